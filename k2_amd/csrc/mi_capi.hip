@@ -1,0 +1,73 @@
+// extern "C" entry points of the MI recursion: argument checks and kernel selection.
+#include "common.h"
+#include "mi_internal.h"
+
+using namespace k2amd;
+
+namespace {
+
+bool ShapeOk(int B, int S, int T) {
+  if (B < 0 || S < 0 || T < 0) return false;
+  // kernels index one sequence's lattice with 32-bit offsets
+  return ((int64_t)S + 1) * ((int64_t)T + 1) < (int64_t)1 << 31;
+}
+
+}  // namespace
+
+extern "C" {
+
+int k2amd_version(void) { return K2AMD_VERSION; }
+
+const char *k2amd_status_string(int status) {
+  switch (status) {
+    case K2AMD_OK: return "ok";
+    case K2AMD_ERR_INVALID_ARGUMENT: return "invalid argument";
+    case K2AMD_ERR_UNSUPPORTED: return "unsupported size for this build";
+    case K2AMD_ERR_WORKSPACE: return "workspace missing or too small";
+    case K2AMD_ERR_LAUNCH: return "HIP launch error";
+    default: return "unknown status";
+  }
+}
+
+size_t k2amd_mi_workspace_bytes(int B, int S, int T, int modified, int dtype) {
+  (void)B; (void)S; (void)T; (void)modified; (void)dtype;
+  return 0;
+}
+
+int k2amd_mi_forward(const void *px, const void *py, const int64_t *boundary, void *p, void *ans,
+                     int B, int S, int T, int modified, int dtype, void *workspace,
+                     size_t workspace_bytes, void *stream) {
+  (void)workspace; (void)workspace_bytes;
+  if (!ShapeOk(B, S, T) || (dtype != K2AMD_F32 && dtype != K2AMD_F64)) return K2AMD_ERR_INVALID_ARGUMENT;
+  if (B == 0) return K2AMD_OK;
+  if (!p || !ans || (!px && S > 0) || (!py && T > 0)) return K2AMD_ERR_INVALID_ARGUMENT;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  modified = modified ? 1 : 0;
+  if (dtype == K2AMD_F32)
+    return MiForwardGeneric<float>((const float *)px, (const float *)py, boundary, (float *)p,
+                                   (float *)ans, B, S, T, modified, st);
+  return MiForwardGeneric<double>((const double *)px, (const double *)py, boundary, (double *)p,
+                                  (double *)ans, B, S, T, modified, st);
+}
+
+int k2amd_mi_backward(const void *px, const void *py, const int64_t *boundary, const void *p,
+                      void *ans_grad, void *px_grad, void *py_grad, int B, int S, int T,
+                      int modified, int dtype, int overwrite_ans_grad, void *workspace,
+                      size_t workspace_bytes, void *stream) {
+  (void)workspace; (void)workspace_bytes; (void)py;
+  if (!ShapeOk(B, S, T) || (dtype != K2AMD_F32 && dtype != K2AMD_F64)) return K2AMD_ERR_INVALID_ARGUMENT;
+  if (B == 0) return K2AMD_OK;
+  if (!p || !ans_grad || (!px && S > 0) || (!px_grad && S > 0) || (!py_grad && T > 0))
+    return K2AMD_ERR_INVALID_ARGUMENT;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  modified = modified ? 1 : 0;
+  if (dtype == K2AMD_F32)
+    return MiBackwardGeneric<float>((const float *)px, (const float *)p, boundary,
+                                    (float *)ans_grad, (float *)px_grad, (float *)py_grad, B, S, T,
+                                    modified, overwrite_ans_grad, st);
+  return MiBackwardGeneric<double>((const double *)px, (const double *)p, boundary,
+                                   (double *)ans_grad, (double *)px_grad, (double *)py_grad, B, S,
+                                   T, modified, overwrite_ans_grad, st);
+}
+
+}  // extern "C"

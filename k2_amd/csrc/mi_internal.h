@@ -1,0 +1,23 @@
+// Launchers shared between the translation units of the MI recursion.
+#ifndef K2_AMD_CSRC_MI_INTERNAL_H_
+#define K2_AMD_CSRC_MI_INTERNAL_H_
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace k2amd {
+
+// Log-domain, one workgroup per sequence (mi_generic.hip).
+template <typename T>
+int MiForwardGeneric(const T *px, const T *py, const int64_t *boundary, T *p, T *ans, int B,
+                     int S, int Tn, int modified, hipStream_t stream);
+template <typename T>
+int MiBackwardGeneric(const T *px, const T *p, const int64_t *boundary, T *ans_grad, T *px_grad,
+                      T *py_grad, int B, int S, int Tn, int modified, int overwrite_ans_grad,
+                      hipStream_t stream);
+size_t MiGenericMaxRows(int dtype);
+
+}  // namespace k2amd
+
+#endif  // K2_AMD_CSRC_MI_INTERNAL_H_
