@@ -1,0 +1,147 @@
+#!/usr/bin/env python3
+"""Headline benchmark: MI recursion forward + backward on one MI355X.
+
+Workload (BASELINE config 4): fp32, modified lattice, B=32, S=200, T=1000, px/py = min(N(-3,1), 0),
+per-sequence boundary with T_b in [600,1000] and S_b in [100,200].  One step = one forward
+launch + one backward launch through the C-ABI, inputs resident in HBM.
+
+Prints ONE JSON line (see README / DESIGN.md for the field meanings).  `value` counts ACTIVE
+lattice cells, sum_b (S_b+1)(T_b+1), per second of fwd+bwd wall time on the GPU.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+# Algorithmic bytes per lattice cell, fp32: forward reads px, py and writes p (12 B); backward
+# reads px, p and writes px_grad, py_grad (16 B; the backward never needs py).
+FWD_BYTES_PER_CELL = 12
+BWD_BYTES_PER_CELL = 16
+
+
+def cpu_baseline(c, budget_s=12.0):
+    """Times the CPU path on this host, single-threaded like the reference's loops
+    (k2/python/csrc/torch/mutual_information_cpu.cu:89,179 have no parallel_for)."""
+    from oracle import mi as omi
+    kind = "reference" if omi.have_ref() else "port"
+    backend = "ref" if kind == "reference" else "port"
+    px, py, bd = c["px"], c["py"], c["boundary"]
+    cells = int(((bd[:, 2] - bd[:, 0] + 1) * (bd[:, 3] - bd[:, 1] + 1)).sum())
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 3 or (time.perf_counter() - t_start < budget_s and len(times) < 50):
+        t0 = time.perf_counter()
+        ans, p = omi.mi_forward(px, py, bd, backend=backend)
+        omi.mi_backward(px, py, bd, p, backend=backend)
+        times.append(time.perf_counter() - t0)
+    med = float(np.median(times))
+    return {
+        "value": cells / med, "unit": "cells/s", "cores": 1, "kind": kind,
+        "sample": f"the same B={c['B']} S={c['S']} T={c['T']} workload, {len(times)} full fwd+bwd "
+                  f"passes, median {med * 1e3:.1f} ms (host has {os.cpu_count()} logical cpus)",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--B", type=int, default=32)
+    ap.add_argument("--S", type=int, default=200)
+    ap.add_argument("--T", type=int, default=1000)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (the batch axis would "
+              "shard trivially, see DESIGN.md); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import cases
+    from k2_amd import capi
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda", 0)
+    c = cases.c4_case(B=args.B, S=args.S, T=args.T)
+    px = torch.from_numpy(c["px"]).to(dev)
+    py = torch.from_numpy(c["py"]).to(dev)
+    bd = torch.from_numpy(c["boundary"]).to(dev)
+    B, S, T = c["B"], c["S"], c["T"]
+    bnp = c["boundary"]
+    active = int(((bnp[:, 2] - bnp[:, 0] + 1) * (bnp[:, 3] - bnp[:, 1] + 1)).sum())
+    full = B * (S + 1) * (T + 1)
+    p = torch.empty(B, S + 1, T + 1, dtype=torch.float32, device=dev)
+    ones = torch.ones(B, dtype=torch.float32, device=dev)
+
+    def step(ev=None):
+        if ev is not None:
+            ev[0].record()
+        capi.mi_forward(px, py, bd, p)
+        if ev is not None:
+            ev[1].record()
+        g = capi.mi_backward(px, py, bd, p, ones, overwrite_ans_grad=False)
+        if ev is not None:
+            ev[2].record()
+        return g
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        step(events[k])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    fwd_ms = np.array([e[0].elapsed_time(e[1]) for e in events])
+    bwd_ms = np.array([e[1].elapsed_time(e[2]) for e in events])
+    ms_per_step = wall / args.steps * 1e3
+
+    # Roofline of the dominant kernel (the one with the longer average launch).
+    fwd_avg, bwd_avg = float(fwd_ms.mean()), float(bwd_ms.mean())
+    if bwd_avg >= fwd_avg:
+        dom, dom_ms, dom_bytes = "mi_backward", bwd_avg, BWD_BYTES_PER_CELL * active
+    else:
+        dom, dom_ms, dom_bytes = "mi_forward", fwd_avg, FWD_BYTES_PER_CELL * active
+    achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
+    both_bytes = (FWD_BYTES_PER_CELL + BWD_BYTES_PER_CELL) * active
+    out = {
+        "metric": "MI recursion fwd+bwd lattice-cells/s (B=32,S=200,T=1000) + % HBM roofline",
+        "value": active / (ms_per_step * 1e-3),
+        "unit": "cells/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"mutual_information_recursion fwd+bwd, fp32, modified, B={B} "
+                               f"S={S} T={T}, random boundary (BASELINE config 4)",
+                   "active_cells": active, "full_box_cells": full},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": dom,
+                     "kernel_avg_us": dom_ms * 1e3},
+        "kernels": {"mi_forward_avg_us": fwd_avg * 1e3, "mi_forward_min_us": float(fwd_ms.min()) * 1e3,
+                    "mi_backward_avg_us": bwd_avg * 1e3, "mi_backward_min_us": float(bwd_ms.min()) * 1e3,
+                    "fwd_bwd_GBps_active_cells": both_bytes / ((fwd_avg + bwd_avg) * 1e-3) / 1e9,
+                    "fwd_bwd_frac_of_hbm_peak": both_bytes / ((fwd_avg + bwd_avg) * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                    "full_box_cells_per_s": full / ((fwd_avg + bwd_avg) * 1e-3)},
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(c)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
