@@ -71,6 +71,81 @@ K2AMD_API int k2amd_mi_backward(const void *px, const void *py, const int64_t *b
                       int modified, int dtype, int overwrite_ans_grad, void *workspace,
                       size_t workspace_bytes, void *stream);
 
+/* ------------------------------------------------------------------ RNN-T log-prob builders
+ *
+ * Common conventions: symbols [B][S] int64 in [0,C); boundary [B][4] int64 or NULL;
+ * px [B][S][T1] with T1 = T+1 for K2AMD_REGULAR (column T is -inf) and T otherwise;
+ * py [B][S+1][T].  "constrained" adds py[b,s+1,t] to px[b,s,t]; "regular" with a boundary sets
+ * px[b,:,t_end[b]] = -inf (k2/python/k2/rnnt_loss.py:25-43,220-223).  The *_backward functions
+ * take the gradients w.r.t. the px / py that the matching forward returned.
+ */
+
+/* Replaces get_rnnt_logprobs (k2/python/k2/rnnt_loss.py:65-225):
+ *   N[b,s,t]  = log(sum_c exp(lm[b,s,c]-lm_max[b,s]) * exp(am[b,t,c]-am_max[b,t]) + tiny) + lm_max + am_max
+ *   px[b,s,t] = am[b,t,sym[b,s]] + lm[b,s,sym[b,s]] - N[b,s,t];  py[b,s,t] = am[b,t,blank] + lm[b,s,blank] - N[b,s,t]
+ * lm [B][S+1][C], am [B][T][C].  The caller provides the buffers that the backward re-uses:
+ * lm_probs [B][S+1][C], am_probs [B][T][C] (the max-shifted exponentials), lm_max [B][S+1],
+ * am_max [B][T] and denom [B][S+1][T] (= the matmul + tiny).                                    */
+K2AMD_API int k2amd_rnnt_logprobs_simple_forward(
+    const void *lm, const void *am, const int64_t *symbols, const int64_t *boundary, void *px,
+    void *py, void *lm_probs, void *am_probs, void *lm_max, void *am_max, void *denom, int B, int S,
+    int T, int C, int termination_symbol, int rnnt_type, int dtype, void *stream);
+
+/* Gradient of the above w.r.t. lm and am (what torch autograd derives from
+ * k2/python/k2/rnnt_loss.py:172-223).  q_scratch [B][S+1][T] is scratch.                         */
+K2AMD_API int k2amd_rnnt_logprobs_simple_backward(
+    const void *px_grad, const void *py_grad, const int64_t *symbols, const int64_t *boundary,
+    const void *lm_probs, const void *am_probs, const void *denom, void *lm_grad, void *am_grad,
+    void *q_scratch, int B, int S, int T, int C, int termination_symbol, int rnnt_type, int dtype,
+    void *stream);
+
+/* Replaces get_rnnt_logprobs_joint (k2/python/k2/rnnt_loss.py:341-447): logits [B][T][S+1][C];
+ * normalizers [B][T][S+1] = logsumexp over C is written for the backward.                        */
+K2AMD_API int k2amd_rnnt_logprobs_joint_forward(
+    const void *logits, const int64_t *symbols, const int64_t *boundary, void *px, void *py,
+    void *normalizers, int B, int S, int T, int C, int termination_symbol, int rnnt_type, int dtype,
+    void *stream);
+K2AMD_API int k2amd_rnnt_logprobs_joint_backward(
+    const void *logits, const void *normalizers, const void *px_grad, const void *py_grad,
+    const int64_t *symbols, const int64_t *boundary, void *logits_grad, int B, int S, int T, int C,
+    int termination_symbol, int rnnt_type, int dtype, void *stream);
+
+/* Replaces get_rnnt_logprobs_pruned (k2/python/k2/rnnt_loss.py:1180-1348): logits [B][T][R][C],
+ * ranges [B][T][R] int64 with values in [0,S]; row k of frame t lands on
+ * s = (ranges[b,t,0] + k) mod (S+1) (k2/python/k2/rnnt_loss.py:957-989), every other element of
+ * px / py is -inf.  normalizers [B][T][R] is written for the backward.                           */
+K2AMD_API int k2amd_rnnt_logprobs_pruned_forward(
+    const void *logits, const int64_t *symbols, const int64_t *ranges, const int64_t *boundary,
+    void *px, void *py, void *normalizers, int B, int S, int T, int R, int C,
+    int termination_symbol, int rnnt_type, int dtype, void *stream);
+K2AMD_API int k2amd_rnnt_logprobs_pruned_backward(
+    const void *logits, const void *normalizers, const void *px_grad, const void *py_grad,
+    const int64_t *symbols, const int64_t *ranges, const int64_t *boundary, void *logits_grad,
+    int B, int S, int T, int R, int C, int termination_symbol, int rnnt_type, int dtype,
+    void *stream);
+
+/* ------------------------------------------------------------------ pruning
+ *
+ * Replaces the device work of get_rnnt_prune_ranges (k2/python/k2/rnnt_loss.py:730-780):
+ * window sum of s_range rows of py_grad (added first row to last), minus px_grad shifted down one
+ * row, first arg-max over the window start, frames t >= t_end-1 pinned to max(s_end-s_range+1, 0),
+ * then the two reverse running minima of _adjust_pruning_lower_bound
+ * (k2/python/k2/rnnt_loss.py:580-630).  s_range is the final value (the caller applies the
+ * adjustments of k2/python/k2/rnnt_loss.py:694-729).  ranges [B][T][s_range] int64.              */
+K2AMD_API int k2amd_rnnt_prune_ranges(const void *px_grad, const void *py_grad,
+                                      const int64_t *boundary, int64_t *ranges, int B, int S, int T,
+                                      int modified, int s_range, int dtype, void *stream);
+
+/* Replaces the gather of do_rnnt_pruning (k2/python/k2/rnnt_loss.py:947-953):
+ * lm_pruned[b,t,k,:] = lm[b, ranges[b,t,k], :]; lm [B][S1][D].  Indices outside [0,S1) yield 0.  */
+K2AMD_API int k2amd_rnnt_prune_gather(const void *lm, const int64_t *ranges, void *lm_pruned, int B,
+                                      int S1, int T, int R, int D, int dtype, void *stream);
+/* Its gradient: lm_grad[b,s,:] = sum over (t,k) with ranges[b,t,k] == s of grad[b,t,k,:].
+ * lm_grad is cleared by the callee.                                                              */
+K2AMD_API int k2amd_rnnt_prune_gather_backward(const void *grad, const int64_t *ranges,
+                                               void *lm_grad, int B, int S1, int T, int R, int D,
+                                               int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

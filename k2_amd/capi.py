@@ -28,6 +28,15 @@ _SIGNATURES = {
     "k2amd_mi_forward": ([_vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp, _sz, _vp], _ci),
     "k2amd_mi_backward": ([_vp, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci,
                            _vp, _sz, _vp], _ci),
+    "k2amd_rnnt_logprobs_simple_forward": ([_vp] * 11 + [_ci] * 7 + [_vp], _ci),
+    "k2amd_rnnt_logprobs_simple_backward": ([_vp] * 10 + [_ci] * 7 + [_vp], _ci),
+    "k2amd_rnnt_logprobs_joint_forward": ([_vp] * 6 + [_ci] * 7 + [_vp], _ci),
+    "k2amd_rnnt_logprobs_joint_backward": ([_vp] * 7 + [_ci] * 7 + [_vp], _ci),
+    "k2amd_rnnt_logprobs_pruned_forward": ([_vp] * 7 + [_ci] * 8 + [_vp], _ci),
+    "k2amd_rnnt_logprobs_pruned_backward": ([_vp] * 8 + [_ci] * 8 + [_vp], _ci),
+    "k2amd_rnnt_prune_ranges": ([_vp] * 4 + [_ci] * 6 + [_vp], _ci),
+    "k2amd_rnnt_prune_gather": ([_vp] * 3 + [_ci] * 6 + [_vp], _ci),
+    "k2amd_rnnt_prune_gather_backward": ([_vp] * 3 + [_ci] * 6 + [_vp], _ci),
 }
 
 
@@ -110,3 +119,133 @@ def mi_backward(px, py, boundary, p, ans_grad, overwrite_ans_grad=True):
                                       int(overwrite_ans_grad), ptr(ws),
                                       0 if ws is None else ws.numel(), stream_ptr(px.device)))
     return px_grad, py_grad
+
+
+def _t1(T, rnnt_type):
+    return T + 1 if rnnt_type == REGULAR else T
+
+
+def logprobs_simple_forward(lm, am, symbols, termination_symbol, rnnt_type, boundary):
+    """C-ABI get_rnnt_logprobs: returns (px, py, saved) with ``saved`` the buffers the backward
+    re-uses (lm_probs, am_probs, denom)."""
+    B, T, C = am.shape
+    S = lm.shape[1] - 1
+    dev, dt = am.device, am.dtype
+    px = torch.empty(B, S, _t1(T, rnnt_type), dtype=dt, device=dev)
+    py = torch.empty(B, S + 1, T, dtype=dt, device=dev)
+    lm_probs = torch.empty_like(lm)
+    am_probs = torch.empty_like(am)
+    lm_max = torch.empty(B, S + 1, dtype=dt, device=dev)
+    am_max = torch.empty(B, T, dtype=dt, device=dev)
+    denom = torch.empty(B, S + 1, T, dtype=dt, device=dev)
+    with torch.cuda.device(dev):
+        check(lib().k2amd_rnnt_logprobs_simple_forward(
+            ptr(lm), ptr(am), ptr(symbols), ptr(boundary), ptr(px), ptr(py), ptr(lm_probs),
+            ptr(am_probs), ptr(lm_max), ptr(am_max), ptr(denom), B, S, T, C, termination_symbol,
+            rnnt_type, dtype_code(am), stream_ptr(dev)))
+    return px, py, (lm_probs, am_probs, denom)
+
+
+def logprobs_simple_backward(px_grad, py_grad, symbols, boundary, saved, termination_symbol,
+                             rnnt_type):
+    lm_probs, am_probs, denom = saved
+    B, T, C = am_probs.shape
+    S = lm_probs.shape[1] - 1
+    lm_grad = torch.empty_like(lm_probs)
+    am_grad = torch.empty_like(am_probs)
+    q = torch.empty_like(denom)
+    dev = am_probs.device
+    with torch.cuda.device(dev):
+        check(lib().k2amd_rnnt_logprobs_simple_backward(
+            ptr(px_grad), ptr(py_grad), ptr(symbols), ptr(boundary), ptr(lm_probs), ptr(am_probs),
+            ptr(denom), ptr(lm_grad), ptr(am_grad), ptr(q), B, S, T, C, termination_symbol,
+            rnnt_type, dtype_code(am_probs), stream_ptr(dev)))
+    return lm_grad, am_grad
+
+
+def logprobs_joint_forward(logits, symbols, termination_symbol, rnnt_type, boundary):
+    B, T, S1, C = logits.shape
+    S = S1 - 1
+    dev, dt = logits.device, logits.dtype
+    px = torch.empty(B, S, _t1(T, rnnt_type), dtype=dt, device=dev)
+    py = torch.empty(B, S + 1, T, dtype=dt, device=dev)
+    norm = torch.empty(B, T, S1, dtype=dt, device=dev)
+    with torch.cuda.device(dev):
+        check(lib().k2amd_rnnt_logprobs_joint_forward(
+            ptr(logits), ptr(symbols), ptr(boundary), ptr(px), ptr(py), ptr(norm), B, S, T, C,
+            termination_symbol, rnnt_type, dtype_code(logits), stream_ptr(dev)))
+    return px, py, norm
+
+
+def logprobs_joint_backward(logits, norm, px_grad, py_grad, symbols, boundary,
+                            termination_symbol, rnnt_type):
+    B, T, S1, C = logits.shape
+    grad = torch.empty_like(logits)
+    dev = logits.device
+    with torch.cuda.device(dev):
+        check(lib().k2amd_rnnt_logprobs_joint_backward(
+            ptr(logits), ptr(norm), ptr(px_grad), ptr(py_grad), ptr(symbols), ptr(boundary),
+            ptr(grad), B, S1 - 1, T, C, termination_symbol, rnnt_type, dtype_code(logits),
+            stream_ptr(dev)))
+    return grad
+
+
+def logprobs_pruned_forward(logits, symbols, ranges, termination_symbol, boundary, rnnt_type):
+    B, T, R, C = logits.shape
+    S = symbols.shape[1]
+    dev, dt = logits.device, logits.dtype
+    px = torch.empty(B, S, _t1(T, rnnt_type), dtype=dt, device=dev)
+    py = torch.empty(B, S + 1, T, dtype=dt, device=dev)
+    norm = torch.empty(B, T, R, dtype=dt, device=dev)
+    with torch.cuda.device(dev):
+        check(lib().k2amd_rnnt_logprobs_pruned_forward(
+            ptr(logits), ptr(symbols), ptr(ranges), ptr(boundary), ptr(px), ptr(py), ptr(norm),
+            B, S, T, R, C, termination_symbol, rnnt_type, dtype_code(logits), stream_ptr(dev)))
+    return px, py, norm
+
+
+def logprobs_pruned_backward(logits, norm, px_grad, py_grad, symbols, ranges, boundary,
+                             termination_symbol, rnnt_type):
+    B, T, R, C = logits.shape
+    S = symbols.shape[1]
+    grad = torch.empty_like(logits)
+    dev = logits.device
+    with torch.cuda.device(dev):
+        check(lib().k2amd_rnnt_logprobs_pruned_backward(
+            ptr(logits), ptr(norm), ptr(px_grad), ptr(py_grad), ptr(symbols), ptr(ranges),
+            ptr(boundary), ptr(grad), B, S, T, R, C, termination_symbol, rnnt_type,
+            dtype_code(logits), stream_ptr(dev)))
+    return grad
+
+
+def prune_ranges(px_grad, py_grad, boundary, s_range):
+    """``s_range`` is the final value (after the adjustments the Python layer applies)."""
+    B, S, T1 = px_grad.shape
+    T = py_grad.shape[2]
+    ranges = torch.empty(B, T, s_range, dtype=torch.int64, device=px_grad.device)
+    dev = px_grad.device
+    with torch.cuda.device(dev):
+        check(lib().k2amd_rnnt_prune_ranges(ptr(px_grad), ptr(py_grad), ptr(boundary), ptr(ranges),
+                                            B, S, T, int(T1 == T), s_range, dtype_code(px_grad),
+                                            stream_ptr(dev)))
+    return ranges
+
+
+def prune_gather(lm, ranges):
+    B, S1, D = lm.shape
+    _, T, R = ranges.shape
+    out = torch.empty(B, T, R, D, dtype=lm.dtype, device=lm.device)
+    with torch.cuda.device(lm.device):
+        check(lib().k2amd_rnnt_prune_gather(ptr(lm), ptr(ranges), ptr(out), B, S1, T, R, D,
+                                            dtype_code(lm), stream_ptr(lm.device)))
+    return out
+
+
+def prune_gather_backward(grad, ranges, S1):
+    B, T, R, D = grad.shape
+    lm_grad = torch.empty(B, S1, D, dtype=grad.dtype, device=grad.device)
+    with torch.cuda.device(grad.device):
+        check(lib().k2amd_rnnt_prune_gather_backward(ptr(grad), ptr(ranges), ptr(lm_grad), B, S1,
+                                                     T, R, D, dtype_code(grad),
+                                                     stream_ptr(grad.device)))
+    return lm_grad

@@ -1,0 +1,284 @@
+// Row-streaming kernels of the RNN-T log-prob builders that take joiner logits:
+//   get_rnnt_logprobs_joint   logits [B][T][S+1][C]   (k2/python/k2/rnnt_loss.py:341-447)
+//   get_rnnt_logprobs_pruned  logits [B][T][R][C]     (k2/python/k2/rnnt_loss.py:1180-1348)
+//
+// Both are one pass over the logits: one 64-lane wavefront owns one row of C logits, keeps it in
+// registers, reduces max and sum(exp) across lanes with DPP-style shuffles, and emits the two
+// values px / py that the row contributes (symbol and termination log-probs).  The backward is the
+// mirror pass: read the row once, write its gradient once.  HBM traffic is the algorithmic
+// minimum (logits read once forward; read once + written once backward).
+#include "common.h"
+
+namespace k2amd {
+namespace {
+
+constexpr int kRowsPerBlock = 4;  // one wavefront per row, 256 threads per workgroup
+constexpr int kMaxRegs = 8;       // register-resident path covers C <= 64 * 8
+
+template <typename T>
+__device__ __forceinline__ T WaveMax(T v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = max(v, __shfl_xor(v, off, kWave));
+  return v;
+}
+template <typename T>
+__device__ __forceinline__ T WaveSum(T v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+  return v;
+}
+
+// logsumexp of one row, torch semantics (an infinite maximum is replaced by 0 before the
+// subtraction, so an all -inf row yields -inf rather than NaN).
+template <typename T>
+__device__ __forceinline__ T RowLogSumExp(const T *__restrict__ x, int C, int lane) {
+  T m = Real<T>::NegInf();
+  T sum = 0;
+  if (C <= kWave * kMaxRegs) {
+    T v[kMaxRegs];
+#pragma unroll
+    for (int i = 0; i < kMaxRegs; ++i) {
+      const int c = lane + i * kWave;
+      v[i] = c < C ? x[c] : Real<T>::NegInf();
+      m = max(m, v[i]);
+    }
+    m = WaveMax(m);
+    if (m - m != 0) m = 0;  // +-inf (or NaN) maximum
+#pragma unroll
+    for (int i = 0; i < kMaxRegs; ++i) sum += Real<T>::Exp(v[i] - m);
+  } else {
+    for (int c = lane; c < C; c += kWave) m = max(m, x[c]);
+    m = WaveMax(m);
+    if (m - m != 0) m = 0;
+    for (int c = lane; c < C; c += kWave) sum += Real<T>::Exp(x[c] - m);
+  }
+  sum = WaveSum(sum);
+  return Real<T>::Log(sum) + m;
+}
+
+struct RowGeom {
+  int B, S, Tn, K, C;  // K rows per frame: S+1 (joint) or R (pruned)
+  int blank, rnnt_type;
+};
+
+// Maps row (b,t,k) to its lattice row s and to the symbol whose log-prob goes to px.
+template <bool kPruned>
+__device__ __forceinline__ void RowTarget(const RowGeom &g, const int64_t *__restrict__ symbols,
+                                          const int64_t *__restrict__ ranges, int b, int t, int k,
+                                          int *s, int *sym) {
+  if (kPruned) {
+    const int64_t *r = ranges + ((size_t)b * g.Tn + t) * g.K;
+    int64_t shift = r[0], src = r[k];
+    int S1 = g.S + 1;
+    int ss = (int)((k + shift) % S1);
+    if (ss < 0) ss += S1;
+    *s = ss;
+    // the symbol is looked up at ranges[b,t,k] in `symbols` extended by the termination symbol
+    if (src >= 0 && src < g.S) *sym = (int)symbols[(size_t)b * g.S + src];
+    else if (src == g.S) *sym = g.blank;
+    else *sym = -1;
+  } else {
+    *s = k;
+    *sym = k < g.S ? (int)symbols[(size_t)b * g.S + k] : -1;
+  }
+}
+
+template <typename T, bool kPruned>
+__global__ __launch_bounds__(kRowsPerBlock *kWave) void RowForwardKernel(
+    const T *__restrict__ logits, const int64_t *__restrict__ symbols,
+    const int64_t *__restrict__ ranges, const int64_t *__restrict__ boundary, T *__restrict__ px,
+    T *__restrict__ py, T *__restrict__ normalizers, RowGeom g) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const long long row = (long long)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
+  const long long rows = (long long)g.B * g.Tn * g.K;
+  if (row >= rows) return;
+  const int k = (int)(row % g.K);
+  const int t = (int)((row / g.K) % g.Tn);
+  const int b = (int)(row / ((long long)g.K * g.Tn));
+  const T *x = logits + (size_t)row * g.C;
+  const T norm = RowLogSumExp<T>(x, g.C, lane);
+  if (lane != 0) return;
+  normalizers[row] = norm;
+  int s, sym;
+  RowTarget<kPruned>(g, symbols, ranges, b, t, k, &s, &sym);
+  const int T1 = g.rnnt_type == K2AMD_REGULAR ? g.Tn + 1 : g.Tn;
+  if (s < g.S) {
+    T v = (sym >= 0 && sym < g.C) ? x[sym] - norm : Real<T>::NegInf();
+    if (g.rnnt_type == K2AMD_REGULAR && boundary != nullptr && boundary[4 * b + 3] == t)
+      v = Real<T>::NegInf();
+    px[((size_t)b * g.S + s) * T1 + t] = v;
+  }
+  py[((size_t)b * (g.S + 1) + s) * g.Tn + t] = x[g.blank] - norm;
+}
+
+template <typename T>
+__global__ void FillKernel(T *__restrict__ dst, size_t n, T value) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (size_t)gridDim.x * blockDim.x)
+    dst[i] = value;
+}
+
+// px[b,s,T] = -inf for a regular lattice (k2/python/k2/rnnt_loss.py:193-205).
+template <typename T>
+__global__ void LastColumnKernel(T *__restrict__ px, int rows, int T1) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < rows) px[(size_t)i * T1 + (T1 - 1)] = Real<T>::NegInf();
+}
+
+// px[b,s,t] += py[b,s+1,t] (k2/python/k2/rnnt_loss.py:222-223); T1 == Tn here.
+template <typename T>
+__global__ void ConstrainedKernel(T *__restrict__ px, const T *__restrict__ py, int B, int S,
+                                  int Tn) {
+  const size_t n = (size_t)B * S * Tn;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (size_t)gridDim.x * blockDim.x) {
+    const size_t b = i / ((size_t)S * Tn), rem = i - b * (size_t)S * Tn;
+    px[i] += py[b * (size_t)(S + 1) * Tn + Tn + rem];
+  }
+}
+
+template <typename T, bool kPruned>
+__global__ __launch_bounds__(kRowsPerBlock *kWave) void RowBackwardKernel(
+    const T *__restrict__ logits, const T *__restrict__ normalizers,
+    const T *__restrict__ px_grad, const T *__restrict__ py_grad,
+    const int64_t *__restrict__ symbols, const int64_t *__restrict__ ranges,
+    const int64_t *__restrict__ boundary, T *__restrict__ logits_grad, RowGeom g) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const long long row = (long long)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
+  const long long rows = (long long)g.B * g.Tn * g.K;
+  if (row >= rows) return;
+  const int k = (int)(row % g.K);
+  const int t = (int)((row / g.K) % g.Tn);
+  const int b = (int)(row / ((long long)g.K * g.Tn));
+  int s, sym;
+  RowTarget<kPruned>(g, symbols, ranges, b, t, k, &s, &sym);
+  const int T1 = g.rnnt_type == K2AMD_REGULAR ? g.Tn + 1 : g.Tn;
+  // gradient reaching this row's px value and py value
+  T gx = 0;
+  if (s < g.S && sym >= 0 && sym < g.C) {
+    const bool cut =
+        g.rnnt_type == K2AMD_REGULAR && boundary != nullptr && boundary[4 * b + 3] == t;
+    if (!cut) gx = px_grad[((size_t)b * g.S + s) * T1 + t];
+  }
+  T gy = py_grad[((size_t)b * (g.S + 1) + s) * g.Tn + t];
+  if (g.rnnt_type == K2AMD_CONSTRAINED && s >= 1)
+    gy += px_grad[((size_t)b * g.S + (s - 1)) * T1 + t];  // px += py[:, 1:]
+  const T norm = normalizers[row];
+  const T tot = gx + gy;
+  const T *x = logits + (size_t)row * g.C;
+  T *dx = logits_grad + (size_t)row * g.C;
+  for (int c = lane; c < g.C; c += kWave) {
+    T v = -Real<T>::Exp(x[c] - norm) * tot;
+    if (c == sym) v += gx;
+    if (c == g.blank) v += gy;
+    dx[c] = v;
+  }
+}
+
+template <typename T, bool kPruned>
+int RowForward(const T *logits, const int64_t *symbols, const int64_t *ranges,
+               const int64_t *boundary, T *px, T *py, T *normalizers, RowGeom g,
+               hipStream_t stream) {
+  const int T1 = g.rnnt_type == K2AMD_REGULAR ? g.Tn + 1 : g.Tn;
+  const size_t n_px = (size_t)g.B * g.S * T1, n_py = (size_t)g.B * (g.S + 1) * g.Tn;
+  if (kPruned) {
+    if (n_px) hipLaunchKernelGGL(FillKernel<T>, dim3(1024), dim3(256), 0, stream, px, n_px, Real<T>::NegInf());
+    if (n_py) hipLaunchKernelGGL(FillKernel<T>, dim3(1024), dim3(256), 0, stream, py, n_py, Real<T>::NegInf());
+  } else if (g.rnnt_type == K2AMD_REGULAR && g.B * g.S > 0) {
+    hipLaunchKernelGGL(LastColumnKernel<T>, dim3((g.B * g.S + 255) / 256), dim3(256), 0, stream, px, g.B * g.S, T1);
+  }
+  const long long rows = (long long)g.B * g.Tn * g.K;
+  if (rows > 0) {
+    const long long blocks = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
+    hipLaunchKernelGGL((RowForwardKernel<T, kPruned>), dim3((unsigned)blocks), dim3(kRowsPerBlock * kWave), 0, stream,
+                       logits, symbols, ranges, boundary, px, py, normalizers, g);
+  }
+  if (g.rnnt_type == K2AMD_CONSTRAINED && n_px > 0)
+    hipLaunchKernelGGL(ConstrainedKernel<T>, dim3(1024), dim3(256), 0, stream, px, py, g.B, g.S, g.Tn);
+  return LaunchStatus();
+}
+
+template <typename T, bool kPruned>
+int RowBackward(const T *logits, const T *normalizers, const T *px_grad, const T *py_grad,
+                const int64_t *symbols, const int64_t *ranges, const int64_t *boundary,
+                T *logits_grad, RowGeom g, hipStream_t stream) {
+  const long long rows = (long long)g.B * g.Tn * g.K;
+  if (rows > 0) {
+    const long long blocks = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
+    hipLaunchKernelGGL((RowBackwardKernel<T, kPruned>), dim3((unsigned)blocks), dim3(kRowsPerBlock * kWave), 0, stream,
+                       logits, normalizers, px_grad, py_grad, symbols, ranges, boundary,
+                       logits_grad, g);
+  }
+  return LaunchStatus();
+}
+
+bool GeomOk(int B, int S, int T, int K, int C, int blank, int rnnt_type, int dtype) {
+  if (B < 0 || S < 0 || T < 0 || K < 0 || C <= 0 || blank < 0 || blank >= C) return false;
+  if (rnnt_type != K2AMD_REGULAR && rnnt_type != K2AMD_MODIFIED && rnnt_type != K2AMD_CONSTRAINED)
+    return false;
+  if (dtype != K2AMD_F32 && dtype != K2AMD_F64) return false;
+  return (long long)B * T * K < (1ll << 31) * kRowsPerBlock;
+}
+
+}  // namespace
+}  // namespace k2amd
+
+using namespace k2amd;
+
+extern "C" {
+
+int k2amd_rnnt_logprobs_joint_forward(const void *logits, const int64_t *symbols,
+                                      const int64_t *boundary, void *px, void *py,
+                                      void *normalizers, int B, int S, int T, int C,
+                                      int termination_symbol, int rnnt_type, int dtype,
+                                      void *stream) {
+  if (!GeomOk(B, S, T, S + 1, C, termination_symbol, rnnt_type, dtype)) return K2AMD_ERR_INVALID_ARGUMENT;
+  RowGeom g{B, S, T, S + 1, C, termination_symbol, rnnt_type};
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == K2AMD_F32)
+    return RowForward<float, false>((const float *)logits, symbols, nullptr, boundary, (float *)px, (float *)py, (float *)normalizers, g, st);
+  return RowForward<double, false>((const double *)logits, symbols, nullptr, boundary, (double *)px, (double *)py, (double *)normalizers, g, st);
+}
+
+int k2amd_rnnt_logprobs_joint_backward(const void *logits, const void *normalizers,
+                                       const void *px_grad, const void *py_grad,
+                                       const int64_t *symbols, const int64_t *boundary,
+                                       void *logits_grad, int B, int S, int T, int C,
+                                       int termination_symbol, int rnnt_type, int dtype,
+                                       void *stream) {
+  if (!GeomOk(B, S, T, S + 1, C, termination_symbol, rnnt_type, dtype)) return K2AMD_ERR_INVALID_ARGUMENT;
+  RowGeom g{B, S, T, S + 1, C, termination_symbol, rnnt_type};
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == K2AMD_F32)
+    return RowBackward<float, false>((const float *)logits, (const float *)normalizers, (const float *)px_grad, (const float *)py_grad, symbols, nullptr, boundary, (float *)logits_grad, g, st);
+  return RowBackward<double, false>((const double *)logits, (const double *)normalizers, (const double *)px_grad, (const double *)py_grad, symbols, nullptr, boundary, (double *)logits_grad, g, st);
+}
+
+int k2amd_rnnt_logprobs_pruned_forward(const void *logits, const int64_t *symbols,
+                                       const int64_t *ranges, const int64_t *boundary, void *px,
+                                       void *py, void *normalizers, int B, int S, int T, int R,
+                                       int C, int termination_symbol, int rnnt_type, int dtype,
+                                       void *stream) {
+  if (!GeomOk(B, S, T, R, C, termination_symbol, rnnt_type, dtype) || R < 1 || R > S + 1) return K2AMD_ERR_INVALID_ARGUMENT;
+  RowGeom g{B, S, T, R, C, termination_symbol, rnnt_type};
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == K2AMD_F32)
+    return RowForward<float, true>((const float *)logits, symbols, ranges, boundary, (float *)px, (float *)py, (float *)normalizers, g, st);
+  return RowForward<double, true>((const double *)logits, symbols, ranges, boundary, (double *)px, (double *)py, (double *)normalizers, g, st);
+}
+
+int k2amd_rnnt_logprobs_pruned_backward(const void *logits, const void *normalizers,
+                                        const void *px_grad, const void *py_grad,
+                                        const int64_t *symbols, const int64_t *ranges,
+                                        const int64_t *boundary, void *logits_grad, int B, int S,
+                                        int T, int R, int C, int termination_symbol, int rnnt_type,
+                                        int dtype, void *stream) {
+  if (!GeomOk(B, S, T, R, C, termination_symbol, rnnt_type, dtype) || R < 1 || R > S + 1) return K2AMD_ERR_INVALID_ARGUMENT;
+  RowGeom g{B, S, T, R, C, termination_symbol, rnnt_type};
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == K2AMD_F32)
+    return RowBackward<float, true>((const float *)logits, (const float *)normalizers, (const float *)px_grad, (const float *)py_grad, symbols, ranges, boundary, (float *)logits_grad, g, st);
+  return RowBackward<double, true>((const double *)logits, (const double *)normalizers, (const double *)px_grad, (const double *)py_grad, symbols, ranges, boundary, (double *)logits_grad, g, st);
+}
+
+}  // extern "C"

@@ -1,0 +1,131 @@
+"""Drop-in for k2/python/k2/mutual_information.py on MI355X.
+
+Same function names, argument meaning, return values and exception classes as the reference;
+the two native calls ``_k2.mutual_information_forward/backward`` are replaced by the HIP
+kernels of libk2amd.so.  Tensors must live on a ROCm device: there is no CPU fallback.
+"""
+from typing import List, Optional, Sequence, Tuple, Union
+
+import torch
+from torch import Tensor
+
+from . import native
+
+
+class MutualInformationRecursionFunction(torch.autograd.Function):
+    """Mirrors k2/python/k2/mutual_information.py:24-182: the forward runs the recursion and, when
+    gradients may be wanted, the backward recursion with ans_grad = 1 straight away; autograd's
+    backward then only scales the saved occupation probabilities."""
+
+    @staticmethod
+    def forward(ctx, px: Tensor, py: Tensor, pxy_grads: List[Optional[Tensor]],
+                boundary: Optional[Tensor] = None, return_grad: bool = False) -> Tensor:
+        (B, S, T1) = px.shape
+        T = py.shape[-1]
+        assert T1 in [T, T + 1], (T1, T)
+        assert py.shape == (B, S + 1, T), (py.shape, S, T)
+        if boundary is not None:
+            assert boundary.shape == (B, 4), (boundary.shape, B)
+
+        p = torch.empty(B, S + 1, T + 1, device=px.device, dtype=px.dtype)
+        ans = native.mutual_information_forward(px, py, boundary, p)
+
+        px_grad, py_grad = None, None
+        if return_grad or px.requires_grad or py.requires_grad:
+            ans_grad = torch.ones(B, device=px.device, dtype=px.dtype)
+            (px_grad, py_grad) = native.mutual_information_backward(px, py, boundary, p, ans_grad)
+            ctx.save_for_backward(px_grad, py_grad)
+        assert len(pxy_grads) == 2, len(pxy_grads)
+        pxy_grads[0] = px_grad
+        pxy_grads[1] = py_grad
+        return ans
+
+    @staticmethod
+    def backward(ctx, ans_grad: Tensor) -> Tuple[Tensor, Tensor, None, None, None]:
+        (px_grad, py_grad) = ctx.saved_tensors
+        (B,) = ans_grad.shape
+        ans_grad = ans_grad.reshape(B, 1, 1)
+        return (px_grad * ans_grad, py_grad * ans_grad, None, None, None)
+
+
+def mutual_information_recursion(
+    px: Tensor,
+    py: Tensor,
+    boundary: Optional[Tensor] = None,
+    return_grad: bool = False,
+) -> Union[Tuple[Tensor, Tuple[Tensor, Tensor]], Tensor]:
+    """k2.mutual_information_recursion (k2/python/k2/mutual_information.py:185-298).
+
+    px: [B][S][T+1] (regular) or [B][S][T] (modified: inferred from the shape); py: [B][S+1][T];
+    boundary: optional int64 [B][4] = (s_begin, t_begin, s_end, t_end).  Returns scores [B], or
+    (scores, (px_grad, py_grad)) when return_grad is set, the grads being the occupation
+    probabilities d scores.sum() / d px, py.
+    """
+    assert px.ndim == 3, px.shape
+    B, S, T1 = px.shape
+    T = py.shape[-1]
+    assert px.shape[-1] in [T, T + 1], (px.shape, T)
+    assert py.shape == (B, S + 1, T), (py.shape, B, S, T)
+    assert px.dtype == py.dtype, (px.dtype, py.dtype)
+    if boundary is not None:
+        assert boundary.dtype == torch.int64, boundary.dtype
+        assert boundary.shape == (B, 4), (boundary.shape, B)
+        for s_begin, t_begin, s_end, t_end in boundary.tolist():
+            assert 0 <= s_begin <= s_end <= S, (s_begin, s_end, S)
+            assert 0 <= t_begin <= t_end <= T, (t_begin, t_end, T)
+
+    px, py = px.contiguous(), py.contiguous()
+    pxy_grads = [None, None]
+    scores = MutualInformationRecursionFunction.apply(px, py, pxy_grads, boundary, return_grad)
+    px_grad, py_grad = pxy_grads
+    return (scores, (px_grad, py_grad)) if return_grad else scores
+
+
+def _inner_product(a: Tensor, b: Tensor) -> Tensor:
+    """Batched dot product over the last axis: [..., N] x [..., N] -> [...]."""
+    return (a * b).sum(dim=-1)
+
+
+def joint_mutual_information_recursion(
+    px: Sequence[Tensor],
+    py: Sequence[Tensor],
+    boundary: Optional[Tensor] = None,
+) -> Sequence[Tensor]:
+    """k2.joint_mutual_information_recursion (k2/python/k2/mutual_information.py:314-423): runs
+    the recursion on the sums of the given px / py and splits the total score over the N inputs
+    with the occupation probabilities, so that the result summed over N equals the joint score."""
+    N = len(px)
+    assert len(py) == N and N > 0
+    B, S, T1 = px[0].shape
+    T = py[0].shape[-1]
+    assert T1 in [T, T + 1]
+    for x in px:
+        assert x.shape == (B, S, T1) and x.dtype == px[0].dtype
+    for y in py:
+        assert y.shape == (B, S + 1, T) and y.dtype == px[0].dtype
+    if boundary is not None:
+        assert boundary.dtype == torch.int64
+        assert boundary.shape == (B, 4)
+        for s_begin, t_begin, s_end, t_end in boundary.tolist():
+            assert 0 <= s_begin <= s_end <= S, (s_begin, s_end, S)
+            assert 0 <= t_begin <= t_end <= T, (t_begin, t_end, T)
+
+    px_cat = torch.stack(list(px), dim=0)  # [N][B][S][T1]
+    py_cat = torch.stack(list(py), dim=0)  # [N][B][S+1][T]
+    px_tot = px_cat.sum(dim=0).contiguous()
+    py_tot = py_cat.sum(dim=0).contiguous()
+    p = torch.empty(B, S + 1, T + 1, device=px_tot.device, dtype=px_tot.dtype)
+    tot_probs = native.mutual_information_forward(px_tot, py_tot, boundary, p)
+    ans_grad = torch.ones(B, device=px_tot.device, dtype=px_tot.dtype)
+    (px_grad, py_grad) = native.mutual_information_backward(px_tot, py_tot, boundary, p, ans_grad)
+    # -inf inputs carry zero occupation: clamp them to the most negative finite value so that
+    # 0 * -inf does not produce NaN (k2/python/k2/mutual_information.py:410-411)
+    lowest = torch.finfo(px_cat.dtype).min
+    x_prods = _inner_product(px_grad.reshape(1, B, -1), px_cat.reshape(N, B, -1).clamp(min=lowest))
+    y_prods = _inner_product(py_grad.reshape(1, B, -1), py_cat.reshape(N, B, -1).clamp(min=lowest))
+    prods = x_prods + y_prods  # [N][B]
+    # the first element absorbs the gap between the sum of logs and the log of the sum
+    with torch.no_grad():
+        offset = tot_probs - prods.sum(dim=0)
+    prods[0] += offset
+    return prods

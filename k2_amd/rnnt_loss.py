@@ -1,0 +1,357 @@
+"""Drop-in for the RNN-T loss functions of k2/python/k2/rnnt_loss.py on MI355X.
+
+Function names, arguments, return values, warnings and exception classes follow the reference.
+Where the reference chains 15-25 torch ops per call, each builder here is one fused HIP kernel
+(plus its hand-written backward), reached through a torch.autograd.Function so that
+``loss.backward()`` works as before.  Tensors must live on a ROCm device.
+"""
+from typing import Optional, Tuple, Union
+
+import torch
+from torch import Tensor
+
+from . import capi
+from .mutual_information import mutual_information_recursion
+
+_RNNT_TYPES = ("regular", "modified", "constrained")
+
+
+def _dev_i64(t: Optional[Tensor], like: Tensor) -> Optional[Tensor]:
+    if t is None:
+        return None
+    assert t.dtype == torch.int64, t.dtype
+    return t.to(like.device).contiguous()
+
+
+def fix_for_boundary(px: Tensor, boundary: Optional[Tensor] = None) -> Tensor:
+    """k2/python/k2/rnnt_loss.py:25-43: px[b, :, boundary[b, 3]] = -inf, in place (the fused
+    builders below already do this; kept for callers that build px themselves)."""
+    if boundary is None:
+        return px
+    B, S, T1 = px.shape
+    index = boundary[:, 3].reshape(B, 1, 1).expand(B, S, T1)
+    return px.scatter_(dim=2, index=index, value=float("-inf"))
+
+
+def _validate_st_lengths(S: int, T: int, is_rnnt_type_regular: bool,
+                         boundary: Optional[Tensor] = None):
+    """k2/python/k2/rnnt_loss.py:46-62."""
+    assert S >= 0, S
+    if boundary is None:
+        assert is_rnnt_type_regular or T >= S, \
+            f"Modified transducer requires T >= S, but got T={T} and S={S}"
+    else:
+        Ss = boundary[:, 2]
+        Ts = boundary[:, 3]
+        assert is_rnnt_type_regular or bool((Ts >= Ss).all()), \
+            f"Modified transducer requires T >= S, but got T={Ts} and S={Ss}"
+
+
+class _LogprobsSimple(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, lm, am, symbols, termination_symbol, rnnt_code, boundary):
+        lm_c, am_c = lm.contiguous(), am.contiguous()
+        px, py, saved = capi.logprobs_simple_forward(lm_c, am_c, symbols, termination_symbol,
+                                                     rnnt_code, boundary)
+        ctx.save_for_backward(*saved)
+        ctx.meta = (symbols, boundary, termination_symbol, rnnt_code)
+        return px, py
+
+    @staticmethod
+    def backward(ctx, px_grad, py_grad):
+        symbols, boundary, termination_symbol, rnnt_code = ctx.meta
+        lm_grad, am_grad = capi.logprobs_simple_backward(
+            px_grad.contiguous(), py_grad.contiguous(), symbols, boundary, ctx.saved_tensors,
+            termination_symbol, rnnt_code)
+        return lm_grad, am_grad, None, None, None, None
+
+
+class _LogprobsJoint(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logits, symbols, termination_symbol, rnnt_code, boundary):
+        logits_c = logits.contiguous()
+        px, py, norm = capi.logprobs_joint_forward(logits_c, symbols, termination_symbol,
+                                                   rnnt_code, boundary)
+        ctx.save_for_backward(logits_c, norm)
+        ctx.meta = (symbols, boundary, termination_symbol, rnnt_code)
+        return px, py
+
+    @staticmethod
+    def backward(ctx, px_grad, py_grad):
+        symbols, boundary, termination_symbol, rnnt_code = ctx.meta
+        logits, norm = ctx.saved_tensors
+        grad = capi.logprobs_joint_backward(logits, norm, px_grad.contiguous(),
+                                            py_grad.contiguous(), symbols, boundary,
+                                            termination_symbol, rnnt_code)
+        return grad, None, None, None, None
+
+
+class _LogprobsPruned(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logits, symbols, ranges, termination_symbol, rnnt_code, boundary):
+        logits_c = logits.contiguous()
+        px, py, norm = capi.logprobs_pruned_forward(logits_c, symbols, ranges, termination_symbol,
+                                                    boundary, rnnt_code)
+        ctx.save_for_backward(logits_c, norm)
+        ctx.meta = (symbols, ranges, boundary, termination_symbol, rnnt_code)
+        return px, py
+
+    @staticmethod
+    def backward(ctx, px_grad, py_grad):
+        symbols, ranges, boundary, termination_symbol, rnnt_code = ctx.meta
+        logits, norm = ctx.saved_tensors
+        grad = capi.logprobs_pruned_backward(logits, norm, px_grad.contiguous(),
+                                             py_grad.contiguous(), symbols, ranges, boundary,
+                                             termination_symbol, rnnt_code)
+        return grad, None, None, None, None, None
+
+
+class _PruneGather(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, lm, ranges):
+        ctx.save_for_backward(ranges)
+        ctx.S1 = lm.shape[1]
+        return capi.prune_gather(lm.contiguous(), ranges)
+
+    @staticmethod
+    def backward(ctx, grad):
+        (ranges,) = ctx.saved_tensors
+        return capi.prune_gather_backward(grad.contiguous(), ranges, ctx.S1), None
+
+
+def get_rnnt_logprobs(
+    lm: Tensor,
+    am: Tensor,
+    symbols: Tensor,
+    termination_symbol: int,
+    rnnt_type: str = "regular",
+    boundary: Optional[Tensor] = None,
+) -> Tuple[Tensor, Tensor]:
+    """k2.get_rnnt_logprobs (k2/python/k2/rnnt_loss.py:65-225): lm [B][S+1][C], am [B][T][C],
+    symbols [B][S] -> px [B][S][T+1 or T], py [B][S+1][T] for mutual_information_recursion."""
+    assert lm.ndim == 3, lm.shape
+    assert am.ndim == 3, am.shape
+    assert lm.shape[0] == am.shape[0], (lm.shape, am.shape)
+    assert lm.shape[2] == am.shape[2], (lm.shape, am.shape)
+    (B, T, C) = am.shape
+    S = lm.shape[1] - 1
+    assert symbols.shape == (B, S), (symbols.shape, B, S)
+    assert rnnt_type in _RNNT_TYPES, rnnt_type
+    _validate_st_lengths(S, T, rnnt_type == "regular", boundary)
+    return _LogprobsSimple.apply(lm, am, _dev_i64(symbols, am), int(termination_symbol),
+                                 capi.RNNT_TYPES[rnnt_type], _dev_i64(boundary, am))
+
+
+def _delay_penalty(px: Tensor, boundary: Optional[Tensor], rnnt_type: str,
+                   delay_penalty: float) -> Tensor:
+    """The penalty block shared by the three losses (k2/python/k2/rnnt_loss.py:307-322):
+    px[b,s,t] += ((T_b - 1) / 2 - t) * delay_penalty."""
+    B, S, T0 = px.shape
+    T = T0 if rnnt_type != "regular" else T0 - 1
+    if boundary is None:
+        offset = torch.tensor((T - 1) / 2, dtype=px.dtype, device=px.device).expand(B, 1, 1)
+    else:
+        offset = (boundary[:, 3] - 1) / 2
+    penalty = offset.reshape(B, 1, 1) - torch.arange(T0, device=px.device).reshape(1, 1, T0)
+    penalty = penalty * delay_penalty
+    return px + penalty.to(px.dtype)
+
+
+def _reduce(negated_loss: Tensor, reduction: Optional[str]) -> Tensor:
+    if reduction == "none":
+        return -negated_loss
+    elif reduction == "mean":
+        return -torch.mean(negated_loss)
+    elif reduction == "sum":
+        return -torch.sum(negated_loss)
+    raise ValueError(f"reduction should be ('none' | 'mean' | 'sum'), given {reduction}")
+
+
+def rnnt_loss_simple(
+    lm: Tensor,
+    am: Tensor,
+    symbols: Tensor,
+    termination_symbol: int,
+    boundary: Optional[Tensor] = None,
+    rnnt_type: str = "regular",
+    delay_penalty: float = 0.0,
+    reduction: Optional[str] = "mean",
+    return_grad: bool = False,
+) -> Union[Tensor, Tuple[Tensor, Tuple[Tensor, Tensor]]]:
+    """k2.rnnt_loss_simple (k2/python/k2/rnnt_loss.py:228-338)."""
+    px, py = get_rnnt_logprobs(lm=lm, am=am, symbols=symbols,
+                               termination_symbol=termination_symbol, boundary=boundary,
+                               rnnt_type=rnnt_type)
+    if delay_penalty > 0.0:
+        px = _delay_penalty(px, boundary, rnnt_type, delay_penalty)
+    scores_and_grads = mutual_information_recursion(px=px, py=py, boundary=boundary,
+                                                    return_grad=return_grad)
+    negated_loss = scores_and_grads[0] if return_grad else scores_and_grads
+    loss = _reduce(negated_loss, reduction)
+    return (loss, scores_and_grads[1]) if return_grad else loss
+
+
+def get_rnnt_logprobs_joint(
+    logits: Tensor,
+    symbols: Tensor,
+    termination_symbol: int,
+    rnnt_type: str = "regular",
+    boundary: Optional[Tensor] = None,
+) -> Tuple[Tensor, Tensor]:
+    """k2.get_rnnt_logprobs_joint (k2/python/k2/rnnt_loss.py:341-447): logits [B][T][S+1][C]."""
+    assert logits.ndim == 4, logits.shape
+    (B, T, S1, C) = logits.shape
+    S = S1 - 1
+    assert symbols.shape == (B, S), (symbols.shape, B, S)
+    assert rnnt_type in _RNNT_TYPES, rnnt_type
+    _validate_st_lengths(S, T, rnnt_type == "regular", boundary)
+    return _LogprobsJoint.apply(logits, _dev_i64(symbols, logits), int(termination_symbol),
+                                capi.RNNT_TYPES[rnnt_type], _dev_i64(boundary, logits))
+
+
+def rnnt_loss(
+    logits: Tensor,
+    symbols: Tensor,
+    termination_symbol: int,
+    boundary: Optional[Tensor] = None,
+    rnnt_type: str = "regular",
+    delay_penalty: float = 0.0,
+    reduction: Optional[str] = "mean",
+) -> Tensor:
+    """k2.rnnt_loss (k2/python/k2/rnnt_loss.py:450-540)."""
+    px, py = get_rnnt_logprobs_joint(logits=logits, symbols=symbols,
+                                     termination_symbol=termination_symbol, boundary=boundary,
+                                     rnnt_type=rnnt_type)
+    if delay_penalty > 0.0:
+        px = _delay_penalty(px, boundary, rnnt_type, delay_penalty)
+    negated_loss = mutual_information_recursion(px=px, py=py, boundary=boundary)
+    return _reduce(negated_loss, reduction)
+
+
+def _monotonic_lower_bound(x: Tensor) -> Tensor:
+    """k2/python/k2/rnnt_loss.py:543-577: reverse running minimum along the last axis."""
+    x = torch.flip(x, dims=(-1,))
+    x, _ = torch.cummin(x, dim=-1)
+    return torch.flip(x, dims=(-1,))
+
+
+def _adjust_pruning_lower_bound(s_begin: Tensor, s_range: int) -> Tensor:
+    """k2/python/k2/rnnt_loss.py:580-630 as torch ops (the fused kernel in
+    get_rnnt_prune_ranges does the same on the device in one launch)."""
+    (B, T) = s_begin.shape
+    ramp = (s_range - 1) * torch.arange(0, T, device=s_begin.device)
+    s_begin = _monotonic_lower_bound(s_begin)
+    s_begin = -(s_begin - ramp)
+    s_begin = _monotonic_lower_bound(s_begin)
+    s_begin = torch.clamp(s_begin, min=0)
+    return -(s_begin - ramp)
+
+
+def get_rnnt_prune_ranges(
+    px_grad: Tensor,
+    py_grad: Tensor,
+    boundary: Tensor,
+    s_range: int,
+) -> Tensor:
+    """k2.get_rnnt_prune_ranges (k2/python/k2/rnnt_loss.py:636-780): int64 [B][T][s_range]."""
+    (B, S, T1) = px_grad.shape
+    T = py_grad.shape[-1]
+    is_regular = T1 != T
+    assert T1 in [T, T + 1], (T1, T)
+    S1 = S + 1
+    assert py_grad.shape == (B, S1, T), (py_grad.shape, B, S1, T)
+    assert boundary.shape == (B, 4), (boundary.shape, B)
+    _validate_st_lengths(S, T, is_regular, boundary)
+
+    if is_regular:
+        Ss = boundary[:, 2]
+        Ts = boundary[:, 3]
+        s_range_min = Ss.sub(1).div(Ts, rounding_mode="trunc").add(2).max().item()
+        if s_range < s_range_min:
+            print(f"Warning: get_rnnt_prune_ranges - got s_range={s_range} "
+                  f"for boundaries S={Ss}, T={Ts}. Adjusting to {s_range_min}")
+            s_range = s_range_min
+    if s_range > S:
+        print(f"Warning: get_rnnt_prune_ranges - got s_range={s_range} "
+              f"for boundaries S={S}. Adjusting to {S + 1}")
+        s_range = S + 1
+    if is_regular:
+        assert s_range >= 2, \
+            f"Pruning range for standard RNN-T should be equal to or greater than 2, " \
+            f"or no valid paths could survive pruning. Given {s_range}"
+    else:
+        assert s_range >= 1, \
+            f"Pruning range for modified RNN-T should be equal to or greater than 1, " \
+            f"or no valid paths could survive pruning. Given {s_range}"
+    return capi.prune_ranges(px_grad.detach().contiguous(), py_grad.detach().contiguous(),
+                             _dev_i64(boundary, px_grad), int(s_range))
+
+
+def do_rnnt_pruning(am: Tensor, lm: Tensor, ranges: Tensor) -> Tuple[Tensor, Tensor]:
+    """k2.do_rnnt_pruning (k2/python/k2/rnnt_loss.py:913-954): am_pruned is a broadcast view
+    [B][T][s_range][E]; lm_pruned[b,t,k,:] = lm[b, ranges[b,t,k], :]."""
+    assert ranges.shape[0] == am.shape[0], (ranges.shape, am.shape)
+    assert ranges.shape[0] == lm.shape[0], (ranges.shape, lm.shape)
+    assert am.shape[1] == ranges.shape[1], (am.shape, ranges.shape)
+    (B, T, s_range) = ranges.shape
+    (B, S1, decoder_dim) = lm.shape
+    encoder_dim = am.shape[-1]
+    assert am.shape == (B, T, encoder_dim), (am.shape, B, T, encoder_dim)
+    am_pruned = am.unsqueeze(2).expand((B, T, s_range, encoder_dim))
+    lm_pruned = _PruneGather.apply(lm, _dev_i64(ranges, lm))
+    return am_pruned, lm_pruned
+
+
+def _roll_by_shifts(src: Tensor, shifts: Tensor) -> Tensor:
+    """k2/python/k2/rnnt_loss.py:957-989: out[b,t,s] = src[b,t,(s - shifts[b,t]) mod S] (the
+    fused pruned builder applies this placement itself; kept for callers)."""
+    assert src.dim() == 3, src.shape
+    (B, T, S) = src.shape
+    assert shifts.shape == (B, T), (shifts.shape, B, T)
+    index = (torch.arange(S, device=src.device).view(1, 1, S) - shifts.reshape(B, T, 1)) % S
+    return torch.gather(src, 2, index)
+
+
+def get_rnnt_logprobs_pruned(
+    logits: Tensor,
+    symbols: Tensor,
+    ranges: Tensor,
+    termination_symbol: int,
+    boundary: Tensor,
+    rnnt_type: str = "regular",
+) -> Tuple[Tensor, Tensor]:
+    """k2.get_rnnt_logprobs_pruned (k2/python/k2/rnnt_loss.py:1180-1348): logits
+    [B][T][s_range][C], ranges [B][T][s_range]."""
+    assert logits.ndim == 4, logits.shape
+    (B, T, s_range, C) = logits.shape
+    assert ranges.shape == (B, T, s_range), (ranges.shape, B, T, s_range)
+    (B, S) = symbols.shape
+    assert rnnt_type in _RNNT_TYPES, rnnt_type
+    _validate_st_lengths(S, T, rnnt_type == "regular", boundary)
+    return _LogprobsPruned.apply(logits, _dev_i64(symbols, logits), _dev_i64(ranges, logits),
+                                 int(termination_symbol), capi.RNNT_TYPES[rnnt_type],
+                                 _dev_i64(boundary, logits))
+
+
+def rnnt_loss_pruned(
+    logits: Tensor,
+    symbols: Tensor,
+    ranges: Tensor,
+    termination_symbol: int,
+    boundary: Tensor = None,
+    rnnt_type: str = "regular",
+    delay_penalty: float = 0.0,
+    reduction: Optional[str] = "mean",
+    use_hat_loss: bool = False,
+) -> Tensor:
+    """k2.rnnt_loss_pruned (k2/python/k2/rnnt_loss.py:1351-1468).  The HAT variant
+    (use_hat_loss=True) is not part of this build."""
+    if use_hat_loss:
+        raise NotImplementedError("k2_amd: use_hat_loss=True (get_hat_logprobs_pruned) is not built")
+    px, py = get_rnnt_logprobs_pruned(logits=logits, symbols=symbols, ranges=ranges,
+                                      termination_symbol=termination_symbol, boundary=boundary,
+                                      rnnt_type=rnnt_type)
+    if delay_penalty > 0.0:
+        px = _delay_penalty(px, boundary, rnnt_type, delay_penalty)
+    negated_loss = mutual_information_recursion(px=px, py=py, boundary=boundary)
+    return _reduce(negated_loss, reduction)

@@ -1,0 +1,78 @@
+"""CPU-side checks of the drop-in boundary: the shared library loads without a GPU, exports every
+symbol include/k2_amd.h declares (and the binding declares the same set), argument validation
+returns error codes instead of launching, and the Python layer mirrors the reference's names."""
+import inspect
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "k2_amd.h")).read()
+    return sorted(set(re.findall(r"K2AMD_API\s+[\w\s\*]*?(k2amd_\w+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported_and_bound():
+    from k2_amd import capi
+    lib = capi.lib()
+    names = _declared()
+    assert len(names) >= 14
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/k2_amd.h but not exported"
+    assert sorted(capi.exported_symbols()) == names
+    assert lib.k2amd_version() == 100
+    assert capi.lib().k2amd_status_string(0) == b"ok"
+
+
+def test_invalid_arguments_return_codes_without_a_gpu():
+    from k2_amd import capi
+    lib = capi.lib()
+    # negative sizes / unknown dtype are rejected before any HIP call
+    assert lib.k2amd_mi_forward(None, None, None, None, None, -1, 1, 1, 0, 0, None, 0, None) == 1
+    assert lib.k2amd_mi_forward(None, None, None, None, None, 1, 1, 1, 0, 7, None, 0, None) == 1
+    assert lib.k2amd_mi_backward(None, None, None, None, None, None, None, 1, 1, 1, 0, 0, 0, None, 0, None) == 1
+    assert lib.k2amd_rnnt_prune_ranges(None, None, None, None, 1, 4, 4, 0, 9, 0, None) == 1
+    assert lib.k2amd_rnnt_logprobs_joint_forward(None, None, None, None, None, None, 1, 1, 1, 4, 9, 0, 0, None) == 1
+    # an empty batch is a no-op
+    assert lib.k2amd_mi_forward(None, None, None, None, None, 0, 3, 3, 0, 0, None, 0, None) == 0
+    with pytest.raises(RuntimeError):
+        capi.check(2)
+
+
+def test_python_api_mirrors_reference_signatures():
+    import k2_amd as k2
+    want = {
+        "mutual_information_recursion": ["px", "py", "boundary", "return_grad"],
+        "joint_mutual_information_recursion": ["px", "py", "boundary"],
+        "get_rnnt_logprobs": ["lm", "am", "symbols", "termination_symbol", "rnnt_type", "boundary"],
+        "rnnt_loss_simple": ["lm", "am", "symbols", "termination_symbol", "boundary", "rnnt_type",
+                             "delay_penalty", "reduction", "return_grad"],
+        "get_rnnt_logprobs_joint": ["logits", "symbols", "termination_symbol", "rnnt_type", "boundary"],
+        "rnnt_loss": ["logits", "symbols", "termination_symbol", "boundary", "rnnt_type", "delay_penalty",
+                      "reduction"],
+        "get_rnnt_prune_ranges": ["px_grad", "py_grad", "boundary", "s_range"],
+        "do_rnnt_pruning": ["am", "lm", "ranges"],
+        "get_rnnt_logprobs_pruned": ["logits", "symbols", "ranges", "termination_symbol", "boundary",
+                                     "rnnt_type"],
+        "rnnt_loss_pruned": ["logits", "symbols", "ranges", "termination_symbol", "boundary", "rnnt_type",
+                             "delay_penalty", "reduction", "use_hat_loss"],
+    }
+    for name, params in want.items():
+        assert list(inspect.signature(getattr(k2, name)).parameters) == params, name
+
+
+def test_cpu_tensors_fail_loudly():
+    import torch
+    import k2_amd as k2
+    px = torch.zeros(1, 2, 4)
+    py = torch.zeros(1, 3, 3)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        k2.mutual_information_recursion(px, py)
+    # the reference's own assertions still come first
+    with pytest.raises(AssertionError):
+        k2.mutual_information_recursion(px, torch.zeros(1, 3, 7))
+    with pytest.raises(AssertionError):
+        k2.mutual_information_recursion(px, py, torch.tensor([[0, 0, 5, 3]]))

@@ -1,0 +1,263 @@
+"""Parity of the fused RNN-T kernels (log-prob builders, prune ranges, pruning gather) and of the
+k2-style Python API against the CPU oracle, plus gradients against plain-torch autograd.
+
+Tolerances: fp32 |a-b| <= 1e-5 + 1e-4*|b|; fp64 1e-10; integer outputs bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+import cases
+import torch_ref
+from oracle import mi as omi
+from oracle import rnnt as orn
+
+pytestmark = pytest.mark.gpu
+
+TOL = {np.dtype(np.float32): dict(rtol=1e-4, atol=1e-5), np.dtype(np.float64): dict(rtol=1e-10, atol=1e-10)}
+TYPES = ["regular", "modified", "constrained"]
+
+
+def three_way(name, got, cpu32, cpu64):
+    """Where |p| reaches the thousands one fp32 ulp of p is ~1e-4, so the fp32 CPU oracle's own
+    gradients carry that much rounding noise; the fp64 oracle arbitrates: the GPU's error against
+    fp64 may exceed the stated tolerance only by the fp32 CPU path's own error against fp64."""
+    cpu_err = np.abs(cpu32 - cpu64)
+    gpu_err = np.abs(got - cpu64)
+    budget = 1e-5 + 1e-4 * np.abs(cpu64) + 2.0 * cpu_err.max()
+    print(f"{name}: max|gpu-fp64|={gpu_err.max():.3e} max|cpu32-fp64|={cpu_err.max():.3e}")
+    assert (gpu_err <= budget).all(), (name, gpu_err.max(), cpu_err.max())
+
+
+def dev(x, device):
+    return None if x is None else torch.from_numpy(np.ascontiguousarray(x)).to(device)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("rnnt_type", TYPES)
+def test_logprobs_simple_forward(device, dtype, rnnt_type):
+    from k2_amd import capi
+    for seed, (B, T, S, C), bd in ((1, (3, 37, 9, 50), True), (2, (2, 70, 66, 130), False), (3, (1, 5, 0, 4), True)):
+        c = cases.rnnt_case(seed, B, T, S, C, dtype=dtype, t_lo=max(T // 2, S if rnnt_type != "regular" else 1),
+                            s_lo=S // 2, with_boundary=bd, modified=rnnt_type != "regular")
+        want = orn.logprobs_simple(c["lm"], c["am"], c["symbols"], 0, rnnt_type, c["boundary"])
+        px, py, _ = capi.logprobs_simple_forward(dev(c["lm"], device), dev(c["am"], device), dev(c["symbols"], device),
+                                                 0, capi.RNNT_TYPES[rnnt_type], dev(c["boundary"], device))
+        np.testing.assert_allclose(px.cpu().numpy(), want[0], **TOL[np.dtype(dtype)])
+        np.testing.assert_allclose(py.cpu().numpy(), want[1], **TOL[np.dtype(dtype)])
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("rnnt_type", TYPES)
+def test_logprobs_joint_forward(device, dtype, rnnt_type):
+    from k2_amd import capi
+    rng = np.random.default_rng(11)
+    for (B, T, S, C), bd in (((2, 21, 6, 40), True), ((1, 9, 8, 600), False), ((2, 12, 3, 513), True)):
+        c = cases.rnnt_case(5, B, T, S, C, dtype=dtype, t_lo=max(T // 2, S), s_lo=S // 2, with_boundary=bd,
+                            modified=rnnt_type != "regular")
+        logits = rng.standard_normal((B, T, S + 1, C)).astype(dtype)
+        logits[0, 0, 0, :] = -np.inf  # an all -inf row: logsumexp must give -inf, not NaN
+        logits[0, 0, 0, 1] = 0.5
+        want = orn.logprobs_joint(logits, c["symbols"], 0, rnnt_type, c["boundary"])
+        px, py, _ = capi.logprobs_joint_forward(dev(logits, device), dev(c["symbols"], device), 0,
+                                                capi.RNNT_TYPES[rnnt_type], dev(c["boundary"], device))
+        np.testing.assert_allclose(px.cpu().numpy(), want[0], **TOL[np.dtype(dtype)])
+        np.testing.assert_allclose(py.cpu().numpy(), want[1], **TOL[np.dtype(dtype)])
+
+
+def _random_ranges(rng, B, T, S, R):
+    start = np.sort(rng.integers(0, S - R + 2, (B, T)), axis=1)
+    return (start[:, :, None] + np.arange(R)).astype(np.int64)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("rnnt_type", TYPES)
+def test_logprobs_pruned_forward(device, dtype, rnnt_type):
+    from k2_amd import capi
+    rng = np.random.default_rng(12)
+    for (B, T, S, R, C) in ((2, 30, 10, 4, 33), (3, 17, 5, 6, 100), (1, 8, 7, 2, 500)):
+        c = cases.rnnt_case(6, B, T, S, C, dtype=dtype, t_lo=max(T // 2, S), s_lo=S // 2,
+                            modified=rnnt_type != "regular")
+        logits = rng.standard_normal((B, T, R, C)).astype(dtype)
+        ranges = _random_ranges(rng, B, T, S, R)
+        want = orn.logprobs_pruned(logits, c["symbols"], ranges, 0, c["boundary"], rnnt_type)
+        px, py, _ = capi.logprobs_pruned_forward(dev(logits, device), dev(c["symbols"], device), dev(ranges, device),
+                                                 0, dev(c["boundary"], device), capi.RNNT_TYPES[rnnt_type])
+        np.testing.assert_allclose(px.cpu().numpy(), want[0], **TOL[np.dtype(dtype)])
+        np.testing.assert_allclose(py.cpu().numpy(), want[1], **TOL[np.dtype(dtype)])
+
+
+@pytest.mark.parametrize("modified", [False, True])
+def test_prune_ranges_bit_exact(device, modified):
+    from k2_amd import capi
+    for seed in range(8):
+        B, T, S, C = 4, 60 + 13 * seed, 14 + seed, 12
+        c = cases.rnnt_case(seed, B, T, S, C, t_lo=T // 2, s_lo=S // 2, modified=modified)
+        rt = "modified" if modified else "regular"
+        px, py = orn.logprobs_simple(c["lm"], c["am"], c["symbols"], 0, rt, c["boundary"])
+        _, gx, gy = omi.mi(px, py, c["boundary"])
+        for R in (2, 5, S + 1):
+            want = orn.prune_ranges(gx, gy, c["boundary"], R)
+            got = capi.prune_ranges(dev(gx, device), dev(gy, device), dev(c["boundary"], device), want.shape[2])
+            assert got.dtype == torch.int64
+            assert np.array_equal(got.cpu().numpy(), want), (seed, R)
+
+
+def test_prune_gather_and_its_gradient(device):
+    from k2_amd import capi
+    rng = np.random.default_rng(3)
+    for dtype in (np.float32, np.float64):
+        lm = rng.standard_normal((3, 11, 37)).astype(dtype)
+        ranges = _random_ranges(rng, 3, 20, 10, 4)
+        _, want = orn.do_pruning(np.zeros((3, 20, 5), dtype), lm, ranges)
+        got = capi.prune_gather(dev(lm, device), dev(ranges, device))
+        assert np.array_equal(got.cpu().numpy(), want)
+        g = rng.standard_normal(want.shape).astype(dtype)
+        want_g = np.zeros_like(lm)
+        np.add.at(want_g, (np.arange(3)[:, None, None], ranges), g)
+        got_g = capi.prune_gather_backward(dev(g, device), dev(ranges, device), 11)
+        np.testing.assert_allclose(got_g.cpu().numpy(), want_g, rtol=1e-5 if dtype == np.float32 else 1e-12,
+                                   atol=1e-5 if dtype == np.float32 else 1e-12)
+
+
+@pytest.mark.parametrize("rnnt_type", TYPES)
+def test_api_losses_and_gradients_vs_autograd(device, rnnt_type):
+    """End-to-end through the k2-style API in fp64 against plain torch autograd on the CPU:
+    rnnt_loss_simple (grads to lm, am), rnnt_loss (grads to logits), rnnt_loss_pruned."""
+    import k2_amd as k2
+    B, T, S, C = 3, 11, 4, 7
+    c = cases.rnnt_case(21, B, T, S, C, dtype=np.float64, t_lo=7, s_lo=2, modified=rnnt_type != "regular")
+    bd_cpu = torch.from_numpy(c["boundary"])
+    sym_cpu = torch.from_numpy(c["symbols"])
+    w = torch.linspace(0.5, 1.5, B, dtype=torch.float64)
+
+    # --- simple
+    lm_r = torch.from_numpy(c["lm"]).requires_grad_(True)
+    am_r = torch.from_numpy(c["am"]).requires_grad_(True)
+    px, py = torch_ref.logprobs_simple(lm_r, am_r, sym_cpu, 0, rnnt_type, bd_cpu)
+    loss_r = -torch_ref.mi_scores(px, py, bd_cpu)
+    (loss_r * w).sum().backward()
+    lm_g = dev(c["lm"], device).requires_grad_(True)
+    am_g = dev(c["am"], device).requires_grad_(True)
+    loss_g = k2.rnnt_loss_simple(lm_g, am_g, dev(c["symbols"], device), 0, dev(c["boundary"], device),
+                                 rnnt_type=rnnt_type, reduction="none")
+    (loss_g * w.to(device)).sum().backward()
+    np.testing.assert_allclose(loss_g.detach().cpu().numpy(), loss_r.detach().numpy(), rtol=1e-10)
+    np.testing.assert_allclose(lm_g.grad.cpu().numpy(), lm_r.grad.numpy(), rtol=1e-8, atol=1e-10)
+    np.testing.assert_allclose(am_g.grad.cpu().numpy(), am_r.grad.numpy(), rtol=1e-8, atol=1e-10)
+
+    # --- joint
+    rng = np.random.default_rng(8)
+    logits = rng.standard_normal((B, T, S + 1, C))
+    lg_r = torch.from_numpy(logits).requires_grad_(True)
+    px, py = torch_ref.logprobs_from_logits(lg_r, sym_cpu, 0, rnnt_type, bd_cpu)
+    loss_r = -torch_ref.mi_scores(px, py, bd_cpu)
+    (loss_r * w).sum().backward()
+    lg_g = dev(logits, device).requires_grad_(True)
+    loss_g = k2.rnnt_loss(lg_g, dev(c["symbols"], device), 0, dev(c["boundary"], device), rnnt_type=rnnt_type,
+                          reduction="none")
+    (loss_g * w.to(device)).sum().backward()
+    np.testing.assert_allclose(loss_g.detach().cpu().numpy(), loss_r.detach().numpy(), rtol=1e-10)
+    np.testing.assert_allclose(lg_g.grad.cpu().numpy(), lg_r.grad.numpy(), rtol=1e-8, atol=1e-10)
+
+    # --- pruned (ranges from the simple pass, as in training)
+    loss_s, (gx, gy) = k2.rnnt_loss_simple(lm_g.detach(), am_g.detach(), dev(c["symbols"], device), 0,
+                                           dev(c["boundary"], device), rnnt_type=rnnt_type, reduction="none",
+                                           return_grad=True)
+    ranges = k2.get_rnnt_prune_ranges(gx, gy, dev(c["boundary"], device), 3)
+    R = ranges.shape[2]
+    am_p, lm_p = k2.do_rnnt_pruning(am_g.detach(), lm_g.detach(), ranges)
+    assert am_p.shape == (B, T, R, C) and lm_p.shape == (B, T, R, C)
+    plog = rng.standard_normal((B, T, R, C))
+    pl_r = torch.from_numpy(plog).requires_grad_(True)
+    px, py = torch_ref.logprobs_pruned(pl_r, sym_cpu, ranges.cpu(), 0, bd_cpu, rnnt_type)
+    loss_r = -torch_ref.mi_scores(px, py, bd_cpu)
+    pl_g = dev(plog, device).requires_grad_(True)
+    loss_g = k2.rnnt_loss_pruned(pl_g, dev(c["symbols"], device), ranges, 0, dev(c["boundary"], device),
+                                 rnnt_type=rnnt_type, reduction="none")
+    np.testing.assert_allclose(loss_g.detach().cpu().numpy(), loss_r.detach().numpy(), rtol=1e-10)
+    ok = torch.isfinite(loss_r)
+    if ok.any():
+        (loss_r[ok] * w[ok]).sum().backward()
+        (loss_g[ok.to(device)] * w[ok].to(device)).sum().backward()
+        np.testing.assert_allclose(pl_g.grad.cpu().numpy(), pl_r.grad.numpy(), rtol=1e-8, atol=1e-10)
+
+
+def test_hand_fixture_and_identities(device):
+    """k2/python/tests/rnnt_loss_test.py:120-244: simple == joint(am+lm); invariant to per-frame
+    constants; the value itself is pinned by brute force in the oracle tests."""
+    import k2_amd as k2
+    lm = torch.tensor([[[0, 0, 1], [0, 1, 1], [1, 0, 1], [2, 2, 0]]], dtype=torch.float, device=device)
+    am = torch.tensor([[[0, 1, 2], [0, 0, 0], [0, 2, 4], [0, 3, 3]]], dtype=torch.float, device=device)
+    symbols = torch.tensor([[0, 1, 0]], dtype=torch.long, device=device)
+    want = orn.rnnt_loss_simple(lm.cpu().numpy(), am.cpu().numpy(), symbols.cpu().numpy(), 2, reduction="none")
+    px, py = k2.get_rnnt_logprobs(lm=lm, am=am, symbols=symbols, termination_symbol=2)
+    assert px.shape == (1, 3, 5) and py.shape == (1, 4, 4)
+    m = k2.mutual_information_recursion(px=px, py=py, boundary=None)
+    np.testing.assert_allclose(-m.cpu().numpy(), want, rtol=1e-5)
+    m = k2.rnnt_loss_simple(lm=lm, am=am, symbols=symbols, termination_symbol=2, boundary=None, reduction="none")
+    np.testing.assert_allclose(m.cpu().numpy(), want, rtol=1e-5)
+    logits = am.unsqueeze(2) + lm.unsqueeze(1)
+    m = k2.rnnt_loss(logits=logits, symbols=symbols, termination_symbol=2, boundary=None, reduction="none")
+    np.testing.assert_allclose(m.cpu().numpy(), want, rtol=1e-5)
+    lm2 = lm + torch.randn(1, 4, 1, device=device)
+    am2 = am + torch.randn(1, 4, 1, device=device)
+    m = k2.rnnt_loss_simple(lm=lm2, am=am2, symbols=symbols, termination_symbol=2, boundary=None, reduction="none")
+    np.testing.assert_allclose(m.cpu().numpy(), want, rtol=1e-5)
+    with pytest.raises(ValueError):
+        k2.rnnt_loss_simple(lm=lm, am=am, symbols=symbols, termination_symbol=2, reduction="bogus")
+    with pytest.raises(AssertionError):
+        k2.get_rnnt_logprobs(lm=lm, am=am[:, :, :2], symbols=symbols, termination_symbol=2)
+
+
+def test_config2_rnnt_loss_simple_full_size(device):
+    """BASELINE config 2: B=16, T=250, S=50, V=500, boundary T_b in [150,250], S_b in [20,50]."""
+    import k2_amd as k2
+    c = cases.rnnt_case(2, 16, 250, 50, 500, t_lo=150, s_lo=20)
+    want, (gx_w, gy_w) = orn.rnnt_loss_simple(c["lm"], c["am"], c["symbols"], 0, c["boundary"], reduction="none",
+                                               return_grad=True)
+    got, (gx, gy) = k2.rnnt_loss_simple(dev(c["lm"], device), dev(c["am"], device), dev(c["symbols"], device), 0,
+                                        dev(c["boundary"], device), reduction="none", return_grad=True)
+    np.testing.assert_allclose(got.cpu().numpy(), want, rtol=1e-4, atol=1e-5)
+    f64 = lambda a: a.astype(np.float64)
+    want64, (gx64, gy64) = orn.rnnt_loss_simple(f64(c["lm"]), f64(c["am"]), c["symbols"], 0, c["boundary"],
+                                                 reduction="none", return_grad=True)
+    np.testing.assert_allclose(got.cpu().numpy(), want64, rtol=1e-4, atol=1e-5)
+    three_way("px_grad", gx.cpu().numpy(), gx_w, gx64)
+    three_way("py_grad", gy.cpu().numpy(), gy_w, gy64)
+
+
+def test_config3_prune_and_pruned_loss_full_size(device):
+    """BASELINE config 3: B=32, T=500, S=100, V=500, s_range=5, regular."""
+    import k2_amd as k2
+    B, T, S, C, R = 32, 500, 100, 500, 5
+    c = cases.rnnt_case(3, B, T, S, C, t_lo=300, s_lo=50)
+    _, (gx_w, gy_w) = orn.rnnt_loss_simple(c["lm"], c["am"], c["symbols"], 0, c["boundary"], reduction="none",
+                                            return_grad=True)
+    # integer output from identical grads: bit-exact
+    want_ranges = orn.prune_ranges(gx_w, gy_w, c["boundary"], R)
+    got_ranges = k2.get_rnnt_prune_ranges(dev(gx_w, device), dev(gy_w, device), dev(c["boundary"], device), R)
+    assert np.array_equal(got_ranges.cpu().numpy(), want_ranges)
+    # and through the device pipeline end to end (grads from the HIP MI kernel)
+    _, (gx, gy) = k2.rnnt_loss_simple(dev(c["lm"], device), dev(c["am"], device), dev(c["symbols"], device), 0,
+                                      dev(c["boundary"], device), reduction="none", return_grad=True)
+    dev_ranges = k2.get_rnnt_prune_ranges(gx, gy, dev(c["boundary"], device), R).cpu().numpy()
+    frac = (dev_ranges == want_ranges).mean()
+    print("ranges identical to the CPU pipeline on", frac, "of elements")
+    assert frac > 0.999
+    logits = np.random.default_rng(33).standard_normal((B, T, R, C)).astype(np.float32)
+    want = orn.rnnt_loss_pruned(logits, c["symbols"], want_ranges, 0, c["boundary"], reduction="none")
+    got = k2.rnnt_loss_pruned(dev(logits, device), dev(c["symbols"], device), dev(want_ranges, device), 0,
+                              dev(c["boundary"], device), reduction="none")
+    np.testing.assert_allclose(got.cpu().numpy(), want, rtol=1e-4, atol=1e-5)
+
+
+def test_config5_rnnt_loss_full_size(device):
+    """BASELINE config 5: B=8, T=300, S=75, V=500, joiner logits [8,300,76,500]."""
+    import k2_amd as k2
+    B, T, S, C = 8, 300, 75, 500
+    c = cases.rnnt_case(5, B, T, S, C, t_lo=200, s_lo=40)
+    logits = np.random.default_rng(55).standard_normal((B, T, S + 1, C)).astype(np.float32)
+    want = orn.rnnt_loss(logits, c["symbols"], 0, c["boundary"], reduction="none")
+    got = k2.rnnt_loss(dev(logits, device), dev(c["symbols"], device), 0, dev(c["boundary"], device),
+                       reduction="none")
+    np.testing.assert_allclose(got.cpu().numpy(), want, rtol=1e-4, atol=1e-5)
