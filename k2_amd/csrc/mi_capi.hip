@@ -1,4 +1,7 @@
 // extern "C" entry points of the MI recursion: argument checks and kernel selection.
+#include <cstdlib>
+#include <cstring>
+
 #include "common.h"
 #include "mi_internal.h"
 
@@ -10,6 +13,12 @@ bool ShapeOk(int B, int S, int T) {
   if (B < 0 || S < 0 || T < 0) return false;
   // kernels index one sequence's lattice with 32-bit offsets
   return ((int64_t)S + 1) * ((int64_t)T + 1) < (int64_t)1 << 31;
+}
+
+// K2AMD_MI_PATH=generic forces the exact log-domain kernels (used by the tests to cover both).
+bool ForceGeneric() {
+  const char *e = std::getenv("K2AMD_MI_PATH");
+  return e != nullptr && std::strcmp(e, "generic") == 0;
 }
 
 }  // namespace
@@ -30,19 +39,26 @@ const char *k2amd_status_string(int status) {
 }
 
 size_t k2amd_mi_workspace_bytes(int B, int S, int T, int modified, int dtype) {
-  (void)B; (void)S; (void)T; (void)modified; (void)dtype;
-  return 0;
+  (void)modified;
+  if (dtype != K2AMD_F32 || !ShapeOk(B, S, T) || B == 0) return 0;
+  return MiFastWorkspaceBytes(B, S, T);
 }
 
 int k2amd_mi_forward(const void *px, const void *py, const int64_t *boundary, void *p, void *ans,
                      int B, int S, int T, int modified, int dtype, void *workspace,
                      size_t workspace_bytes, void *stream) {
-  (void)workspace; (void)workspace_bytes;
   if (!ShapeOk(B, S, T) || (dtype != K2AMD_F32 && dtype != K2AMD_F64)) return K2AMD_ERR_INVALID_ARGUMENT;
   if (B == 0) return K2AMD_OK;
   if (!p || !ans || (!px && S > 0) || (!py && T > 0)) return K2AMD_ERR_INVALID_ARGUMENT;
   hipStream_t st = static_cast<hipStream_t>(stream);
   modified = modified ? 1 : 0;
+  // fp32 with a workspace takes the pipelined throughput path; without one (or for fp64) the
+  // exact one-workgroup-per-sequence kernels run.
+  if (dtype == K2AMD_F32 && workspace != nullptr && !ForceGeneric()) {
+    if (workspace_bytes < MiFastWorkspaceBytes(B, S, T)) return K2AMD_ERR_WORKSPACE;
+    return MiForwardFast((const float *)px, (const float *)py, boundary, (float *)p, (float *)ans,
+                         B, S, T, modified, workspace, workspace_bytes, st);
+  }
   if (dtype == K2AMD_F32)
     return MiForwardGeneric<float>((const float *)px, (const float *)py, boundary, (float *)p,
                                    (float *)ans, B, S, T, modified, st);

@@ -18,6 +18,12 @@ int MiBackwardGeneric(const T *px, const T *p, const int64_t *boundary, T *ans_g
                       hipStream_t stream);
 size_t MiGenericMaxRows(int dtype);
 
+// fp32 throughput path: pipelined 63-row chunks, one chain wavefront per workgroup (mi_fast.hip).
+size_t MiFastWorkspaceBytes(int B, int S, int Tn);
+int MiForwardFast(const float *px, const float *py, const int64_t *boundary, float *p, float *ans,
+                  int B, int S, int Tn, int modified, void *workspace, size_t workspace_bytes,
+                  hipStream_t stream);
+
 }  // namespace k2amd
 
 #endif  // K2_AMD_CSRC_MI_INTERNAL_H_

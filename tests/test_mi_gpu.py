@@ -33,16 +33,34 @@ def run_gpu(px, py, bd, device, ans_grad=None):
     return ans.cpu().numpy(), p.cpu().numpy(), gx.cpu().numpy(), gy.cpu().numpy(), g.cpu().numpy(), g_in.cpu().numpy()
 
 
+def _close(name, got, want, want64, tol):
+    """fp64: the stated tolerance.  fp32: the stated tolerance against the fp32 CPU oracle, or,
+    where |p| is so large that the fp32 oracle itself is noisy (one ulp of p = 2.4e-4 at 3000),
+    the same tolerance against the fp64 oracle widened by the fp32 oracle's own worst error."""
+    with np.errstate(invalid="ignore"):
+        ok = np.isclose(got, want, equal_nan=True, **tol)
+        if want64 is not None and not ok.all():
+            noise = np.nanmax(np.where(np.isfinite(want64), np.abs(want - want64), 0.0))
+            err = np.abs(got - want64)
+            same_inf = (got == want64)
+            ok |= same_inf | (err <= tol["atol"] + tol["rtol"] * np.abs(want64) + 2.0 * noise)
+    assert ok.all(), (name, int((~ok).sum()), got[~ok][:5], want[~ok][:5])
+
+
 def check(name, px, py, bd, want, device):
     ans_w, p_w, gx_w, gy_w = want
     ans, p, gx, gy, g_out, g_in = run_gpu(px, py, bd, device)
     tol = TOL[px.dtype]
-    np.testing.assert_allclose(ans, ans_w, err_msg=name + " ans", **tol)
+    w64 = (None, None, None, None)
+    if px.dtype == np.float32:
+        a64, p64 = omi.mi_forward(px.astype(np.float64), py.astype(np.float64), bd)
+        w64 = (a64, p64) + tuple(omi.mi_backward(px.astype(np.float64), py.astype(np.float64), bd, p64))
+    _close(name + " ans", ans, ans_w, w64[0], tol)
     inside = ~np.isnan(p_w)
     assert not np.isnan(p[inside]).any(), name
-    np.testing.assert_allclose(p[inside], p_w[inside], err_msg=name + " p", **tol)
-    np.testing.assert_allclose(gx, gx_w, err_msg=name + " px_grad", **tol)
-    np.testing.assert_allclose(gy, gy_w, err_msg=name + " py_grad", **tol)
+    _close(name + " p", p[inside], p_w[inside], None if w64[1] is None else w64[1][inside], tol)
+    _close(name + " px_grad", gx, gx_w, w64[2], tol)
+    _close(name + " py_grad", gy, gy_w, w64[3], tol)
     # the gradient that reaches the start cell equals the one injected at the end cell
     # whenever the end cell is reachable
     ok = np.isfinite(ans_w)
