@@ -70,13 +70,19 @@ int k2amd_mi_backward(const void *px, const void *py, const int64_t *boundary, c
                       void *ans_grad, void *px_grad, void *py_grad, int B, int S, int T,
                       int modified, int dtype, int overwrite_ans_grad, void *workspace,
                       size_t workspace_bytes, void *stream) {
-  (void)workspace; (void)workspace_bytes; (void)py;
+  (void)py;
   if (!ShapeOk(B, S, T) || (dtype != K2AMD_F32 && dtype != K2AMD_F64)) return K2AMD_ERR_INVALID_ARGUMENT;
   if (B == 0) return K2AMD_OK;
   if (!p || !ans_grad || (!px && S > 0) || (!px_grad && S > 0) || (!py_grad && T > 0))
     return K2AMD_ERR_INVALID_ARGUMENT;
   hipStream_t st = static_cast<hipStream_t>(stream);
   modified = modified ? 1 : 0;
+  if (dtype == K2AMD_F32 && workspace != nullptr && !ForceGeneric()) {
+    if (workspace_bytes < MiFastWorkspaceBytes(B, S, T)) return K2AMD_ERR_WORKSPACE;
+    return MiBackwardFast((const float *)px, (const float *)p, boundary, (float *)ans_grad,
+                          (float *)px_grad, (float *)py_grad, B, S, T, modified,
+                          overwrite_ans_grad, workspace, workspace_bytes, st);
+  }
   if (dtype == K2AMD_F32)
     return MiBackwardGeneric<float>((const float *)px, (const float *)p, boundary,
                                     (float *)ans_grad, (float *)px_grad, (float *)py_grad, B, S, T,

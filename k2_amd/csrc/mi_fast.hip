@@ -330,6 +330,284 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
   if (!is_chain) store_block(g.nblocks - 1);
 }
 
+
+// ------------------------------------------------------------------------------ backward
+//
+// Mass-flow form of the reference's backward sweep (k2/python/csrc/torch/
+// mutual_information_cpu.cu:179-251).  For a destination cell D = (s, t) that holds gradient g:
+//     d1 = exp(p[s-1][t+o] + px[s-1][t+o] - p[s][t])        (o = -1 modified, 0 regular)
+//     h  = d1 * g        -> px_grad[s-1][t+o], and flows to cell (s-1, t+o)
+//     c  = (1 - d1) * g  -> py_grad[s][t-1],   and flows to cell (s, t-1)
+// so every cell needs ONE exponential, computed by the helper wavefronts (E = d1, OME = 1 - d1,
+// with the reference's guards folded in: first row E = 0, first column of a regular lattice
+// E = 1, non-finite d1 -> both 0).  The chain wavefront then does, per position m (descending),
+//     h = E * G;  c = OME * G;  G = h(lane + 1) + c
+// i.e. two multiplies and one DPP add.  Lane l handles lattice row row0 + l; lane 63 replays the
+// h values of the first row of the chunk below, so here the LOWER chunk runs ahead.
+struct BwdLds {
+  float e[kWave][kStride];    // d1 on the way in, h (px_grad) on the way out
+  float ome[kWave][kStride];  // 1 - d1 on the way in, c (py_grad) on the way out
+  float rin[kRing];
+  unsigned ticket;
+};
+
+__global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
+    const float *__restrict__ px, const float *__restrict__ p,
+    const int64_t *__restrict__ boundary, float *__restrict__ ans_grad,
+    float *__restrict__ px_grad, float *__restrict__ py_grad, FastHeader *hdr, float *edge, int S,
+    int Tn, int modified, int nchunks, int edge_stride, int overwrite_ans_grad) {
+  __shared__ BwdLds lds;
+  if (threadIdx.x == 0) lds.ticket = atomicAdd(&hdr->ticket, 1u);
+  __syncthreads();
+  ChunkGeom g;
+  g.b = lds.ticket / nchunks;
+  g.c = nchunks - 1 - (int)(lds.ticket % nchunks);  // lower chunks take earlier tickets
+  const Box box = LoadBox(boundary, g.b, S, Tn);
+  const int T1 = modified ? Tn : Tn + 1;
+  const int off = modified ? -1 : 0;
+  const float *pxb = px + (size_t)g.b * S * T1;
+  const float *pb = p + (size_t)g.b * (S + 1) * (Tn + 1);
+  float *gxb = px_grad + (size_t)g.b * S * T1;
+  float *gyb = py_grad + (size_t)g.b * (S + 1) * Tn;
+
+  // Zero everything the sweep does not assign, for the rows this workgroup is responsible for
+  // BY ARRAY ROW (independent of the box), so every element of both outputs is written once.
+  {
+    const int r_lo = g.c * kRows, r_hi = min(r_lo + kRows, S + 1);
+    const int xs0 = box.ok ? box.s0 : 0, xs1 = box.ok ? box.s1 : 0;
+    const int xt0 = box.ok ? box.t0 : 0, xt1 = box.ok ? box.t1 + off + 1 : 0;
+    const int ys1 = box.ok ? box.s1 + 1 : 0, yt1 = box.ok ? box.t1 : 0;
+    for (int r = r_lo; r < r_hi; ++r) {
+      if (r < S) {
+        const bool row_in = r >= xs0 && r < xs1;
+        for (int t = threadIdx.x; t < T1; t += kFastThreads)
+          if (!(row_in && t >= xt0 && t < xt1)) gxb[(size_t)r * T1 + t] = 0.0f;
+      }
+      const bool row_in = r >= xs0 && r < ys1;
+      for (int t = threadIdx.x; t < Tn; t += kFastThreads)
+        if (!(row_in && t >= xt0 && t < yt1)) gyb[(size_t)r * Tn + t] = 0.0f;
+    }
+  }
+  if (!box.ok) return;
+  g.s0 = box.s0; g.t0 = box.t0; g.ns = box.s1 - box.s0; g.nt = box.t1 - box.t0;
+  g.row0 = g.c * kRows;
+  if (g.row0 > g.ns) return;
+  g.nrows = min(kRows, g.ns - g.row0 + 1);
+  g.skew = modified ? 0 : 1;
+  const bool has_down = g.row0 + kRows <= g.ns;
+  const bool has_up = g.c > 0;
+  const int npos = g.nt + 2 + (kRows - 1) * g.skew;
+  g.nblocks = (npos + kW - 1) / kW;
+  float *edge_out = edge + ((size_t)g.b * nchunks + g.c) * edge_stride;            // read by c-1
+  const float *edge_in = edge + ((size_t)g.b * nchunks + g.c + 1) * edge_stride;   // from c+1
+
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const bool is_chain = wave == 0;
+  const int hid = threadIdx.x - kWave;
+
+  // lane 63 is the replay lane: its E / OME rows are never used (h is overwritten, c is unused)
+  for (int i = threadIdx.x; i < kRing; i += kFastThreads) {
+    lds.e[kWave - 1][i] = 0.0f;
+    lds.ome[kWave - 1][i] = 0.0f;
+  }
+
+  constexpr int kItems = kRows * (kW / 4);
+  constexpr int kItemsPerLane = (kItems + kHelperLanes - 1) / kHelperLanes;
+  float4 re[kItemsPerLane], ro[kItemsPerLane];
+
+  // E / OME of the four destination cells (row q, positions kb*32 + 4m .. +3)
+  auto load_block = [&](int kb) {
+#pragma unroll
+    for (int it = 0; it < kItemsPerLane; ++it) {
+      const int item = hid + it * kHelperLanes;
+      float ve[4] = {0.f, 0.f, 0.f, 0.f}, vo[4] = {0.f, 0.f, 0.f, 0.f};
+      if (item < kItems && kb >= 0) {
+        const int q = item >> 3, m = item & 7;
+        const int i = g.row0 + q;
+        const int jd = kb * kW + 4 * m - q * g.skew;  // destination column of element 0
+        if (i <= g.ns) {
+          const int s = g.s0 + i;
+          if (i == 0) {
+            // first row: everything flows along py; beyond the end cell nothing flows, except
+            // that the last row carries the seed towards the end cell (see below)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (jd + e >= 1 && jd + e <= g.nt) vo[e] = 1.0f;
+          } else {
+            const int js = jd - 1 + g.skew;  // source column of the px edge of element 0
+            const float *pd = pb + (size_t)s * (Tn + 1) + g.t0 + jd;
+            const float *ps = pb + (size_t)(s - 1) * (Tn + 1) + g.t0 + js;
+            const float *xs = pxb + (size_t)(s - 1) * T1 + g.t0 + js;
+            float vd[4], vs[4], vx[4];
+            if (jd >= 1 && jd + 3 <= g.nt) {
+              const Quad a = *reinterpret_cast<const Quad *>(pd);
+              const Quad bq = *reinterpret_cast<const Quad *>(ps);
+              const Quad cq = *reinterpret_cast<const Quad *>(xs);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) { vd[e] = a.v[e]; vs[e] = bq.v[e]; vx[e] = cq.v[e]; }
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                const bool in = jd + e >= 1 && jd + e <= g.nt;
+                vd[e] = in ? pd[e] : 0.0f;
+                vs[e] = in ? ps[e] : 0.0f;
+                vx[e] = in ? xs[e] : 0.0f;
+              }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int j = jd + e;
+              if (j >= 1 && j <= g.nt) {
+                float total = vd[e];
+                if (total - total != 0.0f) total = 0.0f;
+                const float d1 = __expf((vs[e] + vx[e]) - total);
+                if (d1 - d1 == 0.0f) { ve[e] = d1; vo[e] = 1.0f - d1; }
+              } else if (j == 0 && !modified) {
+                ve[e] = 1.0f;  // first column of a regular lattice: all of it flows up
+              }
+            }
+          }
+          if (i == g.ns) {
+            // virtual cells right of the end cell hand the seed leftwards unchanged
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (jd + e > g.nt) { ve[e] = 0.0f; vo[e] = 1.0f; }
+          }
+        }
+      }
+      re[it] = make_float4(ve[0], ve[1], ve[2], ve[3]);
+      ro[it] = make_float4(vo[0], vo[1], vo[2], vo[3]);
+    }
+  };
+
+  auto commit_block = [&](int kb) {
+    if (kb < 0) return;
+#pragma unroll
+    for (int it = 0; it < kItemsPerLane; ++it) {
+      const int item = hid + it * kHelperLanes;
+      if (item < kItems) {
+        const int q = item >> 3, m = item & 7;
+        const int pos = (kb % 3) * kW + 4 * m;
+        *reinterpret_cast<float4 *>(&lds.e[q][pos]) = re[it];
+        *reinterpret_cast<float4 *>(&lds.ome[q][pos]) = ro[it];
+      }
+    }
+  };
+
+  auto store_block = [&](int kb) {
+#pragma unroll
+    for (int it = 0; it < kItemsPerLane; ++it) {
+      const int item = hid + it * kHelperLanes;
+      if (item < kItems) {
+        const int q = item >> 3, m = item & 7;
+        const int i = g.row0 + q;
+        if (i <= g.ns) {
+          const int pos = (kb % 3) * kW + 4 * m;
+          const float4 h4 = *reinterpret_cast<const float4 *>(&lds.e[q][pos]);
+          const float4 c4 = *reinterpret_cast<const float4 *>(&lds.ome[q][pos]);
+          const float hv[4] = {h4.x, h4.y, h4.z, h4.w}, cv[4] = {c4.x, c4.y, c4.z, c4.w};
+          const int jd = kb * kW + 4 * m - q * g.skew;
+          const int s = g.s0 + i;
+          // py_grad[s][t0 + jd - 1 + e]   for destination columns 1..nt
+          float *dy = gyb + (size_t)s * Tn + g.t0 + jd - 1;
+          if (jd >= 1 && jd + 3 <= g.nt) {
+            Quad o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o.v[e] = cv[e];
+            *reinterpret_cast<Quad *>(dy) = o;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (jd + e >= 1 && jd + e <= g.nt) dy[e] = cv[e];
+          }
+          // px_grad[s-1][t0 + jd - 1 + skew + e]   for destination columns (1 - skew)..nt
+          if (i >= 1) {
+            float *dx = gxb + (size_t)(s - 1) * T1 + g.t0 + jd - 1 + g.skew;
+            const int lo = 1 - g.skew;
+            if (jd >= lo && jd + 3 <= g.nt) {
+              Quad o;
+#pragma unroll
+              for (int e = 0; e < 4; ++e) o.v[e] = hv[e];
+              *reinterpret_cast<Quad *>(dx) = o;
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                if (jd + e >= lo && jd + e <= g.nt) dx[e] = hv[e];
+            }
+          }
+        }
+      }
+    }
+  };
+
+  auto load_rin = [&](int kb) {
+    if (hid >= 0 && hid < kW && kb >= 0) {
+      const int mpos = kb * kW + hid;
+      float v = 0.0f;
+      if (has_down) {
+        const int idx = mpos - kRows * g.skew;
+        if (idx >= 0 && idx < g.nblocks * kW) v = PollEdge(edge_in + idx, hdr);
+      }
+      lds.rin[(kb % 3) * kW + hid] = v;
+    }
+  };
+
+  const int top = g.nblocks - 1;
+  if (!is_chain) {
+    load_block(top);
+    commit_block(top);
+    load_rin(top);
+    load_block(top - 1);
+  }
+  // gradient at the (virtual) right end of each row: the seed on the sequence's last row
+  float G = 0.0f;
+  if (is_chain && g.row0 + lane == g.ns && lane < kRows) G = ans_grad[g.b];
+  float g_origin = 0.0f;
+  __syncthreads();
+
+  for (int kb = top; kb >= 0; --kb) {
+    if (!is_chain) {
+      commit_block(kb - 1);
+      load_rin(kb - 1);
+      load_block(kb - 2);
+      if (kb < top) store_block(kb + 1);
+    } else {
+      const int base = (kb % 3) * kW;
+#pragma unroll 2
+      for (int m = kW / 4 - 1; m >= 0; --m) {
+        const int pos = base + 4 * m;
+        const float4 e4 = *reinterpret_cast<const float4 *>(&lds.e[lane][pos]);
+        const float4 o4 = *reinterpret_cast<const float4 *>(&lds.ome[lane][pos]);
+        const float4 r4 = *reinterpret_cast<const float4 *>(&lds.rin[pos]);
+        const float es[4] = {e4.x, e4.y, e4.z, e4.w};
+        const float os[4] = {o4.x, o4.y, o4.z, o4.w};
+        const float rs[4] = {r4.x, r4.y, r4.z, r4.w};
+        float hs[4], cs[4];
+#pragma unroll
+        for (int e = 3; e >= 0; --e) {
+          if (kb == 0 && m == 0 && e == 0) g_origin = G;
+          float h = es[e] * G;
+          const float c = os[e] * G;
+          if (lane == kWave - 1) h = rs[e];
+          G = WaveShl1(0.0f, h) + c;
+          hs[e] = h;
+          cs[e] = c;
+        }
+        *reinterpret_cast<float4 *>(&lds.e[lane][pos]) = make_float4(hs[0], hs[1], hs[2], hs[3]);
+        *reinterpret_cast<float4 *>(&lds.ome[lane][pos]) = make_float4(cs[0], cs[1], cs[2], cs[3]);
+        if (has_up && lane == 0) {
+          const int mpos = kb * kW + 4 * m;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) PublishEdge(edge_out + mpos + e, hs[e]);
+        }
+      }
+    }
+    __syncthreads();
+  }
+  if (!is_chain) store_block(0);
+  if (overwrite_ans_grad && is_chain && g.c == 0 && lane == 0) ans_grad[g.b] = g_origin;
+}
+
 }  // namespace
 
 size_t MiFastWorkspaceBytes(int B, int S, int Tn) {
@@ -351,6 +629,25 @@ int MiForwardFast(const float *px, const float *py, const int64_t *boundary, flo
                      stream, hdr, reinterpret_cast<unsigned *>(edge), n_edge);
   hipLaunchKernelGGL(MiForwardFastKernel, dim3((unsigned)(B * nchunks)), dim3(kFastThreads), 0, stream,
                      px, py, boundary, p, ans, hdr, edge, S, Tn, modified, nchunks, edge_stride);
+  return LaunchStatus();
+}
+
+
+int MiBackwardFast(const float *px, const float *p, const int64_t *boundary, float *ans_grad,
+                   float *px_grad, float *py_grad, int B, int S, int Tn, int modified,
+                   int overwrite_ans_grad, void *workspace, size_t workspace_bytes,
+                   hipStream_t stream) {
+  if (workspace == nullptr || workspace_bytes < MiFastWorkspaceBytes(B, S, Tn)) return K2AMD_ERR_WORKSPACE;
+  const int nchunks = (S + 1 + kRows - 1) / kRows;
+  const int edge_stride = (int)(((size_t)Tn + 2 + kRows + kW + 3) / 4 * 4 + kW);
+  FastHeader *hdr = static_cast<FastHeader *>(workspace);
+  float *edge = reinterpret_cast<float *>(hdr + 1);
+  const size_t n_edge = (size_t)B * (nchunks + 1) * edge_stride;
+  hipLaunchKernelGGL(FastWsInitKernel, dim3((unsigned)min((size_t)256, (n_edge + 255) / 256)), dim3(256), 0,
+                     stream, hdr, reinterpret_cast<unsigned *>(edge), n_edge);
+  hipLaunchKernelGGL(MiBackwardFastKernel, dim3((unsigned)(B * nchunks)), dim3(kFastThreads), 0, stream,
+                     px, p, boundary, ans_grad, px_grad, py_grad, hdr, edge, S, Tn, modified, nchunks,
+                     edge_stride, overwrite_ans_grad);
   return LaunchStatus();
 }
 

@@ -23,6 +23,10 @@ size_t MiFastWorkspaceBytes(int B, int S, int Tn);
 int MiForwardFast(const float *px, const float *py, const int64_t *boundary, float *p, float *ans,
                   int B, int S, int Tn, int modified, void *workspace, size_t workspace_bytes,
                   hipStream_t stream);
+int MiBackwardFast(const float *px, const float *p, const int64_t *boundary, float *ans_grad,
+                   float *px_grad, float *py_grad, int B, int S, int Tn, int modified,
+                   int overwrite_ans_grad, void *workspace, size_t workspace_bytes,
+                   hipStream_t stream);
 
 }  // namespace k2amd
 
