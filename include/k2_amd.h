@@ -26,7 +26,8 @@ enum k2amd_status {
   K2AMD_ERR_INVALID_ARGUMENT = 1, /* bad shape / null pointer / unknown enum */
   K2AMD_ERR_UNSUPPORTED = 2,      /* valid request this build cannot serve (size limit) */
   K2AMD_ERR_WORKSPACE = 3,        /* workspace missing or too small */
-  K2AMD_ERR_LAUNCH = 4            /* HIP reported a launch error */
+  K2AMD_ERR_LAUNCH = 4,           /* HIP reported a launch error */
+  K2AMD_ERR_TIMEOUT = 5           /* a bounded in-kernel wait expired; re-initialise the workspace */
 };
 
 enum k2amd_dtype { K2AMD_F32 = 0, K2AMD_F64 = 1 };
@@ -46,10 +47,18 @@ K2AMD_API const char *k2amd_status_string(int status);
  *   boundary [B][4] int64 = (s_begin, t_begin, s_end, t_end) or NULL for (0,0,S,T)
  *   ans, ans_grad [B]
  *
- * Workspace: k2amd_mi_workspace_bytes() tells how many bytes of device scratch the
- * forward/backward kernels want for the given shape (may be 0).  The caller owns it.
+ * Workspace (fp32 throughput path): k2amd_mi_workspace_bytes() tells how many bytes of device
+ * scratch the pipelined kernels want for a shape (0 for fp64).  The caller owns the buffer and
+ * must run k2amd_mi_workspace_init() on it ONCE before its first use (and again after a
+ * K2AMD_ERR_TIMEOUT); the kernels leave it ready for the next call, so a buffer sized for the
+ * largest shape can be reused for any smaller one.  One workspace serves one stream at a time.
+ * Passing workspace == NULL selects the exact one-workgroup-per-sequence kernels instead.
  */
 K2AMD_API size_t k2amd_mi_workspace_bytes(int B, int S, int T, int modified, int dtype);
+K2AMD_API int k2amd_mi_workspace_init(void *workspace, size_t workspace_bytes, void *stream);
+/* Synchronises `stream` and returns K2AMD_ERR_TIMEOUT if a pipelined kernel that used this
+ * workspace gave up waiting for a neighbouring workgroup (its results are then invalid). */
+K2AMD_API int k2amd_mi_workspace_status(const void *workspace, void *stream);
 
 /* Replaces _k2.mutual_information_forward (k2/python/csrc/torch/mutual_information.cu:26-44,
  * CPU semantics of k2/python/csrc/torch/mutual_information_cpu.cu:50-124):

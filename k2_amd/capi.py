@@ -25,6 +25,8 @@ _SIGNATURES = {
     "k2amd_version": ([], _ci),
     "k2amd_status_string": ([_ci], ctypes.c_char_p),
     "k2amd_mi_workspace_bytes": ([_ci, _ci, _ci, _ci, _ci], _sz),
+    "k2amd_mi_workspace_init": ([_vp, _sz, _vp], _ci),
+    "k2amd_mi_workspace_status": ([_vp, _vp], _ci),
     "k2amd_mi_forward": ([_vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp, _sz, _vp], _ci),
     "k2amd_mi_backward": ([_vp, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci,
                            _vp, _sz, _vp], _ci),
@@ -84,9 +86,49 @@ def stream_ptr(device):
     return torch.cuda.current_stream(device).cuda_stream
 
 
+_workspaces = {}
+
+
 def mi_workspace(B, S, T, modified, dtype, device):
+    """The scratch buffer of the pipelined fp32 kernels: one per (device, stream), grown on
+    demand and initialised once (the kernels leave it ready for the next call)."""
     n = lib().k2amd_mi_workspace_bytes(B, S, T, int(modified), dtype)
-    return torch.empty(n, dtype=torch.uint8, device=device) if n else None
+    if not n:
+        return None
+    stream = torch.cuda.current_stream(device)
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream.cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < n:
+        ws = torch.empty(max(n, 1 << 20), dtype=torch.uint8, device=device)
+        with torch.cuda.device(device):
+            check(lib().k2amd_mi_workspace_init(ws.data_ptr(), ws.numel(), stream.cuda_stream))
+        _workspaces[key] = ws
+    return ws
+
+
+def mi_workspace_is_clean(device):
+    """True when every edge word of the cached workspace holds the sentinel again and the ticket
+    counters are back to zero, i.e. the last kernel left the buffer ready for the next call."""
+    stream = torch.cuda.current_stream(device)
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream.cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None:
+        return True
+    torch.cuda.synchronize(device)
+    words = ws[: ws.numel() // 4 * 4].view(torch.int32)
+    header_ok = bool((words[:3] == 0).all())
+    sentinel = 0x7FC5A5A5
+    return header_ok and bool((words[64:] == sentinel).all())
+
+
+def mi_workspace_status(device):
+    """Synchronises and raises if a pipelined kernel on this device's current stream timed out."""
+    stream = torch.cuda.current_stream(device)
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream.cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is not None:
+        with torch.cuda.device(device):
+            check(lib().k2amd_mi_workspace_status(ws.data_ptr(), stream.cuda_stream))
 
 
 def mi_forward(px, py, boundary, p):

@@ -34,6 +34,7 @@ const char *k2amd_status_string(int status) {
     case K2AMD_ERR_UNSUPPORTED: return "unsupported size for this build";
     case K2AMD_ERR_WORKSPACE: return "workspace missing or too small";
     case K2AMD_ERR_LAUNCH: return "HIP launch error";
+    case K2AMD_ERR_TIMEOUT: return "in-kernel wait timed out; workspace must be re-initialised";
     default: return "unknown status";
   }
 }
@@ -42,6 +43,20 @@ size_t k2amd_mi_workspace_bytes(int B, int S, int T, int modified, int dtype) {
   (void)modified;
   if (dtype != K2AMD_F32 || !ShapeOk(B, S, T) || B == 0) return 0;
   return MiFastWorkspaceBytes(B, S, T);
+}
+
+int k2amd_mi_workspace_init(void *workspace, size_t workspace_bytes, void *stream) {
+  return MiFastWorkspaceInit(workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+int k2amd_mi_workspace_status(const void *workspace, void *stream) {
+  if (workspace == nullptr) return K2AMD_ERR_INVALID_ARGUMENT;
+  unsigned header[4] = {0, 0, 0, 0};
+  if (hipMemcpyAsync(header, workspace, sizeof(header), hipMemcpyDeviceToHost,
+                     static_cast<hipStream_t>(stream)) != hipSuccess ||
+      hipStreamSynchronize(static_cast<hipStream_t>(stream)) != hipSuccess)
+    return K2AMD_ERR_LAUNCH;
+  return header[2] != 0 ? K2AMD_ERR_TIMEOUT : K2AMD_OK;  // FastHeader::error
 }
 
 int k2amd_mi_forward(const void *px, const void *py, const int64_t *boundary, void *p, void *ans,

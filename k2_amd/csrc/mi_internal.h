@@ -20,6 +20,7 @@ size_t MiGenericMaxRows(int dtype);
 
 // fp32 throughput path: pipelined 63-row chunks, one chain wavefront per workgroup (mi_fast.hip).
 size_t MiFastWorkspaceBytes(int B, int S, int Tn);
+int MiFastWorkspaceInit(void *workspace, size_t workspace_bytes, hipStream_t stream);
 int MiForwardFast(const float *px, const float *py, const int64_t *boundary, float *p, float *ans,
                   int B, int S, int Tn, int modified, void *workspace, size_t workspace_bytes,
                   hipStream_t stream);

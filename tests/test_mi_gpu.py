@@ -30,6 +30,10 @@ def run_gpu(px, py, bd, device, ans_grad=None):
     g_in = g.clone()
     gx, gy = capi.mi_backward(tpx, tpy, tbd, p, g, overwrite_ans_grad=True)
     torch.cuda.synchronize()
+    # the pipelined kernels hand data between workgroups through a scratch buffer that every
+    # call must leave exactly as it found it, and no in-kernel wait may have timed out
+    assert capi.mi_workspace_is_clean(device), "workspace left dirty"
+    capi.mi_workspace_status(device)
     return ans.cpu().numpy(), p.cpu().numpy(), gx.cpu().numpy(), gy.cpu().numpy(), g.cpu().numpy(), g_in.cpu().numpy()
 
 
@@ -96,6 +100,37 @@ def test_wide_lattice_more_rows_than_a_wavefront(device, modified):
     ans, p = omi.mi_forward(px, py, bd)
     gx, gy = omi.mi_backward(px, py, bd, p)
     check("wide", px, py, bd, (ans, p, gx, gy), device)
+
+
+@pytest.mark.parametrize("modified", [False, True])
+def test_fp32_multi_chunk_and_block_edges(device, modified):
+    """fp32 lattices taller than one 64-row chunk, with T chosen around multiples of the 32-step
+    block so that chunk hand-over and the first/last block paths are all exercised."""
+    rng = np.random.default_rng(17)
+    for (B, S, T) in ((2, 70, 95), (3, 130, 160), (2, 200, 127), (1, 64, 128), (2, 63, 129), (1, 129, 191)):
+        px = rng.normal(-2, 1, (B, S, T if modified else T + 1)).astype(np.float32)
+        py = rng.normal(-2, 1, (B, S + 1, T)).astype(np.float32)
+        for with_bd in (False, True):
+            bd = None
+            if with_bd:
+                rows = []
+                for _ in range(B):
+                    s_len = int(rng.integers(S // 2, S + 1)); t_len = int(rng.integers(max(s_len, T // 2), T + 1)) if T >= s_len else T
+                    s_len = min(s_len, t_len) if modified else s_len
+                    s0 = int(rng.integers(0, S - s_len + 1)); t0 = int(rng.integers(0, T - t_len + 1))
+                    rows.append([s0, t0, s0 + s_len, t0 + t_len])
+                bd = np.array(rows, dtype=np.int64)
+            ans, p = omi.mi_forward(px, py, bd)
+            gx, gy = omi.mi_backward(px, py, bd, p)
+            check(f"S{S}T{T}bd{with_bd}", px, py, bd, (ans, p, gx, gy), device)
+    # every T_b around a block boundary, boundaries given
+    B, S, T = 8, 70, 200
+    px = rng.normal(-2, 1, (B, S, T if modified else T + 1)).astype(np.float32)
+    py = rng.normal(-2, 1, (B, S + 1, T)).astype(np.float32)
+    bd = np.array([[0, 0, 66 + b % 4, 92 + b] for b in range(B)], dtype=np.int64)
+    ans, p = omi.mi_forward(px, py, bd)
+    gx, gy = omi.mi_backward(px, py, bd, p)
+    check("block-edge sweep", px, py, bd, (ans, p, gx, gy), device)
 
 
 def test_scaled_ans_grad(device):
