@@ -69,7 +69,7 @@ int k2amd_mi_forward(const void *px, const void *py, const int64_t *boundary, vo
   modified = modified ? 1 : 0;
   // fp32 with a workspace takes the pipelined throughput path; without one (or for fp64) the
   // exact one-workgroup-per-sequence kernels run.
-  if (dtype == K2AMD_F32 && workspace != nullptr && !ForceGeneric()) {
+  if (dtype == K2AMD_F32 && workspace != nullptr && !ForceGeneric() && MiFastSupports(B, S, T, modified)) {
     if (workspace_bytes < MiFastWorkspaceBytes(B, S, T)) return K2AMD_ERR_WORKSPACE;
     return MiForwardFast((const float *)px, (const float *)py, boundary, (float *)p, (float *)ans,
                          B, S, T, modified, workspace, workspace_bytes, st);
@@ -92,7 +92,7 @@ int k2amd_mi_backward(const void *px, const void *py, const int64_t *boundary, c
     return K2AMD_ERR_INVALID_ARGUMENT;
   hipStream_t st = static_cast<hipStream_t>(stream);
   modified = modified ? 1 : 0;
-  if (dtype == K2AMD_F32 && workspace != nullptr && !ForceGeneric()) {
+  if (dtype == K2AMD_F32 && workspace != nullptr && !ForceGeneric() && MiFastSupports(B, S, T, modified)) {
     if (workspace_bytes < MiFastWorkspaceBytes(B, S, T)) return K2AMD_ERR_WORKSPACE;
     return MiBackwardFast((const float *)px, (const float *)p, boundary, (float *)ans_grad,
                           (float *)px_grad, (float *)py_grad, B, S, T, modified,

@@ -19,6 +19,7 @@ int MiBackwardGeneric(const T *px, const T *p, const int64_t *boundary, T *ans_g
 size_t MiGenericMaxRows(int dtype);
 
 // fp32 throughput path: pipelined 63-row chunks, one chain wavefront per workgroup (mi_fast.hip).
+bool MiFastSupports(int B, int S, int Tn, int modified);
 size_t MiFastWorkspaceBytes(int B, int S, int Tn);
 int MiFastWorkspaceInit(void *workspace, size_t workspace_bytes, hipStream_t stream);
 int MiForwardFast(const float *px, const float *py, const int64_t *boundary, float *p, float *ans,
