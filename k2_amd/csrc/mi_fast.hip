@@ -54,9 +54,14 @@ constexpr float kLn2 = 0.69314718055994530942f;
 constexpr int kQuadsPerRow = kStride / 4;
 constexpr int kQuadsPerBlock = kW / 4;
 // One work item = (row q in 0..63, quad m in 0..7) of a block: four consecutive steps of one
-// lattice row; 512 items per block, two per loader lane and two per storer lane (rows q and
-// q + 32, same quad).
-static_assert(kRows * kQuadsPerBlock == 2 * kMoverLanes, "two work items per mover lane");
+// lattice row; 512 items per block.  The four storer wavefronts take two items per lane (rows q
+// and q + 32).  The four loader wavefronts form TWO GROUPS of 128 lanes that alternate blocks
+// (group = block & 1), four items per lane (rows q, q+16, q+32, q+48): a group loads a block,
+// then issues no other memory operation until it commits that block two iterations later, so
+// the wait in front of the commit covers exactly those loads.
+static_assert(kRows * kQuadsPerBlock == 2 * kMoverLanes, "two work items per storer lane");
+constexpr int kGroupLanes = kMoverLanes / 2;
+constexpr int kLoadItems = kRows * kQuadsPerBlock / kGroupLanes;  // 4
 
 struct FastHeader {
   unsigned ticket;  // next chunk to hand out; reset by the last workgroup of a launch
@@ -104,36 +109,36 @@ __device__ __forceinline__ float ShiftAdd(float lane0, float P, float add) {
   return r;
 }
 
-__device__ __forceinline__ float4 LoadQuad(const float *ptr) {
-  const Quad v = *reinterpret_cast<const Quad *>(ptr);
-  return make_float4(v.v[0], v.v[1], v.v[2], v.v[3]);
-}
 __device__ __forceinline__ void StoreQuad(float *ptr, float4 v) {
   Quad o;
   o.v[0] = v.x; o.v[1] = v.y; o.v[2] = v.z; o.v[3] = v.w;
   *reinterpret_cast<Quad *>(ptr) = o;
 }
 
-// A row segment as the loaders see it: `row` points at local column `lo` of the row, valid
-// columns are lo..hi, and `last` is the last address from which four floats may be read without
-// leaving the tensor.
-struct Segment {
-  const float *row;
-  const float *last;
-  int lo, hi;
-};
+// Loads go through raw buffer resources (one per tensor): the hardware range-checks every dword
+// against the tensor's size and returns 0 beyond it, so no load can leave the tensor whatever
+// the boundary tensor holds, and no address clamping code sits in the loaders.
+typedef unsigned uint4v __attribute__((ext_vector_type(4)));
+typedef float float4v __attribute__((ext_vector_type(4)));
 
-// Four columns j0..j0+3 of one row, each clamped into the valid columns lo..hi and into the
-// tensor: element e belongs to column j0 + e whenever that column is valid, and is some other
-// in-bounds value otherwise (the caller masks it).  Static component indices only, so the
-// registers never have to live in scratch.
-__device__ __forceinline__ float4 LoadClamped(const Segment &sg, int j0) {
-  const float *end = sg.last + 3;  // last float of the tensor
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t MakeResource(const float *base, size_t elems) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(base), 0, (int)(elems * sizeof(float)),
+                                           0x00020000);
+}
+// four consecutive floats starting at float index `idx` (idx >= 0)
+__device__ __forceinline__ float4 BufferQuad(__amdgpu_buffer_rsrc_t rs, int idx) {
+  const float4v v = __builtin_bit_cast(float4v, __builtin_amdgcn_raw_buffer_load_b128(rs, idx * 4, 0, 0));
+  return make_float4(v.x, v.y, v.z, v.w);
+}
+// floats idx .. idx+3, each loaded on its own; elements whose flag is false read index 0 instead
+// (they are masked by the caller).  Used where a quad would straddle the valid columns.
+__device__ __forceinline__ float4 BufferFour(__amdgpu_buffer_rsrc_t rs, int idx, bool ok0, bool ok1,
+                                             bool ok2, bool ok3) {
   float4 r;
-  r.x = *min(sg.row + (min(max(j0 + 0, sg.lo), sg.hi) - sg.lo), end);
-  r.y = *min(sg.row + (min(max(j0 + 1, sg.lo), sg.hi) - sg.lo), end);
-  r.z = *min(sg.row + (min(max(j0 + 2, sg.lo), sg.hi) - sg.lo), end);
-  r.w = *min(sg.row + (min(max(j0 + 3, sg.lo), sg.hi) - sg.lo), end);
+  r.x = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, ok0 ? (idx + 0) * 4 : 0, 0, 0));
+  r.y = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, ok1 ? (idx + 1) * 4 : 0, 0, 0));
+  r.z = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, ok2 ? (idx + 2) * 4 : 0, 0, 0));
+  r.w = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, ok3 ? (idx + 3) * 4 : 0, 0, 0));
   return r;
 }
 
@@ -215,7 +220,7 @@ struct FwdLds {
 };
 
 struct FwdRegs {
-  float4 x[2], y[2];
+  float4 x[kLoadItems], y[kLoadItems];
 };
 
 __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
@@ -253,29 +258,29 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
 
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int role = RoleOf(wave);
-  // movers: lane id within the loader (or storer) group, and its two work items
+  // movers: lane id within the loader (or storer) wavefronts
   const int mid = (threadIdx.x - (role == kStorer ? kWave * (2 + kMoverWaves) : 2 * kWave)) &
                   (kMoverLanes - 1);
-  const int mq = mid >> 3, mm = mid & 7;  // rows mq and mq + 32, quad mm
+  const int mq = mid >> 3, mm = mid & 7;  // storers: rows mq and mq + 32, quad mm
+  const int grp = mid >> 7;               // loaders: group, and rows lq + 16*it, quad mm
+  const int lq = (mid & (kGroupLanes - 1)) >> 3;
 
   const int hi_x = g.nt - modified, hi_y = g.nt - 1;  // last valid px / py column
 
   // ---- loaders ---------------------------------------------------------------------------
-  Segment segx[2], segy[2];
-  bool rowx_ok[2], rowy_ok[2];
-  {
-    const float *x_last = px + (size_t)B * S * T1 - 4;
-    const float *y_last = py + (size_t)B * (S + 1) * Tn - 4;
+  const __amdgpu_buffer_rsrc_t rsx = MakeResource(px, (size_t)B * S * T1);
+  const __amdgpu_buffer_rsrc_t rsy = MakeResource(py, (size_t)B * (S + 1) * Tn);
+  int idx_x[kLoadItems], idx_y[kLoadItems];  // float index of local column 0 of the item's row
+  bool rowx_ok[kLoadItems], rowy_ok[kLoadItems];
 #pragma unroll
-    for (int it = 0; it < 2; ++it) {
-      const int row_i = g.row0 + mq + 32 * it;
-      rowx_ok[it] = row_i >= 1 && row_i <= g.ns;
-      rowy_ok[it] = row_i <= g.ns;
-      const int rx = min(max(row_i, 1), max(g.ns, 1)) - 1;  // a px row inside the box if any
-      const int ry = min(row_i, g.ns);
-      segx[it] = Segment{pxb + (size_t)(g.s0 + rx) * T1 + g.t0, x_last, 0, max(hi_x, 0)};
-      segy[it] = Segment{pyb + (size_t)(g.s0 + ry) * Tn + g.t0, y_last, 0, max(hi_y, 0)};
-    }
+  for (int it = 0; it < kLoadItems; ++it) {
+    const int row_i = g.row0 + lq + 16 * it;
+    rowx_ok[it] = row_i >= 1 && row_i <= g.ns;
+    rowy_ok[it] = row_i <= g.ns;
+    const int rx = min(max(row_i, 1), max(g.ns, 1)) - 1;  // a px row inside the box if any
+    const int ry = min(row_i, g.ns);
+    idx_x[it] = (g.b * S + g.s0 + rx) * T1 + g.t0;
+    idx_y[it] = (g.b * (S + 1) + g.s0 + ry) * Tn + g.t0;
   }
   // every quad of every row of block kb inside the valid columns?  (uniform over the workgroup)
   auto interior = [&](int kb) {
@@ -285,14 +290,17 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
     if (kb >= g.nblocks) return;
     const bool inner = interior(kb);
 #pragma unroll
-    for (int it = 0; it < 2; ++it) {
-      const int jp = kb * kW + 4 * mm - 1 - (mq + 32 * it) * g.skew;  // column left of element 0
+    for (int it = 0; it < kLoadItems; ++it) {
+      const int jp = kb * kW + 4 * mm - 1 - (lq + 16 * it) * g.skew;  // column left of element 0
+      const int jx = jp + g.skew;
       if (inner) {
-        r.x[it] = LoadQuad(segx[it].row + jp + g.skew);
-        r.y[it] = LoadQuad(segy[it].row + jp);
+        r.x[it] = BufferQuad(rsx, idx_x[it] + jx);
+        r.y[it] = BufferQuad(rsy, idx_y[it] + jp);
       } else {
-        r.x[it] = LoadClamped(segx[it], jp + g.skew);
-        r.y[it] = LoadClamped(segy[it], jp);
+        r.x[it] = BufferFour(rsx, idx_x[it] + jx, jx >= 0 && jx <= hi_x, jx + 1 >= 0 && jx + 1 <= hi_x,
+                             jx + 2 >= 0 && jx + 2 <= hi_x, jx + 3 >= 0 && jx + 3 <= hi_x);
+        r.y[it] = BufferFour(rsy, idx_y[it] + jp, jp >= 0 && jp <= hi_y, jp + 1 >= 0 && jp + 1 <= hi_y,
+                             jp + 2 >= 0 && jp + 2 <= hi_y, jp + 3 >= 0 && jp + 3 <= hi_y);
       }
     }
   };
@@ -300,8 +308,8 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
     if (kb >= g.nblocks) return;
     const bool inner = interior(kb);
 #pragma unroll
-    for (int it = 0; it < 2; ++it) {
-      const int q = mq + 32 * it;
+    for (int it = 0; it < kLoadItems; ++it) {
+      const int q = lq + 16 * it;
       const int jp = kb * kW + 4 * mm - 1 - q * g.skew;
       const int jx = jp + g.skew;
       float vx[4] = {r.x[it].x, r.x[it].y, r.x[it].z, r.x[it].w};
@@ -410,26 +418,32 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
   };
 
   // ---- prologue: block 0 committed, blocks 1 and 2 in flight ---------------------------------
-  FwdRegs ra, rb;
+  FwdRegs regs;
   if (role == kLoader) {
-    load_block(0, ra);
-    commit_block(0, ra);
-    load_block(1, ra);
-    load_block(2, rb);
+    if (grp == 0) {
+      load_block(0, regs);
+      commit_block(0, regs);
+      load_block(2, regs);
+    } else {
+      load_block(1, regs);
+    }
   } else if (role == kEdge) {
     take_block(0);
   }
   __syncthreads();
 
-  // One iteration: the chain wavefront computes block kb; the loaders commit block kb+1 (loaded
-  // two iterations ago) and start the loads of block kb+3; the storers drain block kb-1; the
-  // edge wavefront publishes block kb-1 downwards and takes block kb+1 from the chunk above.
-  auto iteration = [&](int kb, FwdRegs &r) {
+  // One iteration: the chain wavefront computes block kb; the loader group of block kb+1 commits
+  // it (loaded two iterations ago) and starts the loads of block kb+3; the storers drain block
+  // kb-1; the edge wavefront publishes block kb-1 downwards and takes block kb+1 from the chunk
+  // above.
+  for (int kb = 0; kb < g.nblocks; ++kb) {
     if (role == kChain) {
       chain_block(kb);
     } else if (role == kLoader) {
-      commit_block(kb + 1, r);
-      load_block(kb + 3, r);
+      if (((kb + 1) & 1) == grp) {
+        commit_block(kb + 1, regs);
+        load_block(kb + 3, regs);
+      }
     } else if (role == kStorer) {
       store_block(kb - 1);
     } else {
@@ -437,10 +451,6 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
       take_block(kb + 1);
     }
     __syncthreads();
-  };
-  for (int kb = 0; kb < g.nblocks; kb += 2) {
-    iteration(kb, ra);
-    if (kb + 1 < g.nblocks) iteration(kb + 1, rb);
   }
   if (role == kStorer) store_block(g.nblocks - 1);
   if (role == kEdge) publish_block(g.nblocks - 1);
@@ -469,7 +479,7 @@ struct BwdLds {
 };
 
 struct BwdRegs {
-  float4 d[2], s[2], x[2];  // p[dest], p[src], px[src]
+  float4 d[kLoadItems], s[kLoadItems], x[kLoadItems];  // p[dest], p[src], px[src]
 };
 
 // Clears the four columns c..c+3 of array row r of px_grad / py_grad wherever they lie outside
@@ -565,24 +575,23 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
   const int role = RoleOf(wave);
   const int mid = (threadIdx.x - (role == kStorer ? kWave * (2 + kMoverWaves) : 2 * kWave)) &
                   (kMoverLanes - 1);
-  const int mq = mid >> 3, mm = mid & 7;
+  const int mq = mid >> 3, mm = mid & 7;  // storers: rows mq and mq + 32, quad mm
+  const int grp = mid >> 7;               // loaders: group, and rows lq + 16*it, quad mm
+  const int lq = (mid & (kGroupLanes - 1)) >> 3;
 
   // ---- loaders ---------------------------------------------------------------------------
   // destination cells with both edges exist only for rows 1..ns and columns 1..nt
-  Segment segd[2], segs[2], segx[2];
-  {
-    const float *p_last = p + (size_t)B * (S + 1) * (Tn + 1) - 4;
-    const float *x_last = px + (size_t)B * S * T1 - 4;
+  const __amdgpu_buffer_rsrc_t rsp = MakeResource(p, (size_t)B * (S + 1) * (Tn + 1));
+  const __amdgpu_buffer_rsrc_t rsx = MakeResource(px, (size_t)B * S * T1);
+  // float index of destination column 0 of the item's row: p[dest], and p / px of the source
+  // cell of the px edge (column jd - 1 + skew of the row above)
+  int idx_d[kLoadItems], idx_s[kLoadItems], idx_x[kLoadItems];
 #pragma unroll
-    for (int it = 0; it < 2; ++it) {
-      const int rc = min(max(g.row0 + mq + 32 * it, 1), max(g.ns, 1));  // a row with a row above
-      const int hi = max(g.nt, 1);
-      // local column numbering = destination column jd (valid 1..nt); the source cell of the px
-      // edge sits at column jd - 1 + skew of the row above
-      segd[it] = Segment{pb + (size_t)(g.s0 + rc) * (Tn + 1) + g.t0 + 1, p_last, 1, hi};
-      segs[it] = Segment{pb + (size_t)(g.s0 + rc - 1) * (Tn + 1) + g.t0 + g.skew, p_last, 1, hi};
-      segx[it] = Segment{pxb + (size_t)(g.s0 + rc - 1) * T1 + g.t0 + g.skew, x_last, 1, hi};
-    }
+  for (int it = 0; it < kLoadItems; ++it) {
+    const int rc = min(max(g.row0 + lq + 16 * it, 1), max(g.ns, 1));  // a row with a row above
+    idx_d[it] = (g.b * (S + 1) + g.s0 + rc) * (Tn + 1) + g.t0;
+    idx_s[it] = (g.b * (S + 1) + g.s0 + rc - 1) * (Tn + 1) + g.t0 + g.skew - 1;
+    idx_x[it] = (g.b * S + g.s0 + rc - 1) * T1 + g.t0 + g.skew - 1;
   }
   // every destination cell of block kb has both edges inside the box?  (uniform)
   auto interior = [&](int kb) {
@@ -592,16 +601,18 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
     if (kb < 0) return;
     const bool inner = interior(kb);
 #pragma unroll
-    for (int it = 0; it < 2; ++it) {
-      const int jd = kb * kW + 4 * mm - (mq + 32 * it) * g.skew;  // destination column of element 0
+    for (int it = 0; it < kLoadItems; ++it) {
+      const int jd = kb * kW + 4 * mm - (lq + 16 * it) * g.skew;  // destination column of element 0
       if (inner) {
-        r.d[it] = LoadQuad(segd[it].row + (jd - 1));
-        r.s[it] = LoadQuad(segs[it].row + (jd - 1));
-        r.x[it] = LoadQuad(segx[it].row + (jd - 1));
+        r.d[it] = BufferQuad(rsp, idx_d[it] + jd);
+        r.s[it] = BufferQuad(rsp, idx_s[it] + jd);
+        r.x[it] = BufferQuad(rsx, idx_x[it] + jd);
       } else {
-        r.d[it] = LoadClamped(segd[it], jd);
-        r.s[it] = LoadClamped(segs[it], jd);
-        r.x[it] = LoadClamped(segx[it], jd);
+        const bool ok0 = jd >= 1 && jd <= g.nt, ok1 = jd + 1 >= 1 && jd + 1 <= g.nt,
+                   ok2 = jd + 2 >= 1 && jd + 2 <= g.nt, ok3 = jd + 3 >= 1 && jd + 3 <= g.nt;
+        r.d[it] = BufferFour(rsp, idx_d[it] + jd, ok0, ok1, ok2, ok3);
+        r.s[it] = BufferFour(rsp, idx_s[it] + jd, ok0, ok1, ok2, ok3);
+        r.x[it] = BufferFour(rsx, idx_x[it] + jd, ok0, ok1, ok2, ok3);
       }
     }
   };
@@ -631,8 +642,8 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
     if (kb < 0) return;
     const bool inner = interior(kb);
 #pragma unroll
-    for (int it = 0; it < 2; ++it) {
-      const int q = mq + 32 * it;
+    for (int it = 0; it < kLoadItems; ++it) {
+      const int q = lq + 16 * it;
       const int row_i = g.row0 + q;
       const int jd = kb * kW + 4 * mm - q * g.skew;
       const bool row_ok = row_i <= g.ns, first_row = row_i == 0, last_row = row_i == g.ns;
@@ -754,23 +765,29 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
   };
 
   const int top = g.nblocks - 1;
-  BwdRegs ra, rb;
+  // loader group of a block: blocks top, top-2, ... belong to group 0
+  BwdRegs regs;
   if (role == kLoader) {
-    load_block(top, ra);
-    commit_block(top, ra);
-    load_block(top - 1, ra);
-    load_block(top - 2, rb);
+    if (grp == 0) {
+      load_block(top, regs);
+      commit_block(top, regs);
+      load_block(top - 2, regs);
+    } else {
+      load_block(top - 1, regs);
+    }
   } else if (role == kEdge) {
     take_block(top);
   }
   __syncthreads();
 
-  auto iteration = [&](int kb, BwdRegs &r) {
+  for (int kb = top; kb >= 0; --kb) {
     if (role == kChain) {
       chain_block(kb);
     } else if (role == kLoader) {
-      commit_block(kb - 1, r);
-      load_block(kb - 3, r);
+      if (((top - kb + 1) & 1) == grp) {
+        commit_block(kb - 1, regs);
+        load_block(kb - 3, regs);
+      }
     } else if (role == kStorer) {
       store_block(kb + 1);
       zero_slices(top - kb);
@@ -779,10 +796,6 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
       take_block(kb - 1);
     }
     __syncthreads();
-  };
-  for (int kb = top; kb >= 0; kb -= 2) {
-    iteration(kb, ra);
-    if (kb - 1 >= 0) iteration(kb - 1, rb);
   }
   if (role == kStorer) store_block(0);
   if (role == kEdge) publish_block(0);
@@ -792,10 +805,11 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
 
 }  // namespace
 
-// The throughput kernels read quads; tensors with fewer than four elements take the exact path.
+// The throughput kernels address each tensor through a buffer resource with 32-bit byte offsets:
+// tensors of 2 GiB and more take the exact path.
 bool MiFastSupports(int B, int S, int Tn, int modified) {
-  const int T1 = modified ? Tn : Tn + 1;
-  return S >= 1 && Tn >= 1 && (long long)B * S * T1 >= 4 && (long long)B * (S + 1) * Tn >= 4;
+  (void)modified;
+  return S >= 1 && Tn >= 1 && (long long)B * (S + 1) * (Tn + 1) < (1ll << 29);
 }
 
 size_t MiFastWorkspaceBytes(int B, int S, int Tn) {
