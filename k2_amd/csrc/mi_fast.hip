@@ -55,13 +55,16 @@ constexpr int kQuadsPerRow = kStride / 4;
 constexpr int kQuadsPerBlock = kW / 4;
 // One work item = (row q in 0..63, quad m in 0..7) of a block: four consecutive steps of one
 // lattice row; 512 items per block.  The four storer wavefronts take two items per lane (rows q
-// and q + 32).  The four loader wavefronts form TWO GROUPS of 128 lanes that alternate blocks
-// (group = block & 1), four items per lane (rows q, q+16, q+32, q+48): a group loads a block,
-// then issues no other memory operation until it commits that block two iterations later, so
-// the wait in front of the commit covers exactly those loads.
+// and q + 32).  The loader wavefronts form kGroups groups that take blocks in turn (group =
+// block % kGroups), kLoadItems items per lane (rows q, q + kRowStep, ...): a group loads a
+// block, then issues no other memory operation until it commits that block kGroups iterations
+// later, so the wait in front of the commit covers exactly those loads and kGroups blocks are
+// in flight at any time.
 static_assert(kRows * kQuadsPerBlock == 2 * kMoverLanes, "two work items per storer lane");
-constexpr int kGroupLanes = kMoverLanes / 2;
-constexpr int kLoadItems = kRows * kQuadsPerBlock / kGroupLanes;  // 4
+constexpr int kGroups = 2;
+constexpr int kGroupLanes = kMoverLanes / kGroups;
+constexpr int kLoadItems = kRows * kQuadsPerBlock / kGroupLanes;
+constexpr int kRowStep = kGroupLanes / kQuadsPerBlock;  // rows between a lane's items
 
 struct FastHeader {
   unsigned ticket;  // next chunk to hand out; reset by the last workgroup of a launch
@@ -262,7 +265,7 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
   const int mid = (threadIdx.x - (role == kStorer ? kWave * (2 + kMoverWaves) : 2 * kWave)) &
                   (kMoverLanes - 1);
   const int mq = mid >> 3, mm = mid & 7;  // storers: rows mq and mq + 32, quad mm
-  const int grp = mid >> 7;               // loaders: group, and rows lq + 16*it, quad mm
+  const int grp = mid / kGroupLanes;              // loaders: group, rows lq + kRowStep*it, quad mm
   const int lq = (mid & (kGroupLanes - 1)) >> 3;
 
   const int hi_x = g.nt - modified, hi_y = g.nt - 1;  // last valid px / py column
@@ -274,7 +277,7 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
   bool rowx_ok[kLoadItems], rowy_ok[kLoadItems];
 #pragma unroll
   for (int it = 0; it < kLoadItems; ++it) {
-    const int row_i = g.row0 + lq + 16 * it;
+    const int row_i = g.row0 + lq + kRowStep * it;
     rowx_ok[it] = row_i >= 1 && row_i <= g.ns;
     rowy_ok[it] = row_i <= g.ns;
     const int rx = min(max(row_i, 1), max(g.ns, 1)) - 1;  // a px row inside the box if any
@@ -291,7 +294,7 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
     const bool inner = interior(kb);
 #pragma unroll
     for (int it = 0; it < kLoadItems; ++it) {
-      const int jp = kb * kW + 4 * mm - 1 - (lq + 16 * it) * g.skew;  // column left of element 0
+      const int jp = kb * kW + 4 * mm - 1 - (lq + kRowStep * it) * g.skew;  // column left of element 0
       const int jx = jp + g.skew;
       if (inner) {
         r.x[it] = BufferQuad(rsx, idx_x[it] + jx);
@@ -309,7 +312,7 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
     const bool inner = interior(kb);
 #pragma unroll
     for (int it = 0; it < kLoadItems; ++it) {
-      const int q = lq + 16 * it;
+      const int q = lq + kRowStep * it;
       const int jp = kb * kW + 4 * mm - 1 - q * g.skew;
       const int jx = jp + g.skew;
       float vx[4] = {r.x[it].x, r.x[it].y, r.x[it].z, r.x[it].w};
@@ -418,14 +421,14 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
   };
 
   // ---- prologue: block 0 committed, blocks 1 and 2 in flight ---------------------------------
+  // the chain wavefront is the critical path: it wins the SIMD's issue arbitration
+  if (role == kChain) __builtin_amdgcn_s_setprio(3);
   FwdRegs regs;
   if (role == kLoader) {
+    load_block(grp, regs);
     if (grp == 0) {
-      load_block(0, regs);
       commit_block(0, regs);
-      load_block(2, regs);
-    } else {
-      load_block(1, regs);
+      load_block(kGroups, regs);
     }
   } else if (role == kEdge) {
     take_block(0);
@@ -433,16 +436,16 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
   __syncthreads();
 
   // One iteration: the chain wavefront computes block kb; the loader group of block kb+1 commits
-  // it (loaded two iterations ago) and starts the loads of block kb+3; the storers drain block
+  // it (loaded kGroups iterations ago) and starts the loads of block kb+1+kGroups; the storers drain block
   // kb-1; the edge wavefront publishes block kb-1 downwards and takes block kb+1 from the chunk
   // above.
   for (int kb = 0; kb < g.nblocks; ++kb) {
     if (role == kChain) {
       chain_block(kb);
     } else if (role == kLoader) {
-      if (((kb + 1) & 1) == grp) {
+      if (((kb + 1) & (kGroups - 1)) == grp) {
         commit_block(kb + 1, regs);
-        load_block(kb + 3, regs);
+        load_block(kb + 1 + kGroups, regs);
       }
     } else if (role == kStorer) {
       store_block(kb - 1);
@@ -576,7 +579,7 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
   const int mid = (threadIdx.x - (role == kStorer ? kWave * (2 + kMoverWaves) : 2 * kWave)) &
                   (kMoverLanes - 1);
   const int mq = mid >> 3, mm = mid & 7;  // storers: rows mq and mq + 32, quad mm
-  const int grp = mid >> 7;               // loaders: group, and rows lq + 16*it, quad mm
+  const int grp = mid / kGroupLanes;              // loaders: group, rows lq + kRowStep*it, quad mm
   const int lq = (mid & (kGroupLanes - 1)) >> 3;
 
   // ---- loaders ---------------------------------------------------------------------------
@@ -588,7 +591,7 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
   int idx_d[kLoadItems], idx_s[kLoadItems], idx_x[kLoadItems];
 #pragma unroll
   for (int it = 0; it < kLoadItems; ++it) {
-    const int rc = min(max(g.row0 + lq + 16 * it, 1), max(g.ns, 1));  // a row with a row above
+    const int rc = min(max(g.row0 + lq + kRowStep * it, 1), max(g.ns, 1));  // a row with a row above
     idx_d[it] = (g.b * (S + 1) + g.s0 + rc) * (Tn + 1) + g.t0;
     idx_s[it] = (g.b * (S + 1) + g.s0 + rc - 1) * (Tn + 1) + g.t0 + g.skew - 1;
     idx_x[it] = (g.b * S + g.s0 + rc - 1) * T1 + g.t0 + g.skew - 1;
@@ -602,7 +605,7 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
     const bool inner = interior(kb);
 #pragma unroll
     for (int it = 0; it < kLoadItems; ++it) {
-      const int jd = kb * kW + 4 * mm - (lq + 16 * it) * g.skew;  // destination column of element 0
+      const int jd = kb * kW + 4 * mm - (lq + kRowStep * it) * g.skew;  // destination column of element 0
       if (inner) {
         r.d[it] = BufferQuad(rsp, idx_d[it] + jd);
         r.s[it] = BufferQuad(rsp, idx_s[it] + jd);
@@ -643,7 +646,7 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
     const bool inner = interior(kb);
 #pragma unroll
     for (int it = 0; it < kLoadItems; ++it) {
-      const int q = lq + 16 * it;
+      const int q = lq + kRowStep * it;
       const int row_i = g.row0 + q;
       const int jd = kb * kW + 4 * mm - q * g.skew;
       const bool row_ok = row_i <= g.ns, first_row = row_i == 0, last_row = row_i == g.ns;
@@ -765,15 +768,14 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
   };
 
   const int top = g.nblocks - 1;
-  // loader group of a block: blocks top, top-2, ... belong to group 0
+  // loader group of block kb: (top - kb) % kGroups
+  if (role == kChain) __builtin_amdgcn_s_setprio(3);
   BwdRegs regs;
   if (role == kLoader) {
+    load_block(top - grp, regs);
     if (grp == 0) {
-      load_block(top, regs);
       commit_block(top, regs);
-      load_block(top - 2, regs);
-    } else {
-      load_block(top - 1, regs);
+      load_block(top - kGroups, regs);
     }
   } else if (role == kEdge) {
     take_block(top);
@@ -784,9 +786,9 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
     if (role == kChain) {
       chain_block(kb);
     } else if (role == kLoader) {
-      if (((top - kb + 1) & 1) == grp) {
+      if (((top - kb + 1) & (kGroups - 1)) == grp) {
         commit_block(kb - 1, regs);
-        load_block(kb - 3, regs);
+        load_block(kb - 1 - kGroups, regs);
       }
     } else if (role == kStorer) {
       store_block(kb + 1);
