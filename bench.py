@@ -5,8 +5,9 @@ Workload (BASELINE config 4): fp32, modified lattice, B=32, S=200, T=1000, px/py
 per-sequence boundary with T_b in [600,1000] and S_b in [100,200].  One step = one forward
 launch + one backward launch through the C-ABI, inputs resident in HBM.
 
-Prints ONE JSON line (see README / DESIGN.md for the field meanings).  `value` counts ACTIVE
-lattice cells, sum_b (S_b+1)(T_b+1), per second of fwd+bwd wall time on the GPU.
+Prints ONE JSON line.  `value` counts ACTIVE lattice cells, sum_b (S_b+1)(T_b+1), per second of
+fwd+bwd wall time on the GPU; `roofline` prices the slower of the two kernels against the HBM
+peak with its algorithmic bytes; `cpu_baseline` is the reference's CPU loop on this host.
 """
 import argparse
 import json
@@ -26,6 +27,11 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # reads px, p and writes px_grad, py_grad (16 B; the backward never needs py).
 FWD_BYTES_PER_CELL = 12
 BWD_BYTES_PER_CELL = 16
+
+# HBM bytes per launch on the default workload, from rocprofv3's FETCH_SIZE / WRITE_SIZE counters
+# scaled by a 256 MiB device copy (profiles/mi_fast_kernels_c4_hbm_traffic.md).  Reported only
+# for the default shape; any other --B/--S/--T prints null.
+MEASURED_TRAFFIC_BYTES = {"mi_forward": 49645274, "mi_backward": 86098915}
 
 
 def cpu_baseline(c, budget_s=12.0):
@@ -57,13 +63,17 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also launch one plain device copy of 256 MiB before the warmup: the unit "
+                         "against which rocprofv3's FETCH_SIZE / WRITE_SIZE readings are scaled")
     ap.add_argument("--B", type=int, default=32)
     ap.add_argument("--S", type=int, default=200)
     ap.add_argument("--T", type=int, default=1000)
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (the batch axis would "
-              "shard trivially, see DESIGN.md); run with --gpus 1", file=sys.stderr)
+        print("bench.py measures one GPU: this build has no multi-GPU path (sequences are "
+              "independent, so the batch axis is what would be sharded); run with --gpus 1",
+              file=sys.stderr)
         sys.exit(2)
 
     import torch
@@ -96,6 +106,13 @@ def main():
             ev[2].record()
         return g
 
+    if args.copy_probe:
+        src = torch.zeros(64 << 20, dtype=torch.float32, device=dev)  # 256 MiB read + 256 MiB written
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -130,7 +147,9 @@ def main():
                                f"S={S} T={T}, random boundary (BASELINE config 4)",
                    "active_cells": active, "full_box_cells": full},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": dom,
+                     "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": MEASURED_TRAFFIC_BYTES[dom] if (B, S, T) == (32, 200, 1000) else None,
+                     "kernel": dom,
                      "kernel_avg_us": dom_ms * 1e3},
         "kernels": {"mi_forward_avg_us": fwd_avg * 1e3, "mi_forward_min_us": float(fwd_ms.min()) * 1e3,
                     "mi_backward_avg_us": bwd_avg * 1e3, "mi_backward_min_us": float(bwd_ms.min()) * 1e3,

@@ -78,7 +78,6 @@ def build_pybind(verbose=False):
         f"-L{HERE}", "-lk2amd", "-Wl,-rpath,$ORIGIN",
         f"-L{tdir}/lib", f"-Wl,-rpath,{tdir}/lib",
         "-ltorch", "-ltorch_cpu", "-lc10", "-ltorch_python", "-ltorch_hip", "-lc10_hip",
-        "-L/opt/rocm/lib", "-Wl,-rpath,/opt/rocm/lib", "-lamdhip64",
     ]
     _run(cmd)
     if verbose:

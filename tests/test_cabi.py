@@ -76,3 +76,23 @@ def test_cpu_tensors_fail_loudly():
         k2.mutual_information_recursion(px, torch.zeros(1, 3, 7))
     with pytest.raises(AssertionError):
         k2.mutual_information_recursion(px, py, torch.tensor([[0, 0, 5, 3]]))
+
+
+def test_pybind_host_module_mirrors_k2_native_functions():
+    """The C++ host module carries the two functions of the reference's `_k2` for this path with
+    the same keyword names (k2/python/csrc/torch/mutual_information.cu:26-67) and is the one the
+    Python layer routes through."""
+    import torch
+    from k2_amd import _k2_amd, native
+    assert native._ext is _k2_amd
+    assert _k2_amd.version() == 100
+    doc = _k2_amd.mutual_information_forward.__doc__
+    assert all(k in doc for k in ("px:", "py:", "boundary:", "p:"))
+    doc = _k2_amd.mutual_information_backward.__doc__
+    assert all(k in doc for k in ("px:", "py:", "boundary:", "p:", "ans_grad:"))
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        _k2_amd.mutual_information_forward(px=torch.zeros(1, 2, 3), py=torch.zeros(1, 3, 3),
+                                           boundary=None, p=torch.zeros(1, 3, 4))
+    with pytest.raises(RuntimeError, match="3-dimensional"):
+        _k2_amd.mutual_information_forward(px=torch.zeros(2, 9), py=torch.zeros(1, 3, 3),
+                                           boundary=None, p=torch.zeros(1, 3, 4))

@@ -171,3 +171,35 @@ def test_headline_shape_three_way(device):
         s1 = int(bd[b, 2])
         np.testing.assert_allclose(gx[b, :s1].sum(axis=1), 1.0, rtol=2e-3)
     np.testing.assert_allclose(g_out, g_in, rtol=2e-3)
+
+
+@pytest.mark.gpu
+def test_pybind_host_matches_ctypes_host(device):
+    """The C++ host module and the ctypes binding drive the same kernels: identical bits, on the
+    current stream, with a strided px view made contiguous by the host layer, and ans_grad
+    overwritten by the gradient that reached the origin."""
+    from k2_amd import _k2_amd, capi
+    rng = np.random.default_rng(77)
+    B, S, T = 3, 70, 90
+    px = torch.from_numpy(rng.standard_normal((B, S, T + 1)).astype(np.float32)).to(device)
+    py = torch.from_numpy(rng.standard_normal((B, S + 1, T)).astype(np.float32)).to(device)
+    bd = torch.tensor([[0, 0, S, T], [3, 5, 66, 80], [0, 10, 70, 90]], dtype=torch.int64, device=device)
+    p1 = torch.empty(B, S + 1, T + 1, device=device)
+    p2 = torch.empty_like(p1)
+    ans1 = capi.mi_forward(px, py, bd, p1)
+    px_strided = torch.empty(B, S, 2 * px.shape[2], device=device)[:, :, ::2]
+    px_strided.copy_(px)
+    side = torch.cuda.Stream(device=device)
+    side.wait_stream(torch.cuda.current_stream(device))
+    with torch.cuda.stream(side):
+        ans2 = _k2_amd.mutual_information_forward(px=px_strided, py=py, boundary=bd, p=p2)
+        g2 = torch.full((B,), 2.0, device=device)
+        gx2, gy2 = _k2_amd.mutual_information_backward(px=px, py=py, boundary=bd, p=p2, ans_grad=g2)
+    side.synchronize()
+    g1 = torch.full((B,), 2.0, device=device)
+    gx1, gy1 = capi.mi_backward(px, py, bd, p1, g1, overwrite_ans_grad=True)
+    torch.cuda.synchronize()
+    assert torch.equal(ans1, ans2)
+    assert torch.equal(gx1, gx2) and torch.equal(gy1, gy2)
+    assert torch.equal(g1, g2)
+    np.testing.assert_allclose(g2.cpu().numpy(), 2.0, rtol=1e-3)
