@@ -203,3 +203,41 @@ def test_pybind_host_matches_ctypes_host(device):
     assert torch.equal(gx1, gx2) and torch.equal(gy1, gy2)
     assert torch.equal(g1, g2)
     np.testing.assert_allclose(g2.cpu().numpy(), 2.0, rtol=1e-3)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_joint_recursion_identities(device, dtype):
+    """The checks of k2/python/tests/mutual_information_test.py:137-166: the joint recursion on
+    one input equals the plain one, on two halves it equals it after summing over the inputs,
+    and backprop through either gives the same derivative."""
+    import k2_amd as k2
+    rng = np.random.default_rng(5)
+    for modified in (False, True):
+        B, S, T = 4, 9, 40
+        T1 = T if modified else T + 1
+        npx = rng.standard_normal((B, S, T1))
+        npy = rng.standard_normal((B, S + 1, T))
+        bd = torch.tensor([[0, 0, S, T], [1, 2, 8, 37], [0, 5, 9, 40], [2, 0, 2, 30]],
+                          dtype=torch.int64, device=device)
+        grads = []
+        for which in range(3):
+            px = torch.tensor(npx, dtype=dtype, device=device, requires_grad=True)
+            py = torch.tensor(npy, dtype=dtype, device=device, requires_grad=True)
+            m = k2.mutual_information_recursion(px, py, bd)
+            m2 = k2.joint_mutual_information_recursion((px,), (py,), bd)
+            m3 = k2.joint_mutual_information_recursion((px * 0.5, px * 0.5), (py * 0.5, py * 0.5), bd)
+            assert m2.shape == (1, B) and m3.shape == (2, B)
+            tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=1e-10, atol=1e-10)
+            assert torch.allclose(m, m2[0], **tol)
+            assert torch.allclose(m, m3.sum(dim=0), **tol)
+            ((m, m2, m3)[which].sum() * 3).backward()
+            grads.append((px.grad.clone(), py.grad.clone()))
+        for gx, gy in grads[1:]:
+            assert torch.allclose(gx, grads[0][0], rtol=1e-4, atol=1e-5)
+            assert torch.allclose(gy, grads[0][1], rtol=1e-4, atol=1e-5)
+        # and the plain recursion's derivative is the oracle's occupation probabilities x 3
+        a, p = omi.mi_forward(npx, npy, bd.cpu().numpy())
+        wx, wy = omi.mi_backward(npx, npy, bd.cpu().numpy(), p)
+        np.testing.assert_allclose(grads[0][0].cpu().numpy(), 3 * wx, rtol=1e-4, atol=1e-5)
+        np.testing.assert_allclose(grads[0][1].cpu().numpy(), 3 * wy, rtol=1e-4, atol=1e-5)
