@@ -54,17 +54,14 @@ constexpr float kLn2 = 0.69314718055994530942f;
 constexpr int kQuadsPerRow = kStride / 4;
 constexpr int kQuadsPerBlock = kW / 4;
 // One work item = (row q in 0..63, quad m in 0..7) of a block: four consecutive steps of one
-// lattice row; 512 items per block.  The four storer wavefronts take two items per lane (rows q
-// and q + 32).  The loader wavefronts form kGroups groups that take blocks in turn (group =
-// block % kGroups), kLoadItems items per lane (rows q, q + kRowStep, ...): a group loads a
-// block, then issues no other memory operation until it commits that block kGroups iterations
-// later, so the wait in front of the commit covers exactly those loads and kGroups blocks are
-// in flight at any time.
-static_assert(kRows * kQuadsPerBlock == 2 * kMoverLanes, "two work items per storer lane");
-constexpr int kGroups = 2;
-constexpr int kGroupLanes = kMoverLanes / kGroups;
-constexpr int kLoadItems = kRows * kQuadsPerBlock / kGroupLanes;
-constexpr int kRowStep = kGroupLanes / kQuadsPerBlock;  // rows between a lane's items
+// lattice row; 512 items per block, two per loader lane and two per storer lane (rows q and
+// q + 32, same quad).  A wave-wide 16-byte load or store occupies its wavefront for about a
+// hundred cycles once the memory pipeline is busy, so the movers' work is spread over all their
+// wavefronts in every iteration, and the loaders keep two register sets so that a block's loads
+// stay in flight for two iterations.
+static_assert(kRows * kQuadsPerBlock == 2 * kMoverLanes, "two work items per mover lane");
+constexpr int kLoadItems = 2;
+constexpr int kRowStep = kMoverLanes / kQuadsPerBlock;  // rows between a lane's items (32)
 
 struct FastHeader {
   unsigned ticket;  // next chunk to hand out; reset by the last workgroup of a launch
@@ -121,28 +118,56 @@ __device__ __forceinline__ void StoreQuad(float *ptr, float4 v) {
 // Loads go through raw buffer resources (one per tensor): the hardware range-checks every dword
 // against the tensor's size and returns 0 beyond it, so no load can leave the tensor whatever
 // the boundary tensor holds, and no address clamping code sits in the loaders.
-typedef unsigned uint4v __attribute__((ext_vector_type(4)));
+//
+// The loaders' loads are issued from inline assembly and waited for with explicit s_waitcnt:
+// a block's loads have to stay in flight across two loop iterations, and the compiler's own
+// wait-count insertion falls back to "wait for everything" for loads carried around a loop,
+// which would stall every iteration for a full memory round trip.  The loader loop issues no
+// other vector memory operation, so the counts below are exact.
+typedef int int4v __attribute__((ext_vector_type(4)));
 typedef float float4v __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t MakeResource(const float *base, size_t elems) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(base), 0, (int)(elems * sizeof(float)),
-                                           0x00020000);
-}
-// four consecutive floats starting at float index `idx` (idx >= 0)
-__device__ __forceinline__ float4 BufferQuad(__amdgpu_buffer_rsrc_t rs, int idx) {
-  const float4v v = __builtin_bit_cast(float4v, __builtin_amdgcn_raw_buffer_load_b128(rs, idx * 4, 0, 0));
-  return make_float4(v.x, v.y, v.z, v.w);
-}
-// floats idx .. idx+3, each loaded on its own; elements whose flag is false read index 0 instead
-// (they are masked by the caller).  Used where a quad would straddle the valid columns.
-__device__ __forceinline__ float4 BufferFour(__amdgpu_buffer_rsrc_t rs, int idx, bool ok0, bool ok1,
-                                             bool ok2, bool ok3) {
-  float4 r;
-  r.x = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, ok0 ? (idx + 0) * 4 : 0, 0, 0));
-  r.y = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, ok1 ? (idx + 1) * 4 : 0, 0, 0));
-  r.z = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, ok2 ? (idx + 2) * 4 : 0, 0, 0));
-  r.w = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, ok3 ? (idx + 3) * 4 : 0, 0, 0));
+__device__ __forceinline__ int4v MakeResource(const float *base, size_t elems) {
+  const unsigned long long a = reinterpret_cast<unsigned long long>(base);
+  int4v r;
+  r.x = __builtin_amdgcn_readfirstlane((int)(a & 0xffffffffull));
+  r.y = __builtin_amdgcn_readfirstlane((int)(a >> 32));  // stride 0: a raw buffer
+  r.z = __builtin_amdgcn_readfirstlane((int)(elems * sizeof(float)));
+  r.w = 0x00020000;
   return r;
+}
+// starts the load of four consecutive floats from float index max(idx, 0); the result may be
+// read only after a WaitLoads that covers it
+__device__ __forceinline__ float4v AsyncQuad(int4v rs, int idx) {
+  float4v v;
+  const int off = max(idx, 0) * 4;
+  asm volatile("buffer_load_dwordx4 %0, %1, %2, 0 offen" : "=v"(v) : "v"(off), "s"(rs) : "memory");
+  return v;
+}
+__device__ __forceinline__ float4 AsFloat4(float4v v) { return make_float4(v.x, v.y, v.z, v.w); }
+
+// A quad whose first float would lie in front of the tensor (idx < 0: only possible for the
+// tensor's very first row) is loaded from index 0 instead; this moves the floats back to the
+// positions they were asked for.  The floats in front of the tensor belong to columns outside
+// the box and are masked by the caller.
+__device__ __forceinline__ float4 ShiftQuad(float4 v, int idx) {
+  const int sh = idx < 0 ? -idx : 0;
+  float4 r;
+  r.x = v.x;
+  r.y = sh == 0 ? v.y : v.x;
+  r.z = sh == 0 ? v.z : (sh == 1 ? v.y : v.x);
+  r.w = sh == 0 ? v.w : (sh == 1 ? v.z : (sh == 2 ? v.y : v.x));
+  return r;
+}
+
+// Workgroup barrier that orders LDS traffic only.  Everything the wavefronts of a workgroup hand
+// to each other goes through LDS, so global loads (the loaders' prefetch) and global stores (the
+// storers' output) stay in flight across it; a full __syncthreads() would drain them
+// (s_waitcnt vmcnt(0)) every iteration and serialise the pipeline on HBM latency.
+__device__ __forceinline__ void LdsBarrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
 struct ChunkGeom {
@@ -223,8 +248,18 @@ struct FwdLds {
 };
 
 struct FwdRegs {
-  float4 x[kLoadItems], y[kLoadItems];
+  float4v x[kLoadItems], y[kLoadItems];
 };
+// waits until at most kYounger of this wavefront's loads are outstanding and ties the registers
+// to the wait, so that no read of them moves in front of it
+template <int kYounger>
+__device__ __forceinline__ void WaitLoads(FwdRegs &r) {
+  static_assert(kLoadItems == 2, "operand list below");
+  asm volatile("s_waitcnt vmcnt(%4)"
+               : "+v"(r.x[0]), "+v"(r.y[0]), "+v"(r.x[1]), "+v"(r.y[1])
+               : "n"(kYounger));
+}
+constexpr int kFwdLoadsPerBlock = 2 * kLoadItems;
 
 __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
     const float *__restrict__ px, const float *__restrict__ py,
@@ -265,14 +300,13 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
   const int mid = (threadIdx.x - (role == kStorer ? kWave * (2 + kMoverWaves) : 2 * kWave)) &
                   (kMoverLanes - 1);
   const int mq = mid >> 3, mm = mid & 7;  // storers: rows mq and mq + 32, quad mm
-  const int grp = mid / kGroupLanes;              // loaders: group, rows lq + kRowStep*it, quad mm
-  const int lq = (mid & (kGroupLanes - 1)) >> 3;
+  const int lq = mq;                      // loaders: rows lq + kRowStep*it, quad mm
 
   const int hi_x = g.nt - modified, hi_y = g.nt - 1;  // last valid px / py column
 
   // ---- loaders ---------------------------------------------------------------------------
-  const __amdgpu_buffer_rsrc_t rsx = MakeResource(px, (size_t)B * S * T1);
-  const __amdgpu_buffer_rsrc_t rsy = MakeResource(py, (size_t)B * (S + 1) * Tn);
+  const int4v rsx = MakeResource(px, (size_t)B * S * T1);
+  const int4v rsy = MakeResource(py, (size_t)B * (S + 1) * Tn);
   int idx_x[kLoadItems], idx_y[kLoadItems];  // float index of local column 0 of the item's row
   bool rowx_ok[kLoadItems], rowy_ok[kLoadItems];
 #pragma unroll
@@ -289,25 +323,19 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
   auto interior = [&](int kb) {
     return kb * kW - 1 - (kRows - 1) * g.skew >= 0 && kb * kW + 30 <= g.nt - 1;
   };
+  // One code path for every block: quads that reach outside the valid columns pick up
+  // neighbouring floats (or zeros past the tensor's end) that the commit masks.
+  // Always issues kFwdLoadsPerBlock loads, also for blocks past the last one (they read floats
+  // that nobody uses), so that the counts given to WaitLoads hold in every iteration.
   auto load_block = [&](int kb, FwdRegs &r) {
-    if (kb >= g.nblocks) return;
-    const bool inner = interior(kb);
 #pragma unroll
     for (int it = 0; it < kLoadItems; ++it) {
       const int jp = kb * kW + 4 * mm - 1 - (lq + kRowStep * it) * g.skew;  // column left of element 0
-      const int jx = jp + g.skew;
-      if (inner) {
-        r.x[it] = BufferQuad(rsx, idx_x[it] + jx);
-        r.y[it] = BufferQuad(rsy, idx_y[it] + jp);
-      } else {
-        r.x[it] = BufferFour(rsx, idx_x[it] + jx, jx >= 0 && jx <= hi_x, jx + 1 >= 0 && jx + 1 <= hi_x,
-                             jx + 2 >= 0 && jx + 2 <= hi_x, jx + 3 >= 0 && jx + 3 <= hi_x);
-        r.y[it] = BufferFour(rsy, idx_y[it] + jp, jp >= 0 && jp <= hi_y, jp + 1 >= 0 && jp + 1 <= hi_y,
-                             jp + 2 >= 0 && jp + 2 <= hi_y, jp + 3 >= 0 && jp + 3 <= hi_y);
-      }
+      r.x[it] = AsyncQuad(rsx, idx_x[it] + jp + g.skew);
+      r.y[it] = AsyncQuad(rsy, idx_y[it] + jp);
     }
   };
-  auto commit_block = [&](int kb, const FwdRegs &r) {  // registers -> LDS ring
+  auto commit_block = [&](int kb, FwdRegs &r) {  // registers -> LDS ring
     if (kb >= g.nblocks) return;
     const bool inner = interior(kb);
 #pragma unroll
@@ -315,8 +343,13 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
       const int q = lq + kRowStep * it;
       const int jp = kb * kW + 4 * mm - 1 - q * g.skew;
       const int jx = jp + g.skew;
-      float vx[4] = {r.x[it].x, r.x[it].y, r.x[it].z, r.x[it].w};
-      float vy[4] = {r.y[it].x, r.y[it].y, r.y[it].z, r.y[it].w};
+      float4 qx = AsFloat4(r.x[it]), qy = AsFloat4(r.y[it]);
+      if (!inner && g.b == 0) {  // the only sequence whose rows can start the tensor
+        qx = ShiftQuad(qx, idx_x[it] + jx);
+        qy = ShiftQuad(qy, idx_y[it] + jp);
+      }
+      float vx[4] = {qx.x, qx.y, qx.z, qx.w};
+      float vy[4] = {qy.x, qy.y, qy.z, qy.w};
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const bool okx = rowx_ok[it] && (inner || (jx + e >= 0 && jx + e <= hi_x));
@@ -420,40 +453,55 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
     }
   };
 
-  // ---- prologue: block 0 committed, blocks 1 and 2 in flight ---------------------------------
   // the chain wavefront is the critical path: it wins the SIMD's issue arbitration
   if (role == kChain) __builtin_amdgcn_s_setprio(3);
-  FwdRegs regs;
+  // ---- prologue: block 0 committed, blocks 1 and 2 in flight ---------------------------------
+  FwdRegs ra, rb;
   if (role == kLoader) {
-    load_block(grp, regs);
-    if (grp == 0) {
-      commit_block(0, regs);
-      load_block(kGroups, regs);
-    }
+    load_block(0, ra);
+    WaitLoads<0>(ra);
+    commit_block(0, ra);
+    load_block(1, ra);
+    load_block(2, rb);
   } else if (role == kEdge) {
     take_block(0);
   }
-  __syncthreads();
+  LdsBarrier();
 
-  // One iteration: the chain wavefront computes block kb; the loader group of block kb+1 commits
-  // it (loaded kGroups iterations ago) and starts the loads of block kb+1+kGroups; the storers drain block
-  // kb-1; the edge wavefront publishes block kb-1 downwards and takes block kb+1 from the chunk
-  // above.
-  for (int kb = 0; kb < g.nblocks; ++kb) {
-    if (role == kChain) {
+  // In iteration kb the chain wavefront computes block kb; the loaders commit block kb+1 (loaded
+  // two iterations ago) and start the loads of block kb+3; the storers drain block kb-1; the
+  // edge wavefront publishes block kb-1 downwards and takes block kb+1 from the chunk above.
+  // Every role runs its own loop (same number of barriers), which keeps each loop free of the
+  // other roles' code and lets the compiler count outstanding loads exactly.
+  if (role == kChain) {
+    for (int kb = 0; kb < g.nblocks; ++kb) {
       chain_block(kb);
-    } else if (role == kLoader) {
-      if (((kb + 1) & (kGroups - 1)) == grp) {
-        commit_block(kb + 1, regs);
-        load_block(kb + 1 + kGroups, regs);
+      LdsBarrier();
+    }
+  } else if (role == kLoader) {
+    for (int kb = 0; kb < g.nblocks; kb += 2) {
+      WaitLoads<kFwdLoadsPerBlock>(ra);  // the other set's loads may stay in flight
+      commit_block(kb + 1, ra);
+      load_block(kb + 3, ra);
+      LdsBarrier();
+      if (kb + 1 < g.nblocks) {
+        WaitLoads<kFwdLoadsPerBlock>(rb);
+        commit_block(kb + 2, rb);
+        load_block(kb + 4, rb);
+        LdsBarrier();
       }
-    } else if (role == kStorer) {
+    }
+  } else if (role == kStorer) {
+    for (int kb = 0; kb < g.nblocks; ++kb) {
       store_block(kb - 1);
-    } else {
+      LdsBarrier();
+    }
+  } else {
+    for (int kb = 0; kb < g.nblocks; ++kb) {
       publish_block(kb - 1);
       take_block(kb + 1);
+      LdsBarrier();
     }
-    __syncthreads();
   }
   if (role == kStorer) store_block(g.nblocks - 1);
   if (role == kEdge) publish_block(g.nblocks - 1);
@@ -482,8 +530,16 @@ struct BwdLds {
 };
 
 struct BwdRegs {
-  float4 d[kLoadItems], s[kLoadItems], x[kLoadItems];  // p[dest], p[src], px[src]
+  float4v d[kLoadItems], s[kLoadItems], x[kLoadItems];  // p[dest], p[src], px[src]
 };
+template <int kYounger>
+__device__ __forceinline__ void WaitLoads(BwdRegs &r) {
+  static_assert(kLoadItems == 2, "operand list below");
+  asm volatile("s_waitcnt vmcnt(%6)"
+               : "+v"(r.d[0]), "+v"(r.s[0]), "+v"(r.x[0]), "+v"(r.d[1]), "+v"(r.s[1]), "+v"(r.x[1])
+               : "n"(kYounger));
+}
+constexpr int kBwdLoadsPerBlock = 3 * kLoadItems;
 
 // Clears the four columns c..c+3 of array row r of px_grad / py_grad wherever they lie outside
 // the region the sweep assigns.
@@ -579,13 +635,12 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
   const int mid = (threadIdx.x - (role == kStorer ? kWave * (2 + kMoverWaves) : 2 * kWave)) &
                   (kMoverLanes - 1);
   const int mq = mid >> 3, mm = mid & 7;  // storers: rows mq and mq + 32, quad mm
-  const int grp = mid / kGroupLanes;              // loaders: group, rows lq + kRowStep*it, quad mm
-  const int lq = (mid & (kGroupLanes - 1)) >> 3;
+  const int lq = mq;                      // loaders: rows lq + kRowStep*it, quad mm
 
   // ---- loaders ---------------------------------------------------------------------------
   // destination cells with both edges exist only for rows 1..ns and columns 1..nt
-  const __amdgpu_buffer_rsrc_t rsp = MakeResource(p, (size_t)B * (S + 1) * (Tn + 1));
-  const __amdgpu_buffer_rsrc_t rsx = MakeResource(px, (size_t)B * S * T1);
+  const int4v rsp = MakeResource(p, (size_t)B * (S + 1) * (Tn + 1));
+  const int4v rsx = MakeResource(px, (size_t)B * S * T1);
   // float index of destination column 0 of the item's row: p[dest], and p / px of the source
   // cell of the px edge (column jd - 1 + skew of the row above)
   int idx_d[kLoadItems], idx_s[kLoadItems], idx_x[kLoadItems];
@@ -600,65 +655,92 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
   auto interior = [&](int kb) {
     return kb * kW - (kRows - 1) * g.skew >= 1 && kb * kW + 31 <= g.nt;
   };
+  // Rows past the sequence's last row never change: their E / OME stay at the zeros written
+  // here, the loaders skip them.
+  bool row_ok[kLoadItems];
+#pragma unroll
+  for (int it = 0; it < kLoadItems; ++it) row_ok[it] = g.row0 + lq + kRowStep * it <= g.ns;
+  if (g.row0 + kRows - 1 > g.ns) {
+    const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int i = threadIdx.x; i < kWave * kQuadsPerRow; i += kFastThreads) {
+      const int q = i / kQuadsPerRow, k = i - q * kQuadsPerRow;
+      if (g.row0 + q > g.ns) {
+        lds.e[q][k] = zero4;
+        lds.ome[q][k] = zero4;
+      }
+    }
+  }
+  // One code path for every block: quads that reach outside the valid columns pick up
+  // neighbouring floats (or zeros past the tensor's end) that the commit masks.
+  // Always issues kBwdLoadsPerBlock loads, also for blocks in front of the first one and rows
+  // past the sequence's end (they read floats that nobody uses), so that the counts given to
+  // WaitLoads hold in every iteration.
   auto load_block = [&](int kb, BwdRegs &r) {
-    if (kb < 0) return;
-    const bool inner = interior(kb);
 #pragma unroll
     for (int it = 0; it < kLoadItems; ++it) {
       const int jd = kb * kW + 4 * mm - (lq + kRowStep * it) * g.skew;  // destination column of element 0
-      if (inner) {
-        r.d[it] = BufferQuad(rsp, idx_d[it] + jd);
-        r.s[it] = BufferQuad(rsp, idx_s[it] + jd);
-        r.x[it] = BufferQuad(rsx, idx_x[it] + jd);
-      } else {
-        const bool ok0 = jd >= 1 && jd <= g.nt, ok1 = jd + 1 >= 1 && jd + 1 <= g.nt,
-                   ok2 = jd + 2 >= 1 && jd + 2 <= g.nt, ok3 = jd + 3 >= 1 && jd + 3 <= g.nt;
-        r.d[it] = BufferFour(rsp, idx_d[it] + jd, ok0, ok1, ok2, ok3);
-        r.s[it] = BufferFour(rsp, idx_s[it] + jd, ok0, ok1, ok2, ok3);
-        r.x[it] = BufferFour(rsx, idx_x[it] + jd, ok0, ok1, ok2, ok3);
-      }
+      r.d[it] = AsyncQuad(rsp, idx_d[it] + jd);
+      r.s[it] = AsyncQuad(rsp, idx_s[it] + jd);
+      r.x[it] = AsyncQuad(rsx, idx_x[it] + jd);
     }
   };
-  // E / OME of one destination cell; pd, ps, xs = p[dest], p[src], px[src].  Select-only code: the
-  // reference's guards (k2/python/csrc/torch/mutual_information_cpu.cu:200-211) become masks.
-  auto cell = [&](bool interior_cell, bool first_row, bool last_row, int j, float pd, float ps,
-                  float xs, float *e_out, float *o_out) {
-    const float total = (pd - pd != 0.0f) ? 0.0f : pd;
+  // E / OME of a destination cell that has both edges inside the box; pd, ps, xs = p[dest],
+  // p[src], px[src] (k2/python/csrc/torch/mutual_information_cpu.cu:195-211).
+  auto flow = [&](float pd, float ps, float xs, float *e_out, float *o_out) {
+    const float total = __builtin_isfinite(pd) ? pd : 0.0f;
     const float d1 = __expf((ps + xs) - total);
-    const bool fin = d1 - d1 == 0.0f;
-    float e_v = fin ? d1 : 0.0f, o_v = fin ? 1.0f - d1 : 0.0f;
-    const bool in = interior_cell || (j >= 1 && j <= g.nt);
-    const bool col0_up = !interior_cell && j == 0 && !modified;  // regular first column flows up
-    e_v = in ? e_v : (col0_up ? 1.0f : 0.0f);
-    o_v = in ? o_v : 0.0f;
+    const bool fin = __builtin_isfinite(d1);
+    *e_out = fin ? d1 : 0.0f;
+    *o_out = fin ? 1.0f - d1 : 0.0f;
+  };
+  // The same for a cell on or outside the rim of the box (column j; select-only code).
+  auto rim = [&](bool first_row, bool last_row, int j, float *e_io, float *o_io) {
+    const bool in = j >= 1 && j <= g.nt;
+    const bool col0_up = j == 0 && !modified;  // regular first column flows up
+    float e_v = in ? *e_io : (col0_up ? 1.0f : 0.0f);
+    float o_v = in ? *o_io : 0.0f;
     // first row: everything flows along py
     e_v = first_row ? 0.0f : e_v;
     o_v = first_row ? (in ? 1.0f : 0.0f) : o_v;
     // virtual cells right of the end cell hand the seed leftwards unchanged
     const bool virt = last_row && j > g.nt;
-    e_v = virt ? 0.0f : e_v;
-    o_v = virt ? 1.0f : o_v;
-    *e_out = e_v;
-    *o_out = o_v;
+    *e_io = virt ? 0.0f : e_v;
+    *o_io = virt ? 1.0f : o_v;
   };
-  auto commit_block = [&](int kb, const BwdRegs &r) {
+  auto commit_block = [&](int kb, BwdRegs &r) {
     if (kb < 0) return;
     const bool inner = interior(kb);
 #pragma unroll
     for (int it = 0; it < kLoadItems; ++it) {
+      if (!row_ok[it]) continue;
       const int q = lq + kRowStep * it;
-      const int row_i = g.row0 + q;
-      const int jd = kb * kW + 4 * mm - q * g.skew;
-      const bool row_ok = row_i <= g.ns, first_row = row_i == 0, last_row = row_i == g.ns;
+      float4 qd = AsFloat4(r.d[it]), qs = AsFloat4(r.s[it]), qx = AsFloat4(r.x[it]);
+      if (!inner && g.b == 0) {  // the only sequence whose rows can start the tensor
+        const int jd0 = kb * kW + 4 * mm - q * g.skew;
+        qd = ShiftQuad(qd, idx_d[it] + jd0);
+        qs = ShiftQuad(qs, idx_s[it] + jd0);
+        qx = ShiftQuad(qx, idx_x[it] + jd0);
+      }
       float ve[4], vo[4];
-      cell(inner, first_row, last_row, jd + 0, r.d[it].x, r.s[it].x, r.x[it].x, &ve[0], &vo[0]);
-      cell(inner, first_row, last_row, jd + 1, r.d[it].y, r.s[it].y, r.x[it].y, &ve[1], &vo[1]);
-      cell(inner, first_row, last_row, jd + 2, r.d[it].z, r.s[it].z, r.x[it].z, &ve[2], &vo[2]);
-      cell(inner, first_row, last_row, jd + 3, r.d[it].w, r.s[it].w, r.x[it].w, &ve[3], &vo[3]);
+      flow(qd.x, qs.x, qx.x, &ve[0], &vo[0]);
+      flow(qd.y, qs.y, qx.y, &ve[1], &vo[1]);
+      flow(qd.z, qs.z, qx.z, &ve[2], &vo[2]);
+      flow(qd.w, qs.w, qx.w, &ve[3], &vo[3]);
+      if (inner) {
+        // only the sequence's first row (lane 0 of chunk 0) differs from the plain formula
+        if (it == 0 && g.row0 == 0) {
+          const bool first_row = q == 0;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        ve[e] = row_ok ? ve[e] : 0.0f;
-        vo[e] = row_ok ? vo[e] : 0.0f;
+          for (int e = 0; e < 4; ++e) {
+            ve[e] = first_row ? 0.0f : ve[e];
+            vo[e] = first_row ? 1.0f : vo[e];
+          }
+        }
+      } else {
+        const int row_i = g.row0 + q;
+        const int jd = kb * kW + 4 * mm - q * g.skew;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) rim(row_i == 0, row_i == g.ns, jd + e, &ve[e], &vo[e]);
       }
       const int pq = (kb % 3) * kQuadsPerBlock + mm;
       lds.e[q][pq] = make_float4(ve[0], ve[1], ve[2], ve[3]);
@@ -768,36 +850,52 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
   };
 
   const int top = g.nblocks - 1;
-  // loader group of block kb: (top - kb) % kGroups
-  if (role == kChain) __builtin_amdgcn_s_setprio(3);
-  BwdRegs regs;
+  BwdRegs ra, rb;
   if (role == kLoader) {
-    load_block(top - grp, regs);
-    if (grp == 0) {
-      commit_block(top, regs);
-      load_block(top - kGroups, regs);
-    }
+    load_block(top, ra);
+    WaitLoads<0>(ra);
+    commit_block(top, ra);
+    load_block(top - 1, ra);
+    load_block(top - 2, rb);
   } else if (role == kEdge) {
     take_block(top);
   }
-  __syncthreads();
+  LdsBarrier();
 
-  for (int kb = top; kb >= 0; --kb) {
-    if (role == kChain) {
+  // Descending twin of the forward's loops: in iteration kb the chain computes block kb, the
+  // loaders commit block kb-1 and start the loads of block kb-3, the storers drain block kb+1
+  // and clear a share of the rows' unassigned columns, the edge wavefront publishes block kb+1
+  // upwards and takes block kb-1 from the chunk below.
+  if (role == kChain) {
+    for (int kb = top; kb >= 0; --kb) {
       chain_block(kb);
-    } else if (role == kLoader) {
-      if (((top - kb + 1) & (kGroups - 1)) == grp) {
-        commit_block(kb - 1, regs);
-        load_block(kb - 1 - kGroups, regs);
+      LdsBarrier();
+    }
+  } else if (role == kLoader) {
+    for (int kb = top; kb >= 0; kb -= 2) {
+      WaitLoads<kBwdLoadsPerBlock>(ra);  // the other set's loads may stay in flight
+      commit_block(kb - 1, ra);
+      load_block(kb - 3, ra);
+      LdsBarrier();
+      if (kb - 1 >= 0) {
+        WaitLoads<kBwdLoadsPerBlock>(rb);
+        commit_block(kb - 2, rb);
+        load_block(kb - 4, rb);
+        LdsBarrier();
       }
-    } else if (role == kStorer) {
+    }
+  } else if (role == kStorer) {
+    for (int kb = top; kb >= 0; --kb) {
       store_block(kb + 1);
       zero_slices(top - kb);
-    } else {
+      LdsBarrier();
+    }
+  } else {
+    for (int kb = top; kb >= 0; --kb) {
       publish_block(kb + 1);
       take_block(kb - 1);
+      LdsBarrier();
     }
-    __syncthreads();
   }
   if (role == kStorer) store_block(0);
   if (role == kEdge) publish_block(0);
