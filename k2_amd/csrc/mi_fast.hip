@@ -82,31 +82,29 @@ __device__ __forceinline__ float NegInfF() { return -__builtin_huge_valf(); }
 constexpr float kLogZero = -1.0e30f;
 constexpr float kLogZeroTest = -1.0e29f;  // anything below counts as -inf when p leaves the chain
 
-// value of lane l+1 (lane 63 keeps `keep`)
-__device__ __forceinline__ float WaveShl1(float keep, float v) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(keep), __float_as_int(v), 0x130,
-                                                    0xf, 0xf, false));
-}
-
-// log(exp(a) + exp(b)) for FINITE a, b on the fast transcendental units: max + log1p(exp(-|a-b|)).
-// Matches k2's log-add to within one fp32 rounding of the larger operand: where k2 drops the
-// smaller term (difference below log(eps)) the correction computed here is below 1.2e-7.
-// Dependent chain: sub, mul (|.| and negation are free source modifiers), exp2, add, log2, fma.
-__device__ __forceinline__ float LogAddFinite(float a, float b) {
-  const float mx = __builtin_fmaxf(a, b);  // off the critical path
-  const float e = __builtin_amdgcn_exp2f(-__builtin_fabsf(a - b) * kLog2e);
+// One step of the forward chain for every row (lane) of the chunk:
+//     x   = P + fy                       the path arriving along py (same row, previous column)
+//     inc = P(lane - 1) + fx             the path arriving along px (row above); lane 0, which
+//                                        has no lane above it, takes `lane0_inc` instead
+//     P'  = log(exp(inc) + exp(x)) = max + log2(1 + exp2(-|inc - x| log2e)) ln2   on the fast
+//           transcendental units.  All values are finite (see kLogZero).  This matches k2's
+//           log-add to within one fp32 rounding of the larger operand: where k2 drops the
+//           smaller term (difference below log(eps)) the correction computed here is < 1.2e-7.
+// The first half is spelled out in assembly: the DPP add needs two wait states after the VALU
+// write of P (the add of x and one s_nop provide them; the compiler's hazard recogniser does
+// not look inside), and v_max_f32 on known-finite numbers needs no canonicalising pre-pass.
+__device__ __forceinline__ float ChainStep(float P, float fx, float fy, float lane0_inc) {
+  float x, mx, d, inc = lane0_inc;
+  asm volatile(
+      "v_add_f32 %[x], %[P], %[fy]\n\t"
+      "s_nop 0\n\t"
+      "v_add_f32_dpp %[inc], %[P], %[fx] wave_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32 %[mx], %[inc], %[x]\n\t"
+      "v_sub_f32 %[d], %[inc], %[x]"
+      : [x] "=&v"(x), [inc] "+&v"(inc), [mx] "=&v"(mx), [d] "=&v"(d)
+      : [P] "v"(P), [fx] "v"(fx), [fy] "v"(fy));
+  const float e = __builtin_amdgcn_exp2f(-__builtin_fabsf(d) * kLog2e);
   return __builtin_fmaf(__builtin_amdgcn_logf(1.0f + e), kLn2, mx);
-}
-
-// lane l gets  P(lane l-1) + add ; lane 0, which has no lane below it, keeps `lane0`.
-__device__ __forceinline__ float ShiftAdd(float lane0, float P, float add) {
-  float r = lane0;
-  // a DPP source written by the preceding VALU instruction needs two wait states; inline
-  // assembly is opaque to the compiler's hazard recogniser, so they are spelled out here
-  asm volatile("s_nop 1\n\tv_add_f32_dpp %0, %1, %2 wave_shr:1 row_mask:0xf bank_mask:0xf"
-               : "+v"(r)
-               : "v"(P), "v"(add));
-  return r;
 }
 
 __device__ __forceinline__ void StoreQuad(float *ptr, float4 v) {
@@ -123,7 +121,10 @@ __device__ __forceinline__ void StoreQuad(float *ptr, float4 v) {
 // a block's loads have to stay in flight across two loop iterations, and the compiler's own
 // wait-count insertion falls back to "wait for everything" for loads carried around a loop,
 // which would stall every iteration for a full memory round trip.  The loader loop issues no
-// other vector memory operation, so the counts below are exact.
+// other vector memory operation, so the counts below are exact.  Two rules keep this sound:
+// every register set is drained with WaitLoads<0> before it goes out of scope (a load that
+// lands later would overwrite whatever the compiler has put into its registers by then), and
+// nothing reads or copies a set between AsyncQuad and the WaitLoads that covers it.
 typedef int int4v __attribute__((ext_vector_type(4)));
 typedef float float4v __attribute__((ext_vector_type(4)));
 
@@ -444,9 +445,7 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
       float out[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const float x = P + fys[e];                              // arriving along py
-        const float inc = ShiftAdd(uis[e] + fxs[e], P, fxs[e]);  // arriving along px
-        P = LogAddFinite(inc, x);
+        P = ChainStep(P, fxs[e], fys[e], uis[e] + fxs[e]);
         out[e] = P;
       }
       lds.fy[lane][base + k] = make_float4(out[0], out[1], out[2], out[3]);
@@ -491,6 +490,10 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
         LdsBarrier();
       }
     }
+    // the loads of the blocks past the end are still in flight: they must land before the
+    // compiler may give their registers to anything else
+    WaitLoads<0>(ra);
+    WaitLoads<0>(rb);
   } else if (role == kStorer) {
     for (int kb = 0; kb < g.nblocks; ++kb) {
       store_block(kb - 1);
@@ -588,9 +591,15 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
   const unsigned total_wgs = gridDim.x;
   if (threadIdx.x == 0) lds.ticket = atomicAdd(&hdr->ticket, 1u);
   __syncthreads();
+  // The first B * nchunks tickets sweep; the rest of the grid (as many again) clears what the
+  // sweep does not assign, one workgroup per (sequence, 64 array rows), on compute units the
+  // sweep leaves idle and off its critical path.
+  const unsigned nsweep = (unsigned)B * nchunks;
+  const bool zero_only = lds.ticket >= nsweep;
+  const unsigned unit = zero_only ? lds.ticket - nsweep : lds.ticket;
   ChunkGeom g;
-  g.b = lds.ticket / nchunks;
-  g.c = nchunks - 1 - (int)(lds.ticket % nchunks);  // lower chunks take earlier tickets
+  g.b = unit / nchunks;
+  g.c = nchunks - 1 - (int)(unit % nchunks);  // lower chunks take earlier tickets
   const Box box = LoadBox(boundary, g.b, S, Tn);
   const int T1 = modified ? Tn : Tn + 1;
   const int off = modified ? -1 : 0;
@@ -599,24 +608,23 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
   float *gxb = px_grad + (size_t)g.b * S * T1;
   float *gyb = py_grad + (size_t)g.b * (S + 1) * Tn;
 
-  // Everything the sweep does not assign is zero.  Each workgroup owns 64 ARRAY rows
-  // (independent of the box) and clears them in slices of 32 columns, spread over the pipeline
-  // iterations so that the clearing hides behind the sweep.
-  ZeroGeom zg;
-  zg.gx = gxb; zg.gy = gyb; zg.S = S; zg.T1 = T1; zg.Tn = Tn;
-  zg.xs0 = box.ok ? box.s0 : 0; zg.xs1 = box.ok ? box.s1 : 0;
-  zg.xt0 = box.ok ? box.t0 : 0; zg.xt1 = box.ok ? box.t1 + off + 1 : 0;
-  zg.ys1 = box.ok ? box.s1 + 1 : 0; zg.yt1 = box.ok ? box.t1 : 0;
-  const int zr_lo = g.c * kRows;
-  const int zslices = (T1 + 31) / 32;
+  if (zero_only) {
+    ZeroGeom zg;
+    zg.gx = gxb; zg.gy = gyb; zg.S = S; zg.T1 = T1; zg.Tn = Tn;
+    zg.xs0 = box.ok ? box.s0 : 0; zg.xs1 = box.ok ? box.s1 : 0;
+    zg.xt0 = box.ok ? box.t0 : 0; zg.xt1 = box.ok ? box.t1 + off + 1 : 0;
+    zg.ys1 = box.ok ? box.s1 + 1 : 0; zg.yt1 = box.ok ? box.t1 : 0;
+    const int zslices = (T1 + 31) / 32;
+    if (threadIdx.x < kRows * 8)
+      for (int sl = 0; sl < zslices; ++sl)
+        ZeroItem(zg, g.c * kRows + (threadIdx.x >> 3), sl * 32 + 4 * (threadIdx.x & 7));
+    if (threadIdx.x == 0) FinishWorkgroup(hdr, total_wgs);
+    return;
+  }
 
   g.s0 = box.s0; g.t0 = box.t0; g.ns = box.s1 - box.s0; g.nt = box.t1 - box.t0;
   g.row0 = g.c * kRows;
-  if (!box.ok || g.row0 > g.ns) {
-    // nothing to sweep: clear the rows and leave
-    if (threadIdx.x < kRows * 8)
-      for (int sl = 0; sl < zslices; ++sl)
-        ZeroItem(zg, zr_lo + (threadIdx.x >> 3), sl * 32 + 4 * (threadIdx.x & 7));
+  if (!box.ok || g.row0 > g.ns) {  // nothing to sweep
     if (threadIdx.x == 0) FinishWorkgroup(hdr, total_wgs);
     return;
   }
@@ -628,7 +636,6 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
   const int edge_shift = kRows * g.skew;  // position m here <-> position m - edge_shift one chunk down
   float *edge_out = edge + ((size_t)g.b * nchunks + g.c) * edge_stride;     // read by chunk c-1
   float *edge_in = edge + ((size_t)g.b * nchunks + g.c + 1) * edge_stride;  // from chunk c+1
-  const int zper = (zslices + g.nblocks - 1) / g.nblocks;  // slices cleared per iteration
 
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int role = RoleOf(wave);
@@ -785,12 +792,6 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
       }
     }
   };
-  auto zero_slices = [&](int it) {
-    for (int sl = it * zper; sl < min((it + 1) * zper, zslices); ++sl) {
-      ZeroItem(zg, zr_lo + mq, sl * 32 + 4 * mm);
-      ZeroItem(zg, zr_lo + mq + 32, sl * 32 + 4 * mm);
-    }
-  };
 
   // ---- edge wavefront ----------------------------------------------------------------------
   auto take_block = [&](int kb) {
@@ -819,30 +820,43 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
   float G = 0.0f;
   if (role == kChain && g.row0 + lane == g.ns) G = ans_grad[g.b];
   float g_origin = 0.0f;
+  // Per position (descending): with E, OME of the own row and Edn = E of the row below (lane+1),
+  //     h = E * G;  c = OME * G;                      -> px_grad, py_grad of this cell
+  //     G' = OME * G + Edn * G(lane + 1)              = c + h(lane + 1)
+  // where lane 63 takes, in place of the product, the h arriving from the chunk below (the DPP's
+  // "old" operand).  The two output multiplies sit between the write of G and its DPP read and
+  // provide the wait states that read needs.
+  const int lane_dn = min(lane + 1, kWave - 1);
   auto chain_block = [&](int kb) {
     const int base = (kb % 3) * kQuadsPerBlock;
-    float4 ne = lds.e[lane][base + kQuadsPerBlock - 1],
+    float4 ne = lds.e[lane][base + kQuadsPerBlock - 1], nd = lds.e[lane_dn][base + kQuadsPerBlock - 1],
            no = lds.ome[lane][base + kQuadsPerBlock - 1], nr = lds.rin[base + kQuadsPerBlock - 1];
 #pragma unroll
     for (int k = kQuadsPerBlock - 1; k >= 0; --k) {
-      const float4 e4 = ne, o4 = no, r4 = nr;
+      const float4 e4 = ne, d4 = nd, o4 = no, r4 = nr;
       if (k > 0) {
         ne = lds.e[lane][base + k - 1];
+        nd = lds.e[lane_dn][base + k - 1];
         no = lds.ome[lane][base + k - 1];
         nr = lds.rin[base + k - 1];
       }
       const float es[4] = {e4.x, e4.y, e4.z, e4.w};
+      const float ds[4] = {d4.x, d4.y, d4.z, d4.w};
       const float os[4] = {o4.x, o4.y, o4.z, o4.w};
       const float rs4[4] = {r4.x, r4.y, r4.z, r4.w};
       float hs[4], cs[4];
 #pragma unroll
       for (int e = 3; e >= 0; --e) {
         if (kb == 0 && k == 0 && e == 0) g_origin = G;
-        const float h = es[e] * G;
-        const float c = os[e] * G;
-        G = WaveShl1(rs4[e], h) + c;  // lane 63 takes the h arriving from the chunk below
-        hs[e] = h;
-        cs[e] = c;
+        float t = rs4[e];
+        asm volatile(
+            "v_mul_f32 %[h], %[E], %[G]\n\t"
+            "v_mul_f32 %[c], %[O], %[G]\n\t"
+            "v_mul_f32_dpp %[t], %[G], %[D] wave_shl:1 row_mask:0xf bank_mask:0xf\n\t"
+            "v_fmac_f32 %[t], %[O], %[G]"
+            : [h] "=&v"(hs[e]), [c] "=&v"(cs[e]), [t] "+&v"(t)
+            : [E] "v"(es[e]), [O] "v"(os[e]), [D] "v"(ds[e]), [G] "v"(G));
+        G = t;
       }
       lds.e[lane][base + k] = make_float4(hs[0], hs[1], hs[2], hs[3]);
       lds.ome[lane][base + k] = make_float4(cs[0], cs[1], cs[2], cs[3]);
@@ -863,9 +877,8 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
   LdsBarrier();
 
   // Descending twin of the forward's loops: in iteration kb the chain computes block kb, the
-  // loaders commit block kb-1 and start the loads of block kb-3, the storers drain block kb+1
-  // and clear a share of the rows' unassigned columns, the edge wavefront publishes block kb+1
-  // upwards and takes block kb-1 from the chunk below.
+  // loaders commit block kb-1 and start the loads of block kb-3, the storers drain block kb+1,
+  // the edge wavefront publishes block kb+1 upwards and takes block kb-1 from the chunk below.
   if (role == kChain) {
     for (int kb = top; kb >= 0; --kb) {
       chain_block(kb);
@@ -884,10 +897,13 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
         LdsBarrier();
       }
     }
+    // the loads of the blocks in front of the first one are still in flight: they must land
+    // before the compiler may give their registers to anything else
+    WaitLoads<0>(ra);
+    WaitLoads<0>(rb);
   } else if (role == kStorer) {
     for (int kb = top; kb >= 0; --kb) {
       store_block(kb + 1);
-      zero_slices(top - kb);
       LdsBarrier();
     }
   } else {
@@ -949,7 +965,8 @@ int MiBackwardFast(const float *px, const float *p, const int64_t *boundary, flo
   const int edge_stride = (int)(((size_t)Tn + 2 + kRows + kW + 3) / 4 * 4 + kW);
   FastHeader *hdr = static_cast<FastHeader *>(workspace);
   float *edge = reinterpret_cast<float *>(hdr + 1);
-  hipLaunchKernelGGL(MiBackwardFastKernel, dim3((unsigned)(B * nchunks)), dim3(kFastThreads), 0, stream,
+  // B * nchunks sweeping workgroups + as many that only clear
+  hipLaunchKernelGGL(MiBackwardFastKernel, dim3((unsigned)(2 * B * nchunks)), dim3(kFastThreads), 0, stream,
                      px, p, boundary, ans_grad, px_grad, py_grad, hdr, edge, B, S, Tn, modified,
                      nchunks, edge_stride, overwrite_ans_grad);
   return LaunchStatus();
