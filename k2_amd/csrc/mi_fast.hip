@@ -5,8 +5,8 @@
 // HBM bandwidth from several compute units (a single workgroup tops out near 100 GB/s on this
 // part; 32 sequences alone could never fill 8 TB/s).
 //
-// Inside a workgroup (ten wavefronts, each with one job, so that no wavefront that loads ever
-// has to wait for a store to be acknowledged):
+// Inside a workgroup (twelve wavefronts, each with one job or none, so that no wavefront that
+// loads ever has to wait for a store to be acknowledged):
 //   * one CHAIN wavefront carries the recursion, lane = lattice row.  Lane q works on column
 //     j = n - q*skew at step n (skew = 1 for the regular lattice, 0 for the modified one), so
 //     every cell depends on the previous step only: its own lane's value and the neighbouring
@@ -20,7 +20,10 @@
 //   * four STORER wavefronts drain the ring: results leave as contiguous row segments.
 //   * one EDGE wavefront takes the words published by the adjacent chunk and publishes this
 //     chunk's boundary row.
-//   * one barrier per block of 32 steps.
+//   * two IDLE wavefronts that only join the barriers: they occupy the slots of the chain
+//     wavefront's SIMD, which the chain then has to itself.
+//   * one barrier per block of 32 steps; it orders LDS traffic only, so global loads and stores
+//     stay in flight across it.
 //
 // Between workgroups: the boundary row of a chunk is published per step into a small edge buffer
 // in global memory with device-scope atomic stores; the adjacent chunk polls those words until
@@ -46,7 +49,11 @@ constexpr int kRing = 3 * kW;       // ring positions per row
 constexpr int kStride = kRing + 4;  // floats per LDS row; +4 spreads lanes over banks
 constexpr int kMoverWaves = 4;      // loader wavefronts, and as many storer wavefronts
 constexpr int kMoverLanes = kWave * kMoverWaves;
-constexpr int kFastThreads = kWave * (2 + 2 * kMoverWaves);  // chain + edge + loaders + storers
+// Wavefronts of a workgroup are spread round-robin over the compute unit's four SIMDs.  The chain
+// wavefront (wave 0) is the critical path of the whole kernel, so the two other wavefronts that
+// land on its SIMD (waves 4 and 8) stay idle: they only take part in the barriers.
+constexpr int kIdleWaves = 2;
+constexpr int kFastThreads = kWave * (2 + kIdleWaves + 2 * kMoverWaves);
 constexpr unsigned kSentinel = 0x7fc5a5a5u;  // a quiet-NaN pattern arithmetic never produces
 constexpr int kSpinLimit = 1 << 20;
 constexpr float kLog2e = 1.44269504088896340736f;
@@ -179,11 +186,21 @@ struct ChunkGeom {
   int nblocks;
 };
 
-enum Role { kChain = 0, kEdge = 1, kLoader = 2, kStorer = 3 };
+enum Role { kChain = 0, kEdge = 1, kLoader = 2, kStorer = 3, kIdle = 4 };
 
+// wave:   0      1     2  3  4     5  6  7  8     9  10 11
+// role:   chain  edge  L0 L1 idle  L2 L3 S0 idle  S1 S2 S3
 __device__ __forceinline__ int RoleOf(int wave) {
-  return wave == 0 ? kChain : (wave == 1 ? kEdge : (wave < 2 + kMoverWaves ? kLoader : kStorer));
+  if (wave == 0) return kChain;
+  if (wave == 1) return kEdge;
+  if (wave == 4 || wave == 8) return kIdle;
+  return wave < 7 ? kLoader : kStorer;
 }
+// index of a loader (or storer) wavefront among its kind, 0..kMoverWaves-1
+__device__ __forceinline__ int MoverIndex(int wave) {
+  return wave < 7 ? (wave < 4 ? wave - 2 : wave - 3) : (wave == 7 ? 0 : wave - 8);
+}
+static_assert(kMoverWaves == 4 && kIdleWaves == 2, "the wave table above is written for 12 wavefronts");
 
 __global__ void FastWsInitKernel(FastHeader *hdr, unsigned *edge, size_t n) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -298,8 +315,7 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int role = RoleOf(wave);
   // movers: lane id within the loader (or storer) wavefronts
-  const int mid = (threadIdx.x - (role == kStorer ? kWave * (2 + kMoverWaves) : 2 * kWave)) &
-                  (kMoverLanes - 1);
+  const int mid = (MoverIndex(wave) * kWave + lane) & (kMoverLanes - 1);
   const int mq = mid >> 3, mm = mid & 7;  // storers: rows mq and mq + 32, quad mm
   const int lq = mq;                      // loaders: rows lq + kRowStep*it, quad mm
 
@@ -499,12 +515,14 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
       store_block(kb - 1);
       LdsBarrier();
     }
-  } else {
+  } else if (role == kEdge) {
     for (int kb = 0; kb < g.nblocks; ++kb) {
       publish_block(kb - 1);
       take_block(kb + 1);
       LdsBarrier();
     }
+  } else {
+    for (int kb = 0; kb < g.nblocks; ++kb) LdsBarrier();
   }
   if (role == kStorer) store_block(g.nblocks - 1);
   if (role == kEdge) publish_block(g.nblocks - 1);
@@ -639,8 +657,7 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
 
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int role = RoleOf(wave);
-  const int mid = (threadIdx.x - (role == kStorer ? kWave * (2 + kMoverWaves) : 2 * kWave)) &
-                  (kMoverLanes - 1);
+  const int mid = (MoverIndex(wave) * kWave + lane) & (kMoverLanes - 1);
   const int mq = mid >> 3, mm = mid & 7;  // storers: rows mq and mq + 32, quad mm
   const int lq = mq;                      // loaders: rows lq + kRowStep*it, quad mm
 
@@ -906,12 +923,14 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
       store_block(kb + 1);
       LdsBarrier();
     }
-  } else {
+  } else if (role == kEdge) {
     for (int kb = top; kb >= 0; --kb) {
       publish_block(kb + 1);
       take_block(kb - 1);
       LdsBarrier();
     }
+  } else {
+    for (int kb = top; kb >= 0; --kb) LdsBarrier();
   }
   if (role == kStorer) store_block(0);
   if (role == kEdge) publish_block(0);
