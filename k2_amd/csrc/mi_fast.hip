@@ -91,8 +91,9 @@ constexpr float kLogZeroTest = -1.0e29f;  // anything below counts as -inf when 
 
 // One step of the forward chain for every row (lane) of the chunk:
 //     x   = P + fy                       the path arriving along py (same row, previous column)
-//     inc = P(lane - 1) + fx             the path arriving along px (row above); lane 0, which
-//                                        has no lane above it, takes `lane0_inc` instead
+//     inc = P(lane - 1) + fx             the path arriving along px (row above); lane 0 has no
+//                                        lane above it: the DPP add leaves its register alone,
+//                                        so its `fx` must already be that whole sum
 //     P'  = log(exp(inc) + exp(x)) = max + log2(1 + exp2(-|inc - x| log2e)) ln2   on the fast
 //           transcendental units.  All values are finite (see kLogZero).  This matches k2's
 //           log-add to within one fp32 rounding of the larger operand: where k2 drops the
@@ -100,16 +101,16 @@ constexpr float kLogZeroTest = -1.0e29f;  // anything below counts as -inf when 
 // The first half is spelled out in assembly: the DPP add needs two wait states after the VALU
 // write of P (the add of x and one s_nop provide them; the compiler's hazard recogniser does
 // not look inside), and v_max_f32 on known-finite numbers needs no canonicalising pre-pass.
-__device__ __forceinline__ float ChainStep(float P, float fx, float fy, float lane0_inc) {
-  float x, mx, d, inc = lane0_inc;
+__device__ __forceinline__ float ChainStep(float P, float fx, float fy) {
+  float x, mx, d, inc = fx;
   asm volatile(
       "v_add_f32 %[x], %[P], %[fy]\n\t"
       "s_nop 0\n\t"
-      "v_add_f32_dpp %[inc], %[P], %[fx] wave_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+      "v_add_f32_dpp %[inc], %[P], %[inc] wave_shr:1 row_mask:0xf bank_mask:0xf\n\t"
       "v_max_f32 %[mx], %[inc], %[x]\n\t"
       "v_sub_f32 %[d], %[inc], %[x]"
       : [x] "=&v"(x), [inc] "+&v"(inc), [mx] "=&v"(mx), [d] "=&v"(d)
-      : [P] "v"(P), [fx] "v"(fx), [fy] "v"(fy));
+      : [P] "v"(P), [fy] "v"(fy));
   const float e = __builtin_amdgcn_exp2f(-__builtin_fabsf(d) * kLog2e);
   return __builtin_fmaf(__builtin_amdgcn_logf(1.0f + e), kLn2, mx);
 }
@@ -257,11 +258,11 @@ __device__ __forceinline__ void PublishEdge(float *addr, float v) {
 //     fx[q][n] = px[row-1][jp + skew]   (the px edge arriving from the row above)
 //     fy[q][n] = py[row][jp]            (the py edge arriving from the left),  jp = j - 1
 // and receives p[row][j] in place of fy once the step is done.  Lane 0's "row above" is the
-// last row of the chunk above; its p arrives through uin[n].
+// last row of the chunk above: the edge wavefront adds that row's p and px and stores the sum
+// in row 64 of fx.
 struct FwdLds {
-  float4 fx[kWave][kQuadsPerRow];
+  float4 fx[kWave + 1][kQuadsPerRow];  // row 64: see below
   float4 fy[kWave][kQuadsPerRow];
-  float4 uin[kRing / 4];
   unsigned ticket;
 };
 
@@ -374,8 +375,6 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
         vx[e] = okx ? fmaxf(vx[e], kLogZero) : kLogZero;
         vy[e] = oky ? fmaxf(vy[e], kLogZero) : kLogZero;
       }
-      // the origin: p[s_begin][t_begin] = 0 enters as "0 arriving from above" at step 0
-      if (g.row0 + q == 0 && kb == 0 && mm == 0) vx[0] = 0.0f;
       const int pq = (kb % 3) * kQuadsPerBlock + mm;
       lds.fx[q][pq] = make_float4(vx[0], vx[1], vx[2], vx[3]);
       lds.fy[q][pq] = make_float4(vy[0], vy[1], vy[2], vy[3]);
@@ -415,18 +414,29 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
   };
 
   // ---- edge wavefront ----------------------------------------------------------------------
-  // lanes 0..31: p of the row above lane 0 for block kb
-  auto take_block = [&](int kb) {
+  // Lanes 0..31 prepare, for each step n of block kb, what arrives at lane 0 along px:
+  //     p[row0-1][..] (taken from the chunk above) + px[row0-1][..]
+  // and put it into row 64 of the fx array, which lane 0 of the chain reads in place of a row of
+  // its own (the DPP add of the chain step leaves lane 0's register as it is).  The px values
+  // are loaded by this wavefront itself, one block ahead.
+  auto edge_px = [&](int kb) -> float {
+    const int jx = kb * kW + lane - 1 + g.skew;
+    float v = kLogZero;
+    if (g.c > 0 && lane < kW && jx >= 0 && jx <= hi_x)
+      v = fmaxf(pxb[(size_t)(g.s0 + g.row0 - 1) * T1 + g.t0 + jx], kLogZero);
+    return v;
+  };
+  auto take_block = [&](int kb, float px_above) {
     if (lane < kW && kb < g.nblocks) {
       const int n = kb * kW + lane;
       float v = kLogZero;
       if (g.c == 0) {
-        if (n == 0) v = 0.0f;  // pairs with the 0 placed in fx[0][0]
+        if (n == 0) v = 0.0f;  // the origin: p[s_begin][t_begin] = 0 "arrives" at step 0
       } else {
         const int idx = n + edge_shift;
-        if (idx >= 0 && idx < g.nblocks * kW) v = TakeEdge(edge_in + idx, hdr, kLogZero);
+        if (idx >= 0 && idx < g.nblocks * kW) v = TakeEdge(edge_in + idx, hdr, kLogZero) + px_above;
       }
-      reinterpret_cast<float *>(lds.uin)[(kb % 3) * kW + lane] = v;
+      reinterpret_cast<float *>(lds.fx[kWave])[(kb % 3) * kW + lane] = v;
     }
   };
   // lanes 32..63: hand block kb of the last row to the chunk below.  Only words the chunk below
@@ -443,25 +453,24 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
 
   // ---- chain wavefront ---------------------------------------------------------------------
   float P = kLogZero;
+  const int fx_row = lane == 0 ? kWave : lane;
   auto chain_block = [&](int kb) {
     const int base = (kb % 3) * kQuadsPerBlock;
     P = fmaxf(P, -1.0e36f);  // lanes idling on the stand-in for -inf must never reach -inf itself
-    float4 nfx = lds.fx[lane][base], nfy = lds.fy[lane][base], nu = lds.uin[base];
+    float4 nfx = lds.fx[fx_row][base], nfy = lds.fy[lane][base];
 #pragma unroll
     for (int k = 0; k < kQuadsPerBlock; ++k) {
-      const float4 fx4 = nfx, fy4 = nfy, u4 = nu;
+      const float4 fx4 = nfx, fy4 = nfy;
       if (k + 1 < kQuadsPerBlock) {
-        nfx = lds.fx[lane][base + k + 1];
+        nfx = lds.fx[fx_row][base + k + 1];
         nfy = lds.fy[lane][base + k + 1];
-        nu = lds.uin[base + k + 1];
       }
       const float fxs[4] = {fx4.x, fx4.y, fx4.z, fx4.w};
       const float fys[4] = {fy4.x, fy4.y, fy4.z, fy4.w};
-      const float uis[4] = {u4.x, u4.y, u4.z, u4.w};
       float out[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        P = ChainStep(P, fxs[e], fys[e], uis[e] + fxs[e]);
+        P = ChainStep(P, fxs[e], fys[e]);
         out[e] = P;
       }
       lds.fy[lane][base + k] = make_float4(out[0], out[1], out[2], out[3]);
@@ -479,7 +488,7 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
     load_block(1, ra);
     load_block(2, rb);
   } else if (role == kEdge) {
-    take_block(0);
+    take_block(0, edge_px(0));
   }
   LdsBarrier();
 
@@ -516,9 +525,12 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
       LdsBarrier();
     }
   } else if (role == kEdge) {
+    float px_above = edge_px(1);
     for (int kb = 0; kb < g.nblocks; ++kb) {
       publish_block(kb - 1);
-      take_block(kb + 1);
+      const float px_next = edge_px(kb + 2);
+      take_block(kb + 1, px_above);
+      px_above = px_next;
       LdsBarrier();
     }
   } else {
@@ -544,9 +556,10 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
 // has no lane above it in the wavefront and receives, through the DPP's "old" operand, the h of
 // the first row of the chunk below, so here the LOWER chunk runs ahead.
 struct BwdLds {
-  float4 e[kWave][kQuadsPerRow];    // d1 on the way in, h (px_grad) on the way out
+  // rows 0..63: d1 on the way in, h (px_grad) on the way out; row 64: the h arriving from the
+  // chunk below, laid out like a row so that every lane reads "the row below it" the same way
+  float4 e[kWave + 1][kQuadsPerRow];
   float4 ome[kWave][kQuadsPerRow];  // 1 - d1 on the way in, c (py_grad) on the way out
-  float4 rin[kRing / 4];            // h arriving from the chunk below
   unsigned ticket;
 };
 
@@ -819,7 +832,7 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
         const int idx = mpos - edge_shift;  // position of the same column in the chunk below
         if (idx >= 0) v = TakeEdge(edge_in + idx, hdr, 0.0f);
       }
-      reinterpret_cast<float *>(lds.rin)[(kb % 3) * kW + lane] = v;
+      reinterpret_cast<float *>(lds.e[kWave])[(kb % 3) * kW + lane] = v;
     }
   };
   // only words the chunk above will take are published (positions it maps inside its range)
@@ -840,39 +853,37 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
   // Per position (descending): with E, OME of the own row and Edn = E of the row below (lane+1),
   //     h = E * G;  c = OME * G;                      -> px_grad, py_grad of this cell
   //     G' = OME * G + Edn * G(lane + 1)              = c + h(lane + 1)
-  // where lane 63 takes, in place of the product, the h arriving from the chunk below (the DPP's
-  // "old" operand).  The two output multiplies sit between the write of G and its DPP read and
-  // provide the wait states that read needs.
-  const int lane_dn = min(lane + 1, kWave - 1);
+  // Lane 63 has no lane below it: the DPP multiply leaves its register untouched, and what that
+  // register holds is row 64 of the E array, the h arriving from the chunk below.  The two output
+  // multiplies sit between the write of G and its DPP read and provide the wait states that
+  // read needs.
   auto chain_block = [&](int kb) {
     const int base = (kb % 3) * kQuadsPerBlock;
-    float4 ne = lds.e[lane][base + kQuadsPerBlock - 1], nd = lds.e[lane_dn][base + kQuadsPerBlock - 1],
-           no = lds.ome[lane][base + kQuadsPerBlock - 1], nr = lds.rin[base + kQuadsPerBlock - 1];
+    float4 ne = lds.e[lane][base + kQuadsPerBlock - 1], nd = lds.e[lane + 1][base + kQuadsPerBlock - 1],
+           no = lds.ome[lane][base + kQuadsPerBlock - 1];
 #pragma unroll
     for (int k = kQuadsPerBlock - 1; k >= 0; --k) {
-      const float4 e4 = ne, d4 = nd, o4 = no, r4 = nr;
+      const float4 e4 = ne, d4 = nd, o4 = no;
       if (k > 0) {
         ne = lds.e[lane][base + k - 1];
-        nd = lds.e[lane_dn][base + k - 1];
+        nd = lds.e[lane + 1][base + k - 1];
         no = lds.ome[lane][base + k - 1];
-        nr = lds.rin[base + k - 1];
       }
       const float es[4] = {e4.x, e4.y, e4.z, e4.w};
       const float ds[4] = {d4.x, d4.y, d4.z, d4.w};
       const float os[4] = {o4.x, o4.y, o4.z, o4.w};
-      const float rs4[4] = {r4.x, r4.y, r4.z, r4.w};
       float hs[4], cs[4];
 #pragma unroll
       for (int e = 3; e >= 0; --e) {
         if (kb == 0 && k == 0 && e == 0) g_origin = G;
-        float t = rs4[e];
+        float t = ds[e];
         asm volatile(
             "v_mul_f32 %[h], %[E], %[G]\n\t"
             "v_mul_f32 %[c], %[O], %[G]\n\t"
-            "v_mul_f32_dpp %[t], %[G], %[D] wave_shl:1 row_mask:0xf bank_mask:0xf\n\t"
+            "v_mul_f32_dpp %[t], %[G], %[t] wave_shl:1 row_mask:0xf bank_mask:0xf\n\t"
             "v_fmac_f32 %[t], %[O], %[G]"
             : [h] "=&v"(hs[e]), [c] "=&v"(cs[e]), [t] "+&v"(t)
-            : [E] "v"(es[e]), [O] "v"(os[e]), [D] "v"(ds[e]), [G] "v"(G));
+            : [E] "v"(es[e]), [O] "v"(os[e]), [G] "v"(G));
         G = t;
       }
       lds.e[lane][base + k] = make_float4(hs[0], hs[1], hs[2], hs[3]);
