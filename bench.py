@@ -57,12 +57,124 @@ def cpu_baseline(c, budget_s=12.0):
     }
 
 
+def _cpu_pruned_loss(logits, symbols, ranges, boundary, blank=0):
+    """k2's CPU route for rnnt_loss_pruned, restated with torch CPU ops (the reference is a chain
+    of torch ops, k2/python/k2/rnnt_loss.py:1180-1348, around its CPU recursion
+    k2/python/csrc/torch/mutual_information_cpu.cu): log-softmax, gathers, dense px / py with -inf
+    outside the band, the CPU lattice recursion, autograd back to the logits."""
+    import torch
+    from oracle import mi as omi
+    backend = "ref" if omi.have_ref() else "port"
+    B, T, R, C = logits.shape
+    S = symbols.shape[1]
+
+    class Lattice(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, px, py):
+            npx, npy = px.detach().numpy(), py.detach().numpy()
+            ans, p = omi.mi_forward(npx, npy, boundary.numpy(), backend=backend)
+            gx, gy = omi.mi_backward(npx, npy, boundary.numpy(), p, backend=backend)
+            ctx.save_for_backward(torch.from_numpy(gx), torch.from_numpy(gy))
+            return torch.from_numpy(ans)
+
+        @staticmethod
+        def backward(ctx, g):
+            gx, gy = ctx.saved_tensors
+            return gx * g.reshape(-1, 1, 1), gy * g.reshape(-1, 1, 1)
+
+    lp = torch.log_softmax(logits, dim=-1)
+    s_idx = ranges  # [B,T,R] = s of each kept row
+    sym_pad = torch.cat([symbols, torch.full((B, 1), blank, dtype=symbols.dtype)], dim=1)
+    sym = torch.gather(sym_pad.unsqueeze(1).expand(B, T, S + 1), 2, s_idx)          # [B,T,R]
+    px_band = torch.gather(lp, 3, sym.unsqueeze(-1)).squeeze(-1)                     # [B,T,R]
+    py_band = lp[..., blank]                                                         # [B,T,R]
+    t_end = boundary[:, 3].reshape(B, 1, 1)
+    t_idx = torch.arange(T).reshape(1, T, 1)
+    px_band = torch.where((s_idx < S) & (t_idx != t_end), px_band, torch.full_like(px_band, float("-inf")))
+    px = torch.full((B, T, S + 1), float("-inf")).scatter(2, s_idx, px_band)[:, :, :S]
+    py = torch.full((B, T, S + 1), float("-inf")).scatter(2, s_idx, py_band)
+    px = torch.cat([px.permute(0, 2, 1), torch.full((B, S, 1), float("-inf"))], dim=2).contiguous()
+    py = py.permute(0, 2, 1).contiguous()
+    return -Lattice.apply(px, py).sum()
+
+
+def pruned_secondary(dev, steps=20, cpu=True):
+    """Second figure asked for next to the headline: pruned RNN-T loss forward + backward on
+    BASELINE config 3 (B=32, T=500, S=100, V=500, s_range=5, regular lattice) in utterances/s,
+    beside the CPU route on a sample of the same utterances."""
+    import torch
+    import cases
+    import k2_amd as k2
+    B, T, S, C, R = 32, 500, 100, 500, 5
+    c = cases.rnnt_case(3, B, T, S, C, t_lo=300, s_lo=50)
+    lm, am = torch.from_numpy(c["lm"]).to(dev), torch.from_numpy(c["am"]).to(dev)
+    sym, bd = torch.from_numpy(c["symbols"]).to(dev), torch.from_numpy(c["boundary"]).to(dev)
+    logits = torch.from_numpy(np.random.default_rng(33).standard_normal((B, T, R, C)).astype(np.float32)).to(dev)
+    logits.requires_grad_(True)
+
+    def simple_and_ranges():
+        _, (gx, gy) = k2.rnnt_loss_simple(lm, am, sym, 0, bd, reduction="sum", return_grad=True)
+        return k2.get_rnnt_prune_ranges(gx, gy, bd, R)
+
+    def pruned(ranges):
+        logits.grad = None
+        loss = k2.rnnt_loss_pruned(logits, sym, ranges, 0, bd, reduction="sum")
+        loss.backward()
+        return loss
+
+    ranges = simple_and_ranges()
+    for _ in range(3):
+        pruned(ranges)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+    torch.cuda.synchronize()
+    ev[0].record()
+    for _ in range(steps):
+        ranges = simple_and_ranges()
+    ev[1].record()
+    for _ in range(steps):
+        loss = pruned(ranges)
+    ev[2].record()
+    torch.cuda.synchronize()
+    t_ranges = ev[0].elapsed_time(ev[1]) / steps * 1e-3
+    t_pruned = ev[1].elapsed_time(ev[2]) / steps * 1e-3
+    # one read of the logits forward, one read + one write backward, fp32
+    logits_bytes = 3 * logits.numel() * 4
+    out = {
+        "workload": "rnnt_loss_pruned fwd+bwd, fp32, regular, B=32 T=500 S=100 V=500 s_range=5 "
+                    "(BASELINE config 3), ranges from an rnnt_loss_simple pass",
+        "value": B / t_pruned, "unit": "utterances/s", "ms_per_step": t_pruned * 1e3,
+        "logits_GBps": logits_bytes / t_pruned / 1e9,
+        "frac_of_hbm_peak": logits_bytes / t_pruned / 1e9 / HBM_PEAK_GBS,
+        "simple_pass_plus_prune_ranges_ms": t_ranges * 1e3,
+        "loss": float(loss),
+    }
+    if cpu:
+        n = B  # utterances in the CPU sample: the whole batch
+        cl = logits.detach()[:n].cpu().requires_grad_(True)
+        cs, cb, cr = sym[:n].cpu(), bd[:n].cpu(), ranges[:n].cpu()
+        times = []
+        for _ in range(10):
+            cl.grad = None
+            t0 = time.perf_counter()
+            _cpu_pruned_loss(cl, cs, cr, cb).backward()
+            times.append(time.perf_counter() - t0)
+        med = float(np.median(times))
+        out["cpu_baseline"] = {
+            "value": n / med, "unit": "utterances/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"the same {n} utterances, {len(times)} fwd+bwd passes, median "
+                      f"{med * 1e3:.0f} ms (torch CPU ops with {torch.get_num_threads()} threads + "
+                      "the single-threaded CPU recursion)"}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-secondary", action="store_true",
+                    help="skip the pruned-loss figure (BASELINE config 3) in the 'secondary' field")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch one plain device copy of 256 MiB before the warmup: the unit "
                          "against which rocprofv3's FETCH_SIZE / WRITE_SIZE readings are scaled")
@@ -159,6 +271,9 @@ def main():
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(c)
+    if not args.no_secondary:
+        del px, py, p
+        out["secondary"] = pruned_secondary(dev, cpu=not args.no_cpu)
     print(json.dumps(out))
 
 
