@@ -343,9 +343,10 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
   };
   // One code path for every block: quads that reach outside the valid columns pick up
   // neighbouring floats (or zeros past the tensor's end) that the commit masks.
-  // Always issues kFwdLoadsPerBlock loads, also for blocks past the last one (they read floats
-  // that nobody uses), so that the counts given to WaitLoads hold in every iteration.
+  // Always issues kFwdLoadsPerBlock loads, so that the counts given to WaitLoads hold in every
+  // iteration; for blocks past the last one it reads the last block again (cache hits).
   auto load_block = [&](int kb, FwdRegs &r) {
+    kb = min(kb, g.nblocks - 1);
 #pragma unroll
     for (int it = 0; it < kLoadItems; ++it) {
       const int jp = kb * kW + 4 * mm - 1 - (lq + kRowStep * it) * g.skew;  // column left of element 0
@@ -709,10 +710,11 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
   }
   // One code path for every block: quads that reach outside the valid columns pick up
   // neighbouring floats (or zeros past the tensor's end) that the commit masks.
-  // Always issues kBwdLoadsPerBlock loads, also for blocks in front of the first one and rows
-  // past the sequence's end (they read floats that nobody uses), so that the counts given to
-  // WaitLoads hold in every iteration.
+  // Always issues kBwdLoadsPerBlock loads, so that the counts given to WaitLoads hold in every
+  // iteration; for blocks in front of the first one it reads block 0 again, and rows past the
+  // sequence's end read its last row (cache hits both).
   auto load_block = [&](int kb, BwdRegs &r) {
+    kb = max(kb, 0);
 #pragma unroll
     for (int it = 0; it < kLoadItems; ++it) {
       const int jd = kb * kW + 4 * mm - (lq + kRowStep * it) * g.skew;  // destination column of element 0
