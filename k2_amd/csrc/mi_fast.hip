@@ -5,8 +5,8 @@
 // HBM bandwidth from several compute units (a single workgroup tops out near 100 GB/s on this
 // part; 32 sequences alone could never fill 8 TB/s).
 //
-// Inside a workgroup (twelve wavefronts, each with one job or none, so that no wavefront that
-// loads ever has to wait for a store to be acknowledged):
+// Inside a workgroup (ten wavefronts, each with one job, so that no wavefront that loads ever
+// has to wait for a store to be acknowledged):
 //   * one CHAIN wavefront carries the recursion, lane = lattice row.  Lane q works on column
 //     j = n - q*skew at step n (skew = 1 for the regular lattice, 0 for the modified one), so
 //     every cell depends on the previous step only: its own lane's value and the neighbouring
@@ -20,8 +20,6 @@
 //   * four STORER wavefronts drain the ring: results leave as contiguous row segments.
 //   * one EDGE wavefront takes the words published by the adjacent chunk and publishes this
 //     chunk's boundary row.
-//   * two IDLE wavefronts that only join the barriers: they occupy the slots of the chain
-//     wavefront's SIMD, which the chain then has to itself.
 //   * one barrier per block of 32 steps; it orders LDS traffic only, so global loads and stores
 //     stay in flight across it.
 //
@@ -49,11 +47,7 @@ constexpr int kRing = 3 * kW;       // ring positions per row
 constexpr int kStride = kRing + 4;  // floats per LDS row; +4 spreads lanes over banks
 constexpr int kMoverWaves = 4;      // loader wavefronts, and as many storer wavefronts
 constexpr int kMoverLanes = kWave * kMoverWaves;
-// Wavefronts of a workgroup are spread round-robin over the compute unit's four SIMDs.  The chain
-// wavefront (wave 0) is the critical path of the whole kernel, so the two other wavefronts that
-// land on its SIMD (waves 4 and 8) stay idle: they only take part in the barriers.
-constexpr int kIdleWaves = 2;
-constexpr int kFastThreads = kWave * (2 + kIdleWaves + 2 * kMoverWaves);
+constexpr int kFastThreads = kWave * (2 + 2 * kMoverWaves);  // chain + edge + loaders + storers
 constexpr unsigned kSentinel = 0x7fc5a5a5u;  // a quiet-NaN pattern arithmetic never produces
 constexpr int kSpinLimit = 1 << 20;
 constexpr float kLog2e = 1.44269504088896340736f;
@@ -187,21 +181,15 @@ struct ChunkGeom {
   int nblocks;
 };
 
-enum Role { kChain = 0, kEdge = 1, kLoader = 2, kStorer = 3, kIdle = 4 };
+enum Role { kChain = 0, kEdge = 1, kLoader = 2, kStorer = 3 };
 
-// wave:   0      1     2  3  4     5  6  7  8     9  10 11
-// role:   chain  edge  L0 L1 idle  L2 L3 S0 idle  S1 S2 S3
+// wave:   0      1     2..5     6..9
+// role:   chain  edge  loaders  storers
 __device__ __forceinline__ int RoleOf(int wave) {
-  if (wave == 0) return kChain;
-  if (wave == 1) return kEdge;
-  if (wave == 4 || wave == 8) return kIdle;
-  return wave < 7 ? kLoader : kStorer;
+  return wave == 0 ? kChain : (wave == 1 ? kEdge : (wave < 2 + kMoverWaves ? kLoader : kStorer));
 }
 // index of a loader (or storer) wavefront among its kind, 0..kMoverWaves-1
-__device__ __forceinline__ int MoverIndex(int wave) {
-  return wave < 7 ? (wave < 4 ? wave - 2 : wave - 3) : (wave == 7 ? 0 : wave - 8);
-}
-static_assert(kMoverWaves == 4 && kIdleWaves == 2, "the wave table above is written for 12 wavefronts");
+__device__ __forceinline__ int MoverIndex(int wave) { return (wave - 2) & (kMoverWaves - 1); }
 
 __global__ void FastWsInitKernel(FastHeader *hdr, unsigned *edge, size_t n) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -534,8 +522,6 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
       px_above = px_next;
       LdsBarrier();
     }
-  } else {
-    for (int kb = 0; kb < g.nblocks; ++kb) LdsBarrier();
   }
   if (role == kStorer) store_block(g.nblocks - 1);
   if (role == kEdge) publish_block(g.nblocks - 1);
@@ -942,8 +928,6 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
       take_block(kb - 1);
       LdsBarrier();
     }
-  } else {
-    for (int kb = top; kb >= 0; --kb) LdsBarrier();
   }
   if (role == kStorer) store_block(0);
   if (role == kEdge) publish_block(0);

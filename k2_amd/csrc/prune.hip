@@ -23,44 +23,73 @@ __device__ int *SuffixMin(int *a, int *b, int n) {
   return a;
 }
 
-// One workgroup per sequence.  Frames are spread over the threads for the window search (reads
-// of px_grad / py_grad are then contiguous along t), after which the two monotone passes of
-// _adjust_pruning_lower_bound run as log-step scans in LDS.
+// Step 1 of get_rnnt_prune_ranges: for every frame the window start with the largest
+//   sum_{k<R} py_grad[b, w+k, t]  -  px_grad[b, w-1, t]        (k2/python/k2/rnnt_loss.py:730-747)
+// A workgroup handles 64 frames of one sequence (reads are contiguous along t) and splits the
+// candidate window starts over kArgSplit thread groups, whose results meet in LDS.
 //
-// The window sum adds py_grad[b, s'+0 .. s'+R-1, t] first row to last in the input precision and
-// subtracts px_grad[b, s'-1, t] afterwards (k2/python/k2/rnnt_loss.py:730-744); the arg-max keeps
-// the first maximum (torch.argmax).
+// The window sum adds the rows first to last in the input precision and subtracts px_grad
+// afterwards, exactly as the reference's torch.sum / subtraction does, and the arg-max keeps the
+// first maximum (torch.argmax), so that identical inputs give identical integers.  The raw
+// arg-max goes to ranges[b, t, 0]; step 2 turns it into the final ranges in place.
+constexpr int kArgFrames = 64;
+constexpr int kArgSplit = 4;
+
 template <typename T>
-__global__ __launch_bounds__(kPruneThreads) void PruneRangesKernel(
-    const T *__restrict__ px_grad, const T *__restrict__ py_grad,
-    const int64_t *__restrict__ boundary, int64_t *__restrict__ ranges, int S, int Tn,
-    int modified, int R) {
-  extern __shared__ int lds[];
-  int *buf0 = lds, *buf1 = lds + Tn;
-  const int b = blockIdx.x;
+__global__ __launch_bounds__(kArgFrames * kArgSplit) void PruneArgmaxKernel(
+    const T *__restrict__ px_grad, const T *__restrict__ py_grad, int64_t *__restrict__ ranges,
+    int S, int Tn, int modified, int R) {
+  __shared__ T best_v_s[kArgSplit][kArgFrames];
+  __shared__ int best_w_s[kArgSplit][kArgFrames];
+  const int b = blockIdx.y;
+  const int tx = threadIdx.x % kArgFrames, grp = threadIdx.x / kArgFrames;
+  const int t = blockIdx.x * kArgFrames + tx;
   const int T1 = modified ? Tn : Tn + 1;
   const int S1 = S + 1;
   const int n_win = S1 - R + 1;
   const T *gx = px_grad + (size_t)b * S * T1;
   const T *gy = py_grad + (size_t)b * S1 * Tn;
+  // group g takes the contiguous share [w_lo, w_hi) of the window starts, so that "first
+  // maximum" inside a share and across shares (lower group wins ties) is the global first
+  const int per = (n_win + kArgSplit - 1) / kArgSplit;
+  const int w_lo = grp * per, w_hi = min(n_win, w_lo + per);
+  T best_v = 0;
+  int best = -1;
+  if (t < Tn) {
+    for (int w = w_lo; w < w_hi; ++w) {
+      T acc = gy[(size_t)w * Tn + t];
+      for (int k = 1; k < R; ++k) acc = acc + gy[(size_t)(w + k) * Tn + t];
+      const T v = acc - (w == 0 ? T(0) : gx[(size_t)(w - 1) * T1 + t]);
+      if (best < 0 || v > best_v) { best_v = v; best = w; }
+    }
+  }
+  best_v_s[grp][tx] = best_v;
+  best_w_s[grp][tx] = best;
+  __syncthreads();
+  if (grp == 0 && t < Tn) {
+    for (int g2 = 1; g2 < kArgSplit; ++g2) {
+      const int w2 = best_w_s[g2][tx];
+      const T v2 = best_v_s[g2][tx];
+      if (w2 >= 0 && (best < 0 || v2 > best_v)) { best_v = v2; best = w2; }
+    }
+    ranges[((size_t)b * Tn + t) * R] = best < 0 ? 0 : best;
+  }
+}
+
+// Step 2: one workgroup per sequence.  Frames from t_end - 1 on are pinned to
+// max(s_end - R + 1, 0), then the two monotone passes of _adjust_pruning_lower_bound
+// (k2/python/k2/rnnt_loss.py:580-630, 749-766) run as log-step scans in LDS and the ranges are
+// written over the raw arg-max values.
+__global__ __launch_bounds__(kPruneThreads) void PruneFinishKernel(
+    const int64_t *__restrict__ boundary, int64_t *__restrict__ ranges, int Tn, int modified, int R) {
+  extern __shared__ int lds[];
+  int *buf0 = lds, *buf1 = lds + Tn;
+  const int b = blockIdx.x;
   const int64_t s_end = boundary[4 * b + 2], t_end = boundary[4 * b + 3];
   int64_t pad64 = s_end - R + 1;
   const int pad = pad64 < 0 ? 0 : (int)pad64;
-  for (int t = threadIdx.x; t < Tn; t += kPruneThreads) {
-    int best = 0;
-    if (t < t_end - 1) {
-      T best_v = 0;
-      for (int w = 0; w < n_win; ++w) {
-        T acc = gy[(size_t)w * Tn + t];
-        for (int k = 1; k < R; ++k) acc = acc + gy[(size_t)(w + k) * Tn + t];
-        const T v = acc - (w == 0 ? T(0) : gx[(size_t)(w - 1) * T1 + t]);
-        if (w == 0 || v > best_v) { best_v = v; best = w; }
-      }
-    } else {
-      best = pad;
-    }
-    buf0[t] = best;
-  }
+  for (int t = threadIdx.x; t < Tn; t += kPruneThreads)
+    buf0[t] = t < t_end - 1 ? (int)ranges[((size_t)b * Tn + t) * R] : pad;
   __syncthreads();
   const int ramp = (modified ? 2 : R) - 1;
   int *cur = SuffixMin(buf0, buf1, Tn);
@@ -131,13 +160,15 @@ int k2amd_rnnt_prune_ranges(const void *px_grad, const void *py_grad, const int6
     return K2AMD_ERR_INVALID_ARGUMENT;
   if (B == 0 || T == 0) return K2AMD_OK;
   const size_t smem = 2 * (size_t)T * sizeof(int);
-  if (smem > 64 * 1024 || (long long)S * T >= (1ll << 31)) return K2AMD_ERR_UNSUPPORTED;
+  if (smem > 64 * 1024 || (long long)S * T >= (1ll << 31) || B > 65535) return K2AMD_ERR_UNSUPPORTED;
   hipStream_t st = static_cast<hipStream_t>(stream);
   modified = modified ? 1 : 0;
+  const dim3 grid1((unsigned)((T + kArgFrames - 1) / kArgFrames), (unsigned)B);
   if (dtype == K2AMD_F32)
-    hipLaunchKernelGGL(PruneRangesKernel<float>, dim3(B), dim3(kPruneThreads), smem, st, (const float *)px_grad, (const float *)py_grad, boundary, ranges, S, T, modified, s_range);
+    hipLaunchKernelGGL(PruneArgmaxKernel<float>, grid1, dim3(kArgFrames * kArgSplit), 0, st, (const float *)px_grad, (const float *)py_grad, ranges, S, T, modified, s_range);
   else
-    hipLaunchKernelGGL(PruneRangesKernel<double>, dim3(B), dim3(kPruneThreads), smem, st, (const double *)px_grad, (const double *)py_grad, boundary, ranges, S, T, modified, s_range);
+    hipLaunchKernelGGL(PruneArgmaxKernel<double>, grid1, dim3(kArgFrames * kArgSplit), 0, st, (const double *)px_grad, (const double *)py_grad, ranges, S, T, modified, s_range);
+  hipLaunchKernelGGL(PruneFinishKernel, dim3(B), dim3(kPruneThreads), smem, st, boundary, ranges, T, modified, s_range);
   return LaunchStatus();
 }
 
