@@ -538,10 +538,10 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
 // so every cell needs ONE exponential, computed by the loader wavefronts (E = d1, OME = 1 - d1,
 // with the reference's guards folded in: first row E = 0, first column of a regular lattice
 // E = 1, non-finite d1 -> both 0).  The chain wavefront then does, per position m (descending),
-//     h = E * G;  c = OME * G;  G = h(lane + 1) + c
-// i.e. two multiplies, one DPP move and one add.  Lane l handles lattice row row0 + l; lane 63
-// has no lane above it in the wavefront and receives, through the DPP's "old" operand, the h of
-// the first row of the chunk below, so here the LOWER chunk runs ahead.
+//     h = E * G;  c = OME * G;  G' = c + h(lane + 1) = OME * G + E(lane + 1) * G(lane + 1)
+// i.e. two multiplies for the outputs, one DPP multiply and one FMA for the recursion.  Lane l
+// handles lattice row row0 + l; lane 63 has no lane below it in the wavefront and receives the h
+// of the first row of the chunk below, so here the LOWER chunk runs ahead.
 struct BwdLds {
   // rows 0..63: d1 on the way in, h (px_grad) on the way out; row 64: the h arriving from the
   // chunk below, laid out like a row so that every lane reads "the row below it" the same way
