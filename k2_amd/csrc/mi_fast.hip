@@ -45,9 +45,7 @@ constexpr int kRows = 64;           // lattice rows per chunk, one per lane of t
 constexpr int kW = 32;              // steps per block
 constexpr int kRing = 3 * kW;       // ring positions per row
 constexpr int kStride = kRing + 4;  // floats per LDS row; +4 spreads lanes over banks
-constexpr int kMoverWaves = 4;      // loader wavefronts, and as many storer wavefronts
-constexpr int kMoverLanes = kWave * kMoverWaves;
-constexpr int kFastThreads = kWave * (2 + 2 * kMoverWaves);  // chain + edge + loaders + storers
+constexpr int kStorerWaves = 4;
 constexpr unsigned kSentinel = 0x7fc5a5a5u;  // a quiet-NaN pattern arithmetic never produces
 constexpr int kSpinLimit = 1 << 20;
 constexpr float kLog2e = 1.44269504088896340736f;
@@ -55,14 +53,27 @@ constexpr float kLn2 = 0.69314718055994530942f;
 constexpr int kQuadsPerRow = kStride / 4;
 constexpr int kQuadsPerBlock = kW / 4;
 // One work item = (row q in 0..63, quad m in 0..7) of a block: four consecutive steps of one
-// lattice row; 512 items per block, two per loader lane and two per storer lane (rows q and
-// q + 32, same quad).  A wave-wide 16-byte load or store occupies its wavefront for about a
-// hundred cycles once the memory pipeline is busy, so the movers' work is spread over all their
-// wavefronts in every iteration, and the loaders keep two register sets so that a block's loads
-// stay in flight for two iterations.
-static_assert(kRows * kQuadsPerBlock == 2 * kMoverLanes, "two work items per mover lane");
-constexpr int kLoadItems = 2;
-constexpr int kRowStep = kMoverLanes / kQuadsPerBlock;  // rows between a lane's items (32)
+// lattice row; 512 items per block.  The four storer wavefronts take two items per lane (rows q
+// and q + 32, same quad); the loader wavefronts (four in either kernel: with more of them the
+// compute unit's total instruction issue, which is what the backward's iteration is bound by,
+// does not grow) take 512 / lanes items per lane.  A
+// wave-wide 16-byte load or store occupies its wavefront for about a hundred cycles once the
+// memory pipeline is busy, so the movers' work is spread over all their wavefronts in every
+// iteration, and the loaders keep two register sets so that a block's loads stay in flight for
+// two iterations.
+constexpr int kBlockItems = kRows * kQuadsPerBlock;
+template <int kLoaderWavesT>
+struct Layout {
+  static constexpr int kLoaderWaves = kLoaderWavesT;
+  static constexpr int kLoaderLanes = kWave * kLoaderWaves;
+  static constexpr int kLoadItems = kBlockItems / kLoaderLanes;        // items per loader lane
+  static constexpr int kRowStep = kLoaderLanes / kQuadsPerBlock;       // rows between a lane's items
+  static constexpr int kThreads = kWave * (2 + kLoaderWaves + kStorerWaves);
+  static_assert(kLoadItems * kLoaderLanes == kBlockItems, "loader lanes must divide the block");
+};
+typedef Layout<4> FwdLayout;
+typedef Layout<4> BwdLayout;
+static_assert(kBlockItems == 2 * kWave * kStorerWaves, "two work items per storer lane");
 
 struct FastHeader {
   unsigned ticket;  // next chunk to hand out; reset by the last workgroup of a launch
@@ -183,13 +194,18 @@ struct ChunkGeom {
 
 enum Role { kChain = 0, kEdge = 1, kLoader = 2, kStorer = 3 };
 
-// wave:   0      1     2..5     6..9
-// role:   chain  edge  loaders  storers
+// wave:   0      1     2 ..           .. last
+// role:   chain  edge  loaders        storers (kStorerWaves)
+template <typename L>
 __device__ __forceinline__ int RoleOf(int wave) {
-  return wave == 0 ? kChain : (wave == 1 ? kEdge : (wave < 2 + kMoverWaves ? kLoader : kStorer));
+  return wave == 0 ? kChain : (wave == 1 ? kEdge : (wave < 2 + L::kLoaderWaves ? kLoader : kStorer));
 }
-// index of a loader (or storer) wavefront among its kind, 0..kMoverWaves-1
-__device__ __forceinline__ int MoverIndex(int wave) { return (wave - 2) & (kMoverWaves - 1); }
+// lane id of a loader (or storer) lane among the lanes of its kind
+template <typename L>
+__device__ __forceinline__ int MoverLane(int wave, int lane) {
+  const int first = wave < 2 + L::kLoaderWaves ? 2 : 2 + L::kLoaderWaves;
+  return (wave - first) * kWave + lane;
+}
 
 __global__ void FastWsInitKernel(FastHeader *hdr, unsigned *edge, size_t n) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -255,20 +271,20 @@ struct FwdLds {
 };
 
 struct FwdRegs {
-  float4v x[kLoadItems], y[kLoadItems];
+  float4v x[FwdLayout::kLoadItems], y[FwdLayout::kLoadItems];
 };
 // waits until at most kYounger of this wavefront's loads are outstanding and ties the registers
 // to the wait, so that no read of them moves in front of it
 template <int kYounger>
 __device__ __forceinline__ void WaitLoads(FwdRegs &r) {
-  static_assert(kLoadItems == 2, "operand list below");
+  static_assert(FwdLayout::kLoadItems == 2, "operand list below");
   asm volatile("s_waitcnt vmcnt(%4)"
                : "+v"(r.x[0]), "+v"(r.y[0]), "+v"(r.x[1]), "+v"(r.y[1])
                : "n"(kYounger));
 }
-constexpr int kFwdLoadsPerBlock = 2 * kLoadItems;
+constexpr int kFwdLoadsPerBlock = 2 * FwdLayout::kLoadItems;
 
-__global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
+__global__ __launch_bounds__(FwdLayout::kThreads) void MiForwardFastKernel(
     const float *__restrict__ px, const float *__restrict__ py,
     const int64_t *__restrict__ boundary, float *__restrict__ p, float *__restrict__ ans,
     FastHeader *hdr, float *edge, int B, int S, int Tn, int modified, int nchunks,
@@ -302,11 +318,12 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
   float *edge_in = edge + ((size_t)g.b * nchunks + g.c) * edge_stride;
 
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int role = RoleOf(wave);
-  // movers: lane id within the loader (or storer) wavefronts
-  const int mid = (MoverIndex(wave) * kWave + lane) & (kMoverLanes - 1);
-  const int mq = mid >> 3, mm = mid & 7;  // storers: rows mq and mq + 32, quad mm
-  const int lq = mq;                      // loaders: rows lq + kRowStep*it, quad mm
+  typedef FwdLayout L;
+  constexpr int kLoadItems = L::kLoadItems, kRowStep = L::kRowStep;
+  const int role = RoleOf<L>(wave);
+  const int mid = MoverLane<L>(wave, lane);  // lane id among the loader (or storer) lanes
+  const int mq = mid >> 3, mm = mid & 7;     // storers: rows mq and mq + 32, quad mm
+  const int lq = mq;                         // loaders: rows lq + kRowStep*it, quad mm
 
   const int hi_x = g.nt - modified, hi_y = g.nt - 1;  // last valid px / py column
 
@@ -342,27 +359,40 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
       r.y[it] = AsyncQuad(rsy, idx_y[it] + jp);
     }
   };
+  // `inner` is uniform over the workgroup: the masking code for blocks on the rim of the box is
+  // a real branch (the empty asm statement keeps the compiler from flattening it into selects
+  // that every block would pay for).
   auto commit_block = [&](int kb, FwdRegs &r) {  // registers -> LDS ring
     if (kb >= g.nblocks) return;
     const bool inner = interior(kb);
 #pragma unroll
     for (int it = 0; it < kLoadItems; ++it) {
       const int q = lq + kRowStep * it;
-      const int jp = kb * kW + 4 * mm - 1 - q * g.skew;
-      const int jx = jp + g.skew;
       float4 qx = AsFloat4(r.x[it]), qy = AsFloat4(r.y[it]);
-      if (!inner && g.b == 0) {  // the only sequence whose rows can start the tensor
-        qx = ShiftQuad(qx, idx_x[it] + jx);
-        qy = ShiftQuad(qy, idx_y[it] + jp);
-      }
-      float vx[4] = {qx.x, qx.y, qx.z, qx.w};
-      float vy[4] = {qy.x, qy.y, qy.z, qy.w};
+      float vx[4], vy[4];
+      if (inner) {
+        const float in_x[4] = {qx.x, qx.y, qx.z, qx.w}, in_y[4] = {qy.x, qy.y, qy.z, qy.w};
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const bool okx = rowx_ok[it] && (inner || (jx + e >= 0 && jx + e <= hi_x));
-        const bool oky = rowy_ok[it] && (inner || (jp + e >= 0 && jp + e <= hi_y));
-        vx[e] = okx ? fmaxf(vx[e], kLogZero) : kLogZero;
-        vy[e] = oky ? fmaxf(vy[e], kLogZero) : kLogZero;
+        for (int e = 0; e < 4; ++e) {
+          vx[e] = rowx_ok[it] ? fmaxf(in_x[e], kLogZero) : kLogZero;
+          vy[e] = rowy_ok[it] ? fmaxf(in_y[e], kLogZero) : kLogZero;
+        }
+      } else {
+        asm volatile("");
+        const int jp = kb * kW + 4 * mm - 1 - q * g.skew;
+        const int jx = jp + g.skew;
+        if (g.b == 0) {  // the only sequence whose rows can start the tensor
+          qx = ShiftQuad(qx, idx_x[it] + jx);
+          qy = ShiftQuad(qy, idx_y[it] + jp);
+        }
+        const float in_x[4] = {qx.x, qx.y, qx.z, qx.w}, in_y[4] = {qy.x, qy.y, qy.z, qy.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const bool okx = rowx_ok[it] && jx + e >= 0 && jx + e <= hi_x;
+          const bool oky = rowy_ok[it] && jp + e >= 0 && jp + e <= hi_y;
+          vx[e] = okx ? fmaxf(in_x[e], kLogZero) : kLogZero;
+          vy[e] = oky ? fmaxf(in_y[e], kLogZero) : kLogZero;
+        }
       }
       const int pq = (kb % 3) * kQuadsPerBlock + mm;
       lds.fx[q][pq] = make_float4(vx[0], vx[1], vx[2], vx[3]);
@@ -543,24 +573,28 @@ __global__ __launch_bounds__(kFastThreads) void MiForwardFastKernel(
 // handles lattice row row0 + l; lane 63 has no lane below it in the wavefront and receives the h
 // of the first row of the chunk below, so here the LOWER chunk runs ahead.
 struct BwdLds {
-  // rows 0..63: d1 on the way in, h (px_grad) on the way out; row 64: the h arriving from the
-  // chunk below, laid out like a row so that every lane reads "the row below it" the same way
+  // rows 0..63: d1 of the row's cells; row 64: the h arriving from the chunk below, laid out like
+  // a row so that every lane reads "the row below it" the same way
   float4 e[kWave + 1][kQuadsPerRow];
-  float4 ome[kWave][kQuadsPerRow];  // 1 - d1 on the way in, c (py_grad) on the way out
+  float4 ome[kWave][kQuadsPerRow];  // 1 - d1
+  // what the chain leaves behind: the gradient of each row AFTER the step at a position, which is
+  // the gradient the cell one position to the right saw (the storers multiply it with that cell's
+  // d1 and 1 - d1)
+  float4 g[kWave][kQuadsPerRow];
   unsigned ticket;
 };
 
 struct BwdRegs {
-  float4v d[kLoadItems], s[kLoadItems], x[kLoadItems];  // p[dest], p[src], px[src]
+  float4v d[BwdLayout::kLoadItems], s[BwdLayout::kLoadItems], x[BwdLayout::kLoadItems];  // p[dest], p[src], px[src]
 };
 template <int kYounger>
 __device__ __forceinline__ void WaitLoads(BwdRegs &r) {
-  static_assert(kLoadItems == 2, "operand list below");
+  static_assert(BwdLayout::kLoadItems == 2, "operand list below");
   asm volatile("s_waitcnt vmcnt(%6)"
                : "+v"(r.d[0]), "+v"(r.s[0]), "+v"(r.x[0]), "+v"(r.d[1]), "+v"(r.s[1]), "+v"(r.x[1])
                : "n"(kYounger));
 }
-constexpr int kBwdLoadsPerBlock = 3 * kLoadItems;
+constexpr int kBwdLoadsPerBlock = 3 * BwdLayout::kLoadItems;
 
 // Clears the four columns c..c+3 of array row r of px_grad / py_grad wherever they lie outside
 // the region the sweep assigns.
@@ -600,7 +634,7 @@ __device__ __forceinline__ void ZeroItem(const ZeroGeom &z, int r, int c) {
   }
 }
 
-__global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
+__global__ __launch_bounds__(BwdLayout::kThreads) void MiBackwardFastKernel(
     const float *__restrict__ px, const float *__restrict__ p,
     const int64_t *__restrict__ boundary, float *__restrict__ ans_grad,
     float *__restrict__ px_grad, float *__restrict__ py_grad, FastHeader *hdr, float *edge, int B,
@@ -656,10 +690,12 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
   float *edge_in = edge + ((size_t)g.b * nchunks + g.c + 1) * edge_stride;  // from chunk c+1
 
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int role = RoleOf(wave);
-  const int mid = (MoverIndex(wave) * kWave + lane) & (kMoverLanes - 1);
-  const int mq = mid >> 3, mm = mid & 7;  // storers: rows mq and mq + 32, quad mm
-  const int lq = mq;                      // loaders: rows lq + kRowStep*it, quad mm
+  typedef BwdLayout L;
+  constexpr int kLoadItems = L::kLoadItems, kRowStep = L::kRowStep;
+  const int role = RoleOf<L>(wave);
+  const int mid = MoverLane<L>(wave, lane);  // lane id among the loader (or storer) lanes
+  const int mq = mid >> 3, mm = mid & 7;     // storers: rows mq and mq + 32, quad mm
+  const int lq = mq;                         // loaders: rows lq + kRowStep*it, quad mm
 
   // ---- loaders ---------------------------------------------------------------------------
   // destination cells with both edges exist only for rows 1..ns and columns 1..nt
@@ -686,7 +722,7 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
   for (int it = 0; it < kLoadItems; ++it) row_ok[it] = g.row0 + lq + kRowStep * it <= g.ns;
   if (g.row0 + kRows - 1 > g.ns) {
     const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int i = threadIdx.x; i < kWave * kQuadsPerRow; i += kFastThreads) {
+    for (int i = threadIdx.x; i < kWave * kQuadsPerRow; i += L::kThreads) {
       const int q = i / kQuadsPerRow, k = i - q * kQuadsPerRow;
       if (g.row0 + q > g.ns) {
         lds.e[q][k] = zero4;
@@ -732,6 +768,8 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
     *e_io = virt ? 0.0f : e_v;
     *o_io = virt ? 1.0f : o_v;
   };
+  // `inner` is uniform over the workgroup: the rim code below it is a real branch (the empty asm
+  // statements keep the compiler from flattening it into selects that every block would pay for).
   auto commit_block = [&](int kb, BwdRegs &r) {
     if (kb < 0) return;
     const bool inner = interior(kb);
@@ -741,6 +779,7 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
       const int q = lq + kRowStep * it;
       float4 qd = AsFloat4(r.d[it]), qs = AsFloat4(r.s[it]), qx = AsFloat4(r.x[it]);
       if (!inner && g.b == 0) {  // the only sequence whose rows can start the tensor
+        asm volatile("");
         const int jd0 = kb * kW + 4 * mm - q * g.skew;
         qd = ShiftQuad(qd, idx_d[it] + jd0);
         qs = ShiftQuad(qs, idx_s[it] + jd0);
@@ -762,6 +801,7 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
           }
         }
       } else {
+        asm volatile("");
         const int row_i = g.row0 + q;
         const int jd = kb * kW + 4 * mm - q * g.skew;
 #pragma unroll
@@ -774,6 +814,9 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
   };
 
   // ---- storers ---------------------------------------------------------------------------
+  // The gradient G a cell at position m saw is what the chain left at position m + 1, which for
+  // the last position of a block lies in the block to its right (computed one iteration earlier;
+  // its slot in g is not written again before the chain reaches the block two to the left).
   auto store_block = [&](int kb) {
     if (kb >= g.nblocks) return;
 #pragma unroll
@@ -782,15 +825,17 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
       const int row_i = g.row0 + q;
       if (row_i > g.ns) continue;
       const int pq = (kb % 3) * kQuadsPerBlock + mm;
-      const float4 h4 = lds.e[q][pq];
-      const float4 c4 = lds.ome[q][pq];
-      const float hv[4] = {h4.x, h4.y, h4.z, h4.w}, cv[4] = {c4.x, c4.y, c4.z, c4.w};
+      const int pq_right = mm + 1 < kQuadsPerBlock ? pq + 1 : ((kb + 1) % 3) * kQuadsPerBlock;
+      const float4 e4 = lds.e[q][pq], o4 = lds.ome[q][pq], g4 = lds.g[q][pq], gr = lds.g[q][pq_right];
+      const float gv[4] = {g4.y, g4.z, g4.w, gr.x};
+      const float hv[4] = {e4.x * gv[0], e4.y * gv[1], e4.z * gv[2], e4.w * gv[3]};
+      const float cv[4] = {o4.x * gv[0], o4.y * gv[1], o4.z * gv[2], o4.w * gv[3]};
       const int jd = kb * kW + 4 * mm - q * g.skew;
       const int s = g.s0 + row_i;
       // py_grad[s][t0 + jd - 1 + e]   for destination columns 1..nt
       float *dy = gyb + (size_t)s * Tn + g.t0 + jd - 1;
       if (jd >= 1 && jd + 3 <= g.nt) {
-        StoreQuad(dy, c4);
+        StoreQuad(dy, make_float4(cv[0], cv[1], cv[2], cv[3]));
       } else {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
@@ -801,7 +846,7 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
         float *dx = gxb + (size_t)(s - 1) * T1 + g.t0 + jd - 1 + g.skew;
         const int lo = 1 - g.skew;
         if (jd >= lo && jd + 3 <= g.nt) {
-          StoreQuad(dx, h4);
+          StoreQuad(dx, make_float4(hv[0], hv[1], hv[2], hv[3]));
         } else {
 #pragma unroll
           for (int e = 0; e < 4; ++e)
@@ -823,13 +868,18 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
       reinterpret_cast<float *>(lds.e[kWave])[(kb % 3) * kW + lane] = v;
     }
   };
-  // only words the chunk above will take are published (positions it maps inside its range)
+  // Lanes 32..63 hand the h of the chunk's first row (d1 times the gradient the cell saw, see
+  // store_block) to the chunk above.  Only words that chunk will take are published (positions
+  // it maps inside its range).
   auto publish_block = [&](int kb) {
     if (has_up && kb < g.nblocks && lane >= kW) {
-      const int mpos = kb * kW + (lane - kW);
-      if (mpos + edge_shift < g.nblocks * kW)
-        PublishEdge(edge_out + mpos, reinterpret_cast<const float *>(
-                                         &lds.e[0][0])[(kb % 3) * kW + (lane - kW)]);
+      const int i = lane - kW;
+      const int mpos = kb * kW + i;
+      if (mpos + edge_shift < g.nblocks * kW) {
+        const float e0 = reinterpret_cast<const float *>(&lds.e[0][0])[(kb % 3) * kW + i];
+        const int right = i + 1 < kW ? (kb % 3) * kW + i + 1 : ((kb + 1) % 3) * kW;
+        PublishEdge(edge_out + mpos, e0 * reinterpret_cast<const float *>(&lds.g[0][0])[right]);
+      }
     }
   };
 
@@ -838,48 +888,43 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
   float G = 0.0f;
   if (role == kChain && g.row0 + lane == g.ns) G = ans_grad[g.b];
   float g_origin = 0.0f;
-  // Per position (descending): with E, OME of the own row and Edn = E of the row below (lane+1),
-  //     h = E * G;  c = OME * G;                      -> px_grad, py_grad of this cell
-  //     G' = OME * G + Edn * G(lane + 1)              = c + h(lane + 1)
+  // Per position (descending), with OME of the own row and Edn = d1 of the row below (lane + 1):
+  //     G' = OME * G + Edn * G(lane + 1)
+  // one DPP multiply and one FMA; G' goes to LDS, the storers turn it into px_grad / py_grad.
   // Lane 63 has no lane below it: the DPP multiply leaves its register untouched, and what that
-  // register holds is row 64 of the E array, the h arriving from the chunk below.  The two output
-  // multiplies sit between the write of G and its DPP read and provide the wait states that
-  // read needs.
+  // register holds is row 64 of the E array, the h arriving from the chunk below.  The DPP read
+  // of G needs two wait states after the FMA that wrote it.
   auto chain_block = [&](int kb) {
     const int base = (kb % 3) * kQuadsPerBlock;
-    float4 ne = lds.e[lane][base + kQuadsPerBlock - 1], nd = lds.e[lane + 1][base + kQuadsPerBlock - 1],
-           no = lds.ome[lane][base + kQuadsPerBlock - 1];
+    float4 nd = lds.e[lane + 1][base + kQuadsPerBlock - 1], no = lds.ome[lane][base + kQuadsPerBlock - 1];
 #pragma unroll
     for (int k = kQuadsPerBlock - 1; k >= 0; --k) {
-      const float4 e4 = ne, d4 = nd, o4 = no;
+      const float4 d4 = nd, o4 = no;
       if (k > 0) {
-        ne = lds.e[lane][base + k - 1];
         nd = lds.e[lane + 1][base + k - 1];
         no = lds.ome[lane][base + k - 1];
       }
-      const float es[4] = {e4.x, e4.y, e4.z, e4.w};
-      const float ds[4] = {d4.x, d4.y, d4.z, d4.w};
+      float ts[4] = {d4.x, d4.y, d4.z, d4.w};
       const float os[4] = {o4.x, o4.y, o4.z, o4.w};
-      float hs[4], cs[4];
 #pragma unroll
       for (int e = 3; e >= 0; --e) {
         if (kb == 0 && k == 0 && e == 0) g_origin = G;
-        float t = ds[e];
         asm volatile(
-            "v_mul_f32 %[h], %[E], %[G]\n\t"
-            "v_mul_f32 %[c], %[O], %[G]\n\t"
+            "s_nop 1\n\t"
             "v_mul_f32_dpp %[t], %[G], %[t] wave_shl:1 row_mask:0xf bank_mask:0xf\n\t"
             "v_fmac_f32 %[t], %[O], %[G]"
-            : [h] "=&v"(hs[e]), [c] "=&v"(cs[e]), [t] "+&v"(t)
-            : [E] "v"(es[e]), [O] "v"(os[e]), [G] "v"(G));
-        G = t;
+            : [t] "+&v"(ts[e])
+            : [O] "v"(os[e]), [G] "v"(G));
+        G = ts[e];
       }
-      lds.e[lane][base + k] = make_float4(hs[0], hs[1], hs[2], hs[3]);
-      lds.ome[lane][base + k] = make_float4(cs[0], cs[1], cs[2], cs[3]);
+      lds.g[lane][base + k] = make_float4(ts[0], ts[1], ts[2], ts[3]);
     }
   };
 
   const int top = g.nblocks - 1;
+  // what the cells of the top block's last position saw: the initial gradient
+  if (role == kChain)
+    reinterpret_cast<float *>(&lds.g[lane][((top + 1) % 3) * kQuadsPerBlock])[0] = G;
   BwdRegs ra, rb;
   if (role == kLoader) {
     load_block(top, ra);
@@ -935,6 +980,13 @@ __global__ __launch_bounds__(kFastThreads) void MiBackwardFastKernel(
   if (threadIdx.x == 0) FinishWorkgroup(hdr, total_wgs);
 }
 
+// A sweeping workgroup wants a compute unit to itself (its chain wavefront sets the pace of the
+// whole sequence, and a second workgroup on the unit would share its LDS pipe and issue slots).
+// Asking for more than half of the unit's 160 KB of LDS makes the dispatcher place one workgroup
+// per unit; the bytes beyond the kernels' own structures are never touched.
+constexpr size_t kExclusiveLds = 84 * 1024;
+static_assert(sizeof(FwdLds) < kExclusiveLds && sizeof(BwdLds) < kExclusiveLds, "LDS budget");
+
 }  // namespace
 
 // The throughput kernels address each tensor through a buffer resource with 32-bit byte offsets:
@@ -967,7 +1019,7 @@ int MiForwardFast(const float *px, const float *py, const int64_t *boundary, flo
   const int edge_stride = (int)(((size_t)Tn + 2 + kRows + kW + 3) / 4 * 4 + kW);
   FastHeader *hdr = static_cast<FastHeader *>(workspace);
   float *edge = reinterpret_cast<float *>(hdr + 1);
-  hipLaunchKernelGGL(MiForwardFastKernel, dim3((unsigned)(B * nchunks)), dim3(kFastThreads), 0, stream,
+  hipLaunchKernelGGL(MiForwardFastKernel, dim3((unsigned)(B * nchunks)), dim3(FwdLayout::kThreads), kExclusiveLds - sizeof(FwdLds), stream,
                      px, py, boundary, p, ans, hdr, edge, B, S, Tn, modified, nchunks, edge_stride);
   return LaunchStatus();
 }
@@ -982,7 +1034,7 @@ int MiBackwardFast(const float *px, const float *p, const int64_t *boundary, flo
   FastHeader *hdr = static_cast<FastHeader *>(workspace);
   float *edge = reinterpret_cast<float *>(hdr + 1);
   // B * nchunks sweeping workgroups + as many that only clear
-  hipLaunchKernelGGL(MiBackwardFastKernel, dim3((unsigned)(2 * B * nchunks)), dim3(kFastThreads), 0, stream,
+  hipLaunchKernelGGL(MiBackwardFastKernel, dim3((unsigned)(2 * B * nchunks)), dim3(BwdLayout::kThreads), kExclusiveLds - sizeof(BwdLds), stream,
                      px, p, boundary, ans_grad, px_grad, py_grad, hdr, edge, B, S, Tn, modified,
                      nchunks, edge_stride, overwrite_ans_grad);
   return LaunchStatus();
