@@ -403,6 +403,8 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiForwardFastKernel(
   // ---- storers ---------------------------------------------------------------------------
   auto store_block = [&](int kb) {  // LDS ring -> p
     if (kb < 0) return;
+    // columns kb*32 - 63*skew .. kb*32 + 31 all inside 0..nt-1 (the end cell is never "inner")
+    const bool inner = kb * kW - (kRows - 1) * g.skew >= 0 && kb * kW + kW - 1 <= g.nt - 1;
 #pragma unroll
     for (int it = 0; it < 2; ++it) {
       const int q = mq + 32 * it;
@@ -416,18 +418,19 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiForwardFastKernel(
       v.w = v.w < kLogZeroTest ? ninf : v.w;
       const int j = kb * kW + 4 * mm - q * g.skew;  // column of element 0
       float *dst = pb + (size_t)(g.s0 + row_i) * (Tn + 1) + g.t0 + j;
-      const float vv[4] = {v.x, v.y, v.z, v.w};
-      if (j >= 0 && j + 3 <= g.nt) {
+      if (inner) {  // uniform: every column of the block lies in 0..nt-1 for every row
         StoreQuad(dst, v);
       } else {
+        asm volatile("");  // keeps this path a branch of its own
+        const float vv[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
         for (int e = 0; e < 4; ++e)
           if (j + e >= 0 && j + e <= g.nt) dst[e] = vv[e];
-      }
-      if (row_i == g.ns) {
+        if (row_i == g.ns) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
-          if (j + e == g.nt) ans[g.b] = vv[e];
+          for (int e = 0; e < 4; ++e)
+            if (j + e == g.nt) ans[g.b] = vv[e];
+        }
       }
     }
   };
@@ -819,6 +822,7 @@ __global__ __launch_bounds__(BwdLayout::kThreads) void MiBackwardFastKernel(
   // its slot in g is not written again before the chain reaches the block two to the left).
   auto store_block = [&](int kb) {
     if (kb >= g.nblocks) return;
+    const bool inner = interior(kb);
 #pragma unroll
     for (int it = 0; it < 2; ++it) {
       const int q = mq + 32 * it;
@@ -833,21 +837,19 @@ __global__ __launch_bounds__(BwdLayout::kThreads) void MiBackwardFastKernel(
       const int jd = kb * kW + 4 * mm - q * g.skew;
       const int s = g.s0 + row_i;
       // py_grad[s][t0 + jd - 1 + e]   for destination columns 1..nt
+      // px_grad[s-1][t0 + jd - 1 + skew + e]   for destination columns (1 - skew)..nt
       float *dy = gyb + (size_t)s * Tn + g.t0 + jd - 1;
-      if (jd >= 1 && jd + 3 <= g.nt) {
+      float *dx = gxb + (size_t)(s - 1) * T1 + g.t0 + jd - 1 + g.skew;
+      if (inner) {  // uniform: every cell of the block has both edges inside the box
         StoreQuad(dy, make_float4(cv[0], cv[1], cv[2], cv[3]));
+        if (row_i >= 1) StoreQuad(dx, make_float4(hv[0], hv[1], hv[2], hv[3]));
       } else {
+        asm volatile("");  // keeps this path a branch of its own
 #pragma unroll
         for (int e = 0; e < 4; ++e)
           if (jd + e >= 1 && jd + e <= g.nt) dy[e] = cv[e];
-      }
-      // px_grad[s-1][t0 + jd - 1 + skew + e]   for destination columns (1 - skew)..nt
-      if (row_i >= 1) {
-        float *dx = gxb + (size_t)(s - 1) * T1 + g.t0 + jd - 1 + g.skew;
-        const int lo = 1 - g.skew;
-        if (jd >= lo && jd + 3 <= g.nt) {
-          StoreQuad(dx, make_float4(hv[0], hv[1], hv[2], hv[3]));
-        } else {
+        if (row_i >= 1) {
+          const int lo = 1 - g.skew;
 #pragma unroll
           for (int e = 0; e < 4; ++e)
             if (jd + e >= lo && jd + e <= g.nt) dx[e] = hv[e];
