@@ -2,11 +2,14 @@
 //   get_rnnt_logprobs_joint   logits [B][T][S+1][C]   (k2/python/k2/rnnt_loss.py:341-447)
 //   get_rnnt_logprobs_pruned  logits [B][T][R][C]     (k2/python/k2/rnnt_loss.py:1180-1348)
 //
-// Both are one pass over the logits: one 64-lane wavefront owns one row of C logits, keeps it in
-// registers, reduces max and sum(exp) across lanes with DPP-style shuffles, and emits the two
-// values px / py that the row contributes (symbol and termination log-probs).  The backward is the
-// mirror pass: read the row once, write its gradient once.  HBM traffic is the algorithmic
-// minimum (logits read once forward; read once + written once backward).
+// Both are one streaming pass over the logits, one 64-lane wavefront per row of C logits held
+// in registers (max and sum(exp) reduced across lanes), plus a small pass with one THREAD per
+// row for the look-ups that decide which two log-probs a row contributes and where they go
+// (ranges -> symbols -> logits: dependent round trips that a wavefront should pay for 64 rows
+// at a time, not for one).  The backward mirrors it: a thread-per-row pass gathers each row's
+// two incoming gradients, the streaming pass reads the row once and writes its gradient once.
+// HBM traffic is the algorithmic minimum (logits read once forward; read once + written once
+// backward).
 #include "common.h"
 
 namespace k2amd {
@@ -136,24 +139,38 @@ __device__ __forceinline__ void RowTarget(const RowGeom &g, const int64_t *__res
   }
 }
 
-template <typename T, bool kPruned>
-__global__ __launch_bounds__(kRowsPerBlock *kWave) void RowForwardKernel(
-    const T *__restrict__ logits, const int64_t *__restrict__ symbols,
-    const int64_t *__restrict__ ranges, const int64_t *__restrict__ boundary, T *__restrict__ px,
-    T *__restrict__ py, T *__restrict__ normalizers, RowGeom g) {
+// Forward, pass 1: one wavefront per row streams the row and leaves its log-sum-exp in
+// `normalizers`.  Nothing else: the look-ups that decide where a row's two log-probs go are a
+// chain of dependent memory round trips, and paying that chain once per WAVEFRONT (one row)
+// rather than once per LANE (64 rows, pass 2) cost a third of this kernel's time.
+template <typename T>
+__global__ __launch_bounds__(kRowsPerBlock *kWave) void RowNormKernel(
+    const T *__restrict__ logits, T *__restrict__ normalizers, long long rows, int C) {
   const int lane = threadIdx.x & (kWave - 1);
   const long long row = (long long)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const T *x = logits + (size_t)row * C;
+  const T norm = RowIsVectorisable<T>(C) ? RowLogSumExpVec<T>(x, C, lane) : RowLogSumExp<T>(x, C, lane);
+  if (lane == 0) normalizers[row] = norm;
+}
+
+// Forward, pass 2: one thread per row looks up where the row lands and writes
+//   px[b,s,t] = logits[row, sym] - norm,   py[b,s,t] = logits[row, blank] - norm.
+template <typename T, bool kPruned>
+__global__ void RowEmitKernel(const T *__restrict__ logits, const T *__restrict__ normalizers,
+                              const int64_t *__restrict__ symbols, const int64_t *__restrict__ ranges,
+                              const int64_t *__restrict__ boundary, T *__restrict__ px,
+                              T *__restrict__ py, RowGeom g) {
   const long long rows = (long long)g.B * g.Tn * g.K;
+  const long long row = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (row >= rows) return;
   const int k = (int)(row % g.K);
   const int t = (int)((row / g.K) % g.Tn);
   const int b = (int)(row / ((long long)g.K * g.Tn));
   const T *x = logits + (size_t)row * g.C;
-  const T norm = RowIsVectorisable<T>(g.C) ? RowLogSumExpVec<T>(x, g.C, lane) : RowLogSumExp<T>(x, g.C, lane);
-  if (lane != 0) return;
-  normalizers[row] = norm;
   int s, sym;
   RowTarget<kPruned>(g, symbols, ranges, b, t, k, &s, &sym);
+  const T norm = normalizers[row];
   const int T1 = g.rnnt_type == K2AMD_REGULAR ? g.Tn + 1 : g.Tn;
   if (s < g.S) {
     T v = (sym >= 0 && sym < g.C) ? x[sym] - norm : Real<T>::NegInf();
@@ -190,6 +207,109 @@ __global__ void ConstrainedKernel(T *__restrict__ px, const T *__restrict__ py, 
   }
 }
 
+// d loss / d logits[row, c] = -softmax(row)[c] * (gx + gy) + gx [c == sym] + gy [c == blank], with
+// gx, gy the gradients that reach the row's px and py values.
+//
+// Backward, pass 1: one thread per row gathers what the row's gradient depends on (the look-up
+// chain again, 64 rows per wavefront) and parks it in the first four elements of the row's own
+// slot of logits_grad: {gx, gy, symbol, normaliser}.  Rows therefore need at least four columns.
+template <typename T, bool kPruned>
+__global__ void RowGradPrepKernel(const T *__restrict__ normalizers, const T *__restrict__ px_grad,
+                                  const T *__restrict__ py_grad, const int64_t *__restrict__ symbols,
+                                  const int64_t *__restrict__ ranges,
+                                  const int64_t *__restrict__ boundary, T *__restrict__ logits_grad,
+                                  RowGeom g) {
+  const long long rows = (long long)g.B * g.Tn * g.K;
+  const long long row = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (row >= rows) return;
+  const int k = (int)(row % g.K);
+  const int t = (int)((row / g.K) % g.Tn);
+  const int b = (int)(row / ((long long)g.K * g.Tn));
+  int s, sym;
+  RowTarget<kPruned>(g, symbols, ranges, b, t, k, &s, &sym);
+  const int T1 = g.rnnt_type == K2AMD_REGULAR ? g.Tn + 1 : g.Tn;
+  T gx = 0;
+  if (s < g.S && sym >= 0 && sym < g.C) {
+    const bool cut =
+        g.rnnt_type == K2AMD_REGULAR && boundary != nullptr && boundary[4 * b + 3] == t;
+    if (!cut) gx = px_grad[((size_t)b * g.S + s) * T1 + t];
+  } else {
+    sym = -1;
+  }
+  T gy = py_grad[((size_t)b * (g.S + 1) + s) * g.Tn + t];
+  if (g.rnnt_type == K2AMD_CONSTRAINED && s >= 1)
+    gy += px_grad[((size_t)b * g.S + (s - 1)) * T1 + t];  // px += py[:, 1:]
+  T *rec = logits_grad + (size_t)row * g.C;
+  rec[0] = gx;
+  rec[1] = gy;
+  rec[2] = (T)sym;  // exact: |sym| < 2^24
+  rec[3] = normalizers[row];
+}
+
+// Backward, pass 2: one wavefront per row reads the row and its parked record, and writes the
+// gradient over the whole slot (record included; every lane has read it by then).
+template <typename T>
+__global__ __launch_bounds__(kRowsPerBlock *kWave) void RowGradKernel(
+    const T *__restrict__ logits, T *__restrict__ logits_grad, long long rows, int C, int blank) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const long long row = (long long)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const T *x = logits + (size_t)row * C;
+  T *dx = logits_grad + (size_t)row * C;
+  typedef typename Vec16<T>::type V;
+  constexpr int kN = Vec16<T>::kN;
+  const bool vectorised = RowIsVectorisable<T>(C);
+  const int nv = C / kN;
+  V in[kMaxVecs];
+  if (vectorised) {
+    const V *xv = reinterpret_cast<const V *>(x);
+#pragma unroll
+    for (int i = 0; i < kMaxVecs; ++i) {
+      const int q = lane + i * kWave;
+      if (q < nv) in[i] = xv[q];
+    }
+  }
+  const T gx = dx[0], gy = dx[1], norm = dx[3];
+  const int sym = (int)dx[2];
+  const T tot = gx + gy;
+  if (vectorised) {
+    V *dv = reinterpret_cast<V *>(dx);
+    V outv[kMaxVecs];
+#pragma unroll
+    for (int i = 0; i < kMaxVecs; ++i) {
+      const int q = lane + i * kWave;
+      if (q < nv) {
+        T e[kN];
+        Unpack(in[i], e);
+#pragma unroll
+        for (int k2 = 0; k2 < kN; ++k2) {
+          const int c = q * kN + k2;
+          T v = -FastExp(e[k2] - norm) * tot;
+          if (c == sym) v += gx;
+          if (c == blank) v += gy;
+          e[k2] = v;
+        }
+        outv[i] = Pack(e);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < kMaxVecs; ++i) {
+      const int q = lane + i * kWave;
+      if (q < nv) dv[q] = outv[i];
+    }
+    return;
+  }
+  // rows that are not read as vectors: every lane holds the record in registers before the
+  // first store of the loop below can reach it (a wavefront's loads complete in order)
+  for (int c = lane; c < C; c += kWave) {
+    T v = -Real<T>::Exp(x[c] - norm) * tot;
+    if (c == sym) v += gx;
+    if (c == blank) v += gy;
+    dx[c] = v;
+  }
+}
+
+// The same in one pass, for rows too short to park a record in (C < 4).
 template <typename T, bool kPruned>
 __global__ __launch_bounds__(kRowsPerBlock *kWave) void RowBackwardKernel(
     const T *__restrict__ logits, const T *__restrict__ normalizers,
@@ -274,8 +394,10 @@ int RowForward(const T *logits, const int64_t *symbols, const int64_t *ranges,
   const long long rows = (long long)g.B * g.Tn * g.K;
   if (rows > 0) {
     const long long blocks = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
-    hipLaunchKernelGGL((RowForwardKernel<T, kPruned>), dim3((unsigned)blocks), dim3(kRowsPerBlock * kWave), 0, stream,
-                       logits, symbols, ranges, boundary, px, py, normalizers, g);
+    hipLaunchKernelGGL((RowNormKernel<T>), dim3((unsigned)blocks), dim3(kRowsPerBlock * kWave), 0, stream,
+                       logits, normalizers, rows, g.C);
+    hipLaunchKernelGGL((RowEmitKernel<T, kPruned>), dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, stream,
+                       logits, (const T *)normalizers, symbols, ranges, boundary, px, py, g);
   }
   if (g.rnnt_type == K2AMD_CONSTRAINED && n_px > 0)
     hipLaunchKernelGGL(ConstrainedKernel<T>, dim3(1024), dim3(256), 0, stream, px, py, g.B, g.S, g.Tn);
@@ -289,9 +411,16 @@ int RowBackward(const T *logits, const T *normalizers, const T *px_grad, const T
   const long long rows = (long long)g.B * g.Tn * g.K;
   if (rows > 0) {
     const long long blocks = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
-    hipLaunchKernelGGL((RowBackwardKernel<T, kPruned>), dim3((unsigned)blocks), dim3(kRowsPerBlock * kWave), 0, stream,
-                       logits, normalizers, px_grad, py_grad, symbols, ranges, boundary,
-                       logits_grad, g);
+    if (g.C >= 4) {
+      hipLaunchKernelGGL((RowGradPrepKernel<T, kPruned>), dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, stream,
+                         normalizers, px_grad, py_grad, symbols, ranges, boundary, logits_grad, g);
+      hipLaunchKernelGGL((RowGradKernel<T>), dim3((unsigned)blocks), dim3(kRowsPerBlock * kWave), 0, stream,
+                         logits, logits_grad, rows, g.C, g.blank);
+    } else {
+      hipLaunchKernelGGL((RowBackwardKernel<T, kPruned>), dim3((unsigned)blocks), dim3(kRowsPerBlock * kWave), 0, stream,
+                         logits, normalizers, px_grad, py_grad, symbols, ranges, boundary,
+                         logits_grad, g);
+    }
   }
   return LaunchStatus();
 }
