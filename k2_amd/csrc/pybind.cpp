@@ -1,6 +1,7 @@
 // pybind11 host module `_k2_amd`: the two native functions that k2's Python layer calls for the
 // mutual-information recursion, with the reference's names and keyword arguments
-// (k2/python/csrc/torch/mutual_information.cu:26-67), implemented over the C-ABI of libk2amd.so.
+// (k2/python/csrc/torch/mutual_information.cu:26-67), and host functions for the fused builders
+// that replace the reference's torch-op chains, all implemented over the C-ABI of libk2amd.so.
 //
 // Differences from the reference's host code, on purpose:
 //   * launches go to torch's CURRENT HIP stream of the tensors' device (the reference uses the
@@ -150,6 +151,208 @@ std::vector<torch::Tensor> MutualInformationBackward(torch::Tensor px, torch::Te
   return {px_grad, py_grad};
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// The fused builders that replace the torch-op chains of k2/python/k2/rnnt_loss.py.  Each mirrors
+// the C-ABI entry point of the same name (include/k2_amd.h): outputs are allocated here, raw
+// pointers go down, tensors come back.  Inputs must be contiguous and on one ROCm device.
+
+void *StreamOf(const torch::Tensor &t) {
+  return c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(t.device().index()).stream();
+}
+void RequireDevice(const torch::Tensor &t, const char *name) {
+  TORCH_CHECK(t.is_cuda(), "k2_amd runs on MI355X only: ", name, " is on ", t.device(),
+              " (there is no CPU path)");
+  TORCH_CHECK(t.is_contiguous(), name, " must be contiguous");
+}
+const int64_t *I64(const torch::optional<torch::Tensor> &t) {
+  if (!t.has_value() || !t->defined()) return nullptr;
+  TORCH_CHECK(t->scalar_type() == torch::kLong && t->is_contiguous() && t->is_cuda(),
+              "index tensors must be contiguous int64 device tensors");
+  return t->data_ptr<int64_t>();
+}
+int T1Of(int T, int rnnt_type) { return rnnt_type == K2AMD_REGULAR ? T + 1 : T; }
+
+// get_rnnt_logprobs: returns (px, py, lm_probs, am_probs, denom)
+std::vector<torch::Tensor> LogprobsSimpleForward(torch::Tensor lm, torch::Tensor am,
+                                                 torch::Tensor symbols, int termination_symbol,
+                                                 int rnnt_type,
+                                                 torch::optional<torch::Tensor> boundary) {
+  RequireDevice(lm, "lm");
+  RequireDevice(am, "am");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(am.device());
+  const int B = am.size(0), T = am.size(1), C = am.size(2), S = lm.size(1) - 1;
+  auto opt = am.options();
+  torch::Tensor px = torch::empty({B, S, T1Of(T, rnnt_type)}, opt), py = torch::empty({B, S + 1, T}, opt);
+  torch::Tensor lm_probs = torch::empty_like(lm), am_probs = torch::empty_like(am);
+  torch::Tensor lm_max = torch::empty({B, S + 1}, opt), am_max = torch::empty({B, T}, opt);
+  torch::Tensor denom = torch::empty({B, S + 1, T}, opt);
+  void *stream = StreamOf(am);
+  {
+    pybind11::gil_scoped_release release;
+    Check(k2amd_rnnt_logprobs_simple_forward(
+        lm.data_ptr(), am.data_ptr(), I64(symbols), I64(boundary), px.data_ptr(), py.data_ptr(),
+        lm_probs.data_ptr(), am_probs.data_ptr(), lm_max.data_ptr(), am_max.data_ptr(),
+        denom.data_ptr(), B, S, T, C, termination_symbol, rnnt_type, DtypeCode(am), stream));
+  }
+  return {px, py, lm_probs, am_probs, denom};
+}
+
+std::vector<torch::Tensor> LogprobsSimpleBackward(torch::Tensor px_grad, torch::Tensor py_grad,
+                                                  torch::Tensor symbols,
+                                                  torch::optional<torch::Tensor> boundary,
+                                                  torch::Tensor lm_probs, torch::Tensor am_probs,
+                                                  torch::Tensor denom, int termination_symbol,
+                                                  int rnnt_type) {
+  RequireDevice(px_grad, "px_grad");
+  RequireDevice(py_grad, "py_grad");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(am_probs.device());
+  const int B = am_probs.size(0), T = am_probs.size(1), C = am_probs.size(2), S = lm_probs.size(1) - 1;
+  torch::Tensor lm_grad = torch::empty_like(lm_probs), am_grad = torch::empty_like(am_probs);
+  torch::Tensor q = torch::empty_like(denom);
+  void *stream = StreamOf(am_probs);
+  {
+    pybind11::gil_scoped_release release;
+    Check(k2amd_rnnt_logprobs_simple_backward(
+        px_grad.data_ptr(), py_grad.data_ptr(), I64(symbols), I64(boundary), lm_probs.data_ptr(),
+        am_probs.data_ptr(), denom.data_ptr(), lm_grad.data_ptr(), am_grad.data_ptr(), q.data_ptr(),
+        B, S, T, C, termination_symbol, rnnt_type, DtypeCode(am_probs), stream));
+  }
+  return {lm_grad, am_grad};
+}
+
+// get_rnnt_logprobs_joint: returns (px, py, normalizers)
+std::vector<torch::Tensor> LogprobsJointForward(torch::Tensor logits, torch::Tensor symbols,
+                                                int termination_symbol, int rnnt_type,
+                                                torch::optional<torch::Tensor> boundary) {
+  RequireDevice(logits, "logits");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(logits.device());
+  const int B = logits.size(0), T = logits.size(1), S = logits.size(2) - 1, C = logits.size(3);
+  auto opt = logits.options();
+  torch::Tensor px = torch::empty({B, S, T1Of(T, rnnt_type)}, opt), py = torch::empty({B, S + 1, T}, opt);
+  torch::Tensor norm = torch::empty({B, T, S + 1}, opt);
+  void *stream = StreamOf(logits);
+  {
+    pybind11::gil_scoped_release release;
+    Check(k2amd_rnnt_logprobs_joint_forward(logits.data_ptr(), I64(symbols), I64(boundary),
+                                            px.data_ptr(), py.data_ptr(), norm.data_ptr(), B, S, T, C,
+                                            termination_symbol, rnnt_type, DtypeCode(logits), stream));
+  }
+  return {px, py, norm};
+}
+
+torch::Tensor LogprobsJointBackward(torch::Tensor logits, torch::Tensor norm, torch::Tensor px_grad,
+                                    torch::Tensor py_grad, torch::Tensor symbols,
+                                    torch::optional<torch::Tensor> boundary, int termination_symbol,
+                                    int rnnt_type) {
+  RequireDevice(logits, "logits");
+  RequireDevice(px_grad, "px_grad");
+  RequireDevice(py_grad, "py_grad");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(logits.device());
+  const int B = logits.size(0), T = logits.size(1), S = logits.size(2) - 1, C = logits.size(3);
+  torch::Tensor grad = torch::empty_like(logits);
+  void *stream = StreamOf(logits);
+  {
+    pybind11::gil_scoped_release release;
+    Check(k2amd_rnnt_logprobs_joint_backward(logits.data_ptr(), norm.data_ptr(), px_grad.data_ptr(),
+                                             py_grad.data_ptr(), I64(symbols), I64(boundary),
+                                             grad.data_ptr(), B, S, T, C, termination_symbol, rnnt_type,
+                                             DtypeCode(logits), stream));
+  }
+  return grad;
+}
+
+// get_rnnt_logprobs_pruned: returns (px, py, normalizers)
+std::vector<torch::Tensor> LogprobsPrunedForward(torch::Tensor logits, torch::Tensor symbols,
+                                                 torch::Tensor ranges, int termination_symbol,
+                                                 torch::optional<torch::Tensor> boundary,
+                                                 int rnnt_type) {
+  RequireDevice(logits, "logits");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(logits.device());
+  const int B = logits.size(0), T = logits.size(1), R = logits.size(2), C = logits.size(3);
+  const int S = symbols.size(1);
+  auto opt = logits.options();
+  torch::Tensor px = torch::empty({B, S, T1Of(T, rnnt_type)}, opt), py = torch::empty({B, S + 1, T}, opt);
+  torch::Tensor norm = torch::empty({B, T, R}, opt);
+  void *stream = StreamOf(logits);
+  {
+    pybind11::gil_scoped_release release;
+    Check(k2amd_rnnt_logprobs_pruned_forward(logits.data_ptr(), I64(symbols), I64(ranges),
+                                             I64(boundary), px.data_ptr(), py.data_ptr(),
+                                             norm.data_ptr(), B, S, T, R, C, termination_symbol,
+                                             rnnt_type, DtypeCode(logits), stream));
+  }
+  return {px, py, norm};
+}
+
+torch::Tensor LogprobsPrunedBackward(torch::Tensor logits, torch::Tensor norm, torch::Tensor px_grad,
+                                     torch::Tensor py_grad, torch::Tensor symbols, torch::Tensor ranges,
+                                     torch::optional<torch::Tensor> boundary, int termination_symbol,
+                                     int rnnt_type) {
+  RequireDevice(logits, "logits");
+  RequireDevice(px_grad, "px_grad");
+  RequireDevice(py_grad, "py_grad");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(logits.device());
+  const int B = logits.size(0), T = logits.size(1), R = logits.size(2), C = logits.size(3);
+  const int S = symbols.size(1);
+  torch::Tensor grad = torch::empty_like(logits);
+  void *stream = StreamOf(logits);
+  {
+    pybind11::gil_scoped_release release;
+    Check(k2amd_rnnt_logprobs_pruned_backward(logits.data_ptr(), norm.data_ptr(), px_grad.data_ptr(),
+                                              py_grad.data_ptr(), I64(symbols), I64(ranges),
+                                              I64(boundary), grad.data_ptr(), B, S, T, R, C,
+                                              termination_symbol, rnnt_type, DtypeCode(logits), stream));
+  }
+  return grad;
+}
+
+// device part of get_rnnt_prune_ranges; s_range is the final value
+torch::Tensor PruneRanges(torch::Tensor px_grad, torch::Tensor py_grad, torch::Tensor boundary,
+                          int s_range) {
+  RequireDevice(px_grad, "px_grad");
+  RequireDevice(py_grad, "py_grad");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(px_grad.device());
+  const int B = px_grad.size(0), S = px_grad.size(1), T1 = px_grad.size(2), T = py_grad.size(2);
+  torch::Tensor ranges = torch::empty({B, T, s_range}, px_grad.options().dtype(torch::kLong));
+  void *stream = StreamOf(px_grad);
+  {
+    pybind11::gil_scoped_release release;
+    Check(k2amd_rnnt_prune_ranges(px_grad.data_ptr(), py_grad.data_ptr(), I64(boundary),
+                                  ranges.data_ptr<int64_t>(), B, S, T, T1 == T ? 1 : 0, s_range,
+                                  DtypeCode(px_grad), stream));
+  }
+  return ranges;
+}
+
+torch::Tensor PruneGather(torch::Tensor lm, torch::Tensor ranges) {
+  RequireDevice(lm, "lm");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(lm.device());
+  const int B = lm.size(0), S1 = lm.size(1), D = lm.size(2), T = ranges.size(1), R = ranges.size(2);
+  torch::Tensor out = torch::empty({B, T, R, D}, lm.options());
+  void *stream = StreamOf(lm);
+  {
+    pybind11::gil_scoped_release release;
+    Check(k2amd_rnnt_prune_gather(lm.data_ptr(), I64(ranges), out.data_ptr(), B, S1, T, R, D,
+                                  DtypeCode(lm), stream));
+  }
+  return out;
+}
+
+torch::Tensor PruneGatherBackward(torch::Tensor grad, torch::Tensor ranges, int S1) {
+  RequireDevice(grad, "grad");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(grad.device());
+  const int B = grad.size(0), T = grad.size(1), R = grad.size(2), D = grad.size(3);
+  torch::Tensor lm_grad = torch::empty({B, S1, D}, grad.options());
+  void *stream = StreamOf(grad);
+  {
+    pybind11::gil_scoped_release release;
+    Check(k2amd_rnnt_prune_gather_backward(grad.data_ptr(), I64(ranges), lm_grad.data_ptr(), B, S1, T,
+                                           R, D, DtypeCode(grad), stream));
+  }
+  return lm_grad;
+}
+
 }  // namespace
 
 PYBIND11_MODULE(_k2_amd, m) {
@@ -160,4 +363,13 @@ PYBIND11_MODULE(_k2_amd, m) {
         pybind11::arg("py"), pybind11::arg("boundary"), pybind11::arg("p"),
         pybind11::arg("ans_grad"));
   m.def("version", []() { return k2amd_version(); });
+  m.def("logprobs_simple_forward", &LogprobsSimpleForward);
+  m.def("logprobs_simple_backward", &LogprobsSimpleBackward);
+  m.def("logprobs_joint_forward", &LogprobsJointForward);
+  m.def("logprobs_joint_backward", &LogprobsJointBackward);
+  m.def("logprobs_pruned_forward", &LogprobsPrunedForward);
+  m.def("logprobs_pruned_backward", &LogprobsPrunedBackward);
+  m.def("prune_ranges", &PruneRanges);
+  m.def("prune_gather", &PruneGather);
+  m.def("prune_gather_backward", &PruneGatherBackward);
 }

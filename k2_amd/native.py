@@ -1,7 +1,7 @@
 """The native entry points the Python layer calls, named after the reference's ``_k2`` functions.
 
 Backed by the pybind11 host module ``_k2_amd`` (C++ host code over the C-ABI of libk2amd.so)
-when it has been built, else by the ctypes binding of the same C-ABI.  Either way the work runs
+when it has been built, else by the ctypes binding of the same C-ABI (``capi.py``).  Either way the work runs
 in the HIP kernels; a missing libk2amd.so raises, nothing falls back to the CPU.
 """
 from typing import List, Optional
@@ -44,3 +44,81 @@ def mutual_information_backward(px: torch.Tensor, py: torch.Tensor,
                               None if boundary is None else boundary.contiguous(), p, ans_grad,
                               overwrite_ans_grad=True)
     return [gx, gy]
+
+
+# ---- the fused builders (replacements of the torch-op chains of k2/python/k2/rnnt_loss.py) ----
+# Same signatures and return values in both hosts; see capi.py for what each returns.
+
+def logprobs_simple_forward(lm, am, symbols, termination_symbol, rnnt_type, boundary):
+    _require_device(am)
+    if _ext is not None:
+        px, py, lm_probs, am_probs, denom = _ext.logprobs_simple_forward(
+            lm, am, symbols, termination_symbol, rnnt_type, boundary)
+        return px, py, (lm_probs, am_probs, denom)
+    return capi.logprobs_simple_forward(lm, am, symbols, termination_symbol, rnnt_type, boundary)
+
+
+def logprobs_simple_backward(px_grad, py_grad, symbols, boundary, saved, termination_symbol,
+                             rnnt_type):
+    _require_device(px_grad)
+    if _ext is not None:
+        lm_probs, am_probs, denom = saved
+        return tuple(_ext.logprobs_simple_backward(px_grad, py_grad, symbols, boundary, lm_probs,
+                                                   am_probs, denom, termination_symbol, rnnt_type))
+    return capi.logprobs_simple_backward(px_grad, py_grad, symbols, boundary, saved,
+                                         termination_symbol, rnnt_type)
+
+
+def logprobs_joint_forward(logits, symbols, termination_symbol, rnnt_type, boundary):
+    _require_device(logits)
+    if _ext is not None:
+        return tuple(_ext.logprobs_joint_forward(logits, symbols, termination_symbol, rnnt_type,
+                                                 boundary))
+    return capi.logprobs_joint_forward(logits, symbols, termination_symbol, rnnt_type, boundary)
+
+
+def logprobs_joint_backward(logits, norm, px_grad, py_grad, symbols, boundary, termination_symbol,
+                            rnnt_type):
+    if _ext is not None:
+        return _ext.logprobs_joint_backward(logits, norm, px_grad, py_grad, symbols, boundary,
+                                            termination_symbol, rnnt_type)
+    return capi.logprobs_joint_backward(logits, norm, px_grad, py_grad, symbols, boundary,
+                                        termination_symbol, rnnt_type)
+
+
+def logprobs_pruned_forward(logits, symbols, ranges, termination_symbol, boundary, rnnt_type):
+    _require_device(logits)
+    if _ext is not None:
+        return tuple(_ext.logprobs_pruned_forward(logits, symbols, ranges, termination_symbol,
+                                                  boundary, rnnt_type))
+    return capi.logprobs_pruned_forward(logits, symbols, ranges, termination_symbol, boundary,
+                                        rnnt_type)
+
+
+def logprobs_pruned_backward(logits, norm, px_grad, py_grad, symbols, ranges, boundary,
+                             termination_symbol, rnnt_type):
+    if _ext is not None:
+        return _ext.logprobs_pruned_backward(logits, norm, px_grad, py_grad, symbols, ranges,
+                                             boundary, termination_symbol, rnnt_type)
+    return capi.logprobs_pruned_backward(logits, norm, px_grad, py_grad, symbols, ranges, boundary,
+                                         termination_symbol, rnnt_type)
+
+
+def prune_ranges(px_grad, py_grad, boundary, s_range):
+    _require_device(px_grad)
+    if _ext is not None:
+        return _ext.prune_ranges(px_grad, py_grad, boundary, s_range)
+    return capi.prune_ranges(px_grad, py_grad, boundary, s_range)
+
+
+def prune_gather(lm, ranges):
+    _require_device(lm)
+    if _ext is not None:
+        return _ext.prune_gather(lm, ranges)
+    return capi.prune_gather(lm, ranges)
+
+
+def prune_gather_backward(grad, ranges, S1):
+    if _ext is not None:
+        return _ext.prune_gather_backward(grad, ranges, S1)
+    return capi.prune_gather_backward(grad, ranges, S1)

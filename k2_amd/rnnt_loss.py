@@ -10,7 +10,7 @@ from typing import Optional, Tuple, Union
 import torch
 from torch import Tensor
 
-from . import capi
+from . import capi, native
 from .mutual_information import mutual_information_recursion
 
 _RNNT_TYPES = ("regular", "modified", "constrained")
@@ -51,7 +51,7 @@ class _LogprobsSimple(torch.autograd.Function):
     @staticmethod
     def forward(ctx, lm, am, symbols, termination_symbol, rnnt_code, boundary):
         lm_c, am_c = lm.contiguous(), am.contiguous()
-        px, py, saved = capi.logprobs_simple_forward(lm_c, am_c, symbols, termination_symbol,
+        px, py, saved = native.logprobs_simple_forward(lm_c, am_c, symbols, termination_symbol,
                                                      rnnt_code, boundary)
         ctx.save_for_backward(*saved)
         ctx.meta = (symbols, boundary, termination_symbol, rnnt_code)
@@ -60,7 +60,7 @@ class _LogprobsSimple(torch.autograd.Function):
     @staticmethod
     def backward(ctx, px_grad, py_grad):
         symbols, boundary, termination_symbol, rnnt_code = ctx.meta
-        lm_grad, am_grad = capi.logprobs_simple_backward(
+        lm_grad, am_grad = native.logprobs_simple_backward(
             px_grad.contiguous(), py_grad.contiguous(), symbols, boundary, ctx.saved_tensors,
             termination_symbol, rnnt_code)
         return lm_grad, am_grad, None, None, None, None
@@ -70,7 +70,7 @@ class _LogprobsJoint(torch.autograd.Function):
     @staticmethod
     def forward(ctx, logits, symbols, termination_symbol, rnnt_code, boundary):
         logits_c = logits.contiguous()
-        px, py, norm = capi.logprobs_joint_forward(logits_c, symbols, termination_symbol,
+        px, py, norm = native.logprobs_joint_forward(logits_c, symbols, termination_symbol,
                                                    rnnt_code, boundary)
         ctx.save_for_backward(logits_c, norm)
         ctx.meta = (symbols, boundary, termination_symbol, rnnt_code)
@@ -80,7 +80,7 @@ class _LogprobsJoint(torch.autograd.Function):
     def backward(ctx, px_grad, py_grad):
         symbols, boundary, termination_symbol, rnnt_code = ctx.meta
         logits, norm = ctx.saved_tensors
-        grad = capi.logprobs_joint_backward(logits, norm, px_grad.contiguous(),
+        grad = native.logprobs_joint_backward(logits, norm, px_grad.contiguous(),
                                             py_grad.contiguous(), symbols, boundary,
                                             termination_symbol, rnnt_code)
         return grad, None, None, None, None
@@ -90,7 +90,7 @@ class _LogprobsPruned(torch.autograd.Function):
     @staticmethod
     def forward(ctx, logits, symbols, ranges, termination_symbol, rnnt_code, boundary):
         logits_c = logits.contiguous()
-        px, py, norm = capi.logprobs_pruned_forward(logits_c, symbols, ranges, termination_symbol,
+        px, py, norm = native.logprobs_pruned_forward(logits_c, symbols, ranges, termination_symbol,
                                                     boundary, rnnt_code)
         ctx.save_for_backward(logits_c, norm)
         ctx.meta = (symbols, ranges, boundary, termination_symbol, rnnt_code)
@@ -100,7 +100,7 @@ class _LogprobsPruned(torch.autograd.Function):
     def backward(ctx, px_grad, py_grad):
         symbols, ranges, boundary, termination_symbol, rnnt_code = ctx.meta
         logits, norm = ctx.saved_tensors
-        grad = capi.logprobs_pruned_backward(logits, norm, px_grad.contiguous(),
+        grad = native.logprobs_pruned_backward(logits, norm, px_grad.contiguous(),
                                              py_grad.contiguous(), symbols, ranges, boundary,
                                              termination_symbol, rnnt_code)
         return grad, None, None, None, None, None
@@ -111,12 +111,12 @@ class _PruneGather(torch.autograd.Function):
     def forward(ctx, lm, ranges):
         ctx.save_for_backward(ranges)
         ctx.S1 = lm.shape[1]
-        return capi.prune_gather(lm.contiguous(), ranges)
+        return native.prune_gather(lm.contiguous(), ranges)
 
     @staticmethod
     def backward(ctx, grad):
         (ranges,) = ctx.saved_tensors
-        return capi.prune_gather_backward(grad.contiguous(), ranges, ctx.S1), None
+        return native.prune_gather_backward(grad.contiguous(), ranges, ctx.S1), None
 
 
 def get_rnnt_logprobs(
@@ -283,7 +283,7 @@ def get_rnnt_prune_ranges(
         assert s_range >= 1, \
             f"Pruning range for modified RNN-T should be equal to or greater than 1, " \
             f"or no valid paths could survive pruning. Given {s_range}"
-    return capi.prune_ranges(px_grad.detach().contiguous(), py_grad.detach().contiguous(),
+    return native.prune_ranges(px_grad.detach().contiguous(), py_grad.detach().contiguous(),
                              _dev_i64(boundary, px_grad), int(s_range))
 
 

@@ -96,3 +96,26 @@ def test_pybind_host_module_mirrors_k2_native_functions():
     with pytest.raises(RuntimeError, match="3-dimensional"):
         _k2_amd.mutual_information_forward(px=torch.zeros(2, 9), py=torch.zeros(1, 3, 3),
                                            boundary=None, p=torch.zeros(1, 3, 4))
+
+
+def test_pybind_host_module_covers_every_builder_of_the_c_abi():
+    """Each k2amd_rnnt_* entry point has a C++ host function, the Python layer's `native` module
+    has a wrapper of the same name, and a host tensor is refused rather than computed on."""
+    import torch
+    from k2_amd import _k2_amd, native
+    names = ("logprobs_simple_forward", "logprobs_simple_backward", "logprobs_joint_forward",
+             "logprobs_joint_backward", "logprobs_pruned_forward", "logprobs_pruned_backward",
+             "prune_ranges", "prune_gather", "prune_gather_backward")
+    for n in names:
+        assert callable(getattr(_k2_amd, n)), n
+        assert callable(getattr(native, n)), n
+    sym = torch.zeros(1, 2, dtype=torch.int64)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        _k2_amd.logprobs_simple_forward(torch.zeros(1, 3, 5), torch.zeros(1, 4, 5), sym, 0, 0, None)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        _k2_amd.logprobs_joint_forward(torch.zeros(1, 4, 3, 5), sym, 0, 0, None)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        _k2_amd.prune_gather(torch.zeros(1, 3, 5), torch.zeros(1, 4, 2, dtype=torch.int64))
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        native.prune_ranges(torch.zeros(1, 2, 5), torch.zeros(1, 3, 4),
+                            torch.tensor([[0, 0, 2, 4]]), 2)
