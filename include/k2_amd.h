@@ -133,6 +133,20 @@ K2AMD_API int k2amd_rnnt_logprobs_pruned_backward(
     int B, int S, int T, int R, int C, int termination_symbol, int rnnt_type, int dtype,
     void *stream);
 
+/* Replaces get_hat_logprobs_pruned (k2/python/k2/rnnt_loss.py:992-1177), the hybrid autoregressive
+ * transducer variant that rnnt_loss_pruned(use_hat_loss=True) selects (rnnt_loss.py:1439-1447):
+ * the blank is column 0 and py = log sigmoid(logits[...,0]); normalizers [B][T][R] = logsumexp
+ * over columns 1..C-1; px = logits[..., symbol] - normalizers + log(1 - sigmoid(logits[...,0])).
+ * Placement, -inf fill, boundary fix and the "constrained" add are those of the pruned builder. */
+K2AMD_API int k2amd_rnnt_hat_logprobs_pruned_forward(
+    const void *logits, const int64_t *symbols, const int64_t *ranges, const int64_t *boundary,
+    void *px, void *py, void *normalizers, int B, int S, int T, int R, int C, int rnnt_type,
+    int dtype, void *stream);
+K2AMD_API int k2amd_rnnt_hat_logprobs_pruned_backward(
+    const void *logits, const void *normalizers, const void *px_grad, const void *py_grad,
+    const int64_t *symbols, const int64_t *ranges, const int64_t *boundary, void *logits_grad,
+    int B, int S, int T, int R, int C, int rnnt_type, int dtype, void *stream);
+
 /* ------------------------------------------------------------------ pruning
  *
  * Replaces the device work of get_rnnt_prune_ranges (k2/python/k2/rnnt_loss.py:730-780):

@@ -36,6 +36,8 @@ _SIGNATURES = {
     "k2amd_rnnt_logprobs_joint_backward": ([_vp] * 7 + [_ci] * 7 + [_vp], _ci),
     "k2amd_rnnt_logprobs_pruned_forward": ([_vp] * 7 + [_ci] * 8 + [_vp], _ci),
     "k2amd_rnnt_logprobs_pruned_backward": ([_vp] * 8 + [_ci] * 8 + [_vp], _ci),
+    "k2amd_rnnt_hat_logprobs_pruned_forward": ([_vp] * 7 + [_ci] * 7 + [_vp], _ci),
+    "k2amd_rnnt_hat_logprobs_pruned_backward": ([_vp] * 8 + [_ci] * 7 + [_vp], _ci),
     "k2amd_rnnt_prune_ranges": ([_vp] * 4 + [_ci] * 6 + [_vp], _ci),
     "k2amd_rnnt_prune_gather": ([_vp] * 3 + [_ci] * 6 + [_vp], _ci),
     "k2amd_rnnt_prune_gather_backward": ([_vp] * 3 + [_ci] * 6 + [_vp], _ci),
@@ -232,7 +234,9 @@ def logprobs_joint_backward(logits, norm, px_grad, py_grad, symbols, boundary,
     return grad
 
 
-def logprobs_pruned_forward(logits, symbols, ranges, termination_symbol, boundary, rnnt_type):
+def logprobs_pruned_forward(logits, symbols, ranges, termination_symbol, boundary, rnnt_type,
+                            hat=False):
+    """``hat`` selects get_hat_logprobs_pruned (blank = column 0, termination_symbol unused)."""
     B, T, R, C = logits.shape
     S = symbols.shape[1]
     dev, dt = logits.device, logits.dtype
@@ -240,6 +244,11 @@ def logprobs_pruned_forward(logits, symbols, ranges, termination_symbol, boundar
     py = torch.empty(B, S + 1, T, dtype=dt, device=dev)
     norm = torch.empty(B, T, R, dtype=dt, device=dev)
     with torch.cuda.device(dev):
+        if hat:
+            check(lib().k2amd_rnnt_hat_logprobs_pruned_forward(
+                ptr(logits), ptr(symbols), ptr(ranges), ptr(boundary), ptr(px), ptr(py), ptr(norm),
+                B, S, T, R, C, rnnt_type, dtype_code(logits), stream_ptr(dev)))
+            return px, py, norm
         check(lib().k2amd_rnnt_logprobs_pruned_forward(
             ptr(logits), ptr(symbols), ptr(ranges), ptr(boundary), ptr(px), ptr(py), ptr(norm),
             B, S, T, R, C, termination_symbol, rnnt_type, dtype_code(logits), stream_ptr(dev)))
@@ -247,12 +256,18 @@ def logprobs_pruned_forward(logits, symbols, ranges, termination_symbol, boundar
 
 
 def logprobs_pruned_backward(logits, norm, px_grad, py_grad, symbols, ranges, boundary,
-                             termination_symbol, rnnt_type):
+                             termination_symbol, rnnt_type, hat=False):
     B, T, R, C = logits.shape
     S = symbols.shape[1]
     grad = torch.empty_like(logits)
     dev = logits.device
     with torch.cuda.device(dev):
+        if hat:
+            check(lib().k2amd_rnnt_hat_logprobs_pruned_backward(
+                ptr(logits), ptr(norm), ptr(px_grad), ptr(py_grad), ptr(symbols), ptr(ranges),
+                ptr(boundary), ptr(grad), B, S, T, R, C, rnnt_type, dtype_code(logits),
+                stream_ptr(dev)))
+            return grad
         check(lib().k2amd_rnnt_logprobs_pruned_backward(
             ptr(logits), ptr(norm), ptr(px_grad), ptr(py_grad), ptr(symbols), ptr(ranges),
             ptr(boundary), ptr(grad), B, S, T, R, C, termination_symbol, rnnt_type,

@@ -262,11 +262,12 @@ torch::Tensor LogprobsJointBackward(torch::Tensor logits, torch::Tensor norm, to
   return grad;
 }
 
-// get_rnnt_logprobs_pruned: returns (px, py, normalizers)
+// get_rnnt_logprobs_pruned, or get_hat_logprobs_pruned with hat = true: returns
+// (px, py, normalizers)
 std::vector<torch::Tensor> LogprobsPrunedForward(torch::Tensor logits, torch::Tensor symbols,
                                                  torch::Tensor ranges, int termination_symbol,
                                                  torch::optional<torch::Tensor> boundary,
-                                                 int rnnt_type) {
+                                                 int rnnt_type, bool hat) {
   RequireDevice(logits, "logits");
   c10::hip::HIPGuardMasqueradingAsCUDA guard(logits.device());
   const int B = logits.size(0), T = logits.size(1), R = logits.size(2), C = logits.size(3);
@@ -277,10 +278,16 @@ std::vector<torch::Tensor> LogprobsPrunedForward(torch::Tensor logits, torch::Te
   void *stream = StreamOf(logits);
   {
     pybind11::gil_scoped_release release;
-    Check(k2amd_rnnt_logprobs_pruned_forward(logits.data_ptr(), I64(symbols), I64(ranges),
-                                             I64(boundary), px.data_ptr(), py.data_ptr(),
-                                             norm.data_ptr(), B, S, T, R, C, termination_symbol,
-                                             rnnt_type, DtypeCode(logits), stream));
+    if (hat)
+      Check(k2amd_rnnt_hat_logprobs_pruned_forward(logits.data_ptr(), I64(symbols), I64(ranges),
+                                                   I64(boundary), px.data_ptr(), py.data_ptr(),
+                                                   norm.data_ptr(), B, S, T, R, C, rnnt_type,
+                                                   DtypeCode(logits), stream));
+    else
+      Check(k2amd_rnnt_logprobs_pruned_forward(logits.data_ptr(), I64(symbols), I64(ranges),
+                                               I64(boundary), px.data_ptr(), py.data_ptr(),
+                                               norm.data_ptr(), B, S, T, R, C, termination_symbol,
+                                               rnnt_type, DtypeCode(logits), stream));
   }
   return {px, py, norm};
 }
@@ -288,7 +295,7 @@ std::vector<torch::Tensor> LogprobsPrunedForward(torch::Tensor logits, torch::Te
 torch::Tensor LogprobsPrunedBackward(torch::Tensor logits, torch::Tensor norm, torch::Tensor px_grad,
                                      torch::Tensor py_grad, torch::Tensor symbols, torch::Tensor ranges,
                                      torch::optional<torch::Tensor> boundary, int termination_symbol,
-                                     int rnnt_type) {
+                                     int rnnt_type, bool hat) {
   RequireDevice(logits, "logits");
   RequireDevice(px_grad, "px_grad");
   RequireDevice(py_grad, "py_grad");
@@ -299,10 +306,16 @@ torch::Tensor LogprobsPrunedBackward(torch::Tensor logits, torch::Tensor norm, t
   void *stream = StreamOf(logits);
   {
     pybind11::gil_scoped_release release;
-    Check(k2amd_rnnt_logprobs_pruned_backward(logits.data_ptr(), norm.data_ptr(), px_grad.data_ptr(),
-                                              py_grad.data_ptr(), I64(symbols), I64(ranges),
-                                              I64(boundary), grad.data_ptr(), B, S, T, R, C,
-                                              termination_symbol, rnnt_type, DtypeCode(logits), stream));
+    if (hat)
+      Check(k2amd_rnnt_hat_logprobs_pruned_backward(
+          logits.data_ptr(), norm.data_ptr(), px_grad.data_ptr(), py_grad.data_ptr(), I64(symbols),
+          I64(ranges), I64(boundary), grad.data_ptr(), B, S, T, R, C, rnnt_type, DtypeCode(logits),
+          stream));
+    else
+      Check(k2amd_rnnt_logprobs_pruned_backward(
+          logits.data_ptr(), norm.data_ptr(), px_grad.data_ptr(), py_grad.data_ptr(), I64(symbols),
+          I64(ranges), I64(boundary), grad.data_ptr(), B, S, T, R, C, termination_symbol, rnnt_type,
+          DtypeCode(logits), stream));
   }
   return grad;
 }

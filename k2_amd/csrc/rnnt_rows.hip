@@ -1,6 +1,7 @@
 // Row-streaming kernels of the RNN-T log-prob builders that take joiner logits:
 //   get_rnnt_logprobs_joint   logits [B][T][S+1][C]   (k2/python/k2/rnnt_loss.py:341-447)
 //   get_rnnt_logprobs_pruned  logits [B][T][R][C]     (k2/python/k2/rnnt_loss.py:1180-1348)
+//   get_hat_logprobs_pruned   logits [B][T][R][C]     (k2/python/k2/rnnt_loss.py:992-1177)
 //
 // Both are one streaming pass over the logits, one 64-lane wavefront per row of C logits held
 // in registers (max and sum(exp) reduced across lanes), plus a small pass with one THREAD per
@@ -54,7 +55,8 @@ __device__ __forceinline__ bool RowIsVectorisable(int C) {
 
 // logsumexp of one vectorisable row held in registers; same semantics as RowLogSumExp below
 template <typename T>
-__device__ __forceinline__ T RowLogSumExpVec(const T *__restrict__ x, int C, int lane) {
+__device__ __forceinline__ T RowLogSumExpVec(const T *__restrict__ x, int C, int lane,
+                                             bool skip_first) {
   typedef typename Vec16<T>::type V;
   constexpr int kN = Vec16<T>::kN;
   const int nv = C / kN;
@@ -70,6 +72,7 @@ __device__ __forceinline__ T RowLogSumExpVec(const T *__restrict__ x, int C, int
 #pragma unroll
       for (int e = 0; e < kN; ++e) v[i][e] = Real<T>::NegInf();
     }
+    if (i == 0 && skip_first && lane == 0) v[0][0] = Real<T>::NegInf();  // column 0 left out
 #pragma unroll
     for (int e = 0; e < kN; ++e) m = max(m, v[i][e]);
   }
@@ -87,15 +90,17 @@ __device__ __forceinline__ T RowLogSumExpVec(const T *__restrict__ x, int C, int
 // logsumexp of one row, torch semantics (an infinite maximum is replaced by 0 before the
 // subtraction, so an all -inf row yields -inf rather than NaN).
 template <typename T>
-__device__ __forceinline__ T RowLogSumExp(const T *__restrict__ x, int C, int lane) {
+__device__ __forceinline__ T RowLogSumExp(const T *__restrict__ x, int C, int lane,
+                                          bool skip_first) {
   T m = Real<T>::NegInf();
   T sum = 0;
+  const int first = skip_first ? 1 : 0;
   if (C <= kWave * kMaxRegs) {
     T v[kMaxRegs];
 #pragma unroll
     for (int i = 0; i < kMaxRegs; ++i) {
       const int c = lane + i * kWave;
-      v[i] = c < C ? x[c] : Real<T>::NegInf();
+      v[i] = (c < C && c >= first) ? x[c] : Real<T>::NegInf();
       m = max(m, v[i]);
     }
     m = WaveMax(m);
@@ -103,10 +108,10 @@ __device__ __forceinline__ T RowLogSumExp(const T *__restrict__ x, int C, int la
 #pragma unroll
     for (int i = 0; i < kMaxRegs; ++i) sum += Real<T>::Exp(v[i] - m);
   } else {
-    for (int c = lane; c < C; c += kWave) m = max(m, x[c]);
+    for (int c = lane + first; c < C; c += kWave) m = max(m, x[c]);
     m = WaveMax(m);
     if (m - m != 0) m = 0;
-    for (int c = lane; c < C; c += kWave) sum += Real<T>::Exp(x[c] - m);
+    for (int c = lane + first; c < C; c += kWave) sum += Real<T>::Exp(x[c] - m);
   }
   sum = WaveSum(sum);
   return Real<T>::Log(sum) + m;
@@ -115,7 +120,19 @@ __device__ __forceinline__ T RowLogSumExp(const T *__restrict__ x, int C, int la
 struct RowGeom {
   int B, S, Tn, K, C;  // K rows per frame: S+1 (joint) or R (pruned)
   int blank, rnnt_type;
+  int hat;  // 1: hybrid autoregressive transducer, column 0 is the blank and has its own sigmoid
 };
+
+// log sigmoid(x) = min(x, 0) - log1p(exp(-|x|)), and sigmoid(x) without overflow
+template <typename T>
+__device__ __forceinline__ T LogSigmoid(T x) {
+  return min(x, T(0)) - Real<T>::Log1p(Real<T>::Exp(-fabs(x)));
+}
+template <typename T>
+__device__ __forceinline__ T Sigmoid(T x) {
+  const T e = Real<T>::Exp(-fabs(x));
+  return (x >= 0 ? T(1) : e) / (T(1) + e);
+}
 
 // Maps row (b,t,k) to its lattice row s and to the symbol whose log-prob goes to px.
 template <bool kPruned>
@@ -145,17 +162,21 @@ __device__ __forceinline__ void RowTarget(const RowGeom &g, const int64_t *__res
 // rather than once per LANE (64 rows, pass 2) cost a third of this kernel's time.
 template <typename T>
 __global__ __launch_bounds__(kRowsPerBlock *kWave) void RowNormKernel(
-    const T *__restrict__ logits, T *__restrict__ normalizers, long long rows, int C) {
+    const T *__restrict__ logits, T *__restrict__ normalizers, long long rows, int C,
+    bool skip_first) {
   const int lane = threadIdx.x & (kWave - 1);
   const long long row = (long long)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
   if (row >= rows) return;
   const T *x = logits + (size_t)row * C;
-  const T norm = RowIsVectorisable<T>(C) ? RowLogSumExpVec<T>(x, C, lane) : RowLogSumExp<T>(x, C, lane);
+  const T norm = RowIsVectorisable<T>(C) ? RowLogSumExpVec<T>(x, C, lane, skip_first)
+                                         : RowLogSumExp<T>(x, C, lane, skip_first);
   if (lane == 0) normalizers[row] = norm;
 }
 
 // Forward, pass 2: one thread per row looks up where the row lands and writes
-//   px[b,s,t] = logits[row, sym] - norm,   py[b,s,t] = logits[row, blank] - norm.
+//   px[b,s,t] = logits[row, sym] - norm,   py[b,s,t] = logits[row, blank] - norm,
+// or, for the hybrid autoregressive transducer (norm then covers columns 1..C-1 only),
+//   py = log sigmoid(logits[row, 0]),  px = logits[row, sym] - norm + (py - logits[row, 0]).
 template <typename T, bool kPruned>
 __global__ void RowEmitKernel(const T *__restrict__ logits, const T *__restrict__ normalizers,
                               const int64_t *__restrict__ symbols, const int64_t *__restrict__ ranges,
@@ -172,13 +193,21 @@ __global__ void RowEmitKernel(const T *__restrict__ logits, const T *__restrict_
   RowTarget<kPruned>(g, symbols, ranges, b, t, k, &s, &sym);
   const T norm = normalizers[row];
   const int T1 = g.rnnt_type == K2AMD_REGULAR ? g.Tn + 1 : g.Tn;
+  T shift = 0, yv;
+  if (g.hat) {
+    const T x0 = x[0];
+    yv = LogSigmoid(x0);
+    shift = yv - x0;  // log(1 - sigmoid(x0))
+  } else {
+    yv = x[g.blank] - norm;
+  }
   if (s < g.S) {
-    T v = (sym >= 0 && sym < g.C) ? x[sym] - norm : Real<T>::NegInf();
+    T v = (sym >= 0 && sym < g.C) ? (x[sym] - norm) + shift : Real<T>::NegInf();
     if (g.rnnt_type == K2AMD_REGULAR && boundary != nullptr && boundary[4 * b + 3] == t)
       v = Real<T>::NegInf();
     px[((size_t)b * g.S + s) * T1 + t] = v;
   }
-  py[((size_t)b * (g.S + 1) + s) * g.Tn + t] = x[g.blank] - norm;
+  py[((size_t)b * (g.S + 1) + s) * g.Tn + t] = yv;
 }
 
 template <typename T>
@@ -246,9 +275,33 @@ __global__ void RowGradPrepKernel(const T *__restrict__ normalizers, const T *__
   rec[3] = normalizers[row];
 }
 
+// What one row's gradient is made of.  Softmax rows:
+//   d/d logits[c] = -softmax[c] (gx + gy) + gx [c == sym] + gy [c == blank].
+// Hybrid autoregressive transducer rows (norm covers columns 1..C-1, sg = sigmoid(logits[0])):
+//   d/d logits[c >= 1] = gx ([c == sym] - exp(logits[c] - norm)),
+//   d/d logits[0]      = gy (1 - sg) - gx sg + gx [sym == 0].
+template <typename T, bool kHat>
+struct RowGradTerms {
+  T gx, gy, norm, sg;
+  int sym, blank;
+  template <bool kFast>
+  __device__ __forceinline__ T At(T x, int c) const {
+    const T p = kFast ? FastExp(x - norm) : Real<T>::Exp(x - norm);
+    T v;
+    if (kHat) {
+      v = c == 0 ? gy * (T(1) - sg) - gx * sg : -p * gx;
+    } else {
+      v = -p * (gx + gy);
+      if (c == blank) v += gy;
+    }
+    if (c == sym) v += gx;
+    return v;
+  }
+};
+
 // Backward, pass 2: one wavefront per row reads the row and its parked record, and writes the
 // gradient over the whole slot (record included; every lane has read it by then).
-template <typename T>
+template <typename T, bool kHat>
 __global__ __launch_bounds__(kRowsPerBlock *kWave) void RowGradKernel(
     const T *__restrict__ logits, T *__restrict__ logits_grad, long long rows, int C, int blank) {
   const int lane = threadIdx.x & (kWave - 1);
@@ -269,9 +322,13 @@ __global__ __launch_bounds__(kRowsPerBlock *kWave) void RowGradKernel(
       if (q < nv) in[i] = xv[q];
     }
   }
-  const T gx = dx[0], gy = dx[1], norm = dx[3];
-  const int sym = (int)dx[2];
-  const T tot = gx + gy;
+  RowGradTerms<T, kHat> terms;
+  terms.gx = dx[0];
+  terms.gy = dx[1];
+  terms.sym = (int)dx[2];
+  terms.norm = dx[3];
+  terms.blank = blank;
+  terms.sg = kHat ? Sigmoid(x[0]) : T(0);
   if (vectorised) {
     V *dv = reinterpret_cast<V *>(dx);
     V outv[kMaxVecs];
@@ -282,13 +339,7 @@ __global__ __launch_bounds__(kRowsPerBlock *kWave) void RowGradKernel(
         T e[kN];
         Unpack(in[i], e);
 #pragma unroll
-        for (int k2 = 0; k2 < kN; ++k2) {
-          const int c = q * kN + k2;
-          T v = -FastExp(e[k2] - norm) * tot;
-          if (c == sym) v += gx;
-          if (c == blank) v += gy;
-          e[k2] = v;
-        }
+        for (int k2 = 0; k2 < kN; ++k2) e[k2] = terms.template At<true>(e[k2], q * kN + k2);
         outv[i] = Pack(e);
       }
     }
@@ -301,16 +352,11 @@ __global__ __launch_bounds__(kRowsPerBlock *kWave) void RowGradKernel(
   }
   // rows that are not read as vectors: every lane holds the record in registers before the
   // first store of the loop below can reach it (a wavefront's loads complete in order)
-  for (int c = lane; c < C; c += kWave) {
-    T v = -Real<T>::Exp(x[c] - norm) * tot;
-    if (c == sym) v += gx;
-    if (c == blank) v += gy;
-    dx[c] = v;
-  }
+  for (int c = lane; c < C; c += kWave) dx[c] = terms.template At<false>(x[c], c);
 }
 
 // The same in one pass, for rows too short to park a record in (C < 4).
-template <typename T, bool kPruned>
+template <typename T, bool kPruned, bool kHat>
 __global__ __launch_bounds__(kRowsPerBlock *kWave) void RowBackwardKernel(
     const T *__restrict__ logits, const T *__restrict__ normalizers,
     const T *__restrict__ px_grad, const T *__restrict__ py_grad,
@@ -332,51 +378,22 @@ __global__ __launch_bounds__(kRowsPerBlock *kWave) void RowBackwardKernel(
     const bool cut =
         g.rnnt_type == K2AMD_REGULAR && boundary != nullptr && boundary[4 * b + 3] == t;
     if (!cut) gx = px_grad[((size_t)b * g.S + s) * T1 + t];
+  } else {
+    sym = -1;
   }
   T gy = py_grad[((size_t)b * (g.S + 1) + s) * g.Tn + t];
   if (g.rnnt_type == K2AMD_CONSTRAINED && s >= 1)
     gy += px_grad[((size_t)b * g.S + (s - 1)) * T1 + t];  // px += py[:, 1:]
-  const T norm = normalizers[row];
-  const T tot = gx + gy;
   const T *x = logits + (size_t)row * g.C;
   T *dx = logits_grad + (size_t)row * g.C;
-  if (RowIsVectorisable<T>(g.C)) {
-    typedef typename Vec16<T>::type V;
-    constexpr int kN = Vec16<T>::kN;
-    const int nv = g.C / kN;
-    const V *xv = reinterpret_cast<const V *>(x);
-    V *dv = reinterpret_cast<V *>(dx);
-    V in[kMaxVecs];
-#pragma unroll
-    for (int i = 0; i < kMaxVecs; ++i) {
-      const int q = lane + i * kWave;
-      if (q < nv) in[i] = xv[q];
-    }
-#pragma unroll
-    for (int i = 0; i < kMaxVecs; ++i) {
-      const int q = lane + i * kWave;
-      if (q < nv) {
-        T e[kN];
-        Unpack(in[i], e);
-#pragma unroll
-        for (int k2 = 0; k2 < kN; ++k2) {
-          const int c = q * kN + k2;
-          T v = -FastExp(e[k2] - norm) * tot;
-          if (c == sym) v += gx;
-          if (c == g.blank) v += gy;
-          e[k2] = v;
-        }
-        dv[q] = Pack(e);
-      }
-    }
-    return;
-  }
-  for (int c = lane; c < g.C; c += kWave) {
-    T v = -Real<T>::Exp(x[c] - norm) * tot;
-    if (c == sym) v += gx;
-    if (c == g.blank) v += gy;
-    dx[c] = v;
-  }
+  RowGradTerms<T, kHat> terms;
+  terms.gx = gx;
+  terms.gy = gy;
+  terms.sym = sym;
+  terms.norm = normalizers[row];
+  terms.blank = g.blank;
+  terms.sg = kHat ? Sigmoid(x[0]) : T(0);
+  for (int c = lane; c < g.C; c += kWave) dx[c] = terms.template At<false>(x[c], c);
 }
 
 template <typename T, bool kPruned>
@@ -395,7 +412,7 @@ int RowForward(const T *logits, const int64_t *symbols, const int64_t *ranges,
   if (rows > 0) {
     const long long blocks = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
     hipLaunchKernelGGL((RowNormKernel<T>), dim3((unsigned)blocks), dim3(kRowsPerBlock * kWave), 0, stream,
-                       logits, normalizers, rows, g.C);
+                       logits, normalizers, rows, g.C, g.hat != 0);
     hipLaunchKernelGGL((RowEmitKernel<T, kPruned>), dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, stream,
                        logits, (const T *)normalizers, symbols, ranges, boundary, px, py, g);
   }
@@ -404,7 +421,7 @@ int RowForward(const T *logits, const int64_t *symbols, const int64_t *ranges,
   return LaunchStatus();
 }
 
-template <typename T, bool kPruned>
+template <typename T, bool kPruned, bool kHat>
 int RowBackward(const T *logits, const T *normalizers, const T *px_grad, const T *py_grad,
                 const int64_t *symbols, const int64_t *ranges, const int64_t *boundary,
                 T *logits_grad, RowGeom g, hipStream_t stream) {
@@ -414,10 +431,10 @@ int RowBackward(const T *logits, const T *normalizers, const T *px_grad, const T
     if (g.C >= 4) {
       hipLaunchKernelGGL((RowGradPrepKernel<T, kPruned>), dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, stream,
                          normalizers, px_grad, py_grad, symbols, ranges, boundary, logits_grad, g);
-      hipLaunchKernelGGL((RowGradKernel<T>), dim3((unsigned)blocks), dim3(kRowsPerBlock * kWave), 0, stream,
+      hipLaunchKernelGGL((RowGradKernel<T, kHat>), dim3((unsigned)blocks), dim3(kRowsPerBlock * kWave), 0, stream,
                          logits, logits_grad, rows, g.C, g.blank);
     } else {
-      hipLaunchKernelGGL((RowBackwardKernel<T, kPruned>), dim3((unsigned)blocks), dim3(kRowsPerBlock * kWave), 0, stream,
+      hipLaunchKernelGGL((RowBackwardKernel<T, kPruned, kHat>), dim3((unsigned)blocks), dim3(kRowsPerBlock * kWave), 0, stream,
                          logits, normalizers, px_grad, py_grad, symbols, ranges, boundary,
                          logits_grad, g);
     }
@@ -446,7 +463,7 @@ int k2amd_rnnt_logprobs_joint_forward(const void *logits, const int64_t *symbols
                                       int termination_symbol, int rnnt_type, int dtype,
                                       void *stream) {
   if (!GeomOk(B, S, T, S + 1, C, termination_symbol, rnnt_type, dtype)) return K2AMD_ERR_INVALID_ARGUMENT;
-  RowGeom g{B, S, T, S + 1, C, termination_symbol, rnnt_type};
+  RowGeom g{B, S, T, S + 1, C, termination_symbol, rnnt_type, 0};
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == K2AMD_F32)
     return RowForward<float, false>((const float *)logits, symbols, nullptr, boundary, (float *)px, (float *)py, (float *)normalizers, g, st);
@@ -460,11 +477,11 @@ int k2amd_rnnt_logprobs_joint_backward(const void *logits, const void *normalize
                                        int termination_symbol, int rnnt_type, int dtype,
                                        void *stream) {
   if (!GeomOk(B, S, T, S + 1, C, termination_symbol, rnnt_type, dtype)) return K2AMD_ERR_INVALID_ARGUMENT;
-  RowGeom g{B, S, T, S + 1, C, termination_symbol, rnnt_type};
+  RowGeom g{B, S, T, S + 1, C, termination_symbol, rnnt_type, 0};
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == K2AMD_F32)
-    return RowBackward<float, false>((const float *)logits, (const float *)normalizers, (const float *)px_grad, (const float *)py_grad, symbols, nullptr, boundary, (float *)logits_grad, g, st);
-  return RowBackward<double, false>((const double *)logits, (const double *)normalizers, (const double *)px_grad, (const double *)py_grad, symbols, nullptr, boundary, (double *)logits_grad, g, st);
+    return RowBackward<float, false, false>((const float *)logits, (const float *)normalizers, (const float *)px_grad, (const float *)py_grad, symbols, nullptr, boundary, (float *)logits_grad, g, st);
+  return RowBackward<double, false, false>((const double *)logits, (const double *)normalizers, (const double *)px_grad, (const double *)py_grad, symbols, nullptr, boundary, (double *)logits_grad, g, st);
 }
 
 int k2amd_rnnt_logprobs_pruned_forward(const void *logits, const int64_t *symbols,
@@ -473,7 +490,7 @@ int k2amd_rnnt_logprobs_pruned_forward(const void *logits, const int64_t *symbol
                                        int C, int termination_symbol, int rnnt_type, int dtype,
                                        void *stream) {
   if (!GeomOk(B, S, T, R, C, termination_symbol, rnnt_type, dtype) || R < 1 || R > S + 1) return K2AMD_ERR_INVALID_ARGUMENT;
-  RowGeom g{B, S, T, R, C, termination_symbol, rnnt_type};
+  RowGeom g{B, S, T, R, C, termination_symbol, rnnt_type, 0};
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == K2AMD_F32)
     return RowForward<float, true>((const float *)logits, symbols, ranges, boundary, (float *)px, (float *)py, (float *)normalizers, g, st);
@@ -487,11 +504,38 @@ int k2amd_rnnt_logprobs_pruned_backward(const void *logits, const void *normaliz
                                         int T, int R, int C, int termination_symbol, int rnnt_type,
                                         int dtype, void *stream) {
   if (!GeomOk(B, S, T, R, C, termination_symbol, rnnt_type, dtype) || R < 1 || R > S + 1) return K2AMD_ERR_INVALID_ARGUMENT;
-  RowGeom g{B, S, T, R, C, termination_symbol, rnnt_type};
+  RowGeom g{B, S, T, R, C, termination_symbol, rnnt_type, 0};
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == K2AMD_F32)
-    return RowBackward<float, true>((const float *)logits, (const float *)normalizers, (const float *)px_grad, (const float *)py_grad, symbols, ranges, boundary, (float *)logits_grad, g, st);
-  return RowBackward<double, true>((const double *)logits, (const double *)normalizers, (const double *)px_grad, (const double *)py_grad, symbols, ranges, boundary, (double *)logits_grad, g, st);
+    return RowBackward<float, true, false>((const float *)logits, (const float *)normalizers, (const float *)px_grad, (const float *)py_grad, symbols, ranges, boundary, (float *)logits_grad, g, st);
+  return RowBackward<double, true, false>((const double *)logits, (const double *)normalizers, (const double *)px_grad, (const double *)py_grad, symbols, ranges, boundary, (double *)logits_grad, g, st);
+}
+
+int k2amd_rnnt_hat_logprobs_pruned_forward(const void *logits, const int64_t *symbols,
+                                           const int64_t *ranges, const int64_t *boundary,
+                                           void *px, void *py, void *normalizers, int B, int S,
+                                           int T, int R, int C, int rnnt_type, int dtype,
+                                           void *stream) {
+  if (!GeomOk(B, S, T, R, C, 0, rnnt_type, dtype) || R < 1 || R > S + 1) return K2AMD_ERR_INVALID_ARGUMENT;
+  RowGeom g{B, S, T, R, C, 0, rnnt_type, 1};
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == K2AMD_F32)
+    return RowForward<float, true>((const float *)logits, symbols, ranges, boundary, (float *)px, (float *)py, (float *)normalizers, g, st);
+  return RowForward<double, true>((const double *)logits, symbols, ranges, boundary, (double *)px, (double *)py, (double *)normalizers, g, st);
+}
+
+int k2amd_rnnt_hat_logprobs_pruned_backward(const void *logits, const void *normalizers,
+                                            const void *px_grad, const void *py_grad,
+                                            const int64_t *symbols, const int64_t *ranges,
+                                            const int64_t *boundary, void *logits_grad, int B,
+                                            int S, int T, int R, int C, int rnnt_type, int dtype,
+                                            void *stream) {
+  if (!GeomOk(B, S, T, R, C, 0, rnnt_type, dtype) || R < 1 || R > S + 1) return K2AMD_ERR_INVALID_ARGUMENT;
+  RowGeom g{B, S, T, R, C, 0, rnnt_type, 1};
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == K2AMD_F32)
+    return RowBackward<float, true, true>((const float *)logits, (const float *)normalizers, (const float *)px_grad, (const float *)py_grad, symbols, ranges, boundary, (float *)logits_grad, g, st);
+  return RowBackward<double, true, true>((const double *)logits, (const double *)normalizers, (const double *)px_grad, (const double *)py_grad, symbols, ranges, boundary, (double *)logits_grad, g, st);
 }
 
 }  // extern "C"

@@ -86,22 +86,23 @@ def logprobs_joint_backward(logits, norm, px_grad, py_grad, symbols, boundary, t
                                         termination_symbol, rnnt_type)
 
 
-def logprobs_pruned_forward(logits, symbols, ranges, termination_symbol, boundary, rnnt_type):
+def logprobs_pruned_forward(logits, symbols, ranges, termination_symbol, boundary, rnnt_type,
+                            hat=False):
     _require_device(logits)
     if _ext is not None:
         return tuple(_ext.logprobs_pruned_forward(logits, symbols, ranges, termination_symbol,
-                                                  boundary, rnnt_type))
+                                                  boundary, rnnt_type, hat))
     return capi.logprobs_pruned_forward(logits, symbols, ranges, termination_symbol, boundary,
-                                        rnnt_type)
+                                        rnnt_type, hat)
 
 
 def logprobs_pruned_backward(logits, norm, px_grad, py_grad, symbols, ranges, boundary,
-                             termination_symbol, rnnt_type):
+                             termination_symbol, rnnt_type, hat=False):
     if _ext is not None:
         return _ext.logprobs_pruned_backward(logits, norm, px_grad, py_grad, symbols, ranges,
-                                             boundary, termination_symbol, rnnt_type)
+                                             boundary, termination_symbol, rnnt_type, hat)
     return capi.logprobs_pruned_backward(logits, norm, px_grad, py_grad, symbols, ranges, boundary,
-                                         termination_symbol, rnnt_type)
+                                         termination_symbol, rnnt_type, hat)
 
 
 def prune_ranges(px_grad, py_grad, boundary, s_range):

@@ -88,22 +88,22 @@ class _LogprobsJoint(torch.autograd.Function):
 
 class _LogprobsPruned(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, logits, symbols, ranges, termination_symbol, rnnt_code, boundary):
+    def forward(ctx, logits, symbols, ranges, termination_symbol, rnnt_code, boundary, hat=False):
         logits_c = logits.contiguous()
         px, py, norm = native.logprobs_pruned_forward(logits_c, symbols, ranges, termination_symbol,
-                                                    boundary, rnnt_code)
+                                                      boundary, rnnt_code, hat)
         ctx.save_for_backward(logits_c, norm)
-        ctx.meta = (symbols, ranges, boundary, termination_symbol, rnnt_code)
+        ctx.meta = (symbols, ranges, boundary, termination_symbol, rnnt_code, hat)
         return px, py
 
     @staticmethod
     def backward(ctx, px_grad, py_grad):
-        symbols, ranges, boundary, termination_symbol, rnnt_code = ctx.meta
+        symbols, ranges, boundary, termination_symbol, rnnt_code, hat = ctx.meta
         logits, norm = ctx.saved_tensors
         grad = native.logprobs_pruned_backward(logits, norm, px_grad.contiguous(),
-                                             py_grad.contiguous(), symbols, ranges, boundary,
-                                             termination_symbol, rnnt_code)
-        return grad, None, None, None, None, None
+                                               py_grad.contiguous(), symbols, ranges, boundary,
+                                               termination_symbol, rnnt_code, hat)
+        return grad, None, None, None, None, None, None
 
 
 class _PruneGather(torch.autograd.Function):
@@ -333,6 +333,31 @@ def get_rnnt_logprobs_pruned(
                                  _dev_i64(boundary, logits))
 
 
+def get_hat_logprobs_pruned(
+    logits: Tensor,
+    symbols: Tensor,
+    ranges: Tensor,
+    termination_symbol: int,
+    boundary: Tensor,
+    rnnt_type: str = "regular",
+) -> Tuple[Tensor, Tensor]:
+    """k2.get_hat_logprobs_pruned (k2/python/k2/rnnt_loss.py:992-1177), the hybrid autoregressive
+    transducer: the blank (column 0) has its own sigmoid, py = logsigmoid(logits[..., 0]), and the
+    other symbols share a softmax over columns 1..C-1 scaled by 1 - sigmoid(logits[..., 0])."""
+    assert logits.ndim == 4, logits.shape
+    (B, T, s_range, C) = logits.shape
+    assert ranges.shape == (B, T, s_range), (ranges.shape, B, T, s_range)
+    (B, S) = symbols.shape
+    assert S >= 0, S
+    assert rnnt_type != "modified" or T >= S, \
+        f"Modified transducer requires T >= S, but got T={T} and S={S}"
+    assert rnnt_type in _RNNT_TYPES, rnnt_type
+    assert termination_symbol == 0, \
+        f"Termination symbol must be 0, but got {termination_symbol}"
+    return _LogprobsPruned.apply(logits, _dev_i64(symbols, logits), _dev_i64(ranges, logits), 0,
+                                 capi.RNNT_TYPES[rnnt_type], _dev_i64(boundary, logits), True)
+
+
 def rnnt_loss_pruned(
     logits: Tensor,
     symbols: Tensor,
@@ -344,14 +369,151 @@ def rnnt_loss_pruned(
     reduction: Optional[str] = "mean",
     use_hat_loss: bool = False,
 ) -> Tensor:
-    """k2.rnnt_loss_pruned (k2/python/k2/rnnt_loss.py:1351-1468).  The HAT variant
-    (use_hat_loss=True) is not part of this build."""
-    if use_hat_loss:
-        raise NotImplementedError("k2_amd: use_hat_loss=True (get_hat_logprobs_pruned) is not built")
-    px, py = get_rnnt_logprobs_pruned(logits=logits, symbols=symbols, ranges=ranges,
-                                      termination_symbol=termination_symbol, boundary=boundary,
-                                      rnnt_type=rnnt_type)
+    """k2.rnnt_loss_pruned (k2/python/k2/rnnt_loss.py:1351-1468); ``use_hat_loss`` switches the
+    builder to get_hat_logprobs_pruned (:1430-1447)."""
+    builder = get_hat_logprobs_pruned if use_hat_loss else get_rnnt_logprobs_pruned
+    px, py = builder(logits=logits, symbols=symbols, ranges=ranges,
+                     termination_symbol=termination_symbol, boundary=boundary,
+                     rnnt_type=rnnt_type)
     if delay_penalty > 0.0:
         px = _delay_penalty(px, boundary, rnnt_type, delay_penalty)
     negated_loss = mutual_information_recursion(px=px, py=py, boundary=boundary)
     return _reduce(negated_loss, reduction)
+
+
+def get_rnnt_logprobs_smoothed(
+    lm: Tensor,
+    am: Tensor,
+    symbols: Tensor,
+    termination_symbol: int,
+    lm_only_scale: float = 0.1,
+    am_only_scale: float = 0.1,
+    boundary: Optional[Tensor] = None,
+    rnnt_type: str = "regular",
+) -> Tuple[Tensor, Tensor]:
+    """k2.get_rnnt_logprobs_smoothed (k2/python/k2/rnnt_loss.py:1471-1704): interpolates, in the
+    log domain, the joint log-probs with "lm only" log-probs and "am only" log-probs (the latter
+    against a unigram lm averaged over the batch).
+
+    Not on the accelerated path's critical list: the joint part (the only one of size
+    [B][S+1][T] x C) is the fused kernel of get_rnnt_logprobs; the two marginal parts are a few
+    torch ops on the device over [B][S+1][C] and [B][T][C]."""
+    assert lm.ndim == 3, lm.shape
+    assert am.ndim == 3, am.shape
+    assert lm.shape[0] == am.shape[0], (lm.shape, am.shape)
+    assert lm.shape[2] == am.shape[2], (lm.shape, am.shape)
+    (B, T, C) = am.shape
+    S = lm.shape[1] - 1
+    assert symbols.shape == (B, S), (symbols.shape, B, S)
+    assert rnnt_type in _RNNT_TYPES, rnnt_type
+    _validate_st_lengths(S, T, rnnt_type == "regular", boundary)
+    regular = rnnt_type == "regular"
+    symbols = _dev_i64(symbols, am)
+    blank = int(termination_symbol)
+
+    # joint part, before the boundary fix / the "constrained" add (both come after interpolation)
+    px, py = _LogprobsSimple.apply(lm, am, symbols, blank,
+                                   capi.RNNT_TYPES["regular" if regular else "modified"], None)
+
+    tiny = torch.finfo(lm.dtype).tiny
+    am_top = am.amax(dim=2, keepdim=True)                        # [B][T][1]
+    lm_top = lm.amax(dim=2, keepdim=True)                        # [B][S+1][1]
+    am_lin = (am - am_top).exp()
+    lm_lin = (lm - lm_top).exp()
+    lm_mass = lm_lin.sum(dim=2, keepdim=True)                    # [B][S+1][1]
+    unigram = (lm_lin / lm_mass).mean(dim=(0, 1)) + tiny         # [C]
+    am_only_norm = (torch.mv(am_lin.reshape(-1, C), unigram).reshape(B, 1, T).log()
+                    + am_top.transpose(1, 2))                    # [B][1][T]
+    log_unigram = unigram.log()
+    lm_only_norm = lm_mass.log() + lm_top                        # [B][S+1][1]
+
+    sym_am = torch.gather(am.transpose(1, 2), 1, symbols.unsqueeze(2).expand(B, S, T))  # [B][S][T]
+    sym_lm = torch.gather(lm[:, :S], 2, symbols.unsqueeze(2))                           # [B][S][1]
+    px_am_only = sym_am + log_unigram[symbols].unsqueeze(2) - am_only_norm
+    if regular:  # no symbol can be emitted one past the last frame
+        px_am_only = torch.nn.functional.pad(px_am_only, (0, 1), value=float("-inf"))
+    px_lm_only = sym_lm - lm_only_norm[:, :S]
+
+    blank_am = am[:, :, blank].unsqueeze(1)                      # [B][1][T]
+    blank_lm = lm[:, :, blank].unsqueeze(2)                      # [B][S+1][1]
+    py_am_only = blank_am + log_unigram[blank] - am_only_norm
+    py_lm_only = blank_lm - lm_only_norm
+
+    joint_scale = 1.0 - lm_only_scale - am_only_scale
+    lm_only_scale = 1.0e-20 if lm_only_scale == 0.0 else lm_only_scale
+    am_only_scale = 1.0e-20 if am_only_scale == 0.0 else am_only_scale
+    px_mix = px * joint_scale + px_lm_only * lm_only_scale + px_am_only * am_only_scale
+    py_mix = py * joint_scale + py_lm_only * lm_only_scale + py_am_only * am_only_scale
+
+    if regular:
+        px_mix = fix_for_boundary(px_mix, _dev_i64(boundary, px_mix))
+    elif rnnt_type == "constrained":
+        px_mix = px_mix + py_mix[:, 1:, :]
+    return px_mix, py_mix
+
+
+def rnnt_loss_smoothed(
+    lm: Tensor,
+    am: Tensor,
+    symbols: Tensor,
+    termination_symbol: int,
+    lm_only_scale: float = 0.1,
+    am_only_scale: float = 0.1,
+    boundary: Optional[Tensor] = None,
+    rnnt_type: str = "regular",
+    delay_penalty: float = 0.0,
+    reduction: Optional[str] = "mean",
+    return_grad: bool = False,
+) -> Union[Tuple[Tensor, Tuple[Tensor, Tensor]], Tensor]:
+    """k2.rnnt_loss_smoothed (k2/python/k2/rnnt_loss.py:1707-1829)."""
+    px, py = get_rnnt_logprobs_smoothed(lm=lm, am=am, symbols=symbols,
+                                        termination_symbol=termination_symbol,
+                                        lm_only_scale=lm_only_scale, am_only_scale=am_only_scale,
+                                        boundary=boundary, rnnt_type=rnnt_type)
+    if delay_penalty > 0.0:
+        px = _delay_penalty(px, boundary, rnnt_type, delay_penalty)
+    scores_and_grads = mutual_information_recursion(px=px, py=py, boundary=boundary,
+                                                    return_grad=return_grad)
+    negated_loss = scores_and_grads[0] if return_grad else scores_and_grads
+    loss = _reduce(negated_loss, reduction)
+    return (loss, scores_and_grads[1]) if return_grad else loss
+
+
+def get_rnnt_prune_ranges_deprecated(
+    px_grad: Tensor,
+    py_grad: Tensor,
+    boundary: Tensor,
+    s_range: int,
+) -> Tensor:
+    """k2.get_rnnt_prune_ranges_deprecated (k2/python/k2/rnnt_loss.py:786-910): the older rule,
+    which picks for every frame the window of s_range rows with the largest total occupation
+    px_grad + py_grad (prefix sums over s), then applies the same padding and monotonicity
+    adjustment.  Kept for callers; torch ops on the device, not a fused kernel."""
+    (B, S, T1) = px_grad.shape
+    T = py_grad.shape[-1]
+    assert T1 in [T, T + 1], (T1, T)
+    assert py_grad.shape == (B, S + 1, T), (py_grad.shape, B, S + 1, T)
+    assert boundary.shape == (B, 4), (boundary.shape, B)
+    assert S >= 0, S
+    if s_range > S:
+        s_range = S + 1
+    if T1 == T:
+        assert s_range >= 1, \
+            f"Pruning range for modified RNN-T should be equal to or greater than 1, " \
+            f"or no valid paths could survive pruning. Given {s_range}"
+    else:
+        assert s_range >= 2, \
+            f"Pruning range for standard RNN-T should be equal to or greater than 2, " \
+            f"or no valid paths could survive pruning. Given {s_range}"
+    dev = px_grad.device
+    boundary = boundary.to(dev)
+    pad = torch.nn.functional.pad
+    occupation = pad(px_grad, (0, 0, 0, 1)) + pad(py_grad, (0, T1 - T))   # [B][S+1][T1]
+    prefix = torch.cumsum(pad(occupation, (0, 0, 1, 0)), dim=1)            # [B][S+2][T1]
+    window = prefix[:, s_range:, :] - prefix[:, :-s_range, :]
+    s_begin = torch.argmax(window, dim=1)[:, :T]
+    live = torch.arange(T, device=dev).reshape(1, T) < boundary[:, 3].reshape(B, 1) - 1
+    parked = torch.clamp(boundary[:, 2].reshape(B, 1) - s_range + 1, min=0)
+    s_begin = torch.where(live, s_begin, parked)
+    s_begin = _adjust_pruning_lower_bound(s_begin, 2 if T1 == T else s_range)
+    return s_begin.reshape(B, T, 1) + torch.arange(s_range, device=dev)

@@ -19,6 +19,17 @@ Parity status
     (k2/python/tests/rnnt_loss_test.py:735-760), so its values are **parity unpinned** by
     the reference's tests; tests here additionally compare against torch.sum/argmax on CPU.
 
+  * ``hat_logprobs_pruned``: pinned by the probability identity of the model it states
+    (exp(py) + sum over symbols of exp(px-like terms) = 1 for every row), by direct
+    probability-space evaluation (sigmoid and softmax computed in fp64) and by reduction to
+    ``logprobs_pruned`` when column 0 is pushed to -inf; the reference's test only prints its
+    loss (k2/python/tests/rnnt_loss_test.py:859-925): **parity unpinned** by the reference.
+  * ``logprobs_smoothed``: pinned by the identity the reference tests assert (both scales 0
+    gives rnnt_loss_simple, k2/python/tests/rnnt_loss_test.py:167-178) and invariance to
+    per-frame constants (:436-485), plus direct evaluation of the three normalised
+    distributions on tiny inputs.
+  * ``prune_ranges_deprecated``: restated from the source; invariants only: **parity unpinned**.
+
 Only tests, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` may import this.
 """
 import numpy as np
@@ -225,6 +236,120 @@ def logprobs_pruned(logits, symbols, ranges, termination_symbol, boundary, rnnt_
     return px, py
 
 
+def _log_sigmoid(x):
+    return (np.minimum(x, 0) - np.log1p(np.exp(-np.abs(x)))).astype(x.dtype)
+
+
+def hat_logprobs_pruned(logits, symbols, ranges, termination_symbol, boundary,
+                        rnnt_type="regular"):
+    """k2/python/k2/rnnt_loss.py:992-1177 (get_hat_logprobs_pruned)."""
+    assert logits.ndim == 4
+    B, T, R, C = logits.shape
+    assert ranges.shape == (B, T, R)
+    S = symbols.shape[1]
+    assert symbols.shape == (B, S)
+    assert rnnt_type != "modified" or T >= S
+    assert rnnt_type in ("regular", "modified", "constrained")
+    assert termination_symbol == 0
+    dt = logits.dtype
+    logp_b = _log_sigmoid(logits[..., 0])                     # [B,T,R]
+    nb_normalizers = _logsumexp_last(logits[..., 1:])         # [B,T,R]
+    nb_shift = logp_b - logits[..., 0]
+    sym_ext = np.concatenate([symbols, np.zeros((B, 1), dtype=np.int64)], axis=1)
+    pruned_symbols = sym_ext[np.arange(B)[:, None, None], ranges]
+    px = np.take_along_axis(logits, pruned_symbols[..., None], axis=3)[..., 0]
+    px = px - nb_normalizers + nb_shift
+    px = np.concatenate([px, np.full((B, T, S + 1 - R), -np.inf, dtype=dt)], axis=2)
+    px = roll_by_shifts(px, ranges[:, :, 0])[:, :, :S]
+    px = px.transpose(0, 2, 1)
+    if rnnt_type == "regular":
+        px = np.concatenate([px, np.full((B, S, 1), -np.inf, dtype=dt)], axis=2)
+    px = np.ascontiguousarray(px)
+    py = np.concatenate([logp_b, np.full((B, T, S + 1 - R), -np.inf, dtype=dt)], axis=2)
+    py = roll_by_shifts(py, ranges[:, :, 0])
+    py = np.ascontiguousarray(py.transpose(0, 2, 1))
+    if rnnt_type == "regular":
+        px = fix_for_boundary(px, boundary)
+    elif rnnt_type == "constrained":
+        px += py[:, 1:, :]
+    return px, py
+
+
+def logprobs_smoothed(lm, am, symbols, termination_symbol, lm_only_scale=0.1, am_only_scale=0.1,
+                      boundary=None, rnnt_type="regular"):
+    """k2/python/k2/rnnt_loss.py:1471-1704 (get_rnnt_logprobs_smoothed)."""
+    B, T, C = am.shape
+    S = lm.shape[1] - 1
+    assert symbols.shape == (B, S)
+    validate_st_lengths(S, T, rnnt_type == "regular", boundary)
+    dt = am.dtype
+    tiny = np.finfo(dt).tiny
+    am_max = am.max(axis=2, keepdims=True)
+    lm_max = lm.max(axis=2, keepdims=True)
+    am_probs = np.exp(am - am_max)
+    lm_probs = np.exp(lm - lm_max)
+    normalizers = np.log(np.matmul(lm_probs, am_probs.transpose(0, 2, 1)) + tiny)
+    lmonly = lm_probs.sum(axis=2, keepdims=True)                          # [B,S+1,1]
+    unigram = (lm_probs / lmonly).mean(axis=(0, 1), keepdims=True) + tiny  # [1,1,C]
+    amonly = np.log(am_probs.reshape(-1, C) @ unigram.reshape(C)).reshape(B, T, 1) + am_max
+    amonly = amonly.transpose(0, 2, 1)                                     # [B,1,T]
+    unigram = np.log(unigram)
+    lmonly = np.log(lmonly) + lm_max
+    normalizers = (normalizers + lm_max + am_max.transpose(0, 2, 1)).astype(dt)
+
+    bi = np.arange(B)[:, None, None]
+    px_am = am[bi, np.arange(T)[None, None, :], symbols[:, :, None]]
+    if rnnt_type == "regular":
+        px_am = np.concatenate([px_am, np.full((B, S, 1), -np.inf, dtype=dt)], axis=2)
+    px_lm = lm[bi, np.arange(S)[None, :, None], symbols[:, :, None]]       # [B,S,1]
+    px_lm_unigram = unigram[0, 0][symbols][:, :, None]                     # [B,S,1]
+    px = (px_am + px_lm).astype(dt)
+    px[:, :, :T] -= normalizers[:, :S, :]
+    px_amonly = (px_am + px_lm_unigram).astype(dt)
+    px_amonly[:, :, :T] -= amonly
+    px_lmonly = px_lm - lmonly[:, :S, :]
+    py_am = am[:, :, termination_symbol][:, None, :]
+    py_lm = lm[:, :, termination_symbol][:, :, None]
+    py = py_am + py_lm - normalizers
+    py_amonly = py_am + unigram[0, 0, termination_symbol] - amonly
+    py_lmonly = py_lm - lmonly
+    combined = 1.0 - lm_only_scale - am_only_scale
+    if lm_only_scale == 0.0:
+        lm_only_scale = 1.0e-20
+    if am_only_scale == 0.0:
+        am_only_scale = 1.0e-20
+    with np.errstate(invalid="ignore"):
+        px_i = (px * combined + px_lmonly * lm_only_scale + px_amonly * am_only_scale).astype(dt)
+        py_i = (py * combined + py_lmonly * lm_only_scale + py_amonly * am_only_scale).astype(dt)
+    if rnnt_type == "regular":
+        px_i = fix_for_boundary(px_i, boundary)
+    elif rnnt_type == "constrained":
+        px_i += py_i[:, 1:, :]
+    return px_i, py_i
+
+
+def prune_ranges_deprecated(px_grad, py_grad, boundary, s_range):
+    """k2/python/k2/rnnt_loss.py:786-910 (get_rnnt_prune_ranges_deprecated)."""
+    B, S, T1 = px_grad.shape
+    T = py_grad.shape[-1]
+    assert T1 in (T, T + 1)
+    if s_range > S:
+        s_range = S + 1
+    dt = px_grad.dtype
+    py_p = py_grad if T1 == T else np.concatenate(
+        [py_grad, np.zeros((B, S + 1, 1), dtype=dt)], axis=2)
+    tot = np.concatenate([px_grad, np.zeros((B, 1, T1), dtype=dt)], axis=1) + py_p
+    tot = np.concatenate([np.zeros((B, 1, T1), dtype=dt), tot], axis=1)
+    tot = np.cumsum(tot, axis=1, dtype=dt)
+    diff = tot[:, s_range:, :] - tot[:, :-s_range, :]
+    s_begin = np.argmax(diff, axis=1).astype(np.int64)[:, :T]
+    mask = np.arange(T)[None, :] < (boundary[:, 3][:, None] - 1)
+    pad = np.maximum(boundary[:, 2][:, None] - s_range + 1, 0)
+    s_begin = np.where(mask, s_begin, pad)
+    s_begin = adjust_pruning_lower_bound(s_begin, 2 if T1 == T else s_range)
+    return (s_begin[:, :, None] + np.arange(s_range, dtype=np.int64)[None, None, :]).astype(np.int64)
+
+
 def apply_delay_penalty(px, boundary, rnnt_type, delay_penalty):
     """k2/python/k2/rnnt_loss.py:307-322 (same block at :509-528 and :1441-1456)."""
     if not delay_penalty > 0.0:
@@ -271,10 +396,22 @@ def rnnt_loss(logits, symbols, termination_symbol, boundary=None, rnnt_type="reg
     return _reduce(ans, reduction)
 
 
+def rnnt_loss_smoothed(lm, am, symbols, termination_symbol, lm_only_scale=0.1, am_only_scale=0.1,
+                       boundary=None, rnnt_type="regular", delay_penalty=0.0, reduction="mean"):
+    """k2/python/k2/rnnt_loss.py:1707-1829."""
+    px, py = logprobs_smoothed(lm, am, symbols, termination_symbol, lm_only_scale, am_only_scale,
+                               boundary, rnnt_type)
+    px = apply_delay_penalty(px, boundary, rnnt_type, delay_penalty)
+    ans, _ = _mi.mi_forward(px, py, boundary)
+    return _reduce(ans, reduction)
+
+
 def rnnt_loss_pruned(logits, symbols, ranges, termination_symbol, boundary=None,
-                     rnnt_type="regular", delay_penalty=0.0, reduction="mean"):
-    """k2/python/k2/rnnt_loss.py:1351-1468 (use_hat_loss=False)."""
-    px, py = logprobs_pruned(logits, symbols, ranges, termination_symbol, boundary, rnnt_type)
+                     rnnt_type="regular", delay_penalty=0.0, reduction="mean",
+                     use_hat_loss=False):
+    """k2/python/k2/rnnt_loss.py:1351-1468."""
+    builder = hat_logprobs_pruned if use_hat_loss else logprobs_pruned
+    px, py = builder(logits, symbols, ranges, termination_symbol, boundary, rnnt_type)
     px = apply_delay_penalty(px, boundary, rnnt_type, delay_penalty)
     ans, _ = _mi.mi_forward(px, py, boundary)
     return _reduce(ans, reduction)

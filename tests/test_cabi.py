@@ -59,6 +59,14 @@ def test_python_api_mirrors_reference_signatures():
                                      "rnnt_type"],
         "rnnt_loss_pruned": ["logits", "symbols", "ranges", "termination_symbol", "boundary", "rnnt_type",
                              "delay_penalty", "reduction", "use_hat_loss"],
+        "get_hat_logprobs_pruned": ["logits", "symbols", "ranges", "termination_symbol", "boundary",
+                                    "rnnt_type"],
+        "get_rnnt_logprobs_smoothed": ["lm", "am", "symbols", "termination_symbol", "lm_only_scale",
+                                       "am_only_scale", "boundary", "rnnt_type"],
+        "rnnt_loss_smoothed": ["lm", "am", "symbols", "termination_symbol", "lm_only_scale",
+                               "am_only_scale", "boundary", "rnnt_type", "delay_penalty", "reduction",
+                               "return_grad"],
+        "get_rnnt_prune_ranges_deprecated": ["px_grad", "py_grad", "boundary", "s_range"],
     }
     for name, params in want.items():
         assert list(inspect.signature(getattr(k2, name)).parameters) == params, name

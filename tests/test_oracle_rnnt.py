@@ -202,3 +202,138 @@ def test_delay_penalty_and_reduction():
         pytest.approx(base.mean())
     with pytest.raises(ValueError):
         orn.rnnt_loss_simple(c["lm"], c["am"], c["symbols"], 0, c["boundary"], reduction="bogus")
+
+
+# ---- the variants next to the path: HAT, smoothed, the older range rule ------------------------
+
+def _random_band(rng, B, T, S, R):
+    start = np.sort(rng.integers(0, S - R + 2, (B, T)), axis=1)
+    return (start[:, :, None] + np.arange(R)).astype(np.int64)
+
+
+@pytest.mark.parametrize("rnnt_type", ["regular", "modified", "constrained"])
+def test_hat_matches_probability_space_definition(rnnt_type):
+    """P(blank) = sigmoid(l0), P(c) = (1 - sigmoid(l0)) softmax(l[1:])[c]: evaluated directly with
+    probabilities in fp64 (no logsigmoid, no logsumexp), placed by an explicit loop."""
+    rng = np.random.default_rng(31)
+    B, T, S, R, C = 2, 9, 5, 3, 6
+    logits = rng.standard_normal((B, T, R, C))
+    symbols = rng.integers(1, C, (B, S)).astype(np.int64)
+    ranges = _random_band(rng, B, T, S, R)
+    bd = np.array([[0, 0, S, T], [0, 0, S - 1, T - 2]], dtype=np.int64)
+    px, py = orn.hat_logprobs_pruned(logits, symbols, ranges, 0, bd, rnnt_type)
+    T1 = T + 1 if rnnt_type == "regular" else T
+    want_px = np.full((B, S, T1), -np.inf)
+    want_py = np.full((B, S + 1, T), -np.inf)
+    for b in range(B):
+        for t in range(T):
+            for k in range(R):
+                s = ranges[b, t, k]
+                row = logits[b, t, k]
+                pb = 1.0 / (1.0 + math.exp(-row[0]))
+                nb = np.exp(row[1:]) / np.exp(row[1:]).sum()
+                want_py[b, s, t] = math.log(pb)
+                if s < S:
+                    want_px[b, s, t] = math.log((1.0 - pb) * nb[symbols[b, s] - 1])
+                # the row is a distribution: blank + non-blank mass = 1
+                assert pb + (1.0 - pb) * nb.sum() == pytest.approx(1.0, abs=1e-12)
+    if rnnt_type == "regular":
+        for b in range(B):
+            want_px[b, :, bd[b, 3]] = -np.inf
+    elif rnnt_type == "constrained":
+        want_px = want_px + want_py[:, 1:, :]
+    np.testing.assert_allclose(px, want_px, rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(py, want_py, rtol=1e-12, atol=1e-12)
+
+
+def test_hat_reduces_to_softmax_builder_on_its_non_blank_part():
+    """With the blank logit at -40, 1 - sigmoid = 1 to fp64 precision and the HAT px equals the
+    plain pruned px computed on the row whose column 0 cannot win any mass."""
+    rng = np.random.default_rng(32)
+    B, T, S, R, C = 2, 8, 4, 2, 5
+    logits = rng.standard_normal((B, T, R, C))
+    logits[..., 0] = -40.0
+    symbols = rng.integers(1, C, (B, S)).astype(np.int64)
+    ranges = _random_band(rng, B, T, S, R)
+    bd = np.array([[0, 0, S, T], [0, 0, S, T - 1]], dtype=np.int64)
+    px_hat, py_hat = orn.hat_logprobs_pruned(logits, symbols, ranges, 0, bd, "modified")
+    px, _ = orn.logprobs_pruned(logits, symbols, ranges, 0, bd, "modified")
+    np.testing.assert_allclose(px_hat, px, rtol=0, atol=1e-12)
+    finite = np.isfinite(py_hat)
+    np.testing.assert_allclose(py_hat[finite], -40.0, atol=1e-12)
+
+
+@pytest.mark.parametrize("rnnt_type", ["regular", "modified", "constrained"])
+def test_smoothed_with_zero_scales_is_the_simple_loss(rnnt_type):
+    # k2/python/tests/rnnt_loss_test.py:167-178
+    c = cases.rnnt_case(41, B=3, T=9, S=4, C=6, dtype=np.float64, t_lo=6, s_lo=2,
+                        modified=rnnt_type != "regular")
+    a = orn.rnnt_loss_smoothed(c["lm"], c["am"], c["symbols"], 0, 0.0, 0.0, c["boundary"], rnnt_type,
+                               reduction="none")
+    b = orn.rnnt_loss_simple(c["lm"], c["am"], c["symbols"], 0, c["boundary"], rnnt_type,
+                             reduction="none")
+    np.testing.assert_allclose(a, b, rtol=1e-10)
+
+
+def test_smoothed_parts_are_normalised_distributions_and_shift_invariant():
+    """With all the weight on one part, exp(py) + sum over the vocabulary of exp(px-like terms) is
+    1 for that part's distribution: checked for the lm-only part (softmax of lm) and the am-only
+    part (softmax of am + log unigram) by rebuilding them symbol by symbol; then the invariance
+    the reference asserts (k2/python/tests/rnnt_loss_test.py:436-485)."""
+    lm, am, symbols, blank = _fixture()
+    lm = lm.astype(np.float64); am = am.astype(np.float64)
+    B, S1, C = lm.shape
+    T = am.shape[1]
+    # lm-only: scale 1 on the lm part
+    tot_lm = np.zeros((S1,))
+    tot_am = np.zeros((T,))
+    for sym in range(C):
+        if sym == blank:
+            continue
+        sy = np.full((1, S1 - 1), sym, dtype=np.int64)
+        px, _ = orn.logprobs_smoothed(lm, am, sy, blank, 1.0, 0.0, None, "modified")
+        tot_lm[:S1 - 1] += np.exp(px[0, :, 0])
+        px, _ = orn.logprobs_smoothed(lm, am, sy, blank, 0.0, 1.0, None, "modified")
+        tot_am += np.exp(px[0, 0, :])
+    _, py = orn.logprobs_smoothed(lm, am, symbols, blank, 1.0, 0.0, None, "modified")
+    np.testing.assert_allclose(tot_lm[:S1 - 1] + np.exp(py[0, :S1 - 1, 0]), 1.0, rtol=1e-10)
+    _, py = orn.logprobs_smoothed(lm, am, symbols, blank, 0.0, 1.0, None, "modified")
+    np.testing.assert_allclose(tot_am + np.exp(py[0, 0, :]), 1.0, rtol=1e-10)
+    # and the lm-only symbol probabilities are softmax(lm)
+    px, _ = orn.logprobs_smoothed(lm, am, symbols, blank, 1.0, 0.0, None, "modified")
+    soft = lm[0] - np.log(np.exp(lm[0]).sum(-1, keepdims=True))
+    np.testing.assert_allclose(px[0, :, 0], soft[np.arange(S1 - 1), symbols[0]], rtol=1e-10)
+
+    base = orn.rnnt_loss_smoothed(lm, am, symbols, blank, 0.0, 0.333, None, reduction="none")
+    rng = np.random.default_rng(3)
+    am2 = am + rng.standard_normal((1, T, 1))
+    got = orn.rnnt_loss_smoothed(lm, am2, symbols, blank, 0.0, 0.333, None, reduction="none")
+    np.testing.assert_allclose(got, base, rtol=1e-10)
+
+
+@pytest.mark.parametrize("modified", [False, True])
+def test_deprecated_ranges_invariants(modified):
+    from oracle import mi as omi
+    rt = "modified" if modified else "regular"
+    for seed in range(4):
+        B, T, S, C = 3, 40 + 7 * seed, 9 + seed, 8
+        c = cases.rnnt_case(seed, B, T, S, C, dtype=np.float64, t_lo=T // 2, s_lo=S // 2,
+                            modified=modified)
+        px, py = orn.logprobs_simple(c["lm"], c["am"], c["symbols"], 0, rt, c["boundary"])
+        _, gx, gy = omi.mi(px, py, c["boundary"])
+        for R in (2, 4, S + 3):
+            r = orn.prune_ranges_deprecated(gx, gy, c["boundary"], R)
+            Reff = min(R, S + 1) if R <= S else S + 1
+            assert r.shape == (B, T, Reff) and r.dtype == np.int64
+            s0 = r[:, :, 0]
+            assert (np.diff(r, axis=2) == 1).all()
+            assert (s0 >= 0).all() and (r[:, :, -1] <= S).all()
+            d = np.diff(s0, axis=1)
+            assert (d >= 0).all() and (d < (2 if modified else Reff)).all()
+            # the windows of the true arg-max occupation, before the adjustment, on live frames
+            tot = np.concatenate([gx, np.zeros((B, 1, gx.shape[2]))], axis=1)
+            tot[:, :, :T] += gy
+            for b in range(B):
+                t = 0
+                best = max(range(S + 2 - Reff), key=lambda s: (tot[b, s:s + Reff, t].sum(), -s))
+                assert s0[b, 0] == 0 or s0[b, 0] <= best

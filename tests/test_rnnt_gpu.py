@@ -261,3 +261,150 @@ def test_config5_rnnt_loss_full_size(device):
     got = k2.rnnt_loss(dev(logits, device), dev(c["symbols"], device), 0, dev(c["boundary"], device),
                        reduction="none")
     np.testing.assert_allclose(got.cpu().numpy(), want, rtol=1e-4, atol=1e-5)
+
+
+# ---- the variants next to the path -------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("rnnt_type", TYPES)
+def test_hat_logprobs_pruned_forward(device, dtype, rnnt_type):
+    """get_hat_logprobs_pruned through the C-ABI against the oracle: vectorised rows (C % 4 == 0),
+    odd row lengths, rows longer than the register path and rows of 2 and 3 columns."""
+    from k2_amd import capi
+    rng = np.random.default_rng(52)
+    for (B, T, S, R, C) in ((2, 30, 10, 4, 33), (3, 17, 5, 6, 100), (1, 8, 7, 2, 500), (2, 9, 4, 3, 2),
+                            (2, 9, 4, 3, 3), (1, 6, 3, 2, 1100)):
+        c = cases.rnnt_case(6, B, T, S, max(C, 2), dtype=dtype, t_lo=max(T // 2, S), s_lo=S // 2,
+                            modified=rnnt_type != "regular")
+        symbols = np.minimum(c["symbols"], C - 1)
+        logits = (3 * rng.standard_normal((B, T, R, C))).astype(dtype)
+        ranges = _random_ranges(rng, B, T, S, R)
+        want = orn.hat_logprobs_pruned(logits, symbols, ranges, 0, c["boundary"], rnnt_type)
+        px, py, _ = capi.logprobs_pruned_forward(dev(logits, device), dev(symbols, device), dev(ranges, device),
+                                                 0, dev(c["boundary"], device), capi.RNNT_TYPES[rnnt_type],
+                                                 hat=True)
+        np.testing.assert_allclose(px.cpu().numpy(), want[0], **TOL[np.dtype(dtype)])
+        np.testing.assert_allclose(py.cpu().numpy(), want[1], **TOL[np.dtype(dtype)])
+
+
+@pytest.mark.parametrize("C", [3, 7, 12])
+@pytest.mark.parametrize("rnnt_type", TYPES)
+def test_hat_loss_and_gradient_vs_autograd(device, rnnt_type, C):
+    """rnnt_loss_pruned(use_hat_loss=True) in fp64 against torch autograd on the CPU over the
+    probability-space definition; C = 3 takes the one-kernel backward, 12 the vectorised one."""
+    import k2_amd as k2
+    B, T, S, R = 3, 11, 4, 3
+    c = cases.rnnt_case(23, B, T, S, C, dtype=np.float64, t_lo=7, s_lo=2, modified=rnnt_type != "regular")
+    rng = np.random.default_rng(9)
+    ranges = _random_ranges(rng, B, T, S, R)
+    ranges[:, -3:, :] = np.arange(S - R + 1, S + 1)  # the band reaches the last symbol
+    ranges[:, 0, :] = np.arange(R)
+    ranges = np.maximum.accumulate(ranges, axis=1)
+    plog = rng.standard_normal((B, T, R, C))
+    w = torch.linspace(0.5, 1.5, B, dtype=torch.float64)
+    bd_cpu = torch.from_numpy(c["boundary"])
+    pl_r = torch.from_numpy(plog).requires_grad_(True)
+    px, py = torch_ref.logprobs_pruned(pl_r, torch.from_numpy(c["symbols"]), torch.from_numpy(ranges), 0,
+                                       bd_cpu, rnnt_type, hat=True)
+    loss_r = -torch_ref.mi_scores(px, py, bd_cpu)
+    pl_g = dev(plog, device).requires_grad_(True)
+    loss_g = k2.rnnt_loss_pruned(pl_g, dev(c["symbols"], device), dev(ranges, device), 0,
+                                 dev(c["boundary"], device), rnnt_type=rnnt_type, reduction="none",
+                                 use_hat_loss=True)
+    np.testing.assert_allclose(loss_g.detach().cpu().numpy(), loss_r.detach().numpy(), rtol=1e-10)
+    ok = torch.isfinite(loss_r)
+    assert ok.any()
+    (loss_r[ok] * w[ok]).sum().backward()
+    (loss_g[ok.to(device)] * w[ok].to(device)).sum().backward()
+    np.testing.assert_allclose(pl_g.grad.cpu().numpy(), pl_r.grad.numpy(), rtol=1e-8, atol=1e-10)
+    with pytest.raises(AssertionError):
+        k2.get_hat_logprobs_pruned(pl_g, dev(c["symbols"], device), dev(ranges, device), 1,
+                                   dev(c["boundary"], device), rnnt_type)
+
+
+def test_hat_gradient_fp32_vectorised_rows(device):
+    """fp32, C = 500 (the 16-byte path of the row kernels) against the fp64 result of the same
+    kernels, whose gradient the test above ties to autograd."""
+    import k2_amd as k2
+    B, T, S, R, C = 4, 40, 12, 4, 500
+    c = cases.rnnt_case(29, B, T, S, C, t_lo=T, s_lo=S)  # full lengths: the band below ends at (S, T)
+    rng = np.random.default_rng(10)
+    start = np.minimum(np.arange(T)[None, :] * (S - R + 2) // T, S - R + 1)
+    ranges = (np.repeat(start, B, axis=0)[:, :, None] + np.arange(R)).astype(np.int64)
+    plog = rng.standard_normal((B, T, R, C)).astype(np.float32)
+    res = {}
+    for dt in (torch.float32, torch.float64):
+        x = dev(plog, device).to(dt).requires_grad_(True)
+        loss = k2.rnnt_loss_pruned(x, dev(c["symbols"], device), dev(ranges, device), 0,
+                                   dev(c["boundary"], device), reduction="sum", use_hat_loss=True)
+        loss.backward()
+        res[dt] = (loss.item(), x.grad.double().cpu().numpy())
+    assert np.isfinite(res[torch.float64][0])
+    assert res[torch.float32][0] == pytest.approx(res[torch.float64][0], rel=1e-4)
+    np.testing.assert_allclose(res[torch.float32][1], res[torch.float64][1], rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("rnnt_type", TYPES)
+def test_smoothed_loss_values_gradients_and_identities(device, rnnt_type):
+    """rnnt_loss_smoothed: fp64 values against the oracle, gradients against torch autograd over
+    the three-distribution definition, scales (0, 0) == rnnt_loss_simple
+    (k2/python/tests/rnnt_loss_test.py:167-178) and invariance to per-frame constants (:436-485)."""
+    import k2_amd as k2
+    B, T, S, C = 3, 10, 4, 6
+    c = cases.rnnt_case(61, B, T, S, C, dtype=np.float64, t_lo=7, s_lo=2, modified=rnnt_type != "regular")
+    sym, bd = dev(c["symbols"], device), dev(c["boundary"], device)
+    want = orn.rnnt_loss_smoothed(c["lm"], c["am"], c["symbols"], 0, 0.25, 0.1, c["boundary"], rnnt_type,
+                                  reduction="none")
+    lm_g = dev(c["lm"], device).requires_grad_(True)
+    am_g = dev(c["am"], device).requires_grad_(True)
+    got = k2.rnnt_loss_smoothed(lm_g, am_g, sym, 0, lm_only_scale=0.25, am_only_scale=0.1, boundary=bd,
+                                rnnt_type=rnnt_type, reduction="none")
+    np.testing.assert_allclose(got.detach().cpu().numpy(), want, rtol=1e-10)
+    px, py = k2.get_rnnt_logprobs_smoothed(lm_g, am_g, sym, 0, 0.25, 0.1, bd, rnnt_type)
+    wpx, wpy = orn.logprobs_smoothed(c["lm"], c["am"], c["symbols"], 0, 0.25, 0.1, c["boundary"], rnnt_type)
+    np.testing.assert_allclose(px.detach().cpu().numpy(), wpx, rtol=1e-10, atol=1e-10)
+    np.testing.assert_allclose(py.detach().cpu().numpy(), wpy, rtol=1e-10, atol=1e-10)
+
+    w = torch.linspace(0.5, 1.5, B, dtype=torch.float64)
+    lm_r = torch.from_numpy(c["lm"]).requires_grad_(True)
+    am_r = torch.from_numpy(c["am"]).requires_grad_(True)
+    bd_cpu = torch.from_numpy(c["boundary"])
+    rpx, rpy = torch_ref.logprobs_smoothed(lm_r, am_r, torch.from_numpy(c["symbols"]), 0, 0.25, 0.1,
+                                           rnnt_type, bd_cpu)
+    loss_r = -torch_ref.mi_scores(rpx, rpy, bd_cpu)
+    np.testing.assert_allclose(loss_r.detach().numpy(), want, rtol=1e-10)
+    (loss_r * w).sum().backward()
+    (got * w.to(device)).sum().backward()
+    np.testing.assert_allclose(lm_g.grad.cpu().numpy(), lm_r.grad.numpy(), rtol=1e-8, atol=1e-10)
+    np.testing.assert_allclose(am_g.grad.cpu().numpy(), am_r.grad.numpy(), rtol=1e-8, atol=1e-10)
+
+    plain = k2.rnnt_loss_simple(lm_g.detach(), am_g.detach(), sym, 0, bd, rnnt_type=rnnt_type, reduction="none")
+    zero = k2.rnnt_loss_smoothed(lm_g.detach(), am_g.detach(), sym, 0, lm_only_scale=0.0, am_only_scale=0.0,
+                                 boundary=bd, rnnt_type=rnnt_type, reduction="none")
+    np.testing.assert_allclose(zero.cpu().numpy(), plain.cpu().numpy(), rtol=1e-10)
+    shifted = k2.rnnt_loss_smoothed(lm_g.detach(), am_g.detach() + torch.randn(B, T, 1, device=device, dtype=torch.float64),
+                                    sym, 0, lm_only_scale=0.0, am_only_scale=0.333, boundary=bd,
+                                    rnnt_type=rnnt_type, reduction="none")
+    base = k2.rnnt_loss_smoothed(lm_g.detach(), am_g.detach(), sym, 0, lm_only_scale=0.0, am_only_scale=0.333,
+                                 boundary=bd, rnnt_type=rnnt_type, reduction="none")
+    np.testing.assert_allclose(shifted.cpu().numpy(), base.cpu().numpy(), rtol=1e-9)
+    loss, (gx, gy) = k2.rnnt_loss_smoothed(lm_g.detach(), am_g.detach(), sym, 0, boundary=bd, rnnt_type=rnnt_type,
+                                           return_grad=True)
+    assert loss.ndim == 0 and gx.shape == px.shape and gy.shape == py.shape
+
+
+@pytest.mark.parametrize("modified", [False, True])
+def test_deprecated_prune_ranges_matches_oracle(device, modified):
+    import k2_amd as k2
+    rt = "modified" if modified else "regular"
+    for seed in range(3):
+        B, T, S, C = 3, 50 + 9 * seed, 11 + seed, 9
+        c = cases.rnnt_case(seed, B, T, S, C, dtype=np.float64, t_lo=T // 2, s_lo=S // 2, modified=modified)
+        px, py = orn.logprobs_simple(c["lm"], c["am"], c["symbols"], 0, rt, c["boundary"])
+        _, gx, gy = omi.mi(px, py, c["boundary"])
+        for R in (2, 5, S + 2):
+            want = orn.prune_ranges_deprecated(gx, gy, c["boundary"], R)
+            got = k2.get_rnnt_prune_ranges_deprecated(dev(gx, device), dev(gy, device),
+                                                      dev(c["boundary"], device), R)
+            assert got.dtype == torch.int64
+            assert np.array_equal(got.cpu().numpy(), want), (seed, R)

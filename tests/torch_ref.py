@@ -7,9 +7,27 @@ import torch
 
 def logprobs_from_logits(logits, symbols, blank, rnnt_type="regular", boundary=None):
     """logits [B,T,S+1,C] -> (px [B,S,T1], py [B,S+1,T])."""
-    B, T, S1, C = logits.shape
+    return _from_logprobs(torch.log_softmax(logits, dim=-1), symbols, blank, rnnt_type, boundary)
+
+
+def logprobs_smoothed(lm, am, symbols, blank, lm_only_scale, am_only_scale, rnnt_type="regular",
+                      boundary=None):
+    """Log-linear mix of three normalised distributions over the vocabulary: softmax(am + lm),
+    softmax(lm), and softmax(am + log unigram) with the unigram the batch mean of softmax(lm)."""
+    joint = torch.log_softmax(am.unsqueeze(2) + lm.unsqueeze(1), dim=-1)       # [B,T,S+1,C]
+    lm_only = torch.log_softmax(lm, dim=-1).unsqueeze(1)                        # [B,1,S+1,C]
+    unigram = torch.softmax(lm, dim=-1).mean(dim=(0, 1)) + torch.finfo(lm.dtype).tiny
+    am_only = torch.log_softmax(am + unigram.log(), dim=-1).unsqueeze(2)        # [B,T,1,C]
+    joint_scale = 1.0 - lm_only_scale - am_only_scale
+    lm_only_scale = lm_only_scale or 1.0e-20
+    am_only_scale = am_only_scale or 1.0e-20
+    mix = joint * joint_scale + lm_only * lm_only_scale + am_only * am_only_scale
+    return _from_logprobs(mix, symbols, blank, rnnt_type, boundary)
+
+
+def _from_logprobs(lp, symbols, blank, rnnt_type, boundary):
+    B, T, S1, C = lp.shape
     S = S1 - 1
-    lp = torch.log_softmax(logits, dim=-1)
     idx = symbols.reshape(B, 1, S, 1).expand(B, T, S, 1)
     px = lp[:, :, :S, :].gather(3, idx).squeeze(-1).permute(0, 2, 1)  # [B,S,T]
     py = lp[..., blank].permute(0, 2, 1)  # [B,S+1,T]
@@ -28,11 +46,18 @@ def logprobs_simple(lm, am, symbols, blank, rnnt_type="regular", boundary=None):
     return logprobs_from_logits(am.unsqueeze(2) + lm.unsqueeze(1), symbols, blank, rnnt_type, boundary)
 
 
-def logprobs_pruned(logits, symbols, ranges, blank, boundary, rnnt_type="regular"):
-    """logits [B,T,R,C]; dense px/py with -inf outside the band."""
+def logprobs_pruned(logits, symbols, ranges, blank, boundary, rnnt_type="regular", hat=False):
+    """logits [B,T,R,C]; dense px/py with -inf outside the band.  ``hat``: the blank (column 0)
+    has probability sigmoid(l0) and the others (1 - sigmoid(l0)) softmax(l[1:])."""
     B, T, R, C = logits.shape
     S = symbols.shape[1]
-    lp = torch.log_softmax(logits, dim=-1)
+    if hat:
+        assert blank == 0
+        p_blank = torch.sigmoid(logits[..., :1])
+        lp = torch.cat([p_blank.log(),
+                        (1 - p_blank).log() + torch.log_softmax(logits[..., 1:], dim=-1)], dim=-1)
+    else:
+        lp = torch.log_softmax(logits, dim=-1)
     T1 = T + 1 if rnnt_type == "regular" else T
     px = torch.full((B, S, T1), float("-inf"), dtype=logits.dtype)
     py = torch.full((B, S + 1, T), float("-inf"), dtype=logits.dtype)
