@@ -30,7 +30,7 @@ enum k2amd_status {
   K2AMD_ERR_TIMEOUT = 5           /* a bounded in-kernel wait expired; re-initialise the workspace */
 };
 
-enum k2amd_dtype { K2AMD_F32 = 0, K2AMD_F64 = 1 };
+enum k2amd_dtype { K2AMD_F32 = 0, K2AMD_F64 = 1, K2AMD_F16 = 2 /* lattice scores only */ };
 
 /* rnnt_type of k2/python/k2/rnnt_loss.py:70 ("regular" | "modified" | "constrained") */
 enum k2amd_rnnt_type { K2AMD_REGULAR = 0, K2AMD_MODIFIED = 1, K2AMD_CONSTRAINED = 2 };
@@ -168,6 +168,32 @@ K2AMD_API int k2amd_rnnt_prune_gather(const void *lm, const int64_t *ranges, voi
 K2AMD_API int k2amd_rnnt_prune_gather_backward(const void *grad, const int64_t *ranges,
                                                void *lm_grad, int B, int S1, int T, int R, int D,
                                                int dtype, void *stream);
+
+/* ------------------------------------------------------------------ lattice
+ *
+ * Replaces _k2.pruned_ranges_to_lattice (k2/python/csrc/torch/pruned_ranges_to_lattice.cu:60-263):
+ * the pruned band as one lattice per sequence.  ranges [B][T][R] int32, frames [B] int32,
+ * symbols [B][S] int64, logits [B][T][R][C] (f32 / f64 / f16) with element strides
+ * logits_strides[4] (host memory).  Sequence b has frames[b] * R + 1 states.
+ *
+ * Step 1 (..._count) fills, on the device,
+ *   arc_local  [B][T*R+1]  arcs of sequence b leaving states before the given one (scratch),
+ *   seq_arcs   [B]         (scratch),
+ *   state_splits [B+1]     row splits sequence -> states (k2's row_splits1),
+ *   arc_base   [B+1]       arcs of the sequences before b; arc_base[B] = number of arcs.
+ * The caller reads state_splits[B] and arc_base[B] to size the outputs of step 2 (..._fill):
+ *   arc_splits [states+1]  row splits state -> arcs (k2's row_splits2),
+ *   arcs       [arcs][4]   k2's Arc records {int32 src, int32 dest, int32 label, float score},
+ *   arc_map    [arcs]      element index of the arc's score in logits, or -1.                    */
+K2AMD_API int k2amd_lattice_count(const int32_t *ranges, const int32_t *frames, int32_t *arc_local,
+                                  int32_t *seq_arcs, int32_t *state_splits, int32_t *arc_base,
+                                  int B, int T, int R, void *stream);
+K2AMD_API int k2amd_lattice_fill(const int32_t *ranges, const int32_t *frames,
+                                 const int64_t *symbols, const void *logits,
+                                 const int64_t *logits_strides, const int32_t *state_splits,
+                                 const int32_t *arc_base, const int32_t *arc_local,
+                                 int32_t *arc_splits, void *arcs, int32_t *arc_map, int B, int T,
+                                 int R, int S, int C, int dtype, void *stream);
 
 #ifdef __cplusplus
 }

@@ -5,6 +5,7 @@ Exports the same names as ``import k2`` does for this path
 ``mutual_information_recursion``, ``rnnt_loss_simple``, ``get_rnnt_prune_ranges``,
 ``do_rnnt_pruning``, ``rnnt_loss_pruned``, ``rnnt_loss`` and their log-prob builders.
 """
+from .lattice import pruned_ranges_to_lattice
 from .mutual_information import joint_mutual_information_recursion
 from .mutual_information import mutual_information_recursion
 from .rnnt_loss import do_rnnt_pruning
@@ -27,5 +28,5 @@ __all__ = [
     "get_rnnt_logprobs", "get_rnnt_logprobs_joint", "get_rnnt_logprobs_pruned",
     "get_rnnt_prune_ranges", "rnnt_loss", "rnnt_loss_pruned", "rnnt_loss_simple",
     "get_hat_logprobs_pruned", "get_rnnt_logprobs_smoothed", "rnnt_loss_smoothed",
-    "get_rnnt_prune_ranges_deprecated",
+    "get_rnnt_prune_ranges_deprecated", "pruned_ranges_to_lattice",
 ]

@@ -41,6 +41,8 @@ _SIGNATURES = {
     "k2amd_rnnt_prune_ranges": ([_vp] * 4 + [_ci] * 6 + [_vp], _ci),
     "k2amd_rnnt_prune_gather": ([_vp] * 3 + [_ci] * 6 + [_vp], _ci),
     "k2amd_rnnt_prune_gather_backward": ([_vp] * 3 + [_ci] * 6 + [_vp], _ci),
+    "k2amd_lattice_count": ([_vp] * 6 + [_ci] * 3 + [_vp], _ci),
+    "k2amd_lattice_fill": ([_vp] * 11 + [_ci] * 6 + [_vp], _ci),
 }
 
 
@@ -306,3 +308,39 @@ def prune_gather_backward(grad, ranges, S1):
                                                      T, R, D, dtype_code(grad),
                                                      stream_ptr(grad.device)))
     return lm_grad
+
+
+F16 = 2
+
+
+def pruned_ranges_to_lattice(ranges, frames, symbols, logits):
+    """C-ABI pruned_ranges_to_lattice: returns (state_splits [B+1], arc_splits [states+1],
+    arcs int32 [arcs][4] (score bits in column 3), arc_map int32 [arcs])."""
+    B, T, R = ranges.shape
+    S = symbols.shape[1]
+    C = logits.shape[3]
+    dev = ranges.device
+    i32 = dict(dtype=torch.int32, device=dev)
+    arc_local = torch.empty(B, T * R + 1, **i32)
+    seq_arcs = torch.empty(max(B, 1), **i32)
+    state_splits = torch.empty(B + 1, **i32)
+    arc_base = torch.empty(B + 1, **i32)
+    code = {torch.float32: F32, torch.float64: F64, torch.float16: F16}.get(logits.dtype)
+    if code is None:
+        raise RuntimeError(f"k2_amd: unsupported logits dtype {logits.dtype}")
+    with torch.cuda.device(dev):
+        check(lib().k2amd_lattice_count(ptr(ranges), ptr(frames), ptr(arc_local), ptr(seq_arcs),
+                                        ptr(state_splits), ptr(arc_base), B, T, R, stream_ptr(dev)))
+        n_states, n_arcs = int(state_splits[B]), int(arc_base[B])  # the one host read, as in k2
+        arc_splits = torch.empty(n_states + 1, **i32)
+        arcs = torch.empty(n_arcs, 4, **i32)
+        arc_map = torch.empty(n_arcs, **i32)
+        if B == 0:
+            arc_splits.zero_()
+        strides = (ctypes.c_int64 * 4)(*logits.stride())
+        assert logits.is_cuda
+        check(lib().k2amd_lattice_fill(ptr(ranges), ptr(frames), ptr(symbols), logits.data_ptr(),
+                                       ctypes.addressof(strides), ptr(state_splits), ptr(arc_base),
+                                       ptr(arc_local), ptr(arc_splits), ptr(arcs), ptr(arc_map), B, T,
+                                       R, S, C, code, stream_ptr(dev)))
+    return state_splits, arc_splits, arcs, arc_map

@@ -366,6 +366,57 @@ torch::Tensor PruneGatherBackward(torch::Tensor grad, torch::Tensor ranges, int 
   return lm_grad;
 }
 
+// _k2.pruned_ranges_to_lattice (k2/python/csrc/torch/pruned_ranges_to_lattice.cu:265-281).  The
+// lattice comes back as its parts: (state_splits [B+1], arc_splits [states+1],
+// arcs int32 [arcs][4] with the score's bits in column 3, arc_map int32 [arcs]).
+std::vector<torch::Tensor> PrunedRangesToLattice(torch::Tensor ranges, torch::Tensor frames,
+                                                 torch::Tensor symbols, torch::Tensor logits) {
+  TORCH_CHECK(ranges.dim() == 3, "ranges should be 3-dimensional");
+  TORCH_CHECK(frames.dim() == 1, "frames should be 1-dimensional");
+  TORCH_CHECK(symbols.dim() == 2, "symbols should be 2-dimensional");
+  TORCH_CHECK(logits.dim() == 4, "logits should be 4-dimensional");
+  TORCH_CHECK(ranges.scalar_type() == torch::kInt && frames.scalar_type() == torch::kInt,
+              "ranges and frames must be int32");
+  TORCH_CHECK(symbols.scalar_type() == torch::kLong, "symbols must be int64");
+  RequireDevice(ranges, "ranges");
+  RequireDevice(frames, "frames");
+  RequireDevice(symbols, "symbols");
+  TORCH_CHECK(logits.is_cuda(), "k2_amd runs on MI355X only: logits is on ", logits.device(),
+              " (there is no CPU path)");
+  TORCH_CHECK(frames.device() == ranges.device() && symbols.device() == ranges.device() &&
+                  logits.device() == ranges.device(),
+              "inputs must be on the same device");
+  const int B = ranges.size(0), T = ranges.size(1), R = ranges.size(2);
+  const int S = symbols.size(1), C = logits.size(3);
+  TORCH_CHECK(frames.size(0) == B && symbols.size(0) == B && logits.size(0) == B &&
+                  logits.size(1) == T && logits.size(2) == R,
+              "shapes of ranges, frames, symbols and logits do not agree");
+  int dtype = K2AMD_F32;
+  if (logits.scalar_type() == torch::kDouble) dtype = K2AMD_F64;
+  else if (logits.scalar_type() == torch::kHalf) dtype = K2AMD_F16;
+  else TORCH_CHECK(logits.scalar_type() == torch::kFloat, "logits must be float32, float64 or float16");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(ranges.device());
+  auto i32 = ranges.options();
+  torch::Tensor arc_local = torch::empty({B, T * R + 1}, i32), seq_arcs = torch::empty({std::max(B, 1)}, i32);
+  torch::Tensor state_splits = torch::empty({B + 1}, i32), arc_base = torch::empty({B + 1}, i32);
+  void *stream = StreamOf(ranges);
+  Check(k2amd_lattice_count(ranges.data_ptr<int32_t>(), frames.data_ptr<int32_t>(),
+                            arc_local.data_ptr<int32_t>(), seq_arcs.data_ptr<int32_t>(),
+                            state_splits.data_ptr<int32_t>(), arc_base.data_ptr<int32_t>(), B, T, R,
+                            stream));
+  // the one host read on this path (the reference reads the same totals to size its arrays)
+  const int n_states = state_splits[B].item<int32_t>(), n_arcs = arc_base[B].item<int32_t>();
+  torch::Tensor arc_splits = B > 0 ? torch::empty({n_states + 1}, i32) : torch::zeros({1}, i32);
+  torch::Tensor arcs = torch::empty({n_arcs, 4}, i32), arc_map = torch::empty({n_arcs}, i32);
+  const int64_t strides[4] = {logits.stride(0), logits.stride(1), logits.stride(2), logits.stride(3)};
+  Check(k2amd_lattice_fill(ranges.data_ptr<int32_t>(), frames.data_ptr<int32_t>(), I64(symbols),
+                           logits.data_ptr(), strides, state_splits.data_ptr<int32_t>(),
+                           arc_base.data_ptr<int32_t>(), arc_local.data_ptr<int32_t>(),
+                           arc_splits.data_ptr<int32_t>(), arcs.data_ptr(),
+                           arc_map.data_ptr<int32_t>(), B, T, R, S, C, dtype, stream));
+  return {state_splits, arc_splits, arcs, arc_map};
+}
+
 }  // namespace
 
 PYBIND11_MODULE(_k2_amd, m) {
@@ -385,4 +436,6 @@ PYBIND11_MODULE(_k2_amd, m) {
   m.def("prune_ranges", &PruneRanges);
   m.def("prune_gather", &PruneGather);
   m.def("prune_gather_backward", &PruneGatherBackward);
+  m.def("pruned_ranges_to_lattice", &PrunedRangesToLattice, pybind11::arg("ranges"),
+        pybind11::arg("frames"), pybind11::arg("symbols"), pybind11::arg("logits"));
 }

@@ -123,3 +123,14 @@ def prune_gather_backward(grad, ranges, S1):
     if _ext is not None:
         return _ext.prune_gather_backward(grad, ranges, S1)
     return capi.prune_gather_backward(grad, ranges, S1)
+
+
+def pruned_ranges_to_lattice(ranges, frames, symbols, logits):
+    """The parts of the lattice: (state_splits, arc_splits, arcs [N][4] int32, arc_map [N])."""
+    _require_device(ranges)
+    if _ext is not None:
+        return tuple(_ext.pruned_ranges_to_lattice(ranges, frames, symbols, logits))
+    if ranges.dtype != torch.int32 or frames.dtype != torch.int32 or symbols.dtype != torch.int64:
+        raise RuntimeError("ranges and frames must be int32, symbols int64")
+    return capi.pruned_ranges_to_lattice(ranges.contiguous(), frames.contiguous(),
+                                         symbols.contiguous(), logits)

@@ -67,6 +67,7 @@ def test_python_api_mirrors_reference_signatures():
                                "am_only_scale", "boundary", "rnnt_type", "delay_penalty", "reduction",
                                "return_grad"],
         "get_rnnt_prune_ranges_deprecated": ["px_grad", "py_grad", "boundary", "s_range"],
+        "pruned_ranges_to_lattice": ["ranges", "frames", "symbols", "logits"],
     }
     for name, params in want.items():
         assert list(inspect.signature(getattr(k2, name)).parameters) == params, name
@@ -113,7 +114,7 @@ def test_pybind_host_module_covers_every_builder_of_the_c_abi():
     from k2_amd import _k2_amd, native
     names = ("logprobs_simple_forward", "logprobs_simple_backward", "logprobs_joint_forward",
              "logprobs_joint_backward", "logprobs_pruned_forward", "logprobs_pruned_backward",
-             "prune_ranges", "prune_gather", "prune_gather_backward")
+             "prune_ranges", "prune_gather", "prune_gather_backward", "pruned_ranges_to_lattice")
     for n in names:
         assert callable(getattr(_k2_amd, n)), n
         assert callable(getattr(native, n)), n
