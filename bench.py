@@ -167,6 +167,67 @@ def pruned_secondary(dev, steps=20, cpu=True):
     return out
 
 
+def other_configs(dev, steps=20):
+    """The two remaining BASELINE configurations, forward + backward through the k2-style API with
+    gradients to the network outputs: config 2 (rnnt_loss_simple, B=16 T=250 S=50 V=500) and
+    config 5 (rnnt_loss on the full joiner lattice, B=8 T=300 S=75 V=500)."""
+    import torch
+    import cases
+    import k2_amd as k2
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps * 1e-3
+
+    out = {}
+    B, T, S, C = 16, 250, 50, 500
+    c = cases.rnnt_case(2, B, T, S, C, t_lo=150, s_lo=20)
+    lm = torch.from_numpy(c["lm"]).to(dev).requires_grad_(True)
+    am = torch.from_numpy(c["am"]).to(dev).requires_grad_(True)
+    sym, bd = torch.from_numpy(c["symbols"]).to(dev), torch.from_numpy(c["boundary"]).to(dev)
+
+    def simple():
+        lm.grad = None
+        am.grad = None
+        k2.rnnt_loss_simple(lm, am, sym, 0, bd, reduction="sum").backward()
+
+    t = timed(simple)
+    # lm, am read once forward; their gradients written once backward
+    nbytes = 2 * 4 * (lm.numel() + am.numel())
+    out["c2_rnnt_loss_simple"] = {
+        "workload": "rnnt_loss_simple fwd+bwd, fp32, regular, B=16 T=250 S=50 V=500 (BASELINE config 2)",
+        "ms_per_step": t * 1e3, "utterances_per_s": B / t, "algorithmic_GBps": nbytes / t / 1e9,
+        "frac_of_hbm_peak": nbytes / t / 1e9 / HBM_PEAK_GBS}
+    del lm, am
+
+    B, T, S, C = 8, 300, 75, 500
+    c = cases.rnnt_case(5, B, T, S, C, t_lo=200, s_lo=40)
+    logits = torch.from_numpy(
+        np.random.default_rng(55).standard_normal((B, T, S + 1, C)).astype(np.float32)).to(dev)
+    logits.requires_grad_(True)
+    sym, bd = torch.from_numpy(c["symbols"]).to(dev), torch.from_numpy(c["boundary"]).to(dev)
+
+    def joint():
+        logits.grad = None
+        k2.rnnt_loss(logits, sym, 0, bd, reduction="sum").backward()
+
+    t = timed(joint)
+    nbytes = 3 * 4 * logits.numel()  # read forward; read + write backward
+    out["c5_rnnt_loss"] = {
+        "workload": "rnnt_loss fwd+bwd, fp32, regular, B=8 T=300 S=75 V=500 (BASELINE config 5)",
+        "ms_per_step": t * 1e3, "utterances_per_s": B / t, "logits_GBps": nbytes / t / 1e9,
+        "frac_of_hbm_peak": nbytes / t / 1e9 / HBM_PEAK_GBS}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -274,6 +335,7 @@ def main():
     if not args.no_secondary:
         del px, py, p
         out["secondary"] = pruned_secondary(dev, cpu=not args.no_cpu)
+        out["other_configs"] = other_configs(dev)
     print(json.dumps(out))
 
 
