@@ -428,7 +428,7 @@ int RowBackward(const T *logits, const T *normalizers, const T *px_grad, const T
   const long long rows = (long long)g.B * g.Tn * g.K;
   if (rows > 0) {
     const long long blocks = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
-    if (g.C >= 4) {
+    if (g.C >= 4 && g.C <= (1 << 24)) {  // the record holds the symbol as a float: exact up to 2^24
       hipLaunchKernelGGL((RowGradPrepKernel<T, kPruned>), dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, stream,
                          normalizers, px_grad, py_grad, symbols, ranges, boundary, logits_grad, g);
       hipLaunchKernelGGL((RowGradKernel<T, kHat>), dim3((unsigned)blocks), dim3(kRowsPerBlock * kWave), 0, stream,
