@@ -82,3 +82,23 @@ def test_strided_logits_and_errors(device):
     with pytest.raises(RuntimeError, match="no CPU path"):
         k2.pruned_ranges_to_lattice(torch.from_numpy(c["ranges"]), torch.from_numpy(c["frames"]),
                                     torch.from_numpy(c["symbols"]), torch.from_numpy(c["logits"]))
+
+
+def test_degenerate_shapes(device):
+    """A sequence without frames is a lone final state; an empty batch gives empty outputs."""
+    import k2_amd as k2
+    ranges = torch.zeros(2, 3, 2, dtype=torch.int32, device=device)
+    ranges[..., 1] = 1
+    frames = torch.tensor([0, 3], dtype=torch.int32, device=device)
+    symbols = torch.tensor([[1, 2], [2, 1]], dtype=torch.long, device=device)
+    logits = torch.randn(2, 3, 2, 4, device=device)
+    ofsa, arc_map = k2.pruned_ranges_to_lattice(ranges, frames, symbols, logits)
+    want = olat.pruned_ranges_to_lattice(ranges.cpu().numpy(), frames.cpu().numpy(), symbols.cpu().numpy(),
+                                         logits.cpu().numpy())
+    assert ofsa.row_splits(1).tolist() == [0, 1, 8]
+    assert np.array_equal(ofsa.row_splits(2).cpu().numpy(), want[1])
+    assert np.array_equal(ofsa.values()[:, :3].cpu().numpy(), want[2])
+    assert np.array_equal(arc_map.cpu().numpy(), want[4])
+    empty = k2.pruned_ranges_to_lattice(ranges[:0], frames[:0], symbols[:0], logits[:0])
+    assert empty[0].dim0 == 0 and empty[0].num_elements == 0 and empty[1].numel() == 0
+    assert empty[0].row_splits(1).tolist() == [0] and empty[0].row_splits(2).tolist() == [0]

@@ -408,3 +408,29 @@ def test_deprecated_prune_ranges_matches_oracle(device, modified):
                                                       dev(c["boundary"], device), R)
             assert got.dtype == torch.int64
             assert np.array_equal(got.cpu().numpy(), want), (seed, R)
+
+
+def test_variants_degenerate_shapes(device):
+    """S = 0 (no symbols), s_range = S + 1 (no pruning) and an empty batch through the HAT and
+    smoothed builders."""
+    import k2_amd as k2
+    B, T, C = 2, 5, 4
+    logits = torch.randn(B, T, 1, C, device=device, dtype=torch.float64)
+    sym0 = torch.zeros(B, 0, dtype=torch.long, device=device)
+    ranges0 = torch.zeros(B, T, 1, dtype=torch.long, device=device)
+    bd = torch.tensor([[0, 0, 0, T], [0, 0, 0, T - 1]], device=device)
+    loss = k2.rnnt_loss_pruned(logits, sym0, ranges0, 0, bd, reduction="none", use_hat_loss=True)
+    want = -torch.nn.functional.logsigmoid(logits[..., 0, 0])  # only blanks: sum of log sigmoid
+    assert loss[0].item() == pytest.approx(want[0].sum().item(), rel=1e-10)
+    assert loss[1].item() == pytest.approx(want[1, :T - 1].sum().item(), rel=1e-10)
+    S = 3
+    c = cases.rnnt_case(77, B, T, S, C, dtype=np.float64)
+    full = torch.randn(B, T, S + 1, C, device=device, dtype=torch.float64)
+    ranges = torch.arange(S + 1, device=device).expand(B, T, S + 1).contiguous()
+    a = k2.rnnt_loss_pruned(full, dev(c["symbols"], device), ranges, 0, dev(c["boundary"], device), reduction="none")
+    b = k2.rnnt_loss(full, dev(c["symbols"], device), 0, dev(c["boundary"], device), reduction="none")
+    np.testing.assert_allclose(a.cpu().numpy(), b.cpu().numpy(), rtol=1e-12)
+    lm = torch.randn(0, S + 1, C, device=device)
+    am = torch.randn(0, T, C, device=device)
+    e = k2.rnnt_loss_smoothed(lm, am, torch.zeros(0, S, dtype=torch.long, device=device), 0, reduction="none")
+    assert e.shape == (0,)
