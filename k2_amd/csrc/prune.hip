@@ -35,12 +35,15 @@ __device__ int *SuffixMin(int *a, int *b, int n) {
 constexpr int kArgFrames = 64;
 constexpr int kArgSplit = 4;
 
-template <typename T>
+// kR > 0: the window length as a compile-time constant (the usual s_range of 2..8), which lets the
+// loads of four windows be issued together; kR == 0: any length, one window at a time.
+template <typename T, int kR>
 __global__ __launch_bounds__(kArgFrames * kArgSplit) void PruneArgmaxKernel(
     const T *__restrict__ px_grad, const T *__restrict__ py_grad, int64_t *__restrict__ ranges,
-    int S, int Tn, int modified, int R) {
+    int S, int Tn, int modified, int R_any) {
   __shared__ T best_v_s[kArgSplit][kArgFrames];
   __shared__ int best_w_s[kArgSplit][kArgFrames];
+  const int R = kR > 0 ? kR : R_any;
   const int b = blockIdx.y;
   const int tx = threadIdx.x % kArgFrames, grp = threadIdx.x / kArgFrames;
   const int t = blockIdx.x * kArgFrames + tx;
@@ -55,11 +58,30 @@ __global__ __launch_bounds__(kArgFrames * kArgSplit) void PruneArgmaxKernel(
   const int w_lo = grp * per, w_hi = min(n_win, w_lo + per);
   T best_v = 0;
   int best = -1;
-  if (t < Tn) {
-    for (int w = w_lo; w < w_hi; ++w) {
-      T acc = gy[(size_t)w * Tn + t];
+  auto window = [&](int w) -> T {
+    T acc = gy[(size_t)w * Tn + t];
+    if (kR > 0) {
+#pragma unroll
+      for (int k = 1; k < kR; ++k) acc = acc + gy[(size_t)(w + k) * Tn + t];
+    } else {
       for (int k = 1; k < R; ++k) acc = acc + gy[(size_t)(w + k) * Tn + t];
-      const T v = acc - (w == 0 ? T(0) : gx[(size_t)(w - 1) * T1 + t]);
+    }
+    return acc - (w == 0 ? T(0) : gx[(size_t)(w - 1) * T1 + t]);
+  };
+  if (t < Tn) {
+    int w = w_lo;
+    if (kR > 0) {
+      for (; w + 4 <= w_hi; w += 4) {
+        T v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = window(w + i);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (best < 0 || v[i] > best_v) { best_v = v[i]; best = w + i; }
+      }
+    }
+    for (; w < w_hi; ++w) {
+      const T v = window(w);
       if (best < 0 || v > best_v) { best_v = v; best = w; }
     }
   }
@@ -74,6 +96,26 @@ __global__ __launch_bounds__(kArgFrames * kArgSplit) void PruneArgmaxKernel(
     }
     ranges[((size_t)b * Tn + t) * R] = best < 0 ? 0 : best;
   }
+}
+
+template <typename T>
+void LaunchArgmax(const T *px_grad, const T *py_grad, int64_t *ranges, int S, int Tn, int modified,
+                  int R, dim3 grid, hipStream_t st) {
+  const dim3 block(kArgFrames * kArgSplit);
+#define K2AMD_ARGMAX(KR)                                                                         \
+  hipLaunchKernelGGL((PruneArgmaxKernel<T, KR>), grid, block, 0, st, px_grad, py_grad, ranges, S, \
+                     Tn, modified, R)
+  switch (R) {
+    case 2: K2AMD_ARGMAX(2); break;
+    case 3: K2AMD_ARGMAX(3); break;
+    case 4: K2AMD_ARGMAX(4); break;
+    case 5: K2AMD_ARGMAX(5); break;
+    case 6: K2AMD_ARGMAX(6); break;
+    case 7: K2AMD_ARGMAX(7); break;
+    case 8: K2AMD_ARGMAX(8); break;
+    default: K2AMD_ARGMAX(0); break;
+  }
+#undef K2AMD_ARGMAX
 }
 
 // Step 2: one workgroup per sequence.  Frames from t_end - 1 on are pinned to
@@ -165,9 +207,9 @@ int k2amd_rnnt_prune_ranges(const void *px_grad, const void *py_grad, const int6
   modified = modified ? 1 : 0;
   const dim3 grid1((unsigned)((T + kArgFrames - 1) / kArgFrames), (unsigned)B);
   if (dtype == K2AMD_F32)
-    hipLaunchKernelGGL(PruneArgmaxKernel<float>, grid1, dim3(kArgFrames * kArgSplit), 0, st, (const float *)px_grad, (const float *)py_grad, ranges, S, T, modified, s_range);
+    LaunchArgmax((const float *)px_grad, (const float *)py_grad, ranges, S, T, modified, s_range, grid1, st);
   else
-    hipLaunchKernelGGL(PruneArgmaxKernel<double>, grid1, dim3(kArgFrames * kArgSplit), 0, st, (const double *)px_grad, (const double *)py_grad, ranges, S, T, modified, s_range);
+    LaunchArgmax((const double *)px_grad, (const double *)py_grad, ranges, S, T, modified, s_range, grid1, st);
   hipLaunchKernelGGL(PruneFinishKernel, dim3(B), dim3(kPruneThreads), smem, st, boundary, ranges, T, modified, s_range);
   return LaunchStatus();
 }

@@ -693,7 +693,15 @@ __global__ void AmBlankTermKernel(GradView<T> gv, T *__restrict__ am_grad, int B
   if (i >= B * gv.Tn) return;
   const int b = i / gv.Tn, t = i - b * gv.Tn;
   T sy = 0;
-  for (int s = 0; s <= gv.S; ++s) sy += gv.Gy(b, s, t);
+  int s = 0;
+  for (; s + 8 <= gv.S + 1; s += 8) {  // eight rows' loads in flight at a time
+    T v[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] = gv.Gy(b, s + k, t);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) sy += v[k];
+  }
+  for (; s <= gv.S; ++s) sy += gv.Gy(b, s, t);
   am_grad[(size_t)i * C + blank] += sy;
 }
 
