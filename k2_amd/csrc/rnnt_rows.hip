@@ -210,11 +210,14 @@ __global__ void RowEmitKernel(const T *__restrict__ logits, const T *__restrict_
   py[((size_t)b * (g.S + 1) + s) * g.Tn + t] = yv;
 }
 
+// Both outputs of the pruned builder start as -inf everywhere (one launch for the two tensors).
 template <typename T>
-__global__ void FillKernel(T *__restrict__ dst, size_t n, T value) {
-  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-       i += (size_t)gridDim.x * blockDim.x)
-    dst[i] = value;
+__global__ void FillPairKernel(T *__restrict__ a, size_t na, T *__restrict__ b, size_t nb, T value) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < na + nb; i += stride) {
+    if (i < na) a[i] = value;
+    else b[i - na] = value;
+  }
 }
 
 // px[b,s,T] = -inf for a regular lattice (k2/python/k2/rnnt_loss.py:193-205).
@@ -403,8 +406,7 @@ int RowForward(const T *logits, const int64_t *symbols, const int64_t *ranges,
   const int T1 = g.rnnt_type == K2AMD_REGULAR ? g.Tn + 1 : g.Tn;
   const size_t n_px = (size_t)g.B * g.S * T1, n_py = (size_t)g.B * (g.S + 1) * g.Tn;
   if (kPruned) {
-    if (n_px) hipLaunchKernelGGL(FillKernel<T>, dim3(1024), dim3(256), 0, stream, px, n_px, Real<T>::NegInf());
-    if (n_py) hipLaunchKernelGGL(FillKernel<T>, dim3(1024), dim3(256), 0, stream, py, n_py, Real<T>::NegInf());
+    if (n_px + n_py) hipLaunchKernelGGL(FillPairKernel<T>, dim3(2048), dim3(256), 0, stream, px, n_px, py, n_py, Real<T>::NegInf());
   } else if (g.rnnt_type == K2AMD_REGULAR && g.B * g.S > 0) {
     hipLaunchKernelGGL(LastColumnKernel<T>, dim3((g.B * g.S + 255) / 256), dim3(256), 0, stream, px, g.B * g.S, T1);
   }

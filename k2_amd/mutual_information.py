@@ -4,12 +4,33 @@ Same function names, argument meaning, return values and exception classes as th
 the two native calls ``_k2.mutual_information_forward/backward`` are replaced by the HIP
 kernels of libk2amd.so.  Tensors must live on a ROCm device: there is no CPU fallback.
 """
+import weakref
 from typing import List, Optional, Sequence, Tuple, Union
 
 import torch
 from torch import Tensor
 
 from . import native
+
+
+# boundary tensors whose values passed the range asserts: id(tensor) -> (weak reference, verdict key)
+_checked_boundaries = {}
+
+
+def _check_boundary(boundary: Tensor, S: int, T: int) -> None:
+    """The range asserts of k2/python/k2/mutual_information.py:284-289.  Reading the values is a
+    device-to-host copy that waits for everything queued on the stream, so the verdict is kept
+    per tensor object and reused while the tensor has not been written to (its version counter)
+    and is checked against the same S and T; a new tensor is always read."""
+    ident = id(boundary)
+    key = (boundary._version, S, T)
+    hit = _checked_boundaries.get(ident)
+    if hit is not None and hit[0]() is boundary and hit[1] == key:
+        return
+    for s_begin, t_begin, s_end, t_end in boundary.tolist():
+        assert 0 <= s_begin <= s_end <= S, (s_begin, s_end, S)
+        assert 0 <= t_begin <= t_end <= T, (t_begin, t_end, T)
+    _checked_boundaries[ident] = (weakref.ref(boundary, lambda _, i=ident: _checked_boundaries.pop(i, None)), key)
 
 
 class MutualInformationRecursionFunction(torch.autograd.Function):
@@ -70,9 +91,7 @@ def mutual_information_recursion(
     if boundary is not None:
         assert boundary.dtype == torch.int64, boundary.dtype
         assert boundary.shape == (B, 4), (boundary.shape, B)
-        for s_begin, t_begin, s_end, t_end in boundary.tolist():
-            assert 0 <= s_begin <= s_end <= S, (s_begin, s_end, S)
-            assert 0 <= t_begin <= t_end <= T, (t_begin, t_end, T)
+        _check_boundary(boundary, S, T)
 
     px, py = px.contiguous(), py.contiguous()
     pxy_grads = [None, None]
@@ -106,9 +125,7 @@ def joint_mutual_information_recursion(
     if boundary is not None:
         assert boundary.dtype == torch.int64
         assert boundary.shape == (B, 4)
-        for s_begin, t_begin, s_end, t_end in boundary.tolist():
-            assert 0 <= s_begin <= s_end <= S, (s_begin, s_end, S)
-            assert 0 <= t_begin <= t_end <= T, (t_begin, t_end, T)
+        _check_boundary(boundary, S, T)
 
     px_cat = torch.stack(list(px), dim=0)  # [N][B][S][T1]
     py_cat = torch.stack(list(py), dim=0)  # [N][B][S+1][T]
