@@ -830,7 +830,13 @@ __global__ __launch_bounds__(BwdLayout::kThreads) void MiBackwardFastKernel(
       if (row_i > g.ns) continue;
       const int pq = (kb % 3) * kQuadsPerBlock + mm;
       const int pq_right = mm + 1 < kQuadsPerBlock ? pq + 1 : ((kb + 1) % 3) * kQuadsPerBlock;
-      const float4 e4 = lds.e[q][pq], o4 = lds.ome[q][pq], g4 = lds.g[q][pq], gr = lds.g[q][pq_right];
+      const float4 e4 = lds.e[q][pq], o4 = lds.ome[q][pq];
+      float4 g4 = lds.g[q][pq], gr = lds.g[q][pq_right];
+      // Only three floats of g4 and one of gr are used, and the compiler would fetch just those
+      // with 4-byte reads: lanes that are whole quads apart then share 16 of the 64 banks (4-way
+      // conflicts).  Whole-quad reads are conflict-free.
+      asm volatile("" : "+v"(g4.x), "+v"(g4.y), "+v"(g4.z), "+v"(g4.w));
+      asm volatile("" : "+v"(gr.x), "+v"(gr.y), "+v"(gr.z), "+v"(gr.w));
       const float gv[4] = {g4.y, g4.z, g4.w, gr.x};
       const float hv[4] = {e4.x * gv[0], e4.y * gv[1], e4.z * gv[2], e4.w * gv[3]};
       const float cv[4] = {o4.x * gv[0], o4.y * gv[1], o4.z * gv[2], o4.w * gv[3]};
