@@ -31,7 +31,7 @@ BWD_BYTES_PER_CELL = 16
 # HBM bytes per launch on the default workload, from rocprofv3's FETCH_SIZE / WRITE_SIZE counters
 # scaled by a 256 MiB device copy (profiles/mi_fast_kernels_c4_hbm_traffic.md).  Reported only
 # for the default shape; any other --B/--S/--T prints null.
-MEASURED_TRAFFIC_BYTES = {"mi_forward": 50045338, "mi_backward": 86139378}
+MEASURED_TRAFFIC_BYTES = {"mi_forward": 50049796, "mi_backward": 86230408}
 
 
 def cpu_baseline(c, budget_s=12.0):
