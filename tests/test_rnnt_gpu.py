@@ -434,3 +434,39 @@ def test_variants_degenerate_shapes(device):
     am = torch.randn(0, T, C, device=device)
     e = k2.rnnt_loss_smoothed(lm, am, torch.zeros(0, S, dtype=torch.long, device=device), 0, reduction="none")
     assert e.shape == (0,)
+
+
+@pytest.mark.parametrize("rnnt_type", TYPES)
+def test_logprobs_simple_fp32_products_vs_fp64(device, rnnt_type):
+    """The fp32 batched products run on the matrix cores (two kernels by size, 16-byte and scalar
+    operand loads, ragged edges in M, N and K); fp64 runs on the vector ALUs and is tied to autograd
+    by test_api_losses_and_gradients_vs_autograd.  Same inputs, same incoming gradients: px, py and
+    the gradients with respect to lm and am must agree to the fp32 tolerance (1e-4 relative; the
+    1e-5 absolute part is taken relative to the tensor's largest magnitude, the gradients being
+    sums over up to 500 frames)."""
+    from k2_amd import capi, native
+    code = capi.RNNT_TYPES[rnnt_type]
+    rng = np.random.default_rng(91)
+    shapes = ((3, 37, 9, 50),        # small, rows not a multiple of four: split-K kernel, scalar loads
+              (2, 70, 66, 132),      # split-K kernel, 16-byte loads, K = 132 = 8 x 16 + 4
+              (16, 250, 50, 500),    # config 2: the am gradient takes the LDS kernel
+              (64, 203, 70, 130),    # LDS kernel everywhere, scalar loads, ragged in every axis
+              (32, 500, 100, 500))   # config 3: LDS kernel, 16-byte loads
+    for (B, T, S, C) in shapes:
+        c = cases.rnnt_case(B + T, B, T, S, C, t_lo=max(T // 2, S), s_lo=S // 2, modified=rnnt_type != "regular")
+        sym, bd = dev(c["symbols"], device), dev(c["boundary"], device)
+        T1 = T + 1 if rnnt_type == "regular" else T
+        gpx = rng.random((B, S, T1)).astype(np.float32)
+        gpy = rng.random((B, S + 1, T)).astype(np.float32)
+        res = {}
+        for dt in (torch.float32, torch.float64):
+            lm, am = dev(c["lm"], device).to(dt), dev(c["am"], device).to(dt)
+            px, py, saved = native.logprobs_simple_forward(lm, am, sym, 0, code, bd)
+            lm_g, am_g = native.logprobs_simple_backward(dev(gpx, device).to(dt), dev(gpy, device).to(dt), sym, bd,
+                                                         saved, 0, code)
+            res[dt] = [t.double().cpu().numpy() for t in (px, py, lm_g, am_g)]
+        for name, a, b in zip(("px", "py", "lm_grad", "am_grad"), res[torch.float32], res[torch.float64]):
+            scale = max(1.0, float(np.abs(b[np.isfinite(b)]).max()))
+            with np.errstate(invalid="ignore"):
+                ok = np.isclose(a, b, rtol=1e-4, atol=1e-5 * scale, equal_nan=True) | (a == b)
+            assert ok.all(), (name, (B, T, S, C), int((~ok).sum()), a[~ok][:4], b[~ok][:4])
