@@ -95,7 +95,7 @@ def test_prune_ranges_bit_exact(device, modified):
         rt = "modified" if modified else "regular"
         px, py = orn.logprobs_simple(c["lm"], c["am"], c["symbols"], 0, rt, c["boundary"])
         _, gx, gy = omi.mi(px, py, c["boundary"])
-        for R in (2, 5, S + 1):
+        for R in (2, 3, 4, 5, 6, 7, 8, 9, S + 1):  # 2..8: kernels specialised on the window length
             want = orn.prune_ranges(gx, gy, c["boundary"], R)
             got = capi.prune_ranges(dev(gx, device), dev(gy, device), dev(c["boundary"], device), want.shape[2])
             assert got.dtype == torch.int64
