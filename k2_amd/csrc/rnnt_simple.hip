@@ -7,7 +7,8 @@
 // px / py directly, so the normaliser never makes a round trip through HBM as a separate tensor
 // apart from the `denom` buffer kept for the backward.
 // Backward: Q = (dpx + dpy) / denom, two more batched products (Q * am_probs, Q^T * lm_probs)
-// scaled by the saved exponentials, plus the gathered symbol / termination terms.
+// scaled by the saved exponentials; the symbol terms of the am gradient ride in that product's
+// epilogue, the termination terms and the lm gradient's gathered terms have small kernels.
 #include "common.h"
 
 namespace k2amd {
@@ -80,6 +81,10 @@ struct MatView {
 };
 
 constexpr int kTile = 64, kTileK = 16, kPad = 4;
+// LDS scratch an epilogue may ask for (see AmGradEpilogue): per tile column a count and up to
+// kMaxHits entries
+constexpr int kStageColumns = 64, kMaxHits = 4;
+constexpr int kStageInts = kStageColumns * (1 + kMaxHits);
 
 // fp64: one 64 x 64 output tile per workgroup, K in steps of 16 staged through LDS as As[k][m],
 // Bs[k][n] (scalar, bounds-checked loads: any stride works), 16 x 16 threads with 4 x 4 outputs
@@ -91,6 +96,7 @@ __global__ __launch_bounds__(256) void BatchedProductKernel(const T *__restrict_
                                                             int M, int N, int K, Epilogue epi) {
   __shared__ T As[kTileK][kTile + kPad];
   __shared__ T Bs[kTileK][kTile + kPad];
+  __shared__ int stage[kStageInts];
   const int b = blockIdx.z;
   const int m0 = blockIdx.y * kTile, n0 = blockIdx.x * kTile;
   const T *Ab = A + (size_t)b * av.batch;
@@ -129,11 +135,12 @@ __global__ __launch_bounds__(256) void BatchedProductKernel(const T *__restrict_
     }
     __syncthreads();
   }
+  if constexpr (Epilogue::kStaged) epi.Stage(b, n0, kTile, stage);
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int n = n0 + tx * 4 + j;
     if (n >= N) continue;
-    const auto column = epi.Column(b, n);
+    const auto column = epi.Column(b, n, n - n0, stage);
     typename Epilogue::ElementData pre[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -203,6 +210,7 @@ __global__ __launch_bounds__(256) void ProductSplitKKernel(const float *__restri
                                                          int M, int N, int K, int tiles_n,
                                                          int tiles_m, int total, Epilogue epi) {
   __shared__ float part[4][kMfmaTile][kMfmaTile + 1];
+  __shared__ int stage[kStageInts];
   const int per_xcd = (total + 7) / 8;
   const int id = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if (id >= total) return;
@@ -273,8 +281,9 @@ __global__ __launch_bounds__(256) void ProductSplitKKernel(const float *__restri
 #pragma unroll
   for (int r = 0; r < 16; ++r) part[wave][(r >> 2) * 8 + half * 4 + (r & 3)][col] = acc[r];
   __syncthreads();
+  if constexpr (Epilogue::kStaged) epi.Stage(b, n0, kMfmaTile, stage);
   if (n >= N) return;
-  const auto column = epi.Column(b, n);
+  const auto column = epi.Column(b, n, col, stage);
   typename Epilogue::ElementData pre[4];
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
@@ -377,6 +386,7 @@ __global__ __launch_bounds__(256) void ProductLdsKernel(const float *__restrict_
                                                         int tiles_m, int total, Epilogue epi) {
   __shared__ __attribute__((aligned(16))) float As[2][kKc][kLdsRow];
   __shared__ __attribute__((aligned(16))) float Bs[2][kKc][kLdsRow];
+  __shared__ int stage[kStageInts];
   const int per_xcd = (total + 7) / 8;
   const int id = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if (id >= total) return;
@@ -438,9 +448,10 @@ __global__ __launch_bounds__(256) void ProductLdsKernel(const float *__restrict_
     chunk(c, fa[0], fb[0], fa[1], fb[1]);
     if (c + 1 < chunks) chunk(c + 1, fa[1], fb[1], fa[0], fb[0]);
   }
+  if constexpr (Epilogue::kStaged) epi.Stage(b, n0, kTile, stage);
   const int n = n0 + qn + col;
   if (n >= N) return;
-  const auto column = epi.Column(b, n);
+  const auto column = epi.Column(b, n, qn + col, stage);
   typename Epilogue::ElementData pre[16];
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
@@ -524,12 +535,33 @@ struct Tiny<float> { static constexpr float v = 1.17549435e-38f; };   // torch.f
 template <>
 struct Tiny<double> { static constexpr double v = 2.2250738585072014e-308; };
 
+// Effective gradients of the un-fixed px / py values at (b,s,t), t < T.
+template <typename T>
+struct GradView {
+  const T *px_grad, *py_grad;
+  const int64_t *boundary;
+  int S, Tn, rnnt_type;
+  __device__ __forceinline__ T Gx(int b, int s, int t) const {
+    if (s >= S) return 0;
+    if (rnnt_type == K2AMD_REGULAR && boundary != nullptr && boundary[4 * b + 3] == t) return 0;
+    const int T1 = rnnt_type == K2AMD_REGULAR ? Tn + 1 : Tn;
+    return px_grad[((size_t)b * S + s) * T1 + t];
+  }
+  __device__ __forceinline__ T Gy(int b, int s, int t) const {
+    T g = py_grad[((size_t)b * (S + 1) + s) * Tn + t];
+    if (rnnt_type == K2AMD_CONSTRAINED && s >= 1) g += Gx(b, s - 1, t);
+    return g;
+  }
+};
+
 // Epilogues work in two steps so that a thread can issue the loads of all its elements before
 // the first store (the compiler cannot move a load across a store that might alias it, and one
 // dependent round trip per element is what the tile's epilogue would otherwise cost):
-//   column = epi.Column(b, n)          what depends on (b, n) only
-//   pre    = epi.Prepare(b, m, n, column)   loads for element (m, n)
-//   epi.Finish(b, m, n, acc, column, pre)   arithmetic and stores
+//   epi.Stage(b, n0, width, scratch)          (only if Epilogue::kStaged; whole workgroup, has
+//                                              barriers) what depends on the tile's columns
+//   column = epi.Column(b, n, n - n0, scratch)   what depends on (b, n) only
+//   pre    = epi.Prepare(b, m, n, column)        loads for element (m, n)
+//   epi.Finish(b, m, n, acc, column, pre)        arithmetic and stores
 
 // Forward epilogue: (m, n) = (s, t).  Also writes the -inf column px[b,s,T] of a regular lattice
 // (k2/python/k2/rnnt_loss.py:193-205) from the threads that hold t = T-1.
@@ -547,7 +579,8 @@ struct ForwardEpilogue {
   struct ElementData {
     T lm_max, lm_blank, sym_sum;  // sym_sum = am[b,t,sym] + lm[b,s,sym], -inf without a symbol
   };
-  __device__ __forceinline__ ColumnData Column(int b, int t) const {
+  static constexpr bool kStaged = false;
+  __device__ __forceinline__ ColumnData Column(int b, int t, int, const int *) const {
     ColumnData c;
     c.amr = am + ((size_t)b * Tn + t) * C;
     c.am_max = am_max[(size_t)b * Tn + t];
@@ -592,13 +625,86 @@ struct ScaleEpilogue {
   int M, N;
   struct ColumnData {};
   struct ElementData { T scale; };
-  __device__ __forceinline__ ColumnData Column(int, int) const { return ColumnData(); }
+  static constexpr bool kStaged = false;
+  __device__ __forceinline__ ColumnData Column(int, int, int, const int *) const { return ColumnData(); }
   __device__ __forceinline__ ElementData Prepare(int b, int m, int n, const ColumnData &) const {
     return ElementData{scale[((size_t)b * M + m) * N + n]};
   }
   __device__ __forceinline__ void Finish(int b, int m, int n, T acc, const ColumnData &,
                                          const ElementData &e) const {
     out[((size_t)b * M + m) * N + n] = -e.scale * acc;
+  }
+};
+
+// Epilogue of the am gradient, (m, n) = (t, c):
+//   am_grad[b,t,c] = -am_probs[b,t,c] * acc + sum over s with symbols[b,s] == c of Gx(b,s,t).
+// Stage lists, for each of the tile's columns, the positions s whose symbol is that column (up
+// to kMaxHits, sorted; longer lists are rescanned per element), so that the symbol terms cost a
+// tile one pass over the sequence's symbols instead of a launch of their own.  The terms of an
+// element are added in the order of s: the result does not depend on scheduling.
+template <typename T>
+struct AmGradEpilogue {
+  static constexpr bool kStaged = true;
+  const T *scale;
+  T *out;
+  GradView<T> gv;
+  const int64_t *symbols;
+  int M, N;  // Tn, C
+  struct ColumnData {
+    int hits;  // positions s with symbols[b,s] == c (all of them, also beyond kMaxHits)
+    int s[kMaxHits];
+  };
+  struct ElementData { T scale, sym_sum; };
+  __device__ void Stage(int b, int n0, int width, int *scratch) const {
+    int *count = scratch, *hit = scratch + kStageColumns;
+    for (int i = threadIdx.x; i < kStageColumns; i += blockDim.x) count[i] = 0;
+    __syncthreads();
+    const int64_t *sym = symbols + (size_t)b * gv.S;
+    for (int s = threadIdx.x; s < gv.S; s += blockDim.x) {
+      const int64_t c = sym[s] - n0;
+      if (c >= 0 && c < width) {
+        const int slot = atomicAdd(&count[c], 1);
+        if (slot < kMaxHits) hit[c * kMaxHits + slot] = s;
+      }
+    }
+    __syncthreads();
+    if (threadIdx.x < kStageColumns) {  // ascending s, whatever order the slots were claimed in
+      int *h = hit + threadIdx.x * kMaxHits;
+      const int n = min(count[threadIdx.x], kMaxHits);
+      for (int i = 1; i < n; ++i) {
+        const int v = h[i];
+        int j = i - 1;
+        for (; j >= 0 && h[j] > v; --j) h[j + 1] = h[j];
+        h[j + 1] = v;
+      }
+    }
+    __syncthreads();
+  }
+  __device__ __forceinline__ ColumnData Column(int, int, int local, const int *scratch) const {
+    ColumnData col;
+    col.hits = scratch[local];
+#pragma unroll
+    for (int k = 0; k < kMaxHits; ++k) col.s[k] = scratch[kStageColumns + local * kMaxHits + k];
+    return col;
+  }
+  __device__ __forceinline__ ElementData Prepare(int b, int t, int c, const ColumnData &col) const {
+    ElementData e;
+    e.scale = scale[((size_t)b * M + t) * N + c];
+    e.sym_sum = 0;
+    if (col.hits <= kMaxHits) {
+#pragma unroll
+      for (int k = 0; k < kMaxHits; ++k)
+        if (k < col.hits) e.sym_sum += gv.Gx(b, col.s[k], t);
+    } else {
+      const int64_t *sym = symbols + (size_t)b * gv.S;
+      for (int s = 0; s < gv.S; ++s)
+        if (sym[s] == c) e.sym_sum += gv.Gx(b, s, t);
+    }
+    return e;
+  }
+  __device__ __forceinline__ void Finish(int b, int t, int c, T acc, const ColumnData &,
+                                         const ElementData &e) const {
+    out[((size_t)b * M + t) * N + c] = -e.scale * acc + e.sym_sum;
   }
 };
 
@@ -625,25 +731,6 @@ __global__ void ConstrainedKernelS(T *__restrict__ px, const T *__restrict__ py,
     px[i] += py[b * (size_t)(S + 1) * Tn + Tn + rem];
   }
 }
-
-// Effective gradients of the un-fixed px / py values at (b,s,t), t < T.
-template <typename T>
-struct GradView {
-  const T *px_grad, *py_grad;
-  const int64_t *boundary;
-  int S, Tn, rnnt_type;
-  __device__ __forceinline__ T Gx(int b, int s, int t) const {
-    if (s >= S) return 0;
-    if (rnnt_type == K2AMD_REGULAR && boundary != nullptr && boundary[4 * b + 3] == t) return 0;
-    const int T1 = rnnt_type == K2AMD_REGULAR ? Tn + 1 : Tn;
-    return px_grad[((size_t)b * S + s) * T1 + t];
-  }
-  __device__ __forceinline__ T Gy(int b, int s, int t) const {
-    T g = py_grad[((size_t)b * (S + 1) + s) * Tn + t];
-    if (rnnt_type == K2AMD_CONSTRAINED && s >= 1) g += Gx(b, s - 1, t);
-    return g;
-  }
-};
 
 template <typename T>
 __global__ void QKernel(GradView<T> gv, const T *__restrict__ denom, T *__restrict__ q, int B) {
@@ -705,25 +792,6 @@ __global__ void AmBlankTermKernel(GradView<T> gv, T *__restrict__ am_grad, int B
   am_grad[(size_t)i * C + blank] += sy;
 }
 
-// am_grad[b,t,sym[b,s]] += Gx(b,s,t).  One thread per (b,s,t), hardware floating-point atomics:
-// symbols that repeat within a sequence add to the same element, in no fixed order (the sums
-// differ in the last bit from run to run only where a symbol repeats).
-template <typename T>
-__global__ void AmSymbolTermsKernel(GradView<T> gv, const int64_t *__restrict__ symbols,
-                                    T *__restrict__ am_grad, int B, int C) {
-  const size_t n = (size_t)B * gv.S * gv.Tn;
-  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-       i += (size_t)gridDim.x * blockDim.x) {
-    const int t = (int)(i % gv.Tn);
-    const int s = (int)((i / gv.Tn) % gv.S);
-    const int b = (int)(i / ((size_t)gv.Tn * gv.S));
-    const int64_t sym = symbols[(size_t)b * gv.S + s];
-    if (sym < 0 || sym >= C) continue;
-    const T g = gv.Gx(b, s, t);
-    if (g != 0) unsafeAtomicAdd(am_grad + ((size_t)b * gv.Tn + t) * C + sym, g);
-  }
-}
-
 template <typename T>
 int SimpleForward(const T *lm, const T *am, const int64_t *symbols, const int64_t *boundary, T *px,
                   T *py, T *lm_probs, T *am_probs, T *lm_max, T *am_max, T *denom, int B, int S,
@@ -761,17 +829,12 @@ int SimpleBackward(const T *px_grad, const T *py_grad, const int64_t *symbols,
       LaunchProduct<T, true, false>((const T *)q, av, am_probs, bv, S + 1, C, Tn, B, epi, st);
     }
     {  // am_grad[b][t][c] = -am_probs * sum_s q[b][s][t] * lm_probs[b][s][c]
-      ScaleEpilogue<T> epi{am_probs, am_grad, Tn, C};
+      AmGradEpilogue<T> epi{am_probs, am_grad, gv, symbols, Tn, C};
       MatView av{(size_t)(S + 1) * Tn, 1, Tn};   // A(m=t, k=s) = q[b][s][t]
       MatView bv{(size_t)(S + 1) * C, C, 1};     // B(k=s, n=c) = lm_probs[b][s][c]
       LaunchProduct<T, false, false>((const T *)q, av, lm_probs, bv, Tn, C, S + 1, B, epi, st);
     }
     hipLaunchKernelGGL(AmBlankTermKernel<T>, dim3((B * Tn + 255) / 256), dim3(256), 0, st, gv, am_grad, B, C, blank);
-    if (S > 0) {
-      const size_t n = (size_t)B * S * Tn;
-      const unsigned blocks = (unsigned)((n + 255) / 256 > 16384 ? 16384 : (n + 255) / 256);
-      hipLaunchKernelGGL(AmSymbolTermsKernel<T>, dim3(blocks), dim3(256), 0, st, gv, symbols, am_grad, B, C);
-    }
   } else {
     hipLaunchKernelGGL(ZeroKernelS<T>, dim3(256), dim3(256), 0, st, lm_grad, (size_t)B * (S + 1) * C);
   }
