@@ -470,3 +470,34 @@ def test_logprobs_simple_fp32_products_vs_fp64(device, rnnt_type):
             with np.errstate(invalid="ignore"):
                 ok = np.isclose(a, b, rtol=1e-4, atol=1e-5 * scale, equal_nan=True) | (a == b)
             assert ok.all(), (name, (B, T, S, C), int((~ok).sum()), a[~ok][:4], b[~ok][:4])
+
+
+@pytest.mark.parametrize("rnnt_type", TYPES)
+def test_simple_gradients_with_often_repeated_symbols(device, rnnt_type):
+    """Two non-blank classes and nine symbols: every symbol repeats more often than the am
+    gradient's epilogue lists per column, so it takes its rescanning path; fp64 against torch
+    autograd on the CPU, fp32 against fp64."""
+    import k2_amd as k2
+    B, T, S, C = 2, 13, 9, 3
+    c = cases.rnnt_case(31, B, T, S, C, dtype=np.float64, t_lo=11, s_lo=7, modified=rnnt_type != "regular")
+    assert max(np.bincount(c["symbols"][0])) > 4
+    bd_cpu, sym_cpu = torch.from_numpy(c["boundary"]), torch.from_numpy(c["symbols"])
+    lm_r = torch.from_numpy(c["lm"]).requires_grad_(True)
+    am_r = torch.from_numpy(c["am"]).requires_grad_(True)
+    px, py = torch_ref.logprobs_simple(lm_r, am_r, sym_cpu, 0, rnnt_type, bd_cpu)
+    loss_r = -torch_ref.mi_scores(px, py, bd_cpu)
+    loss_r.sum().backward()
+    grads = {}
+    for dt in (torch.float64, torch.float32):
+        lm_g = dev(c["lm"], device).to(dt).requires_grad_(True)
+        am_g = dev(c["am"], device).to(dt).requires_grad_(True)
+        loss_g = k2.rnnt_loss_simple(lm_g, am_g, dev(c["symbols"], device), 0, dev(c["boundary"], device),
+                                     rnnt_type=rnnt_type, reduction="none")
+        loss_g.sum().backward()
+        grads[dt] = (loss_g.detach().double().cpu().numpy(), lm_g.grad.double().cpu().numpy(),
+                     am_g.grad.double().cpu().numpy())
+    np.testing.assert_allclose(grads[torch.float64][0], loss_r.detach().numpy(), rtol=1e-10)
+    np.testing.assert_allclose(grads[torch.float64][1], lm_r.grad.numpy(), rtol=1e-8, atol=1e-10)
+    np.testing.assert_allclose(grads[torch.float64][2], am_r.grad.numpy(), rtol=1e-8, atol=1e-10)
+    for a, b in zip(grads[torch.float32], grads[torch.float64]):
+        np.testing.assert_allclose(a, b, rtol=1e-4, atol=1e-5)
