@@ -160,10 +160,29 @@ __device__ __forceinline__ void RowTarget(const RowGeom &g, const int64_t *__res
 // `normalizers`.  Nothing else: the look-ups that decide where a row's two log-probs go are a
 // chain of dependent memory round trips, and paying that chain once per WAVEFRONT (one row)
 // rather than once per LANE (64 rows, pass 2) cost a third of this kernel's time.
+// The launch also carries the -inf fills that px / py need before pass 2 writes into them (work
+// that is independent of the normalisers): workgroups past the first `norm_blocks` set
+// a[i * stride_a] (i < na) and b[i] (i < nb) to -inf.  Pruned builder: all of px and py (everything
+// outside the band stays -inf); joint builder, regular lattice: the column px[b,s,T]
+// (k2/python/k2/rnnt_loss.py:193-205).
+template <typename T>
+struct NegInfFill {
+  T *a, *b;
+  size_t na, nb;
+  int stride_a;
+};
+
 template <typename T>
 __global__ __launch_bounds__(kRowsPerBlock *kWave) void RowNormKernel(
     const T *__restrict__ logits, T *__restrict__ normalizers, long long rows, int C,
-    bool skip_first) {
+    bool skip_first, unsigned norm_blocks, NegInfFill<T> fill) {
+  if (blockIdx.x >= norm_blocks) {
+    const size_t first = (size_t)(blockIdx.x - norm_blocks) * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)(gridDim.x - norm_blocks) * blockDim.x;
+    for (size_t i = first; i < fill.na; i += stride) fill.a[i * fill.stride_a] = Real<T>::NegInf();
+    for (size_t i = first; i < fill.nb; i += stride) fill.b[i] = Real<T>::NegInf();
+    return;
+  }
   const int lane = threadIdx.x & (kWave - 1);
   const long long row = (long long)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
   if (row >= rows) return;
@@ -208,23 +227,6 @@ __global__ void RowEmitKernel(const T *__restrict__ logits, const T *__restrict_
     px[((size_t)b * g.S + s) * T1 + t] = v;
   }
   py[((size_t)b * (g.S + 1) + s) * g.Tn + t] = yv;
-}
-
-// Both outputs of the pruned builder start as -inf everywhere (one launch for the two tensors).
-template <typename T>
-__global__ void FillPairKernel(T *__restrict__ a, size_t na, T *__restrict__ b, size_t nb, T value) {
-  const size_t stride = (size_t)gridDim.x * blockDim.x;
-  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < na + nb; i += stride) {
-    if (i < na) a[i] = value;
-    else b[i - na] = value;
-  }
-}
-
-// px[b,s,T] = -inf for a regular lattice (k2/python/k2/rnnt_loss.py:193-205).
-template <typename T>
-__global__ void LastColumnKernel(T *__restrict__ px, int rows, int T1) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < rows) px[(size_t)i * T1 + (T1 - 1)] = Real<T>::NegInf();
 }
 
 // px[b,s,t] += py[b,s+1,t] (k2/python/k2/rnnt_loss.py:222-223); T1 == Tn here.
@@ -405,19 +407,25 @@ int RowForward(const T *logits, const int64_t *symbols, const int64_t *ranges,
                hipStream_t stream) {
   const int T1 = g.rnnt_type == K2AMD_REGULAR ? g.Tn + 1 : g.Tn;
   const size_t n_px = (size_t)g.B * g.S * T1, n_py = (size_t)g.B * (g.S + 1) * g.Tn;
+  NegInfFill<T> fill{px, py, 0, 0, 1};
   if (kPruned) {
-    if (n_px + n_py) hipLaunchKernelGGL(FillPairKernel<T>, dim3(2048), dim3(256), 0, stream, px, n_px, py, n_py, Real<T>::NegInf());
-  } else if (g.rnnt_type == K2AMD_REGULAR && g.B * g.S > 0) {
-    hipLaunchKernelGGL(LastColumnKernel<T>, dim3((g.B * g.S + 255) / 256), dim3(256), 0, stream, px, g.B * g.S, T1);
+    fill.na = n_px;
+    fill.nb = n_py;
+  } else if (g.rnnt_type == K2AMD_REGULAR) {
+    fill.a = px + (T1 - 1);
+    fill.na = (size_t)g.B * g.S;
+    fill.stride_a = T1;
   }
+  const size_t fill_items = fill.na + fill.nb;
+  const unsigned fill_blocks = (unsigned)((fill_items + 4095) / 4096 > 1024 ? 1024 : (fill_items + 4095) / 4096);
   const long long rows = (long long)g.B * g.Tn * g.K;
-  if (rows > 0) {
-    const long long blocks = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
-    hipLaunchKernelGGL((RowNormKernel<T>), dim3((unsigned)blocks), dim3(kRowsPerBlock * kWave), 0, stream,
-                       logits, normalizers, rows, g.C, g.hat != 0);
+  const long long blocks = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
+  if (blocks + fill_blocks > 0)
+    hipLaunchKernelGGL((RowNormKernel<T>), dim3((unsigned)blocks + fill_blocks), dim3(kRowsPerBlock * kWave), 0, stream,
+                       logits, normalizers, rows, g.C, g.hat != 0, (unsigned)blocks, fill);
+  if (rows > 0)
     hipLaunchKernelGGL((RowEmitKernel<T, kPruned>), dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, stream,
                        logits, (const T *)normalizers, symbols, ranges, boundary, px, py, g);
-  }
   if (g.rnnt_type == K2AMD_CONSTRAINED && n_px > 0)
     hipLaunchKernelGGL(ConstrainedKernel<T>, dim3(1024), dim3(256), 0, stream, px, py, g.B, g.S, g.Tn);
   return LaunchStatus();
