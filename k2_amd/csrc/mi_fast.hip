@@ -11,8 +11,9 @@
 //     j = n - q*skew at step n (skew = 1 for the regular lattice, 0 for the modified one), so
 //     every cell depends on the previous step only: its own lane's value and the neighbouring
 //     lane's, fetched with a DPP wave shift (no LDS, no barrier inside a step).  The lane at the
-//     end of the wavefront has no neighbour; the value arriving from the adjacent chunk is
-//     injected there through the DPP's "old" operand.
+//     end of the wavefront has no neighbour: the DPP operation leaves its register as it is, and
+//     what that register holds is the value arriving from the adjacent chunk (an extra LDS row
+//     filled by the edge wavefront).
 //   * four LOADER wavefronts issue coalesced, branch-free quad loads of row segments three blocks
 //     ahead of use and, two iterations later, place them into an LDS ring PRE-SKEWED (element for
 //     lane q, step n at ring position n) so the chain wavefront reads 4 steps per lane with one
@@ -29,7 +30,7 @@
 // is clean again when the kernel ends.  Each word is self-validating, so no fences and no cache
 // flushes are needed.  Workgroups take their chunk from a ticket counter, which guarantees that
 // the chunk a workgroup waits for has already started; the last workgroup to finish resets the
-// counter.  The workspace therefore needs ONE initialisation (MiFastWorkspaceInit) and no
+// counter.  The workspace therefore needs ONE initialisation (k2amd_mi_workspace_init) and no
 // per-call setup kernel.  Every wait is bounded; a timeout raises the header's error flag, after
 // which every later wait returns at once.
 //
