@@ -239,6 +239,8 @@ def main():
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch one plain device copy of 256 MiB before the warmup: the unit "
                          "against which rocprofv3's FETCH_SIZE / WRITE_SIZE readings are scaled")
+    ap.add_argument("--no-keep", action="store_true",
+                    help="run the plain forward/backward pair (no log-derivative tensor between them)")
     ap.add_argument("--B", type=int, default=32)
     ap.add_argument("--S", type=int, default=200)
     ap.add_argument("--T", type=int, default=1000)
@@ -267,14 +269,18 @@ def main():
     full = B * (S + 1) * (T + 1)
     p = torch.empty(B, S + 1, T + 1, dtype=torch.float32, device=dev)
     ones = torch.ones(B, dtype=torch.float32, device=dev)
+    # as mutual_information_recursion does: the forward hands the backward the px-edge
+    # log-derivatives (one more [B][S+1][T+1] tensor written by the forward, read by the backward)
+    keep = not args.no_keep and capi.mi_keeps_log_deriv(px, py)
+    log_deriv = torch.empty_like(p) if keep else None
 
     def step(ev=None):
         if ev is not None:
             ev[0].record()
-        capi.mi_forward(px, py, bd, p)
+        capi.mi_forward(px, py, bd, p, log_deriv=log_deriv)
         if ev is not None:
             ev[1].record()
-        g = capi.mi_backward(px, py, bd, p, ones, overwrite_ans_grad=False)
+        g = capi.mi_backward(px, py, bd, p, ones, overwrite_ans_grad=False, log_deriv=log_deriv)
         if ev is not None:
             ev[2].record()
         return g
@@ -318,7 +324,7 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"mutual_information_recursion fwd+bwd, fp32, modified, B={B} "
                                f"S={S} T={T}, random boundary (BASELINE config 4)",
-                   "active_cells": active, "full_box_cells": full},
+                   "active_cells": active, "full_box_cells": full, "log_deriv_kept": bool(keep)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC_BYTES[dom] if (B, S, T) == (32, 200, 1000) else None,

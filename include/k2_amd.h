@@ -80,6 +80,27 @@ K2AMD_API int k2amd_mi_backward(const void *px, const void *py, const int64_t *b
                       int modified, int dtype, int overwrite_ans_grad, void *workspace,
                       size_t workspace_bytes, void *stream);
 
+/* The pair below is k2amd_mi_forward / k2amd_mi_backward with one more tensor between them, for
+ * callers that run the backward right after the forward, as the reference's autograd function
+ * does (k2/python/k2/mutual_information.py:159-164).  It has no counterpart in the reference.
+ *   log_deriv [B][S+1][T+1], dtype as p: written by the forward, read by the backward.  It holds
+ *   (p[b,s-1,t+o] + px[b,s-1,t+o]) - p[b,s,t], the logarithm of the px edge's derivative at cell
+ *   (s,t) exactly as the backward sweep forms it (mutual_information_cpu.cu:195-211), so the
+ *   backward reads one tensor where it otherwise reads p twice and px once; the gradients are the
+ *   same bits either way.  Elements of a sequence's first row and first column are undefined.
+ * log_deriv == NULL makes each call identical to the plain entry point.  Only the pipelined fp32
+ * kernels use the tensor: k2amd_mi_keeps_log_deriv(...) tells whether the pair will (1) or will
+ * leave it untouched (0) for a shape, so that a host can skip the allocation.  Give the backward
+ * the tensor only if the forward call with the same shape, dtype and workspace wrote it.        */
+K2AMD_API int k2amd_mi_keeps_log_deriv(int B, int S, int T, int modified, int dtype, int has_workspace);
+K2AMD_API int k2amd_mi_forward_keep(const void *px, const void *py, const int64_t *boundary, void *p,
+                          void *ans, void *log_deriv, int B, int S, int T, int modified, int dtype,
+                          void *workspace, size_t workspace_bytes, void *stream);
+K2AMD_API int k2amd_mi_backward_kept(const void *px, const void *py, const int64_t *boundary, const void *p,
+                           const void *log_deriv, void *ans_grad, void *px_grad, void *py_grad,
+                           int B, int S, int T, int modified, int dtype, int overwrite_ans_grad,
+                           void *workspace, size_t workspace_bytes, void *stream);
+
 /* ------------------------------------------------------------------ RNN-T log-prob builders
  *
  * Common conventions: symbols [B][S] int64 in [0,C); boundary [B][4] int64 or NULL;

@@ -30,6 +30,9 @@ _SIGNATURES = {
     "k2amd_mi_forward": ([_vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp, _sz, _vp], _ci),
     "k2amd_mi_backward": ([_vp, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci,
                            _vp, _sz, _vp], _ci),
+    "k2amd_mi_keeps_log_deriv": ([_ci] * 6, _ci),
+    "k2amd_mi_forward_keep": ([_vp] * 6 + [_ci] * 5 + [_vp, _sz, _vp], _ci),
+    "k2amd_mi_backward_kept": ([_vp] * 8 + [_ci] * 6 + [_vp, _sz, _vp], _ci),
     "k2amd_rnnt_logprobs_simple_forward": ([_vp] * 11 + [_ci] * 7 + [_vp], _ci),
     "k2amd_rnnt_logprobs_simple_backward": ([_vp] * 10 + [_ci] * 7 + [_vp], _ci),
     "k2amd_rnnt_logprobs_joint_forward": ([_vp] * 6 + [_ci] * 7 + [_vp], _ci),
@@ -135,8 +138,19 @@ def mi_workspace_status(device):
             check(lib().k2amd_mi_workspace_status(ws.data_ptr(), stream.cuda_stream))
 
 
-def mi_forward(px, py, boundary, p):
-    """C-ABI twin of _k2.mutual_information_forward: fills ``p``, returns ans [B]."""
+def mi_keeps_log_deriv(px, py):
+    """True if mi_forward / mi_backward on these tensors use a ``log_deriv`` tensor when given one
+    (the pipelined fp32 kernels do; the exact kernels leave it untouched)."""
+    B, S, T1 = px.shape
+    T = py.shape[2]
+    dt = dtype_code(px)
+    has_ws = lib().k2amd_mi_workspace_bytes(B, S, T, int(T1 == T), dt) > 0
+    return bool(lib().k2amd_mi_keeps_log_deriv(B, S, T, int(T1 == T), dt, int(has_ws)))
+
+
+def mi_forward(px, py, boundary, p, log_deriv=None):
+    """C-ABI twin of _k2.mutual_information_forward: fills ``p``, returns ans [B].  ``log_deriv``
+    (optional, shaped like ``p``) receives what lets mi_backward skip its reads of p and px."""
     B, S, T1 = px.shape
     T = py.shape[2]
     modified = int(T1 == T)
@@ -144,14 +158,15 @@ def mi_forward(px, py, boundary, p):
     dt = dtype_code(px)
     ws = mi_workspace(B, S, T, modified, dt, px.device)
     with torch.cuda.device(px.device):
-        check(lib().k2amd_mi_forward(ptr(px), ptr(py), ptr(boundary), ptr(p), ptr(ans), B, S, T,
-                                     modified, dt, ptr(ws), 0 if ws is None else ws.numel(),
-                                     stream_ptr(px.device)))
+        check(lib().k2amd_mi_forward_keep(ptr(px), ptr(py), ptr(boundary), ptr(p), ptr(ans),
+                                          ptr(log_deriv), B, S, T, modified, dt, ptr(ws),
+                                          0 if ws is None else ws.numel(), stream_ptr(px.device)))
     return ans
 
 
-def mi_backward(px, py, boundary, p, ans_grad, overwrite_ans_grad=True):
-    """C-ABI twin of _k2.mutual_information_backward: returns (px_grad, py_grad)."""
+def mi_backward(px, py, boundary, p, ans_grad, overwrite_ans_grad=True, log_deriv=None):
+    """C-ABI twin of _k2.mutual_information_backward: returns (px_grad, py_grad).  ``log_deriv``:
+    the tensor the matching mi_forward call filled, or None."""
     B, S, T1 = px.shape
     T = py.shape[2]
     modified = int(T1 == T)
@@ -160,8 +175,8 @@ def mi_backward(px, py, boundary, p, ans_grad, overwrite_ans_grad=True):
     dt = dtype_code(px)
     ws = mi_workspace(B, S, T, modified, dt, px.device)
     with torch.cuda.device(px.device):
-        check(lib().k2amd_mi_backward(ptr(px), ptr(py), ptr(boundary), ptr(p), ptr(ans_grad),
-                                      ptr(px_grad), ptr(py_grad), B, S, T, modified, dt,
+        check(lib().k2amd_mi_backward_kept(ptr(px), ptr(py), ptr(boundary), ptr(p), ptr(log_deriv),
+                                           ptr(ans_grad), ptr(px_grad), ptr(py_grad), B, S, T, modified, dt,
                                       int(overwrite_ans_grad), ptr(ws),
                                       0 if ws is None else ws.numel(), stream_ptr(px.device)))
     return px_grad, py_grad

@@ -59,9 +59,21 @@ int k2amd_mi_workspace_status(const void *workspace, void *stream) {
   return header[2] != 0 ? K2AMD_ERR_TIMEOUT : K2AMD_OK;  // FastHeader::error
 }
 
+int k2amd_mi_keeps_log_deriv(int B, int S, int T, int modified, int dtype, int has_workspace) {
+  return dtype == K2AMD_F32 && has_workspace && ShapeOk(B, S, T) && B > 0 && !ForceGeneric() &&
+         MiFastSupports(B, S, T, modified ? 1 : 0);
+}
+
 int k2amd_mi_forward(const void *px, const void *py, const int64_t *boundary, void *p, void *ans,
                      int B, int S, int T, int modified, int dtype, void *workspace,
                      size_t workspace_bytes, void *stream) {
+  return k2amd_mi_forward_keep(px, py, boundary, p, ans, nullptr, B, S, T, modified, dtype,
+                               workspace, workspace_bytes, stream);
+}
+
+int k2amd_mi_forward_keep(const void *px, const void *py, const int64_t *boundary, void *p,
+                          void *ans, void *log_deriv, int B, int S, int T, int modified, int dtype,
+                          void *workspace, size_t workspace_bytes, void *stream) {
   if (!ShapeOk(B, S, T) || (dtype != K2AMD_F32 && dtype != K2AMD_F64)) return K2AMD_ERR_INVALID_ARGUMENT;
   if (B == 0) return K2AMD_OK;
   if (!p || !ans || (!px && S > 0) || (!py && T > 0)) return K2AMD_ERR_INVALID_ARGUMENT;
@@ -72,7 +84,7 @@ int k2amd_mi_forward(const void *px, const void *py, const int64_t *boundary, vo
   if (dtype == K2AMD_F32 && workspace != nullptr && !ForceGeneric() && MiFastSupports(B, S, T, modified)) {
     if (workspace_bytes < MiFastWorkspaceBytes(B, S, T)) return K2AMD_ERR_WORKSPACE;
     return MiForwardFast((const float *)px, (const float *)py, boundary, (float *)p, (float *)ans,
-                         B, S, T, modified, workspace, workspace_bytes, st);
+                         (float *)log_deriv, B, S, T, modified, workspace, workspace_bytes, st);
   }
   if (dtype == K2AMD_F32)
     return MiForwardGeneric<float>((const float *)px, (const float *)py, boundary, (float *)p,
@@ -85,6 +97,15 @@ int k2amd_mi_backward(const void *px, const void *py, const int64_t *boundary, c
                       void *ans_grad, void *px_grad, void *py_grad, int B, int S, int T,
                       int modified, int dtype, int overwrite_ans_grad, void *workspace,
                       size_t workspace_bytes, void *stream) {
+  return k2amd_mi_backward_kept(px, py, boundary, p, nullptr, ans_grad, px_grad, py_grad, B, S, T,
+                                modified, dtype, overwrite_ans_grad, workspace, workspace_bytes,
+                                stream);
+}
+
+int k2amd_mi_backward_kept(const void *px, const void *py, const int64_t *boundary, const void *p,
+                           const void *log_deriv, void *ans_grad, void *px_grad, void *py_grad,
+                           int B, int S, int T, int modified, int dtype, int overwrite_ans_grad,
+                           void *workspace, size_t workspace_bytes, void *stream) {
   (void)py;
   if (!ShapeOk(B, S, T) || (dtype != K2AMD_F32 && dtype != K2AMD_F64)) return K2AMD_ERR_INVALID_ARGUMENT;
   if (B == 0) return K2AMD_OK;
@@ -94,7 +115,8 @@ int k2amd_mi_backward(const void *px, const void *py, const int64_t *boundary, c
   modified = modified ? 1 : 0;
   if (dtype == K2AMD_F32 && workspace != nullptr && !ForceGeneric() && MiFastSupports(B, S, T, modified)) {
     if (workspace_bytes < MiFastWorkspaceBytes(B, S, T)) return K2AMD_ERR_WORKSPACE;
-    return MiBackwardFast((const float *)px, (const float *)p, boundary, (float *)ans_grad,
+    return MiBackwardFast((const float *)px, (const float *)p, (const float *)log_deriv, boundary,
+                          (float *)ans_grad,
                           (float *)px_grad, (float *)py_grad, B, S, T, modified,
                           overwrite_ans_grad, workspace, workspace_bytes, st);
   }

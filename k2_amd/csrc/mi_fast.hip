@@ -268,6 +268,9 @@ __device__ __forceinline__ void PublishEdge(float *addr, float v) {
 struct FwdLds {
   float4 fx[kWave + 1][kQuadsPerRow];  // row 64: see below
   float4 fy[kWave][kQuadsPerRow];
+  // p of each row at the last position of the three most recent blocks (written by the storers,
+  // only when the launch keeps the px-edge log-derivatives)
+  float last[3][kWave];
   unsigned ticket;
 };
 
@@ -285,11 +288,18 @@ __device__ __forceinline__ void WaitLoads(FwdRegs &r) {
 }
 constexpr int kFwdLoadsPerBlock = 2 * FwdLayout::kLoadItems;
 
+// kKeep: also write log_deriv[b][s][t] = (p[s-1][t+o] + px[s-1][t+o]) - p[s][t], the logarithm of
+// the px edge's share of cell (s, t) exactly as the backward sweep forms it
+// (k2/python/csrc/torch/mutual_information_cpu.cu:195-211), laid out like p.  The chain step has
+// both terms in registers; the storers rebuild them from the ring, so the backward kernel reads
+// one tensor instead of p twice and px once.  Cells of a sequence's first row and first column
+// hold values the backward never uses.
+template <bool kKeep>
 __global__ __launch_bounds__(FwdLayout::kThreads) void MiForwardFastKernel(
     const float *__restrict__ px, const float *__restrict__ py,
     const int64_t *__restrict__ boundary, float *__restrict__ p, float *__restrict__ ans,
-    FastHeader *hdr, float *edge, int B, int S, int Tn, int modified, int nchunks,
-    int edge_stride) {
+    float *__restrict__ log_deriv, FastHeader *hdr, float *edge, int B, int S, int Tn,
+    int modified, int nchunks, int edge_stride) {
   __shared__ FwdLds lds;
   const unsigned total_wgs = gridDim.x;
   if (threadIdx.x == 0) lds.ticket = atomicAdd(&hdr->ticket, 1u);
@@ -315,6 +325,7 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiForwardFastKernel(
   const float *pxb = px + (size_t)g.b * S * T1;
   const float *pyb = py + (size_t)g.b * (S + 1) * Tn;
   float *pb = p + (size_t)g.b * (S + 1) * (Tn + 1);
+  float *ldb = kKeep ? log_deriv + (size_t)g.b * (S + 1) * (Tn + 1) : nullptr;
   float *edge_out = edge + ((size_t)g.b * nchunks + g.c + 1) * edge_stride;  // read by chunk c+1
   float *edge_in = edge + ((size_t)g.b * nchunks + g.c) * edge_stride;
 
@@ -411,22 +422,57 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiForwardFastKernel(
       const int q = mq + 32 * it;
       const int row_i = g.row0 + q;
       if (row_i > g.ns) continue;
-      float4 v = lds.fy[q][(kb % 3) * kQuadsPerBlock + mm];
+      const int pq = (kb % 3) * kQuadsPerBlock + mm;
+      float4 v = lds.fy[q][pq];
       const float ninf = NegInfF();
       v.x = v.x < kLogZeroTest ? ninf : v.x;
       v.y = v.y < kLogZeroTest ? ninf : v.y;
       v.z = v.z < kLogZeroTest ? ninf : v.z;
       v.w = v.w < kLogZeroTest ? ninf : v.w;
       const int j = kb * kW + 4 * mm - q * g.skew;  // column of element 0
-      float *dst = pb + (size_t)(g.s0 + row_i) * (Tn + 1) + g.t0 + j;
+      const size_t at = (size_t)(g.s0 + row_i) * (Tn + 1) + g.t0 + j;
+      float *dst = pb + at;
+      float ld[4] = {0.f, 0.f, 0.f, 0.f};
+      if (kKeep) {
+        // What arrived along px at each step: for row 0 of the chunk the edge wavefront's sum
+        // (row 64 of fx, same position); otherwise p of the row above one position earlier plus
+        // this row's fx.  Stand-ins for -inf need no conversion here: anything that small gives
+        // exp() = 0 in the backward, as -inf does.
+        float t1[4];
+        if (q == 0) {
+          const float4 a = lds.fx[kWave][pq];
+          t1[0] = a.x; t1[1] = a.y; t1[2] = a.z; t1[3] = a.w;
+        } else {
+          const float4 x4 = lds.fx[q][pq];
+          float4 a = lds.fy[q - 1][pq];
+          asm volatile("" : "+v"(a.x), "+v"(a.y), "+v"(a.z), "+v"(a.w));  // one 16-byte read
+          float before;
+          if (mm > 0) {
+            float4 b4 = lds.fy[q - 1][pq - 1];
+            asm volatile("" : "+v"(b4.x), "+v"(b4.y), "+v"(b4.z), "+v"(b4.w));
+            before = b4.w;
+          } else {
+            before = kb > 0 ? lds.last[(kb + 2) % 3][q - 1] : kLogZero;
+          }
+          t1[0] = before + x4.x; t1[1] = a.x + x4.y; t1[2] = a.y + x4.z; t1[3] = a.z + x4.w;
+        }
+        const float own[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) ld[e] = t1[e] - (__builtin_isfinite(own[e]) ? own[e] : 0.0f);
+        if (mm == kQuadsPerBlock - 1) lds.last[kb % 3][q] = v.w;
+      }
       if (inner) {  // uniform: every column of the block lies in 0..nt-1 for every row
         StoreQuad(dst, v);
+        if (kKeep) StoreQuad(ldb + at, make_float4(ld[0], ld[1], ld[2], ld[3]));
       } else {
         asm volatile("");  // keeps this path a branch of its own
         const float vv[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          if (j + e >= 0 && j + e <= g.nt) dst[e] = vv[e];
+          if (j + e >= 0 && j + e <= g.nt) {
+            dst[e] = vv[e];
+            if (kKeep) ldb[at + e] = ld[e];
+          }
         if (row_i == g.ns) {
 #pragma unroll
           for (int e = 0; e < 4; ++e)
@@ -598,7 +644,12 @@ __device__ __forceinline__ void WaitLoads(BwdRegs &r) {
                : "+v"(r.d[0]), "+v"(r.s[0]), "+v"(r.x[0]), "+v"(r.d[1]), "+v"(r.s[1]), "+v"(r.x[1])
                : "n"(kYounger));
 }
-constexpr int kBwdLoadsPerBlock = 3 * BwdLayout::kLoadItems;
+// with kept log-derivatives only r.d is loaded
+template <int kYounger>
+__device__ __forceinline__ void WaitKeptLoads(BwdRegs &r) {
+  static_assert(BwdLayout::kLoadItems == 2, "operand list below");
+  asm volatile("s_waitcnt vmcnt(%2)" : "+v"(r.d[0]), "+v"(r.d[1]) : "n"(kYounger));
+}
 
 // Clears the four columns c..c+3 of array row r of px_grad / py_grad wherever they lie outside
 // the region the sweep assigns.
@@ -638,6 +689,9 @@ __device__ __forceinline__ void ZeroItem(const ZeroGeom &z, int r, int c) {
   }
 }
 
+// kKept: `p` is the log_deriv tensor a kKeep forward launch wrote (same layout as p), px is not
+// read, and every cell's d1 is exp() of one loaded value.
+template <bool kKept>
 __global__ __launch_bounds__(BwdLayout::kThreads) void MiBackwardFastKernel(
     const float *__restrict__ px, const float *__restrict__ p,
     const int64_t *__restrict__ boundary, float *__restrict__ ans_grad,
@@ -659,8 +713,6 @@ __global__ __launch_bounds__(BwdLayout::kThreads) void MiBackwardFastKernel(
   const Box box = LoadBox(boundary, g.b, S, Tn);
   const int T1 = modified ? Tn : Tn + 1;
   const int off = modified ? -1 : 0;
-  const float *pxb = px + (size_t)g.b * S * T1;
-  const float *pb = p + (size_t)g.b * (S + 1) * (Tn + 1);
   float *gxb = px_grad + (size_t)g.b * S * T1;
   float *gyb = py_grad + (size_t)g.b * (S + 1) * Tn;
 
@@ -736,24 +788,39 @@ __global__ __launch_bounds__(BwdLayout::kThreads) void MiBackwardFastKernel(
   }
   // One code path for every block: quads that reach outside the valid columns pick up
   // neighbouring floats (or zeros past the tensor's end) that the commit masks.
-  // Always issues kBwdLoadsPerBlock loads, so that the counts given to WaitLoads hold in every
+  // Always issues kLoadsPerBlock loads, so that the counts given to WaitLoads hold in every
   // iteration; for blocks in front of the first one it reads block 0 again, and rows past the
   // sequence's end read its last row (cache hits both).
+  constexpr int kLoadsPerBlock = (kKept ? 1 : 3) * kLoadItems;
   auto load_block = [&](int kb, BwdRegs &r) {
     kb = max(kb, 0);
 #pragma unroll
     for (int it = 0; it < kLoadItems; ++it) {
       const int jd = kb * kW + 4 * mm - (lq + kRowStep * it) * g.skew;  // destination column of element 0
       r.d[it] = AsyncQuad(rsp, idx_d[it] + jd);
-      r.s[it] = AsyncQuad(rsp, idx_s[it] + jd);
-      r.x[it] = AsyncQuad(rsx, idx_x[it] + jd);
+      if (!kKept) {
+        r.s[it] = AsyncQuad(rsp, idx_s[it] + jd);
+        r.x[it] = AsyncQuad(rsx, idx_x[it] + jd);
+      }
     }
+  };
+  auto wait_all = [&](BwdRegs &r) {
+    if (kKept) WaitKeptLoads<0>(r); else WaitLoads<0>(r);
+  };
+  // A block's loads stay in flight for kSets iterations.  With kept log-derivatives the
+  // loaders' work is light enough for the iteration to drop under half a trip to memory: two
+  // sets (as in the forward, whose iterations are twice as long) would make every iteration wait
+  // for its loads (measured: 42 us per launch with two sets, 31 us with three or more).  The
+  // plain kernel is bound by its movers' instruction issue and gains nothing from a third set.
+  constexpr int kSets = kKept ? 4 : 2;
+  auto wait_older = [&](BwdRegs &r) {  // the younger sets' loads may stay in flight
+    if (kKept) WaitKeptLoads<(kSets - 1) * kLoadsPerBlock>(r); else WaitLoads<(kSets - 1) * kLoadsPerBlock>(r);
   };
   // E / OME of a destination cell that has both edges inside the box; pd, ps, xs = p[dest],
   // p[src], px[src] (k2/python/csrc/torch/mutual_information_cpu.cu:195-211).
   auto flow = [&](float pd, float ps, float xs, float *e_out, float *o_out) {
     const float total = __builtin_isfinite(pd) ? pd : 0.0f;
-    const float d1 = __expf((ps + xs) - total);
+    const float d1 = __expf(kKept ? pd : (ps + xs) - total);
     const bool fin = __builtin_isfinite(d1);
     *e_out = fin ? d1 : 0.0f;
     *o_out = fin ? 1.0f - d1 : 0.0f;
@@ -781,13 +848,16 @@ __global__ __launch_bounds__(BwdLayout::kThreads) void MiBackwardFastKernel(
     for (int it = 0; it < kLoadItems; ++it) {
       if (!row_ok[it]) continue;
       const int q = lq + kRowStep * it;
-      float4 qd = AsFloat4(r.d[it]), qs = AsFloat4(r.s[it]), qx = AsFloat4(r.x[it]);
+      float4 qd = AsFloat4(r.d[it]);
+      float4 qs = kKept ? qd : AsFloat4(r.s[it]), qx = kKept ? qd : AsFloat4(r.x[it]);
       if (!inner && g.b == 0) {  // the only sequence whose rows can start the tensor
         asm volatile("");
         const int jd0 = kb * kW + 4 * mm - q * g.skew;
         qd = ShiftQuad(qd, idx_d[it] + jd0);
-        qs = ShiftQuad(qs, idx_s[it] + jd0);
-        qx = ShiftQuad(qx, idx_x[it] + jd0);
+        if (!kKept) {
+          qs = ShiftQuad(qs, idx_s[it] + jd0);
+          qx = ShiftQuad(qx, idx_x[it] + jd0);
+        }
       }
       float ve[4], vo[4];
       flow(qd.x, qs.x, qx.x, &ve[0], &vo[0]);
@@ -934,13 +1004,13 @@ __global__ __launch_bounds__(BwdLayout::kThreads) void MiBackwardFastKernel(
   // what the cells of the top block's last position saw: the initial gradient
   if (role == kChain)
     reinterpret_cast<float *>(&lds.g[lane][((top + 1) % 3) * kQuadsPerBlock])[0] = G;
-  BwdRegs ra, rb;
+  BwdRegs sets[kSets];
   if (role == kLoader) {
-    load_block(top, ra);
-    WaitLoads<0>(ra);
-    commit_block(top, ra);
-    load_block(top - 1, ra);
-    load_block(top - 2, rb);
+    load_block(top, sets[0]);
+    wait_all(sets[0]);
+    commit_block(top, sets[0]);
+#pragma unroll
+    for (int i = 0; i < kSets; ++i) load_block(top - 1 - i, sets[i]);
   } else if (role == kEdge) {
     take_block(top);
   }
@@ -955,22 +1025,20 @@ __global__ __launch_bounds__(BwdLayout::kThreads) void MiBackwardFastKernel(
       LdsBarrier();
     }
   } else if (role == kLoader) {
-    for (int kb = top; kb >= 0; kb -= 2) {
-      WaitLoads<kBwdLoadsPerBlock>(ra);  // the other set's loads may stay in flight
-      commit_block(kb - 1, ra);
-      load_block(kb - 3, ra);
-      LdsBarrier();
-      if (kb - 1 >= 0) {
-        WaitLoads<kBwdLoadsPerBlock>(rb);
-        commit_block(kb - 2, rb);
-        load_block(kb - 4, rb);
+    for (int kb = top; kb >= 0; kb -= kSets) {
+#pragma unroll
+      for (int i = 0; i < kSets; ++i) {
+        if (kb - i < 0) break;
+        wait_older(sets[i]);
+        commit_block(kb - i - 1, sets[i]);
+        load_block(kb - i - 1 - kSets, sets[i]);
         LdsBarrier();
       }
     }
     // the loads of the blocks in front of the first one are still in flight: they must land
     // before the compiler may give their registers to anything else
-    WaitLoads<0>(ra);
-    WaitLoads<0>(rb);
+#pragma unroll
+    for (int i = 0; i < kSets; ++i) wait_all(sets[i]);
   } else if (role == kStorer) {
     for (int kb = top; kb >= 0; --kb) {
       store_block(kb + 1);
@@ -1021,20 +1089,25 @@ int MiFastWorkspaceInit(void *workspace, size_t workspace_bytes, hipStream_t str
 }
 
 int MiForwardFast(const float *px, const float *py, const int64_t *boundary, float *p, float *ans,
-                  int B, int S, int Tn, int modified, void *workspace, size_t workspace_bytes,
-                  hipStream_t stream) {
+                  float *log_deriv, int B, int S, int Tn, int modified, void *workspace,
+                  size_t workspace_bytes, hipStream_t stream) {
   if (workspace == nullptr || workspace_bytes < MiFastWorkspaceBytes(B, S, Tn)) return K2AMD_ERR_WORKSPACE;
   const int nchunks = (S + 1 + kRows - 1) / kRows;
   const int edge_stride = (int)(((size_t)Tn + 2 + kRows + kW + 3) / 4 * 4 + kW);
   FastHeader *hdr = static_cast<FastHeader *>(workspace);
   float *edge = reinterpret_cast<float *>(hdr + 1);
-  hipLaunchKernelGGL(MiForwardFastKernel, dim3((unsigned)(B * nchunks)), dim3(FwdLayout::kThreads), kExclusiveLds - sizeof(FwdLds), stream,
-                     px, py, boundary, p, ans, hdr, edge, B, S, Tn, modified, nchunks, edge_stride);
+  const dim3 grid((unsigned)(B * nchunks)), block(FwdLayout::kThreads);
+  const size_t pad = kExclusiveLds - sizeof(FwdLds);
+  if (log_deriv != nullptr)
+    hipLaunchKernelGGL(MiForwardFastKernel<true>, grid, block, pad, stream, px, py, boundary, p, ans, log_deriv, hdr, edge, B, S, Tn, modified, nchunks, edge_stride);
+  else
+    hipLaunchKernelGGL(MiForwardFastKernel<false>, grid, block, pad, stream, px, py, boundary, p, ans, log_deriv, hdr, edge, B, S, Tn, modified, nchunks, edge_stride);
   return LaunchStatus();
 }
 
-int MiBackwardFast(const float *px, const float *p, const int64_t *boundary, float *ans_grad,
-                   float *px_grad, float *py_grad, int B, int S, int Tn, int modified,
+int MiBackwardFast(const float *px, const float *p, const float *log_deriv,
+                   const int64_t *boundary, float *ans_grad, float *px_grad, float *py_grad, int B,
+                   int S, int Tn, int modified,
                    int overwrite_ans_grad, void *workspace, size_t workspace_bytes,
                    hipStream_t stream) {
   if (workspace == nullptr || workspace_bytes < MiFastWorkspaceBytes(B, S, Tn)) return K2AMD_ERR_WORKSPACE;
@@ -1043,9 +1116,12 @@ int MiBackwardFast(const float *px, const float *p, const int64_t *boundary, flo
   FastHeader *hdr = static_cast<FastHeader *>(workspace);
   float *edge = reinterpret_cast<float *>(hdr + 1);
   // B * nchunks sweeping workgroups + as many that only clear
-  hipLaunchKernelGGL(MiBackwardFastKernel, dim3((unsigned)(2 * B * nchunks)), dim3(BwdLayout::kThreads), kExclusiveLds - sizeof(BwdLds), stream,
-                     px, p, boundary, ans_grad, px_grad, py_grad, hdr, edge, B, S, Tn, modified,
-                     nchunks, edge_stride, overwrite_ans_grad);
+  const dim3 grid((unsigned)(2 * B * nchunks)), block(BwdLayout::kThreads);
+  const size_t pad = kExclusiveLds - sizeof(BwdLds);
+  if (log_deriv != nullptr)
+    hipLaunchKernelGGL(MiBackwardFastKernel<true>, grid, block, pad, stream, px, log_deriv, boundary, ans_grad, px_grad, py_grad, hdr, edge, B, S, Tn, modified, nchunks, edge_stride, overwrite_ans_grad);
+  else
+    hipLaunchKernelGGL(MiBackwardFastKernel<false>, grid, block, pad, stream, px, p, boundary, ans_grad, px_grad, py_grad, hdr, edge, B, S, Tn, modified, nchunks, edge_stride, overwrite_ans_grad);
   return LaunchStatus();
 }
 

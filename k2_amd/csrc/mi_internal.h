@@ -22,13 +22,16 @@ size_t MiGenericMaxRows(int dtype);
 bool MiFastSupports(int B, int S, int Tn, int modified);
 size_t MiFastWorkspaceBytes(int B, int S, int Tn);
 int MiFastWorkspaceInit(void *workspace, size_t workspace_bytes, hipStream_t stream);
+// log_deriv (may be null): the forward also writes the logarithm of every cell's px-edge
+// derivative there, laid out like p, and the backward given the same tensor reads it instead of
+// p and px.
 int MiForwardFast(const float *px, const float *py, const int64_t *boundary, float *p, float *ans,
-                  int B, int S, int Tn, int modified, void *workspace, size_t workspace_bytes,
-                  hipStream_t stream);
-int MiBackwardFast(const float *px, const float *p, const int64_t *boundary, float *ans_grad,
-                   float *px_grad, float *py_grad, int B, int S, int Tn, int modified,
-                   int overwrite_ans_grad, void *workspace, size_t workspace_bytes,
-                   hipStream_t stream);
+                  float *log_deriv, int B, int S, int Tn, int modified, void *workspace,
+                  size_t workspace_bytes, hipStream_t stream);
+int MiBackwardFast(const float *px, const float *p, const float *log_deriv,
+                   const int64_t *boundary, float *ans_grad, float *px_grad, float *py_grad, int B,
+                   int S, int Tn, int modified, int overwrite_ans_grad, void *workspace,
+                   size_t workspace_bytes, hipStream_t stream);
 
 }  // namespace k2amd
 

@@ -93,9 +93,31 @@ Shape CheckInputs(const torch::Tensor &px, const torch::Tensor &py,
                px.size(2) == T ? 1 : 0};
 }
 
+// log_deriv: optional tensor shaped and typed like p that carries the px-edge log-derivatives
+// from the forward call to the backward call of the same inputs (k2amd_mi_forward_keep /
+// k2amd_mi_backward_kept in include/k2_amd.h).
+void *CheckLogDeriv(const torch::optional<torch::Tensor> &log_deriv, const torch::Tensor &p) {
+  if (!log_deriv.has_value() || !log_deriv->defined()) return nullptr;
+  TORCH_CHECK(log_deriv->sizes() == p.sizes() && log_deriv->scalar_type() == p.scalar_type() &&
+                  log_deriv->device() == p.device() && log_deriv->is_contiguous(),
+              "log_deriv must be a contiguous tensor with p's shape, dtype and device");
+  return log_deriv->data_ptr();
+}
+
+bool MutualInformationKeepsLogDeriv(torch::Tensor px, torch::Tensor py) {
+  TORCH_CHECK(px.dim() == 3 && py.dim() == 3, "px and py must have three dimensions");
+  const int B = static_cast<int>(px.size(0)), S = static_cast<int>(px.size(1)),
+            T = static_cast<int>(py.size(2)), modified = px.size(2) == T ? 1 : 0;
+  const int dt = DtypeCode(px);
+  return k2amd_mi_keeps_log_deriv(B, S, T, modified, dt,
+                                  k2amd_mi_workspace_bytes(B, S, T, modified, dt) > 0) != 0;
+}
+
 torch::Tensor MutualInformationForward(torch::Tensor px, torch::Tensor py,
-                                       torch::optional<torch::Tensor> boundary, torch::Tensor p) {
+                                       torch::optional<torch::Tensor> boundary, torch::Tensor p,
+                                       torch::optional<torch::Tensor> log_deriv) {
   const Shape sh = CheckInputs(px, py, boundary, p);
+  void *kept = CheckLogDeriv(log_deriv, p);
   c10::hip::HIPGuardMasqueradingAsCUDA guard(px.device());
   px = px.contiguous();
   py = py.contiguous();
@@ -108,19 +130,21 @@ torch::Tensor MutualInformationForward(torch::Tensor px, torch::Tensor py,
                                  px.device(), stream);
   {
     pybind11::gil_scoped_release release;
-    Check(k2amd_mi_forward(px.data_ptr(), py.data_ptr(),
-                           bd.defined() ? bd.data_ptr<int64_t>() : nullptr, p.data_ptr(),
-                           ans.data_ptr(), sh.B, sh.S, sh.T, sh.modified, dt,
-                           ws.defined() ? ws.data_ptr() : nullptr,
-                           ws.defined() ? static_cast<size_t>(ws.numel()) : 0, stream));
+    Check(k2amd_mi_forward_keep(px.data_ptr(), py.data_ptr(),
+                                bd.defined() ? bd.data_ptr<int64_t>() : nullptr, p.data_ptr(),
+                                ans.data_ptr(), kept, sh.B, sh.S, sh.T, sh.modified, dt,
+                                ws.defined() ? ws.data_ptr() : nullptr,
+                                ws.defined() ? static_cast<size_t>(ws.numel()) : 0, stream));
   }
   return ans;
 }
 
 std::vector<torch::Tensor> MutualInformationBackward(torch::Tensor px, torch::Tensor py,
                                                      torch::optional<torch::Tensor> boundary,
-                                                     torch::Tensor p, torch::Tensor ans_grad) {
+                                                     torch::Tensor p, torch::Tensor ans_grad,
+                                                     torch::optional<torch::Tensor> log_deriv) {
   const Shape sh = CheckInputs(px, py, boundary, p);
+  const void *kept = CheckLogDeriv(log_deriv, p);
   TORCH_CHECK(ans_grad.dim() == 1 && ans_grad.size(0) == sh.B, "ans_grad must have shape [B]");
   TORCH_CHECK(ans_grad.device() == px.device() && ans_grad.scalar_type() == px.scalar_type(),
               "ans_grad must match px in device and dtype");
@@ -141,12 +165,12 @@ std::vector<torch::Tensor> MutualInformationBackward(torch::Tensor px, torch::Te
     pybind11::gil_scoped_release release;
     // like the reference's device path, ans_grad is overwritten with the gradient that reached
     // the origin (k2/python/csrc/torch/mutual_information_cuda.cu:661-663)
-    Check(k2amd_mi_backward(px.data_ptr(), py.data_ptr(),
-                            bd.defined() ? bd.data_ptr<int64_t>() : nullptr, p.data_ptr(),
-                            ans_grad.data_ptr(), px_grad.data_ptr(), py_grad.data_ptr(), sh.B, sh.S,
-                            sh.T, sh.modified, dt, /*overwrite_ans_grad=*/1,
-                            ws.defined() ? ws.data_ptr() : nullptr,
-                            ws.defined() ? static_cast<size_t>(ws.numel()) : 0, stream));
+    Check(k2amd_mi_backward_kept(px.data_ptr(), py.data_ptr(),
+                                 bd.defined() ? bd.data_ptr<int64_t>() : nullptr, p.data_ptr(), kept,
+                                 ans_grad.data_ptr(), px_grad.data_ptr(), py_grad.data_ptr(), sh.B,
+                                 sh.S, sh.T, sh.modified, dt, /*overwrite_ans_grad=*/1,
+                                 ws.defined() ? ws.data_ptr() : nullptr,
+                                 ws.defined() ? static_cast<size_t>(ws.numel()) : 0, stream));
   }
   return {px_grad, py_grad};
 }
@@ -422,10 +446,13 @@ std::vector<torch::Tensor> PrunedRangesToLattice(torch::Tensor ranges, torch::Te
 PYBIND11_MODULE(_k2_amd, m) {
   m.doc() = "MI355X host layer of the k2 mutual-information recursion";
   m.def("mutual_information_forward", &MutualInformationForward, pybind11::arg("px"),
-        pybind11::arg("py"), pybind11::arg("boundary"), pybind11::arg("p"));
+        pybind11::arg("py"), pybind11::arg("boundary"), pybind11::arg("p"),
+        pybind11::arg("log_deriv") = pybind11::none());
+  m.def("mutual_information_keeps_log_deriv", &MutualInformationKeepsLogDeriv, pybind11::arg("px"),
+        pybind11::arg("py"));
   m.def("mutual_information_backward", &MutualInformationBackward, pybind11::arg("px"),
         pybind11::arg("py"), pybind11::arg("boundary"), pybind11::arg("p"),
-        pybind11::arg("ans_grad"));
+        pybind11::arg("ans_grad"), pybind11::arg("log_deriv") = pybind11::none());
   m.def("version", []() { return k2amd_version(); });
   m.def("logprobs_simple_forward", &LogprobsSimpleForward);
   m.def("logprobs_simple_backward", &LogprobsSimpleBackward);

@@ -33,6 +33,12 @@ def _check_boundary(boundary: Tensor, S: int, T: int) -> None:
     _checked_boundaries[ident] = (weakref.ref(boundary, lambda _, i=ident: _checked_boundaries.pop(i, None)), key)
 
 
+def _log_deriv_like(p: Tensor, px: Tensor, py: Tensor) -> Optional[Tensor]:
+    """The tensor that carries the px-edge log-derivatives from the forward kernel to the backward
+    kernel, or None where the kernels would not use it."""
+    return torch.empty_like(p) if native.mutual_information_keeps_log_deriv(px, py) else None
+
+
 class MutualInformationRecursionFunction(torch.autograd.Function):
     """Mirrors k2/python/k2/mutual_information.py:24-182: the forward runs the recursion and, when
     gradients may be wanted, the backward recursion with ans_grad = 1 straight away; autograd's
@@ -49,12 +55,16 @@ class MutualInformationRecursionFunction(torch.autograd.Function):
             assert boundary.shape == (B, 4), (boundary.shape, B)
 
         p = torch.empty(B, S + 1, T + 1, device=px.device, dtype=px.dtype)
-        ans = native.mutual_information_forward(px, py, boundary, p)
+        want_grad = return_grad or px.requires_grad or py.requires_grad
+        # the backward runs right away, so the forward can hand it the px-edge log-derivatives
+        log_deriv = _log_deriv_like(p, px, py) if want_grad else None
+        ans = native.mutual_information_forward(px, py, boundary, p, log_deriv)
 
         px_grad, py_grad = None, None
-        if return_grad or px.requires_grad or py.requires_grad:
+        if want_grad:
             ans_grad = torch.ones(B, device=px.device, dtype=px.dtype)
-            (px_grad, py_grad) = native.mutual_information_backward(px, py, boundary, p, ans_grad)
+            (px_grad, py_grad) = native.mutual_information_backward(px, py, boundary, p, ans_grad,
+                                                                    log_deriv)
             ctx.save_for_backward(px_grad, py_grad)
         assert len(pxy_grads) == 2, len(pxy_grads)
         pxy_grads[0] = px_grad
@@ -132,9 +142,11 @@ def joint_mutual_information_recursion(
     px_tot = px_cat.sum(dim=0).contiguous()
     py_tot = py_cat.sum(dim=0).contiguous()
     p = torch.empty(B, S + 1, T + 1, device=px_tot.device, dtype=px_tot.dtype)
-    tot_probs = native.mutual_information_forward(px_tot, py_tot, boundary, p)
+    log_deriv = _log_deriv_like(p, px_tot, py_tot)
+    tot_probs = native.mutual_information_forward(px_tot, py_tot, boundary, p, log_deriv)
     ans_grad = torch.ones(B, device=px_tot.device, dtype=px_tot.dtype)
-    (px_grad, py_grad) = native.mutual_information_backward(px_tot, py_tot, boundary, p, ans_grad)
+    (px_grad, py_grad) = native.mutual_information_backward(px_tot, py_tot, boundary, p, ans_grad,
+                                                            log_deriv)
     # -inf inputs carry zero occupation: clamp them to the most negative finite value so that
     # 0 * -inf does not produce NaN (k2/python/k2/mutual_information.py:410-411)
     lowest = torch.finfo(px_cat.dtype).min

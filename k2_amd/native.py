@@ -22,27 +22,43 @@ def _require_device(t: torch.Tensor):
             "k2_amd runs on MI355X only: got a tensor on %s (there is no CPU path)" % t.device)
 
 
-def mutual_information_forward(px: torch.Tensor, py: torch.Tensor,
-                               boundary: Optional[torch.Tensor], p: torch.Tensor) -> torch.Tensor:
-    """_k2.mutual_information_forward (k2/python/csrc/torch/mutual_information.cu:26-44)."""
+def mutual_information_keeps_log_deriv(px: torch.Tensor, py: torch.Tensor) -> bool:
+    """True if the forward / backward pair below uses a ``log_deriv`` tensor for these inputs (the
+    pipelined fp32 kernels do; the exact kernels leave it untouched, so allocating one is
+    wasted)."""
     _require_device(px)
     if _ext is not None:
-        return _ext.mutual_information_forward(px, py, boundary, p)
+        return _ext.mutual_information_keeps_log_deriv(px, py)
+    return capi.mi_keeps_log_deriv(px, py)
+
+
+def mutual_information_forward(px: torch.Tensor, py: torch.Tensor,
+                               boundary: Optional[torch.Tensor], p: torch.Tensor,
+                               log_deriv: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """_k2.mutual_information_forward (k2/python/csrc/torch/mutual_information.cu:26-44).
+    ``log_deriv`` (not in the reference; shaped like ``p``) is filled with what lets the backward
+    call on the same inputs read one tensor instead of three."""
+    _require_device(px)
+    if _ext is not None:
+        return _ext.mutual_information_forward(px, py, boundary, p, log_deriv)
     return capi.mi_forward(px.contiguous(), py.contiguous(),
-                           None if boundary is None else boundary.contiguous(), p)
+                           None if boundary is None else boundary.contiguous(), p,
+                           log_deriv=log_deriv)
 
 
 def mutual_information_backward(px: torch.Tensor, py: torch.Tensor,
                                 boundary: Optional[torch.Tensor], p: torch.Tensor,
-                                ans_grad: torch.Tensor) -> List[torch.Tensor]:
+                                ans_grad: torch.Tensor,
+                                log_deriv: Optional[torch.Tensor] = None) -> List[torch.Tensor]:
     """_k2.mutual_information_backward (k2/python/csrc/torch/mutual_information.cu:46-67);
-    overwrites ``ans_grad`` like the reference's device path."""
+    overwrites ``ans_grad`` like the reference's device path.  ``log_deriv``: the tensor the
+    forward call on the same inputs filled, or None."""
     _require_device(px)
     if _ext is not None:
-        return _ext.mutual_information_backward(px, py, boundary, p, ans_grad)
+        return _ext.mutual_information_backward(px, py, boundary, p, ans_grad, log_deriv)
     gx, gy = capi.mi_backward(px.contiguous(), py.contiguous(),
                               None if boundary is None else boundary.contiguous(), p, ans_grad,
-                              overwrite_ans_grad=True)
+                              overwrite_ans_grad=True, log_deriv=log_deriv)
     return [gx, gy]
 
 

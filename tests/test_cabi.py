@@ -34,6 +34,13 @@ def test_invalid_arguments_return_codes_without_a_gpu():
     assert lib.k2amd_mi_forward(None, None, None, None, None, -1, 1, 1, 0, 0, None, 0, None) == 1
     assert lib.k2amd_mi_forward(None, None, None, None, None, 1, 1, 1, 0, 7, None, 0, None) == 1
     assert lib.k2amd_mi_backward(None, None, None, None, None, None, None, 1, 1, 1, 0, 0, 0, None, 0, None) == 1
+    assert lib.k2amd_mi_forward_keep(None, None, None, None, None, None, -1, 1, 1, 0, 0, None, 0, None) == 1
+    assert lib.k2amd_mi_backward_kept(None, None, None, None, None, None, None, None, 1, 1, 1, 0, 9, 0, None, 0, None) == 1
+    # the log-derivative tensor is only used by the pipelined fp32 kernels, which need a workspace
+    assert lib.k2amd_mi_keeps_log_deriv(4, 10, 20, 0, 0, 1) == 1
+    assert lib.k2amd_mi_keeps_log_deriv(4, 10, 20, 0, 0, 0) == 0
+    assert lib.k2amd_mi_keeps_log_deriv(4, 10, 20, 0, 1, 1) == 0
+    assert lib.k2amd_mi_keeps_log_deriv(0, 10, 20, 0, 0, 1) == 0
     assert lib.k2amd_rnnt_prune_ranges(None, None, None, None, 1, 4, 4, 0, 9, 0, None) == 1
     assert lib.k2amd_rnnt_logprobs_joint_forward(None, None, None, None, None, None, 1, 1, 1, 4, 9, 0, 0, None) == 1
     # an empty batch is a no-op

@@ -34,6 +34,19 @@ def run_gpu(px, py, bd, device, ans_grad=None):
     # call must leave exactly as it found it, and no in-kernel wait may have timed out
     assert capi.mi_workspace_is_clean(device), "workspace left dirty"
     capi.mi_workspace_status(device)
+    if capi.mi_keeps_log_deriv(tpx, tpy):
+        # the same pair with the log-derivative tensor between them: identical bits
+        p2 = torch.full_like(p, float("nan"))
+        log_deriv = torch.full_like(p, float("nan"))
+        ans2 = capi.mi_forward(tpx, tpy, tbd, p2, log_deriv=log_deriv)
+        g2 = g_in.clone()
+        gx2, gy2 = capi.mi_backward(tpx, tpy, tbd, p2, g2, overwrite_ans_grad=True, log_deriv=log_deriv)
+        torch.cuda.synchronize()
+        assert capi.mi_workspace_is_clean(device), "workspace left dirty (kept pair)"
+        capi.mi_workspace_status(device)
+        for name, x, y in (("ans", ans2, ans), ("p", p2, p), ("px_grad", gx2, gx), ("py_grad", gy2, gy),
+                           ("ans_grad", g2, g)):
+            assert torch.equal(x.view(torch.int32), y.view(torch.int32)), "kept pair differs in " + name
     return ans.cpu().numpy(), p.cpu().numpy(), gx.cpu().numpy(), gy.cpu().numpy(), g.cpu().numpy(), g_in.cpu().numpy()
 
 
@@ -195,7 +208,18 @@ def test_pybind_host_matches_ctypes_host(device):
         ans2 = _k2_amd.mutual_information_forward(px=px_strided, py=py, boundary=bd, p=p2)
         g2 = torch.full((B,), 2.0, device=device)
         gx2, gy2 = _k2_amd.mutual_information_backward(px=px, py=py, boundary=bd, p=p2, ans_grad=g2)
+        # the same through the pair that passes the log-derivatives along
+        assert _k2_amd.mutual_information_keeps_log_deriv(px=px, py=py)
+        p3 = torch.empty_like(p1)
+        kept = torch.full_like(p1, float("nan"))
+        ans3 = _k2_amd.mutual_information_forward(px=px_strided, py=py, boundary=bd, p=p3, log_deriv=kept)
+        g3 = torch.full((B,), 2.0, device=device)
+        gx3, gy3 = _k2_amd.mutual_information_backward(px=px, py=py, boundary=bd, p=p3, ans_grad=g3,
+                                                       log_deriv=kept)
     side.synchronize()
+    assert torch.equal(ans3, ans2) and torch.equal(gx3, gx2) and torch.equal(gy3, gy2) and torch.equal(g3, g2)
+    with pytest.raises(RuntimeError):  # wrong shape
+        _k2_amd.mutual_information_forward(px=px, py=py, boundary=bd, p=p3, log_deriv=kept[:, :-1])
     g1 = torch.full((B,), 2.0, device=device)
     gx1, gy1 = capi.mi_backward(px, py, bd, p1, g1, overwrite_ans_grad=True)
     torch.cuda.synchronize()
@@ -241,3 +265,27 @@ def test_joint_recursion_identities(device, dtype):
         wx, wy = omi.mi_backward(npx, npy, bd.cpu().numpy(), p)
         np.testing.assert_allclose(grads[0][0].cpu().numpy(), 3 * wx, rtol=1e-4, atol=1e-5)
         np.testing.assert_allclose(grads[0][1].cpu().numpy(), 3 * wy, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.gpu
+def test_log_deriv_is_left_alone_by_the_exact_kernels(device):
+    """fp64 (and fp32 without a workspace) run the one-workgroup-per-sequence kernels, which
+    neither write nor read the log-derivative tensor: the hosts say so and results are unchanged."""
+    from k2_amd import capi
+    rng = np.random.default_rng(3)
+    B, S, T = 2, 12, 30
+    px = torch.from_numpy(rng.standard_normal((B, S, T + 1))).to(device)
+    py = torch.from_numpy(rng.standard_normal((B, S + 1, T))).to(device)
+    assert not capi.mi_keeps_log_deriv(px, py)
+    p1 = torch.empty(B, S + 1, T + 1, dtype=torch.float64, device=device)
+    p2 = torch.empty_like(p1)
+    kept = torch.full_like(p1, 7.0)
+    a1 = capi.mi_forward(px, py, None, p1)
+    a2 = capi.mi_forward(px, py, None, p2, log_deriv=kept)
+    g1 = torch.ones(B, dtype=torch.float64, device=device)
+    g2 = torch.ones(B, dtype=torch.float64, device=device)
+    x1, y1 = capi.mi_backward(px, py, None, p1, g1)
+    x2, y2 = capi.mi_backward(px, py, None, p2, g2, log_deriv=kept)
+    torch.cuda.synchronize()
+    assert torch.equal(a1, a2) and torch.equal(x1, x2) and torch.equal(y1, y2)
+    assert bool((kept == 7.0).all())
