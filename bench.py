@@ -31,7 +31,8 @@ BWD_BYTES_PER_CELL = 16
 # HBM bytes per launch on the default workload, from rocprofv3's FETCH_SIZE / WRITE_SIZE counters
 # scaled by a 256 MiB device copy (profiles/mi_fast_kernels_c4_hbm_traffic.md).  Reported only
 # for the default shape; any other --B/--S/--T prints null.
-MEASURED_TRAFFIC_BYTES = {"mi_forward": 50049796, "mi_backward": 86230408}
+MEASURED_TRAFFIC_BYTES = {"mi_forward": 65951892, "mi_backward": 69314898}
+MEASURED_TRAFFIC_BYTES_PLAIN_PAIR = {"mi_forward": 50049796, "mi_backward": 86230408}  # --no-keep
 
 
 def cpu_baseline(c, budget_s=12.0):
@@ -327,7 +328,8 @@ def main():
                    "active_cells": active, "full_box_cells": full, "log_deriv_kept": bool(keep)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": MEASURED_TRAFFIC_BYTES[dom] if (B, S, T) == (32, 200, 1000) else None,
+                     "traffic": (MEASURED_TRAFFIC_BYTES if keep else MEASURED_TRAFFIC_BYTES_PLAIN_PAIR)[dom]
+                     if (B, S, T) == (32, 200, 1000) else None,
                      "kernel": dom,
                      "kernel_avg_us": dom_ms * 1e3},
         "kernels": {"mi_forward_avg_us": fwd_avg * 1e3, "mi_forward_min_us": float(fwd_ms.min()) * 1e3,
