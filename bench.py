@@ -31,7 +31,7 @@ BWD_BYTES_PER_CELL = 16
 # HBM bytes per launch on the default workload, from rocprofv3's FETCH_SIZE / WRITE_SIZE counters
 # scaled by a 256 MiB device copy (profiles/mi_fast_kernels_c4_hbm_traffic.md).  Reported only
 # for the default shape; any other --B/--S/--T prints null.
-MEASURED_TRAFFIC_BYTES = {"mi_forward": 65951892, "mi_backward": 69314898}
+MEASURED_TRAFFIC_BYTES = {"mi_forward": 50124982, "mi_backward": 69268852}
 MEASURED_TRAFFIC_BYTES_PLAIN_PAIR = {"mi_forward": 50049796, "mi_backward": 86230408}  # --no-keep
 
 
@@ -268,12 +268,13 @@ def main():
     bnp = c["boundary"]
     active = int(((bnp[:, 2] - bnp[:, 0] + 1) * (bnp[:, 3] - bnp[:, 1] + 1)).sum())
     full = B * (S + 1) * (T + 1)
-    p = torch.empty(B, S + 1, T + 1, dtype=torch.float32, device=dev)
     ones = torch.ones(B, dtype=torch.float32, device=dev)
     # as mutual_information_recursion does: the forward hands the backward the px-edge
     # log-derivatives (one more [B][S+1][T+1] tensor written by the forward, read by the backward)
+    # (the forward then writes that tensor in place of p)
     keep = not args.no_keep and capi.mi_keeps_log_deriv(px, py)
-    log_deriv = torch.empty_like(p) if keep else None
+    lattice = torch.empty(B, S + 1, T + 1, dtype=torch.float32, device=dev)
+    p, log_deriv = (None, lattice) if keep else (lattice, None)
 
     def step(ev=None):
         if ev is not None:

@@ -88,7 +88,10 @@ K2AMD_API int k2amd_mi_backward(const void *px, const void *py, const int64_t *b
  *   (s,t) exactly as the backward sweep forms it (mutual_information_cpu.cu:195-211), so the
  *   backward reads one tensor where it otherwise reads p twice and px once; the gradients are the
  *   same bits either way.  Elements of a sequence's first row and first column are undefined.
- * log_deriv == NULL makes each call identical to the plain entry point.  Only the pipelined fp32
+ * log_deriv == NULL makes each call identical to the plain entry point.  Where the pair uses the
+ * tensor, p may be NULL in both calls: the forward then does not store p at all (ans and the
+ * gradients are all that such a caller gets, which is all the reference's autograd function
+ * keeps, k2/python/k2/mutual_information.py:157-169).  Only the pipelined fp32
  * kernels use the tensor: k2amd_mi_keeps_log_deriv(...) tells whether the pair will (1) or will
  * leave it untouched (0) for a shape, so that a host can skip the allocation.  Give the backward
  * the tensor only if the forward call with the same shape, dtype and workspace wrote it.        */

@@ -150,7 +150,8 @@ def mi_keeps_log_deriv(px, py):
 
 def mi_forward(px, py, boundary, p, log_deriv=None):
     """C-ABI twin of _k2.mutual_information_forward: fills ``p``, returns ans [B].  ``log_deriv``
-    (optional, shaped like ``p``) receives what lets mi_backward skip its reads of p and px."""
+    (optional, shaped like ``p``) receives what lets mi_backward skip its reads of p and px; where
+    mi_keeps_log_deriv(px, py) holds, ``p`` may then be None and is not computed."""
     B, S, T1 = px.shape
     T = py.shape[2]
     modified = int(T1 == T)

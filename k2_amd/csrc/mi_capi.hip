@@ -76,12 +76,15 @@ int k2amd_mi_forward_keep(const void *px, const void *py, const int64_t *boundar
                           void *workspace, size_t workspace_bytes, void *stream) {
   if (!ShapeOk(B, S, T) || (dtype != K2AMD_F32 && dtype != K2AMD_F64)) return K2AMD_ERR_INVALID_ARGUMENT;
   if (B == 0) return K2AMD_OK;
-  if (!p || !ans || (!px && S > 0) || (!py && T > 0)) return K2AMD_ERR_INVALID_ARGUMENT;
+  if (!ans || (!px && S > 0) || (!py && T > 0)) return K2AMD_ERR_INVALID_ARGUMENT;
   hipStream_t st = static_cast<hipStream_t>(stream);
   modified = modified ? 1 : 0;
+  const bool fast = dtype == K2AMD_F32 && workspace != nullptr && !ForceGeneric() && MiFastSupports(B, S, T, modified);
+  // p may be left out only where the log-derivative tensor stands in for it
+  if (!p && !(fast && log_deriv)) return K2AMD_ERR_INVALID_ARGUMENT;
   // fp32 with a workspace takes the pipelined throughput path; without one (or for fp64) the
   // exact one-workgroup-per-sequence kernels run.
-  if (dtype == K2AMD_F32 && workspace != nullptr && !ForceGeneric() && MiFastSupports(B, S, T, modified)) {
+  if (fast) {
     if (workspace_bytes < MiFastWorkspaceBytes(B, S, T)) return K2AMD_ERR_WORKSPACE;
     return MiForwardFast((const float *)px, (const float *)py, boundary, (float *)p, (float *)ans,
                          (float *)log_deriv, B, S, T, modified, workspace, workspace_bytes, st);
@@ -109,11 +112,13 @@ int k2amd_mi_backward_kept(const void *px, const void *py, const int64_t *bounda
   (void)py;
   if (!ShapeOk(B, S, T) || (dtype != K2AMD_F32 && dtype != K2AMD_F64)) return K2AMD_ERR_INVALID_ARGUMENT;
   if (B == 0) return K2AMD_OK;
-  if (!p || !ans_grad || (!px && S > 0) || (!px_grad && S > 0) || (!py_grad && T > 0))
+  if (!ans_grad || (!px && S > 0) || (!px_grad && S > 0) || (!py_grad && T > 0))
     return K2AMD_ERR_INVALID_ARGUMENT;
   hipStream_t st = static_cast<hipStream_t>(stream);
   modified = modified ? 1 : 0;
-  if (dtype == K2AMD_F32 && workspace != nullptr && !ForceGeneric() && MiFastSupports(B, S, T, modified)) {
+  const bool fast = dtype == K2AMD_F32 && workspace != nullptr && !ForceGeneric() && MiFastSupports(B, S, T, modified);
+  if (!p && !(fast && log_deriv)) return K2AMD_ERR_INVALID_ARGUMENT;
+  if (fast) {
     if (workspace_bytes < MiFastWorkspaceBytes(B, S, T)) return K2AMD_ERR_WORKSPACE;
     return MiBackwardFast((const float *)px, (const float *)p, (const float *)log_deriv, boundary,
                           (float *)ans_grad,

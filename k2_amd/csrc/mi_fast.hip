@@ -293,8 +293,9 @@ constexpr int kFwdLoadsPerBlock = 2 * FwdLayout::kLoadItems;
 // (k2/python/csrc/torch/mutual_information_cpu.cu:195-211), laid out like p.  The chain step has
 // both terms in registers; the storers rebuild them from the ring, so the backward kernel reads
 // one tensor instead of p twice and px once.  Cells of a sequence's first row and first column
-// hold values the backward never uses.
-template <bool kKeep>
+// hold values the backward never uses.  kWriteP = false (only with kKeep): p itself is not stored,
+// for callers that want nothing but ans and the gradients.
+template <bool kKeep, bool kWriteP>
 __global__ __launch_bounds__(FwdLayout::kThreads) void MiForwardFastKernel(
     const float *__restrict__ px, const float *__restrict__ py,
     const int64_t *__restrict__ boundary, float *__restrict__ p, float *__restrict__ ans,
@@ -324,7 +325,7 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiForwardFastKernel(
   const int T1 = modified ? Tn : Tn + 1;
   const float *pxb = px + (size_t)g.b * S * T1;
   const float *pyb = py + (size_t)g.b * (S + 1) * Tn;
-  float *pb = p + (size_t)g.b * (S + 1) * (Tn + 1);
+  float *pb = kWriteP ? p + (size_t)g.b * (S + 1) * (Tn + 1) : nullptr;
   float *ldb = kKeep ? log_deriv + (size_t)g.b * (S + 1) * (Tn + 1) : nullptr;
   float *edge_out = edge + ((size_t)g.b * nchunks + g.c + 1) * edge_stride;  // read by chunk c+1
   float *edge_in = edge + ((size_t)g.b * nchunks + g.c) * edge_stride;
@@ -462,7 +463,7 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiForwardFastKernel(
         if (mm == kQuadsPerBlock - 1) lds.last[kb % 3][q] = v.w;
       }
       if (inner) {  // uniform: every column of the block lies in 0..nt-1 for every row
-        StoreQuad(dst, v);
+        if (kWriteP) StoreQuad(dst, v);
         if (kKeep) StoreQuad(ldb + at, make_float4(ld[0], ld[1], ld[2], ld[3]));
       } else {
         asm volatile("");  // keeps this path a branch of its own
@@ -470,7 +471,7 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiForwardFastKernel(
 #pragma unroll
         for (int e = 0; e < 4; ++e)
           if (j + e >= 0 && j + e <= g.nt) {
-            dst[e] = vv[e];
+            if (kWriteP) dst[e] = vv[e];
             if (kKeep) ldb[at + e] = ld[e];
           }
         if (row_i == g.ns) {
@@ -1098,10 +1099,13 @@ int MiForwardFast(const float *px, const float *py, const int64_t *boundary, flo
   float *edge = reinterpret_cast<float *>(hdr + 1);
   const dim3 grid((unsigned)(B * nchunks)), block(FwdLayout::kThreads);
   const size_t pad = kExclusiveLds - sizeof(FwdLds);
-  if (log_deriv != nullptr)
-    hipLaunchKernelGGL(MiForwardFastKernel<true>, grid, block, pad, stream, px, py, boundary, p, ans, log_deriv, hdr, edge, B, S, Tn, modified, nchunks, edge_stride);
+  if (log_deriv == nullptr && p == nullptr) return K2AMD_ERR_INVALID_ARGUMENT;
+  if (log_deriv != nullptr && p != nullptr)
+    hipLaunchKernelGGL((MiForwardFastKernel<true, true>), grid, block, pad, stream, px, py, boundary, p, ans, log_deriv, hdr, edge, B, S, Tn, modified, nchunks, edge_stride);
+  else if (log_deriv != nullptr)
+    hipLaunchKernelGGL((MiForwardFastKernel<true, false>), grid, block, pad, stream, px, py, boundary, p, ans, log_deriv, hdr, edge, B, S, Tn, modified, nchunks, edge_stride);
   else
-    hipLaunchKernelGGL(MiForwardFastKernel<false>, grid, block, pad, stream, px, py, boundary, p, ans, log_deriv, hdr, edge, B, S, Tn, modified, nchunks, edge_stride);
+    hipLaunchKernelGGL((MiForwardFastKernel<false, true>), grid, block, pad, stream, px, py, boundary, p, ans, log_deriv, hdr, edge, B, S, Tn, modified, nchunks, edge_stride);
   return LaunchStatus();
 }
 

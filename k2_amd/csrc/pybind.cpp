@@ -66,8 +66,10 @@ struct Shape {
 };
 
 // The checks of k2/python/csrc/torch/mutual_information_cpu.cu:53-77, as RuntimeError.
+// `p` (or, where p is left out, the log-derivative tensor that stands in for it) is `lattice`.
 Shape CheckInputs(const torch::Tensor &px, const torch::Tensor &py,
-                  const torch::optional<torch::Tensor> &boundary, const torch::Tensor &p) {
+                  const torch::optional<torch::Tensor> &boundary, const torch::Tensor &lattice) {
+  const torch::Tensor &p = lattice;
   TORCH_CHECK(px.dim() == 3, "px must be 3-dimensional");
   TORCH_CHECK(py.dim() == 3, "py must be 3-dimensional");
   TORCH_CHECK(p.dim() == 3, "p must be 3-dimensional");
@@ -96,10 +98,19 @@ Shape CheckInputs(const torch::Tensor &px, const torch::Tensor &py,
 // log_deriv: optional tensor shaped and typed like p that carries the px-edge log-derivatives
 // from the forward call to the backward call of the same inputs (k2amd_mi_forward_keep /
 // k2amd_mi_backward_kept in include/k2_amd.h).
-void *CheckLogDeriv(const torch::optional<torch::Tensor> &log_deriv, const torch::Tensor &p) {
-  if (!log_deriv.has_value() || !log_deriv->defined()) return nullptr;
-  TORCH_CHECK(log_deriv->sizes() == p.sizes() && log_deriv->scalar_type() == p.scalar_type() &&
-                  log_deriv->device() == p.device() && log_deriv->is_contiguous(),
+// p may be None where log_deriv stands in for it (see the header); the one that is given first
+// goes through CheckInputs, the other is compared with it.
+bool Given(const torch::optional<torch::Tensor> &t) { return t.has_value() && t->defined(); }
+const torch::Tensor &LatticeOf(const torch::optional<torch::Tensor> &p,
+                               const torch::optional<torch::Tensor> &log_deriv) {
+  TORCH_CHECK(Given(p) || Given(log_deriv), "p may only be None where log_deriv is given");
+  return Given(p) ? *p : *log_deriv;
+}
+void *CheckLogDeriv(const torch::optional<torch::Tensor> &log_deriv, const torch::Tensor &lattice) {
+  if (!Given(log_deriv)) return nullptr;
+  TORCH_CHECK(log_deriv->sizes() == lattice.sizes() &&
+                  log_deriv->scalar_type() == lattice.scalar_type() &&
+                  log_deriv->device() == lattice.device() && log_deriv->is_contiguous(),
               "log_deriv must be a contiguous tensor with p's shape, dtype and device");
   return log_deriv->data_ptr();
 }
@@ -114,10 +125,13 @@ bool MutualInformationKeepsLogDeriv(torch::Tensor px, torch::Tensor py) {
 }
 
 torch::Tensor MutualInformationForward(torch::Tensor px, torch::Tensor py,
-                                       torch::optional<torch::Tensor> boundary, torch::Tensor p,
+                                       torch::optional<torch::Tensor> boundary,
+                                       torch::optional<torch::Tensor> p,
                                        torch::optional<torch::Tensor> log_deriv) {
-  const Shape sh = CheckInputs(px, py, boundary, p);
-  void *kept = CheckLogDeriv(log_deriv, p);
+  const torch::Tensor &lattice = LatticeOf(p, log_deriv);
+  const Shape sh = CheckInputs(px, py, boundary, lattice);
+  void *kept = CheckLogDeriv(log_deriv, lattice);
+  void *p_ptr = Given(p) ? p->data_ptr() : nullptr;
   c10::hip::HIPGuardMasqueradingAsCUDA guard(px.device());
   px = px.contiguous();
   py = py.contiguous();
@@ -131,7 +145,7 @@ torch::Tensor MutualInformationForward(torch::Tensor px, torch::Tensor py,
   {
     pybind11::gil_scoped_release release;
     Check(k2amd_mi_forward_keep(px.data_ptr(), py.data_ptr(),
-                                bd.defined() ? bd.data_ptr<int64_t>() : nullptr, p.data_ptr(),
+                                bd.defined() ? bd.data_ptr<int64_t>() : nullptr, p_ptr,
                                 ans.data_ptr(), kept, sh.B, sh.S, sh.T, sh.modified, dt,
                                 ws.defined() ? ws.data_ptr() : nullptr,
                                 ws.defined() ? static_cast<size_t>(ws.numel()) : 0, stream));
@@ -141,10 +155,13 @@ torch::Tensor MutualInformationForward(torch::Tensor px, torch::Tensor py,
 
 std::vector<torch::Tensor> MutualInformationBackward(torch::Tensor px, torch::Tensor py,
                                                      torch::optional<torch::Tensor> boundary,
-                                                     torch::Tensor p, torch::Tensor ans_grad,
+                                                     torch::optional<torch::Tensor> p,
+                                                     torch::Tensor ans_grad,
                                                      torch::optional<torch::Tensor> log_deriv) {
-  const Shape sh = CheckInputs(px, py, boundary, p);
-  const void *kept = CheckLogDeriv(log_deriv, p);
+  const torch::Tensor &lattice = LatticeOf(p, log_deriv);
+  const Shape sh = CheckInputs(px, py, boundary, lattice);
+  const void *kept = CheckLogDeriv(log_deriv, lattice);
+  const void *p_ptr = Given(p) ? p->data_ptr() : nullptr;
   TORCH_CHECK(ans_grad.dim() == 1 && ans_grad.size(0) == sh.B, "ans_grad must have shape [B]");
   TORCH_CHECK(ans_grad.device() == px.device() && ans_grad.scalar_type() == px.scalar_type(),
               "ans_grad must match px in device and dtype");
@@ -166,7 +183,7 @@ std::vector<torch::Tensor> MutualInformationBackward(torch::Tensor px, torch::Te
     // like the reference's device path, ans_grad is overwritten with the gradient that reached
     // the origin (k2/python/csrc/torch/mutual_information_cuda.cu:661-663)
     Check(k2amd_mi_backward_kept(px.data_ptr(), py.data_ptr(),
-                                 bd.defined() ? bd.data_ptr<int64_t>() : nullptr, p.data_ptr(), kept,
+                                 bd.defined() ? bd.data_ptr<int64_t>() : nullptr, p_ptr, kept,
                                  ans_grad.data_ptr(), px_grad.data_ptr(), py_grad.data_ptr(), sh.B,
                                  sh.S, sh.T, sh.modified, dt, /*overwrite_ans_grad=*/1,
                                  ws.defined() ? ws.data_ptr() : nullptr,

@@ -33,10 +33,15 @@ def _check_boundary(boundary: Tensor, S: int, T: int) -> None:
     _checked_boundaries[ident] = (weakref.ref(boundary, lambda _, i=ident: _checked_boundaries.pop(i, None)), key)
 
 
-def _log_deriv_like(p: Tensor, px: Tensor, py: Tensor) -> Optional[Tensor]:
-    """The tensor that carries the px-edge log-derivatives from the forward kernel to the backward
-    kernel, or None where the kernels would not use it."""
-    return torch.empty_like(p) if native.mutual_information_keeps_log_deriv(px, py) else None
+def _lattice_buffers(px: Tensor, py: Tensor, want_grad: bool) -> Tuple[Optional[Tensor], Optional[Tensor]]:
+    """(p, log_deriv) for a forward call that a backward call may follow: the [B][S+1][T+1]
+    buffer the reference allocates as ``p`` (k2/python/k2/mutual_information.py:157) is handed over
+    as ``log_deriv`` instead where the kernels pass the px-edge log-derivatives along."""
+    (B, S, _), T = px.shape, py.shape[-1]
+    buf = torch.empty(B, S + 1, T + 1, device=px.device, dtype=px.dtype)
+    if want_grad and native.mutual_information_keeps_log_deriv(px, py):
+        return None, buf
+    return buf, None
 
 
 class MutualInformationRecursionFunction(torch.autograd.Function):
@@ -54,10 +59,10 @@ class MutualInformationRecursionFunction(torch.autograd.Function):
         if boundary is not None:
             assert boundary.shape == (B, 4), (boundary.shape, B)
 
-        p = torch.empty(B, S + 1, T + 1, device=px.device, dtype=px.dtype)
         want_grad = return_grad or px.requires_grad or py.requires_grad
         # the backward runs right away, so the forward can hand it the px-edge log-derivatives
-        log_deriv = _log_deriv_like(p, px, py) if want_grad else None
+        # instead of p (which nothing else reads)
+        p, log_deriv = _lattice_buffers(px, py, want_grad)
         ans = native.mutual_information_forward(px, py, boundary, p, log_deriv)
 
         px_grad, py_grad = None, None
@@ -141,8 +146,7 @@ def joint_mutual_information_recursion(
     py_cat = torch.stack(list(py), dim=0)  # [N][B][S+1][T]
     px_tot = px_cat.sum(dim=0).contiguous()
     py_tot = py_cat.sum(dim=0).contiguous()
-    p = torch.empty(B, S + 1, T + 1, device=px_tot.device, dtype=px_tot.dtype)
-    log_deriv = _log_deriv_like(p, px_tot, py_tot)
+    p, log_deriv = _lattice_buffers(px_tot, py_tot, True)
     tot_probs = native.mutual_information_forward(px_tot, py_tot, boundary, p, log_deriv)
     ans_grad = torch.ones(B, device=px_tot.device, dtype=px_tot.dtype)
     (px_grad, py_grad) = native.mutual_information_backward(px_tot, py_tot, boundary, p, ans_grad,

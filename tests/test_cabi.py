@@ -5,6 +5,8 @@ import inspect
 import os
 import re
 
+import ctypes
+
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -36,6 +38,11 @@ def test_invalid_arguments_return_codes_without_a_gpu():
     assert lib.k2amd_mi_backward(None, None, None, None, None, None, None, 1, 1, 1, 0, 0, 0, None, 0, None) == 1
     assert lib.k2amd_mi_forward_keep(None, None, None, None, None, None, -1, 1, 1, 0, 0, None, 0, None) == 1
     assert lib.k2amd_mi_backward_kept(None, None, None, None, None, None, None, None, 1, 1, 1, 0, 9, 0, None, 0, None) == 1
+    # p may only be left out where the log-derivative tensor stands in for it (fp32 with a workspace)
+    one = ctypes.c_void_p(1)  # never dereferenced: the calls below are rejected on their arguments
+    assert lib.k2amd_mi_forward_keep(one, one, None, None, one, None, 1, 1, 1, 0, 0, one, 1 << 20, None) == 1
+    assert lib.k2amd_mi_forward_keep(one, one, None, None, one, one, 1, 1, 1, 0, 1, one, 1 << 20, None) == 1
+    assert lib.k2amd_mi_forward_keep(one, one, None, None, one, one, 1, 1, 1, 0, 0, None, 0, None) == 1
     # the log-derivative tensor is only used by the pipelined fp32 kernels, which need a workspace
     assert lib.k2amd_mi_keeps_log_deriv(4, 10, 20, 0, 0, 1) == 1
     assert lib.k2amd_mi_keeps_log_deriv(4, 10, 20, 0, 0, 0) == 0

@@ -47,6 +47,15 @@ def run_gpu(px, py, bd, device, ans_grad=None):
         for name, x, y in (("ans", ans2, ans), ("p", p2, p), ("px_grad", gx2, gx), ("py_grad", gy2, gy),
                            ("ans_grad", g2, g)):
             assert torch.equal(x.view(torch.int32), y.view(torch.int32)), "kept pair differs in " + name
+        # and without p at all, as mutual_information_recursion calls it
+        log_deriv.fill_(float("nan"))
+        ans3 = capi.mi_forward(tpx, tpy, tbd, None, log_deriv=log_deriv)
+        g3 = g_in.clone()
+        gx3, gy3 = capi.mi_backward(tpx, tpy, tbd, None, g3, overwrite_ans_grad=True, log_deriv=log_deriv)
+        torch.cuda.synchronize()
+        assert capi.mi_workspace_is_clean(device), "workspace left dirty (kept pair without p)"
+        for name, x, y in (("ans", ans3, ans), ("px_grad", gx3, gx), ("py_grad", gy3, gy), ("ans_grad", g3, g)):
+            assert torch.equal(x.view(torch.int32), y.view(torch.int32)), "kept pair without p differs in " + name
     return ans.cpu().numpy(), p.cpu().numpy(), gx.cpu().numpy(), gy.cpu().numpy(), g.cpu().numpy(), g_in.cpu().numpy()
 
 
