@@ -31,7 +31,7 @@ BWD_BYTES_PER_CELL = 16
 # HBM bytes per launch on the default workload, from rocprofv3's FETCH_SIZE / WRITE_SIZE counters
 # scaled by a 256 MiB device copy (profiles/mi_fast_kernels_c4_hbm_traffic.md).  Reported only
 # for the default shape; any other --B/--S/--T prints null.
-MEASURED_TRAFFIC_BYTES = {"mi_forward": 50124982, "mi_backward": 69268852}
+MEASURED_TRAFFIC_BYTES = {"mi_forward": 50124982, "mi_backward": 69268852}  # + "mi_forward_backward" below
 MEASURED_TRAFFIC_BYTES_PLAIN_PAIR = {"mi_forward": 50049796, "mi_backward": 86230408}  # --no-keep
 
 
@@ -240,6 +240,8 @@ def main():
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch one plain device copy of 256 MiB before the warmup: the unit "
                          "against which rocprofv3's FETCH_SIZE / WRITE_SIZE readings are scaled")
+    ap.add_argument("--two-launches", action="store_true",
+                    help="run the forward and the backward as two launches where one would do")
     ap.add_argument("--no-keep", action="store_true",
                     help="run the plain forward/backward pair (no log-derivative tensor between them)")
     ap.add_argument("--B", type=int, default=32)
@@ -276,7 +278,18 @@ def main():
     lattice = torch.empty(B, S + 1, T + 1, dtype=torch.float32, device=dev)
     p, log_deriv = (None, lattice) if keep else (lattice, None)
 
+    # ... and, where the device holds all of the launch's workgroups at once, both recursions run
+    # in ONE launch, again as mutual_information_recursion does
+    single = keep and not args.two_launches and capi.mi_forward_backward_supported(px, py)
+
     def step(ev=None):
+        if single:
+            if ev is not None:
+                ev[0].record()
+            g = capi.mi_forward_backward(px, py, bd, ones, overwrite_ans_grad=False)
+            if ev is not None:
+                ev[2].record()
+            return g
         if ev is not None:
             ev[0].record()
         capi.mi_forward(px, py, bd, p, log_deriv=log_deriv)
@@ -304,18 +317,29 @@ def main():
         step(events[k])
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    fwd_ms = np.array([e[0].elapsed_time(e[1]) for e in events])
-    bwd_ms = np.array([e[1].elapsed_time(e[2]) for e in events])
     ms_per_step = wall / args.steps * 1e3
-
-    # Roofline of the dominant kernel (the one with the longer average launch).
-    fwd_avg, bwd_avg = float(fwd_ms.mean()), float(bwd_ms.mean())
-    if bwd_avg >= fwd_avg:
-        dom, dom_ms, dom_bytes = "mi_backward", bwd_avg, BWD_BYTES_PER_CELL * active
-    else:
-        dom, dom_ms, dom_bytes = "mi_forward", fwd_avg, FWD_BYTES_PER_CELL * active
-    achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
     both_bytes = (FWD_BYTES_PER_CELL + BWD_BYTES_PER_CELL) * active
+    if single:
+        # one kernel does the step: its algorithmic bytes are the forward's plus the backward's
+        both_ms = np.array([e[0].elapsed_time(e[2]) for e in events])
+        dom, dom_ms, dom_bytes = "mi_forward_backward", float(both_ms.mean()), both_bytes
+        kernel_times = {"mi_forward_backward_avg_us": dom_ms * 1e3,
+                        "mi_forward_backward_min_us": float(both_ms.min()) * 1e3}
+        both_avg = dom_ms
+    else:
+        fwd_ms = np.array([e[0].elapsed_time(e[1]) for e in events])
+        bwd_ms = np.array([e[1].elapsed_time(e[2]) for e in events])
+        # Roofline of the dominant kernel (the one with the longer average launch).
+        fwd_avg, bwd_avg = float(fwd_ms.mean()), float(bwd_ms.mean())
+        if bwd_avg >= fwd_avg:
+            dom, dom_ms, dom_bytes = "mi_backward", bwd_avg, BWD_BYTES_PER_CELL * active
+        else:
+            dom, dom_ms, dom_bytes = "mi_forward", fwd_avg, FWD_BYTES_PER_CELL * active
+        kernel_times = {"mi_forward_avg_us": fwd_avg * 1e3, "mi_forward_min_us": float(fwd_ms.min()) * 1e3,
+                        "mi_backward_avg_us": bwd_avg * 1e3, "mi_backward_min_us": float(bwd_ms.min()) * 1e3}
+        both_avg = fwd_avg + bwd_avg
+    achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
+    traffic_table = (MEASURED_TRAFFIC_BYTES if keep else MEASURED_TRAFFIC_BYTES_PLAIN_PAIR)
     out = {
         "metric": "MI recursion fwd+bwd lattice-cells/s (B=32,S=200,T=1000) + % HBM roofline",
         "value": active / (ms_per_step * 1e-3),
@@ -326,18 +350,17 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"mutual_information_recursion fwd+bwd, fp32, modified, B={B} "
                                f"S={S} T={T}, random boundary (BASELINE config 4)",
-                   "active_cells": active, "full_box_cells": full, "log_deriv_kept": bool(keep)},
+                   "active_cells": active, "full_box_cells": full, "log_deriv_kept": bool(keep),
+                   "launches_per_step": 1 if single else 2},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": (MEASURED_TRAFFIC_BYTES if keep else MEASURED_TRAFFIC_BYTES_PLAIN_PAIR)[dom]
-                     if (B, S, T) == (32, 200, 1000) else None,
+                     "traffic": traffic_table.get(dom) if (B, S, T) == (32, 200, 1000) else None,
                      "kernel": dom,
                      "kernel_avg_us": dom_ms * 1e3},
-        "kernels": {"mi_forward_avg_us": fwd_avg * 1e3, "mi_forward_min_us": float(fwd_ms.min()) * 1e3,
-                    "mi_backward_avg_us": bwd_avg * 1e3, "mi_backward_min_us": float(bwd_ms.min()) * 1e3,
-                    "fwd_bwd_GBps_active_cells": both_bytes / ((fwd_avg + bwd_avg) * 1e-3) / 1e9,
-                    "fwd_bwd_frac_of_hbm_peak": both_bytes / ((fwd_avg + bwd_avg) * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                    "full_box_cells_per_s": full / ((fwd_avg + bwd_avg) * 1e-3)},
+        "kernels": dict(kernel_times,
+                        fwd_bwd_GBps_active_cells=both_bytes / (both_avg * 1e-3) / 1e9,
+                        fwd_bwd_frac_of_hbm_peak=both_bytes / (both_avg * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                        full_box_cells_per_s=full / (both_avg * 1e-3)),
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(c)

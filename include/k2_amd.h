@@ -104,6 +104,25 @@ K2AMD_API int k2amd_mi_backward_kept(const void *px, const void *py, const int64
                            int B, int S, int T, int modified, int dtype, int overwrite_ans_grad,
                            void *workspace, size_t workspace_bytes, void *stream);
 
+/* k2amd_mi_forward_keep followed by k2amd_mi_backward_kept, in ONE launch: what the reference's
+ * autograd function does with two native calls when gradients are wanted
+ * (k2/python/k2/mutual_information.py:157-169).  It has no counterpart in the reference.
+ *   ans [B] out; log_deriv [B][S+1][T+1] scratch (written, then read; contents as above);
+ *   ans_grad [B] in (and out if overwrite_ans_grad); px_grad, py_grad out, every element written.
+ * Same results, bit for bit, as the two calls.  Every workgroup of this launch must be resident
+ * at once, so it only serves shapes with 2 * B * ceil((S+1)/64) <= compute units of the current
+ * device, fp32, with a workspace: k2amd_mi_forward_backward_supported(...) says whether a call
+ * will be served (1) or returns K2AMD_ERR_UNSUPPORTED (0; use the two calls).  It also expects the
+ * device not to be busy with other streams' kernels for as long as a second: a workgroup that
+ * finds no compute unit free keeps others waiting, and a wait that expires ends the launch with
+ * K2AMD_ERR_TIMEOUT in the workspace's status.                                                   */
+K2AMD_API int k2amd_mi_forward_backward_supported(int B, int S, int T, int modified, int dtype,
+                                        int has_workspace);
+K2AMD_API int k2amd_mi_forward_backward(const void *px, const void *py, const int64_t *boundary, void *ans,
+                              void *log_deriv, void *ans_grad, void *px_grad, void *py_grad, int B,
+                              int S, int T, int modified, int dtype, int overwrite_ans_grad,
+                              void *workspace, size_t workspace_bytes, void *stream);
+
 /* ------------------------------------------------------------------ RNN-T log-prob builders
  *
  * Common conventions: symbols [B][S] int64 in [0,C); boundary [B][4] int64 or NULL;

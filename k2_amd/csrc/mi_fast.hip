@@ -295,25 +295,21 @@ constexpr int kFwdLoadsPerBlock = 2 * FwdLayout::kLoadItems;
 // one tensor instead of p twice and px once.  Cells of a sequence's first row and first column
 // hold values the backward never uses.  kWriteP = false (only with kKeep): p itself is not stored,
 // for callers that want nothing but ans and the gradients.
+// The whole workgroup sweeps chunk `chunk` (64 lattice rows) of sequence `seq`.
 template <bool kKeep, bool kWriteP>
-__global__ __launch_bounds__(FwdLayout::kThreads) void MiForwardFastKernel(
-    const float *__restrict__ px, const float *__restrict__ py,
+__device__ __forceinline__ void MiForwardChunk(
+    FwdLds &lds, const float *__restrict__ px, const float *__restrict__ py,
     const int64_t *__restrict__ boundary, float *__restrict__ p, float *__restrict__ ans,
     float *__restrict__ log_deriv, FastHeader *hdr, float *edge, int B, int S, int Tn,
-    int modified, int nchunks, int edge_stride) {
-  __shared__ FwdLds lds;
-  const unsigned total_wgs = gridDim.x;
-  if (threadIdx.x == 0) lds.ticket = atomicAdd(&hdr->ticket, 1u);
-  __syncthreads();
+    int modified, int nchunks, int edge_stride, int seq, int chunk) {
   ChunkGeom g;
-  g.b = lds.ticket / nchunks;
-  g.c = lds.ticket % nchunks;
+  g.b = seq;
+  g.c = chunk;
   const Box box = LoadBox(boundary, g.b, S, Tn);
   g.s0 = box.s0; g.t0 = box.t0; g.ns = box.s1 - box.s0; g.nt = box.t1 - box.t0;
   g.row0 = g.c * kRows;
   if (!box.ok || g.row0 > g.ns) {
     if (!box.ok && g.c == 0 && threadIdx.x == 0) ans[g.b] = __builtin_nanf("");
-    if (threadIdx.x == 0) FinishWorkgroup(hdr, total_wgs);
     return;
   }
   g.skew = modified ? 0 : 1;
@@ -606,7 +602,23 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiForwardFastKernel(
   }
   if (role == kStorer) store_block(g.nblocks - 1);
   if (role == kEdge) publish_block(g.nblocks - 1);
-  if (threadIdx.x == 0) FinishWorkgroup(hdr, total_wgs);
+}
+
+// One workgroup per chunk; the ticket fixes which (see the file header).
+template <bool kKeep, bool kWriteP>
+__global__ __launch_bounds__(FwdLayout::kThreads) void MiForwardFastKernel(
+    const float *__restrict__ px, const float *__restrict__ py,
+    const int64_t *__restrict__ boundary, float *__restrict__ p, float *__restrict__ ans,
+    float *__restrict__ log_deriv, FastHeader *hdr, float *edge, int B, int S, int Tn,
+    int modified, int nchunks, int edge_stride) {
+  __shared__ FwdLds lds;
+  if (threadIdx.x == 0) lds.ticket = atomicAdd(&hdr->ticket, 1u);
+  __syncthreads();
+  const unsigned ticket = lds.ticket;
+  MiForwardChunk<kKeep, kWriteP>(lds, px, py, boundary, p, ans, log_deriv, hdr, edge, B, S, Tn,
+                                 modified, nchunks, edge_stride, (int)(ticket / nchunks),
+                                 (int)(ticket % nchunks));
+  if (threadIdx.x == 0) FinishWorkgroup(hdr, gridDim.x);
 }
 
 // ------------------------------------------------------------------------------ backward
@@ -692,25 +704,18 @@ __device__ __forceinline__ void ZeroItem(const ZeroGeom &z, int r, int c) {
 
 // kKept: `p` is the log_deriv tensor a kKeep forward launch wrote (same layout as p), px is not
 // read, and every cell's d1 is exp() of one loaded value.
+// The whole workgroup sweeps chunk `chunk` of sequence `seq`, or (zero_only) clears what the
+// sweep leaves unassigned in array rows chunk * 64 .. chunk * 64 + 63 of that sequence.
 template <bool kKept>
-__global__ __launch_bounds__(BwdLayout::kThreads) void MiBackwardFastKernel(
-    const float *__restrict__ px, const float *__restrict__ p,
+__device__ __forceinline__ void MiBackwardChunk(
+    BwdLds &lds, const float *__restrict__ px, const float *__restrict__ p,
     const int64_t *__restrict__ boundary, float *__restrict__ ans_grad,
     float *__restrict__ px_grad, float *__restrict__ py_grad, FastHeader *hdr, float *edge, int B,
-    int S, int Tn, int modified, int nchunks, int edge_stride, int overwrite_ans_grad) {
-  __shared__ BwdLds lds;
-  const unsigned total_wgs = gridDim.x;
-  if (threadIdx.x == 0) lds.ticket = atomicAdd(&hdr->ticket, 1u);
-  __syncthreads();
-  // The first B * nchunks tickets sweep; the rest of the grid (as many again) clears what the
-  // sweep does not assign, one workgroup per (sequence, 64 array rows), on compute units the
-  // sweep leaves idle and off its critical path.
-  const unsigned nsweep = (unsigned)B * nchunks;
-  const bool zero_only = lds.ticket >= nsweep;
-  const unsigned unit = zero_only ? lds.ticket - nsweep : lds.ticket;
+    int S, int Tn, int modified, int nchunks, int edge_stride, int overwrite_ans_grad, int seq,
+    int chunk, bool zero_only) {
   ChunkGeom g;
-  g.b = unit / nchunks;
-  g.c = nchunks - 1 - (int)(unit % nchunks);  // lower chunks take earlier tickets
+  g.b = seq;
+  g.c = chunk;
   const Box box = LoadBox(boundary, g.b, S, Tn);
   const int T1 = modified ? Tn : Tn + 1;
   const int off = modified ? -1 : 0;
@@ -727,16 +732,12 @@ __global__ __launch_bounds__(BwdLayout::kThreads) void MiBackwardFastKernel(
     if (threadIdx.x < kRows * 8)
       for (int sl = 0; sl < zslices; ++sl)
         ZeroItem(zg, g.c * kRows + (threadIdx.x >> 3), sl * 32 + 4 * (threadIdx.x & 7));
-    if (threadIdx.x == 0) FinishWorkgroup(hdr, total_wgs);
     return;
   }
 
   g.s0 = box.s0; g.t0 = box.t0; g.ns = box.s1 - box.s0; g.nt = box.t1 - box.t0;
   g.row0 = g.c * kRows;
-  if (!box.ok || g.row0 > g.ns) {  // nothing to sweep
-    if (threadIdx.x == 0) FinishWorkgroup(hdr, total_wgs);
-    return;
-  }
+  if (!box.ok || g.row0 > g.ns) return;  // nothing to sweep
   g.skew = modified ? 0 : 1;
   const bool has_down = g.row0 + kRows <= g.ns;
   const bool has_up = g.c > 0;
@@ -1055,7 +1056,72 @@ __global__ __launch_bounds__(BwdLayout::kThreads) void MiBackwardFastKernel(
   if (role == kStorer) store_block(0);
   if (role == kEdge) publish_block(0);
   if (overwrite_ans_grad && role == kChain && g.c == 0 && lane == 0) ans_grad[g.b] = g_origin;
-  if (threadIdx.x == 0) FinishWorkgroup(hdr, total_wgs);
+}
+
+// The first B * nchunks tickets sweep, lower chunks first; the rest of the grid (as many again)
+// clears what the sweep does not assign, one workgroup per (sequence, 64 array rows), on compute
+// units the sweep leaves idle and off its critical path.
+template <bool kKept>
+__global__ __launch_bounds__(BwdLayout::kThreads) void MiBackwardFastKernel(
+    const float *__restrict__ px, const float *__restrict__ p,
+    const int64_t *__restrict__ boundary, float *__restrict__ ans_grad,
+    float *__restrict__ px_grad, float *__restrict__ py_grad, FastHeader *hdr, float *edge, int B,
+    int S, int Tn, int modified, int nchunks, int edge_stride, int overwrite_ans_grad) {
+  __shared__ BwdLds lds;
+  if (threadIdx.x == 0) lds.ticket = atomicAdd(&hdr->ticket, 1u);
+  __syncthreads();
+  const unsigned ticket = lds.ticket, nsweep = (unsigned)B * nchunks;
+  const bool zero_only = ticket >= nsweep;
+  const unsigned unit = zero_only ? ticket - nsweep : ticket;
+  MiBackwardChunk<kKept>(lds, px, p, boundary, ans_grad, px_grad, py_grad, hdr, edge, B, S, Tn,
+                         modified, nchunks, edge_stride, overwrite_ans_grad, (int)(unit / nchunks),
+                         zero_only ? (int)(unit % nchunks) : nchunks - 1 - (int)(unit % nchunks),
+                         zero_only);
+  if (threadIdx.x == 0) FinishWorkgroup(hdr, gridDim.x);
+}
+
+// Forward and backward of a sequence's chunk in ONE launch, for callers that want ans and the
+// gradients together (the reference's autograd function, k2/python/k2/mutual_information.py:
+// 157-169).  A workgroup sweeps its chunk forward, keeping the log-derivatives, and then sweeps
+// the same chunk backward: everything its backward loads is what its own forward stored, so only
+// the two kinds of edge words cross between workgroups.  The forward runs down a sequence's
+// chunks and the backward comes back up, so the launch costs what the two kernels cost one
+// after the other, less one launch gap and one start-up.  Unlike the separate kernels a workgroup
+// here also waits for a LATER ticket (the chunk below it, in the backward): the launcher only
+// uses this kernel where every sweeping workgroup finds a compute unit at once.
+union FusedLds {
+  FwdLds fwd;
+  BwdLds bwd;
+};
+__global__ __launch_bounds__(FwdLayout::kThreads) void MiForwardBackwardFastKernel(
+    const float *__restrict__ px, const float *__restrict__ py,
+    const int64_t *__restrict__ boundary, float *__restrict__ ans, float *__restrict__ log_deriv,
+    float *__restrict__ ans_grad, float *__restrict__ px_grad, float *__restrict__ py_grad,
+    FastHeader *hdr, float *edge_fwd, float *edge_bwd, int B, int S, int Tn, int modified,
+    int nchunks, int edge_stride, int overwrite_ans_grad) {
+  static_assert(FwdLayout::kThreads == BwdLayout::kThreads, "one workgroup shape for both sweeps");
+  __shared__ FusedLds lds;
+  __shared__ unsigned ticket_slot;
+  if (threadIdx.x == 0) ticket_slot = atomicAdd(&hdr->ticket, 1u);
+  __syncthreads();
+  const unsigned ticket = ticket_slot, nsweep = (unsigned)B * nchunks;
+  if (ticket >= nsweep) {  // clears what the backward sweep does not assign
+    const unsigned unit = ticket - nsweep;
+    MiBackwardChunk<true>(lds.bwd, px, log_deriv, boundary, ans_grad, px_grad, py_grad, hdr,
+                          edge_bwd, B, S, Tn, modified, nchunks, edge_stride, overwrite_ans_grad,
+                          (int)(unit / nchunks), (int)(unit % nchunks), true);
+  } else {
+    const int seq = (int)(ticket / nchunks), chunk = (int)(ticket % nchunks);
+    MiForwardChunk<true, false>(lds.fwd, px, py, boundary, nullptr, ans, log_deriv, hdr, edge_fwd,
+                                B, S, Tn, modified, nchunks, edge_stride, seq, chunk);
+    // __syncthreads() waits for every wavefront's outstanding stores as well: the log-derivatives
+    // are in the L2 this compute unit reads from before any of its loaders asks for them
+    __syncthreads();
+    MiBackwardChunk<true>(lds.bwd, px, log_deriv, boundary, ans_grad, px_grad, py_grad, hdr,
+                          edge_bwd, B, S, Tn, modified, nchunks, edge_stride, overwrite_ans_grad,
+                          seq, chunk, false);
+  }
+  if (threadIdx.x == 0) FinishWorkgroup(hdr, gridDim.x);
 }
 
 // A sweeping workgroup wants a compute unit to itself (its chain wavefront sets the pace of the
@@ -1063,7 +1129,7 @@ __global__ __launch_bounds__(BwdLayout::kThreads) void MiBackwardFastKernel(
 // Asking for more than half of the unit's 160 KB of LDS makes the dispatcher place one workgroup
 // per unit; the bytes beyond the kernels' own structures are never touched.
 constexpr size_t kExclusiveLds = 84 * 1024;
-static_assert(sizeof(FwdLds) < kExclusiveLds && sizeof(BwdLds) < kExclusiveLds, "LDS budget");
+static_assert(sizeof(FusedLds) + 16 < kExclusiveLds, "LDS budget");
 
 }  // namespace
 
@@ -1074,10 +1140,11 @@ bool MiFastSupports(int B, int S, int Tn, int modified) {
   return S >= 1 && Tn >= 1 && (long long)B * (S + 1) * (Tn + 1) < (1ll << 29);
 }
 
+// Two sets of edge rows: the single-launch forward + backward has both kinds in flight at once.
 size_t MiFastWorkspaceBytes(int B, int S, int Tn) {
   const int nchunks = (S + 1 + kRows - 1) / kRows;
   const size_t edge_stride = ((size_t)Tn + 2 + kRows + kW + 3) / 4 * 4 + kW;
-  return sizeof(FastHeader) + (size_t)B * (nchunks + 1) * edge_stride * sizeof(float);
+  return sizeof(FastHeader) + 2 * (size_t)B * (nchunks + 1) * edge_stride * sizeof(float);
 }
 
 int MiFastWorkspaceInit(void *workspace, size_t workspace_bytes, hipStream_t stream) {
@@ -1126,6 +1193,40 @@ int MiBackwardFast(const float *px, const float *p, const float *log_deriv,
     hipLaunchKernelGGL(MiBackwardFastKernel<true>, grid, block, pad, stream, px, log_deriv, boundary, ans_grad, px_grad, py_grad, hdr, edge, B, S, Tn, modified, nchunks, edge_stride, overwrite_ans_grad);
   else
     hipLaunchKernelGGL(MiBackwardFastKernel<false>, grid, block, pad, stream, px, p, boundary, ans_grad, px_grad, py_grad, hdr, edge, B, S, Tn, modified, nchunks, edge_stride, overwrite_ans_grad);
+  return LaunchStatus();
+}
+
+// Whether the single launch may be used on the current device: every sweeping workgroup (and the
+// clearing ones, which never wait) must find a compute unit of its own at once.
+bool MiFusedSupports(int B, int S, int Tn, int modified) {
+  if (!MiFastSupports(B, S, Tn, modified) || B < 1) return false;
+  static int units[64];  // compute units per device ordinal, 0 = not asked yet
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
+  if (units[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return false;
+    units[dev] = n > 0 ? n : -1;
+  }
+  const long long nchunks = (S + 1 + kRows - 1) / kRows;
+  return units[dev] > 0 && 2 * (long long)B * nchunks <= units[dev];
+}
+
+int MiForwardBackwardFast(const float *px, const float *py, const int64_t *boundary, float *ans,
+                          float *log_deriv, float *ans_grad, float *px_grad, float *py_grad, int B,
+                          int S, int Tn, int modified, int overwrite_ans_grad, void *workspace,
+                          size_t workspace_bytes, hipStream_t stream) {
+  if (workspace == nullptr || workspace_bytes < MiFastWorkspaceBytes(B, S, Tn)) return K2AMD_ERR_WORKSPACE;
+  if (log_deriv == nullptr) return K2AMD_ERR_INVALID_ARGUMENT;
+  if (!MiFusedSupports(B, S, Tn, modified)) return K2AMD_ERR_UNSUPPORTED;
+  const int nchunks = (S + 1 + kRows - 1) / kRows;
+  const int edge_stride = (int)(((size_t)Tn + 2 + kRows + kW + 3) / 4 * 4 + kW);
+  FastHeader *hdr = static_cast<FastHeader *>(workspace);
+  float *edge_fwd = reinterpret_cast<float *>(hdr + 1);
+  float *edge_bwd = edge_fwd + (size_t)B * (nchunks + 1) * edge_stride;
+  const dim3 grid((unsigned)(2 * B * nchunks)), block(FwdLayout::kThreads);
+  const size_t pad = kExclusiveLds - sizeof(FusedLds) - 16;
+  hipLaunchKernelGGL(MiForwardBackwardFastKernel, grid, block, pad, stream, px, py, boundary, ans, log_deriv, ans_grad, px_grad, py_grad, hdr, edge_fwd, edge_bwd, B, S, Tn, modified, nchunks, edge_stride, overwrite_ans_grad);
   return LaunchStatus();
 }
 

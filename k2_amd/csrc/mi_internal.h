@@ -33,6 +33,14 @@ int MiBackwardFast(const float *px, const float *p, const float *log_deriv,
                    int S, int Tn, int modified, int overwrite_ans_grad, void *workspace,
                    size_t workspace_bytes, hipStream_t stream);
 
+// Forward and backward in one launch (log_deriv is scratch of p's shape); MiFusedSupports says
+// whether the current device can hold the launch's workgroups at once, which that kernel needs.
+bool MiFusedSupports(int B, int S, int Tn, int modified);
+int MiForwardBackwardFast(const float *px, const float *py, const int64_t *boundary, float *ans,
+                          float *log_deriv, float *ans_grad, float *px_grad, float *py_grad, int B,
+                          int S, int Tn, int modified, int overwrite_ans_grad, void *workspace,
+                          size_t workspace_bytes, hipStream_t stream);
+
 }  // namespace k2amd
 
 #endif  // K2_AMD_CSRC_MI_INTERNAL_H_

@@ -192,6 +192,54 @@ std::vector<torch::Tensor> MutualInformationBackward(torch::Tensor px, torch::Te
   return {px_grad, py_grad};
 }
 
+bool MutualInformationForwardBackwardSupported(torch::Tensor px, torch::Tensor py) {
+  TORCH_CHECK(px.dim() == 3 && py.dim() == 3, "px and py must have three dimensions");
+  if (!px.is_cuda()) return false;
+  const int B = static_cast<int>(px.size(0)), S = static_cast<int>(px.size(1)),
+            T = static_cast<int>(py.size(2)), modified = px.size(2) == T ? 1 : 0;
+  const int dt = DtypeCode(px);
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(px.device());  // the answer depends on the device
+  return k2amd_mi_forward_backward_supported(B, S, T, modified, dt,
+                                             k2amd_mi_workspace_bytes(B, S, T, modified, dt) > 0) != 0;
+}
+
+// The two calls above in one launch (k2amd_mi_forward_backward): returns {ans, px_grad, py_grad}
+// and overwrites ans_grad like MutualInformationBackward.
+std::vector<torch::Tensor> MutualInformationForwardBackward(torch::Tensor px, torch::Tensor py,
+                                                            torch::optional<torch::Tensor> boundary,
+                                                            torch::Tensor ans_grad) {
+  TORCH_CHECK(px.dim() == 3 && py.dim() == 3, "px and py must have three dimensions");
+  TORCH_CHECK(px.is_cuda(), "k2_amd runs on MI355X only: px is on ", px.device(),
+              " (there is no CPU path)");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(px.device());
+  // scratch with p's shape: the forward sweep leaves the px-edge log-derivatives there
+  torch::Tensor log_deriv = torch::empty({px.size(0), px.size(1) + 1, py.size(2) + 1}, px.options());
+  const Shape sh = CheckInputs(px, py, boundary, log_deriv);
+  TORCH_CHECK(ans_grad.dim() == 1 && ans_grad.size(0) == sh.B, "ans_grad must have shape [B]");
+  TORCH_CHECK(ans_grad.device() == px.device() && ans_grad.scalar_type() == px.scalar_type(),
+              "ans_grad must match px in device and dtype");
+  TORCH_CHECK(ans_grad.is_contiguous(), "ans_grad must be contiguous");
+  px = px.contiguous();
+  py = py.contiguous();
+  torch::Tensor bd;
+  if (boundary.has_value() && boundary->defined()) bd = boundary->contiguous();
+  torch::Tensor ans = torch::empty({sh.B}, px.options());
+  torch::Tensor px_grad = torch::empty_like(px), py_grad = torch::empty_like(py);
+  const int dt = DtypeCode(px);
+  void *stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(px.device().index()).stream();
+  torch::Tensor ws = Cache().Get(k2amd_mi_workspace_bytes(sh.B, sh.S, sh.T, sh.modified, dt),
+                                 px.device(), stream);
+  {
+    pybind11::gil_scoped_release release;
+    Check(k2amd_mi_forward_backward(px.data_ptr(), py.data_ptr(),
+                                    bd.defined() ? bd.data_ptr<int64_t>() : nullptr, ans.data_ptr(),
+                                    log_deriv.data_ptr(), ans_grad.data_ptr(), px_grad.data_ptr(),
+                                    py_grad.data_ptr(), sh.B, sh.S, sh.T, sh.modified, dt,
+                                    /*overwrite_ans_grad=*/1, ws.defined() ? ws.data_ptr() : nullptr,
+                                    ws.defined() ? static_cast<size_t>(ws.numel()) : 0, stream));
+  }
+  return {ans, px_grad, py_grad};
+}
 
 // ---------------------------------------------------------------------------------------------
 // The fused builders that replace the torch-op chains of k2/python/k2/rnnt_loss.py.  Each mirrors
@@ -470,6 +518,11 @@ PYBIND11_MODULE(_k2_amd, m) {
   m.def("mutual_information_backward", &MutualInformationBackward, pybind11::arg("px"),
         pybind11::arg("py"), pybind11::arg("boundary"), pybind11::arg("p"),
         pybind11::arg("ans_grad"), pybind11::arg("log_deriv") = pybind11::none());
+  m.def("mutual_information_forward_backward_supported", &MutualInformationForwardBackwardSupported,
+        pybind11::arg("px"), pybind11::arg("py"));
+  m.def("mutual_information_forward_backward", &MutualInformationForwardBackward,
+        pybind11::arg("px"), pybind11::arg("py"), pybind11::arg("boundary"),
+        pybind11::arg("ans_grad"));
   m.def("version", []() { return k2amd_version(); });
   m.def("logprobs_simple_forward", &LogprobsSimpleForward);
   m.def("logprobs_simple_backward", &LogprobsSimpleBackward);

@@ -60,16 +60,21 @@ class MutualInformationRecursionFunction(torch.autograd.Function):
             assert boundary.shape == (B, 4), (boundary.shape, B)
 
         want_grad = return_grad or px.requires_grad or py.requires_grad
-        # the backward runs right away, so the forward can hand it the px-edge log-derivatives
-        # instead of p (which nothing else reads)
-        p, log_deriv = _lattice_buffers(px, py, want_grad)
-        ans = native.mutual_information_forward(px, py, boundary, p, log_deriv)
-
         px_grad, py_grad = None, None
-        if want_grad:
+        if want_grad and native.mutual_information_forward_backward_supported(px, py):
+            # both recursions in one launch
             ans_grad = torch.ones(B, device=px.device, dtype=px.dtype)
-            (px_grad, py_grad) = native.mutual_information_backward(px, py, boundary, p, ans_grad,
-                                                                    log_deriv)
+            (ans, px_grad, py_grad) = native.mutual_information_forward_backward(px, py, boundary, ans_grad)
+        else:
+            # the backward runs right away, so the forward can hand it the px-edge log-derivatives
+            # instead of p (which nothing else reads)
+            p, log_deriv = _lattice_buffers(px, py, want_grad)
+            ans = native.mutual_information_forward(px, py, boundary, p, log_deriv)
+            if want_grad:
+                ans_grad = torch.ones(B, device=px.device, dtype=px.dtype)
+                (px_grad, py_grad) = native.mutual_information_backward(px, py, boundary, p, ans_grad,
+                                                                        log_deriv)
+        if want_grad:
             ctx.save_for_backward(px_grad, py_grad)
         assert len(pxy_grads) == 2, len(pxy_grads)
         pxy_grads[0] = px_grad
@@ -146,11 +151,15 @@ def joint_mutual_information_recursion(
     py_cat = torch.stack(list(py), dim=0)  # [N][B][S+1][T]
     px_tot = px_cat.sum(dim=0).contiguous()
     py_tot = py_cat.sum(dim=0).contiguous()
-    p, log_deriv = _lattice_buffers(px_tot, py_tot, True)
-    tot_probs = native.mutual_information_forward(px_tot, py_tot, boundary, p, log_deriv)
     ans_grad = torch.ones(B, device=px_tot.device, dtype=px_tot.dtype)
-    (px_grad, py_grad) = native.mutual_information_backward(px_tot, py_tot, boundary, p, ans_grad,
-                                                            log_deriv)
+    if native.mutual_information_forward_backward_supported(px_tot, py_tot):
+        (tot_probs, px_grad, py_grad) = native.mutual_information_forward_backward(
+            px_tot, py_tot, boundary, ans_grad)
+    else:
+        p, log_deriv = _lattice_buffers(px_tot, py_tot, True)
+        tot_probs = native.mutual_information_forward(px_tot, py_tot, boundary, p, log_deriv)
+        (px_grad, py_grad) = native.mutual_information_backward(px_tot, py_tot, boundary, p, ans_grad,
+                                                                log_deriv)
     # -inf inputs carry zero occupation: clamp them to the most negative finite value so that
     # 0 * -inf does not produce NaN (k2/python/k2/mutual_information.py:410-411)
     lowest = torch.finfo(px_cat.dtype).min

@@ -62,6 +62,30 @@ def mutual_information_backward(px: torch.Tensor, py: torch.Tensor,
     return [gx, gy]
 
 
+def mutual_information_forward_backward_supported(px: torch.Tensor, py: torch.Tensor) -> bool:
+    """True if mutual_information_forward_backward serves these inputs on their device (fp32, the
+    pipelined kernels, and a compute unit for every workgroup of the launch)."""
+    _require_device(px)
+    if _ext is not None:
+        return _ext.mutual_information_forward_backward_supported(px, py)
+    return capi.mi_forward_backward_supported(px, py)
+
+
+def mutual_information_forward_backward(px: torch.Tensor, py: torch.Tensor,
+                                        boundary: Optional[torch.Tensor],
+                                        ans_grad: torch.Tensor) -> List[torch.Tensor]:
+    """mutual_information_forward followed by mutual_information_backward in one launch, as the
+    reference's autograd function calls them (k2/python/k2/mutual_information.py:157-169):
+    returns [ans, px_grad, py_grad] and overwrites ``ans_grad``."""
+    _require_device(px)
+    if _ext is not None:
+        return _ext.mutual_information_forward_backward(px, py, boundary, ans_grad)
+    ans, gx, gy = capi.mi_forward_backward(px.contiguous(), py.contiguous(),
+                                           None if boundary is None else boundary.contiguous(),
+                                           ans_grad, overwrite_ans_grad=True)
+    return [ans, gx, gy]
+
+
 # ---- the fused builders (replacements of the torch-op chains of k2/python/k2/rnnt_loss.py) ----
 # Same signatures and return values in both hosts; see capi.py for what each returns.
 

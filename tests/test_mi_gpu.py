@@ -56,6 +56,15 @@ def run_gpu(px, py, bd, device, ans_grad=None):
         assert capi.mi_workspace_is_clean(device), "workspace left dirty (kept pair without p)"
         for name, x, y in (("ans", ans3, ans), ("px_grad", gx3, gx), ("py_grad", gy3, gy), ("ans_grad", g3, g)):
             assert torch.equal(x.view(torch.int32), y.view(torch.int32)), "kept pair without p differs in " + name
+    if capi.mi_forward_backward_supported(tpx, tpy):
+        # both recursions in one launch
+        g4 = g_in.clone()
+        ans4, gx4, gy4 = capi.mi_forward_backward(tpx, tpy, tbd, g4, overwrite_ans_grad=True)
+        torch.cuda.synchronize()
+        assert capi.mi_workspace_is_clean(device), "workspace left dirty (single launch)"
+        capi.mi_workspace_status(device)
+        for name, x, y in (("ans", ans4, ans), ("px_grad", gx4, gx), ("py_grad", gy4, gy), ("ans_grad", g4, g)):
+            assert torch.equal(x.view(torch.int32), y.view(torch.int32)), "single launch differs in " + name
     return ans.cpu().numpy(), p.cpu().numpy(), gx.cpu().numpy(), gy.cpu().numpy(), g.cpu().numpy(), g_in.cpu().numpy()
 
 
@@ -227,6 +236,11 @@ def test_pybind_host_matches_ctypes_host(device):
                                                        log_deriv=kept)
     side.synchronize()
     assert torch.equal(ans3, ans2) and torch.equal(gx3, gx2) and torch.equal(gy3, gy2) and torch.equal(g3, g2)
+    assert _k2_amd.mutual_information_forward_backward_supported(px=px, py=py)
+    g5 = torch.full((B,), 2.0, device=device)
+    ans5, gx5, gy5 = _k2_amd.mutual_information_forward_backward(px=px_strided, py=py, boundary=bd, ans_grad=g5)
+    torch.cuda.synchronize()
+    assert torch.equal(ans5, ans2) and torch.equal(gx5, gx2) and torch.equal(gy5, gy2) and torch.equal(g5, g2)
     with pytest.raises(RuntimeError):  # wrong shape
         _k2_amd.mutual_information_forward(px=px, py=py, boundary=bd, p=p3, log_deriv=kept[:, :-1])
     g1 = torch.full((B,), 2.0, device=device)
@@ -298,3 +312,24 @@ def test_log_deriv_is_left_alone_by_the_exact_kernels(device):
     torch.cuda.synchronize()
     assert torch.equal(a1, a2) and torch.equal(x1, x2) and torch.equal(y1, y2)
     assert bool((kept == 7.0).all())
+
+
+@pytest.mark.gpu
+def test_single_launch_is_refused_where_it_cannot_be_resident(device):
+    """More sweeping workgroups than the device has compute units, fp64, or no workspace: the
+    single launch says so (and the Python layer then makes the two calls)."""
+    from k2_amd import capi
+    big = torch.zeros(300, 70, 11, device=device)   # 2 * 300 * 2 workgroups
+    assert not capi.mi_forward_backward_supported(big, torch.zeros(300, 71, 10, device=device))
+    px = torch.zeros(2, 5, 8, dtype=torch.float64, device=device)
+    py = torch.zeros(2, 6, 7, dtype=torch.float64, device=device)
+    assert not capi.mi_forward_backward_supported(px, py)
+    with pytest.raises(RuntimeError):
+        capi.mi_forward_backward(px, py, None, torch.ones(2, dtype=torch.float64, device=device))
+    import k2_amd as k2
+    bx = torch.randn(300, 70, 11, device=device)
+    by = torch.randn(300, 71, 10, device=device)
+    scores, (gx, gy) = k2.mutual_information_recursion(bx, by, None, return_grad=True)
+    small, (sx, sy) = k2.mutual_information_recursion(bx[:4].contiguous(), by[:4].contiguous(), None,
+                                                      return_grad=True)
+    assert torch.equal(scores[:4], small) and torch.equal(gx[:4], sx) and torch.equal(gy[:4], sy)
