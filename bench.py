@@ -284,12 +284,10 @@ def main():
 
     def step(ev=None):
         if single:
+            # one event per launch: launch k lasts from its event to the next launch's
             if ev is not None:
                 ev[0].record()
-            g = capi.mi_forward_backward(px, py, bd, ones, overwrite_ans_grad=False)
-            if ev is not None:
-                ev[2].record()
-            return g
+            return capi.mi_forward_backward(px, py, bd, ones, overwrite_ans_grad=False)
         if ev is not None:
             ev[0].record()
         capi.mi_forward(px, py, bd, p, log_deriv=log_deriv)
@@ -315,13 +313,16 @@ def main():
     t0 = time.perf_counter()
     for k in range(args.steps):
         step(events[k])
+    if single:
+        events[-1][2].record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ms_per_step = wall / args.steps * 1e3
     both_bytes = (FWD_BYTES_PER_CELL + BWD_BYTES_PER_CELL) * active
     if single:
         # one kernel does the step: its algorithmic bytes are the forward's plus the backward's
-        both_ms = np.array([e[0].elapsed_time(e[2]) for e in events])
+        ends = [e[0] for e in events[1:]] + [events[-1][2]]
+        both_ms = np.array([e[0].elapsed_time(end) for e, end in zip(events, ends)])
         dom, dom_ms, dom_bytes = "mi_forward_backward", float(both_ms.mean()), both_bytes
         kernel_times = {"mi_forward_backward_avg_us": dom_ms * 1e3,
                         "mi_forward_backward_min_us": float(both_ms.min()) * 1e3}
