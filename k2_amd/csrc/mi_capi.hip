@@ -15,11 +15,13 @@ bool ShapeOk(int B, int S, int T) {
   return ((int64_t)S + 1) * ((int64_t)T + 1) < (int64_t)1 << 31;
 }
 
-// K2AMD_MI_PATH=generic forces the exact log-domain kernels (used by the tests to cover both).
-bool ForceGeneric() {
+// K2AMD_MI_PATH=generic forces the exact log-domain kernels (used by the tests to cover both);
+// K2AMD_MI_PATH=two-launches keeps the pipelined kernels but never serves the single launch.
+bool PathIs(const char *name) {
   const char *e = std::getenv("K2AMD_MI_PATH");
-  return e != nullptr && std::strcmp(e, "generic") == 0;
+  return e != nullptr && std::strcmp(e, name) == 0;
 }
+bool ForceGeneric() { return PathIs("generic"); }
 
 }  // namespace
 
@@ -137,7 +139,7 @@ int k2amd_mi_backward_kept(const void *px, const void *py, const int64_t *bounda
 int k2amd_mi_forward_backward_supported(int B, int S, int T, int modified, int dtype,
                                         int has_workspace) {
   return dtype == K2AMD_F32 && has_workspace && ShapeOk(B, S, T) && B > 0 && !ForceGeneric() &&
-         MiFusedSupports(B, S, T, modified ? 1 : 0);
+         !PathIs("two-launches") && MiFusedSupports(B, S, T, modified ? 1 : 0);
 }
 
 int k2amd_mi_forward_backward(const void *px, const void *py, const int64_t *boundary, void *ans,

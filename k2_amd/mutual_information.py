@@ -33,6 +33,19 @@ def _check_boundary(boundary: Tensor, S: int, T: int) -> None:
     _checked_boundaries[ident] = (weakref.ref(boundary, lambda _, i=ident: _checked_boundaries.pop(i, None)), key)
 
 
+_single_launch_ok = {}
+
+
+def _single_launch(px: Tensor, py: Tensor) -> bool:
+    """Whether both recursions of these inputs run in one launch (asked of the native layer once
+    per shape, dtype and device)."""
+    key = (px.shape, py.shape[-1], px.dtype, px.device)
+    ok = _single_launch_ok.get(key)
+    if ok is None:
+        ok = _single_launch_ok[key] = bool(native.mutual_information_forward_backward_supported(px, py))
+    return ok
+
+
 def _lattice_buffers(px: Tensor, py: Tensor, want_grad: bool) -> Tuple[Optional[Tensor], Optional[Tensor]]:
     """(p, log_deriv) for a forward call that a backward call may follow: the [B][S+1][T+1]
     buffer the reference allocates as ``p`` (k2/python/k2/mutual_information.py:157) is handed over
@@ -61,7 +74,7 @@ class MutualInformationRecursionFunction(torch.autograd.Function):
 
         want_grad = return_grad or px.requires_grad or py.requires_grad
         px_grad, py_grad = None, None
-        if want_grad and native.mutual_information_forward_backward_supported(px, py):
+        if want_grad and _single_launch(px, py):
             # both recursions in one launch
             ans_grad = torch.ones(B, device=px.device, dtype=px.dtype)
             (ans, px_grad, py_grad) = native.mutual_information_forward_backward(px, py, boundary, ans_grad)
@@ -152,7 +165,7 @@ def joint_mutual_information_recursion(
     px_tot = px_cat.sum(dim=0).contiguous()
     py_tot = py_cat.sum(dim=0).contiguous()
     ans_grad = torch.ones(B, device=px_tot.device, dtype=px_tot.dtype)
-    if native.mutual_information_forward_backward_supported(px_tot, py_tot):
+    if _single_launch(px_tot, py_tot):
         (tot_probs, px_grad, py_grad) = native.mutual_information_forward_backward(
             px_tot, py_tot, boundary, ans_grad)
     else:
