@@ -15,8 +15,9 @@ bool ShapeOk(int B, int S, int T) {
   return ((int64_t)S + 1) * ((int64_t)T + 1) < (int64_t)1 << 31;
 }
 
-// K2AMD_MI_PATH=generic forces the exact log-domain kernels (used by the tests to cover both);
-// K2AMD_MI_PATH=two-launches keeps the pipelined kernels but never serves the single launch.
+// Switches for tests and comparisons, read at every call: K2AMD_MI_PATH=generic forces the exact
+// log-domain kernels; K2AMD_MI_PATH=two-launches keeps the pipelined kernels but never serves the
+// single launch.
 bool PathIs(const char *name) {
   const char *e = std::getenv("K2AMD_MI_PATH");
   return e != nullptr && std::strcmp(e, name) == 0;

@@ -333,3 +333,23 @@ def test_single_launch_is_refused_where_it_cannot_be_resident(device):
     small, (sx, sy) = k2.mutual_information_recursion(bx[:4].contiguous(), by[:4].contiguous(), None,
                                                       return_grad=True)
     assert torch.equal(scores[:4], small) and torch.equal(gx[:4], sx) and torch.equal(gy[:4], sy)
+
+
+@pytest.mark.gpu
+def test_path_switches(device, monkeypatch):
+    """K2AMD_MI_PATH selects the kernels at every call: `generic` runs the exact kernels on fp32
+    input that would otherwise take the pipelined ones (same results within the fp32 tolerance),
+    `two-launches` withdraws the single launch."""
+    from k2_amd import capi
+    c = cases.mi_case(11, dtype=np.float32, max_B=3, max_S=90, max_T=120)
+    want = run_gpu(c["px"], c["py"], c["boundary"], device)
+    tpx = torch.from_numpy(c["px"]).to(device)
+    tpy = torch.from_numpy(c["py"]).to(device)
+    assert capi.mi_keeps_log_deriv(tpx, tpy) and capi.mi_forward_backward_supported(tpx, tpy)
+    monkeypatch.setenv("K2AMD_MI_PATH", "two-launches")
+    assert capi.mi_keeps_log_deriv(tpx, tpy) and not capi.mi_forward_backward_supported(tpx, tpy)
+    monkeypatch.setenv("K2AMD_MI_PATH", "generic")
+    assert not capi.mi_keeps_log_deriv(tpx, tpy) and not capi.mi_forward_backward_supported(tpx, tpy)
+    got = run_gpu(c["px"], c["py"], c["boundary"], device)
+    for name, a, b in zip(("ans", "p", "px_grad", "py_grad"), got, want):
+        _close(name, a, b, None, TOL[np.dtype(np.float32)])
