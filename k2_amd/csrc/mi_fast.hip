@@ -34,6 +34,14 @@
 // per-call setup kernel.  Every wait is bounded; a timeout raises the header's error flag, after
 // which every later wait returns at once.
 //
+// Three kernels share the two sweeps (MiForwardChunk, MiBackwardChunk): the forward alone, the
+// backward alone, and both in one launch for callers that want the gradients with the scores.
+// In that launch, and in the two-call pair that goes with it, the forward hands the backward the
+// logarithm of every cell's px-edge derivative in a tensor that takes p's place, so the backward
+// reads one value per cell.  In the single launch a workgroup also waits for a LATER ticket (the
+// chunk below it, once it sweeps backward), so its launcher requires that all workgroups be
+// resident at once.
+//
 // Arithmetic is the reference's log-domain recursion (k2/python/csrc/torch/
 // mutual_information_cpu.cu:89-121, log-add of k2/csrc/utils.h:511-563) with hardware exp2/log2.
 #include "common.h"
