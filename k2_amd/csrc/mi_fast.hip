@@ -428,12 +428,15 @@ __device__ __forceinline__ void MiForwardChunk(
       const int row_i = g.row0 + q;
       if (row_i > g.ns) continue;
       const int pq = (kb % 3) * kQuadsPerBlock + mm;
-      float4 v = lds.fy[q][pq];
-      const float ninf = NegInfF();
-      v.x = v.x < kLogZeroTest ? ninf : v.x;
-      v.y = v.y < kLogZeroTest ? ninf : v.y;
-      v.z = v.z < kLogZeroTest ? ninf : v.z;
-      v.w = v.w < kLogZeroTest ? ninf : v.w;
+      const float4 raw = lds.fy[q][pq];
+      float4 v = raw;
+      if (kWriteP || !inner) {  // p (or ans, on the rim) leaves the chain: stand-ins become -inf
+        const float ninf = NegInfF();
+        v.x = v.x < kLogZeroTest ? ninf : v.x;
+        v.y = v.y < kLogZeroTest ? ninf : v.y;
+        v.z = v.z < kLogZeroTest ? ninf : v.z;
+        v.w = v.w < kLogZeroTest ? ninf : v.w;
+      }
       const int j = kb * kW + 4 * mm - q * g.skew;  // column of element 0
       const size_t at = (size_t)(g.s0 + row_i) * (Tn + 1) + g.t0 + j;
       float *dst = pb + at;
@@ -461,10 +464,13 @@ __device__ __forceinline__ void MiForwardChunk(
           }
           t1[0] = before + x4.x; t1[1] = a.x + x4.y; t1[2] = a.y + x4.z; t1[3] = a.z + x4.w;
         }
-        const float own[4] = {v.x, v.y, v.z, v.w};
+        // the backward's "total": p of the cell, or 0 where p is not finite (the stand-in for
+        // -inf counts as not finite)
+        const float own[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
-        for (int e = 0; e < 4; ++e) ld[e] = t1[e] - (__builtin_isfinite(own[e]) ? own[e] : 0.0f);
-        if (mm == kQuadsPerBlock - 1) lds.last[kb % 3][q] = v.w;
+        for (int e = 0; e < 4; ++e)
+          ld[e] = t1[e] - (__builtin_fabsf(own[e]) < -kLogZeroTest ? own[e] : 0.0f);
+        if (mm == kQuadsPerBlock - 1) lds.last[kb % 3][q] = raw.w;
       }
       if (inner) {  // uniform: every column of the block lies in 0..nt-1 for every row
         if (kWriteP) StoreQuad(dst, v);
