@@ -44,6 +44,8 @@
 //
 // Arithmetic is the reference's log-domain recursion (k2/python/csrc/torch/
 // mutual_information_cpu.cu:89-121, log-add of k2/csrc/utils.h:511-563) with hardware exp2/log2.
+#include <atomic>
+
 #include "common.h"
 #include "mi_internal.h"
 
@@ -1214,16 +1216,17 @@ int MiBackwardFast(const float *px, const float *p, const float *log_deriv,
 // clearing ones, which never wait) must find a compute unit of its own at once.
 bool MiFusedSupports(int B, int S, int Tn, int modified) {
   if (!MiFastSupports(B, S, Tn, modified) || B < 1) return false;
-  static int units[64];  // compute units per device ordinal, 0 = not asked yet
+  static std::atomic<int> units[64];  // compute units per device ordinal, 0 = not asked yet
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
-  if (units[dev] == 0) {
-    int n = 0;
+  int n = units[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
     if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return false;
-    units[dev] = n > 0 ? n : -1;
+    n = n > 0 ? n : -1;
+    units[dev].store(n, std::memory_order_relaxed);  // every thread would store the same value
   }
   const long long nchunks = (S + 1 + kRows - 1) / kRows;
-  return units[dev] > 0 && 2 * (long long)B * nchunks <= units[dev];
+  return n > 0 && 2 * (long long)B * nchunks <= n;
 }
 
 int MiForwardBackwardFast(const float *px, const float *py, const int64_t *boundary, float *ans,
