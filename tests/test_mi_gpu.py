@@ -353,3 +353,26 @@ def test_path_switches(device, monkeypatch):
     got = run_gpu(c["px"], c["py"], c["boundary"], device)
     for name, a, b in zip(("ans", "p", "px_grad", "py_grad"), got, want):
         _close(name, a, b, None, TOL[np.dtype(np.float32)])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("modified", [False, True])
+def test_blocked_and_improbable_edges(device, modified):
+    """Edges of log-probability -inf (a few per cent of them, so that whole regions of the lattice
+    and some end cells become unreachable) and of -3000 (far below fp32's exp range): all kernels
+    must agree with the CPU code's guards (k2/python/csrc/torch/mutual_information_cpu.cu:195-211)
+    and, as everywhere, with each other bit for bit."""
+    rng = np.random.default_rng(90 + int(modified))
+    B, S, T = 4, 150, 210
+    T1 = T if modified else T + 1
+    for frac_inf in (0.002, 0.05):
+        px = rng.normal(-2.0, 1.0, (B, S, T1)).astype(np.float32)
+        py = rng.normal(-2.0, 1.0, (B, S + 1, T)).astype(np.float32)
+        for a in (px, py):
+            a[rng.random(a.shape) < frac_inf] = -np.inf
+            a[rng.random(a.shape) < 0.02] = -3000.0
+        bd = np.array([[0, 0, S, T], [2, 3, 140, 200], [0, 10, 64, 74 if modified else 30], [5, 0, 5, 100]],
+                      dtype=np.int64)
+        ans, p = omi.mi_forward(px, py, bd)
+        gx, gy = omi.mi_backward(px, py, bd, p)
+        check("blocked %g modified=%s" % (frac_inf, modified), px, py, bd, (ans, p, gx, gy), device)
