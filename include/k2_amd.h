@@ -129,7 +129,11 @@ K2AMD_API int k2amd_mi_forward_backward(const void *px, const void *py, const in
  * px [B][S][T1] with T1 = T+1 for K2AMD_REGULAR (column T is -inf) and T otherwise;
  * py [B][S+1][T].  "constrained" adds py[b,s+1,t] to px[b,s,t]; "regular" with a boundary sets
  * px[b,:,t_end[b]] = -inf (k2/python/k2/rnnt_loss.py:25-43,220-223).  The *_backward functions
- * take the gradients w.r.t. the px / py that the matching forward returned.
+ * take the gradients w.r.t. the px / py that the matching forward returned, and seq_scale [B]
+ * (dtype as the gradients) or NULL: px_grad[b] and py_grad[b] count as multiplied by seq_scale[b].
+ * That is the product the reference's autograd function forms with two elementwise kernels
+ * (k2/python/k2/mutual_information.py:177-182: the occupation probabilities times the gradient
+ * that reaches the sequence's score); here it rides in the kernels that read the gradients.
  */
 
 /* Replaces get_rnnt_logprobs (k2/python/k2/rnnt_loss.py:65-225):
@@ -146,7 +150,8 @@ K2AMD_API int k2amd_rnnt_logprobs_simple_forward(
 /* Gradient of the above w.r.t. lm and am (what torch autograd derives from
  * k2/python/k2/rnnt_loss.py:172-223).  q_scratch [B][S+1][T] is scratch.                         */
 K2AMD_API int k2amd_rnnt_logprobs_simple_backward(
-    const void *px_grad, const void *py_grad, const int64_t *symbols, const int64_t *boundary,
+    const void *px_grad, const void *py_grad, const void *seq_scale, const int64_t *symbols,
+    const int64_t *boundary,
     const void *lm_probs, const void *am_probs, const void *denom, void *lm_grad, void *am_grad,
     void *q_scratch, int B, int S, int T, int C, int termination_symbol, int rnnt_type, int dtype,
     void *stream);
@@ -159,7 +164,7 @@ K2AMD_API int k2amd_rnnt_logprobs_joint_forward(
     void *stream);
 K2AMD_API int k2amd_rnnt_logprobs_joint_backward(
     const void *logits, const void *normalizers, const void *px_grad, const void *py_grad,
-    const int64_t *symbols, const int64_t *boundary, void *logits_grad, int B, int S, int T, int C,
+    const void *seq_scale, const int64_t *symbols, const int64_t *boundary, void *logits_grad, int B, int S, int T, int C,
     int termination_symbol, int rnnt_type, int dtype, void *stream);
 
 /* Replaces get_rnnt_logprobs_pruned (k2/python/k2/rnnt_loss.py:1180-1348): logits [B][T][R][C],
@@ -172,7 +177,7 @@ K2AMD_API int k2amd_rnnt_logprobs_pruned_forward(
     int termination_symbol, int rnnt_type, int dtype, void *stream);
 K2AMD_API int k2amd_rnnt_logprobs_pruned_backward(
     const void *logits, const void *normalizers, const void *px_grad, const void *py_grad,
-    const int64_t *symbols, const int64_t *ranges, const int64_t *boundary, void *logits_grad,
+    const void *seq_scale, const int64_t *symbols, const int64_t *ranges, const int64_t *boundary, void *logits_grad,
     int B, int S, int T, int R, int C, int termination_symbol, int rnnt_type, int dtype,
     void *stream);
 
@@ -187,7 +192,7 @@ K2AMD_API int k2amd_rnnt_hat_logprobs_pruned_forward(
     int dtype, void *stream);
 K2AMD_API int k2amd_rnnt_hat_logprobs_pruned_backward(
     const void *logits, const void *normalizers, const void *px_grad, const void *py_grad,
-    const int64_t *symbols, const int64_t *ranges, const int64_t *boundary, void *logits_grad,
+    const void *seq_scale, const int64_t *symbols, const int64_t *ranges, const int64_t *boundary, void *logits_grad,
     int B, int S, int T, int R, int C, int rnnt_type, int dtype, void *stream);
 
 /* ------------------------------------------------------------------ pruning

@@ -36,13 +36,13 @@ _SIGNATURES = {
     "k2amd_mi_forward_backward_supported": ([_ci] * 6, _ci),
     "k2amd_mi_forward_backward": ([_vp] * 8 + [_ci] * 6 + [_vp, _sz, _vp], _ci),
     "k2amd_rnnt_logprobs_simple_forward": ([_vp] * 11 + [_ci] * 7 + [_vp], _ci),
-    "k2amd_rnnt_logprobs_simple_backward": ([_vp] * 10 + [_ci] * 7 + [_vp], _ci),
+    "k2amd_rnnt_logprobs_simple_backward": ([_vp] * 11 + [_ci] * 7 + [_vp], _ci),
     "k2amd_rnnt_logprobs_joint_forward": ([_vp] * 6 + [_ci] * 7 + [_vp], _ci),
-    "k2amd_rnnt_logprobs_joint_backward": ([_vp] * 7 + [_ci] * 7 + [_vp], _ci),
+    "k2amd_rnnt_logprobs_joint_backward": ([_vp] * 8 + [_ci] * 7 + [_vp], _ci),
     "k2amd_rnnt_logprobs_pruned_forward": ([_vp] * 7 + [_ci] * 8 + [_vp], _ci),
-    "k2amd_rnnt_logprobs_pruned_backward": ([_vp] * 8 + [_ci] * 8 + [_vp], _ci),
+    "k2amd_rnnt_logprobs_pruned_backward": ([_vp] * 9 + [_ci] * 8 + [_vp], _ci),
     "k2amd_rnnt_hat_logprobs_pruned_forward": ([_vp] * 7 + [_ci] * 7 + [_vp], _ci),
-    "k2amd_rnnt_hat_logprobs_pruned_backward": ([_vp] * 8 + [_ci] * 7 + [_vp], _ci),
+    "k2amd_rnnt_hat_logprobs_pruned_backward": ([_vp] * 9 + [_ci] * 7 + [_vp], _ci),
     "k2amd_rnnt_prune_ranges": ([_vp] * 4 + [_ci] * 6 + [_vp], _ci),
     "k2amd_rnnt_prune_gather": ([_vp] * 3 + [_ci] * 6 + [_vp], _ci),
     "k2amd_rnnt_prune_gather_backward": ([_vp] * 3 + [_ci] * 6 + [_vp], _ci),
@@ -241,7 +241,9 @@ def logprobs_simple_forward(lm, am, symbols, termination_symbol, rnnt_type, boun
 
 
 def logprobs_simple_backward(px_grad, py_grad, symbols, boundary, saved, termination_symbol,
-                             rnnt_type):
+                             rnnt_type, seq_scale=None):
+    """``seq_scale`` [B] or None: px_grad[b], py_grad[b] count as multiplied by seq_scale[b] (the
+    same for the two functions below)."""
     lm_probs, am_probs, denom = saved
     B, T, C = am_probs.shape
     S = lm_probs.shape[1] - 1
@@ -251,8 +253,8 @@ def logprobs_simple_backward(px_grad, py_grad, symbols, boundary, saved, termina
     dev = am_probs.device
     with torch.cuda.device(dev):
         check(lib().k2amd_rnnt_logprobs_simple_backward(
-            ptr(px_grad), ptr(py_grad), ptr(symbols), ptr(boundary), ptr(lm_probs), ptr(am_probs),
-            ptr(denom), ptr(lm_grad), ptr(am_grad), ptr(q), B, S, T, C, termination_symbol,
+            ptr(px_grad), ptr(py_grad), ptr(seq_scale), ptr(symbols), ptr(boundary), ptr(lm_probs),
+            ptr(am_probs), ptr(denom), ptr(lm_grad), ptr(am_grad), ptr(q), B, S, T, C, termination_symbol,
             rnnt_type, dtype_code(am_probs), stream_ptr(dev)))
     return lm_grad, am_grad
 
@@ -272,14 +274,14 @@ def logprobs_joint_forward(logits, symbols, termination_symbol, rnnt_type, bound
 
 
 def logprobs_joint_backward(logits, norm, px_grad, py_grad, symbols, boundary,
-                            termination_symbol, rnnt_type):
+                            termination_symbol, rnnt_type, seq_scale=None):
     B, T, S1, C = logits.shape
     grad = torch.empty_like(logits)
     dev = logits.device
     with torch.cuda.device(dev):
         check(lib().k2amd_rnnt_logprobs_joint_backward(
-            ptr(logits), ptr(norm), ptr(px_grad), ptr(py_grad), ptr(symbols), ptr(boundary),
-            ptr(grad), B, S1 - 1, T, C, termination_symbol, rnnt_type, dtype_code(logits),
+            ptr(logits), ptr(norm), ptr(px_grad), ptr(py_grad), ptr(seq_scale), ptr(symbols),
+            ptr(boundary), ptr(grad), B, S1 - 1, T, C, termination_symbol, rnnt_type, dtype_code(logits),
             stream_ptr(dev)))
     return grad
 
@@ -306,7 +308,7 @@ def logprobs_pruned_forward(logits, symbols, ranges, termination_symbol, boundar
 
 
 def logprobs_pruned_backward(logits, norm, px_grad, py_grad, symbols, ranges, boundary,
-                             termination_symbol, rnnt_type, hat=False):
+                             termination_symbol, rnnt_type, hat=False, seq_scale=None):
     B, T, R, C = logits.shape
     S = symbols.shape[1]
     grad = torch.empty_like(logits)
@@ -314,13 +316,13 @@ def logprobs_pruned_backward(logits, norm, px_grad, py_grad, symbols, ranges, bo
     with torch.cuda.device(dev):
         if hat:
             check(lib().k2amd_rnnt_hat_logprobs_pruned_backward(
-                ptr(logits), ptr(norm), ptr(px_grad), ptr(py_grad), ptr(symbols), ptr(ranges),
-                ptr(boundary), ptr(grad), B, S, T, R, C, rnnt_type, dtype_code(logits),
+                ptr(logits), ptr(norm), ptr(px_grad), ptr(py_grad), ptr(seq_scale), ptr(symbols),
+                ptr(ranges), ptr(boundary), ptr(grad), B, S, T, R, C, rnnt_type, dtype_code(logits),
                 stream_ptr(dev)))
             return grad
         check(lib().k2amd_rnnt_logprobs_pruned_backward(
-            ptr(logits), ptr(norm), ptr(px_grad), ptr(py_grad), ptr(symbols), ptr(ranges),
-            ptr(boundary), ptr(grad), B, S, T, R, C, termination_symbol, rnnt_type,
+            ptr(logits), ptr(norm), ptr(px_grad), ptr(py_grad), ptr(seq_scale), ptr(symbols),
+            ptr(ranges), ptr(boundary), ptr(grad), B, S, T, R, C, termination_symbol, rnnt_type,
             dtype_code(logits), stream_ptr(dev)))
     return grad
 

@@ -11,6 +11,18 @@
 
 namespace k2amd {
 
+// a * b rounded on its own: the empty asm statement hides the product from the compiler, which
+// would otherwise fuse it into a following addition (contraction is on for HIP code, and the
+// *_rn intrinsics do not stop it).  Used where a result has to equal what separate elementwise
+// kernels would have produced.
+template <typename T>
+__device__ __forceinline__ T MulRounded(T a, T b) {
+  T r = a * b;
+  asm volatile("" : "+v"(r));
+  return r;
+}
+
+
 constexpr int kWave = 64;  // CDNA wavefront width
 
 // Turns the last HIP error into a status code without clearing sticky state of other streams.

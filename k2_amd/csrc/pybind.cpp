@@ -287,14 +287,26 @@ std::vector<torch::Tensor> LogprobsSimpleForward(torch::Tensor lm, torch::Tensor
   return {px, py, lm_probs, am_probs, denom};
 }
 
+// seq_scale of the *_backward entry points: [B], contiguous, dtype and device of the gradients
+const void *ScalePtr(const torch::optional<torch::Tensor> &seq_scale, const torch::Tensor &px_grad) {
+  if (!seq_scale.has_value() || !seq_scale->defined()) return nullptr;
+  TORCH_CHECK(seq_scale->dim() == 1 && seq_scale->size(0) == px_grad.size(0) &&
+                  seq_scale->scalar_type() == px_grad.scalar_type() &&
+                  seq_scale->device() == px_grad.device() && seq_scale->is_contiguous(),
+              "seq_scale must be a contiguous [B] tensor with the gradients' dtype and device");
+  return seq_scale->data_ptr();
+}
+
 std::vector<torch::Tensor> LogprobsSimpleBackward(torch::Tensor px_grad, torch::Tensor py_grad,
                                                   torch::Tensor symbols,
                                                   torch::optional<torch::Tensor> boundary,
                                                   torch::Tensor lm_probs, torch::Tensor am_probs,
                                                   torch::Tensor denom, int termination_symbol,
-                                                  int rnnt_type) {
+                                                  int rnnt_type,
+                                                  torch::optional<torch::Tensor> seq_scale) {
   RequireDevice(px_grad, "px_grad");
   RequireDevice(py_grad, "py_grad");
+  const void *scale = ScalePtr(seq_scale, px_grad);
   c10::hip::HIPGuardMasqueradingAsCUDA guard(am_probs.device());
   const int B = am_probs.size(0), T = am_probs.size(1), C = am_probs.size(2), S = lm_probs.size(1) - 1;
   torch::Tensor lm_grad = torch::empty_like(lm_probs), am_grad = torch::empty_like(am_probs);
@@ -303,7 +315,7 @@ std::vector<torch::Tensor> LogprobsSimpleBackward(torch::Tensor px_grad, torch::
   {
     pybind11::gil_scoped_release release;
     Check(k2amd_rnnt_logprobs_simple_backward(
-        px_grad.data_ptr(), py_grad.data_ptr(), I64(symbols), I64(boundary), lm_probs.data_ptr(),
+        px_grad.data_ptr(), py_grad.data_ptr(), scale, I64(symbols), I64(boundary), lm_probs.data_ptr(),
         am_probs.data_ptr(), denom.data_ptr(), lm_grad.data_ptr(), am_grad.data_ptr(), q.data_ptr(),
         B, S, T, C, termination_symbol, rnnt_type, DtypeCode(am_probs), stream));
   }
@@ -333,10 +345,11 @@ std::vector<torch::Tensor> LogprobsJointForward(torch::Tensor logits, torch::Ten
 torch::Tensor LogprobsJointBackward(torch::Tensor logits, torch::Tensor norm, torch::Tensor px_grad,
                                     torch::Tensor py_grad, torch::Tensor symbols,
                                     torch::optional<torch::Tensor> boundary, int termination_symbol,
-                                    int rnnt_type) {
+                                    int rnnt_type, torch::optional<torch::Tensor> seq_scale) {
   RequireDevice(logits, "logits");
   RequireDevice(px_grad, "px_grad");
   RequireDevice(py_grad, "py_grad");
+  const void *scale = ScalePtr(seq_scale, px_grad);
   c10::hip::HIPGuardMasqueradingAsCUDA guard(logits.device());
   const int B = logits.size(0), T = logits.size(1), S = logits.size(2) - 1, C = logits.size(3);
   torch::Tensor grad = torch::empty_like(logits);
@@ -344,7 +357,7 @@ torch::Tensor LogprobsJointBackward(torch::Tensor logits, torch::Tensor norm, to
   {
     pybind11::gil_scoped_release release;
     Check(k2amd_rnnt_logprobs_joint_backward(logits.data_ptr(), norm.data_ptr(), px_grad.data_ptr(),
-                                             py_grad.data_ptr(), I64(symbols), I64(boundary),
+                                             py_grad.data_ptr(), scale, I64(symbols), I64(boundary),
                                              grad.data_ptr(), B, S, T, C, termination_symbol, rnnt_type,
                                              DtypeCode(logits), stream));
   }
@@ -384,10 +397,12 @@ std::vector<torch::Tensor> LogprobsPrunedForward(torch::Tensor logits, torch::Te
 torch::Tensor LogprobsPrunedBackward(torch::Tensor logits, torch::Tensor norm, torch::Tensor px_grad,
                                      torch::Tensor py_grad, torch::Tensor symbols, torch::Tensor ranges,
                                      torch::optional<torch::Tensor> boundary, int termination_symbol,
-                                     int rnnt_type, bool hat) {
+                                     int rnnt_type, bool hat,
+                                     torch::optional<torch::Tensor> seq_scale) {
   RequireDevice(logits, "logits");
   RequireDevice(px_grad, "px_grad");
   RequireDevice(py_grad, "py_grad");
+  const void *scale = ScalePtr(seq_scale, px_grad);
   c10::hip::HIPGuardMasqueradingAsCUDA guard(logits.device());
   const int B = logits.size(0), T = logits.size(1), R = logits.size(2), C = logits.size(3);
   const int S = symbols.size(1);
@@ -397,13 +412,13 @@ torch::Tensor LogprobsPrunedBackward(torch::Tensor logits, torch::Tensor norm, t
     pybind11::gil_scoped_release release;
     if (hat)
       Check(k2amd_rnnt_hat_logprobs_pruned_backward(
-          logits.data_ptr(), norm.data_ptr(), px_grad.data_ptr(), py_grad.data_ptr(), I64(symbols),
-          I64(ranges), I64(boundary), grad.data_ptr(), B, S, T, R, C, rnnt_type, DtypeCode(logits),
+          logits.data_ptr(), norm.data_ptr(), px_grad.data_ptr(), py_grad.data_ptr(), scale,
+          I64(symbols), I64(ranges), I64(boundary), grad.data_ptr(), B, S, T, R, C, rnnt_type, DtypeCode(logits),
           stream));
     else
       Check(k2amd_rnnt_logprobs_pruned_backward(
-          logits.data_ptr(), norm.data_ptr(), px_grad.data_ptr(), py_grad.data_ptr(), I64(symbols),
-          I64(ranges), I64(boundary), grad.data_ptr(), B, S, T, R, C, termination_symbol, rnnt_type,
+          logits.data_ptr(), norm.data_ptr(), px_grad.data_ptr(), py_grad.data_ptr(), scale,
+          I64(symbols), I64(ranges), I64(boundary), grad.data_ptr(), B, S, T, R, C, termination_symbol, rnnt_type,
           DtypeCode(logits), stream));
   }
   return grad;

@@ -249,7 +249,8 @@ __global__ void ConstrainedKernel(T *__restrict__ px, const T *__restrict__ py, 
 // slot of logits_grad: {gx, gy, symbol, normaliser}.  Rows therefore need at least four columns.
 template <typename T, bool kPruned>
 __global__ void RowGradPrepKernel(const T *__restrict__ normalizers, const T *__restrict__ px_grad,
-                                  const T *__restrict__ py_grad, const int64_t *__restrict__ symbols,
+                                  const T *__restrict__ py_grad, const T *__restrict__ seq_scale,
+                                  const int64_t *__restrict__ symbols,
                                   const int64_t *__restrict__ ranges,
                                   const int64_t *__restrict__ boundary, T *__restrict__ logits_grad,
                                   RowGeom g) {
@@ -262,17 +263,18 @@ __global__ void RowGradPrepKernel(const T *__restrict__ normalizers, const T *__
   int s, sym;
   RowTarget<kPruned>(g, symbols, ranges, b, t, k, &s, &sym);
   const int T1 = g.rnnt_type == K2AMD_REGULAR ? g.Tn + 1 : g.Tn;
+  const T scale = seq_scale != nullptr ? seq_scale[b] : T(1);  // what reaches the sequence's score
   T gx = 0;
   if (s < g.S && sym >= 0 && sym < g.C) {
     const bool cut =
         g.rnnt_type == K2AMD_REGULAR && boundary != nullptr && boundary[4 * b + 3] == t;
-    if (!cut) gx = px_grad[((size_t)b * g.S + s) * T1 + t];
+    if (!cut) gx = MulRounded(px_grad[((size_t)b * g.S + s) * T1 + t], scale);
   } else {
     sym = -1;
   }
-  T gy = py_grad[((size_t)b * (g.S + 1) + s) * g.Tn + t];
+  T gy = MulRounded(py_grad[((size_t)b * (g.S + 1) + s) * g.Tn + t], scale);
   if (g.rnnt_type == K2AMD_CONSTRAINED && s >= 1)
-    gy += px_grad[((size_t)b * g.S + (s - 1)) * T1 + t];  // px += py[:, 1:]
+    gy += MulRounded(px_grad[((size_t)b * g.S + (s - 1)) * T1 + t], scale);  // px += py[:, 1:]
   T *rec = logits_grad + (size_t)row * g.C;
   rec[0] = gx;
   rec[1] = gy;
@@ -364,7 +366,7 @@ __global__ __launch_bounds__(kRowsPerBlock *kWave) void RowGradKernel(
 template <typename T, bool kPruned, bool kHat>
 __global__ __launch_bounds__(kRowsPerBlock *kWave) void RowBackwardKernel(
     const T *__restrict__ logits, const T *__restrict__ normalizers,
-    const T *__restrict__ px_grad, const T *__restrict__ py_grad,
+    const T *__restrict__ px_grad, const T *__restrict__ py_grad, const T *__restrict__ seq_scale,
     const int64_t *__restrict__ symbols, const int64_t *__restrict__ ranges,
     const int64_t *__restrict__ boundary, T *__restrict__ logits_grad, RowGeom g) {
   const int lane = threadIdx.x & (kWave - 1);
@@ -378,17 +380,18 @@ __global__ __launch_bounds__(kRowsPerBlock *kWave) void RowBackwardKernel(
   RowTarget<kPruned>(g, symbols, ranges, b, t, k, &s, &sym);
   const int T1 = g.rnnt_type == K2AMD_REGULAR ? g.Tn + 1 : g.Tn;
   // gradient reaching this row's px value and py value
+  const T scale = seq_scale != nullptr ? seq_scale[b] : T(1);
   T gx = 0;
   if (s < g.S && sym >= 0 && sym < g.C) {
     const bool cut =
         g.rnnt_type == K2AMD_REGULAR && boundary != nullptr && boundary[4 * b + 3] == t;
-    if (!cut) gx = px_grad[((size_t)b * g.S + s) * T1 + t];
+    if (!cut) gx = MulRounded(px_grad[((size_t)b * g.S + s) * T1 + t], scale);
   } else {
     sym = -1;
   }
-  T gy = py_grad[((size_t)b * (g.S + 1) + s) * g.Tn + t];
+  T gy = MulRounded(py_grad[((size_t)b * (g.S + 1) + s) * g.Tn + t], scale);
   if (g.rnnt_type == K2AMD_CONSTRAINED && s >= 1)
-    gy += px_grad[((size_t)b * g.S + (s - 1)) * T1 + t];  // px += py[:, 1:]
+    gy += MulRounded(px_grad[((size_t)b * g.S + (s - 1)) * T1 + t], scale);  // px += py[:, 1:]
   const T *x = logits + (size_t)row * g.C;
   T *dx = logits_grad + (size_t)row * g.C;
   RowGradTerms<T, kHat> terms;
@@ -433,19 +436,19 @@ int RowForward(const T *logits, const int64_t *symbols, const int64_t *ranges,
 
 template <typename T, bool kPruned, bool kHat>
 int RowBackward(const T *logits, const T *normalizers, const T *px_grad, const T *py_grad,
-                const int64_t *symbols, const int64_t *ranges, const int64_t *boundary,
+                const T *seq_scale, const int64_t *symbols, const int64_t *ranges, const int64_t *boundary,
                 T *logits_grad, RowGeom g, hipStream_t stream) {
   const long long rows = (long long)g.B * g.Tn * g.K;
   if (rows > 0) {
     const long long blocks = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
     if (g.C >= 4 && g.C <= (1 << 24)) {  // the record holds the symbol as a float: exact up to 2^24
       hipLaunchKernelGGL((RowGradPrepKernel<T, kPruned>), dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, stream,
-                         normalizers, px_grad, py_grad, symbols, ranges, boundary, logits_grad, g);
+                         normalizers, px_grad, py_grad, seq_scale, symbols, ranges, boundary, logits_grad, g);
       hipLaunchKernelGGL((RowGradKernel<T, kHat>), dim3((unsigned)blocks), dim3(kRowsPerBlock * kWave), 0, stream,
                          logits, logits_grad, rows, g.C, g.blank);
     } else {
       hipLaunchKernelGGL((RowBackwardKernel<T, kPruned, kHat>), dim3((unsigned)blocks), dim3(kRowsPerBlock * kWave), 0, stream,
-                         logits, normalizers, px_grad, py_grad, symbols, ranges, boundary,
+                         logits, normalizers, px_grad, py_grad, seq_scale, symbols, ranges, boundary,
                          logits_grad, g);
     }
   }
@@ -482,7 +485,7 @@ int k2amd_rnnt_logprobs_joint_forward(const void *logits, const int64_t *symbols
 
 int k2amd_rnnt_logprobs_joint_backward(const void *logits, const void *normalizers,
                                        const void *px_grad, const void *py_grad,
-                                       const int64_t *symbols, const int64_t *boundary,
+                                       const void *seq_scale, const int64_t *symbols, const int64_t *boundary,
                                        void *logits_grad, int B, int S, int T, int C,
                                        int termination_symbol, int rnnt_type, int dtype,
                                        void *stream) {
@@ -490,8 +493,8 @@ int k2amd_rnnt_logprobs_joint_backward(const void *logits, const void *normalize
   RowGeom g{B, S, T, S + 1, C, termination_symbol, rnnt_type, 0};
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == K2AMD_F32)
-    return RowBackward<float, false, false>((const float *)logits, (const float *)normalizers, (const float *)px_grad, (const float *)py_grad, symbols, nullptr, boundary, (float *)logits_grad, g, st);
-  return RowBackward<double, false, false>((const double *)logits, (const double *)normalizers, (const double *)px_grad, (const double *)py_grad, symbols, nullptr, boundary, (double *)logits_grad, g, st);
+    return RowBackward<float, false, false>((const float *)logits, (const float *)normalizers, (const float *)px_grad, (const float *)py_grad, (const float *)seq_scale, symbols, nullptr, boundary, (float *)logits_grad, g, st);
+  return RowBackward<double, false, false>((const double *)logits, (const double *)normalizers, (const double *)px_grad, (const double *)py_grad, (const double *)seq_scale, symbols, nullptr, boundary, (double *)logits_grad, g, st);
 }
 
 int k2amd_rnnt_logprobs_pruned_forward(const void *logits, const int64_t *symbols,
@@ -509,7 +512,7 @@ int k2amd_rnnt_logprobs_pruned_forward(const void *logits, const int64_t *symbol
 
 int k2amd_rnnt_logprobs_pruned_backward(const void *logits, const void *normalizers,
                                         const void *px_grad, const void *py_grad,
-                                        const int64_t *symbols, const int64_t *ranges,
+                                        const void *seq_scale, const int64_t *symbols, const int64_t *ranges,
                                         const int64_t *boundary, void *logits_grad, int B, int S,
                                         int T, int R, int C, int termination_symbol, int rnnt_type,
                                         int dtype, void *stream) {
@@ -517,8 +520,8 @@ int k2amd_rnnt_logprobs_pruned_backward(const void *logits, const void *normaliz
   RowGeom g{B, S, T, R, C, termination_symbol, rnnt_type, 0};
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == K2AMD_F32)
-    return RowBackward<float, true, false>((const float *)logits, (const float *)normalizers, (const float *)px_grad, (const float *)py_grad, symbols, ranges, boundary, (float *)logits_grad, g, st);
-  return RowBackward<double, true, false>((const double *)logits, (const double *)normalizers, (const double *)px_grad, (const double *)py_grad, symbols, ranges, boundary, (double *)logits_grad, g, st);
+    return RowBackward<float, true, false>((const float *)logits, (const float *)normalizers, (const float *)px_grad, (const float *)py_grad, (const float *)seq_scale, symbols, ranges, boundary, (float *)logits_grad, g, st);
+  return RowBackward<double, true, false>((const double *)logits, (const double *)normalizers, (const double *)px_grad, (const double *)py_grad, (const double *)seq_scale, symbols, ranges, boundary, (double *)logits_grad, g, st);
 }
 
 int k2amd_rnnt_hat_logprobs_pruned_forward(const void *logits, const int64_t *symbols,
@@ -536,7 +539,7 @@ int k2amd_rnnt_hat_logprobs_pruned_forward(const void *logits, const int64_t *sy
 
 int k2amd_rnnt_hat_logprobs_pruned_backward(const void *logits, const void *normalizers,
                                             const void *px_grad, const void *py_grad,
-                                            const int64_t *symbols, const int64_t *ranges,
+                                            const void *seq_scale, const int64_t *symbols, const int64_t *ranges,
                                             const int64_t *boundary, void *logits_grad, int B,
                                             int S, int T, int R, int C, int rnnt_type, int dtype,
                                             void *stream) {
@@ -544,8 +547,8 @@ int k2amd_rnnt_hat_logprobs_pruned_backward(const void *logits, const void *norm
   RowGeom g{B, S, T, R, C, 0, rnnt_type, 1};
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == K2AMD_F32)
-    return RowBackward<float, true, true>((const float *)logits, (const float *)normalizers, (const float *)px_grad, (const float *)py_grad, symbols, ranges, boundary, (float *)logits_grad, g, st);
-  return RowBackward<double, true, true>((const double *)logits, (const double *)normalizers, (const double *)px_grad, (const double *)py_grad, symbols, ranges, boundary, (double *)logits_grad, g, st);
+    return RowBackward<float, true, true>((const float *)logits, (const float *)normalizers, (const float *)px_grad, (const float *)py_grad, (const float *)seq_scale, symbols, ranges, boundary, (float *)logits_grad, g, st);
+  return RowBackward<double, true, true>((const double *)logits, (const double *)normalizers, (const double *)px_grad, (const double *)py_grad, (const double *)seq_scale, symbols, ranges, boundary, (double *)logits_grad, g, st);
 }
 
 }  // extern "C"

@@ -539,16 +539,18 @@ struct Tiny<double> { static constexpr double v = 2.2250738585072014e-308; };
 template <typename T>
 struct GradView {
   const T *px_grad, *py_grad;
+  const T *seq_scale;  // what reaches sequence b's score multiplies its gradients (null: 1)
   const int64_t *boundary;
   int S, Tn, rnnt_type;
+  __device__ __forceinline__ T Scale(int b) const { return seq_scale != nullptr ? seq_scale[b] : T(1); }
   __device__ __forceinline__ T Gx(int b, int s, int t) const {
     if (s >= S) return 0;
     if (rnnt_type == K2AMD_REGULAR && boundary != nullptr && boundary[4 * b + 3] == t) return 0;
     const int T1 = rnnt_type == K2AMD_REGULAR ? Tn + 1 : Tn;
-    return px_grad[((size_t)b * S + s) * T1 + t];
+    return MulRounded(px_grad[((size_t)b * S + s) * T1 + t], Scale(b));
   }
   __device__ __forceinline__ T Gy(int b, int s, int t) const {
-    T g = py_grad[((size_t)b * (S + 1) + s) * Tn + t];
+    T g = MulRounded(py_grad[((size_t)b * (S + 1) + s) * Tn + t], Scale(b));
     if (rnnt_type == K2AMD_CONSTRAINED && s >= 1) g += Gx(b, s - 1, t);
     return g;
   }
@@ -814,12 +816,12 @@ int SimpleForward(const T *lm, const T *am, const int64_t *symbols, const int64_
 }
 
 template <typename T>
-int SimpleBackward(const T *px_grad, const T *py_grad, const int64_t *symbols,
+int SimpleBackward(const T *px_grad, const T *py_grad, const T *seq_scale, const int64_t *symbols,
                    const int64_t *boundary, const T *lm_probs, const T *am_probs, const T *denom,
                    T *lm_grad, T *am_grad, T *q, int B, int S, int Tn, int C, int blank,
                    int rnnt_type, hipStream_t st) {
   if (B == 0) return K2AMD_OK;
-  GradView<T> gv{px_grad, py_grad, boundary, S, Tn, rnnt_type};
+  GradView<T> gv{px_grad, py_grad, seq_scale, boundary, S, Tn, rnnt_type};
   if (Tn > 0) {
     hipLaunchKernelGGL(QKernel<T>, dim3(512), dim3(256), 0, st, gv, denom, q, B);
     {  // lm_grad[b][s][c] = -lm_probs * sum_t q[b][s][t] * am_probs[b][t][c]
@@ -874,7 +876,7 @@ int k2amd_rnnt_logprobs_simple_forward(const void *lm, const void *am, const int
 }
 
 int k2amd_rnnt_logprobs_simple_backward(const void *px_grad, const void *py_grad,
-                                        const int64_t *symbols, const int64_t *boundary,
+                                        const void *seq_scale, const int64_t *symbols, const int64_t *boundary,
                                         const void *lm_probs, const void *am_probs,
                                         const void *denom, void *lm_grad, void *am_grad,
                                         void *q_scratch, int B, int S, int T, int C,
@@ -883,8 +885,8 @@ int k2amd_rnnt_logprobs_simple_backward(const void *px_grad, const void *py_grad
   if (!ArgsOk(B, S, T, C, termination_symbol, rnnt_type, dtype)) return K2AMD_ERR_INVALID_ARGUMENT;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == K2AMD_F32)
-    return SimpleBackward<float>((const float *)px_grad, (const float *)py_grad, symbols, boundary, (const float *)lm_probs, (const float *)am_probs, (const float *)denom, (float *)lm_grad, (float *)am_grad, (float *)q_scratch, B, S, T, C, termination_symbol, rnnt_type, st);
-  return SimpleBackward<double>((const double *)px_grad, (const double *)py_grad, symbols, boundary, (const double *)lm_probs, (const double *)am_probs, (const double *)denom, (double *)lm_grad, (double *)am_grad, (double *)q_scratch, B, S, T, C, termination_symbol, rnnt_type, st);
+    return SimpleBackward<float>((const float *)px_grad, (const float *)py_grad, (const float *)seq_scale, symbols, boundary, (const float *)lm_probs, (const float *)am_probs, (const float *)denom, (float *)lm_grad, (float *)am_grad, (float *)q_scratch, B, S, T, C, termination_symbol, rnnt_type, st);
+  return SimpleBackward<double>((const double *)px_grad, (const double *)py_grad, (const double *)seq_scale, symbols, boundary, (const double *)lm_probs, (const double *)am_probs, (const double *)denom, (double *)lm_grad, (double *)am_grad, (double *)q_scratch, B, S, T, C, termination_symbol, rnnt_type, st);
 }
 
 }  // extern "C"

@@ -99,14 +99,17 @@ def logprobs_simple_forward(lm, am, symbols, termination_symbol, rnnt_type, boun
 
 
 def logprobs_simple_backward(px_grad, py_grad, symbols, boundary, saved, termination_symbol,
-                             rnnt_type):
+                             rnnt_type, seq_scale=None):
+    """``seq_scale`` [B] or None (also in the two *_backward functions below): px_grad[b] and
+    py_grad[b] count as multiplied by seq_scale[b]."""
     _require_device(px_grad)
     if _ext is not None:
         lm_probs, am_probs, denom = saved
         return tuple(_ext.logprobs_simple_backward(px_grad, py_grad, symbols, boundary, lm_probs,
-                                                   am_probs, denom, termination_symbol, rnnt_type))
+                                                   am_probs, denom, termination_symbol, rnnt_type,
+                                                   seq_scale))
     return capi.logprobs_simple_backward(px_grad, py_grad, symbols, boundary, saved,
-                                         termination_symbol, rnnt_type)
+                                         termination_symbol, rnnt_type, seq_scale)
 
 
 def logprobs_joint_forward(logits, symbols, termination_symbol, rnnt_type, boundary):
@@ -118,12 +121,12 @@ def logprobs_joint_forward(logits, symbols, termination_symbol, rnnt_type, bound
 
 
 def logprobs_joint_backward(logits, norm, px_grad, py_grad, symbols, boundary, termination_symbol,
-                            rnnt_type):
+                            rnnt_type, seq_scale=None):
     if _ext is not None:
         return _ext.logprobs_joint_backward(logits, norm, px_grad, py_grad, symbols, boundary,
-                                            termination_symbol, rnnt_type)
+                                            termination_symbol, rnnt_type, seq_scale)
     return capi.logprobs_joint_backward(logits, norm, px_grad, py_grad, symbols, boundary,
-                                        termination_symbol, rnnt_type)
+                                        termination_symbol, rnnt_type, seq_scale)
 
 
 def logprobs_pruned_forward(logits, symbols, ranges, termination_symbol, boundary, rnnt_type,
@@ -137,12 +140,12 @@ def logprobs_pruned_forward(logits, symbols, ranges, termination_symbol, boundar
 
 
 def logprobs_pruned_backward(logits, norm, px_grad, py_grad, symbols, ranges, boundary,
-                             termination_symbol, rnnt_type, hat=False):
+                             termination_symbol, rnnt_type, hat=False, seq_scale=None):
     if _ext is not None:
         return _ext.logprobs_pruned_backward(logits, norm, px_grad, py_grad, symbols, ranges,
-                                             boundary, termination_symbol, rnnt_type, hat)
+                                             boundary, termination_symbol, rnnt_type, hat, seq_scale)
     return capi.logprobs_pruned_backward(logits, norm, px_grad, py_grad, symbols, ranges, boundary,
-                                         termination_symbol, rnnt_type, hat)
+                                         termination_symbol, rnnt_type, hat, seq_scale)
 
 
 def prune_ranges(px_grad, py_grad, boundary, s_range):

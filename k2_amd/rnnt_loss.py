@@ -106,6 +106,70 @@ class _LogprobsPruned(torch.autograd.Function):
         return grad, None, None, None, None, None, None
 
 
+class _Scores(torch.autograd.Function):
+    """A builder above and the recursion on its px, py as ONE autograd node, for the loss functions:
+    scores [B] straight from lm / am (``kind`` "simple") or logits ("joint", "pruned").  The
+    recursion has the occupation probabilities ready when it returns (as the reference's does,
+    k2/python/k2/mutual_information.py:162-169); what arrives at the scores in the backward pass
+    scales them per sequence inside the builder's gradient kernels (``seq_scale``), where the
+    reference runs two elementwise products first (mutual_information.py:177-182).  Returns
+    (scores, px_grad, py_grad); the last two are None unless asked for or needed."""
+
+    @staticmethod
+    def forward(ctx, kind, rnnt_type, delay_penalty, return_grad, *args):
+        boundary = args[5] if kind != "joint" else args[4]
+        need = return_grad or any(ctx.needs_input_grad)
+        # no zero tensors for the gradients of px_grad / py_grad, which nothing differentiates
+        ctx.set_materialize_grads(False)
+        if kind == "simple":
+            lm, am, symbols, termination_symbol, rnnt_code, _ = args
+            px, py, saved = native.logprobs_simple_forward(lm.contiguous(), am.contiguous(), symbols,
+                                                         termination_symbol, rnnt_code, boundary)
+        elif kind == "joint":
+            logits, symbols, termination_symbol, rnnt_code, _ = args
+            logits = logits.contiguous()
+            px, py, norm = native.logprobs_joint_forward(logits, symbols, termination_symbol,
+                                                         rnnt_code, boundary)
+            saved = (logits, norm)
+        else:
+            logits, symbols, ranges, termination_symbol, rnnt_code, _, hat = args
+            logits = logits.contiguous()
+            px, py, norm = native.logprobs_pruned_forward(logits, symbols, ranges,
+                                                          termination_symbol, boundary, rnnt_code, hat)
+            saved = (logits, norm)
+        if delay_penalty > 0.0:
+            px = _delay_penalty(px, boundary, rnnt_type, delay_penalty)
+        out = mutual_information_recursion(px=px, py=py, boundary=boundary, return_grad=need)
+        scores, (px_grad, py_grad) = out if need else (out, (None, None))
+        ctx.kind, ctx.args, ctx.n_saved = kind, args, len(saved)
+        if need:
+            ctx.save_for_backward(*saved, px_grad, py_grad)
+            ctx.mark_non_differentiable(px_grad, py_grad)
+        return scores, px_grad, py_grad
+
+    @staticmethod
+    def backward(ctx, scores_grad, _px_grad_grad, _py_grad_grad):
+        args = ctx.args
+        if scores_grad is None:
+            return (None,) * (4 + len(args))
+        saved, (px_grad, py_grad) = ctx.saved_tensors[:ctx.n_saved], ctx.saved_tensors[ctx.n_saved:]
+        scale = scores_grad.contiguous()
+        if ctx.kind == "simple":
+            _, _, symbols, termination_symbol, rnnt_code, boundary = args
+            grads = native.logprobs_simple_backward(px_grad, py_grad, symbols, boundary, saved,
+                                                    termination_symbol, rnnt_code, scale)
+        elif ctx.kind == "joint":
+            _, symbols, termination_symbol, rnnt_code, boundary = args
+            grads = (native.logprobs_joint_backward(saved[0], saved[1], px_grad, py_grad, symbols,
+                                                    boundary, termination_symbol, rnnt_code, scale),)
+        else:
+            _, symbols, ranges, termination_symbol, rnnt_code, boundary, hat = args
+            grads = (native.logprobs_pruned_backward(saved[0], saved[1], px_grad, py_grad, symbols,
+                                                     ranges, boundary, termination_symbol, rnnt_code,
+                                                     hat, scale),)
+        return (None, None, None, None) + tuple(grads) + (None,) * (len(args) - len(grads))
+
+
 class _PruneGather(torch.autograd.Function):
     @staticmethod
     def forward(ctx, lm, ranges):
@@ -129,6 +193,13 @@ def get_rnnt_logprobs(
 ) -> Tuple[Tensor, Tensor]:
     """k2.get_rnnt_logprobs (k2/python/k2/rnnt_loss.py:65-225): lm [B][S+1][C], am [B][T][C],
     symbols [B][S] -> px [B][S][T+1 or T], py [B][S+1][T] for mutual_information_recursion."""
+    return _LogprobsSimple.apply(*_simple_args(lm, am, symbols, termination_symbol, rnnt_type,
+                                               boundary))
+
+
+def _simple_args(lm, am, symbols, termination_symbol, rnnt_type, boundary):
+    """The reference's checks (k2/python/k2/rnnt_loss.py:159-170) and the arguments of
+    _LogprobsSimple."""
     assert lm.ndim == 3, lm.shape
     assert am.ndim == 3, am.shape
     assert lm.shape[0] == am.shape[0], (lm.shape, am.shape)
@@ -138,8 +209,8 @@ def get_rnnt_logprobs(
     assert symbols.shape == (B, S), (symbols.shape, B, S)
     assert rnnt_type in _RNNT_TYPES, rnnt_type
     _validate_st_lengths(S, T, rnnt_type == "regular", boundary)
-    return _LogprobsSimple.apply(lm, am, _dev_i64(symbols, am), int(termination_symbol),
-                                 capi.RNNT_TYPES[rnnt_type], _dev_i64(boundary, am))
+    return (lm, am, _dev_i64(symbols, am), int(termination_symbol), capi.RNNT_TYPES[rnnt_type],
+            _dev_i64(boundary, am))
 
 
 def _delay_penalty(px: Tensor, boundary: Optional[Tensor], rnnt_type: str,
@@ -179,16 +250,11 @@ def rnnt_loss_simple(
     return_grad: bool = False,
 ) -> Union[Tensor, Tuple[Tensor, Tuple[Tensor, Tensor]]]:
     """k2.rnnt_loss_simple (k2/python/k2/rnnt_loss.py:228-338)."""
-    px, py = get_rnnt_logprobs(lm=lm, am=am, symbols=symbols,
-                               termination_symbol=termination_symbol, boundary=boundary,
-                               rnnt_type=rnnt_type)
-    if delay_penalty > 0.0:
-        px = _delay_penalty(px, boundary, rnnt_type, delay_penalty)
-    scores_and_grads = mutual_information_recursion(px=px, py=py, boundary=boundary,
-                                                    return_grad=return_grad)
-    negated_loss = scores_and_grads[0] if return_grad else scores_and_grads
+    args = _simple_args(lm, am, symbols, termination_symbol, rnnt_type, boundary)
+    negated_loss, px_grad, py_grad = _Scores.apply("simple", rnnt_type, float(delay_penalty),
+                                                   bool(return_grad), *args)
     loss = _reduce(negated_loss, reduction)
-    return (loss, scores_and_grads[1]) if return_grad else loss
+    return (loss, (px_grad, py_grad)) if return_grad else loss
 
 
 def get_rnnt_logprobs_joint(
@@ -199,14 +265,20 @@ def get_rnnt_logprobs_joint(
     boundary: Optional[Tensor] = None,
 ) -> Tuple[Tensor, Tensor]:
     """k2.get_rnnt_logprobs_joint (k2/python/k2/rnnt_loss.py:341-447): logits [B][T][S+1][C]."""
+    return _LogprobsJoint.apply(*_joint_args(logits, symbols, termination_symbol, rnnt_type, boundary))
+
+
+def _joint_args(logits, symbols, termination_symbol, rnnt_type, boundary):
+    """The reference's checks (k2/python/k2/rnnt_loss.py:400-408) and the arguments of
+    _LogprobsJoint."""
     assert logits.ndim == 4, logits.shape
     (B, T, S1, C) = logits.shape
     S = S1 - 1
     assert symbols.shape == (B, S), (symbols.shape, B, S)
     assert rnnt_type in _RNNT_TYPES, rnnt_type
     _validate_st_lengths(S, T, rnnt_type == "regular", boundary)
-    return _LogprobsJoint.apply(logits, _dev_i64(symbols, logits), int(termination_symbol),
-                                capi.RNNT_TYPES[rnnt_type], _dev_i64(boundary, logits))
+    return (logits, _dev_i64(symbols, logits), int(termination_symbol), capi.RNNT_TYPES[rnnt_type],
+            _dev_i64(boundary, logits))
 
 
 def rnnt_loss(
@@ -219,12 +291,8 @@ def rnnt_loss(
     reduction: Optional[str] = "mean",
 ) -> Tensor:
     """k2.rnnt_loss (k2/python/k2/rnnt_loss.py:450-540)."""
-    px, py = get_rnnt_logprobs_joint(logits=logits, symbols=symbols,
-                                     termination_symbol=termination_symbol, boundary=boundary,
-                                     rnnt_type=rnnt_type)
-    if delay_penalty > 0.0:
-        px = _delay_penalty(px, boundary, rnnt_type, delay_penalty)
-    negated_loss = mutual_information_recursion(px=px, py=py, boundary=boundary)
+    args = _joint_args(logits, symbols, termination_symbol, rnnt_type, boundary)
+    negated_loss = _Scores.apply("joint", rnnt_type, float(delay_penalty), False, *args)[0]
     return _reduce(negated_loss, reduction)
 
 
@@ -322,15 +390,21 @@ def get_rnnt_logprobs_pruned(
 ) -> Tuple[Tensor, Tensor]:
     """k2.get_rnnt_logprobs_pruned (k2/python/k2/rnnt_loss.py:1180-1348): logits
     [B][T][s_range][C], ranges [B][T][s_range]."""
+    return _LogprobsPruned.apply(*_pruned_args(logits, symbols, ranges, termination_symbol, boundary,
+                                               rnnt_type))
+
+
+def _pruned_args(logits, symbols, ranges, termination_symbol, boundary, rnnt_type):
+    """The reference's checks (k2/python/k2/rnnt_loss.py:1243-1251) and the arguments of
+    _LogprobsPruned."""
     assert logits.ndim == 4, logits.shape
     (B, T, s_range, C) = logits.shape
     assert ranges.shape == (B, T, s_range), (ranges.shape, B, T, s_range)
     (B, S) = symbols.shape
     assert rnnt_type in _RNNT_TYPES, rnnt_type
     _validate_st_lengths(S, T, rnnt_type == "regular", boundary)
-    return _LogprobsPruned.apply(logits, _dev_i64(symbols, logits), _dev_i64(ranges, logits),
-                                 int(termination_symbol), capi.RNNT_TYPES[rnnt_type],
-                                 _dev_i64(boundary, logits))
+    return (logits, _dev_i64(symbols, logits), _dev_i64(ranges, logits), int(termination_symbol),
+            capi.RNNT_TYPES[rnnt_type], _dev_i64(boundary, logits), False)
 
 
 def get_hat_logprobs_pruned(
@@ -344,6 +418,13 @@ def get_hat_logprobs_pruned(
     """k2.get_hat_logprobs_pruned (k2/python/k2/rnnt_loss.py:992-1177), the hybrid autoregressive
     transducer: the blank (column 0) has its own sigmoid, py = logsigmoid(logits[..., 0]), and the
     other symbols share a softmax over columns 1..C-1 scaled by 1 - sigmoid(logits[..., 0])."""
+    return _LogprobsPruned.apply(*_hat_args(logits, symbols, ranges, termination_symbol, boundary,
+                                            rnnt_type))
+
+
+def _hat_args(logits, symbols, ranges, termination_symbol, boundary, rnnt_type):
+    """The reference's checks (k2/python/k2/rnnt_loss.py:1056-1069) and the arguments of
+    _LogprobsPruned."""
     assert logits.ndim == 4, logits.shape
     (B, T, s_range, C) = logits.shape
     assert ranges.shape == (B, T, s_range), (ranges.shape, B, T, s_range)
@@ -354,8 +435,8 @@ def get_hat_logprobs_pruned(
     assert rnnt_type in _RNNT_TYPES, rnnt_type
     assert termination_symbol == 0, \
         f"Termination symbol must be 0, but got {termination_symbol}"
-    return _LogprobsPruned.apply(logits, _dev_i64(symbols, logits), _dev_i64(ranges, logits), 0,
-                                 capi.RNNT_TYPES[rnnt_type], _dev_i64(boundary, logits), True)
+    return (logits, _dev_i64(symbols, logits), _dev_i64(ranges, logits), 0,
+            capi.RNNT_TYPES[rnnt_type], _dev_i64(boundary, logits), True)
 
 
 def rnnt_loss_pruned(
@@ -371,13 +452,9 @@ def rnnt_loss_pruned(
 ) -> Tensor:
     """k2.rnnt_loss_pruned (k2/python/k2/rnnt_loss.py:1351-1468); ``use_hat_loss`` switches the
     builder to get_hat_logprobs_pruned (:1430-1447)."""
-    builder = get_hat_logprobs_pruned if use_hat_loss else get_rnnt_logprobs_pruned
-    px, py = builder(logits=logits, symbols=symbols, ranges=ranges,
-                     termination_symbol=termination_symbol, boundary=boundary,
-                     rnnt_type=rnnt_type)
-    if delay_penalty > 0.0:
-        px = _delay_penalty(px, boundary, rnnt_type, delay_penalty)
-    negated_loss = mutual_information_recursion(px=px, py=py, boundary=boundary)
+    checked = _hat_args if use_hat_loss else _pruned_args
+    args = checked(logits, symbols, ranges, termination_symbol, boundary, rnnt_type)
+    negated_loss = _Scores.apply("pruned", rnnt_type, float(delay_penalty), False, *args)[0]
     return _reduce(negated_loss, reduction)
 
 

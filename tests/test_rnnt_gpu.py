@@ -501,3 +501,83 @@ def test_simple_gradients_with_often_repeated_symbols(device, rnnt_type):
     np.testing.assert_allclose(grads[torch.float64][2], am_r.grad.numpy(), rtol=1e-8, atol=1e-10)
     for a, b in zip(grads[torch.float32], grads[torch.float64]):
         np.testing.assert_allclose(a, b, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("rnnt_type", ["regular", "modified", "constrained"])
+def test_loss_nodes_equal_the_builder_then_recursion_chain(device, rnnt_type):
+    """The loss functions run builder + recursion as one autograd node and scale the gradients per
+    sequence inside the builders' gradient kernels; chaining the public builder, the public
+    recursion and torch's own products (what the reference does, k2/python/k2/rnnt_loss.py:
+    300-338, 520-540, 1430-1468) must give the same bits: per-sequence losses, gradients under
+    arbitrary per-sequence weights, with a delay penalty, and the returned occupation
+    probabilities."""
+    import k2_amd as k2
+    from k2_amd.rnnt_loss import _delay_penalty
+    B, T, S, C, R = 5, 37, 11, 23, 4
+    c = cases.rnnt_case(41, B, T, S, C, t_lo=20, s_lo=5, modified=rnnt_type != "regular")
+    sym = torch.from_numpy(c["symbols"]).to(device)
+    bd = torch.from_numpy(c["boundary"]).to(device)
+    w = torch.tensor([0.3, -1.7, 2.0, 0.0, 1.0], device=device)
+    rng = np.random.default_rng(7)
+
+    def leaf(shape):
+        return torch.from_numpy(rng.standard_normal(shape).astype(np.float32)).to(device).requires_grad_(True)
+
+    def compare(node, chain, leaves):
+        for fn, out in ((node, []), (chain, [])):
+            pass
+        results = []
+        for fn in (node, chain):
+            for x in leaves:
+                x.grad = None
+            loss = fn()
+            (loss * w).sum().backward()
+            results.append((loss.detach().clone(), [x.grad.clone() for x in leaves]))
+        assert torch.equal(results[0][0], results[1][0])
+        for a, b in zip(results[0][1], results[1][1]):
+            assert torch.equal(a, b)
+
+    for penalty in (0.0, 0.01):
+        lm, am = leaf((B, S + 1, C)), leaf((B, T, C))
+
+        def chain_simple():
+            px, py = k2.get_rnnt_logprobs(lm, am, sym, 0, rnnt_type, bd)
+            if penalty:
+                px = _delay_penalty(px, bd, rnnt_type, penalty)
+            return -k2.mutual_information_recursion(px, py, bd)
+        compare(lambda: k2.rnnt_loss_simple(lm, am, sym, 0, bd, rnnt_type, penalty, "none"),
+                chain_simple, [lm, am])
+
+        logits = leaf((B, T, S + 1, C))
+
+        def chain_joint():
+            px, py = k2.get_rnnt_logprobs_joint(logits, sym, 0, rnnt_type, bd)
+            if penalty:
+                px = _delay_penalty(px, bd, rnnt_type, penalty)
+            return -k2.mutual_information_recursion(px, py, bd)
+        compare(lambda: k2.rnnt_loss(logits, sym, 0, bd, rnnt_type, penalty, "none"), chain_joint, [logits])
+
+        _, (gx, gy) = k2.rnnt_loss_simple(lm.detach(), am.detach(), sym, 0, bd, rnnt_type, 0.0, "sum",
+                                          return_grad=True)
+        ranges = k2.get_rnnt_prune_ranges(gx, gy, bd, R)
+        pruned = leaf((B, T, R, C))
+        for hat, builder in ((False, k2.get_rnnt_logprobs_pruned), (True, k2.get_hat_logprobs_pruned)):
+            def chain_pruned():
+                px, py = builder(pruned, sym, ranges, 0, bd, rnnt_type)
+                if penalty:
+                    px = _delay_penalty(px, bd, rnnt_type, penalty)
+                return -k2.mutual_information_recursion(px, py, bd)
+            compare(lambda: k2.rnnt_loss_pruned(pruned, sym, ranges, 0, bd, rnnt_type, penalty, "none", hat),
+                    chain_pruned, [pruned])
+
+    # return_grad hands out the same occupation probabilities as the recursion does
+    lm, am = leaf((B, S + 1, C)), leaf((B, T, C))
+    loss, (gx, gy) = k2.rnnt_loss_simple(lm, am, sym, 0, bd, rnnt_type, 0.0, "sum", return_grad=True)
+    px, py = k2.get_rnnt_logprobs(lm, am, sym, 0, rnnt_type, bd)
+    scores, (hx, hy) = k2.mutual_information_recursion(px, py, bd, return_grad=True)
+    assert torch.equal(gx, hx) and torch.equal(gy, hy) and torch.equal(loss, -scores.sum())
+    assert not gx.requires_grad and not gy.requires_grad
+    # and without gradients nothing of the backward machinery runs
+    with torch.no_grad():
+        plain = k2.rnnt_loss_simple(lm, am, sym, 0, bd, rnnt_type, 0.0, "none")
+    assert torch.equal(plain, -scores.detach()) and not plain.requires_grad
