@@ -108,7 +108,8 @@ K2AMD_API int k2amd_mi_backward_kept(const void *px, const void *py, const int64
  * autograd function does with two native calls when gradients are wanted
  * (k2/python/k2/mutual_information.py:157-169).  It has no counterpart in the reference.
  *   ans [B] out; log_deriv [B][S+1][T+1] scratch (written, then read; contents as above);
- *   ans_grad [B] in (and out if overwrite_ans_grad); px_grad, py_grad out, every element written.
+ *   ans_grad [B] in (and out if overwrite_ans_grad), or NULL for the reference's torch.ones(B)
+ *   (mutual_information.py:163); px_grad, py_grad out, every element written.
  * Same results, bit for bit, as the two calls.  Every workgroup of this launch must be resident
  * at once, so it only serves shapes with 2 * B * ceil((S+1)/64) <= compute units of the current
  * device, fp32, with a workspace: k2amd_mi_forward_backward_supported(...) says whether a call

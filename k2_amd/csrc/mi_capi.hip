@@ -149,7 +149,7 @@ int k2amd_mi_forward_backward(const void *px, const void *py, const int64_t *bou
                               void *workspace, size_t workspace_bytes, void *stream) {
   if (!ShapeOk(B, S, T) || (dtype != K2AMD_F32 && dtype != K2AMD_F64)) return K2AMD_ERR_INVALID_ARGUMENT;
   if (B == 0) return K2AMD_OK;
-  if (!ans || !log_deriv || !ans_grad || (!px && S > 0) || (!py && T > 0) || (!px_grad && S > 0) ||
+  if (!ans || !log_deriv || (!px && S > 0) || (!py && T > 0) || (!px_grad && S > 0) ||
       (!py_grad && T > 0))
     return K2AMD_ERR_INVALID_ARGUMENT;
   if (!k2amd_mi_forward_backward_supported(B, S, T, modified, dtype, workspace != nullptr))

@@ -983,7 +983,8 @@ __device__ __forceinline__ void MiBackwardChunk(
   // ---- chain wavefront ---------------------------------------------------------------------
   // gradient at the (virtual) right end of each row: the seed on the sequence's last row
   float G = 0.0f;
-  if (role == kChain && g.row0 + lane == g.ns) G = ans_grad[g.b];
+  // (the single launch may come without ans_grad: every sequence's score then has gradient 1)
+  if (role == kChain && g.row0 + lane == g.ns) G = ans_grad != nullptr ? ans_grad[g.b] : 1.0f;
   float g_origin = 0.0f;
   // Per position (descending), with OME of the own row and Edn = d1 of the row below (lane + 1):
   //     G' = OME * G + Edn * G(lane + 1)
@@ -1071,7 +1072,8 @@ __device__ __forceinline__ void MiBackwardChunk(
   }
   if (role == kStorer) store_block(0);
   if (role == kEdge) publish_block(0);
-  if (overwrite_ans_grad && role == kChain && g.c == 0 && lane == 0) ans_grad[g.b] = g_origin;
+  if (overwrite_ans_grad && ans_grad != nullptr && role == kChain && g.c == 0 && lane == 0)
+    ans_grad[g.b] = g_origin;
 }
 
 // The first B * nchunks tickets sweep, lower chunks first; the rest of the grid (as many again)

@@ -207,7 +207,7 @@ bool MutualInformationForwardBackwardSupported(torch::Tensor px, torch::Tensor p
 // and overwrites ans_grad like MutualInformationBackward.
 std::vector<torch::Tensor> MutualInformationForwardBackward(torch::Tensor px, torch::Tensor py,
                                                             torch::optional<torch::Tensor> boundary,
-                                                            torch::Tensor ans_grad) {
+                                                            torch::optional<torch::Tensor> ans_grad) {
   TORCH_CHECK(px.dim() == 3 && py.dim() == 3, "px and py must have three dimensions");
   TORCH_CHECK(px.is_cuda(), "k2_amd runs on MI355X only: px is on ", px.device(),
               " (there is no CPU path)");
@@ -215,10 +215,14 @@ std::vector<torch::Tensor> MutualInformationForwardBackward(torch::Tensor px, to
   // scratch with p's shape: the forward sweep leaves the px-edge log-derivatives there
   torch::Tensor log_deriv = torch::empty({px.size(0), px.size(1) + 1, py.size(2) + 1}, px.options());
   const Shape sh = CheckInputs(px, py, boundary, log_deriv);
-  TORCH_CHECK(ans_grad.dim() == 1 && ans_grad.size(0) == sh.B, "ans_grad must have shape [B]");
-  TORCH_CHECK(ans_grad.device() == px.device() && ans_grad.scalar_type() == px.scalar_type(),
-              "ans_grad must match px in device and dtype");
-  TORCH_CHECK(ans_grad.is_contiguous(), "ans_grad must be contiguous");
+  void *seed = nullptr;  // None: every score has gradient 1
+  if (ans_grad.has_value() && ans_grad->defined()) {
+    TORCH_CHECK(ans_grad->dim() == 1 && ans_grad->size(0) == sh.B, "ans_grad must have shape [B]");
+    TORCH_CHECK(ans_grad->device() == px.device() && ans_grad->scalar_type() == px.scalar_type(),
+                "ans_grad must match px in device and dtype");
+    TORCH_CHECK(ans_grad->is_contiguous(), "ans_grad must be contiguous");
+    seed = ans_grad->data_ptr();
+  }
   px = px.contiguous();
   py = py.contiguous();
   torch::Tensor bd;
@@ -233,7 +237,7 @@ std::vector<torch::Tensor> MutualInformationForwardBackward(torch::Tensor px, to
     pybind11::gil_scoped_release release;
     Check(k2amd_mi_forward_backward(px.data_ptr(), py.data_ptr(),
                                     bd.defined() ? bd.data_ptr<int64_t>() : nullptr, ans.data_ptr(),
-                                    log_deriv.data_ptr(), ans_grad.data_ptr(), px_grad.data_ptr(),
+                                    log_deriv.data_ptr(), seed, px_grad.data_ptr(),
                                     py_grad.data_ptr(), sh.B, sh.S, sh.T, sh.modified, dt,
                                     /*overwrite_ans_grad=*/1, ws.defined() ? ws.data_ptr() : nullptr,
                                     ws.defined() ? static_cast<size_t>(ws.numel()) : 0, stream));

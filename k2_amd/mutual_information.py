@@ -75,9 +75,8 @@ class MutualInformationRecursionFunction(torch.autograd.Function):
         want_grad = return_grad or px.requires_grad or py.requires_grad
         px_grad, py_grad = None, None
         if want_grad and _single_launch(px, py):
-            # both recursions in one launch
-            ans_grad = torch.ones(B, device=px.device, dtype=px.dtype)
-            (ans, px_grad, py_grad) = native.mutual_information_forward_backward(px, py, boundary, ans_grad)
+            # both recursions in one launch, seeded with 1 per sequence
+            (ans, px_grad, py_grad) = native.mutual_information_forward_backward(px, py, boundary, None)
         else:
             # the backward runs right away, so the forward can hand it the px-edge log-derivatives
             # instead of p (which nothing else reads)
@@ -164,11 +163,11 @@ def joint_mutual_information_recursion(
     py_cat = torch.stack(list(py), dim=0)  # [N][B][S+1][T]
     px_tot = px_cat.sum(dim=0).contiguous()
     py_tot = py_cat.sum(dim=0).contiguous()
-    ans_grad = torch.ones(B, device=px_tot.device, dtype=px_tot.dtype)
     if _single_launch(px_tot, py_tot):
         (tot_probs, px_grad, py_grad) = native.mutual_information_forward_backward(
-            px_tot, py_tot, boundary, ans_grad)
+            px_tot, py_tot, boundary, None)
     else:
+        ans_grad = torch.ones(B, device=px_tot.device, dtype=px_tot.dtype)
         p, log_deriv = _lattice_buffers(px_tot, py_tot, True)
         tot_probs = native.mutual_information_forward(px_tot, py_tot, boundary, p, log_deriv)
         (px_grad, py_grad) = native.mutual_information_backward(px_tot, py_tot, boundary, p, ans_grad,

@@ -73,10 +73,11 @@ def mutual_information_forward_backward_supported(px: torch.Tensor, py: torch.Te
 
 def mutual_information_forward_backward(px: torch.Tensor, py: torch.Tensor,
                                         boundary: Optional[torch.Tensor],
-                                        ans_grad: torch.Tensor) -> List[torch.Tensor]:
+                                        ans_grad: Optional[torch.Tensor]) -> List[torch.Tensor]:
     """mutual_information_forward followed by mutual_information_backward in one launch, as the
     reference's autograd function calls them (k2/python/k2/mutual_information.py:157-169):
-    returns [ans, px_grad, py_grad] and overwrites ``ans_grad``."""
+    returns [ans, px_grad, py_grad] and overwrites ``ans_grad``; ``ans_grad`` None stands for the
+    reference's torch.ones(B)."""
     _require_device(px)
     if _ext is not None:
         return _ext.mutual_information_forward_backward(px, py, boundary, ans_grad)

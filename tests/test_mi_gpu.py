@@ -65,6 +65,11 @@ def run_gpu(px, py, bd, device, ans_grad=None):
         capi.mi_workspace_status(device)
         for name, x, y in (("ans", ans4, ans), ("px_grad", gx4, gx), ("py_grad", gy4, gy), ("ans_grad", g4, g)):
             assert torch.equal(x.view(torch.int32), y.view(torch.int32)), "single launch differs in " + name
+        if ans_grad is None:  # no seed tensor at all stands for ones
+            ans5, gx5, gy5 = capi.mi_forward_backward(tpx, tpy, tbd, None)
+            torch.cuda.synchronize()
+            for name, x, y in (("ans", ans5, ans), ("px_grad", gx5, gx), ("py_grad", gy5, gy)):
+                assert torch.equal(x.view(torch.int32), y.view(torch.int32)), "seedless single launch differs in " + name
     return ans.cpu().numpy(), p.cpu().numpy(), gx.cpu().numpy(), gy.cpu().numpy(), g.cpu().numpy(), g_in.cpu().numpy()
 
 
