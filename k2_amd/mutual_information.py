@@ -13,24 +13,32 @@ from torch import Tensor
 from . import native
 
 
-# boundary tensors whose values passed the range asserts: id(tensor) -> (weak reference, verdict key)
-_checked_boundaries = {}
+# host copies of boundary tensors: id(tensor) -> (weak reference, version counter, rows)
+_boundary_copies = {}
+
+
+def boundary_rows(boundary: Tensor) -> Tuple[Tuple[int, int, int, int], ...]:
+    """The rows (s_begin, t_begin, s_end, t_end) of a [B][4] boundary tensor as Python integers.
+    Reading them from a device tensor is a copy that waits for everything queued on the stream,
+    and the reference pays it in each of its checks (k2/python/k2/mutual_information.py:284-289,
+    k2/python/k2/rnnt_loss.py:46-62 and 699-705).  Here the copy is kept per tensor object and
+    reused by all of them while the tensor has not been written to (its version counter); a new
+    tensor is always read."""
+    ident = id(boundary)
+    hit = _boundary_copies.get(ident)
+    if hit is not None and hit[0]() is boundary and hit[1] == boundary._version:
+        return hit[2]
+    rows = tuple(tuple(r) for r in boundary.tolist())
+    _boundary_copies[ident] = (weakref.ref(boundary, lambda _, i=ident: _boundary_copies.pop(i, None)),
+                               boundary._version, rows)
+    return rows
 
 
 def _check_boundary(boundary: Tensor, S: int, T: int) -> None:
-    """The range asserts of k2/python/k2/mutual_information.py:284-289.  Reading the values is a
-    device-to-host copy that waits for everything queued on the stream, so the verdict is kept
-    per tensor object and reused while the tensor has not been written to (its version counter)
-    and is checked against the same S and T; a new tensor is always read."""
-    ident = id(boundary)
-    key = (boundary._version, S, T)
-    hit = _checked_boundaries.get(ident)
-    if hit is not None and hit[0]() is boundary and hit[1] == key:
-        return
-    for s_begin, t_begin, s_end, t_end in boundary.tolist():
+    """The range asserts of k2/python/k2/mutual_information.py:284-289."""
+    for s_begin, t_begin, s_end, t_end in boundary_rows(boundary):
         assert 0 <= s_begin <= s_end <= S, (s_begin, s_end, S)
         assert 0 <= t_begin <= t_end <= T, (t_begin, t_end, T)
-    _checked_boundaries[ident] = (weakref.ref(boundary, lambda _, i=ident: _checked_boundaries.pop(i, None)), key)
 
 
 _single_launch_ok = {}

@@ -11,7 +11,7 @@ import torch
 from torch import Tensor
 
 from . import capi, native
-from .mutual_information import mutual_information_recursion
+from .mutual_information import boundary_rows, mutual_information_recursion
 
 _RNNT_TYPES = ("regular", "modified", "constrained")
 
@@ -41,10 +41,14 @@ def _validate_st_lengths(S: int, T: int, is_rnnt_type_regular: bool,
         assert is_rnnt_type_regular or T >= S, \
             f"Modified transducer requires T >= S, but got T={T} and S={S}"
     else:
-        Ss = boundary[:, 2]
-        Ts = boundary[:, 3]
-        assert is_rnnt_type_regular or bool((Ts >= Ss).all()), \
-            f"Modified transducer requires T >= S, but got T={Ts} and S={Ss}"
+        assert is_rnnt_type_regular or all(r[3] >= r[2] for r in boundary_rows(boundary)), \
+            f"Modified transducer requires T >= S, but got T={boundary[:, 3]} and S={boundary[:, 2]}"
+
+
+def _trunc_div(a: int, b: int) -> int:
+    """Integer quotient rounded towards zero, like torch.div(..., rounding_mode="trunc")."""
+    q = abs(a) // abs(b)
+    return q if (a < 0) == (b < 0) else -q
 
 
 class _LogprobsSimple(torch.autograd.Function):
@@ -332,12 +336,14 @@ def get_rnnt_prune_ranges(
     _validate_st_lengths(S, T, is_regular, boundary)
 
     if is_regular:
-        Ss = boundary[:, 2]
-        Ts = boundary[:, 3]
-        s_range_min = Ss.sub(1).div(Ts, rounding_mode="trunc").add(2).max().item()
+        # the smallest s_range that lets a path take all S_b symbols in T_b frames, as
+        # k2/python/k2/rnnt_loss.py:699-705 has it: max over b of trunc((S_b - 1) / T_b) + 2,
+        # from the host copy of the boundary (a sequence without frames asks for nothing)
+        s_range_min = max((_trunc_div(r[2] - 1, r[3]) + 2 for r in boundary_rows(boundary) if r[3] != 0),
+                          default=2)
         if s_range < s_range_min:
             print(f"Warning: get_rnnt_prune_ranges - got s_range={s_range} "
-                  f"for boundaries S={Ss}, T={Ts}. Adjusting to {s_range_min}")
+                  f"for boundaries S={boundary[:, 2]}, T={boundary[:, 3]}. Adjusting to {s_range_min}")
             s_range = s_range_min
     if s_range > S:
         print(f"Warning: get_rnnt_prune_ranges - got s_range={s_range} "

@@ -102,6 +102,27 @@ def test_prune_ranges_bit_exact(device, modified):
             assert np.array_equal(got.cpu().numpy(), want), (seed, R)
 
 
+def test_prune_ranges_widens_a_range_too_small_for_the_boundary(device, capsys):
+    """k2/python/k2/rnnt_loss.py:694-729: a regular lattice needs s_range >= (S_b - 1) / T_b + 2
+    for every sequence, and never more than S + 1 rows."""
+    import k2_amd as k2
+    B, T, S = 3, 6, 17
+    rng = np.random.default_rng(5)
+    boundary = np.array([[0, 0, 17, 4], [0, 0, 9, 6], [0, 0, 1, 3]], np.int64)
+    gx = rng.random((B, S, T + 1)).astype(np.float32)
+    gy = rng.random((B, S + 1, T)).astype(np.float32)
+    bd = dev(boundary, device)
+    for R, R_eff in ((2, 6), (6, 6), (7, 7), (18, 18), (40, 18)):
+        want = orn.prune_ranges(gx, gy, boundary, R)
+        assert want.shape == (B, T, R_eff)
+        got = k2.get_rnnt_prune_ranges(dev(gx, device), dev(gy, device), bd, R)
+        assert np.array_equal(got.cpu().numpy(), want), R
+        # the reference also prints when s_range is S + 1 already (rnnt_loss.py:711-716)
+        assert ("Adjusting" in capsys.readouterr().out) == (R != R_eff or R > S)
+    bd[0, 3] = 2                                            # written in place: read again
+    assert k2.get_rnnt_prune_ranges(dev(gx, device), dev(gy, device), bd, 2).shape[-1] == 10
+
+
 def test_prune_gather_and_its_gradient(device):
     from k2_amd import capi
     rng = np.random.default_rng(3)
