@@ -45,6 +45,7 @@
 // Arithmetic is the reference's log-domain recursion (k2/python/csrc/torch/
 // mutual_information_cpu.cu:89-121, log-add of k2/csrc/utils.h:511-563) with hardware exp2/log2.
 #include <atomic>
+#include <cstdlib>
 
 #include "common.h"
 #include "mi_internal.h"
@@ -1174,6 +1175,34 @@ int MiFastWorkspaceInit(void *workspace, size_t workspace_bytes, hipStream_t str
   return LaunchStatus();
 }
 
+// Compute units of the current device (asked once per device ordinal), or -1.
+static int ComputeUnits() {
+  static std::atomic<int> units[64];  // 0 = not asked yet
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return -1;
+  int n = units[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return -1;
+    n = n > 0 ? n : -1;
+    units[dev].store(n, std::memory_order_relaxed);  // every thread would store the same value
+  }
+  return n;
+}
+
+// LDS bytes to ask for beyond a kernel's own structure.  While the sweeping workgroups of a launch
+// find a compute unit each, every one gets a unit to itself (kExclusiveLds); once there are more
+// chunks than units the launch is bound by how many chains the device steps at a time, and two
+// workgroups share a unit.
+static size_t LdsPad(size_t own, long long sweepers) {
+  static const bool never_share = [] {
+    const char *e = getenv("K2AMD_MI_SHARE_UNITS");
+    return e != nullptr && e[0] == '0';
+  }();
+  const int n = ComputeUnits();
+  if (!never_share && n > 0 && sweepers > n) return 0;
+  return kExclusiveLds - own;
+}
+
 int MiForwardFast(const float *px, const float *py, const int64_t *boundary, float *p, float *ans,
                   float *log_deriv, int B, int S, int Tn, int modified, void *workspace,
                   size_t workspace_bytes, hipStream_t stream) {
@@ -1183,7 +1212,7 @@ int MiForwardFast(const float *px, const float *py, const int64_t *boundary, flo
   FastHeader *hdr = static_cast<FastHeader *>(workspace);
   float *edge = reinterpret_cast<float *>(hdr + 1);
   const dim3 grid((unsigned)(B * nchunks)), block(FwdLayout::kThreads);
-  const size_t pad = kExclusiveLds - sizeof(FwdLds);
+  const size_t pad = LdsPad(sizeof(FwdLds), (long long)B * nchunks);
   if (log_deriv == nullptr && p == nullptr) return K2AMD_ERR_INVALID_ARGUMENT;
   if (log_deriv != nullptr && p != nullptr)
     hipLaunchKernelGGL((MiForwardFastKernel<true, true>), grid, block, pad, stream, px, py, boundary, p, ans, log_deriv, hdr, edge, B, S, Tn, modified, nchunks, edge_stride);
@@ -1206,7 +1235,7 @@ int MiBackwardFast(const float *px, const float *p, const float *log_deriv,
   float *edge = reinterpret_cast<float *>(hdr + 1);
   // B * nchunks sweeping workgroups + as many that only clear
   const dim3 grid((unsigned)(2 * B * nchunks)), block(BwdLayout::kThreads);
-  const size_t pad = kExclusiveLds - sizeof(BwdLds);
+  const size_t pad = LdsPad(sizeof(BwdLds), (long long)B * nchunks);
   if (log_deriv != nullptr)
     hipLaunchKernelGGL(MiBackwardFastKernel<true>, grid, block, pad, stream, px, log_deriv, boundary, ans_grad, px_grad, py_grad, hdr, edge, B, S, Tn, modified, nchunks, edge_stride, overwrite_ans_grad);
   else
@@ -1218,15 +1247,7 @@ int MiBackwardFast(const float *px, const float *p, const float *log_deriv,
 // clearing ones, which never wait) must find a compute unit of its own at once.
 bool MiFusedSupports(int B, int S, int Tn, int modified) {
   if (!MiFastSupports(B, S, Tn, modified) || B < 1) return false;
-  static std::atomic<int> units[64];  // compute units per device ordinal, 0 = not asked yet
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
-  int n = units[dev].load(std::memory_order_relaxed);
-  if (n == 0) {
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return false;
-    n = n > 0 ? n : -1;
-    units[dev].store(n, std::memory_order_relaxed);  // every thread would store the same value
-  }
+  const int n = ComputeUnits();
   const long long nchunks = (S + 1 + kRows - 1) / kRows;
   return n > 0 && 2 * (long long)B * nchunks <= n;
 }

@@ -139,6 +139,20 @@ def test_wide_lattice_more_rows_than_a_wavefront(device, modified):
 
 
 @pytest.mark.parametrize("modified", [False, True])
+def test_more_chunks_than_compute_units(device, modified):
+    """B * ceil((S+1)/64) = 450 sweeping workgroups on 256 compute units: the pair of launches,
+    with two workgroups to a unit."""
+    rng = np.random.default_rng(77)
+    B, S, T = 150, 140, 170
+    px = rng.normal(-2, 1, (B, S, T if modified else T + 1)).astype(np.float32)
+    py = rng.normal(-2, 1, (B, S + 1, T)).astype(np.float32)
+    bd = cases.random_boundary(rng, B, S, T, modified)
+    ans, p = omi.mi_forward(px, py, bd)
+    gx, gy = omi.mi_backward(px, py, bd, p)
+    check("oversubscribed", px, py, bd, (ans, p, gx, gy), device)
+
+
+@pytest.mark.parametrize("modified", [False, True])
 def test_fp32_multi_chunk_and_block_edges(device, modified):
     """fp32 lattices taller than one 64-row chunk, with T chosen around multiples of the 32-step
     block so that chunk hand-over and the first/last block paths are all exercised."""
