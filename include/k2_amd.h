@@ -112,7 +112,8 @@ K2AMD_API int k2amd_mi_backward_kept(const void *px, const void *py, const int64
  *   (mutual_information.py:163); px_grad, py_grad out, every element written.
  * Same results, bit for bit, as the two calls.  Every workgroup of this launch must be resident
  * at once, so it only serves shapes with 2 * B * ceil((S+1)/64) <= compute units of the current
- * device, fp32, with a workspace: k2amd_mi_forward_backward_supported(...) says whether a call
+ * device (twice that where the runtime reports that a unit holds two of its workgroups), fp32,
+ * with a workspace: k2amd_mi_forward_backward_supported(...) says whether a call
  * will be served (1) or returns K2AMD_ERR_UNSUPPORTED (0; use the two calls).  It also expects the
  * device not to be busy with other streams' kernels for as long as a second: a workgroup that
  * finds no compute unit free keeps others waiting, and a wait that expires ends the launch with

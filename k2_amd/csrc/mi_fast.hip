@@ -1243,13 +1243,41 @@ int MiBackwardFast(const float *px, const float *p, const float *log_deriv,
   return LaunchStatus();
 }
 
-// Whether the single launch may be used on the current device: every sweeping workgroup (and the
-// clearing ones, which never wait) must find a compute unit of its own at once.
+// Workgroups of the single launch that one compute unit holds at a time when they ask for no LDS
+// beyond their own structure (asked of the runtime once per device ordinal), or -1.
+static int FusedWorkgroupsPerUnit() {
+  static std::atomic<int> per_unit[64];  // 0 = not asked yet
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return -1;
+  int n = per_unit[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, MiForwardBackwardFastKernel,
+                                                     FwdLayout::kThreads, 0) != hipSuccess)
+      return -1;
+    n = n > 0 ? n : -1;
+    per_unit[dev].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
+
+// Whether the single launch may be used on the current device: every workgroup of the grid must
+// be resident at once (a sweeping workgroup waits, in its backward half, for workgroups that
+// started after it).  Up to one workgroup per compute unit each gets a unit to itself.  Up to two
+// per unit, where the kernel's registers and LDS allow two, the dispatcher still hands the
+// sweeping workgroups (the first half of the grid) a unit each before it doubles up, and the
+// clearing workgroups that join them leave after a few microseconds.
+static bool FusedFits(long long grid, bool *exclusive) {
+  const int n = ComputeUnits();
+  if (n <= 0) return false;
+  *exclusive = grid <= n;
+  return *exclusive || (grid <= 2ll * n && FusedWorkgroupsPerUnit() >= 2);
+}
+
 bool MiFusedSupports(int B, int S, int Tn, int modified) {
   if (!MiFastSupports(B, S, Tn, modified) || B < 1) return false;
-  const int n = ComputeUnits();
   const long long nchunks = (S + 1 + kRows - 1) / kRows;
-  return n > 0 && 2 * (long long)B * nchunks <= n;
+  bool exclusive;
+  return FusedFits(2 * (long long)B * nchunks, &exclusive);
 }
 
 int MiForwardBackwardFast(const float *px, const float *py, const int64_t *boundary, float *ans,
@@ -1258,14 +1286,16 @@ int MiForwardBackwardFast(const float *px, const float *py, const int64_t *bound
                           size_t workspace_bytes, hipStream_t stream) {
   if (workspace == nullptr || workspace_bytes < MiFastWorkspaceBytes(B, S, Tn)) return K2AMD_ERR_WORKSPACE;
   if (log_deriv == nullptr) return K2AMD_ERR_INVALID_ARGUMENT;
-  if (!MiFusedSupports(B, S, Tn, modified)) return K2AMD_ERR_UNSUPPORTED;
   const int nchunks = (S + 1 + kRows - 1) / kRows;
+  bool exclusive = true;
+  if (!MiFastSupports(B, S, Tn, modified) || B < 1 || !FusedFits(2ll * B * nchunks, &exclusive))
+    return K2AMD_ERR_UNSUPPORTED;
   const int edge_stride = (int)(((size_t)Tn + 2 + kRows + kW + 3) / 4 * 4 + kW);
   FastHeader *hdr = static_cast<FastHeader *>(workspace);
   float *edge_fwd = reinterpret_cast<float *>(hdr + 1);
   float *edge_bwd = edge_fwd + (size_t)B * (nchunks + 1) * edge_stride;
   const dim3 grid((unsigned)(2 * B * nchunks)), block(FwdLayout::kThreads);
-  const size_t pad = kExclusiveLds - sizeof(FusedLds) - 16;
+  const size_t pad = exclusive ? kExclusiveLds - sizeof(FusedLds) - 16 : 0;
   hipLaunchKernelGGL(MiForwardBackwardFastKernel, grid, block, pad, stream, px, py, boundary, ans, log_deriv, ans_grad, px_grad, py_grad, hdr, edge_fwd, edge_bwd, B, S, Tn, modified, nchunks, edge_stride, overwrite_ans_grad);
   return LaunchStatus();
 }

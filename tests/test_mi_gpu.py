@@ -138,12 +138,14 @@ def test_wide_lattice_more_rows_than_a_wavefront(device, modified):
     check("wide", px, py, bd, (ans, p, gx, gy), device)
 
 
+@pytest.mark.parametrize("B", [80, 150])
 @pytest.mark.parametrize("modified", [False, True])
-def test_more_chunks_than_compute_units(device, modified):
-    """B * ceil((S+1)/64) = 450 sweeping workgroups on 256 compute units: the pair of launches,
-    with two workgroups to a unit."""
+def test_more_workgroups_than_compute_units(device, modified, B):
+    """Three chunks per sequence on 256 compute units.  B=80: 240 sweeping + 240 clearing
+    workgroups, still one launch, two workgroups to a unit.  B=150: 450 chunks, the pair of
+    launches, two sweeping workgroups to a unit."""
     rng = np.random.default_rng(77)
-    B, S, T = 150, 140, 170
+    S, T = 140, 170
     px = rng.normal(-2, 1, (B, S, T if modified else T + 1)).astype(np.float32)
     py = rng.normal(-2, 1, (B, S + 1, T)).astype(np.float32)
     bd = cases.random_boundary(rng, B, S, T, modified)
