@@ -99,7 +99,7 @@ def _cpu_pruned_loss(logits, symbols, ranges, boundary, blank=0):
     return -Lattice.apply(px, py).sum()
 
 
-def pruned_secondary(dev, steps=20, cpu=True):
+def pruned_secondary(dev, steps=50, cpu=True):
     """Second figure asked for next to the headline: pruned RNN-T loss forward + backward on
     BASELINE config 3 (B=32, T=500, S=100, V=500, s_range=5, regular lattice) in utterances/s,
     beside the CPU route on a sample of the same utterances."""
@@ -168,7 +168,7 @@ def pruned_secondary(dev, steps=20, cpu=True):
     return out
 
 
-def other_configs(dev, steps=20):
+def other_configs(dev, steps=50):
     """The two remaining BASELINE configurations, forward + backward through the k2-style API with
     gradients to the network outputs: config 2 (rnnt_loss_simple, B=16 T=250 S=50 V=500) and
     config 5 (rnnt_loss on the full joiner lattice, B=8 T=300 S=75 V=500)."""

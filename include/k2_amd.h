@@ -57,7 +57,9 @@ K2AMD_API const char *k2amd_status_string(int status);
 K2AMD_API size_t k2amd_mi_workspace_bytes(int B, int S, int T, int modified, int dtype);
 K2AMD_API int k2amd_mi_workspace_init(void *workspace, size_t workspace_bytes, void *stream);
 /* Synchronises `stream` and returns K2AMD_ERR_TIMEOUT if a pipelined kernel that used this
- * workspace gave up waiting for a neighbouring workgroup (its results are then invalid). */
+ * workspace gave up waiting for a neighbouring workgroup.  Its results are then invalid, and so
+ * are those of every later call until the workspace is initialised again; the kernels make that
+ * visible without this call by writing NaN to ans (and to the ans_grad they hand back). */
 K2AMD_API int k2amd_mi_workspace_status(const void *workspace, void *stream);
 
 /* Replaces _k2.mutual_information_forward (k2/python/csrc/torch/mutual_information.cu:26-44,

@@ -251,6 +251,14 @@ __device__ __forceinline__ float TakeEdge(float *addr, FastHeader *hdr, float on
   }
 }
 
+// True once a wait of this or an earlier launch on the workspace has timed out.  Results are then
+// invalid, and the kernels say so where a caller looks first: ans (and the ans_grad they hand
+// back) become NaN, in that launch where the store comes after the timeout and in every later
+// launch until the workspace is initialised again.
+__device__ __forceinline__ bool GaveUp(FastHeader *hdr) {
+  return __hip_atomic_load(&hdr->error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;
+}
+
 // Called by one thread after the workgroup's last barrier.
 __device__ __forceinline__ void FinishWorkgroup(FastHeader *hdr, unsigned total) {
   const unsigned n = atomicAdd(&hdr->done, 1u);
@@ -490,7 +498,7 @@ __device__ __forceinline__ void MiForwardChunk(
         if (row_i == g.ns) {
 #pragma unroll
           for (int e = 0; e < 4; ++e)
-            if (j + e == g.nt) ans[g.b] = vv[e];
+            if (j + e == g.nt) ans[g.b] = GaveUp(hdr) ? __builtin_nanf("") : vv[e];
         }
       }
     }
@@ -1074,7 +1082,7 @@ __device__ __forceinline__ void MiBackwardChunk(
   if (role == kStorer) store_block(0);
   if (role == kEdge) publish_block(0);
   if (overwrite_ans_grad && ans_grad != nullptr && role == kChain && g.c == 0 && lane == 0)
-    ans_grad[g.b] = g_origin;
+    ans_grad[g.b] = GaveUp(hdr) ? __builtin_nanf("") : g_origin;
 }
 
 // The first B * nchunks tickets sweep, lower chunks first; the rest of the grid (as many again)
@@ -1139,6 +1147,7 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiForwardBackwardFastKern
     MiBackwardChunk<true>(lds.bwd, px, log_deriv, boundary, ans_grad, px_grad, py_grad, hdr,
                           edge_bwd, B, S, Tn, modified, nchunks, edge_stride, overwrite_ans_grad,
                           seq, chunk, false);
+    if (threadIdx.x == 0 && GaveUp(hdr)) ans[seq] = __builtin_nanf("");
   }
   if (threadIdx.x == 0) FinishWorkgroup(hdr, gridDim.x);
 }

@@ -397,3 +397,36 @@ def test_blocked_and_improbable_edges(device, modified):
         ans, p = omi.mi_forward(px, py, bd)
         gx, gy = omi.mi_backward(px, py, bd, p)
         check("blocked %g modified=%s" % (frac_inf, modified), px, py, bd, (ans, p, gx, gy), device)
+
+
+def test_a_wait_that_gave_up_is_loud(device):
+    """The workspace's error flag, raised by a kernel whose bounded wait expired, is forced from
+    the host here (every wait then returns after a few polls, so all kernels end normally): ans
+    comes out as NaN from both the forward and the single launch, the status call reports it, and
+    a freshly initialised workspace serves the same call correctly again."""
+    from k2_amd import capi
+    rng = np.random.default_rng(9)
+    B, S, T = 2, 100, 70
+    px = torch.from_numpy(rng.normal(-2, 1, (B, S, T + 1)).astype(np.float32)).to(device)
+    py = torch.from_numpy(rng.normal(-2, 1, (B, S + 1, T)).astype(np.float32)).to(device)
+    p = torch.empty(B, S + 1, T + 1, device=device)
+    good = capi.mi_forward(px, py, None, p).clone()
+    assert torch.isfinite(good).all()
+    capi.mi_workspace_status(device)
+    key = (px.device.index, torch.cuda.current_stream(device).cuda_stream)
+    ws = capi._workspaces[key]
+    try:
+        ws[:16].view(torch.int32)[2] = 1                     # FastHeader::error
+        assert torch.isnan(capi.mi_forward(px, py, None, p)).all()
+        g = torch.ones(B, device=device)
+        capi.mi_backward(px, py, None, p, g, overwrite_ans_grad=True)
+        assert torch.isnan(g).all()
+        ans, _, _ = capi.mi_forward_backward(px, py, None, torch.ones(B, device=device))
+        assert torch.isnan(ans).all()
+        with pytest.raises(RuntimeError, match="timed out"):
+            capi.mi_workspace_status(device)
+    finally:
+        torch.cuda.synchronize(device)
+        del capi._workspaces[key]                            # the next call initialises a new one
+    assert torch.equal(capi.mi_forward(px, py, None, p), good)
+    assert capi.mi_workspace_is_clean(device)
