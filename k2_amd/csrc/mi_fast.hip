@@ -570,21 +570,26 @@ __device__ __forceinline__ void MiForwardChunk(
 
   // the chain wavefront is the critical path: it wins the SIMD's issue arbitration
   if (role == kChain) __builtin_amdgcn_s_setprio(3);
-  // ---- prologue: block 0 committed, blocks 1 and 2 in flight ---------------------------------
-  FwdRegs ra, rb;
+  // ---- prologue: block 0 committed, blocks 1 .. kFwdSets in flight --------------------------
+  // A block's loads stay in flight for kFwdSets iterations (~1 us each).  A third set changes
+  // nothing, neither with inputs that the caches hold nor with inputs that come from HBM
+  // (84 us against 85 us per launch of the B=32 S=200 T=1000 workload), and its registers would
+  // cost the second workgroup on a compute unit.
+  constexpr int kFwdSets = 2;
+  FwdRegs sets[kFwdSets];
   if (role == kLoader) {
-    load_block(0, ra);
-    WaitLoads<0>(ra);
-    commit_block(0, ra);
-    load_block(1, ra);
-    load_block(2, rb);
+    load_block(0, sets[0]);
+    WaitLoads<0>(sets[0]);
+    commit_block(0, sets[0]);
+#pragma unroll
+    for (int i = 0; i < kFwdSets; ++i) load_block(1 + i, sets[i]);
   } else if (role == kEdge) {
     take_block(0, edge_px(0));
   }
   LdsBarrier();
 
   // In iteration kb the chain wavefront computes block kb; the loaders commit block kb+1 (loaded
-  // two iterations ago) and start the loads of block kb+3; the storers drain block kb-1; the
+  // kFwdSets iterations ago) and start the loads of block kb+1+kFwdSets; the storers drain block kb-1; the
   // edge wavefront publishes block kb-1 downwards and takes block kb+1 from the chunk above.
   // Every role runs its own loop (same number of barriers), which keeps each loop free of the
   // other roles' code and lets the compiler count outstanding loads exactly.
@@ -594,22 +599,20 @@ __device__ __forceinline__ void MiForwardChunk(
       LdsBarrier();
     }
   } else if (role == kLoader) {
-    for (int kb = 0; kb < g.nblocks; kb += 2) {
-      WaitLoads<kFwdLoadsPerBlock>(ra);  // the other set's loads may stay in flight
-      commit_block(kb + 1, ra);
-      load_block(kb + 3, ra);
-      LdsBarrier();
-      if (kb + 1 < g.nblocks) {
-        WaitLoads<kFwdLoadsPerBlock>(rb);
-        commit_block(kb + 2, rb);
-        load_block(kb + 4, rb);
+    for (int kb = 0; kb < g.nblocks; kb += kFwdSets) {
+#pragma unroll
+      for (int i = 0; i < kFwdSets; ++i) {
+        if (kb + i >= g.nblocks) break;
+        WaitLoads<(kFwdSets - 1) * kFwdLoadsPerBlock>(sets[i]);  // the other sets' loads may stay in flight
+        commit_block(kb + i + 1, sets[i]);
+        load_block(kb + i + 1 + kFwdSets, sets[i]);
         LdsBarrier();
       }
     }
     // the loads of the blocks past the end are still in flight: they must land before the
     // compiler may give their registers to anything else
-    WaitLoads<0>(ra);
-    WaitLoads<0>(rb);
+#pragma unroll
+    for (int i = 0; i < kFwdSets; ++i) WaitLoads<0>(sets[i]);
   } else if (role == kStorer) {
     for (int kb = 0; kb < g.nblocks; ++kb) {
       store_block(kb - 1);
