@@ -247,7 +247,7 @@ def main():
     ap.add_argument("--input-sets", type=int, default=1,
                     help="rotate over this many copies of px / py in device memory, so that a step's "
                          "inputs are not what the previous steps left in the 256 MB Infinity Cache "
-                         "(8 copies at the default shape: 82-85 us per step against 73)")
+                         "(8 copies at the default shape: 76 us per step against 73)")
     ap.add_argument("--B", type=int, default=32)
     ap.add_argument("--S", type=int, default=200)
     ap.add_argument("--T", type=int, default=1000)

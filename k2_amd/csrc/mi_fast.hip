@@ -290,22 +290,26 @@ struct FwdLds {
   // p of each row at the last position of the three most recent blocks (written by the storers,
   // only when the launch keeps the px-edge log-derivatives)
   float last[3][kWave];
+  // px of the row above the chunk (the last row of the chunk above), block by block: written by
+  // the loaders one block ahead of the rest, read by the edge wavefront
+  float px_above[4][kW];
   unsigned ticket;
 };
 
 struct FwdRegs {
   float4v x[FwdLayout::kLoadItems], y[FwdLayout::kLoadItems];
+  float4v above;  // a quad of the row above the chunk, for the block AFTER the set's block
 };
 // waits until at most kYounger of this wavefront's loads are outstanding and ties the registers
 // to the wait, so that no read of them moves in front of it
 template <int kYounger>
 __device__ __forceinline__ void WaitLoads(FwdRegs &r) {
   static_assert(FwdLayout::kLoadItems == 2, "operand list below");
-  asm volatile("s_waitcnt vmcnt(%4)"
-               : "+v"(r.x[0]), "+v"(r.y[0]), "+v"(r.x[1]), "+v"(r.y[1])
+  asm volatile("s_waitcnt vmcnt(%5)"
+               : "+v"(r.x[0]), "+v"(r.y[0]), "+v"(r.x[1]), "+v"(r.y[1]), "+v"(r.above)
                : "n"(kYounger));
 }
-constexpr int kFwdLoadsPerBlock = 2 * FwdLayout::kLoadItems;
+constexpr int kFwdLoadsPerBlock = 2 * FwdLayout::kLoadItems + 1;
 
 // kKeep: also write log_deriv[b][s][t] = (p[s-1][t+o] + px[s-1][t+o]) - p[s][t], the logarithm of
 // the px edge's share of cell (s, t) exactly as the backward sweep forms it
@@ -370,6 +374,8 @@ __device__ __forceinline__ void MiForwardChunk(
     idx_x[it] = (g.b * S + g.s0 + rx) * T1 + g.t0;
     idx_y[it] = (g.b * (S + 1) + g.s0 + ry) * Tn + g.t0;
   }
+  // float index of local column 0 of the row above the chunk (any px row where there is none)
+  const int idx_above = (g.b * S + g.s0 + max(g.row0 - 1, 0)) * T1 + g.t0;
   // every quad of every row of block kb inside the valid columns?  (uniform over the workgroup)
   auto interior = [&](int kb) {
     return kb * kW - 1 - (kRows - 1) * g.skew >= 0 && kb * kW + 30 <= g.nt - 1;
@@ -386,6 +392,9 @@ __device__ __forceinline__ void MiForwardChunk(
       r.x[it] = AsyncQuad(rsx, idx_x[it] + jp + g.skew);
       r.y[it] = AsyncQuad(rsy, idx_y[it] + jp);
     }
+    // every lane asks (the count of loads in flight is the same for all wavefronts); the eight
+    // lanes of loader row 0 keep what arrives
+    r.above = AsyncQuad(rsx, idx_above + (kb + 1) * kW + 4 * mm - 1 + g.skew);
   };
   // `inner` is uniform over the workgroup: the masking code for blocks on the rim of the box is
   // a real branch (the empty asm statement keeps the compiler from flattening it into selects
@@ -426,6 +435,20 @@ __device__ __forceinline__ void MiForwardChunk(
       lds.fx[q][pq] = make_float4(vx[0], vx[1], vx[2], vx[3]);
       lds.fy[q][pq] = make_float4(vy[0], vy[1], vy[2], vy[3]);
     }
+  };
+
+  // the set of block kb carries the row above the chunk for block kb + 1
+  auto commit_above = [&](int kb, FwdRegs &r) {
+    if (lq != 0 || kb + 1 >= g.nblocks) return;
+    const float4 qa = AsFloat4(r.above);
+    const float in[4] = {qa.x, qa.y, qa.z, qa.w};
+    float v[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int jx = (kb + 1) * kW + 4 * mm + e - 1 + g.skew;
+      v[e] = g.c > 0 && jx >= 0 && jx <= hi_x ? fmaxf(in[e], kLogZero) : kLogZero;
+    }
+    *reinterpret_cast<float4 *>(&lds.px_above[(kb + 1) & 3][4 * mm]) = make_float4(v[0], v[1], v[2], v[3]);
   };
 
   // ---- storers ---------------------------------------------------------------------------
@@ -509,7 +532,9 @@ __device__ __forceinline__ void MiForwardChunk(
   //     p[row0-1][..] (taken from the chunk above) + px[row0-1][..]
   // and put it into row 64 of the fx array, which lane 0 of the chain reads in place of a row of
   // its own (the DPP add of the chain step leaves lane 0's register as it is).  The px values
-  // are loaded by this wavefront itself, one block ahead.
+  // of blocks 0 and 1 are loaded by this wavefront itself; from block 2 on they come from the
+  // loaders' LDS ring, so that no load of this wavefront stands between it and the edge words
+  // (its loads return in order, and a px value that came from HBM kept every hand-over waiting).
   auto edge_px = [&](int kb) -> float {
     const int jx = kb * kW + lane - 1 + g.skew;
     float v = kLogZero;
@@ -581,6 +606,7 @@ __device__ __forceinline__ void MiForwardChunk(
     load_block(0, sets[0]);
     WaitLoads<0>(sets[0]);
     commit_block(0, sets[0]);
+    commit_above(0, sets[0]);
 #pragma unroll
     for (int i = 0; i < kFwdSets; ++i) load_block(1 + i, sets[i]);
   } else if (role == kEdge) {
@@ -605,6 +631,7 @@ __device__ __forceinline__ void MiForwardChunk(
         if (kb + i >= g.nblocks) break;
         WaitLoads<(kFwdSets - 1) * kFwdLoadsPerBlock>(sets[i]);  // the other sets' loads may stay in flight
         commit_block(kb + i + 1, sets[i]);
+        commit_above(kb + i + 1, sets[i]);
         load_block(kb + i + 1 + kFwdSets, sets[i]);
         LdsBarrier();
       }
@@ -622,10 +649,9 @@ __device__ __forceinline__ void MiForwardChunk(
     float px_above = edge_px(1);
     for (int kb = 0; kb < g.nblocks; ++kb) {
       publish_block(kb - 1);
-      const float px_next = edge_px(kb + 2);
       take_block(kb + 1, px_above);
-      px_above = px_next;
       LdsBarrier();
+      px_above = lds.px_above[(kb + 2) & 3][lane & (kW - 1)];  // committed in this iteration
     }
   }
   if (role == kStorer) store_block(g.nblocks - 1);
