@@ -1230,7 +1230,8 @@ static int ComputeUnits() {
 // LDS bytes to ask for beyond a kernel's own structure.  While the sweeping workgroups of a launch
 // find a compute unit each, every one gets a unit to itself (kExclusiveLds); once there are more
 // chunks than units the launch is bound by how many chains the device steps at a time, and two
-// workgroups share a unit.
+// workgroups share a unit (K2AMD_MI_SHARE_UNITS=0 in the environment, read once, keeps one to a
+// unit: for comparisons).
 static size_t LdsPad(size_t own, long long sweepers) {
   static const bool never_share = [] {
     const char *e = getenv("K2AMD_MI_SHARE_UNITS");
