@@ -602,3 +602,52 @@ def test_loss_nodes_equal_the_builder_then_recursion_chain(device, rnnt_type):
     with torch.no_grad():
         plain = k2.rnnt_loss_simple(lm, am, sym, 0, bd, rnnt_type, 0.0, "none")
     assert torch.equal(plain, -scores.detach()) and not plain.requires_grad
+
+
+def test_random_shapes_through_the_api(device):
+    """Random small shapes, lattice types, boundaries, dtypes and delay penalties through the
+    k2-style API against the oracle: rnnt_loss_simple with gradients, get_rnnt_prune_ranges
+    (bit-exact, from the oracle's gradients), rnnt_loss_pruned (and a finite gradient), rnnt_loss."""
+    import k2_amd as k2
+
+    def close(name, seed, got, want, tol):
+        got = got.detach().cpu().numpy()
+        ok = np.isclose(got, want, equal_nan=True, **tol) | (got == want)
+        assert ok.all(), (name, seed, got[~ok][:4], want[~ok][:4])
+
+    for seed in range(7000, 7080):
+        rng = np.random.default_rng(seed)
+        rt = TYPES[int(rng.integers(0, 3))]
+        B, S, C = int(rng.integers(1, 6)), int(rng.integers(1, 40)), int(rng.integers(2, 60))
+        t_min = S if rt != "regular" else 1
+        T = int(rng.integers(t_min, S + 90))
+        dtype = np.float32 if rng.random() < 0.8 else np.float64
+        c = cases.rnnt_case(seed, B, T, S, C, dtype=dtype, t_lo=max(T // 2, t_min), s_lo=S // 2,
+                            with_boundary=bool(rng.random() < 0.7), modified=(rt != "regular"))
+        pen = float(rng.choice([0.0, 0.0, 0.01]))
+        tol, bd, sym = TOL[np.dtype(dtype)], c["boundary"], c["symbols"]
+        want, (gx_w, gy_w) = orn.rnnt_loss_simple(c["lm"], c["am"], sym, 0, bd, rt, pen, "none", True)
+        got, (gx, gy) = k2.rnnt_loss_simple(dev(c["lm"], device), dev(c["am"], device), dev(sym, device), 0,
+                                            dev(bd, device), rt, pen, "none", True)
+        close("simple", seed, got, want, tol)
+        if dtype == np.float64:
+            close("px_grad", seed, gx, gx_w, tol)
+            close("py_grad", seed, gy, gy_w, tol)
+        R = int(rng.integers(2 if rt == "regular" else 1, S + 3))
+        bd_full = np.tile(np.array([[0, 0, S, T]], np.int64), (B, 1)) if bd is None else bd
+        ranges_w = orn.prune_ranges(gx_w, gy_w, bd_full, R)
+        ranges = k2.get_rnnt_prune_ranges(dev(gx_w, device), dev(gy_w, device), dev(bd_full, device), R)
+        assert np.array_equal(ranges.cpu().numpy(), ranges_w), ("ranges", seed)
+        logits = rng.standard_normal((B, T, ranges_w.shape[2], C)).astype(dtype)
+        want = orn.rnnt_loss_pruned(logits, sym, ranges_w, 0, bd, rt, pen, "none")
+        lg = dev(logits, device).requires_grad_(True)
+        got = k2.rnnt_loss_pruned(lg, dev(sym, device), dev(ranges_w, device), 0, dev(bd, device), rt, pen, "none")
+        close("pruned", seed, got, want, tol)
+        fin = np.isfinite(want)
+        if fin.any():
+            (got * dev(fin.astype(dtype), device)).sum().backward()
+            assert torch.isfinite(lg.grad).all(), ("pruned gradient", seed)
+        full = rng.standard_normal((B, T, S + 1, C)).astype(dtype)
+        want = orn.rnnt_loss(full, sym, 0, bd, rt, pen, "none")
+        got = k2.rnnt_loss(dev(full, device), dev(sym, device), 0, dev(bd, device), rt, pen, "none")
+        close("joint", seed, got, want, tol)
