@@ -430,3 +430,29 @@ def test_a_wait_that_gave_up_is_loud(device):
         del capi._workspaces[key]                            # the next call initialises a new one
     assert torch.equal(capi.mi_forward(px, py, None, p), good)
     assert capi.mi_workspace_is_clean(device)
+
+
+def test_single_launches_on_two_streams(device):
+    """Two streams issue the single launch at the same time, each with its own workspace.  The
+    clearing workgroups of a launch never wait and leave, so what must be resident together is
+    the sweeping workgroups of the launches in flight: 2 x 128 here, on 256 compute units."""
+    from k2_amd import capi
+    c = cases.c4_case()
+    px, py, bd = (torch.from_numpy(c[k]).to(device) for k in ("px", "py", "boundary"))
+    ones = torch.ones(px.shape[0], device=device)
+    ref = capi.mi_forward_backward(px, py, bd, ones, overwrite_ans_grad=False)
+    torch.cuda.synchronize(device)
+    streams = [torch.cuda.Stream(device=device) for _ in range(2)]
+    outs = [[], []]
+    for _ in range(20):
+        for i, s in enumerate(streams):
+            with torch.cuda.stream(s):
+                outs[i].append(capi.mi_forward_backward(px, py, bd, ones, overwrite_ans_grad=False))
+    torch.cuda.synchronize(device)
+    for i, s in enumerate(streams):
+        with torch.cuda.stream(s):
+            capi.mi_workspace_status(device)
+            assert capi.mi_workspace_is_clean(device)
+        for o in outs[i]:
+            for a, b in zip(o, ref):
+                assert torch.equal(a, b)
