@@ -125,6 +125,18 @@ def test_random_cases_vs_oracle(device, dtype):
         check(f"seed{seed}", c["px"], c["py"], c["boundary"], (ans, p, gx, gy), device)
 
 
+def test_random_multi_chunk_cases_vs_oracle(device):
+    """Random shapes of up to five 64-row chunks and many 32-column blocks, random boundaries,
+    both lattice types, fp32 (the pipelined kernels in all their launch variants) and fp64."""
+    for seed in range(5000, 5040):
+        shape = (dict(max_B=12, max_S=300, max_T=400), dict(max_B=40, max_S=130, max_T=150),
+                 dict(max_B=3, max_S=70, max_T=1500))[seed % 3]
+        c = cases.mi_case(seed, dtype=np.float64 if seed % 5 == 0 else np.float32, **shape)
+        ans, p = omi.mi_forward(c["px"], c["py"], c["boundary"])
+        gx, gy = omi.mi_backward(c["px"], c["py"], c["boundary"], p)
+        check(f"seed{seed}", c["px"], c["py"], c["boundary"], (ans, p, gx, gy), device)
+
+
 @pytest.mark.parametrize("modified", [False, True])
 def test_wide_lattice_more_rows_than_a_wavefront(device, modified):
     # S+1 > 256 exercises the row loop of a workgroup; long T exercises many steps.
