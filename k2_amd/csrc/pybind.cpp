@@ -56,6 +56,29 @@ struct WorkspaceCache {
   }
 };
 
+WorkspaceCache &Cache();
+
+// Synchronises the stream of every cached workspace and reads its error flag.  A workspace whose
+// kernels gave up a wait (their ans came out as NaN) is initialised again, so that the calls after
+// this one work; returns how many were.  No counterpart in the reference.
+int64_t MutualInformationRecoverWorkspaces() {
+  WorkspaceCache &cache = Cache();
+  std::lock_guard<std::mutex> lock(cache.mu);
+  int64_t recovered = 0;
+  for (auto &kv : cache.bufs) {
+    torch::Tensor &ws = kv.second;
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(ws.device());
+    const int status = k2amd_mi_workspace_status(ws.data_ptr(), kv.first.second);
+    if (status == K2AMD_ERR_TIMEOUT) {
+      Check(k2amd_mi_workspace_init(ws.data_ptr(), static_cast<size_t>(ws.numel()), kv.first.second));
+      ++recovered;
+    } else {
+      Check(status);
+    }
+  }
+  return recovered;
+}
+
 WorkspaceCache &Cache() {
   static WorkspaceCache *cache = new WorkspaceCache();  // never destroyed: outlives torch's teardown
   return *cache;
@@ -532,6 +555,7 @@ PYBIND11_MODULE(_k2_amd, m) {
   m.def("mutual_information_forward", &MutualInformationForward, pybind11::arg("px"),
         pybind11::arg("py"), pybind11::arg("boundary"), pybind11::arg("p"),
         pybind11::arg("log_deriv") = pybind11::none());
+  m.def("mutual_information_recover_workspaces", &MutualInformationRecoverWorkspaces);
   m.def("mutual_information_keeps_log_deriv", &MutualInformationKeepsLogDeriv, pybind11::arg("px"),
         pybind11::arg("py"));
   m.def("mutual_information_backward", &MutualInformationBackward, pybind11::arg("px"),

@@ -22,6 +22,25 @@ def _require_device(t: torch.Tensor):
             "k2_amd runs on MI355X only: got a tensor on %s (there is no CPU path)" % t.device)
 
 
+def mutual_information_recover_workspaces() -> int:
+    """Waits for the streams that the pipelined fp32 kernels have run on and reads the error flag
+    of each scratch buffer.  Where a kernel gave up a bounded wait (its scores came out as NaN,
+    and so would those of every later call), the buffer is initialised again; returns how many
+    were.  Call it when a loss turns NaN to tell that cause from the others."""
+    if _ext is not None:
+        return int(_ext.mutual_information_recover_workspaces())
+    n = 0
+    for key, ws in list(capi._workspaces.items()):
+        with torch.cuda.device(key[0]):
+            status = capi.lib().k2amd_mi_workspace_status(ws.data_ptr(), key[1])
+            if status == 5:  # K2AMD_ERR_TIMEOUT
+                capi.check(capi.lib().k2amd_mi_workspace_init(ws.data_ptr(), ws.numel(), key[1]))
+                n += 1
+            else:
+                capi.check(status)
+    return n
+
+
 def mutual_information_keeps_log_deriv(px: torch.Tensor, py: torch.Tensor) -> bool:
     """True if the forward / backward pair below uses a ``log_deriv`` tensor for these inputs (the
     pipelined fp32 kernels do; the exact kernels leave it untouched, so allocating one is

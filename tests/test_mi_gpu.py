@@ -442,6 +442,11 @@ def test_a_wait_that_gave_up_is_loud(device):
         del capi._workspaces[key]                            # the next call initialises a new one
     assert torch.equal(capi.mi_forward(px, py, None, p), good)
     assert capi.mi_workspace_is_clean(device)
+    # the host module's own buffers: nothing to recover after ordinary calls
+    from k2_amd import native
+    import k2_amd as k2
+    k2.mutual_information_recursion(px, py, None, return_grad=True)
+    assert native.mutual_information_recover_workspaces() == 0
 
 
 def test_single_launches_on_two_streams(device):
