@@ -592,7 +592,9 @@ def get_rnnt_prune_ranges_deprecated(
     boundary = boundary.to(dev)
     pad = torch.nn.functional.pad
     occupation = pad(px_grad, (0, 0, 0, 1)) + pad(py_grad, (0, T1 - T))   # [B][S+1][T1]
-    prefix = torch.cumsum(pad(occupation, (0, 0, 1, 0)), dim=1)            # [B][S+2][T1]
+    # torch's CPU cumsum, which the reference's values come from, accumulates fp32 input in double
+    # and rounds every prefix once; the device scan in fp32 would round along the way
+    prefix = torch.cumsum(pad(occupation, (0, 0, 1, 0)).double(), dim=1).to(occupation.dtype)  # [B][S+2][T1]
     window = prefix[:, s_range:, :] - prefix[:, :-s_range, :]
     s_begin = torch.argmax(window, dim=1)[:, :T]
     live = torch.arange(T, device=dev).reshape(1, T) < boundary[:, 3].reshape(B, 1) - 1

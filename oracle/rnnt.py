@@ -340,7 +340,8 @@ def prune_ranges_deprecated(px_grad, py_grad, boundary, s_range):
         [py_grad, np.zeros((B, S + 1, 1), dtype=dt)], axis=2)
     tot = np.concatenate([px_grad, np.zeros((B, 1, T1), dtype=dt)], axis=1) + py_p
     tot = np.concatenate([np.zeros((B, 1, T1), dtype=dt), tot], axis=1)
-    tot = np.cumsum(tot, axis=1, dtype=dt)
+    # torch's CPU cumsum accumulates fp32 input in double and rounds each prefix once
+    tot = np.cumsum(tot, axis=1, dtype=np.float64).astype(dt)
     diff = tot[:, s_range:, :] - tot[:, :-s_range, :]
     s_begin = np.argmax(diff, axis=1).astype(np.int64)[:, :T]
     mask = np.arange(T)[None, :] < (boundary[:, 3][:, None] - 1)
