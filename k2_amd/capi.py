@@ -1,6 +1,7 @@
 """ctypes binding of libk2amd.so's C-ABI (include/k2_amd.h), taking torch tensors.
 
-This is the thinnest possible host: it checks nothing beyond device/dtype/contiguity, passes
+A thin host: before a pointer goes down it checks that every tensor has the dtype, device and
+exact shape the kernels index with (RuntimeError otherwise, nothing launched), then passes
 ``tensor.data_ptr()`` and torch's current HIP stream, and raises RuntimeError on a non-zero
 status.  The parity tests call the kernels through here.
 """
@@ -91,6 +92,58 @@ def ptr(t):
     return t.data_ptr()
 
 
+def expect(t, name, dtype, device, shape):
+    """Raises RuntimeError unless ``t`` is a contiguous tensor of exactly this dtype, device and
+    shape: the kernels index with the sizes taken from ONE tensor of a call, so a disagreeing
+    tensor would be read out of bounds or at the wrong element size."""
+    if not isinstance(t, torch.Tensor):
+        raise RuntimeError(f"k2_amd: {name} must be a tensor")
+    if not t.is_cuda:
+        raise RuntimeError(f"k2_amd runs on MI355X only: {name} is on {t.device} (there is no CPU path)")
+    if t.dtype != dtype or t.device != device or tuple(t.shape) != tuple(shape):
+        raise RuntimeError(f"k2_amd: {name} must be {dtype} {list(shape)} on {device}, "
+                           f"got {t.dtype} {list(t.shape)} on {t.device}")
+    if not t.is_contiguous():
+        raise RuntimeError(f"k2_amd: {name} must be contiguous")
+
+
+def expect_optional(t, name, dtype, device, shape):
+    if t is not None:
+        expect(t, name, dtype, device, shape)
+
+
+def _float_dtype(t, name):
+    if not isinstance(t, torch.Tensor) or t.dtype not in (torch.float32, torch.float64):
+        raise RuntimeError(f"k2_amd: {name} must be a float32 or float64 tensor")
+    if not t.is_cuda:
+        raise RuntimeError(f"k2_amd runs on MI355X only: {name} is on {t.device} (there is no CPU path)")
+    return t.dtype, t.device
+
+
+def _dims(t, name, n):
+    if t.dim() != n:
+        raise RuntimeError(f"k2_amd: {name} must have {n} dimensions, got {t.dim()}")
+    return tuple(t.shape)
+
+
+def _mi_shapes(px, py, boundary, lattices=()):
+    """(B, S, T, modified) after the checks of k2/python/csrc/torch/mutual_information_cpu.cu:53-77;
+    ``lattices``: (tensor or None, name) pairs that must have p's shape."""
+    dt, dev = _float_dtype(px, "px")
+    B, S, T1 = _dims(px, "px", 3)
+    if py.dim() != 3:
+        raise RuntimeError("k2_amd: py must have 3 dimensions")
+    T = py.shape[2]
+    if T1 not in (T, T + 1):
+        raise RuntimeError("k2_amd: px.size(2) must be T or T+1")
+    expect(px, "px", dt, dev, (B, S, T1))
+    expect(py, "py", dt, dev, (B, S + 1, T))
+    expect_optional(boundary, "boundary", torch.int64, dev, (B, 4))
+    for t, name in lattices:
+        expect_optional(t, name, dt, dev, (B, S + 1, T + 1))
+    return B, S, T, int(T1 == T)
+
+
 def stream_ptr(device):
     return torch.cuda.current_stream(device).cuda_stream
 
@@ -154,9 +207,9 @@ def mi_forward(px, py, boundary, p, log_deriv=None):
     """C-ABI twin of _k2.mutual_information_forward: fills ``p``, returns ans [B].  ``log_deriv``
     (optional, shaped like ``p``) receives what lets mi_backward skip its reads of p and px; where
     mi_keeps_log_deriv(px, py) holds, ``p`` may then be None and is not computed."""
-    B, S, T1 = px.shape
-    T = py.shape[2]
-    modified = int(T1 == T)
+    B, S, T, modified = _mi_shapes(px, py, boundary, ((p, "p"), (log_deriv, "log_deriv")))
+    if p is None and log_deriv is None:
+        raise RuntimeError("k2_amd: p may only be None where log_deriv is given")
     ans = torch.empty(B, dtype=px.dtype, device=px.device)
     dt = dtype_code(px)
     ws = mi_workspace(B, S, T, modified, dt, px.device)
@@ -170,9 +223,10 @@ def mi_forward(px, py, boundary, p, log_deriv=None):
 def mi_backward(px, py, boundary, p, ans_grad, overwrite_ans_grad=True, log_deriv=None):
     """C-ABI twin of _k2.mutual_information_backward: returns (px_grad, py_grad).  ``log_deriv``:
     the tensor the matching mi_forward call filled, or None."""
-    B, S, T1 = px.shape
-    T = py.shape[2]
-    modified = int(T1 == T)
+    B, S, T, modified = _mi_shapes(px, py, boundary, ((p, "p"), (log_deriv, "log_deriv")))
+    if p is None and log_deriv is None:
+        raise RuntimeError("k2_amd: p may only be None where log_deriv is given")
+    expect(ans_grad, "ans_grad", px.dtype, px.device, (B,))
     px_grad = torch.empty_like(px)
     py_grad = torch.empty_like(py)
     dt = dtype_code(px)
@@ -198,9 +252,8 @@ def mi_forward_backward_supported(px, py):
 
 def mi_forward_backward(px, py, boundary, ans_grad, overwrite_ans_grad=True):
     """Forward and backward recursion in one launch: returns (ans, px_grad, py_grad)."""
-    B, S, T1 = px.shape
-    T = py.shape[2]
-    modified = int(T1 == T)
+    B, S, T, modified = _mi_shapes(px, py, boundary)
+    expect_optional(ans_grad, "ans_grad", px.dtype, px.device, (B,))
     ans = torch.empty(B, dtype=px.dtype, device=px.device)
     log_deriv = torch.empty(B, S + 1, T + 1, dtype=px.dtype, device=px.device)
     px_grad = torch.empty_like(px)
@@ -219,12 +272,34 @@ def _t1(T, rnnt_type):
     return T + 1 if rnnt_type == REGULAR else T
 
 
+def _rnnt_type(code):
+    if code not in (REGULAR, MODIFIED, CONSTRAINED):
+        raise RuntimeError(f"k2_amd: unknown rnnt_type code {code}")
+
+
+def _symbol(termination_symbol, C):
+    if not 0 <= int(termination_symbol) < C:
+        raise RuntimeError(f"k2_amd: termination_symbol {termination_symbol} outside [0, {C})")
+
+
+def _expect_lattice_grads(px_grad, py_grad, seq_scale, dt, dev, B, S, T, rnnt_type):
+    expect(px_grad, "px_grad", dt, dev, (B, S, _t1(T, rnnt_type)))
+    expect(py_grad, "py_grad", dt, dev, (B, S + 1, T))
+    expect_optional(seq_scale, "seq_scale", dt, dev, (B,))
+
+
 def logprobs_simple_forward(lm, am, symbols, termination_symbol, rnnt_type, boundary):
     """C-ABI get_rnnt_logprobs: returns (px, py, saved) with ``saved`` the buffers the backward
     re-uses (lm_probs, am_probs, denom)."""
-    B, T, C = am.shape
-    S = lm.shape[1] - 1
-    dev, dt = am.device, am.dtype
+    dt, dev = _float_dtype(am, "am")
+    B, T, C = _dims(am, "am", 3)
+    S = _dims(lm, "lm", 3)[1] - 1
+    _rnnt_type(rnnt_type)
+    expect(am, "am", dt, dev, (B, T, C))
+    expect(lm, "lm", dt, dev, (B, S + 1, C))
+    expect(symbols, "symbols", torch.int64, dev, (B, S))
+    expect_optional(boundary, "boundary", torch.int64, dev, (B, 4))
+    _symbol(termination_symbol, C)
     px = torch.empty(B, S, _t1(T, rnnt_type), dtype=dt, device=dev)
     py = torch.empty(B, S + 1, T, dtype=dt, device=dev)
     lm_probs = torch.empty_like(lm)
@@ -245,8 +320,17 @@ def logprobs_simple_backward(px_grad, py_grad, symbols, boundary, saved, termina
     """``seq_scale`` [B] or None: px_grad[b], py_grad[b] count as multiplied by seq_scale[b] (the
     same for the two functions below)."""
     lm_probs, am_probs, denom = saved
-    B, T, C = am_probs.shape
-    S = lm_probs.shape[1] - 1
+    dt, dev = _float_dtype(am_probs, "am_probs")
+    B, T, C = _dims(am_probs, "am_probs", 3)
+    S = _dims(lm_probs, "lm_probs", 3)[1] - 1
+    _rnnt_type(rnnt_type)
+    expect(am_probs, "am_probs", dt, dev, (B, T, C))
+    expect(lm_probs, "lm_probs", dt, dev, (B, S + 1, C))
+    expect(denom, "denom", dt, dev, (B, S + 1, T))
+    expect(symbols, "symbols", torch.int64, dev, (B, S))
+    expect_optional(boundary, "boundary", torch.int64, dev, (B, 4))
+    _expect_lattice_grads(px_grad, py_grad, seq_scale, dt, dev, B, S, T, rnnt_type)
+    _symbol(termination_symbol, C)
     lm_grad = torch.empty_like(lm_probs)
     am_grad = torch.empty_like(am_probs)
     q = torch.empty_like(denom)
@@ -260,9 +344,14 @@ def logprobs_simple_backward(px_grad, py_grad, symbols, boundary, saved, termina
 
 
 def logprobs_joint_forward(logits, symbols, termination_symbol, rnnt_type, boundary):
-    B, T, S1, C = logits.shape
+    dt, dev = _float_dtype(logits, "logits")
+    B, T, S1, C = _dims(logits, "logits", 4)
     S = S1 - 1
-    dev, dt = logits.device, logits.dtype
+    _rnnt_type(rnnt_type)
+    expect(logits, "logits", dt, dev, (B, T, S1, C))
+    expect(symbols, "symbols", torch.int64, dev, (B, S))
+    expect_optional(boundary, "boundary", torch.int64, dev, (B, 4))
+    _symbol(termination_symbol, C)
     px = torch.empty(B, S, _t1(T, rnnt_type), dtype=dt, device=dev)
     py = torch.empty(B, S + 1, T, dtype=dt, device=dev)
     norm = torch.empty(B, T, S1, dtype=dt, device=dev)
@@ -275,9 +364,16 @@ def logprobs_joint_forward(logits, symbols, termination_symbol, rnnt_type, bound
 
 def logprobs_joint_backward(logits, norm, px_grad, py_grad, symbols, boundary,
                             termination_symbol, rnnt_type, seq_scale=None):
-    B, T, S1, C = logits.shape
+    dt, dev = _float_dtype(logits, "logits")
+    B, T, S1, C = _dims(logits, "logits", 4)
+    _rnnt_type(rnnt_type)
+    expect(logits, "logits", dt, dev, (B, T, S1, C))
+    expect(norm, "normalizers", dt, dev, (B, T, S1))
+    expect(symbols, "symbols", torch.int64, dev, (B, S1 - 1))
+    expect_optional(boundary, "boundary", torch.int64, dev, (B, 4))
+    _expect_lattice_grads(px_grad, py_grad, seq_scale, dt, dev, B, S1 - 1, T, rnnt_type)
+    _symbol(termination_symbol, C)
     grad = torch.empty_like(logits)
-    dev = logits.device
     with torch.cuda.device(dev):
         check(lib().k2amd_rnnt_logprobs_joint_backward(
             ptr(logits), ptr(norm), ptr(px_grad), ptr(py_grad), ptr(seq_scale), ptr(symbols),
@@ -289,9 +385,15 @@ def logprobs_joint_backward(logits, norm, px_grad, py_grad, symbols, boundary,
 def logprobs_pruned_forward(logits, symbols, ranges, termination_symbol, boundary, rnnt_type,
                             hat=False):
     """``hat`` selects get_hat_logprobs_pruned (blank = column 0, termination_symbol unused)."""
-    B, T, R, C = logits.shape
-    S = symbols.shape[1]
-    dev, dt = logits.device, logits.dtype
+    dt, dev = _float_dtype(logits, "logits")
+    B, T, R, C = _dims(logits, "logits", 4)
+    S = _dims(symbols, "symbols", 2)[1]
+    _rnnt_type(rnnt_type)
+    expect(logits, "logits", dt, dev, (B, T, R, C))
+    expect(symbols, "symbols", torch.int64, dev, (B, S))
+    expect(ranges, "ranges", torch.int64, dev, (B, T, R))
+    expect_optional(boundary, "boundary", torch.int64, dev, (B, 4))
+    _symbol(0 if hat else termination_symbol, C)
     px = torch.empty(B, S, _t1(T, rnnt_type), dtype=dt, device=dev)
     py = torch.empty(B, S + 1, T, dtype=dt, device=dev)
     norm = torch.empty(B, T, R, dtype=dt, device=dev)
@@ -309,10 +411,18 @@ def logprobs_pruned_forward(logits, symbols, ranges, termination_symbol, boundar
 
 def logprobs_pruned_backward(logits, norm, px_grad, py_grad, symbols, ranges, boundary,
                              termination_symbol, rnnt_type, hat=False, seq_scale=None):
-    B, T, R, C = logits.shape
-    S = symbols.shape[1]
+    dt, dev = _float_dtype(logits, "logits")
+    B, T, R, C = _dims(logits, "logits", 4)
+    S = _dims(symbols, "symbols", 2)[1]
+    _rnnt_type(rnnt_type)
+    expect(logits, "logits", dt, dev, (B, T, R, C))
+    expect(norm, "normalizers", dt, dev, (B, T, R))
+    expect(symbols, "symbols", torch.int64, dev, (B, S))
+    expect(ranges, "ranges", torch.int64, dev, (B, T, R))
+    expect_optional(boundary, "boundary", torch.int64, dev, (B, 4))
+    _expect_lattice_grads(px_grad, py_grad, seq_scale, dt, dev, B, S, T, rnnt_type)
+    _symbol(0 if hat else termination_symbol, C)
     grad = torch.empty_like(logits)
-    dev = logits.device
     with torch.cuda.device(dev):
         if hat:
             check(lib().k2amd_rnnt_hat_logprobs_pruned_backward(
@@ -329,10 +439,17 @@ def logprobs_pruned_backward(logits, norm, px_grad, py_grad, symbols, ranges, bo
 
 def prune_ranges(px_grad, py_grad, boundary, s_range):
     """``s_range`` is the final value (after the adjustments the Python layer applies)."""
-    B, S, T1 = px_grad.shape
-    T = py_grad.shape[2]
+    dt, dev = _float_dtype(px_grad, "px_grad")
+    B, S, T1 = _dims(px_grad, "px_grad", 3)
+    T = _dims(py_grad, "py_grad", 3)[2]
+    if T1 not in (T, T + 1):
+        raise RuntimeError("k2_amd: px_grad.size(2) must be T or T+1")
+    expect(px_grad, "px_grad", dt, dev, (B, S, T1))
+    expect(py_grad, "py_grad", dt, dev, (B, S + 1, T))
+    expect(boundary, "boundary", torch.int64, dev, (B, 4))
+    if not 1 <= int(s_range) <= S + 1:
+        raise RuntimeError(f"k2_amd: s_range {s_range} outside [1, S + 1 = {S + 1}]")
     ranges = torch.empty(B, T, s_range, dtype=torch.int64, device=px_grad.device)
-    dev = px_grad.device
     with torch.cuda.device(dev):
         check(lib().k2amd_rnnt_prune_ranges(ptr(px_grad), ptr(py_grad), ptr(boundary), ptr(ranges),
                                             B, S, T, int(T1 == T), s_range, dtype_code(px_grad),
@@ -341,8 +458,11 @@ def prune_ranges(px_grad, py_grad, boundary, s_range):
 
 
 def prune_gather(lm, ranges):
-    B, S1, D = lm.shape
-    _, T, R = ranges.shape
+    dt, dev = _float_dtype(lm, "lm")
+    B, S1, D = _dims(lm, "lm", 3)
+    _, T, R = _dims(ranges, "ranges", 3)
+    expect(lm, "lm", dt, dev, (B, S1, D))
+    expect(ranges, "ranges", torch.int64, dev, (B, T, R))
     out = torch.empty(B, T, R, D, dtype=lm.dtype, device=lm.device)
     with torch.cuda.device(lm.device):
         check(lib().k2amd_rnnt_prune_gather(ptr(lm), ptr(ranges), ptr(out), B, S1, T, R, D,
@@ -351,7 +471,12 @@ def prune_gather(lm, ranges):
 
 
 def prune_gather_backward(grad, ranges, S1):
-    B, T, R, D = grad.shape
+    dt, dev = _float_dtype(grad, "grad")
+    B, T, R, D = _dims(grad, "grad", 4)
+    expect(grad, "grad", dt, dev, (B, T, R, D))
+    expect(ranges, "ranges", torch.int64, dev, (B, T, R))
+    if int(S1) < 1:
+        raise RuntimeError("k2_amd: S1 must be positive")
     lm_grad = torch.empty(B, S1, D, dtype=grad.dtype, device=grad.device)
     with torch.cuda.device(grad.device):
         check(lib().k2amd_rnnt_prune_gather_backward(ptr(grad), ptr(ranges), ptr(lm_grad), B, S1,

@@ -281,6 +281,33 @@ void RequireDevice(const torch::Tensor &t, const char *name) {
               " (there is no CPU path)");
   TORCH_CHECK(t.is_contiguous(), name, " must be contiguous");
 }
+// The kernels index every tensor of a call with the sizes taken from ONE of them, so a tensor of
+// another shape, element size or device would be read out of bounds: each host function below
+// checks all of its tensors with these before a pointer goes down (RuntimeError, nothing launched).
+void Expect(const torch::Tensor &t, const char *name, c10::ScalarType dtype, const torch::Device &dev,
+            std::initializer_list<int64_t> shape) {
+  RequireDevice(t, name);
+  TORCH_CHECK(t.scalar_type() == dtype && t.device() == dev && t.sizes() == torch::IntArrayRef(shape),
+              "k2_amd: ", name, " must be ", dtype, " ", torch::IntArrayRef(shape), " on ", dev, ", got ",
+              t.scalar_type(), " ", t.sizes(), " on ", t.device());
+}
+void ExpectOptional(const torch::optional<torch::Tensor> &t, const char *name, c10::ScalarType dtype,
+                    const torch::Device &dev, std::initializer_list<int64_t> shape) {
+  if (t.has_value() && t->defined()) Expect(*t, name, dtype, dev, shape);
+}
+// a float32 / float64 device tensor with n dimensions: the tensor the sizes of a call are read from
+void ExpectFloat(const torch::Tensor &t, const char *name, int64_t n) {
+  RequireDevice(t, name);
+  DtypeCode(t);
+  TORCH_CHECK(t.dim() == n, "k2_amd: ", name, " must have ", n, " dimensions, got ", t.dim());
+}
+void ExpectRnntType(int rnnt_type) {
+  TORCH_CHECK(rnnt_type == K2AMD_REGULAR || rnnt_type == K2AMD_MODIFIED || rnnt_type == K2AMD_CONSTRAINED,
+              "k2_amd: unknown rnnt_type code ", rnnt_type);
+}
+void ExpectSymbol(int symbol, int64_t C) {
+  TORCH_CHECK(symbol >= 0 && symbol < C, "k2_amd: termination_symbol ", symbol, " outside [0, ", C, ")");
+}
 const int64_t *I64(const torch::optional<torch::Tensor> &t) {
   if (!t.has_value() || !t->defined()) return nullptr;
   TORCH_CHECK(t->scalar_type() == torch::kLong && t->is_contiguous() && t->is_cuda(),
@@ -288,16 +315,28 @@ const int64_t *I64(const torch::optional<torch::Tensor> &t) {
   return t->data_ptr<int64_t>();
 }
 int T1Of(int T, int rnnt_type) { return rnnt_type == K2AMD_REGULAR ? T + 1 : T; }
+void ExpectLatticeGrads(const torch::Tensor &px_grad, const torch::Tensor &py_grad,
+                        const torch::optional<torch::Tensor> &seq_scale, c10::ScalarType dtype,
+                        const torch::Device &dev, int64_t B, int64_t S, int64_t T, int rnnt_type) {
+  Expect(px_grad, "px_grad", dtype, dev, {B, S, T1Of(static_cast<int>(T), rnnt_type)});
+  Expect(py_grad, "py_grad", dtype, dev, {B, S + 1, T});
+  ExpectOptional(seq_scale, "seq_scale", dtype, dev, {B});
+}
 
 // get_rnnt_logprobs: returns (px, py, lm_probs, am_probs, denom)
 std::vector<torch::Tensor> LogprobsSimpleForward(torch::Tensor lm, torch::Tensor am,
                                                  torch::Tensor symbols, int termination_symbol,
                                                  int rnnt_type,
                                                  torch::optional<torch::Tensor> boundary) {
-  RequireDevice(lm, "lm");
-  RequireDevice(am, "am");
-  c10::hip::HIPGuardMasqueradingAsCUDA guard(am.device());
+  ExpectFloat(am, "am", 3);
+  ExpectFloat(lm, "lm", 3);
+  ExpectRnntType(rnnt_type);
   const int B = am.size(0), T = am.size(1), C = am.size(2), S = lm.size(1) - 1;
+  Expect(lm, "lm", am.scalar_type(), am.device(), {B, S + 1, C});
+  Expect(symbols, "symbols", torch::kLong, am.device(), {B, S});
+  ExpectOptional(boundary, "boundary", torch::kLong, am.device(), {B, 4});
+  ExpectSymbol(termination_symbol, C);
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(am.device());
   auto opt = am.options();
   torch::Tensor px = torch::empty({B, S, T1Of(T, rnnt_type)}, opt), py = torch::empty({B, S + 1, T}, opt);
   torch::Tensor lm_probs = torch::empty_like(lm), am_probs = torch::empty_like(am);
@@ -331,11 +370,20 @@ std::vector<torch::Tensor> LogprobsSimpleBackward(torch::Tensor px_grad, torch::
                                                   torch::Tensor denom, int termination_symbol,
                                                   int rnnt_type,
                                                   torch::optional<torch::Tensor> seq_scale) {
-  RequireDevice(px_grad, "px_grad");
-  RequireDevice(py_grad, "py_grad");
+  ExpectFloat(am_probs, "am_probs", 3);
+  ExpectFloat(lm_probs, "lm_probs", 3);
+  ExpectRnntType(rnnt_type);
+  const int B = am_probs.size(0), T = am_probs.size(1), C = am_probs.size(2), S = lm_probs.size(1) - 1;
+  const auto dtype = am_probs.scalar_type();
+  const auto dev = am_probs.device();
+  Expect(lm_probs, "lm_probs", dtype, dev, {B, S + 1, C});
+  Expect(denom, "denom", dtype, dev, {B, S + 1, T});
+  Expect(symbols, "symbols", torch::kLong, dev, {B, S});
+  ExpectOptional(boundary, "boundary", torch::kLong, dev, {B, 4});
+  ExpectLatticeGrads(px_grad, py_grad, seq_scale, dtype, dev, B, S, T, rnnt_type);
+  ExpectSymbol(termination_symbol, C);
   const void *scale = ScalePtr(seq_scale, px_grad);
   c10::hip::HIPGuardMasqueradingAsCUDA guard(am_probs.device());
-  const int B = am_probs.size(0), T = am_probs.size(1), C = am_probs.size(2), S = lm_probs.size(1) - 1;
   torch::Tensor lm_grad = torch::empty_like(lm_probs), am_grad = torch::empty_like(am_probs);
   torch::Tensor q = torch::empty_like(denom);
   void *stream = StreamOf(am_probs);
@@ -353,9 +401,13 @@ std::vector<torch::Tensor> LogprobsSimpleBackward(torch::Tensor px_grad, torch::
 std::vector<torch::Tensor> LogprobsJointForward(torch::Tensor logits, torch::Tensor symbols,
                                                 int termination_symbol, int rnnt_type,
                                                 torch::optional<torch::Tensor> boundary) {
-  RequireDevice(logits, "logits");
-  c10::hip::HIPGuardMasqueradingAsCUDA guard(logits.device());
+  ExpectFloat(logits, "logits", 4);
+  ExpectRnntType(rnnt_type);
   const int B = logits.size(0), T = logits.size(1), S = logits.size(2) - 1, C = logits.size(3);
+  Expect(symbols, "symbols", torch::kLong, logits.device(), {B, S});
+  ExpectOptional(boundary, "boundary", torch::kLong, logits.device(), {B, 4});
+  ExpectSymbol(termination_symbol, C);
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(logits.device());
   auto opt = logits.options();
   torch::Tensor px = torch::empty({B, S, T1Of(T, rnnt_type)}, opt), py = torch::empty({B, S + 1, T}, opt);
   torch::Tensor norm = torch::empty({B, T, S + 1}, opt);
@@ -373,12 +425,16 @@ torch::Tensor LogprobsJointBackward(torch::Tensor logits, torch::Tensor norm, to
                                     torch::Tensor py_grad, torch::Tensor symbols,
                                     torch::optional<torch::Tensor> boundary, int termination_symbol,
                                     int rnnt_type, torch::optional<torch::Tensor> seq_scale) {
-  RequireDevice(logits, "logits");
-  RequireDevice(px_grad, "px_grad");
-  RequireDevice(py_grad, "py_grad");
+  ExpectFloat(logits, "logits", 4);
+  ExpectRnntType(rnnt_type);
+  const int B = logits.size(0), T = logits.size(1), S = logits.size(2) - 1, C = logits.size(3);
+  Expect(norm, "normalizers", logits.scalar_type(), logits.device(), {B, T, S + 1});
+  Expect(symbols, "symbols", torch::kLong, logits.device(), {B, S});
+  ExpectOptional(boundary, "boundary", torch::kLong, logits.device(), {B, 4});
+  ExpectLatticeGrads(px_grad, py_grad, seq_scale, logits.scalar_type(), logits.device(), B, S, T, rnnt_type);
+  ExpectSymbol(termination_symbol, C);
   const void *scale = ScalePtr(seq_scale, px_grad);
   c10::hip::HIPGuardMasqueradingAsCUDA guard(logits.device());
-  const int B = logits.size(0), T = logits.size(1), S = logits.size(2) - 1, C = logits.size(3);
   torch::Tensor grad = torch::empty_like(logits);
   void *stream = StreamOf(logits);
   {
@@ -397,10 +453,16 @@ std::vector<torch::Tensor> LogprobsPrunedForward(torch::Tensor logits, torch::Te
                                                  torch::Tensor ranges, int termination_symbol,
                                                  torch::optional<torch::Tensor> boundary,
                                                  int rnnt_type, bool hat) {
-  RequireDevice(logits, "logits");
-  c10::hip::HIPGuardMasqueradingAsCUDA guard(logits.device());
+  ExpectFloat(logits, "logits", 4);
+  ExpectRnntType(rnnt_type);
+  TORCH_CHECK(symbols.dim() == 2, "k2_amd: symbols must have 2 dimensions");
   const int B = logits.size(0), T = logits.size(1), R = logits.size(2), C = logits.size(3);
   const int S = symbols.size(1);
+  Expect(symbols, "symbols", torch::kLong, logits.device(), {B, S});
+  Expect(ranges, "ranges", torch::kLong, logits.device(), {B, T, R});
+  ExpectOptional(boundary, "boundary", torch::kLong, logits.device(), {B, 4});
+  ExpectSymbol(hat ? 0 : termination_symbol, C);
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(logits.device());
   auto opt = logits.options();
   torch::Tensor px = torch::empty({B, S, T1Of(T, rnnt_type)}, opt), py = torch::empty({B, S + 1, T}, opt);
   torch::Tensor norm = torch::empty({B, T, R}, opt);
@@ -426,13 +488,19 @@ torch::Tensor LogprobsPrunedBackward(torch::Tensor logits, torch::Tensor norm, t
                                      torch::optional<torch::Tensor> boundary, int termination_symbol,
                                      int rnnt_type, bool hat,
                                      torch::optional<torch::Tensor> seq_scale) {
-  RequireDevice(logits, "logits");
-  RequireDevice(px_grad, "px_grad");
-  RequireDevice(py_grad, "py_grad");
-  const void *scale = ScalePtr(seq_scale, px_grad);
-  c10::hip::HIPGuardMasqueradingAsCUDA guard(logits.device());
+  ExpectFloat(logits, "logits", 4);
+  ExpectRnntType(rnnt_type);
+  TORCH_CHECK(symbols.dim() == 2, "k2_amd: symbols must have 2 dimensions");
   const int B = logits.size(0), T = logits.size(1), R = logits.size(2), C = logits.size(3);
   const int S = symbols.size(1);
+  Expect(norm, "normalizers", logits.scalar_type(), logits.device(), {B, T, R});
+  Expect(symbols, "symbols", torch::kLong, logits.device(), {B, S});
+  Expect(ranges, "ranges", torch::kLong, logits.device(), {B, T, R});
+  ExpectOptional(boundary, "boundary", torch::kLong, logits.device(), {B, 4});
+  ExpectLatticeGrads(px_grad, py_grad, seq_scale, logits.scalar_type(), logits.device(), B, S, T, rnnt_type);
+  ExpectSymbol(hat ? 0 : termination_symbol, C);
+  const void *scale = ScalePtr(seq_scale, px_grad);
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(logits.device());
   torch::Tensor grad = torch::empty_like(logits);
   void *stream = StreamOf(logits);
   {
@@ -454,10 +522,14 @@ torch::Tensor LogprobsPrunedBackward(torch::Tensor logits, torch::Tensor norm, t
 // device part of get_rnnt_prune_ranges; s_range is the final value
 torch::Tensor PruneRanges(torch::Tensor px_grad, torch::Tensor py_grad, torch::Tensor boundary,
                           int s_range) {
-  RequireDevice(px_grad, "px_grad");
-  RequireDevice(py_grad, "py_grad");
-  c10::hip::HIPGuardMasqueradingAsCUDA guard(px_grad.device());
+  ExpectFloat(px_grad, "px_grad", 3);
+  ExpectFloat(py_grad, "py_grad", 3);
   const int B = px_grad.size(0), S = px_grad.size(1), T1 = px_grad.size(2), T = py_grad.size(2);
+  TORCH_CHECK(T1 == T || T1 == T + 1, "k2_amd: px_grad.size(2) must be T or T+1");
+  Expect(py_grad, "py_grad", px_grad.scalar_type(), px_grad.device(), {B, S + 1, T});
+  Expect(boundary, "boundary", torch::kLong, px_grad.device(), {B, 4});
+  TORCH_CHECK(s_range >= 1 && s_range <= S + 1, "k2_amd: s_range ", s_range, " outside [1, S + 1 = ", S + 1, "]");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(px_grad.device());
   torch::Tensor ranges = torch::empty({B, T, s_range}, px_grad.options().dtype(torch::kLong));
   void *stream = StreamOf(px_grad);
   {
@@ -470,9 +542,11 @@ torch::Tensor PruneRanges(torch::Tensor px_grad, torch::Tensor py_grad, torch::T
 }
 
 torch::Tensor PruneGather(torch::Tensor lm, torch::Tensor ranges) {
-  RequireDevice(lm, "lm");
-  c10::hip::HIPGuardMasqueradingAsCUDA guard(lm.device());
+  ExpectFloat(lm, "lm", 3);
+  TORCH_CHECK(ranges.dim() == 3, "k2_amd: ranges must have 3 dimensions");
   const int B = lm.size(0), S1 = lm.size(1), D = lm.size(2), T = ranges.size(1), R = ranges.size(2);
+  Expect(ranges, "ranges", torch::kLong, lm.device(), {B, T, R});
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(lm.device());
   torch::Tensor out = torch::empty({B, T, R, D}, lm.options());
   void *stream = StreamOf(lm);
   {
@@ -484,9 +558,11 @@ torch::Tensor PruneGather(torch::Tensor lm, torch::Tensor ranges) {
 }
 
 torch::Tensor PruneGatherBackward(torch::Tensor grad, torch::Tensor ranges, int S1) {
-  RequireDevice(grad, "grad");
-  c10::hip::HIPGuardMasqueradingAsCUDA guard(grad.device());
+  ExpectFloat(grad, "grad", 4);
   const int B = grad.size(0), T = grad.size(1), R = grad.size(2), D = grad.size(3);
+  Expect(ranges, "ranges", torch::kLong, grad.device(), {B, T, R});
+  TORCH_CHECK(S1 >= 1, "k2_amd: S1 must be positive");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(grad.device());
   torch::Tensor lm_grad = torch::empty({B, S1, D}, grad.options());
   void *stream = StreamOf(grad);
   {

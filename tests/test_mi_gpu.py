@@ -74,7 +74,7 @@ def run_gpu(px, py, bd, device, ans_grad=None):
     return ans.cpu().numpy(), p.cpu().numpy(), gx.cpu().numpy(), gy.cpu().numpy(), g.cpu().numpy(), g_in.cpu().numpy()
 
 
-def _close(name, got, want, want64, tol, p_scale=None, relative_floor=True):
+def _close(name, got, want, want64, tol, mode="relative"):
     """fp64: the stated tolerance.  fp32: the stated tolerance against the fp32 CPU oracle; the
     elements that miss it are arbitrated by the fp64 oracle element by element (tolerance.py)."""
     if tol["rtol"] < 1e-6 or want64 is None:
@@ -82,7 +82,7 @@ def _close(name, got, want, want64, tol, p_scale=None, relative_floor=True):
             ok = np.isclose(got, want, equal_nan=True, **tol)
         assert ok.all(), (name, int((~ok).sum()), got[~ok][:5], want[~ok][:5])
         return None
-    return tolerance.close_f32(name, got, want, want64, p_scale, relative_floor=relative_floor)
+    return tolerance.close_f32(name, got, want, want64, mode=mode)
 
 
 def check(name, px, py, bd, want, device):
@@ -90,22 +90,20 @@ def check(name, px, py, bd, want, device):
     ans, p, gx, gy, g_out, g_in = run_gpu(px, py, bd, device)
     tol = TOL[px.dtype]
     w64 = (None, None, None, None)
-    scale = None
     if px.dtype == np.float32:
         a64, p64 = omi.mi_forward(px.astype(np.float64), py.astype(np.float64), bd)
         w64 = (a64, p64) + tuple(omi.mi_backward(px.astype(np.float64), py.astype(np.float64), bd, p64))
-        scale = tolerance.p_scale_of(p64)
-    _close(name + " ans", ans, ans_w, w64[0], tol, scale, relative_floor=False)
+    _close(name + " ans", ans, ans_w, w64[0], tol, mode="absolute")
     inside = ~np.isnan(p_w)
     assert not np.isnan(p[inside]).any(), name
     if w64[1] is not None:
         with np.errstate(invalid="ignore"):
             p_g, p_32, p_64 = (np.where(inside, a, 0.0) for a in (p, p_w, w64[1]))
-        _close(name + " p", p_g, p_32, p_64, tol, scale, relative_floor=False)
+        _close(name + " p", p_g, p_32, p_64, tol, mode="absolute")
     else:
         _close(name + " p", p[inside], p_w[inside], None, tol)
-    _close(name + " px_grad", gx, gx_w, w64[2], tol, scale)
-    _close(name + " py_grad", gy, gy_w, w64[3], tol, scale)
+    _close(name + " px_grad", gx, gx_w, w64[2], tol)
+    _close(name + " py_grad", gy, gy_w, w64[3], tol)
     # the gradient that reaches the start cell equals the one injected at the end cell
     # whenever the end cell is reachable
     ok = np.isfinite(ans_w)
@@ -228,12 +226,12 @@ def test_headline_shape_three_way(device):
     # loss: the stated tolerance holds directly
     np.testing.assert_allclose(ans, ans32, rtol=1e-4, atol=1e-5)
     np.testing.assert_allclose(ans, ans64, rtol=1e-4, atol=1e-5)
-    scale = tolerance.p_scale_of(p64)
     for name, g, g32, g64 in (("px_grad", gx, gx32, gx64), ("py_grad", gy, gy32, gy64)):
-        st = tolerance.close_f32("c4 " + name, g, g32, g64, scale, max_arbitrated=0.02)
+        st = tolerance.close_f32("c4 " + name, g, g32, g64, max_arbitrated=0.05)
         print(f"c4 {name}: max|gpu-fp64|={st['max_gpu_vs_fp64']:.3e}  max|cpu32-fp64|={st['max_cpu32_vs_fp64']:.3e}  "
               f"max|gpu-cpu32|={st['max_gpu_vs_cpu32']:.3e}  arbitrated {st['arbitrated']} of {st['n']} "
-              f"({100 * st['arbitrated_frac']:.4f} %)")
+              f"({100 * st['arbitrated_frac']:.4f} %), reference's own 99.9th-percentile relative error "
+              f"{st.get('reference_error_quantile_max', 0):.3e}")
     # flow conservation at full size: each symbol row is emitted exactly once
     for b in range(c["B"]):
         s1 = int(bd[b, 2])
