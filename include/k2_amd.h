@@ -27,7 +27,8 @@ enum k2amd_status {
   K2AMD_ERR_UNSUPPORTED = 2,      /* valid request this build cannot serve (size limit) */
   K2AMD_ERR_WORKSPACE = 3,        /* workspace missing or too small */
   K2AMD_ERR_LAUNCH = 4,           /* HIP reported a launch error */
-  K2AMD_ERR_TIMEOUT = 5           /* a bounded in-kernel wait expired; re-initialise the workspace */
+  K2AMD_ERR_TIMEOUT = 5,          /* a bounded in-kernel wait expired; re-initialise the workspace */
+  K2AMD_ERR_SCRATCH_LIMIT = 6     /* k2amd_mi_forward_noalloc: shape beyond its static scratch array */
 };
 
 enum k2amd_dtype { K2AMD_F32 = 0, K2AMD_F64 = 1, K2AMD_F16 = 2 /* lattice scores only */ };
@@ -70,6 +71,24 @@ K2AMD_API int k2amd_mi_workspace_status(const void *workspace, void *stream);
 K2AMD_API int k2amd_mi_forward(const void *px, const void *py, const int64_t *boundary, void *p, void *ans,
                      int B, int S, int T, int modified, int dtype, void *workspace,
                      size_t workspace_bytes, void *stream);
+
+/* k2amd_mi_forward for callers that cannot allocate or bring a workspace: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference.  Same arguments, results and kernels as k2amd_mi_forward, except that the scratch of
+ * the pipelined fp32 kernels is a static device array of K2AMD_MI_NOALLOC_SCRATCH_BYTES inside the
+ * library (each GPU the library runs on holds its own copy until the process ends); the call
+ * itself allocates and frees nothing and synchronises nothing.  A shape whose
+ * k2amd_mi_workspace_bytes(...) exceeds that size is refused with K2AMD_ERR_SCRATCH_LIMIT (the
+ * headline shape B=32, S=200, T=1000 needs 1.45 MB).  fp64 runs the exact kernels, which use no
+ * scratch.  Every call re-initialises the part of the array it uses with a fill kernel in front of
+ * the recursion, so a call never inherits anything from the one before it.  All calls on one GPU
+ * share that GPU's array: calls that overlap in time on one GPU (two streams, two threads) race
+ * and must be serialised by the caller.  The first call on a device looks up the array's address;
+ * a call with B == 0 does only that.                                                             */
+#define K2AMD_MI_NOALLOC_SCRATCH_BYTES (8u << 20)
+K2AMD_API int k2amd_mi_forward_noalloc(const void *px, const void *py, const int64_t *boundary,
+                                       void *p, void *ans, int B, int S, int T, int modified,
+                                       int dtype, void *stream);
 
 /* Replaces _k2.mutual_information_backward (k2/python/csrc/torch/mutual_information.cu:46-67,
  * semantics of k2/python/csrc/torch/mutual_information_cpu.cu:128-255).  Writes EVERY element of

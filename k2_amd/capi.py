@@ -29,6 +29,7 @@ _SIGNATURES = {
     "k2amd_mi_workspace_init": ([_vp, _sz, _vp], _ci),
     "k2amd_mi_workspace_status": ([_vp, _vp], _ci),
     "k2amd_mi_forward": ([_vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp, _sz, _vp], _ci),
+    "k2amd_mi_forward_noalloc": ([_vp] * 5 + [_ci] * 5 + [_vp], _ci),
     "k2amd_mi_backward": ([_vp, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci,
                            _vp, _sz, _vp], _ci),
     "k2amd_mi_keeps_log_deriv": ([_ci] * 6, _ci),
@@ -217,6 +218,18 @@ def mi_forward(px, py, boundary, p, log_deriv=None):
         check(lib().k2amd_mi_forward_keep(ptr(px), ptr(py), ptr(boundary), ptr(p), ptr(ans),
                                           ptr(log_deriv), B, S, T, modified, dt, ptr(ws),
                                           0 if ws is None else ws.numel(), stream_ptr(px.device)))
+    return ans
+
+
+def mi_forward_noalloc(px, py, boundary, p, ans):
+    """k2amd_mi_forward_noalloc: like mi_forward, but the library brings its own static scratch and
+    the caller brings ``ans`` [B] as well, so that nothing is allocated by the call."""
+    B, S, T, modified = _mi_shapes(px, py, boundary, ((p, "p"),))
+    expect(p, "p", px.dtype, px.device, (B, S + 1, T + 1))
+    expect(ans, "ans", px.dtype, px.device, (B,))
+    with torch.cuda.device(px.device):
+        check(lib().k2amd_mi_forward_noalloc(ptr(px), ptr(py), ptr(boundary), ptr(p), ptr(ans), B, S, T,
+                                             modified, dtype_code(px), stream_ptr(px.device)))
     return ans
 
 

@@ -1,4 +1,5 @@
 // extern "C" entry points of the MI recursion: argument checks and kernel selection.
+#include <atomic>
 #include <cstdlib>
 #include <cstring>
 
@@ -24,6 +25,30 @@ bool PathIs(const char *name) {
 }
 bool ForceGeneric() { return PathIs("generic"); }
 
+// ---- scratch of the entry point that allocates nothing (k2amd_mi_forward_noalloc) --------------
+// One array per device that loads this library, held until the process ends.  The name below is a
+// host-side stand-in for the symbol, NOT a device address: host code only ever uses the pointer
+// that hipGetSymbolAddress returned for the device that is current (ScratchOfCurrentDevice).
+constexpr size_t kScratchBytes = K2AMD_MI_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+// Device address of `scratch` on the current device (asked of the runtime once per device
+// ordinal, with that device current), or nullptr.
+void *ScratchOfCurrentDevice() {
+  static std::atomic<void *> ptrs[64];  // nullptr = not asked yet
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+  void *ptr = ptrs[dev].load(std::memory_order_acquire);
+  if (ptr == nullptr) {
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    ptrs[dev].store(ptr, std::memory_order_release);  // every thread would store the same address
+  }
+  return ptr;
+}
+
 }  // namespace
 
 extern "C" {
@@ -38,6 +63,7 @@ const char *k2amd_status_string(int status) {
     case K2AMD_ERR_WORKSPACE: return "workspace missing or too small";
     case K2AMD_ERR_LAUNCH: return "HIP launch error";
     case K2AMD_ERR_TIMEOUT: return "in-kernel wait timed out; workspace must be re-initialised";
+    case K2AMD_ERR_SCRATCH_LIMIT: return "shape needs more scratch than the static array of the no-allocation entry point holds";
     default: return "unknown status";
   }
 }
@@ -97,6 +123,27 @@ int k2amd_mi_forward_keep(const void *px, const void *py, const int64_t *boundar
                                    (float *)ans, B, S, T, modified, st);
   return MiForwardGeneric<double>((const double *)px, (const double *)py, boundary, (double *)p,
                                   (double *)ans, B, S, T, modified, st);
+}
+
+int k2amd_mi_forward_noalloc(const void *px, const void *py, const int64_t *boundary, void *p,
+                             void *ans, int B, int S, int T, int modified, int dtype, void *stream) {
+  if (!ShapeOk(B, S, T) || (dtype != K2AMD_F32 && dtype != K2AMD_F64)) return K2AMD_ERR_INVALID_ARGUMENT;
+  const size_t need = k2amd_mi_workspace_bytes(B, S, T, modified, dtype);
+  if (need > kScratchBytes) return K2AMD_ERR_SCRATCH_LIMIT;
+  // set-up (also for B == 0, so that a caller can have it done ahead of its first real call)
+  void *ws = ScratchOfCurrentDevice();
+  if (ws == nullptr) return K2AMD_ERR_LAUNCH;
+  if (B == 0) return K2AMD_OK;
+  if (need > 0) {
+    // The array keeps what the last call on this device left in it, whichever stream and shape
+    // that was, and a launch that gave up a wait leaves words behind: every call starts by
+    // putting the part it uses back into the initial state (a fill kernel, stream-ordered in
+    // front of the recursion).
+    const int status = MiFastWorkspaceInit(ws, need, static_cast<hipStream_t>(stream));
+    if (status != K2AMD_OK) return status;
+  }
+  return k2amd_mi_forward_keep(px, py, boundary, p, ans, nullptr, B, S, T, modified, dtype,
+                               need > 0 ? ws : nullptr, need, stream);
 }
 
 int k2amd_mi_backward(const void *px, const void *py, const int64_t *boundary, const void *p,
