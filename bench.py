@@ -2,12 +2,16 @@
 """Headline benchmark: MI recursion forward + backward on one MI355X.
 
 Workload (BASELINE config 4): fp32, modified lattice, B=32, S=200, T=1000, px/py = min(N(-3,1), 0),
-per-sequence boundary with T_b in [600,1000] and S_b in [100,200].  One step = one forward
-launch + one backward launch through the C-ABI, inputs resident in HBM.
+per-sequence boundary with T_b in [600,1000] and S_b in [100,200].  One step = the forward and
+the backward recursion through the C-ABI (one launch: k2amd_mi_forward_backward), inputs resident
+in HBM and taken in turn from eight copies, so that every step reads them from HBM rather than
+from what the step before left in the 256 MB Infinity Cache.
 
 Prints ONE JSON line.  `value` counts ACTIVE lattice cells, sum_b (S_b+1)(T_b+1), per second of
-fwd+bwd wall time on the GPU; `roofline` prices the slower of the two kernels against the HBM
-peak with its algorithmic bytes; `cpu_baseline` is the reference's CPU loop on this host.
+fwd+bwd wall time on the GPU; `roofline` prices the step's kernel (the slower of the two where
+two launches are asked for) against the HBM peak with its algorithmic bytes; `cache_resident` is
+the same measurement with one copy of the inputs; `cpu_baseline` is the reference's CPU loop on
+this host.
 """
 import argparse
 import json
@@ -31,7 +35,7 @@ BWD_BYTES_PER_CELL = 16
 # HBM bytes per launch on the default workload, from rocprofv3's FETCH_SIZE / WRITE_SIZE counters
 # scaled by a 256 MiB device copy (profiles/mi_fast_kernels_c4_hbm_traffic.md).  Reported only
 # for the default shape; any other --B/--S/--T prints null.
-MEASURED_TRAFFIC_BYTES = {"mi_forward_backward": 119547667, "mi_forward": 50265553, "mi_backward": 69316719}
+MEASURED_TRAFFIC_BYTES = {"mi_forward_backward": None, "mi_forward": 50265553, "mi_backward": 69316719}
 MEASURED_TRAFFIC_BYTES_PLAIN_PAIR = {"mi_forward": 50049796, "mi_backward": 86230408}  # --no-keep
 
 
@@ -113,13 +117,17 @@ def pruned_secondary(dev, steps=50, cpu=True):
     logits = torch.from_numpy(np.random.default_rng(33).standard_normal((B, T, R, C)).astype(np.float32)).to(dev)
     logits.requires_grad_(True)
 
+    # A training loop brings a new boundary tensor with every batch, and the functions read its
+    # values on the host once per tensor (a device-to-host copy that waits for the stream): every
+    # timed step gets a fresh clone, so that the figure includes that read.
     def simple_and_ranges():
-        _, (gx, gy) = k2.rnnt_loss_simple(lm, am, sym, 0, bd, reduction="sum", return_grad=True)
-        return k2.get_rnnt_prune_ranges(gx, gy, bd, R)
+        b = bd.clone()
+        _, (gx, gy) = k2.rnnt_loss_simple(lm, am, sym, 0, b, reduction="sum", return_grad=True)
+        return k2.get_rnnt_prune_ranges(gx, gy, b, R)
 
     def pruned(ranges):
         logits.grad = None
-        loss = k2.rnnt_loss_pruned(logits, sym, ranges, 0, bd, reduction="sum")
+        loss = k2.rnnt_loss_pruned(logits, sym, ranges, 0, bd.clone(), reduction="sum")
         loss.backward()
         return loss
 
@@ -142,7 +150,8 @@ def pruned_secondary(dev, steps=50, cpu=True):
     logits_bytes = 3 * logits.numel() * 4
     out = {
         "workload": "rnnt_loss_pruned fwd+bwd, fp32, regular, B=32 T=500 S=100 V=500 s_range=5 "
-                    "(BASELINE config 3), ranges from an rnnt_loss_simple pass",
+                    "(BASELINE config 3), ranges from an rnnt_loss_simple pass; a fresh boundary "
+                    "tensor in every step (one host read of it per step, as in a training loop)",
         "value": B / t_pruned, "unit": "utterances/s", "ms_per_step": t_pruned * 1e3,
         "logits_GBps": logits_bytes / t_pruned / 1e9,
         "frac_of_hbm_peak": logits_bytes / t_pruned / 1e9 / HBM_PEAK_GBS,
@@ -198,7 +207,7 @@ def other_configs(dev, steps=50):
     def simple():
         lm.grad = None
         am.grad = None
-        k2.rnnt_loss_simple(lm, am, sym, 0, bd, reduction="sum").backward()
+        k2.rnnt_loss_simple(lm, am, sym, 0, bd.clone(), reduction="sum").backward()
 
     t = timed(simple)
     # lm, am read once forward; their gradients written once backward
@@ -218,7 +227,7 @@ def other_configs(dev, steps=50):
 
     def joint():
         logits.grad = None
-        k2.rnnt_loss(logits, sym, 0, bd, reduction="sum").backward()
+        k2.rnnt_loss(logits, sym, 0, bd.clone(), reduction="sum").backward()
 
     t = timed(joint)
     nbytes = 3 * 4 * logits.numel()  # read forward; read + write backward
@@ -244,10 +253,12 @@ def main():
                     help="run the forward and the backward as two launches where one would do")
     ap.add_argument("--no-keep", action="store_true",
                     help="run the plain forward/backward pair (no log-derivative tensor between them)")
-    ap.add_argument("--input-sets", type=int, default=1,
+    ap.add_argument("--input-sets", type=int, default=8,
                     help="rotate over this many copies of px / py in device memory, so that a step's "
                          "inputs are not what the previous steps left in the 256 MB Infinity Cache "
-                         "(8 copies at the default shape: 76 us per step against 73)")
+                         "(8 copies at the default shape are 410 MB); 1 = the same inputs every step")
+    ap.add_argument("--no-cache-resident", action="store_true",
+                    help="skip the second measurement on one copy of the inputs ('cache_resident')")
     ap.add_argument("--B", type=int, default=32)
     ap.add_argument("--S", type=int, default=200)
     ap.add_argument("--T", type=int, default=1000)
@@ -282,30 +293,67 @@ def main():
     lattice = torch.empty(B, S + 1, T + 1, dtype=torch.float32, device=dev)
     p, log_deriv = (None, lattice) if keep else (lattice, None)
 
-    # ... and, where the device holds all of the launch's workgroups at once, both recursions run
-    # in ONE launch, again as mutual_information_recursion does
+    # ... and both recursions run in ONE launch, again as mutual_information_recursion does
     single = keep and not args.two_launches and capi.mi_forward_backward_supported(px, py)
 
-    sets = [(px, py)] + [(px.clone(), py.clone()) for _ in range(args.input_sets - 1)]
-    turn = [0]
+    def measure(n_sets):
+        """Times args.steps steps after args.warmup; px / py taken in turn from n_sets copies."""
+        sets = [(px, py)] + [(px.clone(), py.clone()) for _ in range(n_sets - 1)]
+        turn = [0]
 
-    def step(ev=None):
-        px, py = sets[turn[0] % len(sets)]
-        turn[0] += 1
-        if single:
-            # one event per launch: launch k lasts from its event to the next launch's
+        def step(ev=None):
+            x, y = sets[turn[0] % len(sets)]
+            turn[0] += 1
+            if single:
+                # one event per launch: launch k lasts from its event to the next launch's
+                if ev is not None:
+                    ev[0].record()
+                return capi.mi_forward_backward(x, y, bd, ones, overwrite_ans_grad=False)
             if ev is not None:
                 ev[0].record()
-            return capi.mi_forward_backward(px, py, bd, ones, overwrite_ans_grad=False)
-        if ev is not None:
-            ev[0].record()
-        capi.mi_forward(px, py, bd, p, log_deriv=log_deriv)
-        if ev is not None:
-            ev[1].record()
-        g = capi.mi_backward(px, py, bd, p, ones, overwrite_ans_grad=False, log_deriv=log_deriv)
-        if ev is not None:
-            ev[2].record()
-        return g
+            capi.mi_forward(x, y, bd, p, log_deriv=log_deriv)
+            if ev is not None:
+                ev[1].record()
+            g = capi.mi_backward(x, y, bd, p, ones, overwrite_ans_grad=False, log_deriv=log_deriv)
+            if ev is not None:
+                ev[2].record()
+            return g
+
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for k in range(args.steps):
+            step(events[k])
+        if single:
+            events[-1][2].record()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        m = {"ms_per_step": wall / args.steps * 1e3, "input_mb": len(sets) * (px.numel() + py.numel()) * 4 // 1000000}
+        if single:
+            # one kernel does the step: its algorithmic bytes are the forward's plus the backward's
+            ends = [e[0] for e in events[1:]] + [events[-1][2]]
+            both_ms = np.array([e[0].elapsed_time(end) for e, end in zip(events, ends)])
+            m.update(dom="mi_forward_backward", dom_ms=float(both_ms.mean()), dom_bytes=both_bytes,
+                     both_avg=float(both_ms.mean()),
+                     kernel_times={"mi_forward_backward_avg_us": float(both_ms.mean()) * 1e3,
+                                   "mi_forward_backward_min_us": float(both_ms.min()) * 1e3})
+        else:
+            fwd_ms = np.array([e[0].elapsed_time(e[1]) for e in events])
+            bwd_ms = np.array([e[1].elapsed_time(e[2]) for e in events])
+            # Roofline of the dominant kernel (the one with the longer average launch).
+            fwd_avg, bwd_avg = float(fwd_ms.mean()), float(bwd_ms.mean())
+            if bwd_avg >= fwd_avg:
+                m.update(dom="mi_backward", dom_ms=bwd_avg, dom_bytes=BWD_BYTES_PER_CELL * active)
+            else:
+                m.update(dom="mi_forward", dom_ms=fwd_avg, dom_bytes=FWD_BYTES_PER_CELL * active)
+            m.update(both_avg=fwd_avg + bwd_avg,
+                     kernel_times={"mi_forward_avg_us": fwd_avg * 1e3, "mi_forward_min_us": float(fwd_ms.min()) * 1e3,
+                                   "mi_backward_avg_us": bwd_avg * 1e3, "mi_backward_min_us": float(bwd_ms.min()) * 1e3})
+        del sets
+        return m
 
     if args.copy_probe:
         src = torch.zeros(64 << 20, dtype=torch.float32, device=dev)  # 256 MiB read + 256 MiB written
@@ -314,40 +362,9 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for k in range(args.steps):
-        step(events[k])
-    if single:
-        events[-1][2].record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_per_step = wall / args.steps * 1e3
     both_bytes = (FWD_BYTES_PER_CELL + BWD_BYTES_PER_CELL) * active
-    if single:
-        # one kernel does the step: its algorithmic bytes are the forward's plus the backward's
-        ends = [e[0] for e in events[1:]] + [events[-1][2]]
-        both_ms = np.array([e[0].elapsed_time(end) for e, end in zip(events, ends)])
-        dom, dom_ms, dom_bytes = "mi_forward_backward", float(both_ms.mean()), both_bytes
-        kernel_times = {"mi_forward_backward_avg_us": dom_ms * 1e3,
-                        "mi_forward_backward_min_us": float(both_ms.min()) * 1e3}
-        both_avg = dom_ms
-    else:
-        fwd_ms = np.array([e[0].elapsed_time(e[1]) for e in events])
-        bwd_ms = np.array([e[1].elapsed_time(e[2]) for e in events])
-        # Roofline of the dominant kernel (the one with the longer average launch).
-        fwd_avg, bwd_avg = float(fwd_ms.mean()), float(bwd_ms.mean())
-        if bwd_avg >= fwd_avg:
-            dom, dom_ms, dom_bytes = "mi_backward", bwd_avg, BWD_BYTES_PER_CELL * active
-        else:
-            dom, dom_ms, dom_bytes = "mi_forward", fwd_avg, FWD_BYTES_PER_CELL * active
-        kernel_times = {"mi_forward_avg_us": fwd_avg * 1e3, "mi_forward_min_us": float(fwd_ms.min()) * 1e3,
-                        "mi_backward_avg_us": bwd_avg * 1e3, "mi_backward_min_us": float(bwd_ms.min()) * 1e3}
-        both_avg = fwd_avg + bwd_avg
+    m = measure(args.input_sets)
+    ms_per_step, dom, dom_ms, dom_bytes, both_avg = m["ms_per_step"], m["dom"], m["dom_ms"], m["dom_bytes"], m["both_avg"]
     achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
     traffic_table = (MEASURED_TRAFFIC_BYTES if keep else MEASURED_TRAFFIC_BYTES_PLAIN_PAIR)
     out = {
@@ -361,22 +378,31 @@ def main():
         "config": {"workload": f"mutual_information_recursion fwd+bwd, fp32, modified, B={B} "
                                f"S={S} T={T}, random boundary (BASELINE config 4)",
                    "active_cells": active, "full_box_cells": full, "log_deriv_kept": bool(keep),
-                   "launches_per_step": 1 if single else 2, "input_sets": len(sets),
+                   "launches_per_step": 1 if single else 2, "input_sets": args.input_sets,
                    "inputs": ("the same px / py every step: at this size the Infinity Cache serves them from "
                               "the second step on, as it does after the builder kernels of the loss functions"
-                              if len(sets) == 1 else
+                              if args.input_sets == 1 else
                               "px / py taken in turn from %d copies, %d MB in all: they come from HBM"
-                              % (len(sets), len(sets) * (px.numel() + py.numel()) * 4 // 1000000))},
+                              % (args.input_sets, m["input_mb"]))},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
                      "traffic": traffic_table.get(dom) if (B, S, T) == (32, 200, 1000) else None,
                      "kernel": dom,
                      "kernel_avg_us": dom_ms * 1e3},
-        "kernels": dict(kernel_times,
+        "kernels": dict(m["kernel_times"],
                         fwd_bwd_GBps_active_cells=both_bytes / (both_avg * 1e-3) / 1e9,
                         fwd_bwd_frac_of_hbm_peak=both_bytes / (both_avg * 1e-3) / 1e9 / HBM_PEAK_GBS,
                         full_box_cells_per_s=full / (both_avg * 1e-3)),
     }
+    if args.input_sets > 1 and not args.no_cache_resident:
+        # the same steps on ONE copy of the inputs, which the Infinity Cache then serves (the
+        # situation inside the loss functions, where a builder kernel has just written px / py)
+        r = measure(1)
+        out["cache_resident"] = {
+            "inputs": "the same px / py every step",
+            "ms_per_step": r["ms_per_step"], "value": active / (r["ms_per_step"] * 1e-3), "unit": "cells/s",
+            "kernel": r["dom"], "kernel_avg_us": r["dom_ms"] * 1e3,
+            "frac_of_hbm_peak": r["dom_bytes"] / (r["dom_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS}
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(c)
     if not args.no_secondary:

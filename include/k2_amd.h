@@ -125,26 +125,34 @@ K2AMD_API int k2amd_mi_backward_kept(const void *px, const void *py, const int64
                            int B, int S, int T, int modified, int dtype, int overwrite_ans_grad,
                            void *workspace, size_t workspace_bytes, void *stream);
 
-/* k2amd_mi_forward_keep followed by k2amd_mi_backward_kept, in ONE launch: what the reference's
- * autograd function does with two native calls when gradients are wanted
- * (k2/python/k2/mutual_information.py:157-169).  It has no counterpart in the reference.
- *   ans [B] out; log_deriv [B][S+1][T+1] scratch (written, then read; contents as above);
- *   ans_grad [B] in (and out if overwrite_ans_grad), or NULL for the reference's torch.ones(B)
- *   (mutual_information.py:163); px_grad, py_grad out, every element written.
- * Same results, bit for bit, as the two calls.  Every workgroup of this launch must be resident
- * at once, so it only serves shapes with 2 * B * ceil((S+1)/64) <= compute units of the current
- * device (twice that where the runtime reports that a unit holds two of its workgroups), fp32,
- * with a workspace: k2amd_mi_forward_backward_supported(...) says whether a call
- * will be served (1) or returns K2AMD_ERR_UNSUPPORTED (0; use the two calls).  It also expects the
- * device not to be busy with other streams' kernels for as long as a second: a workgroup that
- * finds no compute unit free keeps others waiting, and a wait that expires ends the launch with
- * K2AMD_ERR_TIMEOUT in the workspace's status.                                                   */
+/* Forward and backward recursion in ONE launch: what the reference's autograd function does with
+ * two native calls when gradients are wanted (k2/python/k2/mutual_information.py:157-169).  It has
+ * no counterpart in the reference.
+ *   ans [B] out; ans_grad [B] in (and out if overwrite_ans_grad), or NULL for the reference's
+ *   torch.ones(B) (mutual_information.py:163); px_grad, py_grad out, every element written;
+ *   scratch: k2amd_mi_forward_backward_scratch_bytes(...) bytes of device memory that the launch
+ *   writes and then reads (nothing in it is an output).
+ * Every lattice is swept from both ends at once: the first half of its diagonals forward from
+ * the origin, the second half backward from the end cell (the same recursion on px / py read in
+ * reverse); where the two meet, alpha + beta of a cell is the log-weight of all paths through
+ * it, which gives the score and the gradient that each half then carries back to its own end.
+ * The results are those of the two calls to within fp32 rounding of p (not the same bits: the
+ * second half's occupation counts come from beta instead of alpha).  A sequence whose end cell no
+ * path reaches (score -inf) gets the reference's result for that case from the exact kernels'
+ * code inside the same launch.
+ * Work is handed to a fixed set of workgroups in an order in which every wait is for work handed
+ * out earlier, so the launch needs no particular number of resident workgroups and is safe next
+ * to other streams' kernels.  It serves fp32 with a workspace and S + 2 <= 2056:
+ * k2amd_mi_forward_backward_supported(...) says whether a call will be served (1) or returns
+ * K2AMD_ERR_UNSUPPORTED (0; use the two calls).                                                  */
 K2AMD_API int k2amd_mi_forward_backward_supported(int B, int S, int T, int modified, int dtype,
                                         int has_workspace);
+K2AMD_API size_t k2amd_mi_forward_backward_scratch_bytes(int B, int S, int T, int modified, int dtype);
 K2AMD_API int k2amd_mi_forward_backward(const void *px, const void *py, const int64_t *boundary, void *ans,
-                              void *log_deriv, void *ans_grad, void *px_grad, void *py_grad, int B,
-                              int S, int T, int modified, int dtype, int overwrite_ans_grad,
-                              void *workspace, size_t workspace_bytes, void *stream);
+                              void *scratch, size_t scratch_bytes, void *ans_grad, void *px_grad,
+                              void *py_grad, int B, int S, int T, int modified, int dtype,
+                              int overwrite_ans_grad, void *workspace, size_t workspace_bytes,
+                              void *stream);
 
 /* ------------------------------------------------------------------ RNN-T log-prob builders
  *

@@ -36,7 +36,8 @@ _SIGNATURES = {
     "k2amd_mi_forward_keep": ([_vp] * 6 + [_ci] * 5 + [_vp, _sz, _vp], _ci),
     "k2amd_mi_backward_kept": ([_vp] * 8 + [_ci] * 6 + [_vp, _sz, _vp], _ci),
     "k2amd_mi_forward_backward_supported": ([_ci] * 6, _ci),
-    "k2amd_mi_forward_backward": ([_vp] * 8 + [_ci] * 6 + [_vp, _sz, _vp], _ci),
+    "k2amd_mi_forward_backward_scratch_bytes": ([_ci] * 5, _sz),
+    "k2amd_mi_forward_backward": ([_vp] * 5 + [_sz] + [_vp] * 3 + [_ci] * 6 + [_vp, _sz, _vp], _ci),
     "k2amd_rnnt_logprobs_simple_forward": ([_vp] * 11 + [_ci] * 7 + [_vp], _ci),
     "k2amd_rnnt_logprobs_simple_backward": ([_vp] * 11 + [_ci] * 7 + [_vp], _ci),
     "k2amd_rnnt_logprobs_joint_forward": ([_vp] * 6 + [_ci] * 7 + [_vp], _ci),
@@ -253,8 +254,7 @@ def mi_backward(px, py, boundary, p, ans_grad, overwrite_ans_grad=True, log_deri
 
 
 def mi_forward_backward_supported(px, py):
-    """True if mi_forward_backward serves these tensors (fp32, pipelined kernels, and a device with
-    a compute unit for every workgroup of the launch)."""
+    """True if mi_forward_backward serves these tensors (fp32, the pipelined kernels' shapes)."""
     B, S, T1 = px.shape
     T = py.shape[2]
     dt = dtype_code(px)
@@ -268,15 +268,16 @@ def mi_forward_backward(px, py, boundary, ans_grad, overwrite_ans_grad=True):
     B, S, T, modified = _mi_shapes(px, py, boundary)
     expect_optional(ans_grad, "ans_grad", px.dtype, px.device, (B,))
     ans = torch.empty(B, dtype=px.dtype, device=px.device)
-    log_deriv = torch.empty(B, S + 1, T + 1, dtype=px.dtype, device=px.device)
     px_grad = torch.empty_like(px)
     py_grad = torch.empty_like(py)
     dt = dtype_code(px)
+    nbytes = lib().k2amd_mi_forward_backward_scratch_bytes(B, S, T, modified, dt)
+    scratch = torch.empty(max(nbytes, 4), dtype=torch.uint8, device=px.device)
     ws = mi_workspace(B, S, T, modified, dt, px.device)
     with torch.cuda.device(px.device):
-        check(lib().k2amd_mi_forward_backward(ptr(px), ptr(py), ptr(boundary), ptr(ans), ptr(log_deriv),
-                                              ptr(ans_grad), ptr(px_grad), ptr(py_grad), B, S, T,
-                                              modified, dt, int(overwrite_ans_grad), ptr(ws),
+        check(lib().k2amd_mi_forward_backward(ptr(px), ptr(py), ptr(boundary), ptr(ans), ptr(scratch),
+                                              scratch.numel(), ptr(ans_grad), ptr(px_grad), ptr(py_grad),
+                                              B, S, T, modified, dt, int(overwrite_ans_grad), ptr(ws),
                                               0 if ws is None else ws.numel(), stream_ptr(px.device)))
     return ans, px_grad, py_grad
 

@@ -190,20 +190,28 @@ int k2amd_mi_forward_backward_supported(int B, int S, int T, int modified, int d
          !PathIs("two-launches") && MiFusedSupports(B, S, T, modified ? 1 : 0);
 }
 
+size_t k2amd_mi_forward_backward_scratch_bytes(int B, int S, int T, int modified, int dtype) {
+  if (!k2amd_mi_forward_backward_supported(B, S, T, modified, dtype, 1)) return 0;
+  return MiFusedScratchElems(B, S, T) * sizeof(float);
+}
+
 int k2amd_mi_forward_backward(const void *px, const void *py, const int64_t *boundary, void *ans,
-                              void *log_deriv, void *ans_grad, void *px_grad, void *py_grad, int B,
-                              int S, int T, int modified, int dtype, int overwrite_ans_grad,
-                              void *workspace, size_t workspace_bytes, void *stream) {
+                              void *scratch, size_t scratch_bytes, void *ans_grad, void *px_grad,
+                              void *py_grad, int B, int S, int T, int modified, int dtype,
+                              int overwrite_ans_grad, void *workspace, size_t workspace_bytes,
+                              void *stream) {
   if (!ShapeOk(B, S, T) || (dtype != K2AMD_F32 && dtype != K2AMD_F64)) return K2AMD_ERR_INVALID_ARGUMENT;
   if (B == 0) return K2AMD_OK;
-  if (!ans || !log_deriv || (!px && S > 0) || (!py && T > 0) || (!px_grad && S > 0) ||
+  if (!ans || !scratch || (!px && S > 0) || (!py && T > 0) || (!px_grad && S > 0) ||
       (!py_grad && T > 0))
     return K2AMD_ERR_INVALID_ARGUMENT;
   if (!k2amd_mi_forward_backward_supported(B, S, T, modified, dtype, workspace != nullptr))
     return K2AMD_ERR_UNSUPPORTED;
-  if (workspace_bytes < MiFastWorkspaceBytes(B, S, T)) return K2AMD_ERR_WORKSPACE;
+  if (workspace_bytes < MiFastWorkspaceBytes(B, S, T) ||
+      scratch_bytes < k2amd_mi_forward_backward_scratch_bytes(B, S, T, modified, dtype))
+    return K2AMD_ERR_WORKSPACE;
   return MiForwardBackwardFast((const float *)px, (const float *)py, boundary, (float *)ans,
-                               (float *)log_deriv, (float *)ans_grad, (float *)px_grad,
+                               (float *)scratch, (float *)ans_grad, (float *)px_grad,
                                (float *)py_grad, B, S, T, modified ? 1 : 0, overwrite_ans_grad,
                                workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }

@@ -44,10 +44,14 @@
 //
 // Arithmetic is the reference's log-domain recursion (k2/python/csrc/torch/
 // mutual_information_cpu.cu:89-121, log-add of k2/csrc/utils.h:511-563) with hardware exp2/log2.
+#include <algorithm>
 #include <atomic>
 #include <cstdlib>
 
+#include <cstddef>
+
 #include "common.h"
+#include "mi_generic_impl.h"
 #include "mi_internal.h"
 
 namespace k2amd {
@@ -172,6 +176,28 @@ __device__ __forceinline__ float4v AsyncQuad(int4v rs, int idx) {
 }
 __device__ __forceinline__ float4 AsFloat4(float4v v) { return make_float4(v.x, v.y, v.z, v.w); }
 
+// The same load, and a 16-byte store, at device coherence (sc1): they are performed where every
+// compute unit of the device sees them, past the L2 of the issuing unit's XCD, as the
+// device-scope atomic accesses of the edge words are.  The single launch moves the
+// log-derivatives between workgroups this way: a forward sweep's stores are read, later in the
+// same launch, by whichever compute unit sweeps that chunk back, and handing them over with a
+// device-scope release / acquire pair instead would write back and invalidate a whole L2 at
+// every hand-over (measured: 7 us each, and every other workgroup of the XCD slowed down).
+__device__ __forceinline__ float4v AsyncQuadCoherent(int4v rs, int idx) {
+  float4v v;
+  const int off = max(idx, 0) * 4;
+  asm volatile("buffer_load_dwordx4 %0, %1, %2, 0 offen sc1" : "=v"(v) : "v"(off), "s"(rs) : "memory");
+  return v;
+}
+__device__ __forceinline__ void StoreQuadCoherent(float *ptr, float4 v) {
+  float4v w;
+  w.x = v.x; w.y = v.y; w.z = v.z; w.w = v.w;
+  asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(ptr), "v"(w) : "memory");
+}
+__device__ __forceinline__ void StoreCoherent(float *ptr, float v) {
+  __hip_atomic_store(ptr, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // A quad whose first float would lie in front of the tensor (idx < 0: only possible for the
 // tensor's very first row) is loaded from index 0 instead; this moves the floats back to the
 // positions they were asked for.  The floats in front of the tensor belong to columns outside
@@ -203,6 +229,31 @@ struct ChunkGeom {
   int skew;
   int nblocks;
 };
+
+// The part of a sequence's lattice that one sweep covers.  The single launch splits every lattice
+// at a "cut" diagonal (cells with s + t = const on a regular lattice, a column on a modified
+// one) into two halves that are swept at the same time: the first half in the lattice's own
+// coordinates from the origin up to the cut, the second half MIRRORED, i.e. from the end cell
+// back to the cut in coordinates s' = ns - s, t' = nt - t, in which the recursion for
+//     beta[s][t] = log_add(px[s][t] + beta[s+1][t-o], py[s][t] + beta[s][t+1])
+// is the forward recursion again, on px and py read backwards along both axes.  A sweep over a
+// half works in ITS coordinates throughout; only the addresses of what it loads and stores know
+// about the mirror.  dmax = last diagonal of the half (own coordinates).  The two-kernel pair
+// sweeps whole lattices: kBidir = false compiles all of this away.
+struct Half {
+  int mirror;  // 0: own coordinates = the lattice's; 1: reversed along both axes
+  int dmax;    // cells with row * skew + column <= dmax belong to the half
+#ifdef K2AMD_MI_TRACE
+  unsigned long long *trace;
+#endif
+};
+#ifdef K2AMD_MI_TRACE
+#define K2AMD_TRACE_MARK(half, i) do { if ((half).trace != nullptr && threadIdx.x == 0) (half).trace[i] = wall_clock64(); } while (0)
+#else
+#define K2AMD_TRACE_MARK(half, i) do { } while (0)
+#endif
+
+__device__ __forceinline__ float4 Rev4(float4 v) { return make_float4(v.w, v.z, v.y, v.x); }
 
 enum Role { kChain = 0, kEdge = 1, kLoader = 2, kStorer = 3 };
 
@@ -275,6 +326,16 @@ __device__ __forceinline__ void PublishEdge(float *addr, float v) {
                      __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// Values on the cut diagonal go through device-coherent stores and loads like the edge words (the
+// reader is another workgroup, on any compute unit), but need no sentinel: a counter says when
+// all of a sequence's values are there.
+__device__ __forceinline__ void PublishCut(float *addr, float v) {
+  __hip_atomic_store(addr, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float ReadCut(const float *addr) {
+  return __hip_atomic_load(addr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // ------------------------------------------------------------------------------ forward
 //
 // Lane q of the chain wavefront owns lattice row row0 + q and is at column j = n - q*skew at step
@@ -319,33 +380,52 @@ constexpr int kFwdLoadsPerBlock = 2 * FwdLayout::kLoadItems + 1;
 // hold values the backward never uses.  kWriteP = false (only with kKeep): p itself is not stored,
 // for callers that want nothing but ans and the gradients.
 // The whole workgroup sweeps chunk `chunk` (64 lattice rows) of sequence `seq`.
-template <bool kKeep, bool kWriteP>
+// kBidir: the sweep covers the half `half` of the lattice (see Half) and ends on its cut
+// diagonal; what the chain holds there (p of the half's last cell of every row) goes to
+// cut_out[0..63] (the chunk's 64 own rows; the finite stand-in for -inf where a row has no cell
+// on the cut or lies past the sequence's last row), ans is not written, and log_deriv has rows of
+// Tn + 2 floats (the two halves of a sequence share one slab: the mirrored half's cells lie one
+// column to the right of their place, where no cell of the other half is).
+template <bool kKeep, bool kWriteP, bool kBidir>
 __device__ __forceinline__ void MiForwardChunk(
-    FwdLds &lds, const float *__restrict__ px, const float *__restrict__ py,
-    const int64_t *__restrict__ boundary, float *__restrict__ p, float *__restrict__ ans,
+    FwdLds &lds, const float *__restrict__ px, const float *__restrict__ py, const Box &box,
+    float *__restrict__ p, float *__restrict__ ans,
     float *__restrict__ log_deriv, FastHeader *hdr, float *edge, int B, int S, int Tn,
-    int modified, int nchunks, int edge_stride, int seq, int chunk) {
+    int modified, int nchunks, int edge_stride, int seq, int chunk, Half half, float *cut_out) {
+  static_assert(!kBidir || (kKeep && !kWriteP), "the halves keep the log-derivatives only");
   ChunkGeom g;
   g.b = seq;
   g.c = chunk;
-  const Box box = LoadBox(boundary, g.b, S, Tn);
   g.s0 = box.s0; g.t0 = box.t0; g.ns = box.s1 - box.s0; g.nt = box.t1 - box.t0;
   g.row0 = g.c * kRows;
   if (!box.ok || g.row0 > g.ns) {
-    if (!box.ok && g.c == 0 && threadIdx.x == 0) ans[g.b] = __builtin_nanf("");
+    if (!kBidir && !box.ok && g.c == 0 && threadIdx.x == 0) ans[g.b] = __builtin_nanf("");
     return;
   }
   g.skew = modified ? 0 : 1;
-  const bool has_down = g.row0 + kRows <= g.ns;
-  const int nsteps = g.nt + 1 + (kRows - 1) * g.skew;  // last needed step index + 1
-  g.nblocks = (nsteps + kW - 1) / kW;
+  const int mirror = kBidir ? half.mirror : 0;
+  const int nsteps_full = g.nt + 1 + (kRows - 1) * g.skew;  // last needed step index + 1
+  // steps (and 32-step blocks) that the chunk at local row r0 runs: up to the cut diagonal
+  auto steps_of = [&](int r0) { return kBidir ? min(nsteps_full, half.dmax - r0 * g.skew + 1) : nsteps_full; };
+  auto blocks_of = [&](int r0) { return max(steps_of(r0) + kW - 1, 0) / kW; };
+  const int nsteps = steps_of(g.row0);
+  const int n_last = nsteps - 1;  // the chunk's step on the cut diagonal (kBidir)
+  g.nblocks = blocks_of(g.row0);
+  if (kBidir && g.nblocks == 0) {  // no cell of these rows lies in the half
+    if (threadIdx.x < kRows) PublishCut(cut_out + threadIdx.x, kLogZero);
+    return;
+  }
+  const bool has_down = g.row0 + kRows <= g.ns && blocks_of(g.row0 + kRows) > 0;
+  const int nblocks_down = has_down ? blocks_of(g.row0 + kRows) : 0;
+  const int nblocks_up = g.c > 0 ? blocks_of(g.row0 - kRows) : 0;
   const int edge_shift = kRows * g.skew - 1;  // step n here <-> step n + edge_shift one chunk up
 
   const int T1 = modified ? Tn : Tn + 1;
+  const int LS = kBidir ? Tn + 2 : Tn + 1;  // floats per row of log_deriv
   const float *pxb = px + (size_t)g.b * S * T1;
   const float *pyb = py + (size_t)g.b * (S + 1) * Tn;
   float *pb = kWriteP ? p + (size_t)g.b * (S + 1) * (Tn + 1) : nullptr;
-  float *ldb = kKeep ? log_deriv + (size_t)g.b * (S + 1) * (Tn + 1) : nullptr;
+  float *ldb = kKeep ? log_deriv + (size_t)g.b * (S + 1) * LS : nullptr;
   float *edge_out = edge + ((size_t)g.b * nchunks + g.c + 1) * edge_stride;  // read by chunk c+1
   float *edge_in = edge + ((size_t)g.b * nchunks + g.c) * edge_stride;
 
@@ -371,11 +451,20 @@ __device__ __forceinline__ void MiForwardChunk(
     rowy_ok[it] = row_i <= g.ns;
     const int rx = min(max(row_i, 1), max(g.ns, 1)) - 1;  // a px row inside the box if any
     const int ry = min(row_i, g.ns);
-    idx_x[it] = (g.b * S + g.s0 + rx) * T1 + g.t0;
-    idx_y[it] = (g.b * (S + 1) + g.s0 + ry) * Tn + g.t0;
+    // mirrored: own row r of px is the lattice's row ns-1-r, own column c its column hi_x-c (py:
+    // row ns-r, column nt-1-c), so own column c lies at index idx - c
+    idx_x[it] = mirror ? (g.b * S + g.s0 + max(g.ns - 1 - rx, 0)) * T1 + g.t0 + hi_x
+                       : (g.b * S + g.s0 + rx) * T1 + g.t0;
+    idx_y[it] = mirror ? (g.b * (S + 1) + g.s0 + g.ns - ry) * Tn + g.t0 + hi_y
+                       : (g.b * (S + 1) + g.s0 + ry) * Tn + g.t0;
   }
   // float index of local column 0 of the row above the chunk (any px row where there is none)
-  const int idx_above = (g.b * S + g.s0 + max(g.row0 - 1, 0)) * T1 + g.t0;
+  const int row_above = max(g.row0 - 1, 0);
+  const int idx_above = mirror ? (g.b * S + g.s0 + max(g.ns - 1 - row_above, 0)) * T1 + g.t0 + hi_x
+                               : (g.b * S + g.s0 + row_above) * T1 + g.t0;
+  // index of the quad that holds own columns c .. c+3 of a row whose column 0 is at idx (mirrored:
+  // the quad comes back in descending column order, see Unmirror)
+  auto quad_at = [&](int idx, int c) { return mirror ? idx - c - 3 : idx + c; };
   // every quad of every row of block kb inside the valid columns?  (uniform over the workgroup)
   auto interior = [&](int kb) {
     return kb * kW - 1 - (kRows - 1) * g.skew >= 0 && kb * kW + 30 <= g.nt - 1;
@@ -389,12 +478,17 @@ __device__ __forceinline__ void MiForwardChunk(
 #pragma unroll
     for (int it = 0; it < kLoadItems; ++it) {
       const int jp = kb * kW + 4 * mm - 1 - (lq + kRowStep * it) * g.skew;  // column left of element 0
-      r.x[it] = AsyncQuad(rsx, idx_x[it] + jp + g.skew);
-      r.y[it] = AsyncQuad(rsy, idx_y[it] + jp);
+      r.x[it] = AsyncQuad(rsx, quad_at(idx_x[it], jp + g.skew));
+      r.y[it] = AsyncQuad(rsy, quad_at(idx_y[it], jp));
     }
     // every lane asks (the count of loads in flight is the same for all wavefronts); the eight
     // lanes of loader row 0 keep what arrives
-    r.above = AsyncQuad(rsx, idx_above + (kb + 1) * kW + 4 * mm - 1 + g.skew);
+    r.above = AsyncQuad(rsx, quad_at(idx_above, (kb + 1) * kW + 4 * mm - 1 + g.skew));
+  };
+  // a loaded quad in ascending order of own columns (`at` = the index it was loaded from)
+  auto unmirror = [&](float4 v, int at, bool rim) {
+    if (rim && g.b == 0) v = ShiftQuad(v, at);  // the only sequence whose rows can start the tensor
+    return mirror ? Rev4(v) : v;
   };
   // `inner` is uniform over the workgroup: the masking code for blocks on the rim of the box is
   // a real branch (the empty asm statement keeps the compiler from flattening it into selects
@@ -408,6 +502,10 @@ __device__ __forceinline__ void MiForwardChunk(
       float4 qx = AsFloat4(r.x[it]), qy = AsFloat4(r.y[it]);
       float vx[4], vy[4];
       if (inner) {
+        if (kBidir) {
+          qx = unmirror(qx, 0, false);
+          qy = unmirror(qy, 0, false);
+        }
         const float in_x[4] = {qx.x, qx.y, qx.z, qx.w}, in_y[4] = {qy.x, qy.y, qy.z, qy.w};
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -418,10 +516,8 @@ __device__ __forceinline__ void MiForwardChunk(
         asm volatile("");
         const int jp = kb * kW + 4 * mm - 1 - q * g.skew;
         const int jx = jp + g.skew;
-        if (g.b == 0) {  // the only sequence whose rows can start the tensor
-          qx = ShiftQuad(qx, idx_x[it] + jx);
-          qy = ShiftQuad(qy, idx_y[it] + jp);
-        }
+        qx = unmirror(qx, quad_at(idx_x[it], jx), true);
+        qy = unmirror(qy, quad_at(idx_y[it], jp), true);
         const float in_x[4] = {qx.x, qx.y, qx.z, qx.w}, in_y[4] = {qy.x, qy.y, qy.z, qy.w};
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -440,7 +536,7 @@ __device__ __forceinline__ void MiForwardChunk(
   // the set of block kb carries the row above the chunk for block kb + 1
   auto commit_above = [&](int kb, FwdRegs &r) {
     if (lq != 0 || kb + 1 >= g.nblocks) return;
-    const float4 qa = AsFloat4(r.above);
+    const float4 qa = unmirror(AsFloat4(r.above), quad_at(idx_above, (kb + 1) * kW + 4 * mm - 1 + g.skew), true);
     const float in[4] = {qa.x, qa.y, qa.z, qa.w};
     float v[4];
 #pragma unroll
@@ -454,8 +550,10 @@ __device__ __forceinline__ void MiForwardChunk(
   // ---- storers ---------------------------------------------------------------------------
   auto store_block = [&](int kb) {  // LDS ring -> p
     if (kb < 0) return;
-    // columns kb*32 - 63*skew .. kb*32 + 31 all inside 0..nt-1 (the end cell is never "inner")
-    const bool inner = kb * kW - (kRows - 1) * g.skew >= 0 && kb * kW + kW - 1 <= g.nt - 1;
+    // columns kb*32 - 63*skew .. kb*32 + 31 all inside 0..nt-1 (the end cell is never "inner"),
+    // and every step of the block inside the half
+    const bool inner = kb * kW - (kRows - 1) * g.skew >= 0 && kb * kW + kW - 1 <= g.nt - 1 &&
+                       (!kBidir || kb * kW + kW - 1 <= n_last);
 #pragma unroll
     for (int it = 0; it < 2; ++it) {
       const int q = mq + 32 * it;
@@ -472,7 +570,10 @@ __device__ __forceinline__ void MiForwardChunk(
         v.w = v.w < kLogZeroTest ? ninf : v.w;
       }
       const int j = kb * kW + 4 * mm - q * g.skew;  // column of element 0
-      const size_t at = (size_t)(g.s0 + row_i) * (Tn + 1) + g.t0 + j;
+      // where own columns j .. j+3 of the row lie: the mirrored half stores the lattice's cell
+      // (ns - row, nt - column) one column to the right of its place, columns descending
+      const ptrdiff_t at = mirror ? (ptrdiff_t)(g.s0 + g.ns - row_i) * LS + g.t0 + g.nt - j - 2
+                                  : (ptrdiff_t)(g.s0 + row_i) * LS + g.t0 + j;
       float *dst = pb + at;
       float ld[4] = {0.f, 0.f, 0.f, 0.f};
       if (kKeep) {
@@ -508,17 +609,24 @@ __device__ __forceinline__ void MiForwardChunk(
       }
       if (inner) {  // uniform: every column of the block lies in 0..nt-1 for every row
         if (kWriteP) StoreQuad(dst, v);
-        if (kKeep) StoreQuad(ldb + at, make_float4(ld[0], ld[1], ld[2], ld[3]));
+        if (kKeep) {
+          const float4 l4 = make_float4(ld[0], ld[1], ld[2], ld[3]);
+          if (kBidir) StoreQuadCoherent(ldb + at, mirror ? Rev4(l4) : l4);
+          else StoreQuad(ldb + at, l4);
+        }
       } else {
         asm volatile("");  // keeps this path a branch of its own
         const float vv[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          if (j + e >= 0 && j + e <= g.nt) {
+          if (j + e >= 0 && j + e <= g.nt && (!kBidir || j + e + q * g.skew <= n_last)) {
             if (kWriteP) dst[e] = vv[e];
-            if (kKeep) ldb[at + e] = ld[e];
+            if (kKeep) {
+              if (kBidir) StoreCoherent(ldb + at + (mirror ? 3 - e : e), ld[e]);
+              else ldb[at + e] = ld[e];
+            }
           }
-        if (row_i == g.ns) {
+        if (!kBidir && row_i == g.ns) {
 #pragma unroll
           for (int e = 0; e < 4; ++e)
             if (j + e == g.nt) ans[g.b] = GaveUp(hdr) ? __builtin_nanf("") : vv[e];
@@ -539,7 +647,8 @@ __device__ __forceinline__ void MiForwardChunk(
     const int jx = kb * kW + lane - 1 + g.skew;
     float v = kLogZero;
     if (g.c > 0 && lane < kW && jx >= 0 && jx <= hi_x)
-      v = fmaxf(pxb[(size_t)(g.s0 + g.row0 - 1) * T1 + g.t0 + jx], kLogZero);
+      v = fmaxf(mirror ? pxb[(size_t)(g.s0 + g.ns - g.row0) * T1 + g.t0 + hi_x - jx]
+                       : pxb[(size_t)(g.s0 + g.row0 - 1) * T1 + g.t0 + jx], kLogZero);
     return v;
   };
   auto take_block = [&](int kb, float px_above) {
@@ -550,7 +659,7 @@ __device__ __forceinline__ void MiForwardChunk(
         if (n == 0) v = 0.0f;  // the origin: p[s_begin][t_begin] = 0 "arrives" at step 0
       } else {
         const int idx = n + edge_shift;
-        if (idx >= 0 && idx < g.nblocks * kW) v = TakeEdge(edge_in + idx, hdr, kLogZero) + px_above;
+        if (idx >= 0 && idx < nblocks_up * kW) v = TakeEdge(edge_in + idx, hdr, kLogZero) + px_above;
       }
       reinterpret_cast<float *>(lds.fx[kWave])[(kb % 3) * kW + lane] = v;
     }
@@ -561,7 +670,7 @@ __device__ __forceinline__ void MiForwardChunk(
     if (has_down && kb >= 0 && lane >= kW) {
       const int n = kb * kW + (lane - kW);
       // the chunk below takes word n at its step n - edge_shift, which must exist
-      if (n >= edge_shift && n - edge_shift < g.nblocks * kW)
+      if (n >= edge_shift && n - edge_shift < nblocks_down * kW)
         PublishEdge(edge_out + n, reinterpret_cast<const float *>(
                                       &lds.fy[kWave - 1][0])[(kb % 3) * kW + (lane - kW)]);
     }
@@ -612,7 +721,9 @@ __device__ __forceinline__ void MiForwardChunk(
   } else if (role == kEdge) {
     take_block(0, edge_px(0));
   }
+  K2AMD_TRACE_MARK(half, 4);
   LdsBarrier();
+  K2AMD_TRACE_MARK(half, 5);
 
   // In iteration kb the chain wavefront computes block kb; the loaders commit block kb+1 (loaded
   // kFwdSets iterations ago) and start the loads of block kb+1+kFwdSets; the storers drain block kb-1; the
@@ -654,8 +765,18 @@ __device__ __forceinline__ void MiForwardChunk(
       px_above = lds.px_above[(kb + 2) & 3][lane & (kW - 1)];  // committed in this iteration
     }
   }
+  K2AMD_TRACE_MARK(half, 6);
   if (role == kStorer) store_block(g.nblocks - 1);
   if (role == kEdge) publish_block(g.nblocks - 1);
+  if (kBidir) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the coherent stores above
+  if (kBidir && wave == 2 + L::kLoaderWaves) {
+    // What the chain left on the cut diagonal: step n_last of every row, still in the ring.  (A
+    // chunk that ran out of columns before the cut has no cell on it; a row whose cell on the cut
+    // lies outside the columns holds a stand-in for -inf there already.)
+    const int at = ((g.nblocks - 1) % 3) * kW + (n_last - (g.nblocks - 1) * kW);
+    const bool on_cut = half.dmax - g.row0 * g.skew == n_last && g.row0 + lane <= g.ns;
+    PublishCut(cut_out + lane, on_cut ? reinterpret_cast<const float *>(&lds.fy[lane][0])[at] : kLogZero);
+  }
 }
 
 // One workgroup per chunk; the ticket fixes which (see the file header).
@@ -669,9 +790,10 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiForwardFastKernel(
   if (threadIdx.x == 0) lds.ticket = atomicAdd(&hdr->ticket, 1u);
   __syncthreads();
   const unsigned ticket = lds.ticket;
-  MiForwardChunk<kKeep, kWriteP>(lds, px, py, boundary, p, ans, log_deriv, hdr, edge, B, S, Tn,
-                                 modified, nchunks, edge_stride, (int)(ticket / nchunks),
-                                 (int)(ticket % nchunks));
+  MiForwardChunk<kKeep, kWriteP, false>(lds, px, py, LoadBox(boundary, (int)(ticket / nchunks), S, Tn), p,
+                                        ans, log_deriv, hdr, edge, B, S, Tn, modified, nchunks,
+                                        edge_stride, (int)(ticket / nchunks), (int)(ticket % nchunks),
+                                        Half{}, nullptr);
   if (threadIdx.x == 0) FinishWorkgroup(hdr, gridDim.x);
 }
 
@@ -760,17 +882,21 @@ __device__ __forceinline__ void ZeroItem(const ZeroGeom &z, int r, int c) {
 // read, and every cell's d1 is exp() of one loaded value.
 // The whole workgroup sweeps chunk `chunk` of sequence `seq`, or (zero_only) clears what the
 // sweep leaves unassigned in array rows chunk * 64 .. chunk * 64 + 63 of that sequence.
-template <bool kKept>
+// kBidir: the sweep covers the half `half` (see Half), whose forward sweep left its
+// log-derivatives in `p` (rows of Tn + 2 floats); it starts on the cut diagonal, where row
+// row0 + q of the half holds gradient seeds[q] (its cell's share of all paths, times the
+// gradient of the sequence's score), instead of at the end cell.
+template <bool kKept, bool kBidir>
 __device__ __forceinline__ void MiBackwardChunk(
-    BwdLds &lds, const float *__restrict__ px, const float *__restrict__ p,
-    const int64_t *__restrict__ boundary, float *__restrict__ ans_grad,
+    BwdLds &lds, const float *__restrict__ px, const float *__restrict__ p, const Box &box,
+    float *__restrict__ ans_grad,
     float *__restrict__ px_grad, float *__restrict__ py_grad, FastHeader *hdr, float *edge, int B,
     int S, int Tn, int modified, int nchunks, int edge_stride, int overwrite_ans_grad, int seq,
-    int chunk, bool zero_only) {
+    int chunk, bool zero_only, Half half, const float *seeds) {
+  static_assert(!kBidir || kKept, "the halves hand over log-derivatives");
   ChunkGeom g;
   g.b = seq;
   g.c = chunk;
-  const Box box = LoadBox(boundary, g.b, S, Tn);
   const int T1 = modified ? Tn : Tn + 1;
   const int off = modified ? -1 : 0;
   float *gxb = px_grad + (size_t)g.b * S * T1;
@@ -793,10 +919,20 @@ __device__ __forceinline__ void MiBackwardChunk(
   g.row0 = g.c * kRows;
   if (!box.ok || g.row0 > g.ns) return;  // nothing to sweep
   g.skew = modified ? 0 : 1;
-  const bool has_down = g.row0 + kRows <= g.ns;
+  const int mirror = kBidir ? half.mirror : 0;
+  const int npos_full = g.nt + 2 + (kRows - 1) * g.skew;  // one virtual column right of the end cell
+  // positions (and 32-position blocks) of the chunk at local row r0: one past its step on the cut
+  auto npos_of = [&](int r0) { return kBidir ? min(npos_full, half.dmax - r0 * g.skew + 2) : npos_full; };
+  auto blocks_of = [&](int r0) { return npos_of(r0) >= 2 ? (npos_of(r0) + kW - 1) / kW : 0; };
+  const int npos = npos_of(g.row0);
+  const int n_last = npos - 2;  // the chunk's position on the cut diagonal (kBidir)
+  g.nblocks = blocks_of(g.row0);
+  if (kBidir && g.nblocks == 0) return;  // no cell of these rows lies in the half
+  const bool has_down = g.row0 + kRows <= g.ns && blocks_of(g.row0 + kRows) > 0;
   const bool has_up = g.c > 0;
-  const int npos = g.nt + 2 + (kRows - 1) * g.skew;  // one virtual column right of the end cell
-  g.nblocks = (npos + kW - 1) / kW;
+  const int nblocks_down = has_down ? blocks_of(g.row0 + kRows) : 0;
+  const int nblocks_up = has_up ? blocks_of(g.row0 - kRows) : 0;
+  const int LS = kBidir ? Tn + 2 : Tn + 1;  // floats per row of p / the log-derivatives
   const int edge_shift = kRows * g.skew;  // position m here <-> position m - edge_shift one chunk down
   float *edge_out = edge + ((size_t)g.b * nchunks + g.c) * edge_stride;     // read by chunk c-1
   float *edge_in = edge + ((size_t)g.b * nchunks + g.c + 1) * edge_stride;  // from chunk c+1
@@ -811,7 +947,7 @@ __device__ __forceinline__ void MiBackwardChunk(
 
   // ---- loaders ---------------------------------------------------------------------------
   // destination cells with both edges exist only for rows 1..ns and columns 1..nt
-  const int4v rsp = MakeResource(p, (size_t)B * (S + 1) * (Tn + 1));
+  const int4v rsp = MakeResource(p, (size_t)B * (S + 1) * LS);
   const int4v rsx = MakeResource(px, (size_t)B * S * T1);
   // float index of destination column 0 of the item's row: p[dest], and p / px of the source
   // cell of the px edge (column jd - 1 + skew of the row above)
@@ -819,13 +955,21 @@ __device__ __forceinline__ void MiBackwardChunk(
 #pragma unroll
   for (int it = 0; it < kLoadItems; ++it) {
     const int rc = min(max(g.row0 + lq + kRowStep * it, 1), max(g.ns, 1));  // a row with a row above
-    idx_d[it] = (g.b * (S + 1) + g.s0 + rc) * (Tn + 1) + g.t0;
+    // the mirrored half's cell (row, column) lies at lattice cell (ns - row, nt - column), one
+    // column to the right: own column c of the row is at index idx - c
+    idx_d[it] = mirror ? (g.b * (S + 1) + g.s0 + g.ns - rc) * LS + g.t0 + g.nt + 1
+                       : (g.b * (S + 1) + g.s0 + rc) * LS + g.t0;
     idx_s[it] = (g.b * (S + 1) + g.s0 + rc - 1) * (Tn + 1) + g.t0 + g.skew - 1;
     idx_x[it] = (g.b * S + g.s0 + rc - 1) * T1 + g.t0 + g.skew - 1;
   }
-  // every destination cell of block kb has both edges inside the box?  (uniform)
+  // index of the quad that holds own columns c .. c+3 of a row whose column 0 is at idx (mirrored:
+  // the quad comes back in descending column order)
+  auto quad_at = [&](int idx, int c) { return mirror ? idx - c - 3 : idx + c; };
+  // every destination cell of block kb has both edges inside the box (and lies in the half)?
+  // (uniform)
   auto interior = [&](int kb) {
-    return kb * kW - (kRows - 1) * g.skew >= 1 && kb * kW + 31 <= g.nt;
+    return kb * kW - (kRows - 1) * g.skew >= 1 && kb * kW + 31 <= g.nt &&
+           (!kBidir || kb * kW + 31 <= n_last);
   };
   // Rows past the sequence's last row never change: their E / OME stay at the zeros written
   // here, the loaders skip them.
@@ -853,7 +997,7 @@ __device__ __forceinline__ void MiBackwardChunk(
 #pragma unroll
     for (int it = 0; it < kLoadItems; ++it) {
       const int jd = kb * kW + 4 * mm - (lq + kRowStep * it) * g.skew;  // destination column of element 0
-      r.d[it] = AsyncQuad(rsp, idx_d[it] + jd);
+      r.d[it] = kBidir ? AsyncQuadCoherent(rsp, quad_at(idx_d[it], jd)) : AsyncQuad(rsp, quad_at(idx_d[it], jd));
       if (!kKept) {
         r.s[it] = AsyncQuad(rsp, idx_s[it] + jd);
         r.x[it] = AsyncQuad(rsx, idx_x[it] + jd);
@@ -882,7 +1026,7 @@ __device__ __forceinline__ void MiBackwardChunk(
     *o_out = fin ? 1.0f - d1 : 0.0f;
   };
   // The same for a cell on or outside the rim of the box (column j; select-only code).
-  auto rim = [&](bool first_row, bool last_row, int j, float *e_io, float *o_io) {
+  auto rim = [&](bool first_row, bool last_row, int j, int m, float *e_io, float *o_io) {
     const bool in = j >= 1 && j <= g.nt;
     const bool col0_up = j == 0 && !modified;  // regular first column flows up
     float e_v = in ? *e_io : (col0_up ? 1.0f : 0.0f);
@@ -890,8 +1034,9 @@ __device__ __forceinline__ void MiBackwardChunk(
     // first row: everything flows along py
     e_v = first_row ? 0.0f : e_v;
     o_v = first_row ? (in ? 1.0f : 0.0f) : o_v;
-    // virtual cells right of the end cell hand the seed leftwards unchanged
-    const bool virt = last_row && j > g.nt;
+    // virtual cells right of the end cell hand the seed leftwards unchanged; so do, in a half,
+    // the positions past the cut diagonal in every row
+    const bool virt = kBidir ? m > n_last : last_row && j > g.nt;
     *e_io = virt ? 0.0f : e_v;
     *o_io = virt ? 1.0f : o_v;
   };
@@ -909,12 +1054,13 @@ __device__ __forceinline__ void MiBackwardChunk(
       if (!inner && g.b == 0) {  // the only sequence whose rows can start the tensor
         asm volatile("");
         const int jd0 = kb * kW + 4 * mm - q * g.skew;
-        qd = ShiftQuad(qd, idx_d[it] + jd0);
+        qd = ShiftQuad(qd, quad_at(idx_d[it], jd0));
         if (!kKept) {
           qs = ShiftQuad(qs, idx_s[it] + jd0);
           qx = ShiftQuad(qx, idx_x[it] + jd0);
         }
       }
+      if (kBidir && mirror) qd = Rev4(qd);
       float ve[4], vo[4];
       flow(qd.x, qs.x, qx.x, &ve[0], &vo[0]);
       flow(qd.y, qs.y, qx.y, &ve[1], &vo[1]);
@@ -935,7 +1081,8 @@ __device__ __forceinline__ void MiBackwardChunk(
         const int row_i = g.row0 + q;
         const int jd = kb * kW + 4 * mm - q * g.skew;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) rim(row_i == 0, row_i == g.ns, jd + e, &ve[e], &vo[e]);
+        for (int e = 0; e < 4; ++e)
+          rim(row_i == 0, row_i == g.ns, jd + e, jd + e + q * g.skew, &ve[e], &vo[e]);
       }
       const int pq = (kb % 3) * kQuadsPerBlock + mm;
       lds.e[q][pq] = make_float4(ve[0], ve[1], ve[2], ve[3]);
@@ -971,21 +1118,31 @@ __device__ __forceinline__ void MiBackwardChunk(
       const int s = g.s0 + row_i;
       // py_grad[s][t0 + jd - 1 + e]   for destination columns 1..nt
       // px_grad[s-1][t0 + jd - 1 + skew + e]   for destination columns (1 - skew)..nt
-      float *dy = gyb + (size_t)s * Tn + g.t0 + jd - 1;
-      float *dx = gxb + (size_t)(s - 1) * T1 + g.t0 + jd - 1 + g.skew;
+      // The mirrored half's destination cell (row, column) is the lattice's cell
+      // (ns - row, nt - column), and what flows into it along its px / py edge is the flow
+      // OUT of that lattice cell along px / py: both gradients land at that cell's own index,
+      // columns descending.
+      const int sm = g.s0 + g.ns - row_i;
+      float *dy = mirror ? gyb + (ptrdiff_t)sm * Tn + g.t0 + g.nt - jd - 3
+                         : gyb + (ptrdiff_t)s * Tn + g.t0 + jd - 1;
+      float *dx = mirror ? gxb + (ptrdiff_t)sm * T1 + g.t0 + g.nt - jd - 3
+                         : gxb + (ptrdiff_t)(s - 1) * T1 + g.t0 + jd - 1 + g.skew;
       if (inner) {  // uniform: every cell of the block has both edges inside the box
-        StoreQuad(dy, make_float4(cv[0], cv[1], cv[2], cv[3]));
-        if (row_i >= 1) StoreQuad(dx, make_float4(hv[0], hv[1], hv[2], hv[3]));
+        const float4 c4 = make_float4(cv[0], cv[1], cv[2], cv[3]), h4 = make_float4(hv[0], hv[1], hv[2], hv[3]);
+        StoreQuad(dy, kBidir && mirror ? Rev4(c4) : c4);
+        if (row_i >= 1) StoreQuad(dx, kBidir && mirror ? Rev4(h4) : h4);
       } else {
         asm volatile("");  // keeps this path a branch of its own
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          if (jd + e >= 1 && jd + e <= g.nt) dy[e] = cv[e];
+          if (jd + e >= 1 && jd + e <= g.nt && (!kBidir || jd + e + q * g.skew <= n_last))
+            dy[kBidir && mirror ? 3 - e : e] = cv[e];
         if (row_i >= 1) {
           const int lo = 1 - g.skew;
 #pragma unroll
           for (int e = 0; e < 4; ++e)
-            if (jd + e >= lo && jd + e <= g.nt) dx[e] = hv[e];
+            if (jd + e >= lo && jd + e <= g.nt && (!kBidir || jd + e + q * g.skew <= n_last))
+              dx[kBidir && mirror ? 3 - e : e] = hv[e];
         }
       }
     }
@@ -998,7 +1155,7 @@ __device__ __forceinline__ void MiBackwardChunk(
       float v = 0.0f;
       if (has_down) {
         const int idx = mpos - edge_shift;  // position of the same column in the chunk below
-        if (idx >= 0) v = TakeEdge(edge_in + idx, hdr, 0.0f);
+        if (idx >= 0 && idx < nblocks_down * kW) v = TakeEdge(edge_in + idx, hdr, 0.0f);
       }
       reinterpret_cast<float *>(lds.e[kWave])[(kb % 3) * kW + lane] = v;
     }
@@ -1010,7 +1167,7 @@ __device__ __forceinline__ void MiBackwardChunk(
     if (has_up && kb < g.nblocks && lane >= kW) {
       const int i = lane - kW;
       const int mpos = kb * kW + i;
-      if (mpos + edge_shift < g.nblocks * kW) {
+      if (mpos + edge_shift < nblocks_up * kW) {
         const float e0 = reinterpret_cast<const float *>(&lds.e[0][0])[(kb % 3) * kW + i];
         const int right = i + 1 < kW ? (kb % 3) * kW + i + 1 : ((kb + 1) % 3) * kW;
         PublishEdge(edge_out + mpos, e0 * reinterpret_cast<const float *>(&lds.g[0][0])[right]);
@@ -1022,7 +1179,11 @@ __device__ __forceinline__ void MiBackwardChunk(
   // gradient at the (virtual) right end of each row: the seed on the sequence's last row
   float G = 0.0f;
   // (the single launch may come without ans_grad: every sequence's score then has gradient 1)
-  if (role == kChain && g.row0 + lane == g.ns) G = ans_grad != nullptr ? ans_grad[g.b] : 1.0f;
+  if (kBidir) {
+    if (role == kChain) G = seeds[lane];
+  } else if (role == kChain && g.row0 + lane == g.ns) {
+    G = ans_grad != nullptr ? ans_grad[g.b] : 1.0f;
+  }
   float g_origin = 0.0f;
   // Per position (descending), with OME of the own row and Edn = d1 of the row below (lane + 1):
   //     G' = OME * G + Edn * G(lane + 1)
@@ -1071,7 +1232,9 @@ __device__ __forceinline__ void MiBackwardChunk(
   } else if (role == kEdge) {
     take_block(top);
   }
+  K2AMD_TRACE_MARK(half, 4);
   LdsBarrier();
+  K2AMD_TRACE_MARK(half, 5);
 
   // Descending twin of the forward's loops: in iteration kb the chain computes block kb, the
   // loaders commit block kb-1 and start the loads of block kb-3, the storers drain block kb+1,
@@ -1108,9 +1271,10 @@ __device__ __forceinline__ void MiBackwardChunk(
       LdsBarrier();
     }
   }
+  K2AMD_TRACE_MARK(half, 6);
   if (role == kStorer) store_block(0);
   if (role == kEdge) publish_block(0);
-  if (overwrite_ans_grad && ans_grad != nullptr && role == kChain && g.c == 0 && lane == 0)
+  if (overwrite_ans_grad && ans_grad != nullptr && role == kChain && g.c == 0 && lane == 0 && !mirror)
     ans_grad[g.b] = GaveUp(hdr) ? __builtin_nanf("") : g_origin;
 }
 
@@ -1129,56 +1293,334 @@ __global__ __launch_bounds__(BwdLayout::kThreads) void MiBackwardFastKernel(
   const unsigned ticket = lds.ticket, nsweep = (unsigned)B * nchunks;
   const bool zero_only = ticket >= nsweep;
   const unsigned unit = zero_only ? ticket - nsweep : ticket;
-  MiBackwardChunk<kKept>(lds, px, p, boundary, ans_grad, px_grad, py_grad, hdr, edge, B, S, Tn,
-                         modified, nchunks, edge_stride, overwrite_ans_grad, (int)(unit / nchunks),
-                         zero_only ? (int)(unit % nchunks) : nchunks - 1 - (int)(unit % nchunks),
-                         zero_only);
+  MiBackwardChunk<kKept, false>(lds, px, p, LoadBox(boundary, (int)(unit / nchunks), S, Tn), ans_grad,
+                                px_grad, py_grad, hdr, edge, B, S,
+                                Tn, modified, nchunks, edge_stride, overwrite_ans_grad,
+                                (int)(unit / nchunks),
+                                zero_only ? (int)(unit % nchunks) : nchunks - 1 - (int)(unit % nchunks),
+                                zero_only, Half{}, nullptr);
   if (threadIdx.x == 0) FinishWorkgroup(hdr, gridDim.x);
 }
 
-// Forward and backward of a sequence's chunk in ONE launch, for callers that want ans and the
+// ------------------------------------------------------------------------------ single launch
+//
+// Forward and backward of every sequence in ONE launch, for callers that want ans and the
 // gradients together (the reference's autograd function, k2/python/k2/mutual_information.py:
-// 157-169).  A workgroup sweeps its chunk forward, keeping the log-derivatives, and then sweeps
-// the same chunk backward: everything its backward loads is what its own forward stored, so only
-// the two kinds of edge words cross between workgroups.  The forward runs down a sequence's
-// chunks and the backward comes back up, so the launch costs what the two kernels cost one
-// after the other, less one launch gap and one start-up.  Unlike the separate kernels a workgroup
-// here also waits for a LATER ticket (the chunk below it, in the backward): the launcher only
-// uses this kernel where every sweeping workgroup finds a compute unit at once.
+// 157-169).  Every lattice is split at a cut diagonal half way along its longest path (see Half)
+// and swept from both ends at once:
+//   1. the first half forward from the origin (alpha), the second half "forward" in its mirrored
+//      coordinates from the end cell (beta), each keeping its px-edge log-derivatives;
+//   2. on the cut, where every path has exactly one cell, alpha + beta of a cell is the log of
+//      the total weight of the paths through it: the score is their log-sum, and a cell's share
+//      of the paths, exp(alpha + beta - score), is the gradient that reaches it;
+//   3. each half sweeps back from the cut with the ordinary backward chunk sweep, seeded with
+//      those shares on every row instead of with the sequence's gradient at the end cell.  In the
+//      mirrored half a cell's log-derivative is the log-probability of LEAVING the lattice cell
+//      along px given that a path is there, which is what the occupation counts need on that
+//      side: the same code yields px_grad / py_grad of the edges that leave each cell.
+// So the longest chain of dependent steps is half the lattice's, both ways.
+//
+// Work is handed out as TASKS through the ticket counter to a fixed set of persistent workgroups
+// (one per compute unit): first the forward sweeps of all (sequence, half, 64-row chunk), then the
+// clearing of what lies outside the boxes, then the backward sweeps, then one task per sequence
+// for the lattices the split cannot serve.  A task only ever waits for tasks with EARLIER
+// tickets (a chunk's producer; for the backward sweeps and the last kind of task, all forward
+// sweeps of the sequence), and a ticket is only taken by a workgroup that is running, so the
+// launch makes progress with any number of resident workgroups: nothing depends on the whole grid
+// being resident at once.
+//
+// A lattice whose end cell no path reaches has no finite score to normalise with; its gradients
+// are then DEFINED by the reference's loop order (k2/python/csrc/torch/
+// mutual_information_cpu.cu:195-211).  Such a sequence is left to its last task, which runs the
+// exact one-workgroup recursion of mi_generic_impl.h on it.
+constexpr int kCutRows = 2056;  // lattice rows (S + 2 at most) the single launch serves
+constexpr int kCutWordsPerSeqHeader = 16;
+
+struct CutShared {
+  // alpha / beta of the sequence's cut cells by lattice row, then exp(alpha + beta - best); also
+  // the two rotating rows of the exact recursion
+  float a[kCutRows];
+  float b[kCutRows];
+  float red_val[16];
+  int red_idx[16];
+  float seeds[kRows];
+  float total;
+  float scale;
+  int best;
+  int last;
+  unsigned ticket;
+};
+
+// Per sequence, in the workspace: arrive (forward sweeps finished), depart (readers of the cut
+// finished), the gradient of the sequence's score, then alpha by own row of the first half and
+// beta by own row of the second.  Counters count up from the sentinel, which is what the
+// workspace is initialised to.
+struct CutWords {
+  unsigned *arrive, *depart;
+  float *scale, *alpha, *beta;
+  int words;
+};
+__device__ __forceinline__ CutWords CutOf(float *cut, int b, int nchunks) {
+  CutWords w;
+  w.words = kCutWordsPerSeqHeader + 2 * nchunks * kRows;
+  float *base = cut + (size_t)b * w.words;
+  w.arrive = reinterpret_cast<unsigned *>(base);
+  w.depart = reinterpret_cast<unsigned *>(base) + 1;
+  w.scale = base + 2;
+  w.alpha = base + kCutWordsPerSeqHeader;
+  w.beta = w.alpha + nchunks * kRows;
+  return w;
+}
+
+// One thread waits until a counter has reached a value (bounded, like TakeEdge).
+__device__ __forceinline__ void WaitCount(unsigned *word, unsigned want, FastHeader *hdr) {
+  int spins = 0;
+  for (;;) {
+    if (__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == want) return;
+    ++spins;
+    if ((spins & 255) == 0 &&
+        __hip_atomic_load(&hdr->error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)
+      return;
+    if (spins > kSpinLimit) {
+      __hip_atomic_store(&hdr->error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      return;
+    }
+    __builtin_amdgcn_s_sleep(2);
+  }
+}
+
+// (value, index) of the largest value over the workgroup, the smallest index among equals.
+__device__ __forceinline__ void BlockArgMax(CutShared &sh, float v, int idx) {
+  for (int d = 32; d >= 1; d >>= 1) {
+    const float ov = __shfl_xor(v, d);
+    const int oi = __shfl_xor(idx, d);
+    if (ov > v || (ov == v && oi < idx)) { v = ov; idx = oi; }
+  }
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (lane == 0) { sh.red_val[wave] = v; sh.red_idx[wave] = idx; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const int nw = blockDim.x >> 6;
+    for (int w = 1; w < nw; ++w)
+      if (sh.red_val[w] > v || (sh.red_val[w] == v && sh.red_idx[w] < idx)) { v = sh.red_val[w]; idx = sh.red_idx[w]; }
+    sh.best = idx;
+  }
+  __syncthreads();
+}
+// Sum over the workgroup in a fixed order (the same bits in every workgroup that adds the same
+// numbers).
+__device__ __forceinline__ float BlockSum(CutShared &sh, float v) {
+  for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  __syncthreads();
+  if (lane == 0) sh.red_val[wave] = v;
+  __syncthreads();
+  float t = sh.red_val[0];
+  const int nw = blockDim.x >> 6;
+  for (int w = 1; w < nw; ++w) t += sh.red_val[w];
+  return t;
+}
+
+// The join on the cut of a sequence with ns + 1 rows: returns the score (to every thread; -inf
+// when no path reaches the end cell) and leaves in sh.seeds the gradient seeds of the 64 own rows
+// row0 .. row0 + 63 of a half (lattice row = own row, or ns - own row when mirrored).
+// alpha and beta are of the size of the score (thousands, where one ulp is 2.4e-4) while their
+// sum only matters relative to the largest one: both are taken relative to the best cell's
+// values BEFORE they are added, which keeps the shares exact to a few ulps of themselves.
+__device__ __attribute__((noinline)) float CutJoin(CutShared &sh, const CutWords &cw, int ns, int row0, int mirror) {
+  float best = -3.0e38f;
+  int best_s = 0x7fffffff;
+  for (int s = threadIdx.x; s <= ns; s += blockDim.x) {
+    const float a = ReadCut(cw.alpha + s), b = ReadCut(cw.beta + (ns - s));
+    sh.a[s] = a;
+    sh.b[s] = b;
+    const float u = a + b;
+    if (u > best) { best = u; best_s = s; }
+  }
+  if (threadIdx.x == 0) sh.scale = ReadCut(cw.scale);
+  BlockArgMax(sh, best, best_s);
+  const int at = sh.best <= ns ? sh.best : 0;  // (no candidate at all: every sum was NaN)
+  const float a_ref = sh.a[at], b_ref = sh.b[at];
+  const bool reachable = a_ref + b_ref > kLogZeroTest;
+  float part = 0.0f;
+  __syncthreads();  // everyone has a_ref, b_ref before sh.a is overwritten
+  for (int s = threadIdx.x; s <= ns; s += blockDim.x) {
+    const float w = reachable ? expf((sh.a[s] - a_ref) + (sh.b[s] - b_ref)) : 0.0f;
+    sh.a[s] = w;
+    part += w;
+  }
+  const float sum = BlockSum(sh, part);  // >= 1 when reachable
+  if (threadIdx.x < kRows) {
+    const int own = row0 + threadIdx.x;
+    const int s = mirror ? ns - own : own;
+    sh.seeds[threadIdx.x] = reachable && own <= ns ? sh.a[s] / sum * sh.scale : 0.0f;
+  }
+  __syncthreads();
+  return reachable ? (a_ref + b_ref) + logf(sum) : NegInfF();
+}
+
 union FusedLds {
   FwdLds fwd;
   BwdLds bwd;
 };
-__global__ __launch_bounds__(FwdLayout::kThreads) void MiForwardBackwardFastKernel(
-    const float *__restrict__ px, const float *__restrict__ py,
-    const int64_t *__restrict__ boundary, float *__restrict__ ans, float *__restrict__ log_deriv,
-    float *__restrict__ ans_grad, float *__restrict__ px_grad, float *__restrict__ py_grad,
-    FastHeader *hdr, float *edge_fwd, float *edge_bwd, int B, int S, int Tn, int modified,
-    int nchunks, int edge_stride, int overwrite_ans_grad) {
+
+// What every task of the single launch needs (the kernel's arguments).
+struct BidirArgs {
+  const float *px, *py;
+  const int64_t *boundary;
+  float *ans, *scratch, *ans_grad, *px_grad, *py_grad;
+  FastHeader *hdr;
+  float *edge0, *edge1, *cut;
+  int B, S, Tn, modified, nchunks, edge_stride, overwrite_ans_grad;
+#ifdef K2AMD_MI_TRACE
+  unsigned long long *trace;  // per ticket: start, cut reached, end (100 MHz clock), compute unit
+#endif
+};
+
+// The tasks are functions of their own (not inlined into the kernel's loop), so that each gets the
+// registers IT needs: the sweeps' loaders keep several blocks of loads in flight in registers and
+// count them by hand, which a spill in their loops would upset.  What they need of the kernel's
+// arguments and of the sequence's box they read from LDS (a copy made once per workgroup, once per
+// task): a reference into any other memory would cost a trip there at the start of every task.
+struct TaskShared {
+  BidirArgs k;
+  Box box;
+};
+__device__ __attribute__((noinline)) void BidirForwardTask(FwdLds &lds, const TaskShared &t, int seq,
+                                                           int chunk, Half half, float *cut_out) {
+  const BidirArgs &k = t.k;
+  MiForwardChunk<true, false, true>(lds, k.px, k.py, t.box, nullptr, k.ans, k.scratch, k.hdr,
+                                    half.mirror ? k.edge1 : k.edge0, k.B, k.S, k.Tn, k.modified,
+                                    k.nchunks, k.edge_stride, seq, chunk, half, cut_out);
+}
+__device__ __attribute__((noinline)) void BidirBackwardTask(BwdLds &lds, const TaskShared &t, int seq,
+                                                            int chunk, Half half, const float *seeds) {
+  const BidirArgs &k = t.k;
+  MiBackwardChunk<true, true>(lds, k.px, k.scratch, t.box, k.ans_grad, k.px_grad, k.py_grad, k.hdr,
+                              half.mirror ? k.edge1 : k.edge0, k.B, k.S, k.Tn, k.modified, k.nchunks,
+                              k.edge_stride, k.overwrite_ans_grad, seq, chunk, false, half, seeds);
+}
+__device__ __attribute__((noinline)) void BidirClearTask(BwdLds &lds, const TaskShared &t, int seq, int chunk) {
+  const BidirArgs &k = t.k;
+  MiBackwardChunk<true, false>(lds, k.px, k.scratch, t.box, k.ans_grad, k.px_grad, k.py_grad, k.hdr,
+                               k.edge0, k.B, k.S, k.Tn, k.modified, k.nchunks, k.edge_stride,
+                               k.overwrite_ans_grad, seq, chunk, true, Half{}, nullptr);
+}
+// No path reaches the end cell: the exact recursion, whose loop order defines the result.
+__device__ __attribute__((noinline)) void BidirExactTask(CutShared &sh, const TaskShared &t, int seq,
+                                                         float seed) {
+  const BidirArgs &k = t.k;
+  const Box box = t.box;
+  float *prev = sh.a, *cur = sh.a + (k.S + 2);
+  static_assert(offsetof(CutShared, b) == sizeof(float) * kCutRows, "a and b are one array here");
+  const float end = MiForwardGenericSeq<float>(k.px, k.py, box, k.scratch, seq, k.S, k.Tn, k.modified,
+                                               k.Tn + 2, prev, cur);
+  if (threadIdx.x == 0) k.ans[seq] = GaveUp(k.hdr) ? __builtin_nanf("") : end;
+  __syncthreads();
+  const float at_origin = MiBackwardGenericSeq<float>(k.px, k.scratch, box, seed, k.px_grad, k.py_grad,
+                                                      seq, k.S, k.Tn, k.modified, k.Tn + 2, prev, cur);
+  if (k.overwrite_ans_grad && k.ans_grad != nullptr && threadIdx.x == 0) k.ans_grad[seq] = at_origin;
+}
+
+__global__ __launch_bounds__(FwdLayout::kThreads) void MiBidirKernel(const BidirArgs k) {
   static_assert(FwdLayout::kThreads == BwdLayout::kThreads, "one workgroup shape for both sweeps");
   __shared__ FusedLds lds;
-  __shared__ unsigned ticket_slot;
-  if (threadIdx.x == 0) ticket_slot = atomicAdd(&hdr->ticket, 1u);
-  __syncthreads();
-  const unsigned ticket = ticket_slot, nsweep = (unsigned)B * nchunks;
-  if (ticket >= nsweep) {  // clears what the backward sweep does not assign
-    const unsigned unit = ticket - nsweep;
-    MiBackwardChunk<true>(lds.bwd, px, log_deriv, boundary, ans_grad, px_grad, py_grad, hdr,
-                          edge_bwd, B, S, Tn, modified, nchunks, edge_stride, overwrite_ans_grad,
-                          (int)(unit / nchunks), (int)(unit % nchunks), true);
-  } else {
-    const int seq = (int)(ticket / nchunks), chunk = (int)(ticket % nchunks);
-    MiForwardChunk<true, false>(lds.fwd, px, py, boundary, nullptr, ans, log_deriv, hdr, edge_fwd,
-                                B, S, Tn, modified, nchunks, edge_stride, seq, chunk);
-    // __syncthreads() waits for every wavefront's outstanding stores as well: the log-derivatives
-    // are in the L2 this compute unit reads from before any of its loaders asks for them
+  __shared__ CutShared sh;
+  __shared__ TaskShared ts;
+  if (threadIdx.x == 0) ts.k = k;
+  const int nchunks = k.nchunks;
+  const unsigned per_seq = 2u * nchunks, nsweep = (unsigned)k.B * per_seq;
+  const unsigned first_clear = nsweep, first_bwd = first_clear + (unsigned)k.B * nchunks;
+  const unsigned first_last = first_bwd + nsweep, ntasks = first_last + (unsigned)k.B;
+  const int skew = k.modified ? 0 : 1;
+  for (;;) {
+    __syncthreads();  // the previous task's last LDS reads are done, its stores complete
+    if (threadIdx.x == 0) sh.ticket = atomicAdd(&k.hdr->ticket, 1u);
     __syncthreads();
-    MiBackwardChunk<true>(lds.bwd, px, log_deriv, boundary, ans_grad, px_grad, py_grad, hdr,
-                          edge_bwd, B, S, Tn, modified, nchunks, edge_stride, overwrite_ans_grad,
-                          seq, chunk, false);
-    if (threadIdx.x == 0 && GaveUp(hdr)) ans[seq] = __builtin_nanf("");
+    const unsigned ticket = sh.ticket;
+    if (ticket >= ntasks) break;
+#ifdef K2AMD_MI_TRACE
+    struct Tracer {
+      unsigned long long *at;
+      __device__ void mark(int i) { if (at != nullptr && threadIdx.x == 0) at[i] = wall_clock64(); }
+      __device__ ~Tracer() { mark(2); }
+    } tracer{k.trace != nullptr ? k.trace + 8 * (size_t)ticket : nullptr};
+    tracer.mark(0);
+    if (tracer.at != nullptr && threadIdx.x == 0) tracer.at[3] = blockIdx.x;
+#endif
+
+    if (ticket >= first_clear && ticket < first_bwd) {  // what no sweep assigns
+      const unsigned unit = ticket - first_clear;
+      if (threadIdx.x == 0) ts.box = LoadBox(k.boundary, (int)(unit / nchunks), k.S, k.Tn);
+      __syncthreads();
+      BidirClearTask(lds.bwd, ts, (int)(unit / nchunks), (int)(unit % nchunks));
+      continue;
+    }
+
+    const bool fwd = ticket < first_clear, last = ticket >= first_last;
+    const unsigned unit = fwd ? ticket : (last ? 0u : ticket - first_bwd);
+    const int seq = last ? (int)(ticket - first_last) : (int)(unit / per_seq);
+    const int mirror = last ? 0 : (int)((unit % per_seq) / nchunks);
+    const int cidx = last ? 0 : (int)(unit % nchunks);
+    const int chunk = fwd || last ? cidx : nchunks - 1 - cidx;  // backward: lower chunks first
+    if (threadIdx.x == 0) ts.box = LoadBox(k.boundary, seq, k.S, k.Tn);
+    __syncthreads();
+    const Box box = ts.box;
+    const int ns = box.s1 - box.s0, nt = box.t1 - box.t0;
+    const int diagonals = nt + ns * skew, dcut = diagonals / 2;
+    Half half{};
+    half.mirror = mirror;
+    half.dmax = mirror ? diagonals - dcut : dcut;
+#ifdef K2AMD_MI_TRACE
+    half.trace = k.trace != nullptr ? k.trace + 8 * (size_t)ticket : nullptr;
+#endif
+    const CutWords cw = CutOf(k.cut, seq, nchunks);
+
+    if (fwd) {
+      if (!mirror && chunk == 0 && threadIdx.x == 0)
+        PublishCut(cw.scale, k.ans_grad != nullptr ? k.ans_grad[seq] : 1.0f);
+      BidirForwardTask(lds.fwd, ts, seq, chunk, half, (mirror ? cw.beta : cw.alpha) + chunk * kRows);
+      // every wavefront has waited for its stores (device-coherent ones, see StoreQuadCoherent)
+      // before this barrier: whichever compute unit sweeps this chunk back will see them
+      __syncthreads();
+      if (threadIdx.x == 0)
+        __hip_atomic_fetch_add(cw.arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      continue;
+    }
+
+    // backward sweep of a chunk, or the sequence's last task: both start from the cut
+    if (threadIdx.x == 0) WaitCount(cw.arrive, kSentinel + per_seq, k.hdr);
+    __syncthreads();
+    float total = 0.0f;
+#ifdef K2AMD_MI_TRACE
+    tracer.mark(1);
+#endif
+    if (box.ok) total = CutJoin(sh, cw, ns, chunk * kRows, mirror);
+    const float seed = sh.scale;
+    // This task has read the sequence's cut words.  The last of their readers puts them back into
+    // their initial state; the count comes back while the sweep below runs and is looked at after it.
+    unsigned departed = 0;
+    if (threadIdx.x == 0)
+      departed = __hip_atomic_fetch_add(cw.depart, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const bool split_ok = box.ok && total > kLogZeroTest;  // a finite score
+    if (!last) {
+      if (!mirror && chunk == 0 && threadIdx.x == 0) {
+        if (!box.ok || GaveUp(k.hdr)) k.ans[seq] = __builtin_nanf("");
+        else if (split_ok) k.ans[seq] = total;
+      }
+      if (split_ok) BidirBackwardTask(lds.bwd, ts, seq, chunk, half, sh.seeds);
+    } else if (box.ok && !split_ok) {
+      BidirExactTask(sh, ts, seq, seed);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) sh.last = departed + 1 == kSentinel + per_seq + 1;
+    __syncthreads();
+    if (sh.last)
+      for (int i = threadIdx.x; i < cw.words; i += blockDim.x)
+        __hip_atomic_store(reinterpret_cast<unsigned *>(cw.arrive) + i, kSentinel, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
   }
-  if (threadIdx.x == 0) FinishWorkgroup(hdr, gridDim.x);
+  if (threadIdx.x == 0) FinishWorkgroup(k.hdr, gridDim.x);
 }
 
 // A sweeping workgroup wants a compute unit to itself (its chain wavefront sets the pace of the
@@ -1186,7 +1628,10 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiForwardBackwardFastKern
 // Asking for more than half of the unit's 160 KB of LDS makes the dispatcher place one workgroup
 // per unit; the bytes beyond the kernels' own structures are never touched.
 constexpr size_t kExclusiveLds = 84 * 1024;
-static_assert(sizeof(FusedLds) + 16 < kExclusiveLds, "LDS budget");
+static_assert(sizeof(FwdLds) + 16 < kExclusiveLds && sizeof(BwdLds) + 16 < kExclusiveLds, "LDS budget");
+// the single launch's own structures already are more than half a unit's LDS
+static_assert(sizeof(FusedLds) + sizeof(CutShared) > 80 * 1024 && sizeof(FusedLds) + sizeof(CutShared) < 160 * 1024,
+              "one workgroup of the single launch per compute unit");
 
 }  // namespace
 
@@ -1197,11 +1642,13 @@ bool MiFastSupports(int B, int S, int Tn, int modified) {
   return S >= 1 && Tn >= 1 && (long long)B * (S + 1) * (Tn + 1) < (1ll << 29);
 }
 
-// Two sets of edge rows: the single-launch forward + backward has both kinds in flight at once.
+// Two sets of edge rows (the single launch sweeps the two halves of every lattice at once), then
+// the words of the cut of every sequence.
 size_t MiFastWorkspaceBytes(int B, int S, int Tn) {
   const int nchunks = (S + 1 + kRows - 1) / kRows;
   const size_t edge_stride = ((size_t)Tn + 2 + kRows + kW + 3) / 4 * 4 + kW;
-  return sizeof(FastHeader) + 2 * (size_t)B * (nchunks + 1) * edge_stride * sizeof(float);
+  const size_t cut_words = kCutWordsPerSeqHeader + 2 * (size_t)nchunks * kRows;
+  return sizeof(FastHeader) + (2 * (size_t)B * (nchunks + 1) * edge_stride + (size_t)B * cut_words) * sizeof(float);
 }
 
 int MiFastWorkspaceInit(void *workspace, size_t workspace_bytes, hipStream_t stream) {
@@ -1282,60 +1729,42 @@ int MiBackwardFast(const float *px, const float *p, const float *log_deriv,
   return LaunchStatus();
 }
 
-// Workgroups of the single launch that one compute unit holds at a time when they ask for no LDS
-// beyond their own structure (asked of the runtime once per device ordinal), or -1.
-static int FusedWorkgroupsPerUnit() {
-  static std::atomic<int> per_unit[64];  // 0 = not asked yet
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return -1;
-  int n = per_unit[dev].load(std::memory_order_relaxed);
-  if (n == 0) {
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, MiForwardBackwardFastKernel,
-                                                     FwdLayout::kThreads, 0) != hipSuccess)
-      return -1;
-    n = n > 0 ? n : -1;
-    per_unit[dev].store(n, std::memory_order_relaxed);
-  }
-  return n;
-}
-
-// Whether the single launch may be used on the current device: every workgroup of the grid must
-// be resident at once (a sweeping workgroup waits, in its backward half, for workgroups that
-// started after it).  Up to one workgroup per compute unit each gets a unit to itself.  Up to two
-// per unit, where the kernel's registers and LDS allow two, the dispatcher still hands the
-// sweeping workgroups (the first half of the grid) a unit each before it doubles up, and the
-// clearing workgroups that join them leave after a few microseconds.
-static bool FusedFits(long long grid, bool *exclusive) {
-  const int n = ComputeUnits();
-  if (n <= 0) return false;
-  *exclusive = grid <= n;
-  return *exclusive || (grid <= 2ll * n && FusedWorkgroupsPerUnit() >= 2);
-}
-
+// The single launch serves what the pipelined kernels serve, up to the number of lattice rows that
+// its join on the cut keeps in LDS.  It needs no particular number of resident workgroups.
 bool MiFusedSupports(int B, int S, int Tn, int modified) {
-  if (!MiFastSupports(B, S, Tn, modified) || B < 1) return false;
-  const long long nchunks = (S + 1 + kRows - 1) / kRows;
-  bool exclusive;
-  return FusedFits(2 * (long long)B * nchunks, &exclusive);
+  return MiFastSupports(B, S, Tn, modified) && B >= 1 && S + 2 <= kCutRows;
 }
+
+// Floats of scratch per call of the single launch: one slab of (S + 1) rows of Tn + 2 per sequence
+// (the log-derivatives of both halves, the mirrored half's one column to the right).
+size_t MiFusedScratchElems(int B, int S, int Tn) { return (size_t)B * (S + 1) * ((size_t)Tn + 2); }
 
 int MiForwardBackwardFast(const float *px, const float *py, const int64_t *boundary, float *ans,
-                          float *log_deriv, float *ans_grad, float *px_grad, float *py_grad, int B,
+                          float *scratch, float *ans_grad, float *px_grad, float *py_grad, int B,
                           int S, int Tn, int modified, int overwrite_ans_grad, void *workspace,
                           size_t workspace_bytes, hipStream_t stream) {
   if (workspace == nullptr || workspace_bytes < MiFastWorkspaceBytes(B, S, Tn)) return K2AMD_ERR_WORKSPACE;
-  if (log_deriv == nullptr) return K2AMD_ERR_INVALID_ARGUMENT;
-  const int nchunks = (S + 1 + kRows - 1) / kRows;
-  bool exclusive = true;
-  if (!MiFastSupports(B, S, Tn, modified) || B < 1 || !FusedFits(2ll * B * nchunks, &exclusive))
+  if (scratch == nullptr) return K2AMD_ERR_INVALID_ARGUMENT;
+  if (!MiFusedSupports(B, S, Tn, modified) || MiFusedScratchElems(B, S, Tn) >= (1ull << 29))
     return K2AMD_ERR_UNSUPPORTED;
+  const int units = ComputeUnits();
+  if (units <= 0) return K2AMD_ERR_LAUNCH;
+  const int nchunks = (S + 1 + kRows - 1) / kRows;
   const int edge_stride = (int)(((size_t)Tn + 2 + kRows + kW + 3) / 4 * 4 + kW);
   FastHeader *hdr = static_cast<FastHeader *>(workspace);
-  float *edge_fwd = reinterpret_cast<float *>(hdr + 1);
-  float *edge_bwd = edge_fwd + (size_t)B * (nchunks + 1) * edge_stride;
-  const dim3 grid((unsigned)(2 * B * nchunks)), block(FwdLayout::kThreads);
-  const size_t pad = exclusive ? kExclusiveLds - sizeof(FusedLds) - 16 : 0;
-  hipLaunchKernelGGL(MiForwardBackwardFastKernel, grid, block, pad, stream, px, py, boundary, ans, log_deriv, ans_grad, px_grad, py_grad, hdr, edge_fwd, edge_bwd, B, S, Tn, modified, nchunks, edge_stride, overwrite_ans_grad);
+  float *edge0 = reinterpret_cast<float *>(hdr + 1);
+  float *edge1 = edge0 + (size_t)B * (nchunks + 1) * edge_stride;
+  float *cut = edge1 + (size_t)B * (nchunks + 1) * edge_stride;
+  // forward sweeps of both halves, clearing, backward sweeps, one last task per sequence
+  const long long ntasks = 5ll * B * nchunks + B;
+  const dim3 grid((unsigned)std::min<long long>(ntasks, units)), block(FwdLayout::kThreads);
+  BidirArgs args{px, py, boundary, ans, scratch, ans_grad, px_grad, py_grad, hdr, edge0, edge1, cut,
+                 B, S, Tn, modified, nchunks, edge_stride, overwrite_ans_grad};
+#ifdef K2AMD_MI_TRACE
+  const char *trace_at = getenv("K2AMD_MI_TRACE_PTR");
+  args.trace = trace_at != nullptr ? reinterpret_cast<unsigned long long *>(strtoull(trace_at, nullptr, 0)) : nullptr;
+#endif
+  hipLaunchKernelGGL(MiBidirKernel, grid, block, 0, stream, args);
   return LaunchStatus();
 }
 

@@ -1,14 +1,12 @@
 // Robust log-domain kernels for the mutual-information recursion (fp32 and fp64).
 //
-// One workgroup owns one sequence and sweeps its lattice one wavefront step at a time:
-//   regular lattice : step k holds the anti-diagonal  s + t = k   (cell (s,t) needs (s-1,t), (s,t-1))
-//   modified lattice: step k holds the column         t = k       (cell (s,t) needs (s-1,t-1), (s,t-1))
-// so in both cases a step depends on the previous step only, which lives in LDS (two rotating
-// rows of S+1 values).  Arithmetic follows k2's CPU loops term for term
-// (k2/python/csrc/torch/mutual_information_cpu.cu:89-121 forward, :179-251 backward), so these
-// kernels are the exact-semantics path: every dtype, every size, every -inf / NaN corner.
+// One workgroup owns one sequence and sweeps its lattice one wavefront step at a time (the sweeps
+// themselves are the device functions of mi_generic_impl.h).  Arithmetic follows k2's CPU loops
+// term for term, so these kernels are the exact-semantics path: every dtype, every size, every
+// -inf / NaN corner.
 // They are latency-bound by design; the throughput path for fp32 lives in mi_fast.hip.
 #include "common.h"
+#include "mi_generic_impl.h"
 #include "mi_internal.h"
 
 namespace k2amd {
@@ -29,46 +27,8 @@ __global__ __launch_bounds__(kThreads) void MiForwardGenericKernel(
     if (threadIdx.x == 0) ans[b] = std::numeric_limits<T>::quiet_NaN();
     return;
   }
-  const int T1 = modified ? Tn : Tn + 1;
-  const int off = modified ? -1 : 0;
-  const int skew = modified ? 0 : 1;
-  const int ns = box.s1 - box.s0, nt = box.t1 - box.t0;
-  const T *pxb = px + (size_t)b * S * T1;
-  const T *pyb = py + (size_t)b * (S + 1) * Tn;
-  T *pb = p + (size_t)b * (S + 1) * (Tn + 1);
-  const int K = nt + ns * skew;
-  for (int k = 0; k <= K; ++k) {
-    for (int i = threadIdx.x; i <= ns; i += kThreads) {
-      const int j = k - i * skew;
-      if (j < 0 || j > nt) continue;
-      const int s = box.s0 + i, t = box.t0 + j;
-      T v;
-      if (i == 0) {
-        v = (j == 0) ? T(0) : prev[0] + pyb[(size_t)s * Tn + t - 1];
-      } else if (j == 0) {
-        v = modified ? Real<T>::NegInf() : prev[i - 1] + pxb[(size_t)(s - 1) * T1 + t];
-      } else {
-        v = LogAdd<T>(prev[i - 1] + pxb[(size_t)(s - 1) * T1 + t + off],
-                      prev[i] + pyb[(size_t)s * Tn + t - 1]);
-      }
-      cur[i] = v;
-      pb[(size_t)s * (Tn + 1) + t] = v;
-    }
-    __syncthreads();
-    T *tmp = prev; prev = cur; cur = tmp;
-  }
-  if (threadIdx.x == 0) ans[b] = prev[ns];
-}
-
-// exp(term1 - total) with the reference's guards
-// (k2/python/csrc/torch/mutual_information_cpu.cu:195-211): a non-finite total counts as 0;
-// a non-finite derivative sends no gradient either way (ok = false).
-template <typename T>
-__device__ __forceinline__ T PxDeriv(T term1, T total, bool *ok) {
-  if (total - total != 0) total = 0;
-  T d = Real<T>::Exp(term1 - total);
-  *ok = (d - d == 0);
-  return d;
+  const T end = MiForwardGenericSeq<T>(px, py, box, p, b, S, Tn, modified, Tn + 1, prev, cur);
+  if (threadIdx.x == 0) ans[b] = end;
 }
 
 template <typename T>
@@ -83,9 +43,6 @@ __global__ __launch_bounds__(kThreads) void MiBackwardGenericKernel(
   const Box box = LoadBox(boundary, b, S, Tn);
   const int T1 = modified ? Tn : Tn + 1;
   const int off = modified ? -1 : 0;
-  const int skew = modified ? 0 : 1;
-  const T *pxb = px + (size_t)b * S * T1;
-  const T *pb = p + (size_t)b * (S + 1) * (Tn + 1);
   T *gx = px_grad + (size_t)b * S * T1;
   T *gy = py_grad + (size_t)b * (S + 1) * Tn;
 
@@ -107,51 +64,9 @@ __global__ __launch_bounds__(kThreads) void MiBackwardGenericKernel(
     }
   }
   if (!box.ok) return;
-
-  const int ns = box.s1 - box.s0, nt = box.t1 - box.t0;
-  const int K = nt + ns * skew;
-  const T seed = ans_grad[b];
-  for (int k = K; k >= 0; --k) {
-    for (int i = threadIdx.x; i <= ns; i += kThreads) {
-      const int j = k - i * skew;
-      if (j < 0 || j > nt) continue;
-      const int s = box.s0 + i, t = box.t0 + j;
-      T a = 0, c = 0;
-      // Gradient arriving through px[s][t]: from cell (s+1, t-off).
-      const int jd = j - off;
-      if (i < ns && jd <= nt) {
-        const T gd = gprev[i + 1];
-        if (jd == 0) {
-          a = gd;  // first column of a regular lattice: p[s+1][t0] = p[s][t0] + px[s][t0]
-        } else {
-          bool ok;
-          const T d1 = PxDeriv<T>(pb[(size_t)s * (Tn + 1) + t] + pxb[(size_t)s * T1 + t],
-                                  pb[(size_t)(s + 1) * (Tn + 1) + t - off], &ok);
-          a = ok ? d1 * gd : T(0);
-        }
-        gx[(size_t)s * T1 + t] = a;
-      }
-      // Gradient arriving through py[s][t]: from cell (s, t+1).
-      if (j < nt) {
-        const T gd = gprev[i];
-        if (i == 0) {
-          c = gd;  // first row: p[s0][t+1] = p[s0][t] + py[s0][t]
-        } else {
-          bool ok;
-          const T d1 =
-              PxDeriv<T>(pb[(size_t)(s - 1) * (Tn + 1) + t + 1 + off] +
-                             pxb[(size_t)(s - 1) * T1 + t + 1 + off],
-                         pb[(size_t)s * (Tn + 1) + t + 1], &ok);
-          c = ok ? (T(1) - d1) * gd : T(0);
-        }
-        gy[(size_t)s * Tn + t] = c;
-      }
-      gcur[i] = (i == ns && j == nt) ? seed : a + c;
-    }
-    __syncthreads();
-    T *tmp = gprev; gprev = gcur; gcur = tmp;
-  }
-  if (overwrite_ans_grad && threadIdx.x == 0) ans_grad[b] = gprev[0];
+  const T at_origin = MiBackwardGenericSeq<T>(px, p, box, ans_grad[b], px_grad, py_grad, b, S, Tn,
+                                              modified, Tn + 1, gprev, gcur);
+  if (overwrite_ans_grad && threadIdx.x == 0) ans_grad[b] = at_origin;
 }
 
 }  // namespace

@@ -33,11 +33,12 @@ int MiBackwardFast(const float *px, const float *p, const float *log_deriv,
                    int S, int Tn, int modified, int overwrite_ans_grad, void *workspace,
                    size_t workspace_bytes, hipStream_t stream);
 
-// Forward and backward in one launch (log_deriv is scratch of p's shape); MiFusedSupports says
-// whether the current device can hold the launch's workgroups at once, which that kernel needs.
+// Forward and backward in one launch; scratch holds MiFusedScratchElems floats (written, then
+// read, by the launch itself).  MiFusedSupports: whether that kernel serves the shape.
 bool MiFusedSupports(int B, int S, int Tn, int modified);
+size_t MiFusedScratchElems(int B, int S, int Tn);
 int MiForwardBackwardFast(const float *px, const float *py, const int64_t *boundary, float *ans,
-                          float *log_deriv, float *ans_grad, float *px_grad, float *py_grad, int B,
+                          float *scratch, float *ans_grad, float *px_grad, float *py_grad, int B,
                           int S, int Tn, int modified, int overwrite_ans_grad, void *workspace,
                           size_t workspace_bytes, hipStream_t stream);
 

@@ -14,6 +14,7 @@
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 
+#include <algorithm>
 #include <map>
 #include <mutex>
 #include <utility>
@@ -89,25 +90,28 @@ struct Shape {
 };
 
 // The checks of k2/python/csrc/torch/mutual_information_cpu.cu:53-77, as RuntimeError.
-// `p` (or, where p is left out, the log-derivative tensor that stands in for it) is `lattice`.
+// `lattice`: p (or, where p is left out, the log-derivative tensor that stands in for it); null
+// for a call without either.
 Shape CheckInputs(const torch::Tensor &px, const torch::Tensor &py,
-                  const torch::optional<torch::Tensor> &boundary, const torch::Tensor &lattice) {
-  const torch::Tensor &p = lattice;
+                  const torch::optional<torch::Tensor> &boundary, const torch::Tensor *lattice) {
   TORCH_CHECK(px.dim() == 3, "px must be 3-dimensional");
   TORCH_CHECK(py.dim() == 3, "py must be 3-dimensional");
-  TORCH_CHECK(p.dim() == 3, "p must be 3-dimensional");
   TORCH_CHECK(px.is_cuda(), "k2_amd runs on MI355X only: px is on ", px.device(),
               " (there is no CPU path)");
-  TORCH_CHECK(py.device() == px.device() && p.device() == px.device(),
-              "inputs must be on the same device");
-  TORCH_CHECK(px.scalar_type() == py.scalar_type() && px.scalar_type() == p.scalar_type(),
-              "px, py and p must have the same dtype");
+  TORCH_CHECK(py.device() == px.device(), "inputs must be on the same device");
+  TORCH_CHECK(px.scalar_type() == py.scalar_type(), "px and py must have the same dtype");
   const int64_t B = px.size(0), S = px.size(1), T = py.size(2);
   TORCH_CHECK(px.size(2) == T || px.size(2) == T + 1, "px.size(2) must be T or T+1");
   TORCH_CHECK(py.size(0) == B && py.size(1) == S + 1, "py must have shape [B][S+1][T]");
-  TORCH_CHECK(p.size(0) == B && p.size(1) == S + 1 && p.size(2) == T + 1,
-              "p must have shape [B][S+1][T+1]");
-  TORCH_CHECK(p.is_contiguous(), "p must be contiguous");
+  if (lattice != nullptr) {
+    const torch::Tensor &p = *lattice;
+    TORCH_CHECK(p.dim() == 3, "p must be 3-dimensional");
+    TORCH_CHECK(p.device() == px.device(), "inputs must be on the same device");
+    TORCH_CHECK(px.scalar_type() == p.scalar_type(), "px, py and p must have the same dtype");
+    TORCH_CHECK(p.size(0) == B && p.size(1) == S + 1 && p.size(2) == T + 1,
+                "p must have shape [B][S+1][T+1]");
+    TORCH_CHECK(p.is_contiguous(), "p must be contiguous");
+  }
   if (boundary.has_value() && boundary->defined()) {
     TORCH_CHECK(boundary->scalar_type() == torch::kLong, "boundary must be int64");
     TORCH_CHECK(boundary->dim() == 2 && boundary->size(0) == B && boundary->size(1) == 4,
@@ -152,7 +156,7 @@ torch::Tensor MutualInformationForward(torch::Tensor px, torch::Tensor py,
                                        torch::optional<torch::Tensor> p,
                                        torch::optional<torch::Tensor> log_deriv) {
   const torch::Tensor &lattice = LatticeOf(p, log_deriv);
-  const Shape sh = CheckInputs(px, py, boundary, lattice);
+  const Shape sh = CheckInputs(px, py, boundary, &lattice);
   void *kept = CheckLogDeriv(log_deriv, lattice);
   void *p_ptr = Given(p) ? p->data_ptr() : nullptr;
   c10::hip::HIPGuardMasqueradingAsCUDA guard(px.device());
@@ -182,7 +186,7 @@ std::vector<torch::Tensor> MutualInformationBackward(torch::Tensor px, torch::Te
                                                      torch::Tensor ans_grad,
                                                      torch::optional<torch::Tensor> log_deriv) {
   const torch::Tensor &lattice = LatticeOf(p, log_deriv);
-  const Shape sh = CheckInputs(px, py, boundary, lattice);
+  const Shape sh = CheckInputs(px, py, boundary, &lattice);
   const void *kept = CheckLogDeriv(log_deriv, lattice);
   const void *p_ptr = Given(p) ? p->data_ptr() : nullptr;
   TORCH_CHECK(ans_grad.dim() == 1 && ans_grad.size(0) == sh.B, "ans_grad must have shape [B]");
@@ -235,9 +239,7 @@ std::vector<torch::Tensor> MutualInformationForwardBackward(torch::Tensor px, to
   TORCH_CHECK(px.is_cuda(), "k2_amd runs on MI355X only: px is on ", px.device(),
               " (there is no CPU path)");
   c10::hip::HIPGuardMasqueradingAsCUDA guard(px.device());
-  // scratch with p's shape: the forward sweep leaves the px-edge log-derivatives there
-  torch::Tensor log_deriv = torch::empty({px.size(0), px.size(1) + 1, py.size(2) + 1}, px.options());
-  const Shape sh = CheckInputs(px, py, boundary, log_deriv);
+  const Shape sh = CheckInputs(px, py, boundary, nullptr);
   void *seed = nullptr;  // None: every score has gradient 1
   if (ans_grad.has_value() && ans_grad->defined()) {
     TORCH_CHECK(ans_grad->dim() == 1 && ans_grad->size(0) == sh.B, "ans_grad must have shape [B]");
@@ -253,6 +255,10 @@ std::vector<torch::Tensor> MutualInformationForwardBackward(torch::Tensor px, to
   torch::Tensor ans = torch::empty({sh.B}, px.options());
   torch::Tensor px_grad = torch::empty_like(px), py_grad = torch::empty_like(py);
   const int dt = DtypeCode(px);
+  // the launch's scratch (the px-edge log-derivatives of both halves of every lattice)
+  const size_t scratch_bytes = k2amd_mi_forward_backward_scratch_bytes(sh.B, sh.S, sh.T, sh.modified, dt);
+  torch::Tensor scratch = torch::empty({static_cast<int64_t>(std::max<size_t>(scratch_bytes, 4))},
+                                       px.options().dtype(torch::kUInt8));
   void *stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(px.device().index()).stream();
   torch::Tensor ws = Cache().Get(k2amd_mi_workspace_bytes(sh.B, sh.S, sh.T, sh.modified, dt),
                                  px.device(), stream);
@@ -260,8 +266,8 @@ std::vector<torch::Tensor> MutualInformationForwardBackward(torch::Tensor px, to
     pybind11::gil_scoped_release release;
     Check(k2amd_mi_forward_backward(px.data_ptr(), py.data_ptr(),
                                     bd.defined() ? bd.data_ptr<int64_t>() : nullptr, ans.data_ptr(),
-                                    log_deriv.data_ptr(), seed, px_grad.data_ptr(),
-                                    py_grad.data_ptr(), sh.B, sh.S, sh.T, sh.modified, dt,
+                                    scratch.data_ptr(), static_cast<size_t>(scratch.numel()), seed,
+                                    px_grad.data_ptr(), py_grad.data_ptr(), sh.B, sh.S, sh.T, sh.modified, dt,
                                     /*overwrite_ans_grad=*/1, ws.defined() ? ws.data_ptr() : nullptr,
                                     ws.defined() ? static_cast<size_t>(ws.numel()) : 0, stream));
   }

@@ -43,11 +43,21 @@ def test_invalid_arguments_return_codes_without_a_gpu():
     assert lib.k2amd_mi_forward_keep(one, one, None, None, one, None, 1, 1, 1, 0, 0, one, 1 << 20, None) == 1
     assert lib.k2amd_mi_forward_keep(one, one, None, None, one, one, 1, 1, 1, 0, 1, one, 1 << 20, None) == 1
     assert lib.k2amd_mi_forward_keep(one, one, None, None, one, one, 1, 1, 1, 0, 0, None, 0, None) == 1
-    assert lib.k2amd_mi_forward_backward(one, one, None, one, None, one, one, one, 1, 1, 1, 0, 0, 1, one, 1 << 20, None) == 1
-    assert lib.k2amd_mi_forward_backward(one, one, None, one, one, one, one, one, 1, 1, 1, 0, 1, 1, one, 1 << 20, None) == 2
-    assert lib.k2amd_mi_forward_backward(None, None, None, None, None, None, None, None, 0, 1, 1, 0, 0, 1, None, 0, None) == 0
+    big = 1 << 20
+    assert lib.k2amd_mi_forward_backward(one, one, None, one, None, big, one, one, one, 1, 1, 1, 0, 0, 1, one, big, None) == 1
+    assert lib.k2amd_mi_forward_backward(one, one, None, one, one, big, one, one, one, 1, 1, 1, 0, 1, 1, one, big, None) == 2
+    assert lib.k2amd_mi_forward_backward(None, None, None, None, None, 0, None, None, None, 0, 1, 1, 0, 0, 1, None, 0, None) == 0
+    # scratch or workspace too small for the shape: refused before anything is launched
+    assert lib.k2amd_mi_forward_backward(one, one, None, one, one, 16, one, one, one, 4, 10, 20, 0, 0, 1, one, big, None) == 3
+    assert lib.k2amd_mi_forward_backward(one, one, None, one, one, big, one, one, one, 4, 10, 20, 0, 0, 1, one, 16, None) == 3
     assert lib.k2amd_mi_forward_backward_supported(4, 10, 20, 0, 1, 1) == 0
     assert lib.k2amd_mi_forward_backward_supported(4, 10, 20, 0, 0, 0) == 0
+    # the single launch needs no particular number of resident workgroups: any batch is served
+    assert lib.k2amd_mi_forward_backward_supported(4, 10, 20, 0, 0, 1) == 1
+    assert lib.k2amd_mi_forward_backward_supported(2000, 200, 1000, 1, 0, 1) == 1
+    assert lib.k2amd_mi_forward_backward_supported(4, 2055, 3000, 1, 0, 1) == 0   # more rows than its join keeps
+    assert lib.k2amd_mi_forward_backward_scratch_bytes(4, 10, 20, 0, 0) == 4 * 11 * 22 * 4
+    assert lib.k2amd_mi_forward_backward_scratch_bytes(4, 10, 20, 0, 1) == 0
     # the log-derivative tensor is only used by the pipelined fp32 kernels, which need a workspace
     assert lib.k2amd_mi_keeps_log_deriv(4, 10, 20, 0, 0, 1) == 1
     assert lib.k2amd_mi_keeps_log_deriv(4, 10, 20, 0, 0, 0) == 0

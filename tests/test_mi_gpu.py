@@ -57,20 +57,30 @@ def run_gpu(px, py, bd, device, ans_grad=None):
         assert capi.mi_workspace_is_clean(device), "workspace left dirty (kept pair without p)"
         for name, x, y in (("ans", ans3, ans), ("px_grad", gx3, gx), ("py_grad", gy3, gy), ("ans_grad", g3, g)):
             assert torch.equal(x.view(torch.int32), y.view(torch.int32)), "kept pair without p differs in " + name
+    single = None
     if capi.mi_forward_backward_supported(tpx, tpy):
-        # both recursions in one launch
+        # Both recursions in one launch.  That launch sweeps every lattice from both ends and joins
+        # the halves in the middle, so its results are not the pair's bits: they are returned for
+        # the caller to compare with the oracle like the pair's.  What must be identical is the
+        # launch with itself: a second run, and a run without a seed tensor (which stands for ones).
         g4 = g_in.clone()
         ans4, gx4, gy4 = capi.mi_forward_backward(tpx, tpy, tbd, g4, overwrite_ans_grad=True)
         torch.cuda.synchronize()
         assert capi.mi_workspace_is_clean(device), "workspace left dirty (single launch)"
         capi.mi_workspace_status(device)
-        for name, x, y in (("ans", ans4, ans), ("px_grad", gx4, gx), ("py_grad", gy4, gy), ("ans_grad", g4, g)):
-            assert torch.equal(x.view(torch.int32), y.view(torch.int32)), "single launch differs in " + name
+        g6 = g_in.clone()
+        ans6, gx6, gy6 = capi.mi_forward_backward(tpx, tpy, tbd, g6, overwrite_ans_grad=True)
+        torch.cuda.synchronize()
+        assert capi.mi_workspace_is_clean(device), "workspace left dirty (single launch, again)"
+        for name, x, y in (("ans", ans6, ans4), ("px_grad", gx6, gx4), ("py_grad", gy6, gy4), ("ans_grad", g6, g4)):
+            assert torch.equal(x.view(torch.int32), y.view(torch.int32)), "single launch not reproducible in " + name
         if ans_grad is None:  # no seed tensor at all stands for ones
             ans5, gx5, gy5 = capi.mi_forward_backward(tpx, tpy, tbd, None)
             torch.cuda.synchronize()
-            for name, x, y in (("ans", ans5, ans), ("px_grad", gx5, gx), ("py_grad", gy5, gy)):
+            for name, x, y in (("ans", ans5, ans4), ("px_grad", gx5, gx4), ("py_grad", gy5, gy4)):
                 assert torch.equal(x.view(torch.int32), y.view(torch.int32)), "seedless single launch differs in " + name
+        single = (ans4.cpu().numpy(), gx4.cpu().numpy(), gy4.cpu().numpy(), g4.cpu().numpy())
+    run_gpu.single = single
     return ans.cpu().numpy(), p.cpu().numpy(), gx.cpu().numpy(), gy.cpu().numpy(), g.cpu().numpy(), g_in.cpu().numpy()
 
 
@@ -108,6 +118,12 @@ def check(name, px, py, bd, want, device):
     # whenever the end cell is reachable
     ok = np.isfinite(ans_w)
     np.testing.assert_allclose(g_out[ok], g_in[ok], rtol=1e-3)
+    if run_gpu.single is not None:  # the single launch, against the same oracles
+        ans1, gx1, gy1, g1 = run_gpu.single
+        _close(name + " ans (single launch)", ans1, ans_w, w64[0], tol, mode="absolute")
+        _close(name + " px_grad (single launch)", gx1, gx_w, w64[2], tol)
+        _close(name + " py_grad (single launch)", gy1, gy_w, w64[3], tol)
+        np.testing.assert_allclose(g1[ok], g_in[ok], rtol=1e-3)
 
 
 def test_reference_fixtures(device):
@@ -232,11 +248,168 @@ def test_headline_shape_three_way(device):
               f"max|gpu-cpu32|={st['max_gpu_vs_cpu32']:.3e}  arbitrated {st['arbitrated']} of {st['n']} "
               f"({100 * st['arbitrated_frac']:.4f} %), reference's own 99.9th-percentile relative error "
               f"{st.get('reference_error_quantile_max', 0):.3e}")
+    ans1, gx1, gy1, g1 = run_gpu.single
+    np.testing.assert_allclose(ans1, ans32, rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(ans1, ans64, rtol=1e-4, atol=1e-5)
+    for name, g, g32, g64 in (("px_grad", gx1, gx32, gx64), ("py_grad", gy1, gy32, gy64)):
+        st = tolerance.close_f32("c4 single launch " + name, g, g32, g64, max_arbitrated=0.05)
+        print(f"c4 single launch {name}: max|gpu-fp64|={st['max_gpu_vs_fp64']:.3e}  max|cpu32-fp64|={st['max_cpu32_vs_fp64']:.3e}  "
+              f"max|gpu-cpu32|={st['max_gpu_vs_cpu32']:.3e}  arbitrated {st['arbitrated']} of {st['n']} "
+              f"({100 * st['arbitrated_frac']:.4f} %)")
     # flow conservation at full size: each symbol row is emitted exactly once
-    for b in range(c["B"]):
-        s1 = int(bd[b, 2])
-        np.testing.assert_allclose(gx[b, :s1].sum(axis=1), 1.0, rtol=2e-3)
+    for grads in (gx, gx1):
+        for b in range(c["B"]):
+            s1 = int(bd[b, 2])
+            np.testing.assert_allclose(grads[b, :s1].sum(axis=1), 1.0, rtol=2e-3)
     np.testing.assert_allclose(g_out, g_in, rtol=2e-3)
+    np.testing.assert_allclose(g1, g_in, rtol=2e-3)
+
+
+@pytest.mark.gpu
+def test_pybind_host_matches_ctypes_host(device):
+    """The C++ host module and the ctypes binding drive the same kernels: identical bits, on the
+    current stream, with a strided px view made contiguous by the host layer, and ans_grad
+    overwritten by the gradient that reached the origin."""
+    from k2_amd import _k2_amd, capi
+    rng = np.random.default_rng(77)
+    B, S, T = 3, 70, 90
+    px = torch.from_numpy(rng.standard_normal((B, S, T + 1)).astype(np.float32)).to(device)
+    py = torch.from_numpy(rng.standard_normal((B, S + 1, T)).astype(np.float32)).to(device)
+    bd = torch.tensor([[0, 0, S, T], [3, 5, 66, 80], [0, 10, 70, 90]], dtype=torch.int64, device=device)
+    p1 = torch.empty(B, S + 1, T + 1, device=device)
+    p2 = torch.empty_like(p1)
+    ans1 = capi.mi_forward(px, py, bd, p1)
+    px_strided = torch.empty(B, S, 2 * px.shape[2], device=device)[:, :, ::2]
+    px_strided.copy_(px)
+    side = torch.cuda.Stream(device=device)
+    side.wait_stream(torch.cuda.current_stream(device))
+    with torch.cuda.stream(side):
+        ans2 = _k2_amd.mutual_information_forward(px=px_strided, py=py, boundary=bd, p=p2)
+        g2 = torch.full((B,), 2.0, device=device)
+        gx2, gy2 = _k2_amd.mutual_information_backward(px=px, py=py, boundary=bd, p=p2, ans_grad=g2)
+        # the same through the pair that passes the log-derivatives along
+        assert _k2_amd.mutual_information_keeps_log_deriv(px=px, py=py)
+        p3 = torch.empty_like(p1)
+        kept = torch.full_like(p1, float("nan"))
+        ans3 = _k2_amd.mutual_information_forward(px=px_strided, py=py, boundary=bd, p=p3, log_deriv=kept)
+        g3 = torch.full((B,), 2.0, device=device)
+        gx3, gy3 = _k2_amd.mutual_information_backward(px=px, py=py, boundary=bd, p=p3, ans_grad=g3,
+                                                       log_deriv=kept)
+    side.synchronize()
+    assert torch.equal(ans3, ans2) and torch.equal(gx3, gx2) and torch.equal(gy3, gy2) and torch.equal(g3, g2)
+    assert _k2_amd.mutual_information_forward_backward_supported(px=px, py=py)
+    # the single launch sweeps the lattices from both ends: the hosts agree with each other bit
+    # for bit, and with the pair to the fp32 tolerance
+    g5 = torch.full((B,), 2.0, device=device)
+    ans5, gx5, gy5 = _k2_amd.mutual_information_forward_backward(px=px_strided, py=py, boundary=bd, ans_grad=g5)
+    g6 = torch.full((B,), 2.0, device=device)
+    ans6, gx6, gy6 = capi.mi_forward_backward(px, py, bd, g6, overwrite_ans_grad=True)
+    torch.cuda.synchronize()
+    assert torch.equal(ans5, ans6) and torch.equal(gx5, gx6) and torch.equal(gy5, gy6) and torch.equal(g5, g6)
+    for a, b in ((ans5, ans2), (gx5, gx2), (gy5, gy2), (g5, g2)):
+        np.testing.assert_allclose(a.cpu().numpy(), b.cpu().numpy(), rtol=1e-4, atol=1e-5)
+    with pytest.raises(RuntimeError):  # wrong shape
+        _k2_amd.mutual_information_forward(px=px, py=py, boundary=bd, p=p3, log_deriv=kept[:, :-1])
+    g1 = torch.full((B,), 2.0, device=device)
+    gx1, gy1 = capi.mi_backward(px, py, bd, p1, g1, overwrite_ans_grad=True)
+    torch.cuda.synchronize()
+    assert torch.equal(ans1, ans2)
+    assert torch.equal(gx1, gx2) and torch.equal(gy1, gy2)
+    assert torch.equal(g1, g2)
+    np.testing.assert_allclose(g2.cpu().numpy(), 2.0, rtol=1e-3)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_joint_recursion_identities(device, dtype):
+    """The checks of k2/python/tests/mutual_information_test.py:137-166: the joint recursion on
+    one input equals the plain one, on two halves it equals it after summing over the inputs,
+    and backprop through either gives the same derivative."""
+    import k2_amd as k2
+    rng = np.random.default_rng(5)
+    for modified in (False, True):
+        B, S, T = 4, 9, 40
+        T1 = T if modified else T + 1
+        npx = rng.standard_normal((B, S, T1))
+        npy = rng.standard_normal((B, S + 1, T))
+        bd = torch.tensor([[0, 0, S, T], [1, 2, 8, 37], [0, 5, 9, 40], [2, 0, 2, 30]],
+                          dtype=torch.int64, device=device)
+        grads = []
+        for which in range(3):
+            px = torch.tensor(npx, dtype=dtype, device=device, requires_grad=True)
+            py = torch.tensor(npy, dtype=dtype, device=device, requires_grad=True)
+            m = k2.mutual_information_recursion(px, py, bd)
+            m2 = k2.joint_mutual_information_recursion((px,), (py,), bd)
+            m3 = k2.joint_mutual_information_recursion((px * 0.5, px * 0.5), (py * 0.5, py * 0.5), bd)
+            assert m2.shape == (1, B) and m3.shape == (2, B)
+            tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=1e-10, atol=1e-10)
+            assert torch.allclose(m, m2[0], **tol)
+            assert torch.allclose(m, m3.sum(dim=0), **tol)
+            ((m, m2, m3)[which].sum() * 3).backward()
+            grads.append((px.grad.clone(), py.grad.clone()))
+        for gx, gy in grads[1:]:
+            assert torch.allclose(gx, grads[0][0], rtol=1e-4, atol=1e-5)
+            assert torch.allclose(gy, grads[0][1], rtol=1e-4, atol=1e-5)
+        # and the plain recursion's derivative is the oracle's occupation probabilities x 3
+        a, p = omi.mi_forward(npx, npy, bd.cpu().numpy())
+        wx, wy = omi.mi_backward(npx, npy, bd.cpu().numpy(), p)
+        np.testing.assert_allclose(grads[0][0].cpu().numpy(), 3 * wx, rtol=1e-4, atol=1e-5)
+        np.testing.assert_allclose(grads[0][1].cpu().numpy(), 3 * wy, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.gpu
+def test_log_deriv_is_left_alone_by_the_exact_kernels(device):
+    """fp64 (and fp32 without a workspace) run the one-workgroup-per-sequence kernels, which
+    neither write nor read the log-derivative tensor: the hosts say so and results are unchanged."""
+    from k2_amd import capi
+    rng = np.random.default_rng(3)
+    B, S, T = 2, 12, 30
+    px = torch.from_numpy(rng.standard_normal((B, S, T + 1))).to(device)
+    py = torch.from_numpy(rng.standard_normal((B, S + 1, T))).to(device)
+    assert not capi.mi_keeps_log_deriv(px, py)
+    p1 = torch.empty(B, S + 1, T + 1, dtype=torch.float64, device=device)
+    p2 = torch.empty_like(p1)
+    kept = torch.full_like(p1, 7.0)
+    a1 = capi.mi_forward(px, py, None, p1)
+    a2 = capi.mi_forward(px, py, None, p2, log_deriv=kept)
+    g1 = torch.ones(B, dtype=torch.float64, device=device)
+    g2 = torch.ones(B, dtype=torch.float64, device=device)
+    x1, y1 = capi.mi_backward(px, py, None, p1, g1)
+    x2, y2 = capi.mi_backward(px, py, None, p2, g2, log_deriv=kept)
+    torch.cuda.synchronize()
+    assert torch.equal(a1, a2) and torch.equal(x1, x2) and torch.equal(y1, y2)
+    assert bool((kept == 7.0).all())
+
+
+@pytest.mark.gpu
+def test_single_launch_serves_any_batch_and_says_what_it_does_not(device):
+    """The single launch hands its work to a fixed set of workgroups in an order in which every
+    wait is for work handed out earlier, so it needs no particular number of resident workgroups:
+    a batch with several times more chunks than the device has compute units is one launch like
+    any other.  fp64 and lattices of more rows than its join keeps are refused (the Python layer
+    then makes the two calls)."""
+    from k2_amd import capi
+    big = torch.zeros(300, 70, 11, device=device)   # 2 * 300 * 2 sweeps each way on 256 compute units
+    assert capi.mi_forward_backward_supported(big, torch.zeros(300, 71, 10, device=device))
+    px = torch.zeros(2, 5, 8, dtype=torch.float64, device=device)
+    py = torch.zeros(2, 6, 7, dtype=torch.float64, device=device)
+    assert not capi.mi_forward_backward_supported(px, py)
+    with pytest.raises(RuntimeError):
+        capi.mi_forward_backward(px, py, None, torch.ones(2, dtype=torch.float64, device=device))
+    tall = torch.zeros(1, 2100, 2101, device=device)
+    assert not capi.mi_forward_backward_supported(tall, torch.zeros(1, 2101, 2100, device=device))
+    import k2_amd as k2
+    bx = torch.randn(300, 70, 11, device=device)
+    by = torch.randn(300, 71, 10, device=device)
+    scores, (gx, gy) = k2.mutual_information_recursion(bx, by, None, return_grad=True)
+    small, (sx, sy) = k2.mutual_information_recursion(bx[:4].contiguous(), by[:4].contiguous(), None,
+                                                      return_grad=True)
+    assert torch.equal(scores[:4], small) and torch.equal(gx[:4], sx) and torch.equal(gy[:4], sy)
+    a, p = omi.mi_forward(bx.cpu().numpy(), by.cpu().numpy(), None)
+    wx, wy = omi.mi_backward(bx.cpu().numpy(), by.cpu().numpy(), None, p)
+    np.testing.assert_allclose(scores.cpu().numpy(), a, rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(gx.cpu().numpy(), wx, rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(gy.cpu().numpy(), wy, rtol=1e-4, atol=1e-5)
 
 
 @pytest.mark.gpu
@@ -265,7 +438,8 @@ def test_blocked_and_improbable_edges(device, modified):
     """Edges of log-probability -inf (a few per cent of them, so that whole regions of the lattice
     and some end cells become unreachable) and of -3000 (far below fp32's exp range): all kernels
     must agree with the CPU code's guards (k2/python/csrc/torch/mutual_information_cpu.cu:195-211)
-    and, as everywhere, with each other bit for bit."""
+    and the pairs of launches with each other bit for bit.  Sequences whose end cell no path reaches
+    take the exact recursion inside the single launch."""
     rng = np.random.default_rng(90 + int(modified))
     B, S, T = 4, 150, 210
     T1 = T if modified else T + 1

@@ -261,13 +261,21 @@ def test_config3_prune_and_pruned_loss_full_size(device):
     want_ranges = orn.prune_ranges(gx_w, gy_w, c["boundary"], R)
     got_ranges = k2.get_rnnt_prune_ranges(dev(gx_w, device), dev(gy_w, device), dev(c["boundary"], device), R)
     assert np.array_equal(got_ranges.cpu().numpy(), want_ranges)
-    # and through the device pipeline end to end (grads from the HIP MI kernel)
+    # And through the device pipeline end to end (occupation probabilities from the HIP kernels).
+    # Two fp32 pipelines round differently, and a frame whose two best windows are within that
+    # noise may go either way: the yardstick is the fp64 pipeline, with which the device's ranges
+    # must agree about as often as the reference's own fp32 pipeline does (within one per cent).
     _, (gx, gy) = k2.rnnt_loss_simple(dev(c["lm"], device), dev(c["am"], device), dev(c["symbols"], device), 0,
                                       dev(c["boundary"], device), reduction="none", return_grad=True)
     dev_ranges = k2.get_rnnt_prune_ranges(gx, gy, dev(c["boundary"], device), R).cpu().numpy()
-    frac = (dev_ranges == want_ranges).mean()
-    print("ranges identical to the CPU pipeline on", frac, "of elements")
-    assert frac > 0.999
+    f64 = lambda a: a.astype(np.float64)
+    _, (gx64, gy64) = orn.rnnt_loss_simple(f64(c["lm"]), f64(c["am"]), c["symbols"], 0, c["boundary"],
+                                            reduction="none", return_grad=True)
+    ranges64 = orn.prune_ranges(gx64, gy64, c["boundary"], R)
+    frac_dev, frac_cpu = (dev_ranges == ranges64).mean(), (want_ranges == ranges64).mean()
+    print("ranges identical to the fp64 pipeline's: device", frac_dev, " fp32 CPU", frac_cpu,
+          " device vs fp32 CPU", (dev_ranges == want_ranges).mean())
+    assert frac_dev > frac_cpu - 0.01
     logits = np.random.default_rng(33).standard_normal((B, T, R, C)).astype(np.float32)
     want = orn.rnnt_loss_pruned(logits, c["symbols"], want_ranges, 0, c["boundary"], reduction="none")
     got = k2.rnnt_loss_pruned(dev(logits, device), dev(c["symbols"], device), dev(want_ranges, device), 0,

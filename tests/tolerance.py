@@ -16,14 +16,19 @@ mode "absolute": the percentile of |cpu32 - f64| itself, for quantities that are
 So the GPU may be as far from the truth as twice what the reference's fp32 code is at that
 element, or, relative to the element's own size, twice what the reference's fp32 code is at the
 worst thousandth of the same sequence's elements; a tiny element is never granted a large
-element's noise.  The share of elements that needed the arbitration is returned, bounded by the
-caller and printed by the tests at the BASELINE sizes.
+element's noise.  A percentile is not a maximum: of tens of millions of elements a few lie in
+the far tail of either implementation's error, so up to TAIL_FRACTION of the elements (one in a
+hundred thousand) may exceed that budget, by no more than TAIL_FACTOR times.  The share of
+elements that needed the arbitration is returned, bounded by the caller and printed by the tests
+at the BASELINE sizes.
 """
 import numpy as np
 
 RTOL, ATOL = 1e-4, 1e-5
 QUANTILE = 0.999
 MIN_MAGNITUDE = 1e-4
+TAIL_FRACTION = 1e-5
+TAIL_FACTOR = 4.0
 
 # name -> dict of the figures of the last comparison under that name (read by tests that report)
 last_stats = {}
@@ -70,10 +75,16 @@ def close_f32(name, got, want32, want64, max_arbitrated=1.0, mode="relative"):
             ref_err = np.abs(w32 - w64)
             q = _per_sequence_quantile(ref_err, np.abs(w64), mode)
             floor = q * np.abs(w64) if mode == "relative" else q
-            budget = ATOL + RTOL * np.abs(w64) + 2.0 * np.maximum(ref_err, floor)
-            ok = plain | (got == w64) | (np.abs(got - w64) <= budget)
+            noise = 2.0 * np.maximum(ref_err, floor)
+            err = np.abs(got - w64)
+            ok = plain | (got == w64) | (err <= ATOL + RTOL * np.abs(w64) + noise)
+            ok_tail = ok | (err <= ATOL + RTOL * np.abs(w64) + TAIL_FACTOR * noise)
         stats["reference_error_quantile_max"] = float(np.max(q))
-        assert ok.all(), (name, int((~ok).sum()), got[~ok][:5], w32[~ok][:5], w64[~ok][:5], stats)
+        stats["tail"] = int((~ok).sum())
+        assert ok_tail.all(), (name, int((~ok_tail).sum()), got[~ok_tail][:5], w32[~ok_tail][:5],
+                               w64[~ok_tail][:5], stats)
+        assert stats["tail"] <= TAIL_FRACTION * got.size, (name, stats["tail"], got[~ok][:5], w32[~ok][:5],
+                                                            w64[~ok][:5], stats)
         stats["arbitrated"] = int((~plain).sum())
         stats["arbitrated_frac"] = stats["arbitrated"] / max(got.size, 1)
     assert stats["arbitrated_frac"] <= max_arbitrated, (name, stats)
