@@ -383,7 +383,8 @@ constexpr int kFwdLoadsPerBlock = 2 * FwdLayout::kLoadItems + 1;
 // kBidir: the sweep covers the half `half` of the lattice (see Half) and ends on its cut
 // diagonal; what the chain holds there (p of the half's last cell of every row) goes to
 // cut_out[0..63] (the chunk's 64 own rows; the finite stand-in for -inf where a row has no cell
-// on the cut or lies past the sequence's last row), ans is not written, and log_deriv has rows of
+// on the cut or lies past the sequence's last row) and *cut_arrive is then incremented (once per
+// call, whatever the chunk holds), ans is not written, and log_deriv has rows of
 // Tn + 2 floats (the two halves of a sequence share one slab: the mirrored half's cells lie one
 // column to the right of their place, where no cell of the other half is).
 template <bool kKeep, bool kWriteP, bool kBidir>
@@ -391,7 +392,8 @@ __device__ __forceinline__ void MiForwardChunk(
     FwdLds &lds, const float *__restrict__ px, const float *__restrict__ py, const Box &box,
     float *__restrict__ p, float *__restrict__ ans,
     float *__restrict__ log_deriv, FastHeader *hdr, float *edge, int B, int S, int Tn,
-    int modified, int nchunks, int edge_stride, int seq, int chunk, Half half, float *cut_out) {
+    int modified, int nchunks, int edge_stride, int seq, int chunk, Half half, float *cut_out,
+    unsigned *cut_arrive) {
   static_assert(!kBidir || (kKeep && !kWriteP), "the halves keep the log-derivatives only");
   ChunkGeom g;
   g.b = seq;
@@ -400,6 +402,8 @@ __device__ __forceinline__ void MiForwardChunk(
   g.row0 = g.c * kRows;
   if (!box.ok || g.row0 > g.ns) {
     if (!kBidir && !box.ok && g.c == 0 && threadIdx.x == 0) ans[g.b] = __builtin_nanf("");
+    if (kBidir && threadIdx.x == 0)
+      __hip_atomic_fetch_add(cut_arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return;
   }
   g.skew = modified ? 0 : 1;
@@ -412,7 +416,11 @@ __device__ __forceinline__ void MiForwardChunk(
   const int n_last = nsteps - 1;  // the chunk's step on the cut diagonal (kBidir)
   g.nblocks = blocks_of(g.row0);
   if (kBidir && g.nblocks == 0) {  // no cell of these rows lies in the half
-    if (threadIdx.x < kRows) PublishCut(cut_out + threadIdx.x, kLogZero);
+    if (threadIdx.x < kRows) {
+      PublishCut(cut_out + threadIdx.x, kLogZero);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      if (threadIdx.x == 0) __hip_atomic_fetch_add(cut_arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
     return;
   }
   const bool has_down = g.row0 + kRows <= g.ns && blocks_of(g.row0 + kRows) > 0;
@@ -705,11 +713,15 @@ __device__ __forceinline__ void MiForwardChunk(
   // the chain wavefront is the critical path: it wins the SIMD's issue arbitration
   if (role == kChain) __builtin_amdgcn_s_setprio(3);
   // ---- prologue: block 0 committed, blocks 1 .. kFwdSets in flight --------------------------
-  // A block's loads stay in flight for kFwdSets iterations (~1 us each).  A third set changes
-  // nothing, neither with inputs that the caches hold nor with inputs that come from HBM
-  // (84 us against 85 us per launch of the B=32 S=200 T=1000 workload), and its registers would
-  // cost the second workgroup on a compute unit.
-  constexpr int kFwdSets = 2;
+  // A block's loads stay in flight for kFwdSets iterations (~1.2 us each).  Two sets serve the
+  // separate forward kernel, whose registers decide whether a second workgroup fits a compute
+  // unit.  The single launch has a unit per workgroup, and 2 x 256 of its sweeps read from HBM at
+  // once: there two sets leave every iteration waiting for its loads when the inputs are not in
+  // the Infinity Cache (1.55 us per block against 1.2).
+#ifndef K2AMD_FWD_SETS
+#define K2AMD_FWD_SETS 2
+#endif
+  constexpr int kFwdSets = kBidir ? K2AMD_FWD_SETS : 2;
   FwdRegs sets[kFwdSets];
   if (role == kLoader) {
     load_block(0, sets[0]);
@@ -768,15 +780,20 @@ __device__ __forceinline__ void MiForwardChunk(
   K2AMD_TRACE_MARK(half, 6);
   if (role == kStorer) store_block(g.nblocks - 1);
   if (role == kEdge) publish_block(g.nblocks - 1);
-  if (kBidir) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the coherent stores above
-  if (kBidir && wave == 2 + L::kLoaderWaves) {
+  if (kBidir && role == kChain) {
     // What the chain left on the cut diagonal: step n_last of every row, still in the ring.  (A
     // chunk that ran out of columns before the cut has no cell on it; a row whose cell on the cut
-    // lies outside the columns holds a stand-in for -inf there already.)
+    // lies outside the columns holds a stand-in for -inf there already.)  The chain wavefront
+    // has no other store in flight, so its wait below is for these 64 words only: the sequence's
+    // join on the cut can start while the other wavefronts' log-derivatives are still on
+    // their way.
     const int at = ((g.nblocks - 1) % 3) * kW + (n_last - (g.nblocks - 1) * kW);
     const bool on_cut = half.dmax - g.row0 * g.skew == n_last && g.row0 + lane <= g.ns;
     PublishCut(cut_out + lane, on_cut ? reinterpret_cast<const float *>(&lds.fy[lane][0])[at] : kLogZero);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (lane == 0) __hip_atomic_fetch_add(cut_arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
+  if (kBidir) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the coherent stores above
 }
 
 // One workgroup per chunk; the ticket fixes which (see the file header).
@@ -793,7 +810,7 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiForwardFastKernel(
   MiForwardChunk<kKeep, kWriteP, false>(lds, px, py, LoadBox(boundary, (int)(ticket / nchunks), S, Tn), p,
                                         ans, log_deriv, hdr, edge, B, S, Tn, modified, nchunks,
                                         edge_stride, (int)(ticket / nchunks), (int)(ticket % nchunks),
-                                        Half{}, nullptr);
+                                        Half{}, nullptr, nullptr);
   if (threadIdx.x == 0) FinishWorkgroup(hdr, gridDim.x);
 }
 
@@ -1351,12 +1368,13 @@ struct CutShared {
   unsigned ticket;
 };
 
-// Per sequence, in the workspace: arrive (forward sweeps finished), depart (readers of the cut
-// finished), the gradient of the sequence's score, then alpha by own row of the first half and
-// beta by own row of the second.  Counters count up from the sentinel, which is what the
+// Per sequence, in the workspace: arrive (forward sweeps whose values on the cut are there),
+// depart (readers of the cut finished), the gradient of the sequence's score, stored (forward
+// sweeps whose log-derivatives have all reached memory), then alpha by own row of the first half
+// and beta by own row of the second.  Counters count up from the sentinel, which is what the
 // workspace is initialised to.
 struct CutWords {
-  unsigned *arrive, *depart;
+  unsigned *arrive, *depart, *stored;
   float *scale, *alpha, *beta;
   int words;
 };
@@ -1367,6 +1385,7 @@ __device__ __forceinline__ CutWords CutOf(float *cut, int b, int nchunks) {
   w.arrive = reinterpret_cast<unsigned *>(base);
   w.depart = reinterpret_cast<unsigned *>(base) + 1;
   w.scale = base + 2;
+  w.stored = reinterpret_cast<unsigned *>(base) + 3;
   w.alpha = base + kCutWordsPerSeqHeader;
   w.beta = w.alpha + nchunks * kRows;
   return w;
@@ -1487,11 +1506,12 @@ struct TaskShared {
   Box box;
 };
 __device__ __attribute__((noinline)) void BidirForwardTask(FwdLds &lds, const TaskShared &t, int seq,
-                                                           int chunk, Half half, float *cut_out) {
+                                                           int chunk, Half half, float *cut_out,
+                                                           unsigned *cut_arrive) {
   const BidirArgs &k = t.k;
   MiForwardChunk<true, false, true>(lds, k.px, k.py, t.box, nullptr, k.ans, k.scratch, k.hdr,
                                     half.mirror ? k.edge1 : k.edge0, k.B, k.S, k.Tn, k.modified,
-                                    k.nchunks, k.edge_stride, seq, chunk, half, cut_out);
+                                    k.nchunks, k.edge_stride, seq, chunk, half, cut_out, cut_arrive);
 }
 __device__ __attribute__((noinline)) void BidirBackwardTask(BwdLds &lds, const TaskShared &t, int seq,
                                                             int chunk, Half half, const float *seeds) {
@@ -1579,12 +1599,13 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiBidirKernel(const Bidir
     if (fwd) {
       if (!mirror && chunk == 0 && threadIdx.x == 0)
         PublishCut(cw.scale, k.ans_grad != nullptr ? k.ans_grad[seq] : 1.0f);
-      BidirForwardTask(lds.fwd, ts, seq, chunk, half, (mirror ? cw.beta : cw.alpha) + chunk * kRows);
+      BidirForwardTask(lds.fwd, ts, seq, chunk, half, (mirror ? cw.beta : cw.alpha) + chunk * kRows,
+                       cw.arrive);
       // every wavefront has waited for its stores (device-coherent ones, see StoreQuadCoherent)
       // before this barrier: whichever compute unit sweeps this chunk back will see them
       __syncthreads();
       if (threadIdx.x == 0)
-        __hip_atomic_fetch_add(cw.arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_fetch_add(cw.stored, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       continue;
     }
 
@@ -1595,8 +1616,15 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiBidirKernel(const Bidir
 #ifdef K2AMD_MI_TRACE
     tracer.mark(1);
 #endif
+    // The join runs while the last log-derivatives are on their way; they are needed after it.
+    // (The look at their counter is asked for before the join and used after it: one trip to
+    // memory less where they have all arrived by then.)
+    unsigned stored = 0;
+    if (threadIdx.x == 0) stored = __hip_atomic_load(cw.stored, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (box.ok) total = CutJoin(sh, cw, ns, chunk * kRows, mirror);
     const float seed = sh.scale;
+    if (threadIdx.x == 0 && stored != kSentinel + per_seq) WaitCount(cw.stored, kSentinel + per_seq, k.hdr);
+    __syncthreads();
     // This task has read the sequence's cut words.  The last of their readers puts them back into
     // their initial state; the count comes back while the sweep below runs and is looked at after it.
     unsigned departed = 0;
