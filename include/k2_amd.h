@@ -144,9 +144,14 @@ K2AMD_API int k2amd_mi_backward_kept(const void *px, const void *py, const int64
  * out earlier, so the launch needs no particular number of resident workgroups and is safe next
  * to other streams' kernels.  It serves fp32 with a workspace and S + 2 <= 2056:
  * k2amd_mi_forward_backward_supported(...) says whether a call will be served (1) or returns
- * K2AMD_ERR_UNSUPPORTED (0; use the two calls).                                                  */
+ * K2AMD_ERR_UNSUPPORTED (0; use the two calls).  k2amd_mi_forward_backward_advised(...) says
+ * whether it is also the faster way on the current device (1): it is while the device has a compute
+ * unit for every half-sweep, 2 * B * ceil((S+1)/64) of them, at once; beyond that the two calls,
+ * whose kernels share compute units, take less time, and a host that has the choice makes them. */
 K2AMD_API int k2amd_mi_forward_backward_supported(int B, int S, int T, int modified, int dtype,
                                         int has_workspace);
+K2AMD_API int k2amd_mi_forward_backward_advised(int B, int S, int T, int modified, int dtype,
+                                      int has_workspace);
 K2AMD_API size_t k2amd_mi_forward_backward_scratch_bytes(int B, int S, int T, int modified, int dtype);
 K2AMD_API int k2amd_mi_forward_backward(const void *px, const void *py, const int64_t *boundary, void *ans,
                               void *scratch, size_t scratch_bytes, void *ans_grad, void *px_grad,
@@ -247,6 +252,41 @@ K2AMD_API int k2amd_rnnt_prune_gather(const void *lm, const int64_t *ranges, voi
 K2AMD_API int k2amd_rnnt_prune_gather_backward(const void *grad, const int64_t *ranges,
                                                void *lm_grad, int B, int S1, int T, int R, int D,
                                                int dtype, void *stream);
+
+/* ------------------------------------------------------------------ pruned joiner, fused
+ *
+ * What stands between do_rnnt_pruning (k2/python/k2/rnnt_loss.py:913-954) and rnnt_loss_pruned
+ * (rnnt_loss.py:1351-1468) in the reference's recipes is the caller's joiner; these two calls run
+ * the usual one, logits = tanh(am_pruned + lm_pruned) . weight^T + bias, TOGETHER with the gather
+ * before it and get_rnnt_logprobs_pruned (rnnt_loss.py:1180-1348) after it, so that the
+ * [B][T][R][C] logits never exist in memory (the reference has no such call; its torch-op chain
+ * do_rnnt_pruning -> tanh -> linear -> get_rnnt_logprobs_pruned is what they are checked against).
+ *   am [B][T][D], lm [B][S+1][D], ranges [B][T][R] int64, weight [C][D] (torch.nn.Linear's
+ *   layout), bias [C] or NULL, symbols [B][S]; all floating tensors fp32.
+ *   px, py, normalizers [B][T][R]: as k2amd_rnnt_logprobs_pruned_forward.
+ *   precision: K2AMD_JOINER_F32 multiplies in fp32 on the matrix cores; K2AMD_JOINER_BF16 rounds the
+ *   activations, the weight and the logits' gradients to bfloat16 for the products (fp32 sums).
+ *   workspace: k2amd_rnnt_joiner_pruned_workspace_bytes(...) bytes of device memory (0 = shape
+ *   not served: D a multiple of 64 up to 512, R <= 32; K2AMD_ERR_UNSUPPORTED also where C is too
+ *   large for the backward's tiles); contents need not survive between the two calls.
+ * The backward takes what the forward took, the normalizers it wrote and the gradients w.r.t. its
+ * px / py (seq_scale as for the other builders), and writes am_grad [B][T][D], lm_grad [B][S+1][D],
+ * weight_grad [C][D], bias_grad [C] (or NULL).  lm_grad, weight_grad and bias_grad are sums formed
+ * with floating-point atomic adds: their last bits vary from run to run.                        */
+enum k2amd_joiner_precision { K2AMD_JOINER_F32 = 0, K2AMD_JOINER_BF16 = 1 };
+K2AMD_API size_t k2amd_rnnt_joiner_pruned_workspace_bytes(int B, int S, int T, int R, int C, int D,
+                                                          int precision);
+K2AMD_API int k2amd_rnnt_joiner_pruned_forward(
+    const void *am, const void *lm, const int64_t *ranges, const void *weight, const void *bias,
+    const int64_t *symbols, const int64_t *boundary, void *px, void *py, void *normalizers, int B,
+    int S, int T, int R, int C, int D, int termination_symbol, int rnnt_type, int precision,
+    void *workspace, size_t workspace_bytes, void *stream);
+K2AMD_API int k2amd_rnnt_joiner_pruned_backward(
+    const void *am, const void *lm, const int64_t *ranges, const void *weight, const void *bias,
+    const int64_t *symbols, const int64_t *boundary, const void *normalizers, const void *px_grad,
+    const void *py_grad, const void *seq_scale, void *am_grad, void *lm_grad, void *weight_grad,
+    void *bias_grad, int B, int S, int T, int R, int C, int D, int termination_symbol, int rnnt_type,
+    int precision, void *workspace, size_t workspace_bytes, void *stream);
 
 /* ------------------------------------------------------------------ lattice
  *

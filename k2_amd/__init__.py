@@ -18,6 +18,7 @@ from .rnnt_loss import get_rnnt_prune_ranges
 from .rnnt_loss import get_rnnt_prune_ranges_deprecated
 from .rnnt_loss import rnnt_loss
 from .rnnt_loss import rnnt_loss_pruned
+from .rnnt_loss import rnnt_loss_pruned_joiner
 from .rnnt_loss import rnnt_loss_simple
 from .rnnt_loss import rnnt_loss_smoothed
 
@@ -28,5 +29,5 @@ __all__ = [
     "get_rnnt_logprobs", "get_rnnt_logprobs_joint", "get_rnnt_logprobs_pruned",
     "get_rnnt_prune_ranges", "rnnt_loss", "rnnt_loss_pruned", "rnnt_loss_simple",
     "get_hat_logprobs_pruned", "get_rnnt_logprobs_smoothed", "rnnt_loss_smoothed",
-    "get_rnnt_prune_ranges_deprecated", "pruned_ranges_to_lattice",
+    "get_rnnt_prune_ranges_deprecated", "pruned_ranges_to_lattice", "rnnt_loss_pruned_joiner",
 ]

@@ -36,6 +36,7 @@ _SIGNATURES = {
     "k2amd_mi_forward_keep": ([_vp] * 6 + [_ci] * 5 + [_vp, _sz, _vp], _ci),
     "k2amd_mi_backward_kept": ([_vp] * 8 + [_ci] * 6 + [_vp, _sz, _vp], _ci),
     "k2amd_mi_forward_backward_supported": ([_ci] * 6, _ci),
+    "k2amd_mi_forward_backward_advised": ([_ci] * 6, _ci),
     "k2amd_mi_forward_backward_scratch_bytes": ([_ci] * 5, _sz),
     "k2amd_mi_forward_backward": ([_vp] * 5 + [_sz] + [_vp] * 3 + [_ci] * 6 + [_vp, _sz, _vp], _ci),
     "k2amd_rnnt_logprobs_simple_forward": ([_vp] * 11 + [_ci] * 7 + [_vp], _ci),
@@ -46,6 +47,9 @@ _SIGNATURES = {
     "k2amd_rnnt_logprobs_pruned_backward": ([_vp] * 9 + [_ci] * 8 + [_vp], _ci),
     "k2amd_rnnt_hat_logprobs_pruned_forward": ([_vp] * 7 + [_ci] * 7 + [_vp], _ci),
     "k2amd_rnnt_hat_logprobs_pruned_backward": ([_vp] * 9 + [_ci] * 7 + [_vp], _ci),
+    "k2amd_rnnt_joiner_pruned_workspace_bytes": ([_ci] * 7, _sz),
+    "k2amd_rnnt_joiner_pruned_forward": ([_vp] * 10 + [_ci] * 9 + [_vp, _sz, _vp], _ci),
+    "k2amd_rnnt_joiner_pruned_backward": ([_vp] * 15 + [_ci] * 9 + [_vp, _sz, _vp], _ci),
     "k2amd_rnnt_prune_ranges": ([_vp] * 4 + [_ci] * 6 + [_vp], _ci),
     "k2amd_rnnt_prune_gather": ([_vp] * 3 + [_ci] * 6 + [_vp], _ci),
     "k2amd_rnnt_prune_gather_backward": ([_vp] * 3 + [_ci] * 6 + [_vp], _ci),
@@ -263,6 +267,17 @@ def mi_forward_backward_supported(px, py):
         return bool(lib().k2amd_mi_forward_backward_supported(B, S, T, int(T1 == T), dt, int(has_ws)))
 
 
+def mi_forward_backward_advised(px, py):
+    """True if mi_forward_backward serves these tensors and is the faster way on their device (the
+    device has a compute unit for every half-sweep of the launch at once)."""
+    B, S, T1 = px.shape
+    T = py.shape[2]
+    dt = dtype_code(px)
+    has_ws = lib().k2amd_mi_workspace_bytes(B, S, T, int(T1 == T), dt) > 0
+    with torch.cuda.device(px.device):
+        return bool(lib().k2amd_mi_forward_backward_advised(B, S, T, int(T1 == T), dt, int(has_ws)))
+
+
 def mi_forward_backward(px, py, boundary, ans_grad, overwrite_ans_grad=True):
     """Forward and backward recursion in one launch: returns (ans, px_grad, py_grad)."""
     B, S, T, modified = _mi_shapes(px, py, boundary)
@@ -449,6 +464,79 @@ def logprobs_pruned_backward(logits, norm, px_grad, py_grad, symbols, ranges, bo
             ptr(ranges), ptr(boundary), ptr(grad), B, S, T, R, C, termination_symbol, rnnt_type,
             dtype_code(logits), stream_ptr(dev)))
     return grad
+
+
+JOINER_PRECISIONS = {"fp32": 0, "bf16": 1}
+
+
+def _joiner_shapes(am, lm, ranges, weight, bias, symbols, boundary, termination_symbol, rnnt_type,
+                   precision):
+    """Checks every tensor of the fused joiner calls; returns (B, S, T, R, C, D, workspace)."""
+    dev = am.device
+    if am.dtype != torch.float32:
+        raise RuntimeError(f"k2_amd: the fused joiner takes float32 tensors, am is {am.dtype}")
+    if precision not in (0, 1):
+        raise RuntimeError(f"k2_amd: unknown joiner precision code {precision}")
+    B, T, D = _dims(am, "am", 3)
+    S1 = _dims(lm, "lm", 3)[1]
+    R = _dims(ranges, "ranges", 3)[2]
+    C = _dims(weight, "weight", 2)[0]
+    S = S1 - 1
+    _rnnt_type(rnnt_type)
+    expect(am, "am", torch.float32, dev, (B, T, D))
+    expect(lm, "lm", torch.float32, dev, (B, S1, D))
+    expect(ranges, "ranges", torch.int64, dev, (B, T, R))
+    expect(weight, "weight", torch.float32, dev, (C, D))
+    expect_optional(bias, "bias", torch.float32, dev, (C,))
+    expect(symbols, "symbols", torch.int64, dev, (B, S))
+    expect_optional(boundary, "boundary", torch.int64, dev, (B, 4))
+    _symbol(termination_symbol, C)
+    nbytes = lib().k2amd_rnnt_joiner_pruned_workspace_bytes(B, S, T, R, C, D, precision)
+    if nbytes == 0:
+        raise RuntimeError(f"k2_amd: the fused joiner does not serve B={B} S={S} T={T} R={R} C={C} D={D} "
+                           "(D must be a multiple of 64 up to 512, R at most 32 and S + 1)")
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    return B, S, T, R, C, D, ws
+
+
+def joiner_pruned_forward(am, lm, ranges, weight, bias, symbols, termination_symbol, boundary,
+                          rnnt_type, precision=0):
+    """tanh(am[b,t] + lm[b,ranges[b,t,k]]) . weight^T + bias and get_rnnt_logprobs_pruned on it in one
+    pass: returns (px, py, normalizers [B][T][R]); the logits never exist in memory."""
+    B, S, T, R, C, D, ws = _joiner_shapes(am, lm, ranges, weight, bias, symbols, boundary,
+                                          termination_symbol, rnnt_type, precision)
+    dev = am.device
+    px = torch.empty(B, S, _t1(T, rnnt_type), dtype=torch.float32, device=dev)
+    py = torch.empty(B, S + 1, T, dtype=torch.float32, device=dev)
+    norm = torch.empty(B, T, R, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        check(lib().k2amd_rnnt_joiner_pruned_forward(
+            ptr(am), ptr(lm), ptr(ranges), ptr(weight), ptr(bias), ptr(symbols), ptr(boundary),
+            ptr(px), ptr(py), ptr(norm), B, S, T, R, C, D, termination_symbol, rnnt_type, precision,
+            ptr(ws), ws.numel(), stream_ptr(dev)))
+    return px, py, norm
+
+
+def joiner_pruned_backward(am, lm, ranges, weight, bias, symbols, termination_symbol, boundary,
+                           rnnt_type, norm, px_grad, py_grad, seq_scale=None, precision=0):
+    """Gradients of sum_b seq_scale[b] * score_b through the fused joiner: returns (am_grad, lm_grad,
+    weight_grad, bias_grad or None)."""
+    B, S, T, R, C, D, ws = _joiner_shapes(am, lm, ranges, weight, bias, symbols, boundary,
+                                          termination_symbol, rnnt_type, precision)
+    dev = am.device
+    expect(norm, "normalizers", torch.float32, dev, (B, T, R))
+    _expect_lattice_grads(px_grad, py_grad, seq_scale, torch.float32, dev, B, S, T, rnnt_type)
+    am_grad = torch.empty_like(am)
+    lm_grad = torch.empty_like(lm)
+    weight_grad = torch.empty_like(weight)
+    bias_grad = torch.empty_like(bias) if bias is not None else None
+    with torch.cuda.device(dev):
+        check(lib().k2amd_rnnt_joiner_pruned_backward(
+            ptr(am), ptr(lm), ptr(ranges), ptr(weight), ptr(bias), ptr(symbols), ptr(boundary),
+            ptr(norm), ptr(px_grad), ptr(py_grad), ptr(seq_scale), ptr(am_grad), ptr(lm_grad),
+            ptr(weight_grad), ptr(bias_grad), B, S, T, R, C, D, termination_symbol, rnnt_type,
+            precision, ptr(ws), ws.numel(), stream_ptr(dev)))
+    return am_grad, lm_grad, weight_grad, bias_grad
 
 
 def prune_ranges(px_grad, py_grad, boundary, s_range):

@@ -1,0 +1,806 @@
+// The pruned joiner fused with the log-prob builder that consumes its output:
+//
+//   logits[b,t,k,:] = tanh(am[b,t,:] + lm[b, ranges[b,t,k], :]) . weight^T + bias
+//   px, py          = get_rnnt_logprobs_pruned(logits, ...)
+//
+// i.e. do_rnnt_pruning (k2/python/k2/rnnt_loss.py:913-954), the joiner the reference leaves to the
+// caller between it and rnnt_loss_pruned, and get_rnnt_logprobs_pruned (rnnt_loss.py:1180-1348).
+// The [B][T][R][C] logits only ever exist as tiles in registers: the forward multiplies a tile of
+// rows by the weight on the matrix cores, folds each tile of columns into a running log-sum-exp and
+// picks out the two logits a row contributes; the backward multiplies again and forms
+// d logits = -softmax (gx + gy) + gx [c == symbol] + gy [c == blank] on the fly, once per tile of
+// rows (for the gradients of am and lm) and once per slice of columns (for those of the weight).
+//
+// One row of the product is (b, t, k); a tile holds whole frames (b, t), R rows each, so the sum
+// over k that am's gradient needs stays inside a tile.  Operands: `F32` multiplies fp32 by fp32
+// (v_mfma_f32_32x32x2_f32: the products and sums of an fp32 matrix multiply), `Bf16` rounds
+// tanh(..), the weight and d logits to bfloat16 and multiplies with v_mfma_f32_32x32x16_bf16; both
+// accumulate in fp32, and everything outside the products is fp32.
+//
+// Data movement: the activations tanh(..) of a tile are formed once and kept in LDS ([row][k], k
+// contiguous); the weight is read from a copy prepared per call in the operand type, padded with
+// zeros to whole tiles, once with k = D contiguous (for logits) and once with k = C contiguous (for
+// d logits . weight).  A lane's share of an operand per step of k is 64 contiguous bytes (16 floats
+// or 32 bfloat16) of its row: four 16-byte loads from LDS or from the weight copy (which stays in
+// L2).  Which k a lane feeds to which multiply is the same for both operands, which is all the
+// instruction needs.
+#include "common.h"
+
+namespace k2amd {
+namespace {
+
+typedef float Acc16 __attribute__((ext_vector_type(16)));
+typedef __bf16 Bf8 __attribute__((ext_vector_type(8)));
+
+constexpr int kThreads = 256;   // four wavefronts
+constexpr int kNTile = 128;     // columns of a product per pass: 32 per wavefront
+constexpr int kSliceCols = 64;  // columns of d logits a workgroup of the weight-gradient kernel owns
+constexpr int kMaxD = 512;      // joiner dimension the LDS tiles are sized for
+constexpr int kMaxDBlocks = kMaxD / 64;  // 32-column blocks of D per wavefront in the weight gradient
+
+struct Frag {
+  uint4 q[4];
+};
+
+__device__ __forceinline__ float AsFloat(unsigned u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ unsigned AsBits(float f) { return __builtin_bit_cast(unsigned, f); }
+
+// round to nearest even; NaN stays NaN
+__device__ __forceinline__ unsigned short ToBf16(float f) {
+  unsigned u = AsBits(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (unsigned short)(u >> 16);
+}
+__device__ __forceinline__ float FromBf16(unsigned short h) { return AsFloat((unsigned)h << 16); }
+
+// tanh(x) = sign(x) (1 - e) / (1 + e), e = exp(-2|x|): absolute error ~1e-7, which is what the
+// logits (sums of D such values times weights) are sensitive to.
+__device__ __forceinline__ float Tanh(float x) {
+  const float e = __expf(-2.0f * fabsf(x));
+  const float t = (1.0f - e) / (1.0f + e);
+  return x < 0 ? -t : t;
+}
+
+struct F32 {
+  typedef float Elem;
+  static constexpr int kChunk = 32;  // k per step
+  static constexpr int kPad = 4;     // elements: rows 16 bytes apart modulo 256 (LDS banks)
+  static __device__ __forceinline__ Elem From(float f) { return f; }
+  static __device__ __forceinline__ float To(Elem e) { return e; }
+  static __device__ __forceinline__ void Mma(Acc16 &acc, const Frag &a, const Frag &b) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(AsFloat(a.q[i].x), AsFloat(b.q[i].x), acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(AsFloat(a.q[i].y), AsFloat(b.q[i].y), acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(AsFloat(a.q[i].z), AsFloat(b.q[i].z), acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(AsFloat(a.q[i].w), AsFloat(b.q[i].w), acc, 0, 0, 0);
+    }
+  }
+  static __device__ __forceinline__ void Store4(Elem *dst, float4 v) {
+    *reinterpret_cast<float4 *>(dst) = v;
+  }
+};
+
+struct Bf16 {
+  typedef unsigned short Elem;
+  static constexpr int kChunk = 64;
+  static constexpr int kPad = 8;
+  static __device__ __forceinline__ Elem From(float f) { return ToBf16(f); }
+  static __device__ __forceinline__ float To(Elem e) { return FromBf16(e); }
+  static __device__ __forceinline__ void Mma(Acc16 &acc, const Frag &a, const Frag &b) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(Bf8, a.q[i]),
+                                                    __builtin_bit_cast(Bf8, b.q[i]), acc, 0, 0, 0);
+  }
+  static __device__ __forceinline__ void Store4(Elem *dst, float4 v) {
+    uint2 p;
+    p.x = (unsigned)ToBf16(v.x) | ((unsigned)ToBf16(v.y) << 16);
+    p.y = (unsigned)ToBf16(v.z) | ((unsigned)ToBf16(v.w) << 16);
+    *reinterpret_cast<uint2 *>(dst) = p;
+  }
+};
+
+// 64 bytes of an operand row (16-byte aligned by construction of every caller)
+template <typename Elem>
+__device__ __forceinline__ Frag LoadFrag(const Elem *p) {
+  const uint4 *v = reinterpret_cast<const uint4 *>(p);
+  Frag f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) f.q[i] = v[i];
+  return f;
+}
+
+struct JoinerArgs {
+  const float *am, *lm, *bias;  // bias may be null
+  const int64_t *ranges, *symbols, *boundary;
+  const void *wk;   // weight copy [Cpad][D], k = D contiguous
+  const void *wc;   // weight copy [Dpad][Cpad], k = C contiguous
+  float *px, *py, *norm;        // forward outputs (norm [B][T][R])
+  const float4 *hdr;            // backward: per row {gx, gy, symbol, norm}
+  float *am_grad, *lm_grad, *weight_grad, *bias_grad;
+  int B, S, Tn, R, C, D, blank, rnnt_type;
+  int Cpad, Dpad;               // C, D rounded up to whole tiles of kNTile
+  int tpt;                      // frames per tile of rows
+  long long frames;             // B * Tn
+};
+
+struct RowMeta {
+  int bt;     // frame b * Tn + t
+  int lmrow;  // b * (S + 1) + ranges[b,t,k] (clamped into the sequence's rows)
+  int s;      // lattice row (ranges[b,t,0] + k) mod (S + 1)
+  int sym;    // symbol whose logit goes to px, or -1
+};
+
+// Where row (b, t, k) takes its lm vector from, where it lands in the lattice and which symbol it
+// scores (k2/python/k2/rnnt_loss.py:1282-1316).
+__device__ __forceinline__ RowMeta MetaOf(const JoinerArgs &a, long long frame, int k) {
+  RowMeta m;
+  const int b = (int)(frame / a.Tn);
+  const int64_t *r = a.ranges + (size_t)frame * a.R;
+  const int64_t shift = r[0], src = r[k];
+  const int S1 = a.S + 1;
+  int ss = (int)((k + shift) % S1);
+  if (ss < 0) ss += S1;
+  m.bt = (int)frame;
+  m.s = ss;
+  const int64_t clamped = src < 0 ? 0 : (src > a.S ? a.S : src);
+  m.lmrow = b * S1 + (int)clamped;
+  if (src >= 0 && src < a.S) m.sym = (int)a.symbols[(size_t)b * a.S + src];
+  else if (src == a.S) m.sym = a.blank;
+  else m.sym = -1;
+  if (m.sym < 0 || m.sym >= a.C) m.sym = -1;
+  return m;
+}
+
+// The rows of a tile: frames f0 .. f0 + nf - 1, row = (frame - f0) * R + k.
+template <int MT>
+__device__ __forceinline__ int LoadMeta(const JoinerArgs &a, long long f0, RowMeta *meta) {
+  const long long left = a.frames - f0;
+  const int nf = (int)(left < a.tpt ? left : a.tpt);
+  const int rows = nf * a.R;
+  for (int m = threadIdx.x; m < MT; m += kThreads) {
+    if (m < rows) {
+      meta[m] = MetaOf(a, f0 + m / a.R, m % a.R);
+    } else {
+      RowMeta z; z.bt = 0; z.lmrow = 0; z.s = 0; z.sym = -1;
+      meta[m] = z;
+    }
+  }
+  return rows;
+}
+
+// h[m][:] = tanh(am[frame] + lm[lmrow]) for the tile's rows (zeros beyond them), in the operand
+// type; kTransposed also keeps a copy ht[d][m] (k = row contiguous, for the weight gradient).
+template <typename Mode, int MT, bool kTransposed>
+__device__ __forceinline__ void StageActivations(const JoinerArgs &a, const RowMeta *meta, int rows,
+                                                 typename Mode::Elem *h, int ldh,
+                                                 typename Mode::Elem *ht, int ldt) {
+  const int qpr = a.D >> 2;
+  for (int idx = threadIdx.x; idx < MT * qpr; idx += kThreads) {
+    const int m = idx / qpr, q = idx - m * qpr;
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (m < rows) {
+      const RowMeta rm = meta[m];
+      const float4 x = *reinterpret_cast<const float4 *>(a.am + (size_t)rm.bt * a.D + 4 * q);
+      const float4 y = *reinterpret_cast<const float4 *>(a.lm + (size_t)rm.lmrow * a.D + 4 * q);
+      v = make_float4(Tanh(x.x + y.x), Tanh(x.y + y.y), Tanh(x.z + y.z), Tanh(x.w + y.w));
+    }
+    Mode::Store4(h + (size_t)m * ldh + 4 * q, v);
+    if (kTransposed) {
+      ht[(size_t)(4 * q + 0) * ldt + m] = Mode::From(v.x);
+      ht[(size_t)(4 * q + 1) * ldt + m] = Mode::From(v.y);
+      ht[(size_t)(4 * q + 2) * ldt + m] = Mode::From(v.z);
+      ht[(size_t)(4 * q + 3) * ldt + m] = Mode::From(v.w);
+    }
+  }
+}
+
+// acc[rb] += A[rows rb*32 .. +31][0..K) . B[n][0..K)^T for the wavefront's 32 columns n: A in LDS
+// (row stride lda elements), B rows in global memory (row stride ldb), both k-contiguous.
+template <typename Mode, int RB>
+__device__ __forceinline__ void TileProduct(Acc16 (&acc)[RB], const typename Mode::Elem *a_lane,
+                                            int lda, const typename Mode::Elem *b_lane, int K) {
+  constexpr int kChunk = Mode::kChunk;
+  const int chunks = K / kChunk;
+  Frag fb = LoadFrag(b_lane);
+  for (int kc = 0; kc < chunks; ++kc) {
+    const int next = kc + 1 < chunks ? kc + 1 : kc;
+    const Frag fbn = LoadFrag(b_lane + (size_t)next * kChunk);
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      const Frag fa = LoadFrag(a_lane + (size_t)rb * 32 * lda + (size_t)kc * kChunk);
+      Mode::Mma(acc[rb], fa, fb);
+    }
+    fb = fbn;
+  }
+}
+
+// accumulator element r of a lane: row (r >> 2) * 8 + half * 4 + (r & 3) of the 32 x 32 block,
+// column lane & 31
+__device__ __forceinline__ int AccRow(int r, int half) { return (r >> 2) * 8 + half * 4 + (r & 3); }
+
+constexpr float kLowest = -3.0e38f;  // start of a running maximum (finite: -inf - -inf is NaN)
+
+// ---------------------------------------------------------------------------------- forward
+//
+// LDS: h [MT][D + pad]; row meta; the two picked logits per row; per wavefront (max, sum) per row.
+template <typename Mode, int RB>
+__global__ __launch_bounds__(kThreads) void JoinerForwardKernel(const JoinerArgs a) {
+  constexpr int MT = 32 * RB;
+  typedef typename Mode::Elem Elem;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int ldh = a.D + Mode::kPad;
+  Elem *h = reinterpret_cast<Elem *>(smem);
+  RowMeta *meta = reinterpret_cast<RowMeta *>(smem + (size_t)MT * ldh * sizeof(Elem));
+  float *zsym = reinterpret_cast<float *>(meta + MT);
+  float *zblank = zsym + MT;
+  float *part_m = zblank + MT;  // [4][MT]
+  float *part_s = part_m + 4 * MT;
+
+  const long long f0 = (long long)blockIdx.x * a.tpt;
+  const int rows = LoadMeta<MT>(a, f0, meta);
+  for (int m = threadIdx.x; m < MT; m += kThreads) { zsym[m] = 0.f; zblank[m] = 0.f; }
+  __syncthreads();
+  StageActivations<Mode, MT, false>(a, meta, rows, h, ldh, nullptr, 0);
+  __syncthreads();
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 31, half = lane >> 5;
+  const Elem *wk = static_cast<const Elem *>(a.wk);
+  const Elem *a_lane = h + (size_t)col * ldh + half * (Mode::kChunk / 2);
+  float run_m[RB][16], run_s[RB][16];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { run_m[rb][r] = kLowest; run_s[rb][r] = 0.f; }
+
+  for (int n0 = 0; n0 < a.Cpad; n0 += kNTile) {
+    const int n = n0 + wave * 32 + col;
+    Acc16 acc[RB];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[rb][r] = 0.f;
+    TileProduct<Mode, RB>(acc, a_lane, ldh, wk + (size_t)n * a.D + half * (Mode::kChunk / 2), a.D);
+    if (n < a.C) {
+      const float bn = a.bias != nullptr ? a.bias[n] : 0.f;
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = rb * 32 + AccRow(r, half);
+          const float z = acc[rb][r] + bn;
+          const float m = run_m[rb][r];
+          if (z > m) {
+            run_s[rb][r] = run_s[rb][r] * __expf(m - z) + 1.0f;
+            run_m[rb][r] = z;
+          } else {
+            run_s[rb][r] += __expf(z - m);
+          }
+          if (n == meta[row].sym) zsym[row] = z;
+          if (n == a.blank) zblank[row] = z;
+        }
+    }
+  }
+  // (max, sum) of a row: over the 32 lanes that hold its columns, then over the wavefronts
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      float m = run_m[rb][r], s = run_s[rb][r];
+#pragma unroll
+      for (int off = 16; off >= 1; off >>= 1) {
+        const float om = __shfl_xor(m, off, kWave), os = __shfl_xor(s, off, kWave);
+        const float mm = fmaxf(m, om);
+        s = s * __expf(m - mm) + os * __expf(om - mm);
+        m = mm;
+      }
+      if (col == 0) {
+        const int row = rb * 32 + AccRow(r, half);
+        part_m[wave * MT + row] = m;
+        part_s[wave * MT + row] = s;
+      }
+    }
+  __syncthreads();
+  for (int row = threadIdx.x; row < rows; row += kThreads) {
+    float m = part_m[row], s = part_s[row];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) {
+      const float om = part_m[w * MT + row], os = part_s[w * MT + row];
+      const float mm = fmaxf(m, om);
+      s = s * __expf(m - mm) + os * __expf(om - mm);
+      m = mm;
+    }
+    const float norm = m + logf(s);
+    const RowMeta rm = meta[row];
+    const int b = rm.bt / a.Tn, t = rm.bt - b * a.Tn;
+    a.norm[(size_t)f0 * a.R + row] = norm;
+    const int T1 = a.rnnt_type == K2AMD_REGULAR ? a.Tn + 1 : a.Tn;
+    const bool has_blank = a.blank >= 0 && a.blank < a.C;
+    a.py[((size_t)b * (a.S + 1) + rm.s) * a.Tn + t] = has_blank ? zblank[row] - norm : Real<float>::NegInf();
+    if (rm.s < a.S) {
+      float v = rm.sym >= 0 ? zsym[row] - norm : Real<float>::NegInf();
+      if (a.rnnt_type == K2AMD_REGULAR && a.boundary != nullptr && a.boundary[4 * b + 3] == t)
+        v = Real<float>::NegInf();
+      a.px[((size_t)b * a.S + rm.s) * T1 + t] = v;
+    }
+  }
+}
+
+// ------------------------------------------------------------ backward, gradients of am and lm
+//
+// One tile of 32 rows per workgroup: d logits [32][Cpad] into LDS, then d h = d logits . weight,
+// d pre = d h (1 - h^2); am_grad[frame] is the sum over the frame's R rows (plain stores: a frame
+// lies in one tile), lm_grad[b, s] collects its rows with atomic adds (runs of equal s along t are
+// added up first).
+template <typename Mode>
+__global__ __launch_bounds__(kThreads) void JoinerBackwardRowsKernel(const JoinerArgs a) {
+  constexpr int MT = 32;
+  typedef typename Mode::Elem Elem;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int ldh = a.D + Mode::kPad, ldc = a.Cpad + Mode::kPad;
+  constexpr int kLdStage = kNTile + 4;
+  Elem *h = reinterpret_cast<Elem *>(smem);
+  Elem *dz = h + (size_t)MT * ldh;
+  float *stage = reinterpret_cast<float *>(dz + (size_t)MT * ldc);
+  float4 *hdr = reinterpret_cast<float4 *>(stage + MT * kLdStage);
+  RowMeta *meta = reinterpret_cast<RowMeta *>(hdr + MT);
+
+  const long long f0 = (long long)blockIdx.x * a.tpt;
+  const int rows = LoadMeta<MT>(a, f0, meta);
+  for (int m = threadIdx.x; m < MT; m += kThreads)
+    hdr[m] = m < rows ? a.hdr[(size_t)f0 * a.R + m] : make_float4(0.f, 0.f, -1.f, 3.0e38f);  // padding: exp(. - norm) = 0
+  __syncthreads();
+  StageActivations<Mode, MT, false>(a, meta, rows, h, ldh, nullptr, 0);
+  __syncthreads();
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 31, half = lane >> 5;
+  const int koff = half * (Mode::kChunk / 2);
+  const Elem *wk = static_cast<const Elem *>(a.wk), *wc = static_cast<const Elem *>(a.wc);
+  for (int n0 = 0; n0 < a.Cpad; n0 += kNTile) {
+    const int n = n0 + wave * 32 + col;
+    Acc16 acc[1];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[0][r] = 0.f;
+    TileProduct<Mode, 1>(acc, h + (size_t)col * ldh + koff, ldh, wk + (size_t)n * a.D + koff, a.D);
+    const float bn = (n < a.C && a.bias != nullptr) ? a.bias[n] : 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = AccRow(r, half);
+      const float4 g = hdr[row];  // gx, gy, symbol, norm
+      float v = 0.f;
+      if (n < a.C) {
+        v = -__expf(acc[0][r] + bn - g.w) * (g.x + g.y);
+        if (n == (int)g.z) v += g.x;
+        if (n == a.blank) v += g.y;
+      }
+      dz[(size_t)row * ldc + n] = Mode::From(v);
+    }
+  }
+  __syncthreads();
+  const int part = threadIdx.x >> 7, c = threadIdx.x & 127;
+  const int nf = rows / a.R;
+  for (int d0 = 0; d0 < a.Dpad; d0 += kNTile) {
+    const int d = d0 + wave * 32 + col;
+    Acc16 acc[1];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[0][r] = 0.f;
+    TileProduct<Mode, 1>(acc, dz + (size_t)col * ldc + koff, ldc, wc + (size_t)d * a.Cpad + koff, a.Cpad);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = AccRow(r, half);
+      const float hv = d < a.D ? Mode::To(h[(size_t)row * ldh + d]) : 0.f;
+      stage[row * kLdStage + wave * 32 + col] = acc[0][r] * (1.0f - hv * hv);
+    }
+    __syncthreads();
+    if (d0 + c < a.D) {
+      for (int fl = part; fl < nf; fl += 2) {
+        float sum = 0.f;
+        for (int k = 0; k < a.R; ++k) sum += stage[(fl * a.R + k) * kLdStage + c];
+        a.am_grad[(size_t)(f0 + fl) * a.D + d0 + c] = sum;
+      }
+      for (int k = part; k < a.R; k += 2) {
+        int key = -1;
+        float sum = 0.f;
+        for (int fl = 0; fl < nf; ++fl) {
+          const int row = fl * a.R + k;
+          const int lmrow = meta[row].lmrow;
+          if (lmrow != key) {
+            if (key >= 0) atomicAdd(a.lm_grad + (size_t)key * a.D + d0 + c, sum);
+            key = lmrow;
+            sum = 0.f;
+          }
+          sum += stage[row * kLdStage + c];
+        }
+        if (key >= 0) atomicAdd(a.lm_grad + (size_t)key * a.D + d0 + c, sum);
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// ------------------------------------------------------- backward, gradients of weight and bias
+//
+// A workgroup owns 64 columns c of d logits and every kGroups-th share of the tiles of 64 rows; it
+// keeps its [64][D] block of the weight's gradient in accumulators over all of its tiles:
+//   logits slice = h . weight[c-slice]^T     (k = D)
+//   d logits slice -> LDS, transposed [c][row]
+//   weight_grad[c][d] += sum over rows of d logits[row][c] h[row][d]   (k = rows of the tile)
+// and adds it to weight_grad (zeroed by the launcher) with atomic adds at the end.
+template <typename Mode>
+__global__ __launch_bounds__(kThreads) void JoinerBackwardWeightKernel(const JoinerArgs a, int tiles,
+                                                                        int groups) {
+  constexpr int MT = 64;
+  constexpr bool kBf = sizeof(typename Mode::Elem) == 2;
+  typedef typename Mode::Elem Elem;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int ldh = a.D + Mode::kPad;
+  constexpr int ldz = MT + Mode::kPad;  // d logits, transposed: [c][row]
+  constexpr int ldt = MT + Mode::kPad;  // h, transposed: [d][row] (bfloat16 only)
+  Elem *h = reinterpret_cast<Elem *>(smem);
+  Elem *dzt = h + (size_t)MT * ldh;
+  Elem *ht = dzt + (size_t)kSliceCols * ldz;
+  float4 *hdr = reinterpret_cast<float4 *>(ht + (kBf ? (size_t)a.D * ldt : 0));
+  RowMeta *meta = reinterpret_cast<RowMeta *>(hdr + MT);
+
+  const int slice = blockIdx.x / groups, group = blockIdx.x - slice * groups;
+  const int c0 = slice * kSliceCols;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 31, half = lane >> 5;
+  const int koff = half * (Mode::kChunk / 2);
+  const int rb = wave >> 1, cb = wave & 1;  // block of the logits slice this wavefront multiplies
+  const int n = c0 + cb * 32 + col;         // its column of logits (< Cpad: slices tile Cpad)
+  const Elem *wk = static_cast<const Elem *>(a.wk);
+  // its blocks of the gradient: columns c0 + cb*32 .. +31, d blocks dhalf * ndb .. + ndb - 1
+  const int ndb = a.D / 64, dhalf = wave >> 1;
+  Acc16 wacc[kMaxDBlocks];
+#pragma unroll
+  for (int i = 0; i < kMaxDBlocks; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) wacc[i][r] = 0.f;
+  float bsum = 0.f;
+  const float bn = (n < a.C && a.bias != nullptr) ? a.bias[n] : 0.f;
+
+  for (int tile = group; tile < tiles; tile += groups) {
+    const long long f0 = (long long)tile * a.tpt;
+    const int rows = LoadMeta<MT>(a, f0, meta);
+    for (int m = threadIdx.x; m < MT; m += kThreads)
+      hdr[m] = m < rows ? a.hdr[(size_t)f0 * a.R + m] : make_float4(0.f, 0.f, -1.f, 3.0e38f);  // padding: exp(. - norm) = 0
+    __syncthreads();
+    StageActivations<Mode, MT, kBf>(a, meta, rows, h, ldh, ht, ldt);
+    __syncthreads();
+    Acc16 acc[1];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[0][r] = 0.f;
+    TileProduct<Mode, 1>(acc, h + (size_t)(rb * 32 + col) * ldh + koff, ldh,
+                         wk + (size_t)n * a.D + koff, a.D);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = rb * 32 + AccRow(r, half);
+      const float4 g = hdr[row];
+      float v = 0.f;
+      if (n < a.C) {
+        v = -__expf(acc[0][r] + bn - g.w) * (g.x + g.y);
+        if (n == (int)g.z) v += g.x;
+        if (n == a.blank) v += g.y;
+      }
+      dzt[(size_t)(cb * 32 + col) * ldz + row] = Mode::From(v);
+    }
+    __syncthreads();
+    if (threadIdx.x < kSliceCols) {
+      float s = 0.f;
+      for (int m = 0; m < MT; ++m) s += Mode::To(dzt[(size_t)threadIdx.x * ldz + m]);
+      bsum += s;
+    }
+#pragma unroll
+    for (int kc = 0; kc < MT / Mode::kChunk; ++kc) {
+      const Frag fa = LoadFrag(dzt + (size_t)(cb * 32 + col) * ldz + kc * Mode::kChunk + koff);
+#pragma unroll
+      for (int i = 0; i < kMaxDBlocks; ++i) {
+        if (i < ndb) {
+          const int d = (dhalf * ndb + i) * 32 + col;
+          Frag fb;
+          if (kBf) {
+            fb = LoadFrag(ht + (size_t)d * ldt + kc * Mode::kChunk + koff);
+          } else {
+            const float *hf = reinterpret_cast<const float *>(h);
+            unsigned u[16];
+#pragma unroll
+            for (int j = 0; j < 16; ++j)
+              u[j] = AsBits(hf[(size_t)(kc * 32 + half * 16 + j) * ldh + d]);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) fb.q[q] = make_uint4(u[4 * q], u[4 * q + 1], u[4 * q + 2], u[4 * q + 3]);
+          }
+          Mode::Mma(wacc[i], fa, fb);
+        }
+      }
+    }
+    __syncthreads();  // the next tile's staging overwrites h, dzt, hdr
+  }
+#pragma unroll
+  for (int i = 0; i < kMaxDBlocks; ++i) {
+    if (i < ndb) {
+      const int d = (dhalf * ndb + i) * 32 + col;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int c = c0 + cb * 32 + AccRow(r, half);
+        if (c < a.C) atomicAdd(a.weight_grad + (size_t)c * a.D + d, wacc[i][r]);
+      }
+    }
+  }
+  if (threadIdx.x < kSliceCols && c0 + (int)threadIdx.x < a.C && a.bias_grad != nullptr)
+    atomicAdd(a.bias_grad + c0 + threadIdx.x, bsum);
+}
+
+// ---------------------------------------------------------------------------- small kernels
+
+// The weight [C][D] in the operand type: wk [Cpad][D] and wc [Dpad][Cpad], zeros in the padding.
+template <typename Mode>
+__global__ void JoinerPrepWeightKernel(const float *__restrict__ weight, typename Mode::Elem *wk,
+                                       typename Mode::Elem *wc, int C, int D, int Cpad, int Dpad) {
+  const size_t nk = (size_t)Cpad * D, nc = (size_t)Dpad * Cpad;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nk + nc;
+       i += (size_t)gridDim.x * blockDim.x) {
+    if (i < nk) {
+      const int c = (int)(i / D), d = (int)(i - (size_t)c * D);
+      wk[i] = Mode::From(c < C ? weight[(size_t)c * D + d] : 0.f);
+    } else if (wc != nullptr) {
+      const size_t j = i - nk;
+      const int d = (int)(j / Cpad), c = (int)(j - (size_t)d * Cpad);
+      wc[j] = Mode::From(c < C && d < D ? weight[(size_t)c * D + d] : 0.f);
+    }
+  }
+}
+
+__global__ void JoinerFillKernel(float *a, size_t na, float va, float *b, size_t nb, float vb) {
+  const size_t first = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = first; i < na; i += stride) a[i] = va;
+  for (size_t i = first; i < nb; i += stride) b[i] = vb;
+}
+
+// px[b,s,t] += py[b,s+1,t] (k2/python/k2/rnnt_loss.py:1345-1346); T1 == Tn here.
+__global__ void JoinerConstrainedKernel(float *__restrict__ px, const float *__restrict__ py, int B,
+                                        int S, int Tn) {
+  const size_t n = (size_t)B * S * Tn;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (size_t)gridDim.x * blockDim.x) {
+    const size_t b = i / ((size_t)S * Tn), rem = i - b * (size_t)S * Tn;
+    px[i] += py[b * (size_t)(S + 1) * Tn + Tn + rem];
+  }
+}
+
+// Per row {gx, gy, symbol, norm}: the gradients that reach the row's px and py values, times what
+// reaches the sequence's score (one thread per row pays the look-up chain for 64 rows at a time).
+__global__ void JoinerRowHeaderKernel(const JoinerArgs a, const float *__restrict__ px_grad,
+                                      const float *__restrict__ py_grad,
+                                      const float *__restrict__ seq_scale, float4 *__restrict__ hdr) {
+  const long long rows = a.frames * a.R;
+  const long long row = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (row >= rows) return;
+  const long long frame = row / a.R;
+  const int k = (int)(row - frame * a.R);
+  const RowMeta rm = MetaOf(a, frame, k);
+  const int b = rm.bt / a.Tn, t = rm.bt - b * a.Tn;
+  const int T1 = a.rnnt_type == K2AMD_REGULAR ? a.Tn + 1 : a.Tn;
+  const float scale = seq_scale != nullptr ? seq_scale[b] : 1.0f;
+  float gx = 0.f;
+  int sym = rm.sym;
+  if (rm.s < a.S && sym >= 0) {
+    const bool cut = a.rnnt_type == K2AMD_REGULAR && a.boundary != nullptr && a.boundary[4 * b + 3] == t;
+    if (!cut) gx = MulRounded(px_grad[((size_t)b * a.S + rm.s) * T1 + t], scale);
+  } else {
+    sym = -1;
+  }
+  float gy = MulRounded(py_grad[((size_t)b * (a.S + 1) + rm.s) * a.Tn + t], scale);
+  if (a.rnnt_type == K2AMD_CONSTRAINED && rm.s >= 1)
+    gy += MulRounded(px_grad[((size_t)b * a.S + (rm.s - 1)) * T1 + t], scale);  // px += py[:, 1:]
+  hdr[row] = make_float4(gx, gy, (float)sym, a.norm[row]);
+}
+
+// ------------------------------------------------------------------------------- launchers
+
+int RoundUp(int v, int m) { return (v + m - 1) / m * m; }
+size_t ElemBytes(int precision) { return precision == K2AMD_JOINER_BF16 ? 2 : 4; }
+
+bool JoinerShapeOk(int B, int S, int T, int R, int C, int D) {
+  if (B < 0 || S < 0 || T < 0 || R < 1 || C < 1) return false;
+  if (D < 64 || D > kMaxD || D % 64 != 0 || R > 32 || R > S + 1 || C > (1 << 20)) return false;
+  const long long rows = (long long)B * T * R;
+  return rows * 4 < (1ll << 31) && (long long)B * (S + 1) * (T + 1) < (1ll << 31) &&
+         (long long)B * (S + 1) * D < (1ll << 31) && (long long)B * T * D < (1ll << 31);
+}
+
+struct WorkspaceLayout {
+  size_t wk, wc, hdr, total;
+};
+WorkspaceLayout LayoutOf(int B, int T, int R, int C, int D, int precision) {
+  const size_t e = ElemBytes(precision);
+  const size_t Cpad = RoundUp(C, kNTile), Dpad = RoundUp(D, kNTile);
+  WorkspaceLayout w;
+  w.wk = 0;
+  w.wc = (Cpad * D * e + 255) / 256 * 256;
+  w.hdr = w.wc + (Dpad * Cpad * e + 255) / 256 * 256;
+  w.total = w.hdr + (size_t)B * T * R * sizeof(float4);
+  return w;
+}
+
+template <typename K>
+int AllowLds(K kernel, size_t bytes) {
+  if (bytes > 160 * 1024) return K2AMD_ERR_UNSUPPORTED;
+  return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) == hipSuccess
+             ? K2AMD_OK
+             : K2AMD_ERR_LAUNCH;
+}
+
+JoinerArgs MakeArgs(const float *am, const float *lm, const int64_t *ranges, const float *bias,
+                    const int64_t *symbols, const int64_t *boundary, int B, int S, int T, int R,
+                    int C, int D, int blank, int rnnt_type, int rows_per_tile, void *workspace,
+                    int precision) {
+  JoinerArgs a{};
+  a.am = am; a.lm = lm; a.bias = bias; a.ranges = ranges; a.symbols = symbols; a.boundary = boundary;
+  a.B = B; a.S = S; a.Tn = T; a.R = R; a.C = C; a.D = D; a.blank = blank; a.rnnt_type = rnnt_type;
+  a.Cpad = RoundUp(C, kNTile); a.Dpad = RoundUp(D, kNTile);
+  a.tpt = rows_per_tile / R;
+  a.frames = (long long)B * T;
+  const WorkspaceLayout w = LayoutOf(B, T, R, C, D, precision);
+  unsigned char *ws = static_cast<unsigned char *>(workspace);
+  a.wk = ws + w.wk;
+  a.wc = ws + w.wc;
+  a.hdr = reinterpret_cast<const float4 *>(ws + w.hdr);
+  return a;
+}
+
+template <typename Mode>
+int PrepWeights(const float *weight, const JoinerArgs &a, bool both, hipStream_t st) {
+  typedef typename Mode::Elem Elem;
+  hipLaunchKernelGGL(JoinerPrepWeightKernel<Mode>, dim3(512), dim3(256), 0, st, weight,
+                     static_cast<Elem *>(const_cast<void *>(a.wk)),
+                     both ? static_cast<Elem *>(const_cast<void *>(a.wc)) : nullptr, a.C, a.D, a.Cpad, a.Dpad);
+  return LaunchStatus();
+}
+
+template <typename Mode, int RB>
+int ForwardImpl(const float *weight, JoinerArgs a, hipStream_t st) {
+  constexpr int MT = 32 * RB;
+  int rc = PrepWeights<Mode>(weight, a, false, st);
+  if (rc != K2AMD_OK) return rc;
+  const size_t npx = (size_t)a.B * a.S * (a.rnnt_type == K2AMD_REGULAR ? a.Tn + 1 : a.Tn);
+  const size_t npy = (size_t)a.B * (a.S + 1) * a.Tn;
+  hipLaunchKernelGGL(JoinerFillKernel, dim3(512), dim3(256), 0, st, a.px, npx, Real<float>::NegInf(),
+                     a.py, npy, Real<float>::NegInf());
+  const size_t lds = (size_t)MT * (a.D + Mode::kPad) * sizeof(typename Mode::Elem) +
+                     MT * (sizeof(RowMeta) + 10 * sizeof(float));
+  rc = AllowLds(JoinerForwardKernel<Mode, RB>, lds);
+  if (rc != K2AMD_OK) return rc;
+  const long long tiles = (a.frames + a.tpt - 1) / a.tpt;
+  if (tiles > 0)
+    hipLaunchKernelGGL((JoinerForwardKernel<Mode, RB>), dim3((unsigned)tiles), dim3(kThreads), lds, st, a);
+  if (a.rnnt_type == K2AMD_CONSTRAINED && a.S > 0 && a.frames > 0)
+    hipLaunchKernelGGL(JoinerConstrainedKernel, dim3(512), dim3(256), 0, st, a.px, a.py, a.B, a.S, a.Tn);
+  return LaunchStatus();
+}
+
+template <typename Mode>
+int BackwardImpl(const float *weight, JoinerArgs a, const float *px_grad, const float *py_grad,
+                 const float *seq_scale, hipStream_t st) {
+  typedef typename Mode::Elem Elem;
+  constexpr bool kBf = sizeof(Elem) == 2;
+  int rc = PrepWeights<Mode>(weight, a, true, st);
+  if (rc != K2AMD_OK) return rc;
+  const long long rows = a.frames * a.R;
+  hipLaunchKernelGGL(JoinerFillKernel, dim3(512), dim3(256), 0, st, a.lm_grad,
+                     (size_t)a.B * (a.S + 1) * a.D, 0.f, a.weight_grad, (size_t)a.C * a.D, 0.f);
+  if (a.bias_grad != nullptr)
+    hipLaunchKernelGGL(JoinerFillKernel, dim3(4), dim3(256), 0, st, a.bias_grad, (size_t)a.C, 0.f,
+                       static_cast<float *>(nullptr), (size_t)0, 0.f);
+  if (rows == 0) return LaunchStatus();
+  hipLaunchKernelGGL(JoinerRowHeaderKernel, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, st, a,
+                     px_grad, py_grad, seq_scale, const_cast<float4 *>(a.hdr));
+  {  // gradients of am and lm: tiles of 32 rows
+    JoinerArgs r = a;
+    r.tpt = 32 / a.R;
+    const size_t lds = (size_t)32 * (a.D + Mode::kPad + a.Cpad + Mode::kPad) * sizeof(Elem) +
+                       32 * ((kNTile + 4) * sizeof(float) + sizeof(float4) + sizeof(RowMeta));
+    rc = AllowLds(JoinerBackwardRowsKernel<Mode>, lds);
+    if (rc != K2AMD_OK) return rc;
+    const long long tiles = (a.frames + r.tpt - 1) / r.tpt;
+    hipLaunchKernelGGL(JoinerBackwardRowsKernel<Mode>, dim3((unsigned)tiles), dim3(kThreads), lds, st, r);
+  }
+  {  // gradients of weight and bias: slices of 64 columns x groups of tiles of 64 rows
+    JoinerArgs w = a;
+    w.tpt = 64 / a.R;
+    const size_t lds = (size_t)64 * (a.D + Mode::kPad) * sizeof(Elem) +
+                       (size_t)kSliceCols * (64 + Mode::kPad) * sizeof(Elem) +
+                       (kBf ? (size_t)a.D * (64 + Mode::kPad) * sizeof(Elem) : 0) +
+                       64 * (sizeof(float4) + sizeof(RowMeta));
+    rc = AllowLds(JoinerBackwardWeightKernel<Mode>, lds);
+    if (rc != K2AMD_OK) return rc;
+    const long long tiles = (a.frames + w.tpt - 1) / w.tpt;
+    const int slices = a.Cpad / kSliceCols;
+    int groups = 512 / slices;
+    if (groups < 1) groups = 1;
+    if (groups > tiles) groups = (int)tiles;
+    hipLaunchKernelGGL(JoinerBackwardWeightKernel<Mode>, dim3((unsigned)(slices * groups)),
+                       dim3(kThreads), lds, st, w, (int)tiles, groups);
+  }
+  return LaunchStatus();
+}
+
+}  // namespace
+}  // namespace k2amd
+
+using namespace k2amd;
+
+extern "C" {
+
+size_t k2amd_rnnt_joiner_pruned_workspace_bytes(int B, int S, int T, int R, int C, int D,
+                                                int precision) {
+  if (!JoinerShapeOk(B, S, T, R, C, D)) return 0;
+  if (precision != K2AMD_JOINER_F32 && precision != K2AMD_JOINER_BF16) return 0;
+  return LayoutOf(B, T, R, C, D, precision).total;
+}
+
+int k2amd_rnnt_joiner_pruned_forward(const void *am, const void *lm, const int64_t *ranges,
+                                     const void *weight, const void *bias, const int64_t *symbols,
+                                     const int64_t *boundary, void *px, void *py, void *normalizers,
+                                     int B, int S, int T, int R, int C, int D, int termination_symbol,
+                                     int rnnt_type, int precision, void *workspace,
+                                     size_t workspace_bytes, void *stream) {
+  if (!JoinerShapeOk(B, S, T, R, C, D)) return K2AMD_ERR_UNSUPPORTED;
+  if (precision != K2AMD_JOINER_F32 && precision != K2AMD_JOINER_BF16) return K2AMD_ERR_INVALID_ARGUMENT;
+  if (rnnt_type != K2AMD_REGULAR && rnnt_type != K2AMD_MODIFIED && rnnt_type != K2AMD_CONSTRAINED)
+    return K2AMD_ERR_INVALID_ARGUMENT;
+  if (rnnt_type != K2AMD_REGULAR && T < S) return K2AMD_ERR_INVALID_ARGUMENT;
+  if (B == 0 || T == 0) return K2AMD_OK;
+  if (!am || !lm || !ranges || !weight || !px || !py || !normalizers || (!symbols && S > 0))
+    return K2AMD_ERR_INVALID_ARGUMENT;
+  if (workspace == nullptr ||
+      workspace_bytes < k2amd_rnnt_joiner_pruned_workspace_bytes(B, S, T, R, C, D, precision))
+    return K2AMD_ERR_WORKSPACE;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool bf = precision == K2AMD_JOINER_BF16;
+  JoinerArgs a = MakeArgs((const float *)am, (const float *)lm, ranges, (const float *)bias, symbols,
+                          boundary, B, S, T, R, C, D, termination_symbol, rnnt_type, bf ? 128 : 64,
+                          workspace, precision);
+  a.px = (float *)px; a.py = (float *)py; a.norm = (float *)normalizers;
+  return bf ? ForwardImpl<Bf16, 4>((const float *)weight, a, st)
+            : ForwardImpl<F32, 2>((const float *)weight, a, st);
+}
+
+int k2amd_rnnt_joiner_pruned_backward(const void *am, const void *lm, const int64_t *ranges,
+                                      const void *weight, const void *bias, const int64_t *symbols,
+                                      const int64_t *boundary, const void *normalizers,
+                                      const void *px_grad, const void *py_grad, const void *seq_scale,
+                                      void *am_grad, void *lm_grad, void *weight_grad, void *bias_grad,
+                                      int B, int S, int T, int R, int C, int D, int termination_symbol,
+                                      int rnnt_type, int precision, void *workspace,
+                                      size_t workspace_bytes, void *stream) {
+  if (!JoinerShapeOk(B, S, T, R, C, D)) return K2AMD_ERR_UNSUPPORTED;
+  if (precision != K2AMD_JOINER_F32 && precision != K2AMD_JOINER_BF16) return K2AMD_ERR_INVALID_ARGUMENT;
+  if (rnnt_type != K2AMD_REGULAR && rnnt_type != K2AMD_MODIFIED && rnnt_type != K2AMD_CONSTRAINED)
+    return K2AMD_ERR_INVALID_ARGUMENT;
+  if (!weight_grad || (!lm_grad && B > 0)) return K2AMD_ERR_INVALID_ARGUMENT;
+  if (B > 0 && T > 0 &&
+      (!am || !lm || !ranges || !weight || !normalizers || !px_grad || !py_grad || !am_grad ||
+       (!symbols && S > 0)))
+    return K2AMD_ERR_INVALID_ARGUMENT;
+  if (workspace == nullptr ||
+      workspace_bytes < k2amd_rnnt_joiner_pruned_workspace_bytes(B, S, T, R, C, D, precision))
+    return K2AMD_ERR_WORKSPACE;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool bf = precision == K2AMD_JOINER_BF16;
+  JoinerArgs a = MakeArgs((const float *)am, (const float *)lm, ranges, (const float *)bias, symbols,
+                          boundary, B, S, T, R, C, D, termination_symbol, rnnt_type, 32, workspace,
+                          precision);
+  a.norm = (float *)const_cast<void *>(normalizers);
+  a.am_grad = (float *)am_grad; a.lm_grad = (float *)lm_grad;
+  a.weight_grad = (float *)weight_grad; a.bias_grad = (float *)bias_grad;
+  return bf ? BackwardImpl<Bf16>((const float *)weight, a, (const float *)px_grad,
+                                 (const float *)py_grad, (const float *)seq_scale, st)
+            : BackwardImpl<F32>((const float *)weight, a, (const float *)px_grad,
+                                (const float *)py_grad, (const float *)seq_scale, st);
+}
+
+}  // extern "C"

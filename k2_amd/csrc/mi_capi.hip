@@ -18,7 +18,7 @@ bool ShapeOk(int B, int S, int T) {
 
 // Switches for tests and comparisons, read at every call: K2AMD_MI_PATH=generic forces the exact
 // log-domain kernels; K2AMD_MI_PATH=two-launches keeps the pipelined kernels but never serves the
-// single launch.
+// single launch; K2AMD_MI_PATH=single-launch advises the single launch wherever it is served.
 bool PathIs(const char *name) {
   const char *e = std::getenv("K2AMD_MI_PATH");
   return e != nullptr && std::strcmp(e, name) == 0;
@@ -188,6 +188,12 @@ int k2amd_mi_forward_backward_supported(int B, int S, int T, int modified, int d
                                         int has_workspace) {
   return dtype == K2AMD_F32 && has_workspace && ShapeOk(B, S, T) && B > 0 && !ForceGeneric() &&
          !PathIs("two-launches") && MiFusedSupports(B, S, T, modified ? 1 : 0);
+}
+
+int k2amd_mi_forward_backward_advised(int B, int S, int T, int modified, int dtype,
+                                      int has_workspace) {
+  return k2amd_mi_forward_backward_supported(B, S, T, modified, dtype, has_workspace) &&
+         (MiFusedAdvised(B, S) || PathIs("single-launch"));
 }
 
 size_t k2amd_mi_forward_backward_scratch_bytes(int B, int S, int T, int modified, int dtype) {

@@ -1763,6 +1763,17 @@ bool MiFusedSupports(int B, int S, int Tn, int modified) {
   return MiFastSupports(B, S, Tn, modified) && B >= 1 && S + 2 <= kCutRows;
 }
 
+// Whether the single launch is the faster way to run both recursions of this shape on the current
+// device: it is while every forward half-sweep finds a compute unit at once (the launch then lasts
+// as long as one sequence's two half-length fronts).  With more half-sweeps than units they queue,
+// one workgroup to a unit, and the two launches, which place two workgroups on a unit, take less
+// time (B = 128 at S = 200, T = 1000: 181 us against 201).
+bool MiFusedAdvised(int B, int S) {
+  const int units = ComputeUnits();
+  const long long nchunks = (S + 1 + kRows - 1) / kRows;
+  return units > 0 && 2ll * B * nchunks <= units;
+}
+
 // Floats of scratch per call of the single launch: one slab of (S + 1) rows of Tn + 2 per sequence
 // (the log-derivatives of both halves, the mirrored half's one column to the right).
 size_t MiFusedScratchElems(int B, int S, int Tn) { return (size_t)B * (S + 1) * ((size_t)Tn + 2); }

@@ -36,6 +36,8 @@ int MiBackwardFast(const float *px, const float *p, const float *log_deriv,
 // Forward and backward in one launch; scratch holds MiFusedScratchElems floats (written, then
 // read, by the launch itself).  MiFusedSupports: whether that kernel serves the shape.
 bool MiFusedSupports(int B, int S, int Tn, int modified);
+// Whether it is also the faster way on the current device (else: the two launches).
+bool MiFusedAdvised(int B, int S);
 size_t MiFusedScratchElems(int B, int S, int Tn);
 int MiForwardBackwardFast(const float *px, const float *py, const int64_t *boundary, float *ans,
                           float *scratch, float *ans_grad, float *px_grad, float *py_grad, int B,

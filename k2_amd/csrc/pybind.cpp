@@ -230,6 +230,17 @@ bool MutualInformationForwardBackwardSupported(torch::Tensor px, torch::Tensor p
                                              k2amd_mi_workspace_bytes(B, S, T, modified, dt) > 0) != 0;
 }
 
+bool MutualInformationForwardBackwardAdvised(torch::Tensor px, torch::Tensor py) {
+  TORCH_CHECK(px.dim() == 3 && py.dim() == 3, "px and py must have three dimensions");
+  if (!px.is_cuda()) return false;
+  const int B = static_cast<int>(px.size(0)), S = static_cast<int>(px.size(1)),
+            T = static_cast<int>(py.size(2)), modified = px.size(2) == T ? 1 : 0;
+  const int dt = DtypeCode(px);
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(px.device());  // the answer depends on the device
+  return k2amd_mi_forward_backward_advised(B, S, T, modified, dt,
+                                           k2amd_mi_workspace_bytes(B, S, T, modified, dt) > 0) != 0;
+}
+
 // The two calls above in one launch (k2amd_mi_forward_backward): returns {ans, px_grad, py_grad}
 // and overwrites ans_grad like MutualInformationBackward.
 std::vector<torch::Tensor> MutualInformationForwardBackward(torch::Tensor px, torch::Tensor py,
@@ -644,6 +655,8 @@ PYBIND11_MODULE(_k2_amd, m) {
         pybind11::arg("py"), pybind11::arg("boundary"), pybind11::arg("p"),
         pybind11::arg("ans_grad"), pybind11::arg("log_deriv") = pybind11::none());
   m.def("mutual_information_forward_backward_supported", &MutualInformationForwardBackwardSupported,
+        pybind11::arg("px"), pybind11::arg("py"));
+  m.def("mutual_information_forward_backward_advised", &MutualInformationForwardBackwardAdvised,
         pybind11::arg("px"), pybind11::arg("py"));
   m.def("mutual_information_forward_backward", &MutualInformationForwardBackward,
         pybind11::arg("px"), pybind11::arg("py"), pybind11::arg("boundary"),

@@ -45,12 +45,12 @@ _single_launch_ok = {}
 
 
 def _single_launch(px: Tensor, py: Tensor) -> bool:
-    """Whether both recursions of these inputs run in one launch (asked of the native layer once
-    per shape, dtype and device)."""
+    """Whether both recursions of these inputs run in one launch: where the native layer serves it
+    and says it is the faster way on the device (asked once per shape, dtype and device)."""
     key = (px.shape, py.shape[-1], px.dtype, px.device)
     ok = _single_launch_ok.get(key)
     if ok is None:
-        ok = _single_launch_ok[key] = bool(native.mutual_information_forward_backward_supported(px, py))
+        ok = _single_launch_ok[key] = bool(native.mutual_information_forward_backward_advised(px, py))
     return ok
 
 

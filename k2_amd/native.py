@@ -81,9 +81,18 @@ def mutual_information_backward(px: torch.Tensor, py: torch.Tensor,
     return [gx, gy]
 
 
+def mutual_information_forward_backward_advised(px: torch.Tensor, py: torch.Tensor) -> bool:
+    """True if mutual_information_forward_backward serves these inputs and is the faster way on
+    their device (a compute unit for every half-sweep of the launch at once)."""
+    _require_device(px)
+    if _ext is not None:
+        return _ext.mutual_information_forward_backward_advised(px, py)
+    return capi.mi_forward_backward_advised(px, py)
+
+
 def mutual_information_forward_backward_supported(px: torch.Tensor, py: torch.Tensor) -> bool:
     """True if mutual_information_forward_backward serves these inputs on their device (fp32, the
-    pipelined kernels, and a compute unit for every workgroup of the launch)."""
+    pipelined kernels' shapes)."""
     _require_device(px)
     if _ext is not None:
         return _ext.mutual_information_forward_backward_supported(px, py)
@@ -166,6 +175,19 @@ def logprobs_pruned_backward(logits, norm, px_grad, py_grad, symbols, ranges, bo
                                              boundary, termination_symbol, rnnt_type, hat, seq_scale)
     return capi.logprobs_pruned_backward(logits, norm, px_grad, py_grad, symbols, ranges, boundary,
                                          termination_symbol, rnnt_type, hat, seq_scale)
+
+
+def joiner_pruned_forward(am, lm, ranges, weight, bias, symbols, termination_symbol, boundary,
+                          rnnt_type, precision):
+    _require_device(am)
+    return capi.joiner_pruned_forward(am, lm, ranges, weight, bias, symbols, termination_symbol,
+                                      boundary, rnnt_type, precision)
+
+
+def joiner_pruned_backward(am, lm, ranges, weight, bias, symbols, termination_symbol, boundary,
+                           rnnt_type, norm, px_grad, py_grad, seq_scale, precision):
+    return capi.joiner_pruned_backward(am, lm, ranges, weight, bias, symbols, termination_symbol,
+                                       boundary, rnnt_type, norm, px_grad, py_grad, seq_scale, precision)
 
 
 def prune_ranges(px_grad, py_grad, boundary, s_range):

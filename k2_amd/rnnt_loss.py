@@ -121,7 +121,8 @@ class _Scores(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, kind, rnnt_type, delay_penalty, return_grad, *args):
-        boundary = args[5] if kind != "joint" else args[4]
+        boundary = {"joint": 4, "joiner": 8}.get(kind, 5)
+        boundary = args[boundary]
         need = return_grad or any(ctx.needs_input_grad)
         # no zero tensors for the gradients of px_grad / py_grad, which nothing differentiates
         ctx.set_materialize_grads(False)
@@ -135,6 +136,13 @@ class _Scores(torch.autograd.Function):
             px, py, norm = native.logprobs_joint_forward(logits, symbols, termination_symbol,
                                                          rnnt_code, boundary)
             saved = (logits, norm)
+        elif kind == "joiner":
+            am, lm, ranges, weight, bias, symbols, termination_symbol, rnnt_code, _, precision = args
+            am, lm, weight = am.contiguous(), lm.contiguous(), weight.contiguous()
+            bias = bias.contiguous() if bias is not None else None
+            px, py, norm = native.joiner_pruned_forward(am, lm, ranges, weight, bias, symbols,
+                                                        termination_symbol, boundary, rnnt_code, precision)
+            saved = (am, lm, weight, norm) + ((bias,) if bias is not None else ())
         else:
             logits, symbols, ranges, termination_symbol, rnnt_code, _, hat = args
             logits = logits.contiguous()
@@ -166,6 +174,13 @@ class _Scores(torch.autograd.Function):
             _, symbols, termination_symbol, rnnt_code, boundary = args
             grads = (native.logprobs_joint_backward(saved[0], saved[1], px_grad, py_grad, symbols,
                                                     boundary, termination_symbol, rnnt_code, scale),)
+        elif ctx.kind == "joiner":
+            _, _, ranges, _, bias, symbols, termination_symbol, rnnt_code, boundary, precision = args
+            am, lm, weight, norm = saved[:4]
+            d_am, d_lm, d_w, d_b = native.joiner_pruned_backward(
+                am, lm, ranges, weight, saved[4] if bias is not None else None, symbols,
+                termination_symbol, boundary, rnnt_code, norm, px_grad, py_grad, scale, precision)
+            grads = (d_am, d_lm, None, d_w, d_b)
         else:
             _, symbols, ranges, termination_symbol, rnnt_code, boundary, hat = args
             grads = (native.logprobs_pruned_backward(saved[0], saved[1], px_grad, py_grad, symbols,
@@ -461,6 +476,47 @@ def rnnt_loss_pruned(
     checked = _hat_args if use_hat_loss else _pruned_args
     args = checked(logits, symbols, ranges, termination_symbol, boundary, rnnt_type)
     negated_loss = _Scores.apply("pruned", rnnt_type, float(delay_penalty), False, *args)[0]
+    return _reduce(negated_loss, reduction)
+
+
+def rnnt_loss_pruned_joiner(
+    am: Tensor,
+    lm: Tensor,
+    ranges: Tensor,
+    weight: Tensor,
+    bias: Optional[Tensor],
+    symbols: Tensor,
+    termination_symbol: int,
+    boundary: Tensor = None,
+    rnnt_type: str = "regular",
+    delay_penalty: float = 0.0,
+    reduction: Optional[str] = "mean",
+    precision: str = "fp32",
+) -> Tensor:
+    """do_rnnt_pruning -> joiner -> rnnt_loss_pruned (k2/python/k2/rnnt_loss.py:913-954, the
+    caller's joiner, :1351-1468) as one call for the usual joiner,
+
+        logits = torch.nn.functional.linear(torch.tanh(am_pruned + lm_pruned), weight, bias),
+
+    with am [B][T][D] and lm [B][S+1][D] the projected encoder / decoder outputs, ranges from
+    get_rnnt_prune_ranges, weight [C][D] and bias [C] (or None) those of the output layer.  The
+    [B][T][s_range][C] logits are never stored; gradients flow to am, lm, weight and bias.
+    ``precision``: "fp32" multiplies in fp32; "bf16" rounds the activations, the weight and the logits'
+    gradients to bfloat16 for the matrix products (fp32 accumulation), as autocast would."""
+    assert am.ndim == 3 and lm.ndim == 3, (am.shape, lm.shape)
+    (B, T, D) = am.shape
+    assert lm.shape[0] == B and lm.shape[2] == D, (am.shape, lm.shape)
+    S = lm.shape[1] - 1
+    assert ranges.ndim == 3 and ranges.shape[:2] == (B, T), (ranges.shape, B, T)
+    assert weight.ndim == 2 and weight.shape[1] == D, (weight.shape, D)
+    assert bias is None or bias.shape == (weight.shape[0],), (bias.shape, weight.shape)
+    assert symbols.shape == (B, S), (symbols.shape, B, S)
+    assert rnnt_type in _RNNT_TYPES, rnnt_type
+    assert precision in capi.JOINER_PRECISIONS, precision
+    _validate_st_lengths(S, T, rnnt_type == "regular", boundary)
+    args = (am, lm, _dev_i64(ranges, am), weight, bias, _dev_i64(symbols, am), int(termination_symbol),
+            capi.RNNT_TYPES[rnnt_type], _dev_i64(boundary, am), capi.JOINER_PRECISIONS[precision])
+    negated_loss = _Scores.apply("joiner", rnnt_type, float(delay_penalty), False, *args)[0]
     return _reduce(negated_loss, reduction)
 
 

@@ -196,6 +196,18 @@ def do_pruning(am, lm, ranges):
     return am_pruned, lm_pruned
 
 
+def joiner_pruned_logits(am, lm, ranges, weight, bias=None):
+    """The joiner that the reference's recipes place between do_rnnt_pruning and
+    rnnt_loss_pruned (k2/python/k2/rnnt_loss.py:913-954 describes the step: "am_pruned + lm_pruned"
+    goes to the joiner): logits = tanh(am_pruned + lm_pruned) . weight^T + bias, [B][T][R][C], with
+    weight [C][D] in torch.nn.Linear's layout.  Plain numpy on the arrays' own dtype."""
+    am_pruned, lm_pruned = do_pruning(am, lm, ranges)
+    logits = np.tanh(am_pruned + lm_pruned) @ weight.T
+    if bias is not None:
+        logits = logits + bias
+    return logits.astype(am.dtype)
+
+
 def roll_by_shifts(src, shifts):
     """k2/python/k2/rnnt_loss.py:957-989: out[b,t,s] = src[b,t,(s - shifts[b,t]) mod S]."""
     B, T, S = src.shape

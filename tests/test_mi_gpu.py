@@ -401,15 +401,27 @@ def test_single_launch_serves_any_batch_and_says_what_it_does_not(device):
     import k2_amd as k2
     bx = torch.randn(300, 70, 11, device=device)
     by = torch.randn(300, 71, 10, device=device)
-    scores, (gx, gy) = k2.mutual_information_recursion(bx, by, None, return_grad=True)
-    small, (sx, sy) = k2.mutual_information_recursion(bx[:4].contiguous(), by[:4].contiguous(), None,
-                                                      return_grad=True)
+    ones = torch.ones(300, device=device)
+    scores, gx, gy = capi.mi_forward_backward(bx, by, None, ones)
+    small, sx, sy = capi.mi_forward_backward(bx[:4].contiguous(), by[:4].contiguous(), None, ones[:4].clone())
+    torch.cuda.synchronize()
     assert torch.equal(scores[:4], small) and torch.equal(gx[:4], sx) and torch.equal(gy[:4], sy)
     a, p = omi.mi_forward(bx.cpu().numpy(), by.cpu().numpy(), None)
     wx, wy = omi.mi_backward(bx.cpu().numpy(), by.cpu().numpy(), None, p)
     np.testing.assert_allclose(scores.cpu().numpy(), a, rtol=1e-4, atol=1e-5)
     np.testing.assert_allclose(gx.cpu().numpy(), wx, rtol=1e-4, atol=1e-5)
     np.testing.assert_allclose(gy.cpu().numpy(), wy, rtol=1e-4, atol=1e-5)
+    # With more half-sweeps than compute units the two launches are the faster way, the library says
+    # so, and the Python layer follows: its results are then the pair's bits.
+    assert capi.mi_forward_backward_advised(bx[:4].contiguous(), by[:4].contiguous())
+    assert not capi.mi_forward_backward_advised(bx, by)
+    assert not capi.mi_forward_backward_advised(px, py)
+    api_scores, (ax, ay) = k2.mutual_information_recursion(bx, by, None, return_grad=True)
+    kept = torch.empty(300, 71, 11, device=device)
+    pair_scores = capi.mi_forward(bx, by, None, None, log_deriv=kept)
+    qx, qy = capi.mi_backward(bx, by, None, None, torch.ones(300, device=device), log_deriv=kept)
+    torch.cuda.synchronize()
+    assert torch.equal(api_scores, pair_scores) and torch.equal(ax, qx) and torch.equal(ay, qy)
 
 
 @pytest.mark.gpu
