@@ -177,6 +177,78 @@ def pruned_secondary(dev, steps=50, cpu=True):
     return out
 
 
+MFMA_PEAK_TFLOPS = {"fp32": 157.3, "bf16": 2500.0}  # MI355X published dense matrix rates
+
+
+def fused_joiner(dev, steps=20):
+    """The pruned loss with the joiner inside it (k2_amd.rnnt_loss_pruned_joiner) on BASELINE config
+    3's shape with a joiner of D=512, forward + backward, beside the chain it replaces on the same
+    device (do_rnnt_pruning, torch's tanh and linear, rnnt_loss_pruned).  FLOPs counted: the three
+    products an implementation cannot avoid (logits, their gradient times the weight, the
+    weight's gradient), 2 * B*T*s_range * D * V each; what the fused kernels multiply again when they
+    recompute is not counted."""
+    import torch
+    import cases
+    import k2_amd as k2
+    B, T, S, C, R, D = 32, 500, 100, 500, 5, 512
+    c = cases.rnnt_case(3, B, T, S, C, t_lo=300, s_lo=50)
+    lm0, am0 = torch.from_numpy(c["lm"]).to(dev), torch.from_numpy(c["am"]).to(dev)
+    sym, bd = torch.from_numpy(c["symbols"]).to(dev), torch.from_numpy(c["boundary"]).to(dev)
+    _, (gx, gy) = k2.rnnt_loss_simple(lm0, am0, sym, 0, bd, reduction="sum", return_grad=True)
+    ranges = k2.get_rnnt_prune_ranges(gx, gy, bd, R)
+    g = torch.Generator(device="cpu").manual_seed(7)
+    am = (0.8 * torch.randn(B, T, D, generator=g)).to(dev).requires_grad_(True)
+    lm = (0.8 * torch.randn(B, S + 1, D, generator=g)).to(dev).requires_grad_(True)
+    weight = (2.0 / D ** 0.5 * torch.randn(C, D, generator=g)).to(dev).requires_grad_(True)
+    bias = (0.5 * torch.randn(C, generator=g)).to(dev).requires_grad_(True)
+
+    def fused(precision):
+        return k2.rnnt_loss_pruned_joiner(am, lm, ranges, weight, bias, sym, 0, bd, reduction="sum",
+                                          precision=precision)
+
+    def chain(autocast):
+        am_p, lm_p = k2.do_rnnt_pruning(am, lm, ranges)
+        with torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast):
+            logits = torch.nn.functional.linear(torch.tanh(am_p + lm_p), weight, bias)
+        return k2.rnnt_loss_pruned(logits.float(), sym, ranges, 0, bd, reduction="sum")
+
+    def timed(fn):
+        for _ in range(3):
+            for t in (am, lm, weight, bias):
+                t.grad = None
+            loss = fn()
+            loss.backward()
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+        torch.cuda.synchronize()
+        ev[0].record()
+        for _ in range(steps):
+            for t in (am, lm, weight, bias):
+                t.grad = None
+            loss = fn()
+            loss.backward()
+        ev[1].record()
+        torch.cuda.synchronize()
+        return ev[0].elapsed_time(ev[1]) / steps, float(loss)
+
+    flops = 3 * 2.0 * B * T * R * D * C
+    out = {"workload": "do_rnnt_pruning -> tanh -> linear(D=512 -> V=500) -> rnnt_loss_pruned fwd+bwd, "
+                       "B=32 T=500 S=100 s_range=5 (BASELINE config 3's shape), gradients to am, lm, "
+                       "weight, bias; the fused call never stores the [B,T,s_range,V] logits",
+           "algorithmic_GFLOP": flops / 1e9}
+    for precision in ("fp32", "bf16"):
+        ms, loss = timed(lambda: fused(precision))
+        ms_chain, loss_chain = timed(lambda: chain(precision == "bf16"))
+        out[precision] = {
+            "ms_per_step": ms, "value": B / (ms * 1e-3), "unit": "utterances/s", "loss": loss,
+            "roofline": {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12,
+                         "peak": MFMA_PEAK_TFLOPS[precision], "unit": "TFLOP/s",
+                         "frac": flops / (ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS[precision]},
+            "unfused_chain_ms_per_step": ms_chain, "unfused_chain_loss": loss_chain,
+            "unfused_chain": "torch ops for the joiner" + (" under autocast(bfloat16)" if precision == "bf16" else "")
+                             + " + k2_amd.rnnt_loss_pruned on its fp32 logits"}
+    return out
+
+
 def other_configs(dev, steps=50):
     """The two remaining BASELINE configurations, forward + backward through the k2-style API with
     gradients to the network outputs: config 2 (rnnt_loss_simple, B=16 T=250 S=50 V=500) and
@@ -409,6 +481,7 @@ def main():
         del px, py, p
         out["secondary"] = pruned_secondary(dev, cpu=not args.no_cpu)
         out["other_configs"] = other_configs(dev)
+        out["fused_joiner"] = fused_joiner(dev)
     print(json.dumps(out))
 
 

@@ -18,12 +18,13 @@
 // accumulate in fp32, and everything outside the products is fp32.
 //
 // Data movement: the activations tanh(..) of a tile are formed once and kept in LDS ([row][k], k
-// contiguous); the weight is read from a copy prepared per call in the operand type, padded with
-// zeros to whole tiles, once with k = D contiguous (for logits) and once with k = C contiguous (for
-// d logits . weight).  A lane's share of an operand per step of k is 64 contiguous bytes (16 floats
-// or 32 bfloat16) of its row: four 16-byte loads from LDS or from the weight copy (which stays in
-// L2).  Which k a lane feeds to which multiply is the same for both operands, which is all the
-// instruction needs.
+// contiguous, rows 16 bytes apart modulo 256 so that 16-byte reads of 32 rows miss each other's
+// banks); the weight is read from copies prepared per call in the operand type, padded with zeros
+// to whole tiles and stored in the order the multiplies consume them (BOperand), once with k = D
+// (for logits) and once with k = C (for d logits . weight); they stay in L2.  A lane's share of an
+// operand per step of k is 64 bytes (16 floats or 32 bfloat16): four 16-byte loads.  Which k a lane
+// feeds to which multiply is the same for both operands, which is all the instruction needs.
+// Workgroups are eight wavefronts, two per SIMD.
 #include "common.h"
 
 namespace k2amd {
@@ -32,11 +33,11 @@ namespace {
 typedef float Acc16 __attribute__((ext_vector_type(16)));
 typedef __bf16 Bf8 __attribute__((ext_vector_type(8)));
 
-constexpr int kThreads = 256;   // four wavefronts
-constexpr int kNTile = 128;     // columns of a product per pass: 32 per wavefront
-constexpr int kSliceCols = 64;  // columns of d logits a workgroup of the weight-gradient kernel owns
+constexpr int kThreads = 512;   // eight wavefronts: two per SIMD, one computes while the other waits
+constexpr int kWaves = kThreads / 64;
+constexpr int kNTile = 256;     // columns of a product per pass: 32 per wavefront
 constexpr int kMaxD = 512;      // joiner dimension the LDS tiles are sized for
-constexpr int kMaxDBlocks = kMaxD / 64;  // 32-column blocks of D per wavefront in the weight gradient
+constexpr int kStageCols = 128; // columns of d pre-activation reduced at a time
 
 struct Frag {
   uint4 q[4];
@@ -58,13 +59,14 @@ __device__ __forceinline__ float FromBf16(unsigned short h) { return AsFloat((un
 // logits (sums of D such values times weights) are sensitive to.
 __device__ __forceinline__ float Tanh(float x) {
   const float e = __expf(-2.0f * fabsf(x));
-  const float t = (1.0f - e) / (1.0f + e);
+  const float t = (1.0f - e) * __builtin_amdgcn_rcpf(1.0f + e);  // 1 + e in [1, 2]: rcp is good to 1 ulp
   return x < 0 ? -t : t;
 }
 
 struct F32 {
   typedef float Elem;
   static constexpr int kChunk = 32;  // k per step
+  static constexpr int kAhead = 1;   // a step is 16 multiplies per block of rows: one step hides a trip to L2
   static constexpr int kPad = 4;     // elements: rows 16 bytes apart modulo 256 (LDS banks)
   static __device__ __forceinline__ Elem From(float f) { return f; }
   static __device__ __forceinline__ float To(Elem e) { return e; }
@@ -85,6 +87,7 @@ struct F32 {
 struct Bf16 {
   typedef unsigned short Elem;
   static constexpr int kChunk = 64;
+  static constexpr int kAhead = 1;
   static constexpr int kPad = 8;
   static __device__ __forceinline__ Elem From(float f) { return ToBf16(f); }
   static __device__ __forceinline__ float To(Elem e) { return FromBf16(e); }
@@ -112,11 +115,30 @@ __device__ __forceinline__ Frag LoadFrag(const Elem *p) {
   return f;
 }
 
+// The weight copies are stored in the order the multiplies consume them: for each block of 32 rows n
+// and each step of k, four groups of 64 x 16 bytes, group i holding for lane l the 16 bytes at
+// k = step * kChunk + (l >> 5) * kChunk / 2 + i * (16 / sizeof(Elem)) of row n = block * 32 + (l & 31):
+// one load instruction of a wavefront then reads 1 KB of consecutive memory.
+constexpr int kFragQuads = 4 * 64;  // 16-byte groups per (block of rows, step of k)
+// `block` is the same for all lanes (a scalar register), so the loads take the form scalar base +
+// lane offset + immediate and need no per-load address registers.
+__device__ __forceinline__ Frag LoadFragB(const uint4 *block, int lane) {
+  Frag f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) f.q[i] = block[i * 64 + lane];
+  return f;
+}
+// groups of block `nb`, step `step0`, in a copy with `ksteps` steps per block (all arguments the
+// same for all lanes)
+__device__ __forceinline__ const uint4 *BOperand(const void *w, int nb, int ksteps, int step0) {
+  return static_cast<const uint4 *>(w) + ((size_t)nb * ksteps + step0) * kFragQuads;
+}
+
 struct JoinerArgs {
   const float *am, *lm, *bias;  // bias may be null
   const int64_t *ranges, *symbols, *boundary;
-  const void *wk;   // weight copy [Cpad][D], k = D contiguous
-  const void *wc;   // weight copy [Dpad][Cpad], k = C contiguous
+  const void *wk;   // weight copy, rows c (Cpad), k = d: see BOperand
+  const void *wc;   // weight copy, rows d (Dpad), k = c (Cpad)
   float *px, *py, *norm;        // forward outputs (norm [B][T][R])
   const float4 *hdr;            // backward: per row {gx, gy, symbol, norm}
   float *am_grad, *lm_grad, *weight_grad, *bias_grad;
@@ -173,81 +195,152 @@ __device__ __forceinline__ int LoadMeta(const JoinerArgs &a, long long f0, RowMe
 
 // h[m][:] = tanh(am[frame] + lm[lmrow]) for the tile's rows (zeros beyond them), in the operand
 // type; kTransposed also keeps a copy ht[d][m] (k = row contiguous, for the weight gradient).
-template <typename Mode, int MT, bool kTransposed>
+template <typename Mode, int MT, bool kTransposed, int kBatch>
 __device__ __forceinline__ void StageActivations(const JoinerArgs &a, const RowMeta *meta, int rows,
                                                  typename Mode::Elem *h, int ldh,
                                                  typename Mode::Elem *ht, int ldt) {
-  const int qpr = a.D >> 2;
-  for (int idx = threadIdx.x; idx < MT * qpr; idx += kThreads) {
-    const int m = idx / qpr, q = idx - m * qpr;
-    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (m < rows) {
-      const RowMeta rm = meta[m];
-      const float4 x = *reinterpret_cast<const float4 *>(a.am + (size_t)rm.bt * a.D + 4 * q);
-      const float4 y = *reinterpret_cast<const float4 *>(a.lm + (size_t)rm.lmrow * a.D + 4 * q);
-      v = make_float4(Tanh(x.x + y.x), Tanh(x.y + y.y), Tanh(x.z + y.z), Tanh(x.w + y.w));
+  // A thread's items in batches of kBatch: all loads of a batch are asked for before the first is
+  // used (one trip to memory per batch instead of one per item; the batch is sized to the registers
+  // the caller has left).
+  const int qpr = a.D >> 2, items = MT * qpr;
+  for (int base = threadIdx.x; base < items; base += kThreads * kBatch) {
+    float4 x[kBatch], y[kBatch];
+    int at[kBatch];  // m * qpr + q, or -1 beyond the tile's items
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) {
+      const int idx = base + j * kThreads;
+      at[j] = idx < items ? idx : -1;
+      x[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+      y[j] = x[j];
+      if (idx < items) {
+        const int m = idx / qpr, q = idx - m * qpr;
+        if (m < rows) {
+          const RowMeta rm = meta[m];
+          x[j] = *reinterpret_cast<const float4 *>(a.am + (size_t)rm.bt * a.D + 4 * q);
+          y[j] = *reinterpret_cast<const float4 *>(a.lm + (size_t)rm.lmrow * a.D + 4 * q);
+        }
+      }
     }
-    Mode::Store4(h + (size_t)m * ldh + 4 * q, v);
-    if (kTransposed) {
-      ht[(size_t)(4 * q + 0) * ldt + m] = Mode::From(v.x);
-      ht[(size_t)(4 * q + 1) * ldt + m] = Mode::From(v.y);
-      ht[(size_t)(4 * q + 2) * ldt + m] = Mode::From(v.z);
-      ht[(size_t)(4 * q + 3) * ldt + m] = Mode::From(v.w);
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) {
+      if (at[j] < 0) continue;
+      const int m = at[j] / qpr, q = at[j] - m * qpr;
+      // rows beyond the tile's: tanh(0 + 0) = 0
+      const float4 v = make_float4(Tanh(x[j].x + y[j].x), Tanh(x[j].y + y[j].y), Tanh(x[j].z + y[j].z),
+                                   Tanh(x[j].w + y[j].w));
+      Mode::Store4(h + (size_t)m * ldh + 4 * q, v);
+      if (kTransposed) {
+        ht[(size_t)(4 * q + 0) * ldt + m] = Mode::From(v.x);
+        ht[(size_t)(4 * q + 1) * ldt + m] = Mode::From(v.y);
+        ht[(size_t)(4 * q + 2) * ldt + m] = Mode::From(v.z);
+        ht[(size_t)(4 * q + 3) * ldt + m] = Mode::From(v.w);
+      }
     }
   }
 }
 
 // acc[rb] += A[rows rb*32 .. +31][0..K) . B[n][0..K)^T for the wavefront's 32 columns n: A in LDS
-// (row stride lda elements), B rows in global memory (row stride ldb), both k-contiguous.
-template <typename Mode, int RB>
+// (row stride lda elements), B rows in global memory, both k-contiguous.  kSteps > 0: the number of
+// steps of k is known when compiling and the loop is unrolled completely, B asked for Mode::kAhead steps
+// and A one step ahead of their use (the compiler counts outstanding loads exactly in straight-line
+// code; around a loop it waits for all of them at every iteration).  kSteps == 0: any K, that loop.
+template <typename Mode, int RB, int kSteps>
 __device__ __forceinline__ void TileProduct(Acc16 (&acc)[RB], const typename Mode::Elem *a_lane,
-                                            int lda, const typename Mode::Elem *b_lane, int K) {
+                                            int lda, const uint4 *b_block, int lane, int K) {
   constexpr int kChunk = Mode::kChunk;
-  const int chunks = K / kChunk;
-  Frag fb = LoadFrag(b_lane);
-  for (int kc = 0; kc < chunks; ++kc) {
-    const int next = kc + 1 < chunks ? kc + 1 : kc;
-    const Frag fbn = LoadFrag(b_lane + (size_t)next * kChunk);
+  if constexpr (kSteps > 0) {
+    constexpr int kAhead = Mode::kAhead;  // steps of k between asking for B and using it
+    Frag fb[kAhead + 1], fa[2][RB];
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb) {
-      const Frag fa = LoadFrag(a_lane + (size_t)rb * 32 * lda + (size_t)kc * kChunk);
-      Mode::Mma(acc[rb], fa, fb);
+    for (int i = 0; i < kAhead; ++i)
+      if (i < kSteps) fb[i] = LoadFragB(b_block + (size_t)i * kFragQuads, lane);
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) fa[0][rb] = LoadFrag(a_lane + (size_t)rb * 32 * lda);
+#pragma unroll
+    for (int kc = 0; kc < kSteps; ++kc) {
+      if (kc + kAhead < kSteps)
+        fb[(kc + kAhead) % (kAhead + 1)] = LoadFragB(b_block + (size_t)(kc + kAhead) * kFragQuads, lane);
+      if (kc + 1 < kSteps) {
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+          fa[(kc + 1) & 1][rb] = LoadFrag(a_lane + (size_t)rb * 32 * lda + (size_t)(kc + 1) * kChunk);
+      }
+      __builtin_amdgcn_sched_barrier(0);  // the requests above stay above the multiplies below
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) Mode::Mma(acc[rb], fa[kc & 1][rb], fb[kc % (kAhead + 1)]);
+      __builtin_amdgcn_sched_barrier(0);
     }
-    fb = fbn;
+  } else {
+    const int chunks = K / kChunk, last = chunks - 1;
+    Frag f0 = LoadFragB(b_block, lane);
+    Frag f1 = LoadFragB(b_block + (size_t)(1 < last ? 1 : last) * kFragQuads, lane);
+    for (int kc = 0; kc < chunks; ++kc) {
+      const int ahead = kc + 2 < last ? kc + 2 : last;
+      const Frag f2 = LoadFragB(b_block + (size_t)ahead * kFragQuads, lane);
+      Frag fa[RB];
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) fa[rb] = LoadFrag(a_lane + (size_t)rb * 32 * lda + (size_t)kc * kChunk);
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) Mode::Mma(acc[rb], fa[rb], f0);
+      f0 = f1;
+      f1 = f2;
+    }
   }
 }
 
+// A lane's value as seen by the lane that a DPP control pairs it with (within rows of 16 lanes).
+template <int kCtrl>
+__device__ __forceinline__ float Dpp(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), kCtrl, 0xf, 0xf, true));
+}
+// (max, sum of exp relative to it) of two sets of logits merged
+__device__ __forceinline__ void MergeLse(float &m, float &s, float om, float os) {
+  const float d = m - om;
+  const float e = __expf(-fabsf(d));
+  s = d >= 0 ? s + os * e : s * e + os;
+  m = fmaxf(m, om);
+}
 // accumulator element r of a lane: row (r >> 2) * 8 + half * 4 + (r & 3) of the 32 x 32 block,
 // column lane & 31
 __device__ __forceinline__ int AccRow(int r, int half) { return (r >> 2) * 8 + half * 4 + (r & 3); }
 
 constexpr float kLowest = -3.0e38f;  // start of a running maximum (finite: -inf - -inf is NaN)
 
+// d logits of one element: -softmax (gx + gy) + gx [n == symbol] + gy [n == blank]; g = {gx, gy,
+// symbol, norm}
+__device__ __forceinline__ float LogitGrad(float z, int n, const float4 g, int blank) {
+  float v = -__expf(z - g.w) * (g.x + g.y);
+  if (n == (int)g.z) v += g.x;
+  if (n == blank) v += g.y;
+  return v;
+}
+
 // ---------------------------------------------------------------------------------- forward
 //
 // LDS: h [MT][D + pad]; row meta; the two picked logits per row; per wavefront (max, sum) per row.
-template <typename Mode, int RB>
+template <typename Mode, int RB, int kD>
 __global__ __launch_bounds__(kThreads) void JoinerForwardKernel(const JoinerArgs a) {
+  constexpr int kStepsD = kD / Mode::kChunk;  // 0: D only known at run time
   constexpr int MT = 32 * RB;
   typedef typename Mode::Elem Elem;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  const int ldh = a.D + Mode::kPad;
+  const int ldh = (kD > 0 ? kD : a.D) + Mode::kPad;  // a constant where D is one: LDS offsets become immediates
   Elem *h = reinterpret_cast<Elem *>(smem);
   RowMeta *meta = reinterpret_cast<RowMeta *>(smem + (size_t)MT * ldh * sizeof(Elem));
   float *zsym = reinterpret_cast<float *>(meta + MT);
   float *zblank = zsym + MT;
-  float *part_m = zblank + MT;  // [4][MT]
-  float *part_s = part_m + 4 * MT;
+  float *part_m = zblank + MT;  // [kWaves][MT]
+  float *part_s = part_m + kWaves * MT;
 
   const long long f0 = (long long)blockIdx.x * a.tpt;
   const int rows = LoadMeta<MT>(a, f0, meta);
   for (int m = threadIdx.x; m < MT; m += kThreads) { zsym[m] = 0.f; zblank[m] = 0.f; }
   __syncthreads();
-  StageActivations<Mode, MT, false>(a, meta, rows, h, ldh, nullptr, 0);
+  StageActivations<Mode, MT, false, 8>(a, meta, rows, h, ldh, nullptr, 0);
   __syncthreads();
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 31, half = lane >> 5;
-  const Elem *wk = static_cast<const Elem *>(a.wk);
+  const int lane = threadIdx.x & 63, col = lane & 31, half = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the same in all lanes: a scalar
   const Elem *a_lane = h + (size_t)col * ldh + half * (Mode::kChunk / 2);
   float run_m[RB][16], run_s[RB][16];
 #pragma unroll
@@ -262,7 +355,7 @@ __global__ __launch_bounds__(kThreads) void JoinerForwardKernel(const JoinerArgs
     for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[rb][r] = 0.f;
-    TileProduct<Mode, RB>(acc, a_lane, ldh, wk + (size_t)n * a.D + half * (Mode::kChunk / 2), a.D);
+    TileProduct<Mode, RB, kStepsD>(acc, a_lane, ldh, BOperand(a.wk, (n0 >> 5) + wave, a.D / Mode::kChunk, 0), lane, a.D);
     if (n < a.C) {
       const float bn = a.bias != nullptr ? a.bias[n] : 0.f;
 #pragma unroll
@@ -271,47 +364,76 @@ __global__ __launch_bounds__(kThreads) void JoinerForwardKernel(const JoinerArgs
         for (int r = 0; r < 16; ++r) {
           const int row = rb * 32 + AccRow(r, half);
           const float z = acc[rb][r] + bn;
-          const float m = run_m[rb][r];
-          if (z > m) {
-            run_s[rb][r] = run_s[rb][r] * __expf(m - z) + 1.0f;
-            run_m[rb][r] = z;
-          } else {
-            run_s[rb][r] += __expf(z - m);
-          }
+          const float m = run_m[rb][r], d = z - m;
+          const float e = __expf(-fabsf(d));
+          run_s[rb][r] = d > 0 ? run_s[rb][r] * e + 1.0f : run_s[rb][r] + e;
+          run_m[rb][r] = d > 0 ? z : m;
           if (n == meta[row].sym) zsym[row] = z;
           if (n == a.blank) zblank[row] = z;
         }
     }
   }
-  // (max, sum) of a row: over the 32 lanes that hold its columns, then over the wavefronts
+  // (max, sum) of a row: over the 32 lanes that hold its columns, then over the wavefronts.  The
+  // lanes of a half wavefront hold the same 16 RB rows; at each step a lane keeps one half of the
+  // rows it still holds and hands the other half to its partner (xor 1, 2 inside quads on the vector
+  // ALU, xor 4, 8, 16 through the LDS crossbar), so every merge is done once, and after five steps
+  // (six with RB = 2) each lane holds the merged pair of the rows that the bits of its number select.
+  {
+    constexpr int kN = 16 * RB;
+    float vm[kN], vs[kN];
 #pragma unroll
-  for (int rb = 0; rb < RB; ++rb)
+    for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      float m = run_m[rb][r], s = run_s[rb][r];
-#pragma unroll
-      for (int off = 16; off >= 1; off >>= 1) {
-        const float om = __shfl_xor(m, off, kWave), os = __shfl_xor(s, off, kWave);
-        const float mm = fmaxf(m, om);
-        s = s * __expf(m - mm) + os * __expf(om - mm);
-        m = mm;
-      }
-      if (col == 0) {
-        const int row = rb * 32 + AccRow(r, half);
-        part_m[wave * MT + row] = m;
-        part_s[wave * MT + row] = s;
+      for (int r = 0; r < 16; ++r) { vm[rb * 16 + r] = run_m[rb][r]; vs[rb * 16 + r] = run_s[rb][r]; }
+    int mine = 0;  // index rb * 16 + r of the first row this lane ends up with
+#define K2AMD_SCATTER_STEP(COUNT, BIT, EXCHANGE)                              \
+    {                                                                         \
+      const bool up = (col & (BIT)) != 0;                                     \
+      _Pragma("unroll") for (int j = 0; j < (COUNT) / 2; ++j) {               \
+        float km = up ? vm[j + (COUNT) / 2] : vm[j], ks = up ? vs[j + (COUNT) / 2] : vs[j]; \
+        const float sm = up ? vm[j] : vm[j + (COUNT) / 2], ss = up ? vs[j] : vs[j + (COUNT) / 2]; \
+        MergeLse(km, ks, EXCHANGE(sm), EXCHANGE(ss));                         \
+        vm[j] = km;                                                           \
+        vs[j] = ks;                                                           \
+      }                                                                       \
+      if (up) mine += (COUNT) / 2;                                            \
+    }
+#define K2AMD_X1(v) Dpp<0xB1>(v)
+#define K2AMD_X2(v) Dpp<0x4E>(v)
+#define K2AMD_X4(v) __shfl_xor(v, 4, kWave)
+#define K2AMD_X8(v) __shfl_xor(v, 8, kWave)
+#define K2AMD_X16(v) __shfl_xor(v, 16, kWave)
+    K2AMD_SCATTER_STEP(kN, 1, K2AMD_X1)
+    K2AMD_SCATTER_STEP(kN / 2, 2, K2AMD_X2)
+    K2AMD_SCATTER_STEP(kN / 4, 4, K2AMD_X4)
+    K2AMD_SCATTER_STEP(kN / 8, 8, K2AMD_X8)
+    if constexpr (RB == 2) {
+      K2AMD_SCATTER_STEP(kN / 16, 16, K2AMD_X16)
+      const int row = (mine >> 4) * 32 + AccRow(mine & 15, half);
+      part_m[wave * MT + row] = vm[0];
+      part_s[wave * MT + row] = vs[0];
+    } else {
+      // RB == 1: one row left per pair of lanes 16 apart; merge it, the lower lane stores
+      float km = vm[0], ks = vs[0];
+      MergeLse(km, ks, K2AMD_X16(vm[0]), K2AMD_X16(vs[0]));
+      if ((col & 16) == 0) {
+        const int row = AccRow(mine & 15, half);
+        part_m[wave * MT + row] = km;
+        part_s[wave * MT + row] = ks;
       }
     }
+#undef K2AMD_SCATTER_STEP
+#undef K2AMD_X1
+#undef K2AMD_X2
+#undef K2AMD_X4
+#undef K2AMD_X8
+#undef K2AMD_X16
+  }
   __syncthreads();
   for (int row = threadIdx.x; row < rows; row += kThreads) {
     float m = part_m[row], s = part_s[row];
 #pragma unroll
-    for (int w = 1; w < 4; ++w) {
-      const float om = part_m[w * MT + row], os = part_s[w * MT + row];
-      const float mm = fmaxf(m, om);
-      s = s * __expf(m - mm) + os * __expf(om - mm);
-      m = mm;
-    }
+    for (int w = 1; w < kWaves; ++w) MergeLse(m, s, part_m[w * MT + row], part_s[w * MT + row]);
     const float norm = m + logf(s);
     const RowMeta rm = meta[row];
     const int b = rm.bt / a.Tn, t = rm.bt - b * a.Tn;
@@ -330,21 +452,26 @@ __global__ __launch_bounds__(kThreads) void JoinerForwardKernel(const JoinerArgs
 
 // ------------------------------------------------------------ backward, gradients of am and lm
 //
-// One tile of 32 rows per workgroup: d logits [32][Cpad] into LDS, then d h = d logits . weight,
-// d pre = d h (1 - h^2); am_grad[frame] is the sum over the frame's R rows (plain stores: a frame
-// lies in one tile), lm_grad[b, s] collects its rows with atomic adds (runs of equal s along t are
-// added up first).
-template <typename Mode>
+// One tile of MT rows per workgroup.  Per tile of 256 columns c: logits -> d logits into LDS, then
+// d h += d logits . weight[c-tile] with d h [MT][D] kept in accumulators over all column tiles
+// (wavefront w owns the 32-column blocks w and w + 8 of D).  At the end d pre = d h (1 - h^2) goes
+// through LDS 128 columns at a time: am_grad[frame] is the sum over the frame's R rows (plain
+// stores: a frame lies in one tile), lm_grad[b, s] collects its rows with atomic adds (runs of
+// equal s along t are added up first).
+template <typename Mode, int RB, int kD>
 __global__ __launch_bounds__(kThreads) void JoinerBackwardRowsKernel(const JoinerArgs a) {
-  constexpr int MT = 32;
+  constexpr int kStepsD = kD / Mode::kChunk;  // 0: D only known at run time
+  constexpr int MT = 32 * RB;
   typedef typename Mode::Elem Elem;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  const int ldh = a.D + Mode::kPad, ldc = a.Cpad + Mode::kPad;
-  constexpr int kLdStage = kNTile + 4;
+  const int ldh = (kD > 0 ? kD : a.D) + Mode::kPad;  // a constant where D is one: LDS offsets become immediates
+  constexpr int ldz = kNTile + Mode::kPad;
+  constexpr int kLdStage = kStageCols + 4;
+  static_assert((size_t)MT * kLdStage * sizeof(float) <= (size_t)MT * ldz * sizeof(Elem), "stage fits dz");
   Elem *h = reinterpret_cast<Elem *>(smem);
   Elem *dz = h + (size_t)MT * ldh;
-  float *stage = reinterpret_cast<float *>(dz + (size_t)MT * ldc);
-  float4 *hdr = reinterpret_cast<float4 *>(stage + MT * kLdStage);
+  float *stage = reinterpret_cast<float *>(dz);  // after the last column tile
+  float4 *hdr = reinterpret_cast<float4 *>(dz + (size_t)MT * ldz);
   RowMeta *meta = reinterpret_cast<RowMeta *>(hdr + MT);
 
   const long long f0 = (long long)blockIdx.x * a.tpt;
@@ -352,55 +479,75 @@ __global__ __launch_bounds__(kThreads) void JoinerBackwardRowsKernel(const Joine
   for (int m = threadIdx.x; m < MT; m += kThreads)
     hdr[m] = m < rows ? a.hdr[(size_t)f0 * a.R + m] : make_float4(0.f, 0.f, -1.f, 3.0e38f);  // padding: exp(. - norm) = 0
   __syncthreads();
-  StageActivations<Mode, MT, false>(a, meta, rows, h, ldh, nullptr, 0);
+  StageActivations<Mode, MT, false, 8>(a, meta, rows, h, ldh, nullptr, 0);
   __syncthreads();
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 31, half = lane >> 5;
+  const int lane = threadIdx.x & 63, col = lane & 31, half = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the same in all lanes: a scalar
   const int koff = half * (Mode::kChunk / 2);
-  const Elem *wk = static_cast<const Elem *>(a.wk), *wc = static_cast<const Elem *>(a.wc);
+  Acc16 dh[2][RB];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dh[i][rb][r] = 0.f;
+
   for (int n0 = 0; n0 < a.Cpad; n0 += kNTile) {
     const int n = n0 + wave * 32 + col;
-    Acc16 acc[1];
+    Acc16 acc[RB];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[0][r] = 0.f;
-    TileProduct<Mode, 1>(acc, h + (size_t)col * ldh + koff, ldh, wk + (size_t)n * a.D + koff, a.D);
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[rb][r] = 0.f;
+    TileProduct<Mode, RB, kStepsD>(acc, h + (size_t)col * ldh + koff, ldh,
+                                   BOperand(a.wk, (n0 >> 5) + wave, a.D / Mode::kChunk, 0), lane, a.D);
     const float bn = (n < a.C && a.bias != nullptr) ? a.bias[n] : 0.f;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int row = AccRow(r, half);
-      const float4 g = hdr[row];  // gx, gy, symbol, norm
-      float v = 0.f;
-      if (n < a.C) {
-        v = -__expf(acc[0][r] + bn - g.w) * (g.x + g.y);
-        if (n == (int)g.z) v += g.x;
-        if (n == a.blank) v += g.y;
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = rb * 32 + AccRow(r, half);
+        const float v = n < a.C ? LogitGrad(acc[rb][r] + bn, n, hdr[row], a.blank) : 0.f;
+        dz[(size_t)row * ldz + wave * 32 + col] = Mode::From(v);
       }
-      dz[(size_t)row * ldc + n] = Mode::From(v);
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      if ((wave + kWaves * i) * 32 < a.D)
+        TileProduct<Mode, RB, kNTile / Mode::kChunk>(dh[i], dz + (size_t)col * ldz + koff, ldz,
+                                                     BOperand(a.wc, wave + kWaves * i, a.Cpad / Mode::kChunk, n0 / Mode::kChunk), lane, kNTile);
     }
+    __syncthreads();
   }
-  __syncthreads();
-  const int part = threadIdx.x >> 7, c = threadIdx.x & 127;
+
+  const int part = threadIdx.x / kStageCols, c = threadIdx.x % kStageCols;
+  constexpr int kParts = kThreads / kStageCols;
   const int nf = rows / a.R;
-  for (int d0 = 0; d0 < a.Dpad; d0 += kNTile) {
-    const int d = d0 + wave * 32 + col;
-    Acc16 acc[1];
+  for (int d0 = 0; d0 < a.D; d0 += kStageCols) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[0][r] = 0.f;
-    TileProduct<Mode, 1>(acc, dz + (size_t)col * ldc + koff, ldc, wc + (size_t)d * a.Cpad + koff, a.Cpad);
+    for (int i = 0; i < 2; ++i) {
+      const int db = wave + kWaves * i;
+      if (db * 32 >= d0 && db * 32 < d0 + kStageCols && db * 32 < a.D) {
+        const int d = db * 32 + col;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int row = AccRow(r, half);
-      const float hv = d < a.D ? Mode::To(h[(size_t)row * ldh + d]) : 0.f;
-      stage[row * kLdStage + wave * 32 + col] = acc[0][r] * (1.0f - hv * hv);
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int row = rb * 32 + AccRow(r, half);
+            const float hv = Mode::To(h[(size_t)row * ldh + d]);
+            stage[row * kLdStage + d - d0] = dh[i][rb][r] * (1.0f - hv * hv);
+          }
+      }
     }
     __syncthreads();
     if (d0 + c < a.D) {
-      for (int fl = part; fl < nf; fl += 2) {
+      for (int fl = part; fl < nf; fl += kParts) {
         float sum = 0.f;
         for (int k = 0; k < a.R; ++k) sum += stage[(fl * a.R + k) * kLdStage + c];
         a.am_grad[(size_t)(f0 + fl) * a.D + d0 + c] = sum;
       }
-      for (int k = part; k < a.R; k += 2) {
+      for (int k = part; k < a.R; k += kParts) {
         int key = -1;
         float sum = 0.f;
         for (int fl = 0; fl < nf; ++fl) {
@@ -422,40 +569,49 @@ __global__ __launch_bounds__(kThreads) void JoinerBackwardRowsKernel(const Joine
 
 // ------------------------------------------------------- backward, gradients of weight and bias
 //
-// A workgroup owns 64 columns c of d logits and every kGroups-th share of the tiles of 64 rows; it
-// keeps its [64][D] block of the weight's gradient in accumulators over all of its tiles:
-//   logits slice = h . weight[c-slice]^T     (k = D)
+// A workgroup owns kSlice columns c of d logits and every `groups`-th tile of 64 rows; it keeps its
+// [kSlice][D] block of the weight's gradient in accumulators over all of its tiles:
+//   logits slice = h . weight[c-slice]^T     (k = D; with fewer 32 x 32 blocks than wavefronts, k is
+//                                             split between them and the halves meet in LDS)
 //   d logits slice -> LDS, transposed [c][row]
 //   weight_grad[c][d] += sum over rows of d logits[row][c] h[row][d]   (k = rows of the tile)
 // and adds it to weight_grad (zeroed by the launcher) with atomic adds at the end.
-template <typename Mode>
+template <typename Mode, int kSlice, int kD>
 __global__ __launch_bounds__(kThreads) void JoinerBackwardWeightKernel(const JoinerArgs a, int tiles,
                                                                         int groups) {
   constexpr int MT = 64;
   constexpr bool kBf = sizeof(typename Mode::Elem) == 2;
+  constexpr int kColBlocks = kSlice / 32;               // 32-column blocks of the slice
+  constexpr int kBlocks = 2 * kColBlocks;               // blocks of the logits slice
+  constexpr int kSplit = kWaves / kBlocks;              // wavefronts per block: shares of k
+  constexpr int kDGroups = kWaves / kColBlocks;         // wavefronts per column block in the gradient
+  constexpr int kMaxDB = (kMaxD / 32) / kDGroups;       // 32-column blocks of D per wavefront
+  static_assert(kBlocks * kSplit == kWaves && (kSplit == 1 || kSplit == 2), "wavefront roles");
   typedef typename Mode::Elem Elem;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  const int ldh = a.D + Mode::kPad;
+  const int ldh = (kD > 0 ? kD : a.D) + Mode::kPad;  // a constant where D is one: LDS offsets become immediates
   constexpr int ldz = MT + Mode::kPad;  // d logits, transposed: [c][row]
   constexpr int ldt = MT + Mode::kPad;  // h, transposed: [d][row] (bfloat16 only)
   Elem *h = reinterpret_cast<Elem *>(smem);
   Elem *dzt = h + (size_t)MT * ldh;
-  Elem *ht = dzt + (size_t)kSliceCols * ldz;
+  Elem *ht = dzt + (size_t)kSlice * ldz;
   float4 *hdr = reinterpret_cast<float4 *>(ht + (kBf ? (size_t)a.D * ldt : 0));
   RowMeta *meta = reinterpret_cast<RowMeta *>(hdr + MT);
 
   const int slice = blockIdx.x / groups, group = blockIdx.x - slice * groups;
-  const int c0 = slice * kSliceCols;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 31, half = lane >> 5;
+  const int c0 = slice * kSlice;
+  const int lane = threadIdx.x & 63, col = lane & 31, half = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the same in all lanes: a scalar
   const int koff = half * (Mode::kChunk / 2);
-  const int rb = wave >> 1, cb = wave & 1;  // block of the logits slice this wavefront multiplies
-  const int n = c0 + cb * 32 + col;         // its column of logits (< Cpad: slices tile Cpad)
-  const Elem *wk = static_cast<const Elem *>(a.wk);
-  // its blocks of the gradient: columns c0 + cb*32 .. +31, d blocks dhalf * ndb .. + ndb - 1
-  const int ndb = a.D / 64, dhalf = wave >> 1;
-  Acc16 wacc[kMaxDBlocks];
+  // the block of the logits slice this wavefront multiplies, and its share of k
+  const int blk = wave % kBlocks, ks = wave / kBlocks, rb = blk / kColBlocks, cb = blk % kColBlocks;
+  const int n = c0 + cb * 32 + col;  // its column of logits (< Cpad: slices tile Cpad)
+  const int kshare = a.D / kSplit;
+  // its blocks of the gradient: columns c0 + gcb*32 .. +31, d blocks dgrp, dgrp + kDGroups, ..
+  const int gcb = wave % kColBlocks, dgrp = wave / kColBlocks, ndb = a.D / 32;
+  Acc16 wacc[kMaxDB];
 #pragma unroll
-  for (int i = 0; i < kMaxDBlocks; ++i)
+  for (int i = 0; i < kMaxDB; ++i)
 #pragma unroll
     for (int r = 0; r < 16; ++r) wacc[i][r] = 0.f;
   float bsum = 0.f;
@@ -467,38 +623,49 @@ __global__ __launch_bounds__(kThreads) void JoinerBackwardWeightKernel(const Joi
     for (int m = threadIdx.x; m < MT; m += kThreads)
       hdr[m] = m < rows ? a.hdr[(size_t)f0 * a.R + m] : make_float4(0.f, 0.f, -1.f, 3.0e38f);  // padding: exp(. - norm) = 0
     __syncthreads();
-    StageActivations<Mode, MT, kBf>(a, meta, rows, h, ldh, ht, ldt);
+    StageActivations<Mode, MT, kBf, kBf ? 4 : 2>(a, meta, rows, h, ldh, ht, ldt);
     __syncthreads();
     Acc16 acc[1];
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[0][r] = 0.f;
-    TileProduct<Mode, 1>(acc, h + (size_t)(rb * 32 + col) * ldh + koff, ldh,
-                         wk + (size_t)n * a.D + koff, a.D);
+    TileProduct<Mode, 1, kD / kSplit / Mode::kChunk>(acc, h + (size_t)(rb * 32 + col) * ldh + ks * kshare + koff,
+                                                     ldh, BOperand(a.wk, (c0 >> 5) + cb, a.D / Mode::kChunk, ks * kshare / Mode::kChunk), lane, kshare);
+    if constexpr (kSplit == 2) {  // the upper share of k parks its sums where the block's d logits will go
+      float *park = reinterpret_cast<float *>(dzt);
+      if (ks == 1) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int row = rb * 32 + AccRow(r, half);
-      const float4 g = hdr[row];
-      float v = 0.f;
-      if (n < a.C) {
-        v = -__expf(acc[0][r] + bn - g.w) * (g.x + g.y);
-        if (n == (int)g.z) v += g.x;
-        if (n == a.blank) v += g.y;
+        for (int r = 0; r < 16; ++r)
+          park[(size_t)(cb * 32 + col) * ldz + rb * 32 + AccRow(r, half)] = acc[0][r];
       }
-      dzt[(size_t)(cb * 32 + col) * ldz + row] = Mode::From(v);
+      __syncthreads();
+      if (ks == 0) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          acc[0][r] += park[(size_t)(cb * 32 + col) * ldz + rb * 32 + AccRow(r, half)];
+      }
+    }
+    if (ks == 0) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = rb * 32 + AccRow(r, half);
+        const float v = n < a.C ? LogitGrad(acc[0][r] + bn, n, hdr[row], a.blank) : 0.f;
+        dzt[(size_t)(cb * 32 + col) * ldz + row] = Mode::From(v);
+      }
     }
     __syncthreads();
-    if (threadIdx.x < kSliceCols) {
+    if (threadIdx.x < kSlice) {
       float s = 0.f;
       for (int m = 0; m < MT; ++m) s += Mode::To(dzt[(size_t)threadIdx.x * ldz + m]);
       bsum += s;
     }
 #pragma unroll
     for (int kc = 0; kc < MT / Mode::kChunk; ++kc) {
-      const Frag fa = LoadFrag(dzt + (size_t)(cb * 32 + col) * ldz + kc * Mode::kChunk + koff);
+      const Frag fa = LoadFrag(dzt + (size_t)(gcb * 32 + col) * ldz + kc * Mode::kChunk + koff);
 #pragma unroll
-      for (int i = 0; i < kMaxDBlocks; ++i) {
-        if (i < ndb) {
-          const int d = (dhalf * ndb + i) * 32 + col;
+      for (int i = 0; i < kMaxDB; ++i) {
+        const int db = dgrp + kDGroups * i;
+        if (db < ndb) {
+          const int d = db * 32 + col;
           Frag fb;
           if (kBf) {
             fb = LoadFrag(ht + (size_t)d * ldt + kc * Mode::kChunk + koff);
@@ -518,37 +685,59 @@ __global__ __launch_bounds__(kThreads) void JoinerBackwardWeightKernel(const Joi
     __syncthreads();  // the next tile's staging overwrites h, dzt, hdr
   }
 #pragma unroll
-  for (int i = 0; i < kMaxDBlocks; ++i) {
-    if (i < ndb) {
-      const int d = (dhalf * ndb + i) * 32 + col;
+  for (int i = 0; i < kMaxDB; ++i) {
+    const int db = dgrp + kDGroups * i;
+    if (db < ndb) {
+      const int d = db * 32 + col;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int c = c0 + cb * 32 + AccRow(r, half);
+        const int c = c0 + gcb * 32 + AccRow(r, half);
         if (c < a.C) atomicAdd(a.weight_grad + (size_t)c * a.D + d, wacc[i][r]);
       }
     }
   }
-  if (threadIdx.x < kSliceCols && c0 + (int)threadIdx.x < a.C && a.bias_grad != nullptr)
+  if (threadIdx.x < kSlice && c0 + (int)threadIdx.x < a.C && a.bias_grad != nullptr)
     atomicAdd(a.bias_grad + c0 + threadIdx.x, bsum);
 }
 
 // ---------------------------------------------------------------------------- small kernels
 
-// The weight [C][D] in the operand type: wk [Cpad][D] and wc [Dpad][Cpad], zeros in the padding.
+// The weight [C][D] in the operand type and in the order the multiplies read it (see BOperand):
+// wk with rows n = c (Cpad of them, zeros beyond C) and k = d; wc with rows n = d (Dpad) and k = c
+// (Cpad, zeros beyond C and D).  One thread per 16-byte group.
 template <typename Mode>
-__global__ void JoinerPrepWeightKernel(const float *__restrict__ weight, typename Mode::Elem *wk,
-                                       typename Mode::Elem *wc, int C, int D, int Cpad, int Dpad) {
-  const size_t nk = (size_t)Cpad * D, nc = (size_t)Dpad * Cpad;
-  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nk + nc;
-       i += (size_t)gridDim.x * blockDim.x) {
-    if (i < nk) {
-      const int c = (int)(i / D), d = (int)(i - (size_t)c * D);
-      wk[i] = Mode::From(c < C ? weight[(size_t)c * D + d] : 0.f);
-    } else if (wc != nullptr) {
-      const size_t j = i - nk;
-      const int d = (int)(j / Cpad), c = (int)(j - (size_t)d * Cpad);
-      wc[j] = Mode::From(c < C && d < D ? weight[(size_t)c * D + d] : 0.f);
+__global__ void JoinerPrepWeightKernel(const float *__restrict__ weight, uint4 *wk, uint4 *wc, int C,
+                                       int D, int Cpad, int Dpad) {
+  typedef typename Mode::Elem Elem;
+  constexpr int kPer = 16 / sizeof(Elem);  // elements per group
+  const size_t nk = (size_t)Cpad * D / kPer, nc = wc != nullptr ? (size_t)Dpad * Cpad / kPer : 0;
+  for (size_t g = (size_t)blockIdx.x * blockDim.x + threadIdx.x; g < nk + nc;
+       g += (size_t)gridDim.x * blockDim.x) {
+    const bool second = g >= nk;
+    const size_t j = second ? g - nk : g;
+    const int ksteps = (second ? Cpad : D) / Mode::kChunk;
+    const int lane = (int)(j & 63), i = (int)((j >> 6) & 3);
+    const size_t blockstep = j >> 8;
+    const int step = (int)(blockstep % ksteps), nb = (int)(blockstep / ksteps);
+    const int n = nb * 32 + (lane & 31);
+    const int k0 = step * Mode::kChunk + (lane >> 5) * (Mode::kChunk / 2) + i * kPer;
+    Elem v[kPer];
+#pragma unroll
+    for (int e = 0; e < kPer; ++e) {
+      const int c = second ? k0 + e : n, d = second ? n : k0 + e;
+      v[e] = Mode::From(c < C && d < D ? weight[(size_t)c * D + d] : 0.f);
     }
+    uint4 out;
+    if (sizeof(Elem) == 4) {
+      out = make_uint4(AsBits(Mode::To(v[0])), AsBits(Mode::To(v[1])), AsBits(Mode::To(v[2])), AsBits(Mode::To(v[3])));
+    } else {
+      unsigned w32[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        w32[e] = (unsigned)(unsigned short)v[(2 * e) % kPer] | ((unsigned)(unsigned short)v[(2 * e + 1) % kPer] << 16);
+      out = make_uint4(w32[0], w32[1], w32[2], w32[3]);
+    }
+    (second ? wc : wk)[j] = out;
   }
 }
 
@@ -654,10 +843,9 @@ JoinerArgs MakeArgs(const float *am, const float *lm, const int64_t *ranges, con
 
 template <typename Mode>
 int PrepWeights(const float *weight, const JoinerArgs &a, bool both, hipStream_t st) {
-  typedef typename Mode::Elem Elem;
   hipLaunchKernelGGL(JoinerPrepWeightKernel<Mode>, dim3(512), dim3(256), 0, st, weight,
-                     static_cast<Elem *>(const_cast<void *>(a.wk)),
-                     both ? static_cast<Elem *>(const_cast<void *>(a.wc)) : nullptr, a.C, a.D, a.Cpad, a.Dpad);
+                     static_cast<uint4 *>(const_cast<void *>(a.wk)),
+                     both ? static_cast<uint4 *>(const_cast<void *>(a.wc)) : nullptr, a.C, a.D, a.Cpad, a.Dpad);
   return LaunchStatus();
 }
 
@@ -671,12 +859,12 @@ int ForwardImpl(const float *weight, JoinerArgs a, hipStream_t st) {
   hipLaunchKernelGGL(JoinerFillKernel, dim3(512), dim3(256), 0, st, a.px, npx, Real<float>::NegInf(),
                      a.py, npy, Real<float>::NegInf());
   const size_t lds = (size_t)MT * (a.D + Mode::kPad) * sizeof(typename Mode::Elem) +
-                     MT * (sizeof(RowMeta) + 10 * sizeof(float));
-  rc = AllowLds(JoinerForwardKernel<Mode, RB>, lds);
+                     MT * (sizeof(RowMeta) + (2 + 2 * kWaves) * sizeof(float));
+  auto kernel = a.D == kMaxD ? JoinerForwardKernel<Mode, RB, kMaxD> : JoinerForwardKernel<Mode, RB, 0>;
+  rc = AllowLds(kernel, lds);
   if (rc != K2AMD_OK) return rc;
   const long long tiles = (a.frames + a.tpt - 1) / a.tpt;
-  if (tiles > 0)
-    hipLaunchKernelGGL((JoinerForwardKernel<Mode, RB>), dim3((unsigned)tiles), dim3(kThreads), lds, st, a);
+  if (tiles > 0) hipLaunchKernelGGL(kernel, dim3((unsigned)tiles), dim3(kThreads), lds, st, a);
   if (a.rnnt_type == K2AMD_CONSTRAINED && a.S > 0 && a.frames > 0)
     hipLaunchKernelGGL(JoinerConstrainedKernel, dim3(512), dim3(256), 0, st, a.px, a.py, a.B, a.S, a.Tn);
   return LaunchStatus();
@@ -698,32 +886,37 @@ int BackwardImpl(const float *weight, JoinerArgs a, const float *px_grad, const 
   if (rows == 0) return LaunchStatus();
   hipLaunchKernelGGL(JoinerRowHeaderKernel, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, st, a,
                      px_grad, py_grad, seq_scale, const_cast<float4 *>(a.hdr));
-  {  // gradients of am and lm: tiles of 32 rows
+  {  // gradients of am and lm: tiles of 32 (fp32) or 64 (bfloat16) rows
+    constexpr int RB = kBf ? 2 : 1, MT = 32 * RB;
     JoinerArgs r = a;
-    r.tpt = 32 / a.R;
-    const size_t lds = (size_t)32 * (a.D + Mode::kPad + a.Cpad + Mode::kPad) * sizeof(Elem) +
-                       32 * ((kNTile + 4) * sizeof(float) + sizeof(float4) + sizeof(RowMeta));
-    rc = AllowLds(JoinerBackwardRowsKernel<Mode>, lds);
+    r.tpt = MT / a.R;
+    const size_t lds = (size_t)MT * (a.D + Mode::kPad + kNTile + Mode::kPad) * sizeof(Elem) +
+                       MT * (sizeof(float4) + sizeof(RowMeta));
+    auto kernel = a.D == kMaxD ? JoinerBackwardRowsKernel<Mode, RB, kMaxD> : JoinerBackwardRowsKernel<Mode, RB, 0>;
+    rc = AllowLds(kernel, lds);
     if (rc != K2AMD_OK) return rc;
     const long long tiles = (a.frames + r.tpt - 1) / r.tpt;
-    hipLaunchKernelGGL(JoinerBackwardRowsKernel<Mode>, dim3((unsigned)tiles), dim3(kThreads), lds, st, r);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)tiles), dim3(kThreads), lds, st, r);
   }
-  {  // gradients of weight and bias: slices of 64 columns x groups of tiles of 64 rows
+  {  // gradients of weight and bias: slices of columns x groups of tiles of 64 rows
+    constexpr int kSlice = kBf ? 128 : 64;
     JoinerArgs w = a;
     w.tpt = 64 / a.R;
     const size_t lds = (size_t)64 * (a.D + Mode::kPad) * sizeof(Elem) +
-                       (size_t)kSliceCols * (64 + Mode::kPad) * sizeof(Elem) +
+                       (size_t)kSlice * (64 + Mode::kPad) * sizeof(Elem) +
                        (kBf ? (size_t)a.D * (64 + Mode::kPad) * sizeof(Elem) : 0) +
                        64 * (sizeof(float4) + sizeof(RowMeta));
-    rc = AllowLds(JoinerBackwardWeightKernel<Mode>, lds);
+    auto kernel = a.D == kMaxD ? JoinerBackwardWeightKernel<Mode, kSlice, kMaxD>
+                               : JoinerBackwardWeightKernel<Mode, kSlice, 0>;
+    rc = AllowLds(kernel, lds);
     if (rc != K2AMD_OK) return rc;
     const long long tiles = (a.frames + w.tpt - 1) / w.tpt;
-    const int slices = a.Cpad / kSliceCols;
-    int groups = 512 / slices;
+    const int slices = a.Cpad / kSlice;
+    int groups = 256 / slices;  // one workgroup per compute unit
     if (groups < 1) groups = 1;
     if (groups > tiles) groups = (int)tiles;
-    hipLaunchKernelGGL(JoinerBackwardWeightKernel<Mode>, dim3((unsigned)(slices * groups)),
-                       dim3(kThreads), lds, st, w, (int)tiles, groups);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(slices * groups)), dim3(kThreads), lds, st, w, (int)tiles,
+                       groups);
   }
   return LaunchStatus();
 }
@@ -762,10 +955,10 @@ int k2amd_rnnt_joiner_pruned_forward(const void *am, const void *lm, const int64
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool bf = precision == K2AMD_JOINER_BF16;
   JoinerArgs a = MakeArgs((const float *)am, (const float *)lm, ranges, (const float *)bias, symbols,
-                          boundary, B, S, T, R, C, D, termination_symbol, rnnt_type, bf ? 128 : 64,
-                          workspace, precision);
+                          boundary, B, S, T, R, C, D, termination_symbol, rnnt_type, 64, workspace,
+                          precision);
   a.px = (float *)px; a.py = (float *)py; a.norm = (float *)normalizers;
-  return bf ? ForwardImpl<Bf16, 4>((const float *)weight, a, st)
+  return bf ? ForwardImpl<Bf16, 2>((const float *)weight, a, st)
             : ForwardImpl<F32, 2>((const float *)weight, a, st);
 }
 

@@ -337,3 +337,31 @@ def test_deprecated_ranges_invariants(modified):
                 t = 0
                 best = max(range(S + 2 - Reff), key=lambda s: (tot[b, s:s + Reff, t].sum(), -s))
                 assert s0[b, 0] == 0 or s0[b, 0] <= best
+
+
+def test_joiner_pruned_logits_against_torch_ops_and_loops():
+    """oracle.rnnt.joiner_pruned_logits is the joiner the reference's recipes put between
+    do_rnnt_pruning and rnnt_loss_pruned, tanh(am_pruned + lm_pruned) through a linear layer.  Pinned
+    by torch's own ops on the same numbers (torch.gather as in k2/python/k2/rnnt_loss.py:947-953,
+    torch.tanh, torch.nn.functional.linear) and by explicit loops on a tiny case."""
+    rng = np.random.default_rng(21)
+    B, T, S, R, D, C = 2, 7, 4, 3, 5, 6
+    am = rng.standard_normal((B, T, D))
+    lm = rng.standard_normal((B, S + 1, D))
+    weight = rng.standard_normal((C, D))
+    bias = rng.standard_normal(C)
+    start = np.sort(rng.integers(0, S + 2 - R, size=(B, T)), axis=1)
+    ranges = (start[:, :, None] + np.arange(R)).astype(np.int64)
+    got = orn.joiner_pruned_logits(am, lm, ranges, weight, bias)
+    tam, tlm, trg = torch.from_numpy(am), torch.from_numpy(lm), torch.from_numpy(ranges)
+    am_pruned = tam.unsqueeze(2).expand(B, T, R, D)
+    lm_pruned = torch.gather(tlm.unsqueeze(1).expand(B, T, S + 1, D), dim=2,
+                             index=trg.reshape(B, T, R, 1).expand(B, T, R, D))
+    want = torch.nn.functional.linear(torch.tanh(am_pruned + lm_pruned), torch.from_numpy(weight),
+                                      torch.from_numpy(bias)).numpy()
+    np.testing.assert_allclose(got, want, rtol=1e-12, atol=1e-12)
+    for b, t, k, c in itertools.product(range(B), range(T), range(R), range(C)):
+        z = bias[c] + sum(math.tanh(am[b, t, d] + lm[b, ranges[b, t, k], d]) * weight[c, d] for d in range(D))
+        assert abs(got[b, t, k, c] - z) < 1e-12
+    no_bias = orn.joiner_pruned_logits(am, lm, ranges, weight)
+    np.testing.assert_allclose(no_bias + bias, got, rtol=1e-12, atol=1e-12)
