@@ -182,6 +182,45 @@ __global__ void ScatterAddKernel(const T *__restrict__ grad, const int64_t *__re
   }
 }
 
+// The same sums without atomics, the terms of each one added in the order of (t, k): one workgroup
+// per lm row (b, s) lists the rows of grad that point at it (each thread looks at a contiguous
+// share of ranges[b], an exclusive scan over the threads' counts places its finds), then every
+// thread adds up its columns d over that list.  The result does not depend on the run.
+constexpr int kGatherThreads = 256;
+template <typename T>
+__global__ __launch_bounds__(kGatherThreads) void GatherBackwardKernel(
+    const T *__restrict__ grad, const int64_t *__restrict__ ranges, T *__restrict__ lm_grad, int S1,
+    int TR, int D) {
+  extern __shared__ int found[];  // [TR] row numbers, in order
+  __shared__ int counts[kGatherThreads + 1];
+  const int b = blockIdx.x / S1, s = blockIdx.x - b * S1;
+  const int64_t *r = ranges + (size_t)b * TR;
+  const int per = (TR + kGatherThreads - 1) / kGatherThreads;
+  const int lo = min((int)threadIdx.x * per, TR), hi = min(lo + per, TR);
+  int mine = 0;
+  for (int i = lo; i < hi; ++i) mine += r[i] == s;
+  counts[threadIdx.x + 1] = mine;
+  if (threadIdx.x == 0) counts[0] = 0;
+  __syncthreads();
+  for (int step = 1; step < kGatherThreads; step <<= 1) {  // inclusive scan of counts[1..]
+    const int add = (int)threadIdx.x + 1 > step ? counts[threadIdx.x + 1 - step] : 0;
+    __syncthreads();
+    counts[threadIdx.x + 1] += add;
+    __syncthreads();
+  }
+  int at = counts[threadIdx.x];
+  for (int i = lo; i < hi; ++i)
+    if (r[i] == s) found[at++] = i;
+  __syncthreads();
+  const int n = counts[kGatherThreads];
+  const T *g = grad + (size_t)b * TR * D;
+  for (int d = threadIdx.x; d < D; d += kGatherThreads) {
+    T sum = 0;
+    for (int j = 0; j < n; ++j) sum += g[(size_t)found[j] * D + d];
+    lm_grad[((size_t)b * S1 + s) * D + d] = sum;
+  }
+}
+
 unsigned GridFor(size_t n) {
   size_t blocks = (n + 255) / 256;
   return (unsigned)(blocks > 8192 ? 8192 : (blocks == 0 ? 1 : blocks));
@@ -235,6 +274,16 @@ int k2amd_rnnt_prune_gather_backward(const void *grad, const int64_t *ranges, vo
   hipStream_t st = static_cast<hipStream_t>(stream);
   const size_t n_out = (size_t)B * S1 * D, n = (size_t)B * T * R * D;
   if (n_out == 0) return K2AMD_OK;
+  const size_t list_bytes = (size_t)T * R * sizeof(int);
+  if (list_bytes <= 48 * 1024 && (long long)B * S1 < (1ll << 31) && (long long)T * R * D < (1ll << 31)) {
+    // the order-preserving kernel (a sequence's list of T * R row numbers fits its LDS)
+    const dim3 grid((unsigned)(B * S1)), block(kGatherThreads);
+    if (dtype == K2AMD_F32)
+      hipLaunchKernelGGL(GatherBackwardKernel<float>, grid, block, list_bytes, st, (const float *)grad, ranges, (float *)lm_grad, S1, T * R, D);
+    else
+      hipLaunchKernelGGL(GatherBackwardKernel<double>, grid, block, list_bytes, st, (const double *)grad, ranges, (double *)lm_grad, S1, T * R, D);
+    return LaunchStatus();
+  }
   if (dtype == K2AMD_F32) {
     hipLaunchKernelGGL(ZeroKernel<float>, dim3(GridFor(n_out)), dim3(256), 0, st, (float *)lm_grad, n_out);
     if (n) hipLaunchKernelGGL(ScatterAddKernel<float>, dim3(GridFor(n)), dim3(256), 0, st, (const float *)grad, ranges, (float *)lm_grad, S1, T * R, D, n);

@@ -141,6 +141,19 @@ def test_prune_gather_and_its_gradient(device):
         got_g = capi.prune_gather_backward(dev(g, device), dev(ranges, device), 11)
         np.testing.assert_allclose(got_g.cpu().numpy(), want_g, rtol=1e-5 if dtype == np.float32 else 1e-12,
                                    atol=1e-5 if dtype == np.float32 else 1e-12)
+    # config 3's shape (T * s_range = 2500 rows per sequence, D = 512): the sums are formed in the
+    # order of (t, k), so two runs give the same bits, and the result is that ordered sum exactly
+    B, T, S, R, D = 32, 500, 100, 5, 512
+    ranges = _random_ranges(rng, B, T, S, R)
+    g = rng.standard_normal((B, T, R, D)).astype(np.float32)
+    first = capi.prune_gather_backward(dev(g, device), dev(ranges, device), S + 1)
+    again = capi.prune_gather_backward(dev(g, device), dev(ranges, device), S + 1)
+    assert torch.equal(first, again)
+    want_g = np.zeros((B, S + 1, D), np.float32)
+    for t in range(T):
+        for k in range(R):   # the same order of additions, in fp32
+            want_g[np.arange(B), ranges[:, t, k]] += g[:, t, k]
+    assert np.array_equal(first.cpu().numpy(), want_g)
 
 
 @pytest.mark.parametrize("rnnt_type", TYPES)
