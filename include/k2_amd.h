@@ -248,9 +248,9 @@ K2AMD_API int k2amd_rnnt_prune_ranges(const void *px_grad, const void *py_grad,
 K2AMD_API int k2amd_rnnt_prune_gather(const void *lm, const int64_t *ranges, void *lm_pruned, int B,
                                       int S1, int T, int R, int D, int dtype, void *stream);
 /* Its gradient: lm_grad[b,s,:] = sum over (t,k) with ranges[b,t,k] == s of grad[b,t,k,:], every
- * element of lm_grad written.  The terms of a sum are added in the order of (t, k), so the result is
- * the same in every run, while T * R <= 12288; beyond that the sums are formed with floating-point
- * atomic adds and their last bits vary.                                                          */
+ * element of lm_grad written.  Which terms meet in which partial sum is fixed by ranges alone, so
+ * the result is the same in every run, while T * R <= 10240; beyond that the sums are formed with
+ * floating-point atomic adds and their last bits vary.                                           */
 K2AMD_API int k2amd_rnnt_prune_gather_backward(const void *grad, const int64_t *ranges,
                                                void *lm_grad, int B, int S1, int T, int R, int D,
                                                int dtype, void *stream);

@@ -182,16 +182,22 @@ __global__ void ScatterAddKernel(const T *__restrict__ grad, const int64_t *__re
   }
 }
 
-// The same sums without atomics, the terms of each one added in the order of (t, k): one workgroup
-// per lm row (b, s) lists the rows of grad that point at it (each thread looks at a contiguous
-// share of ranges[b], an exclusive scan over the threads' counts places its finds), then every
-// thread adds up its columns d over that list.  The result does not depend on the run.
+// The same sums without atomics and in a fixed order: one workgroup per lm row (b, s) lists the rows
+// of grad that point at it, in the order of (t, k) (each thread looks at a contiguous share of
+// ranges[b], an exclusive scan over the threads' counts places its finds).  The threads then split
+// into kParts groups; group p adds up rows p, p + kParts, .. of the list for its columns, with four
+// independent partial sums (rows j, j + kParts, j + 2 kParts, j + 3 kParts in flight together: a
+// frame-synchronous lattice sends hundreds of rows to the same s, and one chain of dependent loads
+// per column would take as long as the rest of the launch), and the groups' sums are added in order
+// through LDS.  Which terms meet in which partial sum depends only on the list: the same bits in
+// every run.
 constexpr int kGatherThreads = 256;
-template <typename T>
+template <typename T, int kVec>
 __global__ __launch_bounds__(kGatherThreads) void GatherBackwardKernel(
     const T *__restrict__ grad, const int64_t *__restrict__ ranges, T *__restrict__ lm_grad, int S1,
     int TR, int D) {
-  extern __shared__ int found[];  // [TR] row numbers, in order
+  extern __shared__ unsigned char gather_smem[];
+  int *found = reinterpret_cast<int *>(gather_smem);  // [TR] row numbers, in order
   __shared__ int counts[kGatherThreads + 1];
   const int b = blockIdx.x / S1, s = blockIdx.x - b * S1;
   const int64_t *r = ranges + (size_t)b * TR;
@@ -214,10 +220,48 @@ __global__ __launch_bounds__(kGatherThreads) void GatherBackwardKernel(
   __syncthreads();
   const int n = counts[kGatherThreads];
   const T *g = grad + (size_t)b * TR * D;
-  for (int d = threadIdx.x; d < D; d += kGatherThreads) {
-    T sum = 0;
-    for (int j = 0; j < n; ++j) sum += g[(size_t)found[j] * D + d];
-    lm_grad[((size_t)b * S1 + s) * D + d] = sum;
+  T *out = lm_grad + ((size_t)b * S1 + s) * D;
+  // groups of `width` threads, each thread kVec adjacent columns; the columns in passes of
+  // width * kVec where D is wider than that
+  const int groups_of = D / kVec;  // threads that cover a row once
+  const int width = groups_of < kGatherThreads ? groups_of : kGatherThreads;
+  const int parts = kGatherThreads / width, part = threadIdx.x / width, lane = threadIdx.x - part * width;
+  T *partial = reinterpret_cast<T *>(gather_smem + (((size_t)TR * sizeof(int) + 15) / 16) * 16);  // [parts][width * kVec]
+  for (int c0 = 0; c0 < D; c0 += width * kVec) {
+    const int c = c0 + lane * kVec;
+    T acc[4][kVec];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) acc[u][e] = 0;
+    if (part < parts && c < D) {
+      for (int j = part; j < n; j += 4 * parts) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int jj = j + u * parts;
+          if (jj < n) {
+            const T *src = g + (size_t)found[jj] * D + c;
+#pragma unroll
+            for (int e = 0; e < kVec; ++e) acc[u][e] += src[e];
+          }
+        }
+      }
+    }
+    if (part < parts && c < D) {
+#pragma unroll
+      for (int e = 0; e < kVec; ++e)
+        partial[(size_t)part * width * kVec + lane * kVec + e] = (acc[0][e] + acc[1][e]) + (acc[2][e] + acc[3][e]);
+    }
+    __syncthreads();
+    if (part == 0 && c < D) {
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) {
+        T sum = partial[lane * kVec + e];
+        for (int p = 1; p < parts; ++p) sum += partial[(size_t)p * width * kVec + lane * kVec + e];
+        out[c + e] = sum;
+      }
+    }
+    __syncthreads();
   }
 }
 
@@ -274,14 +318,20 @@ int k2amd_rnnt_prune_gather_backward(const void *grad, const int64_t *ranges, vo
   hipStream_t st = static_cast<hipStream_t>(stream);
   const size_t n_out = (size_t)B * S1 * D, n = (size_t)B * T * R * D;
   if (n_out == 0) return K2AMD_OK;
-  const size_t list_bytes = (size_t)T * R * sizeof(int);
-  if (list_bytes <= 48 * 1024 && (long long)B * S1 < (1ll << 31) && (long long)T * R * D < (1ll << 31)) {
+  const size_t list_bytes = (((size_t)T * R * sizeof(int) + 15) / 16) * 16;
+  if (list_bytes <= 40 * 1024 && D >= 1 && (long long)B * S1 < (1ll << 31) && (long long)T * R * D < (1ll << 31)) {
     // the order-preserving kernel (a sequence's list of T * R row numbers fits its LDS)
     const dim3 grid((unsigned)(B * S1)), block(kGatherThreads);
-    if (dtype == K2AMD_F32)
-      hipLaunchKernelGGL(GatherBackwardKernel<float>, grid, block, list_bytes, st, (const float *)grad, ranges, (float *)lm_grad, S1, T * R, D);
-    else
-      hipLaunchKernelGGL(GatherBackwardKernel<double>, grid, block, list_bytes, st, (const double *)grad, ranges, (double *)lm_grad, S1, T * R, D);
+    const bool vec = D % 4 == 0;  // 16-byte (fp32) / 32-byte (fp64) groups of columns per thread
+    const size_t esz = dtype == K2AMD_F32 ? 4 : 8;
+    const size_t smem = list_bytes + (size_t)kGatherThreads * (vec ? 4 : 1) * esz;
+    if (dtype == K2AMD_F32) {
+      if (vec) hipLaunchKernelGGL((GatherBackwardKernel<float, 4>), grid, block, smem, st, (const float *)grad, ranges, (float *)lm_grad, S1, T * R, D);
+      else hipLaunchKernelGGL((GatherBackwardKernel<float, 1>), grid, block, smem, st, (const float *)grad, ranges, (float *)lm_grad, S1, T * R, D);
+    } else {
+      if (vec) hipLaunchKernelGGL((GatherBackwardKernel<double, 4>), grid, block, smem, st, (const double *)grad, ranges, (double *)lm_grad, S1, T * R, D);
+      else hipLaunchKernelGGL((GatherBackwardKernel<double, 1>), grid, block, smem, st, (const double *)grad, ranges, (double *)lm_grad, S1, T * R, D);
+    }
     return LaunchStatus();
   }
   if (dtype == K2AMD_F32) {

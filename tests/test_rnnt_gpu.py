@@ -141,19 +141,26 @@ def test_prune_gather_and_its_gradient(device):
         got_g = capi.prune_gather_backward(dev(g, device), dev(ranges, device), 11)
         np.testing.assert_allclose(got_g.cpu().numpy(), want_g, rtol=1e-5 if dtype == np.float32 else 1e-12,
                                    atol=1e-5 if dtype == np.float32 else 1e-12)
-    # config 3's shape (T * s_range = 2500 rows per sequence, D = 512): the sums are formed in the
-    # order of (t, k), so two runs give the same bits, and the result is that ordered sum exactly
+    # config 3's shape (T * s_range = 2500 rows per sequence, D = 512), with ranges that stay on one
+    # row for many frames as a real lattice's do: the order of the additions is fixed by ranges, so
+    # two runs give the same bits
     B, T, S, R, D = 32, 500, 100, 5, 512
     ranges = _random_ranges(rng, B, T, S, R)
+    ranges[: B // 2, : T // 2] = np.arange(R)       # 250 frames of 16 sequences on rows 0..4
     g = rng.standard_normal((B, T, R, D)).astype(np.float32)
     first = capi.prune_gather_backward(dev(g, device), dev(ranges, device), S + 1)
     again = capi.prune_gather_backward(dev(g, device), dev(ranges, device), S + 1)
     assert torch.equal(first, again)
-    want_g = np.zeros((B, S + 1, D), np.float32)
-    for t in range(T):
-        for k in range(R):   # the same order of additions, in fp32
-            want_g[np.arange(B), ranges[:, t, k]] += g[:, t, k]
-    assert np.array_equal(first.cpu().numpy(), want_g)
+    want_g = np.zeros((B, S + 1, D), np.float64)
+    np.add.at(want_g, (np.arange(B)[:, None, None], ranges), g.astype(np.float64))
+    np.testing.assert_allclose(first.cpu().numpy(), want_g, rtol=1e-5, atol=1e-4)
+    for D in (1, 6, 36, 1100):                       # columns that are no multiple of four; more than 1024
+        ranges = _random_ranges(rng, 2, 9, 5, 3)
+        g = rng.standard_normal((2, 9, 3, D))
+        want_g = np.zeros((2, 6, D))
+        np.add.at(want_g, (np.arange(2)[:, None, None], ranges), g)
+        got_g = capi.prune_gather_backward(dev(g, device), dev(ranges, device), 6)
+        np.testing.assert_allclose(got_g.cpu().numpy(), want_g, rtol=1e-12, atol=1e-12)
 
 
 @pytest.mark.parametrize("rnnt_type", TYPES)
