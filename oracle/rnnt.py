@@ -6,29 +6,28 @@ the inputs (fp32 stays fp32) and in the reference's order of operations where th
 visible in its source; reductions inside numpy (``max``, ``sum``, ``matmul``) may round
 differently from torch's, which is within the stated float tolerances.
 
-Parity status
-  * ``logprobs_simple`` / ``logprobs_joint`` / ``logprobs_pruned``: pinned by the hand fixture of
-    k2/python/tests/rnnt_loss_test.py:127-139 through brute-force enumeration of its
-    alignments, by the identities the reference tests assert (simple == joint on am+lm,
-    invariance to per-frame constants) and by the no-pruning identity (s_range = S+1 gives
-    the joint loss).  The reference's tests hold no numeric golden values for them.
-  * ``roll_by_shifts``, ``monotonic_lower_bound``: pinned by the doc-test vectors at
+Parity status: every function below is pinned.
+  * By what the reference's OWN Python chain computes: tests/golden/rnnt_ref_fixtures.npz, written
+    by tests/golden/make_rnnt_fixtures.py from k2/python/k2/rnnt_loss.py and mutual_information.py
+    loaded by path over the reference's compiled CPU recursion (whole chains simple loss ->
+    gradients -> prune ranges -> pruning -> pruned log-probs -> pruned loss for the three lattice
+    types, delay penalty, HAT, smoothed, deprecated ranges; cases around arg-max ties and around
+    the ``+ tiny`` floor).  tests/test_oracle_rnnt_fixtures.py: integers bit for bit, floats to
+    the stated tolerances.  (That comparison is why ``prune_ranges_deprecated`` accumulates its
+    cumulative sums in float64: torch's CPU cumsum does.)
+  * ``logprobs_simple`` / ``logprobs_joint`` / ``logprobs_pruned`` also by the hand fixture of
+    k2/python/tests/rnnt_loss_test.py:127-139 through brute-force enumeration of its alignments,
+    by the identities the reference tests assert (simple == joint on am+lm, invariance to
+    per-frame constants) and by the no-pruning identity (s_range = S+1 gives the joint loss).
+  * ``apply_delay_penalty`` also by brute force over alignments with the per-symbol term.
+  * ``roll_by_shifts``, ``monotonic_lower_bound`` also by the doc-test vectors at
     k2/python/k2/rnnt_loss.py:965-976 and :551-565.
-  * ``prune_ranges``: integer part pinned by those vectors and by the invariants stated at
-    k2/python/k2/rnnt_loss.py:583-589; the reference's own tests only print its output
-    (k2/python/tests/rnnt_loss_test.py:735-760), so its values are **parity unpinned** by
-    the reference's tests; tests here additionally compare against torch.sum/argmax on CPU.
-
-  * ``hat_logprobs_pruned``: pinned by the probability identity of the model it states
-    (exp(py) + sum over symbols of exp(px-like terms) = 1 for every row), by direct
-    probability-space evaluation (sigmoid and softmax computed in fp64) and by reduction to
-    ``logprobs_pruned`` when column 0 is pushed to -inf; the reference's test only prints its
-    loss (k2/python/tests/rnnt_loss_test.py:859-925): **parity unpinned** by the reference.
-  * ``logprobs_smoothed``: pinned by the identity the reference tests assert (both scales 0
-    gives rnnt_loss_simple, k2/python/tests/rnnt_loss_test.py:167-178) and invariance to
-    per-frame constants (:436-485), plus direct evaluation of the three normalised
-    distributions on tiny inputs.
-  * ``prune_ranges_deprecated``: restated from the source; invariants only: **parity unpinned**.
+  * ``hat_logprobs_pruned`` also by the probability identity of the model, by direct
+    probability-space evaluation and by reduction to ``logprobs_pruned``.
+  * ``logprobs_smoothed`` also by the identity the reference tests assert (both scales 0 gives
+    rnnt_loss_simple, k2/python/tests/rnnt_loss_test.py:167-178) and shift invariance (:436-485).
+  * ``joiner_pruned_logits`` (the step the reference leaves to the caller) by torch's own gather /
+    tanh / linear on the same numbers and by explicit loops.
 
 Only tests, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` may import this.
 """
