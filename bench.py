@@ -11,7 +11,8 @@ Prints ONE JSON line.  `value` counts ACTIVE lattice cells, sum_b (S_b+1)(T_b+1)
 fwd+bwd wall time on the GPU; `roofline` prices the step's kernel (the slower of the two where
 two launches are asked for) against the HBM peak with its algorithmic bytes; `cache_resident` is
 the same measurement with one copy of the inputs; `cpu_baseline` is the reference's CPU loop on
-this host.
+this host.  `secondary`, `other_configs` and `fused_joiner` are further workloads through the Python
+API (configs 3, 2, 5, and config 3's shape with the joiner inside the loss), none of them `value`.
 """
 import argparse
 import json
