@@ -48,8 +48,10 @@ K2AMD_API const char *k2amd_status_string(int status);
  *   boundary [B][4] int64 = (s_begin, t_begin, s_end, t_end) or NULL for (0,0,S,T)
  *   ans, ans_grad [B]
  *
- * Workspace (fp32 throughput path): k2amd_mi_workspace_bytes() tells how many bytes of device
- * scratch the pipelined kernels want for a shape (0 for fp64).  The caller owns the buffer and
+ * Workspace (throughput paths): k2amd_mi_workspace_bytes() tells how many bytes of device
+ * scratch the pipelined kernels want for a shape and dtype (fp32: chunks of 64 rows as workgroups
+ * of specialised wavefronts; fp64: one wavefront per chunk; 0 = no pipelined kernel serves the
+ * shape).  The layout and the initial state are the same for both.  The caller owns the buffer and
  * must run k2amd_mi_workspace_init() on it ONCE before its first use (and again after a
  * K2AMD_ERR_TIMEOUT); the kernels leave it ready for the next call, so a buffer sized for the
  * largest shape can be reused for any smaller one.  One workspace serves one stream at a time.
@@ -79,8 +81,7 @@ K2AMD_API int k2amd_mi_forward(const void *px, const void *py, const int64_t *bo
  * library (each GPU the library runs on holds its own copy until the process ends); the call
  * itself allocates and frees nothing and synchronises nothing.  A shape whose
  * k2amd_mi_workspace_bytes(...) exceeds that size is refused with K2AMD_ERR_SCRATCH_LIMIT (the
- * headline shape B=32, S=200, T=1000 needs 1.45 MB).  fp64 runs the exact kernels, which use no
- * scratch.  Every call re-initialises the part of the array it uses with a fill kernel in front of
+ * headline shape B=32, S=200, T=1000 needs 1.5 MB in fp32, 1.4 MB in fp64).  Every call re-initialises the part of the array it uses with a fill kernel in front of
  * the recursion, so a call never inherits anything from the one before it.  All calls on one GPU
  * share that GPU's array: calls that overlap in time on one GPU (two streams, two threads) race
  * and must be serialised by the caller.  The first call on a device looks up the array's address;

@@ -70,7 +70,9 @@ const char *k2amd_status_string(int status) {
 
 size_t k2amd_mi_workspace_bytes(int B, int S, int T, int modified, int dtype) {
   (void)modified;
-  if (dtype != K2AMD_F32 || !ShapeOk(B, S, T) || B == 0) return 0;
+  if (!ShapeOk(B, S, T) || B == 0) return 0;
+  if (dtype == K2AMD_F64) return MiWaveSupports(B, S, T) ? MiWaveWorkspaceBytes(B, S, T) : 0;
+  if (dtype != K2AMD_F32) return 0;
   return MiFastWorkspaceBytes(B, S, T);
 }
 
@@ -121,6 +123,12 @@ int k2amd_mi_forward_keep(const void *px, const void *py, const int64_t *boundar
   if (dtype == K2AMD_F32)
     return MiForwardGeneric<float>((const float *)px, (const float *)py, boundary, (float *)p,
                                    (float *)ans, B, S, T, modified, st);
+  // fp64 with a workspace: one wavefront per 64-row chunk, pipelined
+  if (workspace != nullptr && !ForceGeneric() && MiWaveSupports(B, S, T)) {
+    if (workspace_bytes < MiWaveWorkspaceBytes(B, S, T)) return K2AMD_ERR_WORKSPACE;
+    return MiForwardWave((const double *)px, (const double *)py, boundary, (double *)p, (double *)ans,
+                         B, S, T, modified, workspace, workspace_bytes, st);
+  }
   return MiForwardGeneric<double>((const double *)px, (const double *)py, boundary, (double *)p,
                                   (double *)ans, B, S, T, modified, st);
 }
@@ -179,6 +187,12 @@ int k2amd_mi_backward_kept(const void *px, const void *py, const int64_t *bounda
     return MiBackwardGeneric<float>((const float *)px, (const float *)p, boundary,
                                     (float *)ans_grad, (float *)px_grad, (float *)py_grad, B, S, T,
                                     modified, overwrite_ans_grad, st);
+  if (dtype == K2AMD_F64 && workspace != nullptr && !ForceGeneric() && MiWaveSupports(B, S, T)) {
+    if (workspace_bytes < MiWaveWorkspaceBytes(B, S, T)) return K2AMD_ERR_WORKSPACE;
+    return MiBackwardWave((const double *)px, (const double *)p, boundary, (double *)ans_grad,
+                          (double *)px_grad, (double *)py_grad, B, S, T, modified, overwrite_ans_grad,
+                          workspace, workspace_bytes, st);
+  }
   return MiBackwardGeneric<double>((const double *)px, (const double *)p, boundary,
                                    (double *)ans_grad, (double *)px_grad, (double *)py_grad, B, S,
                                    T, modified, overwrite_ans_grad, st);

@@ -44,6 +44,17 @@ int MiForwardBackwardFast(const float *px, const float *py, const int64_t *bound
                           int S, int Tn, int modified, int overwrite_ans_grad, void *workspace,
                           size_t workspace_bytes, hipStream_t stream);
 
+// fp64 throughput path: pipelined 64-row chunks, one wavefront per chunk (mi_wave.hip); the
+// workspace has the layout and the initial state of the fp32 one (MiFastWorkspaceInit).
+bool MiWaveSupports(int B, int S, int Tn);
+size_t MiWaveWorkspaceBytes(int B, int S, int Tn);
+int MiForwardWave(const double *px, const double *py, const int64_t *boundary, double *p, double *ans,
+                  int B, int S, int Tn, int modified, void *workspace, size_t workspace_bytes,
+                  hipStream_t stream);
+int MiBackwardWave(const double *px, const double *p, const int64_t *boundary, double *ans_grad,
+                   double *px_grad, double *py_grad, int B, int S, int Tn, int modified,
+                   int overwrite_ans_grad, void *workspace, size_t workspace_bytes, hipStream_t stream);
+
 }  // namespace k2amd
 
 #endif  // K2_AMD_CSRC_MI_INTERNAL_H_

@@ -531,3 +531,36 @@ def test_single_launches_on_two_streams(device):
         for o in outs[i]:
             for a, b in zip(o, ref):
                 assert torch.equal(a, b)
+
+
+@pytest.mark.gpu
+def test_fp64_headline_shape_on_the_wave_kernels(device, monkeypatch):
+    """fp64 with a workspace takes the kernels of mi_wave.hip (one wavefront per 64-row chunk,
+    pipelined): at BASELINE config 4's shape within 1e-10 of the fp64 oracle, like the exact
+    one-workgroup-per-sequence kernels, which K2AMD_MI_PATH=generic still selects; and on shapes
+    that put chunk borders, the 32-word hand-over blocks and the column clamps at their edges."""
+    from k2_amd import capi
+    c = cases.c4_case(dtype=np.float64)
+    assert capi.lib().k2amd_mi_workspace_bytes(32, 200, 1000, 1, capi.F64) > 0
+
+    def against_oracle(name, px, py, bd):
+        ans, p = omi.mi_forward(px, py, bd)
+        gx, gy = omi.mi_backward(px, py, bd, p)
+        check(name, px, py, bd, (ans, p, gx, gy), device)
+
+    against_oracle("c4 fp64", c["px"], c["py"], c["boundary"])
+    monkeypatch.setenv("K2AMD_MI_PATH", "generic")
+    against_oracle("c4 fp64, exact kernels", c["px"], c["py"], c["boundary"])
+    monkeypatch.delenv("K2AMD_MI_PATH")
+    rng = np.random.default_rng(64)
+    for modified in (False, True):
+        for B, S, T in ((3, 63, 40), (2, 64, 33), (2, 130, 70), (1, 0, 5), (2, 5, 5), (2, 200, 31),
+                        (1, 65, 32), (2, 127, 129), (1, 1, 1)):
+            if modified and T < S:
+                continue
+            T1 = T if modified else T + 1
+            px = rng.standard_normal((B, S, T1))
+            py = rng.standard_normal((B, S + 1, T))
+            bd = cases.random_boundary(rng, B, S, T, modified)
+            for boundary in (None, bd):
+                against_oracle(f"modified={modified} B={B} S={S} T={T} bd={boundary is not None}", px, py, boundary)

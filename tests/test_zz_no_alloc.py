@@ -42,7 +42,7 @@ def test_noalloc_forward_equals_the_workspace_entry_point(device):
     small = cases.mi_case(5003, dtype=np.float32, max_B=5, max_S=130, max_T=150,
                           force=dict(modified=False, rand_bd=True))
     _both(small, device)
-    _both(cases.mi_case(77, dtype=np.float64, max_B=3, max_S=20, max_T=40), device)   # exact kernels, no scratch
+    _both(cases.mi_case(77, dtype=np.float64, max_B=3, max_S=20, max_T=40), device)   # the fp64 kernels, same array
     _both(big, device)
     # beyond the static array: refused with its own status, nothing launched
     lib = capi.lib()
