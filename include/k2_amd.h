@@ -270,8 +270,8 @@ K2AMD_API int k2amd_rnnt_prune_gather_backward(const void *grad, const int64_t *
  *   precision: K2AMD_JOINER_F32 multiplies in fp32 on the matrix cores; K2AMD_JOINER_BF16 rounds the
  *   activations, the weight and the logits' gradients to bfloat16 for the products (fp32 sums).
  *   workspace: k2amd_rnnt_joiner_pruned_workspace_bytes(...) bytes of device memory (0 = shape
- *   not served: D a multiple of 64 up to 512, R <= 32; K2AMD_ERR_UNSUPPORTED also where C is too
- *   large for the backward's tiles); contents need not survive between the two calls.
+ *   not served: D a multiple of 64 up to 512, R <= 32 and <= S + 1; any C); contents need not
+ *   survive between the two calls.
  * The backward takes what the forward took, the normalizers it wrote and the gradients w.r.t. its
  * px / py (seq_scale as for the other builders), and writes am_grad [B][T][D], lm_grad [B][S+1][D],
  * weight_grad [C][D], bias_grad [C] (or NULL).  lm_grad, weight_grad and bias_grad are sums formed

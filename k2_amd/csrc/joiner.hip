@@ -46,21 +46,18 @@ struct Frag {
 __device__ __forceinline__ float AsFloat(unsigned u) { return __builtin_bit_cast(float, u); }
 __device__ __forceinline__ unsigned AsBits(float f) { return __builtin_bit_cast(unsigned, f); }
 
-// round to nearest even; NaN stays NaN
+// float -> bfloat16, round to nearest even (the hardware's conversion)
 __device__ __forceinline__ unsigned short ToBf16(float f) {
-  unsigned u = AsBits(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (unsigned short)(u >> 16);
+  return __builtin_bit_cast(unsigned short, static_cast<__bf16>(f));
 }
 __device__ __forceinline__ float FromBf16(unsigned short h) { return AsFloat((unsigned)h << 16); }
 
-// tanh(x) = sign(x) (1 - e) / (1 + e), e = exp(-2|x|): absolute error ~1e-7, which is what the
-// logits (sums of D such values times weights) are sensitive to.
+// tanh(x) = 1 - 2 / (1 + exp(2 x)): five instructions (the exponential saturates to 0 or inf at
+// the ends, which gives -1 and 1); absolute error ~1e-7, which is what the logits (sums of D such
+// values times weights) are sensitive to.
 __device__ __forceinline__ float Tanh(float x) {
-  const float e = __expf(-2.0f * fabsf(x));
-  const float t = (1.0f - e) * __builtin_amdgcn_rcpf(1.0f + e);  // 1 + e in [1, 2]: rcp is good to 1 ulp
-  return x < 0 ? -t : t;
+  const float e = __builtin_amdgcn_exp2f(x * 2.8853900817779268f);  // exp(2 x)
+  return fmaf(-2.0f, __builtin_amdgcn_rcpf(1.0f + e), 1.0f);
 }
 
 struct F32 {
@@ -235,6 +232,53 @@ __device__ __forceinline__ void StageActivations(const JoinerArgs &a, const RowM
         ht[(size_t)(4 * q + 2) * ldt + m] = Mode::From(v.z);
         ht[(size_t)(4 * q + 3) * ldt + m] = Mode::From(v.w);
       }
+    }
+  }
+}
+
+// The same for the weight gradient in bfloat16, which also wants the activations transposed,
+// ht[d][m] (k = row contiguous).  An item is four adjacent columns of four adjacent rows: the
+// transposed copy is then written eight bytes at a time (four rows of one column) instead of one
+// two-byte store per element, whose lanes fell sixteen to an LDS bank.  Consecutive threads take
+// consecutive groups of rows first, so that those stores of a wavefront are contiguous.
+template <typename Mode, int MT>
+__device__ __forceinline__ void StageActivationsBoth(const JoinerArgs &a, const RowMeta *meta, int rows,
+                                                     typename Mode::Elem *h, int ldh,
+                                                     typename Mode::Elem *ht, int ldt) {
+  static_assert(sizeof(typename Mode::Elem) == 2, "bfloat16 tiles");
+  constexpr int kGroups = MT / 4;
+  const int qpr = a.D >> 2, items = kGroups * qpr;
+  for (int it = threadIdx.x; it < items; it += kThreads) {
+    const int mg = it % kGroups, q = it / kGroups;
+    float4 x[4], y[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int m = mg * 4 + r;
+      x[r] = make_float4(0.f, 0.f, 0.f, 0.f);
+      y[r] = x[r];
+      if (m < rows) {
+        const RowMeta rm = meta[m];
+        x[r] = *reinterpret_cast<const float4 *>(a.am + (size_t)rm.bt * a.D + 4 * q);
+        y[r] = *reinterpret_cast<const float4 *>(a.lm + (size_t)rm.lmrow * a.D + 4 * q);
+      }
+    }
+    unsigned short t[4][4];  // [row][column]
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float4 v = make_float4(Tanh(x[r].x + y[r].x), Tanh(x[r].y + y[r].y), Tanh(x[r].z + y[r].z),
+                                   Tanh(x[r].w + y[r].w));
+      t[r][0] = ToBf16(v.x); t[r][1] = ToBf16(v.y); t[r][2] = ToBf16(v.z); t[r][3] = ToBf16(v.w);
+      uint2 row;
+      row.x = (unsigned)t[r][0] | ((unsigned)t[r][1] << 16);
+      row.y = (unsigned)t[r][2] | ((unsigned)t[r][3] << 16);
+      *reinterpret_cast<uint2 *>(h + (size_t)(mg * 4 + r) * ldh + 4 * q) = row;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      uint2 colv;
+      colv.x = (unsigned)t[0][e] | ((unsigned)t[1][e] << 16);
+      colv.y = (unsigned)t[2][e] | ((unsigned)t[3][e] << 16);
+      *reinterpret_cast<uint2 *>(ht + (size_t)(4 * q + e) * ldt + mg * 4) = colv;
     }
   }
 }
@@ -623,7 +667,8 @@ __global__ __launch_bounds__(kThreads) void JoinerBackwardWeightKernel(const Joi
     for (int m = threadIdx.x; m < MT; m += kThreads)
       hdr[m] = m < rows ? a.hdr[(size_t)f0 * a.R + m] : make_float4(0.f, 0.f, -1.f, 3.0e38f);  // padding: exp(. - norm) = 0
     __syncthreads();
-    StageActivations<Mode, MT, kBf, kBf ? 4 : 2>(a, meta, rows, h, ldh, ht, ldt);
+    if constexpr (kBf) StageActivationsBoth<Mode, MT>(a, meta, rows, h, ldh, ht, ldt);
+    else StageActivations<Mode, MT, false, 2>(a, meta, rows, h, ldh, nullptr, 0);
     __syncthreads();
     Acc16 acc[1];
 #pragma unroll

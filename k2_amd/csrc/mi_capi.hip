@@ -113,8 +113,8 @@ int k2amd_mi_forward_keep(const void *px, const void *py, const int64_t *boundar
   const bool fast = dtype == K2AMD_F32 && workspace != nullptr && !ForceGeneric() && MiFastSupports(B, S, T, modified);
   // p may be left out only where the log-derivative tensor stands in for it
   if (!p && !(fast && log_deriv)) return K2AMD_ERR_INVALID_ARGUMENT;
-  // fp32 with a workspace takes the pipelined throughput path; without one (or for fp64) the
-  // exact one-workgroup-per-sequence kernels run.
+  // fp32 with a workspace takes the pipelined throughput path (fp64 has its own, further down);
+  // without a workspace the exact one-workgroup-per-sequence kernels run.
   if (fast) {
     if (workspace_bytes < MiFastWorkspaceBytes(B, S, T)) return K2AMD_ERR_WORKSPACE;
     return MiForwardFast((const float *)px, (const float *)py, boundary, (float *)p, (float *)ans,

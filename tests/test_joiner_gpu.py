@@ -107,6 +107,7 @@ SMALL = [  # seed, B, T, S, C, D, R, bias
     (3, 1, 70, 30, 500, 192, 4, True),   # C = 500 as in the configs; D not a multiple of 128
     (4, 4, 33, 6, 64, 320, 2, True),     # smallest window
     (5, 2, 50, 20, 257, 512, 7, True),   # largest D; R does not divide the tile rows
+    (6, 1, 30, 12, 700, 64, 4, True),    # three tiles of 256 columns, smallest D
 ]
 
 

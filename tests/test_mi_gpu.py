@@ -359,8 +359,8 @@ def test_joint_recursion_identities(device, dtype):
 
 @pytest.mark.gpu
 def test_log_deriv_is_left_alone_by_the_exact_kernels(device):
-    """fp64 (and fp32 without a workspace) run the one-workgroup-per-sequence kernels, which
-    neither write nor read the log-derivative tensor: the hosts say so and results are unchanged."""
+    """The fp64 kernels (and the exact kernels that run without a workspace) neither write nor read
+    the log-derivative tensor: the hosts say so and results are unchanged."""
     from k2_amd import capi
     rng = np.random.default_rng(3)
     B, S, T = 2, 12, 30
