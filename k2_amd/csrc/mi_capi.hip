@@ -212,7 +212,7 @@ int k2amd_mi_forward_backward_advised(int B, int S, int T, int modified, int dty
 
 size_t k2amd_mi_forward_backward_scratch_bytes(int B, int S, int T, int modified, int dtype) {
   if (!k2amd_mi_forward_backward_supported(B, S, T, modified, dtype, 1)) return 0;
-  return MiFusedScratchElems(B, S, T) * sizeof(float);
+  return MiFusedScratchElems(B, S, T, modified ? 1 : 0) * sizeof(float);
 }
 
 int k2amd_mi_forward_backward(const void *px, const void *py, const int64_t *boundary, void *ans,

@@ -253,6 +253,24 @@ struct Half {
 #define K2AMD_TRACE_MARK(half, i) do { } while (0)
 #endif
 
+// The single launch keeps the log-derivatives of every half-sweep in a slab of its own, laid out
+// the way they are produced and consumed: per (sequence, half, chunk) a run of 32-position blocks,
+// each 64 rows x 32 positions of the half's own coordinates.  A wavefront's 16-byte accesses then
+// cover 1 KB of consecutive bytes and every 128-byte line is written whole, by one instruction
+// (rows of a [S + 1][T + 2] array would put 128-byte runs 4 KB apart, straddling two lines each,
+// which device-coherent stores send to memory as the partial lines they are).
+// Blocks a chunk of a half can have: its positions end one past the cut diagonal, and the cut
+// lies half way along the lattice's longest path.
+constexpr int kSlabBlockFloats = kRows * kW;
+__host__ __device__ inline int SlabBlocks(int S, int Tn, int modified) {
+  const int diagonals = Tn + (modified ? 0 : S);
+  return (diagonals - diagonals / 2 + 2 + kW - 1) / kW;
+}
+__host__ __device__ inline size_t SlabFloatsPerSequence(int S, int Tn, int modified) {
+  const int nchunks = (S + 1 + kRows - 1) / kRows;
+  return 2 * (size_t)nchunks * SlabBlocks(S, Tn, modified) * kSlabBlockFloats;
+}
+
 __device__ __forceinline__ float4 Rev4(float4 v) { return make_float4(v.w, v.z, v.y, v.x); }
 
 enum Role { kChain = 0, kEdge = 1, kLoader = 2, kStorer = 3 };
@@ -429,11 +447,15 @@ __device__ __forceinline__ void MiForwardChunk(
   const int edge_shift = kRows * g.skew - 1;  // step n here <-> step n + edge_shift one chunk up
 
   const int T1 = modified ? Tn : Tn + 1;
-  const int LS = kBidir ? Tn + 2 : Tn + 1;  // floats per row of log_deriv
+  const int LS = Tn + 1;  // floats per row of log_deriv (the two-kernel pair's tensor)
   const float *pxb = px + (size_t)g.b * S * T1;
   const float *pyb = py + (size_t)g.b * (S + 1) * Tn;
   float *pb = kWriteP ? p + (size_t)g.b * (S + 1) * (Tn + 1) : nullptr;
-  float *ldb = kKeep ? log_deriv + (size_t)g.b * (S + 1) * LS : nullptr;
+  // (kBidir: the run of blocks of this chunk of this half in the launch's slab)
+  float *ldb = !kKeep ? nullptr
+               : kBidir ? log_deriv + (size_t)g.b * SlabFloatsPerSequence(S, Tn, modified) +
+                              (size_t)(mirror * nchunks + g.c) * SlabBlocks(S, Tn, modified) * kSlabBlockFloats
+                        : log_deriv + (size_t)g.b * (S + 1) * LS;
   float *edge_out = edge + ((size_t)g.b * nchunks + g.c + 1) * edge_stride;  // read by chunk c+1
   float *edge_in = edge + ((size_t)g.b * nchunks + g.c) * edge_stride;
 
@@ -580,8 +602,7 @@ __device__ __forceinline__ void MiForwardChunk(
       const int j = kb * kW + 4 * mm - q * g.skew;  // column of element 0
       // where own columns j .. j+3 of the row lie: the mirrored half stores the lattice's cell
       // (ns - row, nt - column) one column to the right of its place, columns descending
-      const ptrdiff_t at = mirror ? (ptrdiff_t)(g.s0 + g.ns - row_i) * LS + g.t0 + g.nt - j - 2
-                                  : (ptrdiff_t)(g.s0 + row_i) * LS + g.t0 + j;
+      const ptrdiff_t at = (ptrdiff_t)(g.s0 + row_i) * LS + g.t0 + j;
       float *dst = pb + at;
       float ld[4] = {0.f, 0.f, 0.f, 0.f};
       if (kKeep) {
@@ -615,24 +636,22 @@ __device__ __forceinline__ void MiForwardChunk(
           ld[e] = t1[e] - (__builtin_fabsf(own[e]) < -kLogZeroTest ? own[e] : 0.0f);
         if (mm == kQuadsPerBlock - 1) lds.last[kb % 3][q] = raw.w;
       }
-      if (inner) {  // uniform: every column of the block lies in 0..nt-1 for every row
+      if (kBidir) {
+        // Whole quads in the half's own order, also where the block reaches outside the box or
+        // past the cut: the backward sweep decides by position what it uses.
+        StoreQuadCoherent(ldb + (size_t)kb * kSlabBlockFloats + q * kW + 4 * mm,
+                          make_float4(ld[0], ld[1], ld[2], ld[3]));
+      } else if (inner) {  // uniform: every column of the block lies in 0..nt-1 for every row
         if (kWriteP) StoreQuad(dst, v);
-        if (kKeep) {
-          const float4 l4 = make_float4(ld[0], ld[1], ld[2], ld[3]);
-          if (kBidir) StoreQuadCoherent(ldb + at, mirror ? Rev4(l4) : l4);
-          else StoreQuad(ldb + at, l4);
-        }
+        if (kKeep) StoreQuad(ldb + at, make_float4(ld[0], ld[1], ld[2], ld[3]));
       } else {
         asm volatile("");  // keeps this path a branch of its own
         const float vv[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          if (j + e >= 0 && j + e <= g.nt && (!kBidir || j + e + q * g.skew <= n_last)) {
+          if (j + e >= 0 && j + e <= g.nt) {
             if (kWriteP) dst[e] = vv[e];
-            if (kKeep) {
-              if (kBidir) StoreCoherent(ldb + at + (mirror ? 3 - e : e), ld[e]);
-              else ldb[at + e] = ld[e];
-            }
+            if (kKeep) ldb[at + e] = ld[e];
           }
         if (!kBidir && row_i == g.ns) {
 #pragma unroll
@@ -949,7 +968,7 @@ __device__ __forceinline__ void MiBackwardChunk(
   const bool has_up = g.c > 0;
   const int nblocks_down = has_down ? blocks_of(g.row0 + kRows) : 0;
   const int nblocks_up = has_up ? blocks_of(g.row0 - kRows) : 0;
-  const int LS = kBidir ? Tn + 2 : Tn + 1;  // floats per row of p / the log-derivatives
+  const int LS = Tn + 1;  // floats per row of p / the log-derivatives (the two-kernel pair's tensors)
   const int edge_shift = kRows * g.skew;  // position m here <-> position m - edge_shift one chunk down
   float *edge_out = edge + ((size_t)g.b * nchunks + g.c) * edge_stride;     // read by chunk c-1
   float *edge_in = edge + ((size_t)g.b * nchunks + g.c + 1) * edge_stride;  // from chunk c+1
@@ -964,7 +983,12 @@ __device__ __forceinline__ void MiBackwardChunk(
 
   // ---- loaders ---------------------------------------------------------------------------
   // destination cells with both edges exist only for rows 1..ns and columns 1..nt
-  const int4v rsp = MakeResource(p, (size_t)B * (S + 1) * LS);
+  // (kBidir: `p` is the launch's slab, and this chunk of this half has a run of blocks in it)
+  const int slab_blocks = SlabBlocks(S, Tn, modified);
+  const int4v rsp = kBidir ? MakeResource(p + (size_t)g.b * SlabFloatsPerSequence(S, Tn, modified) +
+                                              (size_t)(mirror * nchunks + g.c) * slab_blocks * kSlabBlockFloats,
+                                          (size_t)slab_blocks * kSlabBlockFloats)
+                           : MakeResource(p, (size_t)B * (S + 1) * LS);
   const int4v rsx = MakeResource(px, (size_t)B * S * T1);
   // float index of destination column 0 of the item's row: p[dest], and p / px of the source
   // cell of the px edge (column jd - 1 + skew of the row above)
@@ -972,16 +996,11 @@ __device__ __forceinline__ void MiBackwardChunk(
 #pragma unroll
   for (int it = 0; it < kLoadItems; ++it) {
     const int rc = min(max(g.row0 + lq + kRowStep * it, 1), max(g.ns, 1));  // a row with a row above
-    // the mirrored half's cell (row, column) lies at lattice cell (ns - row, nt - column), one
-    // column to the right: own column c of the row is at index idx - c
-    idx_d[it] = mirror ? (g.b * (S + 1) + g.s0 + g.ns - rc) * LS + g.t0 + g.nt + 1
-                       : (g.b * (S + 1) + g.s0 + rc) * LS + g.t0;
+    // (kBidir: the item's row inside a block of the slab)
+    idx_d[it] = kBidir ? (lq + kRowStep * it) * kW : (g.b * (S + 1) + g.s0 + rc) * LS + g.t0;
     idx_s[it] = (g.b * (S + 1) + g.s0 + rc - 1) * (Tn + 1) + g.t0 + g.skew - 1;
     idx_x[it] = (g.b * S + g.s0 + rc - 1) * T1 + g.t0 + g.skew - 1;
   }
-  // index of the quad that holds own columns c .. c+3 of a row whose column 0 is at idx (mirrored:
-  // the quad comes back in descending column order)
-  auto quad_at = [&](int idx, int c) { return mirror ? idx - c - 3 : idx + c; };
   // every destination cell of block kb has both edges inside the box (and lies in the half)?
   // (uniform)
   auto interior = [&](int kb) {
@@ -1014,7 +1033,8 @@ __device__ __forceinline__ void MiBackwardChunk(
 #pragma unroll
     for (int it = 0; it < kLoadItems; ++it) {
       const int jd = kb * kW + 4 * mm - (lq + kRowStep * it) * g.skew;  // destination column of element 0
-      r.d[it] = kBidir ? AsyncQuadCoherent(rsp, quad_at(idx_d[it], jd)) : AsyncQuad(rsp, quad_at(idx_d[it], jd));
+      r.d[it] = kBidir ? AsyncQuadCoherent(rsp, idx_d[it] + kb * kSlabBlockFloats + 4 * mm)
+                       : AsyncQuad(rsp, idx_d[it] + jd);
       if (!kKept) {
         r.s[it] = AsyncQuad(rsp, idx_s[it] + jd);
         r.x[it] = AsyncQuad(rsx, idx_x[it] + jd);
@@ -1068,16 +1088,16 @@ __device__ __forceinline__ void MiBackwardChunk(
       const int q = lq + kRowStep * it;
       float4 qd = AsFloat4(r.d[it]);
       float4 qs = kKept ? qd : AsFloat4(r.s[it]), qx = kKept ? qd : AsFloat4(r.x[it]);
-      if (!inner && g.b == 0) {  // the only sequence whose rows can start the tensor
+      // (the slab's quads are whole by construction)
+      if (!kBidir && !inner && g.b == 0) {  // the only sequence whose rows can start the tensor
         asm volatile("");
         const int jd0 = kb * kW + 4 * mm - q * g.skew;
-        qd = ShiftQuad(qd, quad_at(idx_d[it], jd0));
+        qd = ShiftQuad(qd, idx_d[it] + jd0);
         if (!kKept) {
           qs = ShiftQuad(qs, idx_s[it] + jd0);
           qx = ShiftQuad(qx, idx_x[it] + jd0);
         }
       }
-      if (kBidir && mirror) qd = Rev4(qd);
       float ve[4], vo[4];
       flow(qd.x, qs.x, qx.x, &ve[0], &vo[0]);
       flow(qd.y, qs.y, qx.y, &ve[1], &vo[1]);
@@ -1532,12 +1552,16 @@ __device__ __attribute__((noinline)) void BidirExactTask(CutShared &sh, const Ta
   const BidirArgs &k = t.k;
   const Box box = t.box;
   float *prev = sh.a, *cur = sh.a + (k.S + 2);
+  // p goes where the sequence's blocks would have gone: the sequence's part of the slab is at
+  // least (S + 1) rows of Tn + 2 (the exact recursion adds seq * (S + 1) * (Tn + 2) itself)
+  float *p_seq = k.scratch + (size_t)seq * (SlabFloatsPerSequence(k.S, k.Tn, k.modified) -
+                                            (size_t)(k.S + 1) * (k.Tn + 2));
   static_assert(offsetof(CutShared, b) == sizeof(float) * kCutRows, "a and b are one array here");
-  const float end = MiForwardGenericSeq<float>(k.px, k.py, box, k.scratch, seq, k.S, k.Tn, k.modified,
+  const float end = MiForwardGenericSeq<float>(k.px, k.py, box, p_seq, seq, k.S, k.Tn, k.modified,
                                                k.Tn + 2, prev, cur);
   if (threadIdx.x == 0) k.ans[seq] = GaveUp(k.hdr) ? __builtin_nanf("") : end;
   __syncthreads();
-  const float at_origin = MiBackwardGenericSeq<float>(k.px, k.scratch, box, seed, k.px_grad, k.py_grad,
+  const float at_origin = MiBackwardGenericSeq<float>(k.px, p_seq, box, seed, k.px_grad, k.py_grad,
                                                       seq, k.S, k.Tn, k.modified, k.Tn + 2, prev, cur);
   if (k.overwrite_ans_grad && k.ans_grad != nullptr && threadIdx.x == 0) k.ans_grad[seq] = at_origin;
 }
@@ -1774,9 +1798,11 @@ bool MiFusedAdvised(int B, int S) {
   return units > 0 && 2ll * B * nchunks <= units;
 }
 
-// Floats of scratch per call of the single launch: one slab of (S + 1) rows of Tn + 2 per sequence
-// (the log-derivatives of both halves, the mirrored half's one column to the right).
-size_t MiFusedScratchElems(int B, int S, int Tn) { return (size_t)B * (S + 1) * ((size_t)Tn + 2); }
+// Floats of scratch per call of the single launch: the log-derivatives of both halves of every
+// sequence, in blocks (SlabBlocks).
+size_t MiFusedScratchElems(int B, int S, int Tn, int modified) {
+  return (size_t)B * SlabFloatsPerSequence(S, Tn, modified);
+}
 
 int MiForwardBackwardFast(const float *px, const float *py, const int64_t *boundary, float *ans,
                           float *scratch, float *ans_grad, float *px_grad, float *py_grad, int B,
@@ -1784,8 +1810,7 @@ int MiForwardBackwardFast(const float *px, const float *py, const int64_t *bound
                           size_t workspace_bytes, hipStream_t stream) {
   if (workspace == nullptr || workspace_bytes < MiFastWorkspaceBytes(B, S, Tn)) return K2AMD_ERR_WORKSPACE;
   if (scratch == nullptr) return K2AMD_ERR_INVALID_ARGUMENT;
-  if (!MiFusedSupports(B, S, Tn, modified) || MiFusedScratchElems(B, S, Tn) >= (1ull << 29))
-    return K2AMD_ERR_UNSUPPORTED;
+  if (!MiFusedSupports(B, S, Tn, modified)) return K2AMD_ERR_UNSUPPORTED;
   const int units = ComputeUnits();
   if (units <= 0) return K2AMD_ERR_LAUNCH;
   const int nchunks = (S + 1 + kRows - 1) / kRows;

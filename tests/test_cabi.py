@@ -56,7 +56,10 @@ def test_invalid_arguments_return_codes_without_a_gpu():
     assert lib.k2amd_mi_forward_backward_supported(4, 10, 20, 0, 0, 1) == 1
     assert lib.k2amd_mi_forward_backward_supported(2000, 200, 1000, 1, 0, 1) == 1
     assert lib.k2amd_mi_forward_backward_supported(4, 2055, 3000, 1, 0, 1) == 0   # more rows than its join keeps
-    assert lib.k2amd_mi_forward_backward_scratch_bytes(4, 10, 20, 0, 0) == 4 * 11 * 22 * 4
+    # per sequence: two halves x one chunk of 64 rows x one block of 32 positions (the cut of a
+    # regular 10 x 20 lattice lies 15 diagonals in), in floats
+    assert lib.k2amd_mi_forward_backward_scratch_bytes(4, 10, 20, 0, 0) == 4 * 2 * 64 * 32 * 4
+    assert lib.k2amd_mi_forward_backward_scratch_bytes(32, 200, 1000, 1, 0) == 32 * 2 * 4 * 16 * 64 * 32 * 4
     assert lib.k2amd_mi_forward_backward_scratch_bytes(4, 10, 20, 0, 1) == 0
     # the log-derivative tensor is only used by the pipelined fp32 kernels, which need a workspace
     assert lib.k2amd_mi_keeps_log_deriv(4, 10, 20, 0, 0, 1) == 1
