@@ -249,8 +249,10 @@ struct Half {
 };
 #ifdef K2AMD_MI_TRACE
 #define K2AMD_TRACE_MARK(half, i) do { if ((half).trace != nullptr && threadIdx.x == 0) (half).trace[i] = wall_clock64(); } while (0)
+#define K2AMD_TRACE_MARK_IF(half, i, cond) do { if ((half).trace != nullptr && (cond)) (half).trace[i] = wall_clock64(); } while (0)
 #else
 #define K2AMD_TRACE_MARK(half, i) do { } while (0)
+#define K2AMD_TRACE_MARK_IF(half, i, cond) do { } while (0)
 #endif
 
 // The single launch keeps the log-derivatives of every half-sweep in a slab of its own, laid out
@@ -345,13 +347,199 @@ __device__ __forceinline__ void PublishEdge(float *addr, float v) {
 }
 
 // Values on the cut diagonal go through device-coherent stores and loads like the edge words (the
-// reader is another workgroup, on any compute unit), but need no sentinel: a counter says when
-// all of a sequence's values are there.
-__device__ __forceinline__ void PublishCut(float *addr, float v) {
-  __hip_atomic_store(addr, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+// readers are other workgroups, on any compute unit) and validate themselves the same way; they
+// have several readers, so a reader leaves them as they are (the last one to finish puts the
+// sentinels back, see MiBidirKernel).
+__device__ __forceinline__ void PublishCut(float *addr, float v) { PublishEdge(addr, v); }
+
+
+// ---- the cut of the single launch (see MiBidirKernel) ----
+constexpr int kCutRows = 2056;  // lattice rows (S + 2 at most) the single launch serves
+constexpr int kCutWordsPerSeqHeader = 16;
+
+struct CutShared {
+  // alpha / beta of the sequence's cut cells by lattice row, then exp(alpha + beta - best); also
+  // the two rotating rows of the exact recursion
+  float a[kCutRows];
+  float b[kCutRows];
+  float total;   // the sequence's score, from the join of this task
+  float scale;   // the gradient of the sequence's score
+  int split_ok;  // the score is finite: the halves sweep back from the cut
+  int last;
+  unsigned ticket;
+};
+
+// Per sequence, in the workspace: depart (readers of the cut finished), the gradient of the
+// sequence's score, stored (forward sweeps whose log-derivatives have all reached memory), then
+// alpha by own row of the first half and beta by own row of the second.  Counters count up from
+// the sentinel, which is what the workspace is initialised to.
+struct CutWords {
+  unsigned *depart, *stored;
+  float *scale, *alpha, *beta;
+  int words;
+};
+__device__ __forceinline__ CutWords CutOf(float *cut, int b, int nchunks) {
+  CutWords w;
+  w.words = kCutWordsPerSeqHeader + 2 * nchunks * kRows;
+  float *base = cut + (size_t)b * w.words;
+  w.depart = reinterpret_cast<unsigned *>(base) + 1;
+  w.scale = base + 2;
+  w.stored = reinterpret_cast<unsigned *>(base) + 3;
+  w.alpha = base + kCutWordsPerSeqHeader;
+  w.beta = w.alpha + nchunks * kRows;
+  return w;
 }
-__device__ __forceinline__ float ReadCut(const float *addr) {
-  return __hip_atomic_load(addr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
+// One thread waits until a counter has reached a value (bounded, like TakeEdge).
+__device__ __forceinline__ void WaitCount(unsigned *word, unsigned want, FastHeader *hdr) {
+  int spins = 0;
+  for (;;) {
+    if (__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == want) return;
+    ++spins;
+    if ((spins & 255) == 0 &&
+        __hip_atomic_load(&hdr->error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)
+      return;
+    if (spins > kSpinLimit) {
+      __hip_atomic_store(&hdr->error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      return;
+    }
+    __builtin_amdgcn_s_sleep(2);
+  }
+}
+
+// Reductions over a wavefront through the data-parallel lane permutations (a few cycles per step;
+// the LDS crossbar that __shfl goes through costs a hundred).  Four steps leave the result of
+// each row of 16 lanes in all of its lanes, the four rows are combined in a fixed order: every
+// lane gets the same bits.
+template <int kCtrl>
+__device__ __forceinline__ float DppF(float v) {
+  return __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), kCtrl, 0xf, 0xf, true));
+}
+template <int kCtrl>
+__device__ __forceinline__ int DppI(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, kCtrl, 0xf, 0xf, true);
+}
+// quad_perm [1,0,3,2], quad_perm [2,3,0,1], row_half_mirror, row_mirror
+#define K2AMD_ROW_BUTTERFLY(v, Dpp, op)  \
+  v = op(v, Dpp<0xB1>(v));               \
+  v = op(v, Dpp<0x4E>(v));               \
+  v = op(v, Dpp<0x141>(v));              \
+  v = op(v, Dpp<0x140>(v))
+__device__ __forceinline__ float LaneF(float v, int lane) {
+  return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), lane));
+}
+__device__ __forceinline__ float AddF(float a, float b) { return a + b; }
+__device__ __forceinline__ int MinI(int a, int b) { return a < b ? a : b; }
+__device__ __forceinline__ float WaveMaxF(float v) {
+  K2AMD_ROW_BUTTERFLY(v, DppF, fmaxf);
+  return fmaxf(fmaxf(LaneF(v, 0), LaneF(v, 16)), fmaxf(LaneF(v, 32), LaneF(v, 48)));
+}
+__device__ __forceinline__ float WaveSumF(float v) {
+  K2AMD_ROW_BUTTERFLY(v, DppF, AddF);
+  return (LaneF(v, 0) + LaneF(v, 16)) + (LaneF(v, 32) + LaneF(v, 48));
+}
+__device__ __forceinline__ int WaveMinI(int v) {
+  K2AMD_ROW_BUTTERFLY(v, DppI, MinI);
+  return MinI(MinI(__builtin_amdgcn_readlane(v, 0), __builtin_amdgcn_readlane(v, 16)),
+              MinI(__builtin_amdgcn_readlane(v, 32), __builtin_amdgcn_readlane(v, 48)));
+}
+#undef K2AMD_ROW_BUTTERFLY
+
+// What a backward task needs for the join on its sequence's cut.
+struct BidirJoin {
+  CutShared *sh;
+  CutWords cw;
+  float *ans;  // where the sequence's score goes (the task of chunk 0 of the first half), or null
+};
+
+// The join on the cut of a sequence with ns + 1 rows, by ONE wavefront (the others of the
+// workgroup are fetching the sweep's first blocks meanwhile): waits for the sequence's alpha and
+// beta, returns the score (to every lane; -inf when no path reaches the end cell) and, to lane q,
+// the gradient seed of own row row0 + q of a half (lattice row = own row, or ns - own row when
+// mirrored).  Every task of a sequence adds the same numbers in the same order, so all of them
+// get the same bits.
+// alpha and beta are of the size of the score (thousands, where one ulp is 2.4e-4) while their
+// sum only matters relative to the largest one: both are taken relative to the best cell's
+// values BEFORE they are added, which keeps the shares exact to a few ulps of themselves.
+// (Inlined: as a function of its own it would take the words' addresses and hand back its results
+// through scratch memory, a trip there for each.)
+__device__ __forceinline__ float WaveCutJoin(CutShared &sh, const CutWords cw, int ns, int row0,
+                                             int mirror, FastHeader *hdr, float *seed_out,
+                                             float *scale_out) {
+  const int lane = threadIdx.x & (kWave - 1);
+  // Every pass asks for all of the sequence's words before it looks at any (one trip to memory
+  // per pass, whatever the number of rows), until none of them is the sentinel.
+  constexpr int kBatch = 4;
+  const unsigned *wa = reinterpret_cast<const unsigned *>(cw.alpha);
+  const unsigned *wb = reinterpret_cast<const unsigned *>(cw.beta);
+  float scale = 0.0f;
+  for (int spins = 0;; ++spins) {
+    const unsigned us = __hip_atomic_load(reinterpret_cast<const unsigned *>(cw.scale), __ATOMIC_RELAXED,
+                                          __HIP_MEMORY_SCOPE_AGENT);
+    bool missing = false;
+    for (int s0 = lane; s0 <= ns; s0 += kWave * kBatch) {
+      unsigned ua[kBatch], ub[kBatch];
+#pragma unroll
+      for (int i = 0; i < kBatch; ++i) {
+        const int s = min(s0 + i * kWave, ns);
+        ua[i] = __hip_atomic_load(wa + s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ub[i] = __hip_atomic_load(wb + (ns - s), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+#pragma unroll
+      for (int i = 0; i < kBatch; ++i) {
+        const int s = s0 + i * kWave;
+        if (s <= ns) {
+          missing |= ua[i] == kSentinel || ub[i] == kSentinel;
+          sh.a[s] = __uint_as_float(ua[i]);
+          sh.b[s] = __uint_as_float(ub[i]);
+        }
+      }
+    }
+    missing |= us == kSentinel;
+    scale = __uint_as_float(us);
+    if (!__any(missing)) break;
+    // bounded like every wait: what is missing stays a NaN, the score comes out as not finite
+    // and the error flag turns the results into NaN
+    if ((spins & 255) == 255 &&
+        __hip_atomic_load(&hdr->error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)
+      break;
+    if (spins > kSpinLimit) {
+      __hip_atomic_store(&hdr->error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      break;
+    }
+    __builtin_amdgcn_s_sleep(1);
+  }
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  float best = -3.0e38f;
+  int best_s = 0x7fffffff;
+  for (int s = lane; s <= ns; s += kWave) {
+    const float u = sh.a[s] + sh.b[s];
+    if (u > best) { best = u; best_s = s; }
+  }
+  // the largest sum, the smallest row among equals
+  const float wave_best = WaveMaxF(best);
+  best_s = WaveMinI(best == wave_best ? best_s : 0x7fffffff);
+  const int at = best_s <= ns ? best_s : 0;  // (no candidate at all: every sum was NaN)
+  // One wavefront's LDS accesses are served in the order it issues them: the fences only keep
+  // the compiler from moving them.
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  const float a_ref = sh.a[at], b_ref = sh.b[at];
+  const bool reachable = a_ref + b_ref > kLogZeroTest;
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  float sum = 0.0f;
+  for (int s = lane; s <= ns; s += kWave) {
+    const float w = reachable ? expf((sh.a[s] - a_ref) + (sh.b[s] - b_ref)) : 0.0f;
+    sh.a[s] = w;
+    sum += w;
+  }
+  sum = WaveSumF(sum);  // >= 1 when reachable
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  const int own = row0 + lane;
+  const int s_own = min(max(mirror ? ns - own : own, 0), ns);
+  const float share = sh.a[s_own];
+  *seed_out = reachable && own <= ns ? share / sum * scale : 0.0f;
+  *scale_out = scale;
+  return reachable ? (a_ref + b_ref) + logf(sum) : NegInfF();
 }
 
 // ------------------------------------------------------------------------------ forward
@@ -401,17 +589,14 @@ constexpr int kFwdLoadsPerBlock = 2 * FwdLayout::kLoadItems + 1;
 // kBidir: the sweep covers the half `half` of the lattice (see Half) and ends on its cut
 // diagonal; what the chain holds there (p of the half's last cell of every row) goes to
 // cut_out[0..63] (the chunk's 64 own rows; the finite stand-in for -inf where a row has no cell
-// on the cut or lies past the sequence's last row) and *cut_arrive is then incremented (once per
-// call, whatever the chunk holds), ans is not written, and log_deriv has rows of
-// Tn + 2 floats (the two halves of a sequence share one slab: the mirrored half's cells lie one
-// column to the right of their place, where no cell of the other half is).
+// on the cut; nothing for rows of a chunk that lies past the sequence's last row altogether), ans
+// is not written, and log_deriv is the launch's slab of blocks (SlabBlocks).
 template <bool kKeep, bool kWriteP, bool kBidir>
 __device__ __forceinline__ void MiForwardChunk(
     FwdLds &lds, const float *__restrict__ px, const float *__restrict__ py, const Box &box,
     float *__restrict__ p, float *__restrict__ ans,
     float *__restrict__ log_deriv, FastHeader *hdr, float *edge, int B, int S, int Tn,
-    int modified, int nchunks, int edge_stride, int seq, int chunk, Half half, float *cut_out,
-    unsigned *cut_arrive) {
+    int modified, int nchunks, int edge_stride, int seq, int chunk, Half half, float *cut_out) {
   static_assert(!kBidir || (kKeep && !kWriteP), "the halves keep the log-derivatives only");
   ChunkGeom g;
   g.b = seq;
@@ -420,8 +605,6 @@ __device__ __forceinline__ void MiForwardChunk(
   g.row0 = g.c * kRows;
   if (!box.ok || g.row0 > g.ns) {
     if (!kBidir && !box.ok && g.c == 0 && threadIdx.x == 0) ans[g.b] = __builtin_nanf("");
-    if (kBidir && threadIdx.x == 0)
-      __hip_atomic_fetch_add(cut_arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return;
   }
   g.skew = modified ? 0 : 1;
@@ -434,11 +617,7 @@ __device__ __forceinline__ void MiForwardChunk(
   const int n_last = nsteps - 1;  // the chunk's step on the cut diagonal (kBidir)
   g.nblocks = blocks_of(g.row0);
   if (kBidir && g.nblocks == 0) {  // no cell of these rows lies in the half
-    if (threadIdx.x < kRows) {
-      PublishCut(cut_out + threadIdx.x, kLogZero);
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      if (threadIdx.x == 0) __hip_atomic_fetch_add(cut_arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
+    if (threadIdx.x < kRows) PublishCut(cut_out + threadIdx.x, kLogZero);
     return;
   }
   const bool has_down = g.row0 + kRows <= g.ns && blocks_of(g.row0 + kRows) > 0;
@@ -802,15 +981,12 @@ __device__ __forceinline__ void MiForwardChunk(
   if (kBidir && role == kChain) {
     // What the chain left on the cut diagonal: step n_last of every row, still in the ring.  (A
     // chunk that ran out of columns before the cut has no cell on it; a row whose cell on the cut
-    // lies outside the columns holds a stand-in for -inf there already.)  The chain wavefront
-    // has no other store in flight, so its wait below is for these 64 words only: the sequence's
-    // join on the cut can start while the other wavefronts' log-derivatives are still on
-    // their way.
+    // lies outside the columns holds a stand-in for -inf there already.)  The words validate
+    // themselves, so the sequence's join on the cut starts as soon as they land, while the other
+    // wavefronts' log-derivatives are still on their way.
     const int at = ((g.nblocks - 1) % 3) * kW + (n_last - (g.nblocks - 1) * kW);
     const bool on_cut = half.dmax - g.row0 * g.skew == n_last && g.row0 + lane <= g.ns;
     PublishCut(cut_out + lane, on_cut ? reinterpret_cast<const float *>(&lds.fy[lane][0])[at] : kLogZero);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    if (lane == 0) __hip_atomic_fetch_add(cut_arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   if (kBidir) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the coherent stores above
 }
@@ -829,7 +1005,7 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiForwardFastKernel(
   MiForwardChunk<kKeep, kWriteP, false>(lds, px, py, LoadBox(boundary, (int)(ticket / nchunks), S, Tn), p,
                                         ans, log_deriv, hdr, edge, B, S, Tn, modified, nchunks,
                                         edge_stride, (int)(ticket / nchunks), (int)(ticket % nchunks),
-                                        Half{}, nullptr, nullptr);
+                                        Half{}, nullptr);
   if (threadIdx.x == 0) FinishWorkgroup(hdr, gridDim.x);
 }
 
@@ -919,16 +1095,17 @@ __device__ __forceinline__ void ZeroItem(const ZeroGeom &z, int r, int c) {
 // The whole workgroup sweeps chunk `chunk` of sequence `seq`, or (zero_only) clears what the
 // sweep leaves unassigned in array rows chunk * 64 .. chunk * 64 + 63 of that sequence.
 // kBidir: the sweep covers the half `half` (see Half), whose forward sweep left its
-// log-derivatives in `p` (rows of Tn + 2 floats); it starts on the cut diagonal, where row
-// row0 + q of the half holds gradient seeds[q] (its cell's share of all paths, times the
-// gradient of the sequence's score), instead of at the end cell.
+// log-derivatives in `p` (the launch's slab of blocks); it starts on the cut diagonal, where
+// every row of the half holds its cell's share of all paths times the gradient of the sequence's
+// score (WaveCutJoin, run by the chain wavefront while the loaders fetch the first blocks),
+// instead of at the end cell.
 template <bool kKept, bool kBidir>
 __device__ __forceinline__ void MiBackwardChunk(
     BwdLds &lds, const float *__restrict__ px, const float *__restrict__ p, const Box &box,
     float *__restrict__ ans_grad,
     float *__restrict__ px_grad, float *__restrict__ py_grad, FastHeader *hdr, float *edge, int B,
     int S, int Tn, int modified, int nchunks, int edge_stride, int overwrite_ans_grad, int seq,
-    int chunk, bool zero_only, Half half, const float *seeds) {
+    int chunk, bool zero_only, Half half, const BidirJoin *join) {
   static_assert(!kBidir || kKept, "the halves hand over log-derivatives");
   ChunkGeom g;
   g.b = seq;
@@ -1215,12 +1392,7 @@ __device__ __forceinline__ void MiBackwardChunk(
   // ---- chain wavefront ---------------------------------------------------------------------
   // gradient at the (virtual) right end of each row: the seed on the sequence's last row
   float G = 0.0f;
-  // (the single launch may come without ans_grad: every sequence's score then has gradient 1)
-  if (kBidir) {
-    if (role == kChain) G = seeds[lane];
-  } else if (role == kChain && g.row0 + lane == g.ns) {
-    G = ans_grad != nullptr ? ans_grad[g.b] : 1.0f;
-  }
+  if (!kBidir && role == kChain && g.row0 + lane == g.ns) G = ans_grad != nullptr ? ans_grad[g.b] : 1.0f;
   float g_origin = 0.0f;
   // Per position (descending), with OME of the own row and Edn = d1 of the row below (lane + 1):
   //     G' = OME * G + Edn * G(lane + 1)
@@ -1256,22 +1428,65 @@ __device__ __forceinline__ void MiBackwardChunk(
   };
 
   const int top = g.nblocks - 1;
-  // what the cells of the top block's last position saw: the initial gradient
-  if (role == kChain)
-    reinterpret_cast<float *>(&lds.g[lane][((top + 1) % 3) * kQuadsPerBlock])[0] = G;
   BwdRegs sets[kSets];
-  if (role == kLoader) {
-    load_block(top, sets[0]);
-    wait_all(sets[0]);
-    commit_block(top, sets[0]);
+  if (kBidir) {
+    // The chain wavefront joins the halves on the cut; the loaders wait for the forward sweeps'
+    // last log-derivatives (all of the sequence's: the counter is per sequence) and fetch the
+    // first blocks meanwhile.  The edge wavefront asks the chunk below for nothing before the
+    // join has said that the halves sweep back at all: where the score is not finite no chunk
+    // of the sequence publishes anything.
+    CutShared &sh = *join->sh;
+    if (role == kChain) {
+      float scale;
+      K2AMD_TRACE_MARK(half, 7);
+      const float total = WaveCutJoin(sh, join->cw, g.ns, g.row0, mirror, hdr, &G, &scale);
+      K2AMD_TRACE_MARK(half, 3);
+      if (lane == 0) {
+        const bool ok = total > kLogZeroTest;  // a finite score
+        sh.total = total;
+        sh.scale = scale;
+        sh.split_ok = ok;
+        if (join->ans != nullptr && ok) *join->ans = GaveUp(hdr) ? __builtin_nanf("") : total;
+      }
+      K2AMD_TRACE_MARK(half, 1);
+    } else if (role == kLoader) {
+      const unsigned per_seq = 2u * nchunks;
+      if (lane == 0) WaitCount(join->cw.stored, kSentinel + per_seq, hdr);
+      load_block(top, sets[0]);
+      wait_all(sets[0]);
+      commit_block(top, sets[0]);
 #pragma unroll
-    for (int i = 0; i < kSets; ++i) load_block(top - 1 - i, sets[i]);
-  } else if (role == kEdge) {
-    take_block(top);
+      for (int i = 0; i < kSets; ++i) load_block(top - 1 - i, sets[i]);
+    }
+    LdsBarrier();
+    if (!sh.split_ok) {
+      if (role == kLoader) {
+#pragma unroll
+        for (int i = 0; i < kSets; ++i) wait_all(sets[i]);
+      }
+      return;
+    }
+    // what the cells of the top block's last position saw: the initial gradient
+    if (role == kChain) reinterpret_cast<float *>(&lds.g[lane][((top + 1) % 3) * kQuadsPerBlock])[0] = G;
+    if (role == kEdge) take_block(top);
+    K2AMD_TRACE_MARK(half, 4);
+    LdsBarrier();
+    K2AMD_TRACE_MARK(half, 5);
+  } else {
+    // what the cells of the top block's last position saw: the initial gradient
+    if (role == kChain)
+      reinterpret_cast<float *>(&lds.g[lane][((top + 1) % 3) * kQuadsPerBlock])[0] = G;
+    if (role == kLoader) {
+      load_block(top, sets[0]);
+      wait_all(sets[0]);
+      commit_block(top, sets[0]);
+#pragma unroll
+      for (int i = 0; i < kSets; ++i) load_block(top - 1 - i, sets[i]);
+    } else if (role == kEdge) {
+      take_block(top);
+    }
+    LdsBarrier();
   }
-  K2AMD_TRACE_MARK(half, 4);
-  LdsBarrier();
-  K2AMD_TRACE_MARK(half, 5);
 
   // Descending twin of the forward's loops: in iteration kb the chain computes block kb, the
   // loaders commit block kb-1 and start the loads of block kb-3, the storers drain block kb+1,
@@ -1370,134 +1585,6 @@ __global__ __launch_bounds__(BwdLayout::kThreads) void MiBackwardFastKernel(
 // are then DEFINED by the reference's loop order (k2/python/csrc/torch/
 // mutual_information_cpu.cu:195-211).  Such a sequence is left to its last task, which runs the
 // exact one-workgroup recursion of mi_generic_impl.h on it.
-constexpr int kCutRows = 2056;  // lattice rows (S + 2 at most) the single launch serves
-constexpr int kCutWordsPerSeqHeader = 16;
-
-struct CutShared {
-  // alpha / beta of the sequence's cut cells by lattice row, then exp(alpha + beta - best); also
-  // the two rotating rows of the exact recursion
-  float a[kCutRows];
-  float b[kCutRows];
-  float red_val[16];
-  int red_idx[16];
-  float seeds[kRows];
-  float total;
-  float scale;
-  int best;
-  int last;
-  unsigned ticket;
-};
-
-// Per sequence, in the workspace: arrive (forward sweeps whose values on the cut are there),
-// depart (readers of the cut finished), the gradient of the sequence's score, stored (forward
-// sweeps whose log-derivatives have all reached memory), then alpha by own row of the first half
-// and beta by own row of the second.  Counters count up from the sentinel, which is what the
-// workspace is initialised to.
-struct CutWords {
-  unsigned *arrive, *depart, *stored;
-  float *scale, *alpha, *beta;
-  int words;
-};
-__device__ __forceinline__ CutWords CutOf(float *cut, int b, int nchunks) {
-  CutWords w;
-  w.words = kCutWordsPerSeqHeader + 2 * nchunks * kRows;
-  float *base = cut + (size_t)b * w.words;
-  w.arrive = reinterpret_cast<unsigned *>(base);
-  w.depart = reinterpret_cast<unsigned *>(base) + 1;
-  w.scale = base + 2;
-  w.stored = reinterpret_cast<unsigned *>(base) + 3;
-  w.alpha = base + kCutWordsPerSeqHeader;
-  w.beta = w.alpha + nchunks * kRows;
-  return w;
-}
-
-// One thread waits until a counter has reached a value (bounded, like TakeEdge).
-__device__ __forceinline__ void WaitCount(unsigned *word, unsigned want, FastHeader *hdr) {
-  int spins = 0;
-  for (;;) {
-    if (__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == want) return;
-    ++spins;
-    if ((spins & 255) == 0 &&
-        __hip_atomic_load(&hdr->error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)
-      return;
-    if (spins > kSpinLimit) {
-      __hip_atomic_store(&hdr->error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      return;
-    }
-    __builtin_amdgcn_s_sleep(2);
-  }
-}
-
-// (value, index) of the largest value over the workgroup, the smallest index among equals.
-__device__ __forceinline__ void BlockArgMax(CutShared &sh, float v, int idx) {
-  for (int d = 32; d >= 1; d >>= 1) {
-    const float ov = __shfl_xor(v, d);
-    const int oi = __shfl_xor(idx, d);
-    if (ov > v || (ov == v && oi < idx)) { v = ov; idx = oi; }
-  }
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  if (lane == 0) { sh.red_val[wave] = v; sh.red_idx[wave] = idx; }
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    const int nw = blockDim.x >> 6;
-    for (int w = 1; w < nw; ++w)
-      if (sh.red_val[w] > v || (sh.red_val[w] == v && sh.red_idx[w] < idx)) { v = sh.red_val[w]; idx = sh.red_idx[w]; }
-    sh.best = idx;
-  }
-  __syncthreads();
-}
-// Sum over the workgroup in a fixed order (the same bits in every workgroup that adds the same
-// numbers).
-__device__ __forceinline__ float BlockSum(CutShared &sh, float v) {
-  for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d);
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  __syncthreads();
-  if (lane == 0) sh.red_val[wave] = v;
-  __syncthreads();
-  float t = sh.red_val[0];
-  const int nw = blockDim.x >> 6;
-  for (int w = 1; w < nw; ++w) t += sh.red_val[w];
-  return t;
-}
-
-// The join on the cut of a sequence with ns + 1 rows: returns the score (to every thread; -inf
-// when no path reaches the end cell) and leaves in sh.seeds the gradient seeds of the 64 own rows
-// row0 .. row0 + 63 of a half (lattice row = own row, or ns - own row when mirrored).
-// alpha and beta are of the size of the score (thousands, where one ulp is 2.4e-4) while their
-// sum only matters relative to the largest one: both are taken relative to the best cell's
-// values BEFORE they are added, which keeps the shares exact to a few ulps of themselves.
-__device__ __attribute__((noinline)) float CutJoin(CutShared &sh, const CutWords &cw, int ns, int row0, int mirror) {
-  float best = -3.0e38f;
-  int best_s = 0x7fffffff;
-  for (int s = threadIdx.x; s <= ns; s += blockDim.x) {
-    const float a = ReadCut(cw.alpha + s), b = ReadCut(cw.beta + (ns - s));
-    sh.a[s] = a;
-    sh.b[s] = b;
-    const float u = a + b;
-    if (u > best) { best = u; best_s = s; }
-  }
-  if (threadIdx.x == 0) sh.scale = ReadCut(cw.scale);
-  BlockArgMax(sh, best, best_s);
-  const int at = sh.best <= ns ? sh.best : 0;  // (no candidate at all: every sum was NaN)
-  const float a_ref = sh.a[at], b_ref = sh.b[at];
-  const bool reachable = a_ref + b_ref > kLogZeroTest;
-  float part = 0.0f;
-  __syncthreads();  // everyone has a_ref, b_ref before sh.a is overwritten
-  for (int s = threadIdx.x; s <= ns; s += blockDim.x) {
-    const float w = reachable ? expf((sh.a[s] - a_ref) + (sh.b[s] - b_ref)) : 0.0f;
-    sh.a[s] = w;
-    part += w;
-  }
-  const float sum = BlockSum(sh, part);  // >= 1 when reachable
-  if (threadIdx.x < kRows) {
-    const int own = row0 + threadIdx.x;
-    const int s = mirror ? ns - own : own;
-    sh.seeds[threadIdx.x] = reachable && own <= ns ? sh.a[s] / sum * sh.scale : 0.0f;
-  }
-  __syncthreads();
-  return reachable ? (a_ref + b_ref) + logf(sum) : NegInfF();
-}
-
 union FusedLds {
   FwdLds fwd;
   BwdLds bwd;
@@ -1526,19 +1613,23 @@ struct TaskShared {
   Box box;
 };
 __device__ __attribute__((noinline)) void BidirForwardTask(FwdLds &lds, const TaskShared &t, int seq,
-                                                           int chunk, Half half, float *cut_out,
-                                                           unsigned *cut_arrive) {
+                                                           int chunk, Half half, float *cut_out) {
   const BidirArgs &k = t.k;
   MiForwardChunk<true, false, true>(lds, k.px, k.py, t.box, nullptr, k.ans, k.scratch, k.hdr,
                                     half.mirror ? k.edge1 : k.edge0, k.B, k.S, k.Tn, k.modified,
-                                    k.nchunks, k.edge_stride, seq, chunk, half, cut_out, cut_arrive);
+                                    k.nchunks, k.edge_stride, seq, chunk, half, cut_out);
 }
+// (what the join needs comes as arguments of its own: a structure handed over by address would
+// live in scratch memory, a trip there for every field the sweep reads)
 __device__ __attribute__((noinline)) void BidirBackwardTask(BwdLds &lds, const TaskShared &t, int seq,
-                                                            int chunk, Half half, const float *seeds) {
+                                                            int chunk, Half half, CutShared *sh,
+                                                            float *ans_out) {
   const BidirArgs &k = t.k;
+  const BidirJoin join_words{sh, CutOf(k.cut, seq, k.nchunks), ans_out};
+  const BidirJoin *join = &join_words;  // (never leaves this function: stays in registers)
   MiBackwardChunk<true, true>(lds, k.px, k.scratch, t.box, k.ans_grad, k.px_grad, k.py_grad, k.hdr,
                               half.mirror ? k.edge1 : k.edge0, k.B, k.S, k.Tn, k.modified, k.nchunks,
-                              k.edge_stride, k.overwrite_ans_grad, seq, chunk, false, half, seeds);
+                              k.edge_stride, k.overwrite_ans_grad, seq, chunk, false, half, join);
 }
 __device__ __attribute__((noinline)) void BidirClearTask(BwdLds &lds, const TaskShared &t, int seq, int chunk) {
   const BidirArgs &k = t.k;
@@ -1571,15 +1662,27 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiBidirKernel(const Bidir
   __shared__ FusedLds lds;
   __shared__ CutShared sh;
   __shared__ TaskShared ts;
-  if (threadIdx.x == 0) ts.k = k;
+  // The boxes of the first sequences, read once per workgroup while its first ticket is on its
+  // way: a task then starts without a trip to memory for its box.
+  constexpr int kBoxes = 256;
+  __shared__ Box boxes[kBoxes];
+  if (threadIdx.x == 0) {
+    ts.k = k;
+    sh.ticket = atomicAdd(&k.hdr->ticket, 1u);
+  }
+  for (int i = (int)threadIdx.x - kWave; i >= 0 && i < min(k.B, kBoxes); i += blockDim.x - kWave)
+    boxes[i] = LoadBox(k.boundary, i, k.S, k.Tn);
+  auto box_of = [&](int seq) { return seq < kBoxes ? boxes[seq] : LoadBox(k.boundary, seq, k.S, k.Tn); };
   const int nchunks = k.nchunks;
   const unsigned per_seq = 2u * nchunks, nsweep = (unsigned)k.B * per_seq;
   const unsigned first_clear = nsweep, first_bwd = first_clear + (unsigned)k.B * nchunks;
   const unsigned first_last = first_bwd + nsweep, ntasks = first_last + (unsigned)k.B;
   const int skew = k.modified ? 0 : 1;
-  for (;;) {
-    __syncthreads();  // the previous task's last LDS reads are done, its stores complete
-    if (threadIdx.x == 0) sh.ticket = atomicAdd(&k.hdr->ticket, 1u);
+  for (bool first = true;; first = false) {
+    if (!first) {
+      __syncthreads();  // the previous task's last LDS reads are done, its stores complete
+      if (threadIdx.x == 0) sh.ticket = atomicAdd(&k.hdr->ticket, 1u);
+    }
     __syncthreads();
     const unsigned ticket = sh.ticket;
     if (ticket >= ntasks) break;
@@ -1590,12 +1693,11 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiBidirKernel(const Bidir
       __device__ ~Tracer() { mark(2); }
     } tracer{k.trace != nullptr ? k.trace + 8 * (size_t)ticket : nullptr};
     tracer.mark(0);
-    if (tracer.at != nullptr && threadIdx.x == 0) tracer.at[3] = blockIdx.x;
 #endif
 
     if (ticket >= first_clear && ticket < first_bwd) {  // what no sweep assigns
       const unsigned unit = ticket - first_clear;
-      if (threadIdx.x == 0) ts.box = LoadBox(k.boundary, (int)(unit / nchunks), k.S, k.Tn);
+      if (threadIdx.x == 0) ts.box = box_of((int)(unit / nchunks));
       __syncthreads();
       BidirClearTask(lds.bwd, ts, (int)(unit / nchunks), (int)(unit % nchunks));
       continue;
@@ -1607,7 +1709,7 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiBidirKernel(const Bidir
     const int mirror = last ? 0 : (int)((unit % per_seq) / nchunks);
     const int cidx = last ? 0 : (int)(unit % nchunks);
     const int chunk = fwd || last ? cidx : nchunks - 1 - cidx;  // backward: lower chunks first
-    if (threadIdx.x == 0) ts.box = LoadBox(k.boundary, seq, k.S, k.Tn);
+    if (threadIdx.x == 0) ts.box = box_of(seq);
     __syncthreads();
     const Box box = ts.box;
     const int ns = box.s1 - box.s0, nt = box.t1 - box.t0;
@@ -1623,8 +1725,7 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiBidirKernel(const Bidir
     if (fwd) {
       if (!mirror && chunk == 0 && threadIdx.x == 0)
         PublishCut(cw.scale, k.ans_grad != nullptr ? k.ans_grad[seq] : 1.0f);
-      BidirForwardTask(lds.fwd, ts, seq, chunk, half, (mirror ? cw.beta : cw.alpha) + chunk * kRows,
-                       cw.arrive);
+      BidirForwardTask(lds.fwd, ts, seq, chunk, half, (mirror ? cw.beta : cw.alpha) + chunk * kRows);
       // every wavefront has waited for its stores (device-coherent ones, see StoreQuadCoherent)
       // before this barrier: whichever compute unit sweeps this chunk back will see them
       __syncthreads();
@@ -1633,43 +1734,40 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiBidirKernel(const Bidir
       continue;
     }
 
-    // backward sweep of a chunk, or the sequence's last task: both start from the cut
-    if (threadIdx.x == 0) WaitCount(cw.arrive, kSentinel + per_seq, k.hdr);
-    __syncthreads();
-    float total = 0.0f;
-#ifdef K2AMD_MI_TRACE
-    tracer.mark(1);
-#endif
-    // The join runs while the last log-derivatives are on their way; they are needed after it.
-    // (The look at their counter is asked for before the join and used after it: one trip to
-    // memory less where they have all arrived by then.)
-    unsigned stored = 0;
-    if (threadIdx.x == 0) stored = __hip_atomic_load(cw.stored, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (box.ok) total = CutJoin(sh, cw, ns, chunk * kRows, mirror);
-    const float seed = sh.scale;
-    if (threadIdx.x == 0 && stored != kSentinel + per_seq) WaitCount(cw.stored, kSentinel + per_seq, k.hdr);
-    __syncthreads();
-    // This task has read the sequence's cut words.  The last of their readers puts them back into
-    // their initial state; the count comes back while the sweep below runs and is looked at after it.
-    unsigned departed = 0;
-    if (threadIdx.x == 0)
-      departed = __hip_atomic_fetch_add(cw.depart, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const bool split_ok = box.ok && total > kLogZeroTest;  // a finite score
+    // Backward sweep of a chunk, or the sequence's last task: both start from the cut, whose
+    // words they wait for themselves.
     if (!last) {
-      if (!mirror && chunk == 0 && threadIdx.x == 0) {
-        if (!box.ok || GaveUp(k.hdr)) k.ans[seq] = __builtin_nanf("");
-        else if (split_ok) k.ans[seq] = total;
+      if (threadIdx.x == 0 && !mirror && chunk == 0 && !box.ok) k.ans[seq] = __builtin_nanf("");
+      if (box.ok)
+        BidirBackwardTask(lds.bwd, ts, seq, chunk, half, &sh, !mirror && chunk == 0 ? k.ans + seq : nullptr);
+    } else {
+      // The sequence's last task: the exact recursion where the halves could not be joined (no
+      // path reaches the end cell), once no forward sweep has a store on its way into the slab.
+      // It waits for the forward sweeps' stores in any case: they include the words of the cut,
+      // which the last task to leave the sequence resets, and this task is among those.
+      if (threadIdx.x < kWave) {
+        float seed, scale = 0.0f;
+        const float total = box.ok ? WaveCutJoin(sh, cw, ns, 0, 0, k.hdr, &seed, &scale) : 0.0f;
+        if (threadIdx.x == 0) {
+          sh.total = total;
+          sh.scale = scale;
+          WaitCount(cw.stored, kSentinel + per_seq, k.hdr);
+        }
       }
-      if (split_ok) BidirBackwardTask(lds.bwd, ts, seq, chunk, half, sh.seeds);
-    } else if (box.ok && !split_ok) {
-      BidirExactTask(sh, ts, seq, seed);
+      __syncthreads();
+      const float seed = sh.scale;
+      if (box.ok && !(sh.total > kLogZeroTest)) BidirExactTask(sh, ts, seq, seed);
     }
+    // This task is through with the sequence's cut words (where it read them at all).  The last
+    // task to say so puts them back into their initial state.
     __syncthreads();
-    if (threadIdx.x == 0) sh.last = departed + 1 == kSentinel + per_seq + 1;
+    if (threadIdx.x == 0)
+      sh.last = __hip_atomic_fetch_add(cw.depart, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
+                kSentinel + per_seq;
     __syncthreads();
     if (sh.last)
       for (int i = threadIdx.x; i < cw.words; i += blockDim.x)
-        __hip_atomic_store(reinterpret_cast<unsigned *>(cw.arrive) + i, kSentinel, __ATOMIC_RELAXED,
+        __hip_atomic_store(reinterpret_cast<unsigned *>(cw.depart) - 1 + i, kSentinel, __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_AGENT);
   }
   if (threadIdx.x == 0) FinishWorkgroup(k.hdr, gridDim.x);
