@@ -98,10 +98,6 @@ struct FastHeader {
   unsigned pad[61];
 };
 
-struct __attribute__((packed, aligned(4))) Quad {
-  float v[4];
-};
-
 __device__ __forceinline__ float NegInfF() { return -__builtin_huge_valf(); }
 
 // Inside the forward chain "minus infinity" is this finite stand-in: differences of two such
@@ -136,11 +132,25 @@ __device__ __forceinline__ float ChainStep(float P, float fx, float fy) {
   return __builtin_fmaf(__builtin_amdgcn_logf(1.0f + e), kLn2, mx);
 }
 
-__device__ __forceinline__ void StoreQuad(float *ptr, float4 v) {
-  Quad o;
-  o.v[0] = v.x; o.v[1] = v.y; o.v[2] = v.z; o.v[3] = v.w;
-  *reinterpret_cast<Quad *>(ptr) = o;
+// Everything these kernels reach through a pointer is device memory, and they say so: the tasks
+// of the single launch get their pointers from a structure in LDS, where the compiler cannot see
+// that, and an access through a pointer of unknown kind is a FLAT one, which also goes through
+// the LDS queue and counts against the waits for LDS data (the storers' gradient stores then
+// held up their own LDS reads: 6 us of a 56 us launch).
+typedef __attribute__((address_space(1))) float GFloat;
+typedef __attribute__((address_space(1))) unsigned GWord;
+__device__ __forceinline__ GFloat *Global(float *p) { return (GFloat *)p; }
+__device__ __forceinline__ const GFloat *Global(const float *p) { return (const GFloat *)p; }
+__device__ __forceinline__ GWord *Global(unsigned *p) { return (GWord *)p; }
+__device__ __forceinline__ const GWord *Global(const unsigned *p) { return (const GWord *)p; }
+
+typedef float QuadU __attribute__((ext_vector_type(4), aligned(4)));  // four floats at any float
+__device__ __forceinline__ void StoreQuad(GFloat *ptr, float4 v) {
+  QuadU o;
+  o.x = v.x; o.y = v.y; o.z = v.z; o.w = v.w;
+  *(__attribute__((address_space(1))) QuadU *)ptr = o;
 }
+__device__ __forceinline__ void StoreQuad(float *ptr, float4 v) { StoreQuad(Global(ptr), v); }
 
 // Loads go through raw buffer resources (one per tensor): the hardware range-checks every dword
 // against the tensor's size and returns 0 beyond it, so no load can leave the tensor whatever
@@ -195,7 +205,7 @@ __device__ __forceinline__ void StoreQuadCoherent(float *ptr, float4 v) {
   asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(ptr), "v"(w) : "memory");
 }
 __device__ __forceinline__ void StoreCoherent(float *ptr, float v) {
-  __hip_atomic_store(ptr, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(Global(ptr), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // A quad whose first float would lie in front of the tensor (idx < 0: only possible for the
@@ -305,17 +315,17 @@ __device__ __forceinline__ float TakeEdge(float *addr, FastHeader *hdr, float on
   unsigned *word = reinterpret_cast<unsigned *>(addr);
   int spins = 0;
   for (;;) {
-    const unsigned v = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned v = __hip_atomic_load(Global(word), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (v != kSentinel) {
-      __hip_atomic_store(word, kSentinel, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(Global(word), kSentinel, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       return __uint_as_float(v);
     }
     ++spins;
     if ((spins & 255) == 0 &&
-        __hip_atomic_load(&hdr->error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)
+        __hip_atomic_load(Global(&hdr->error), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)
       return on_timeout;
     if (spins > kSpinLimit) {
-      __hip_atomic_store(&hdr->error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(Global(&hdr->error), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       return on_timeout;
     }
     __builtin_amdgcn_s_sleep(1);
@@ -327,22 +337,22 @@ __device__ __forceinline__ float TakeEdge(float *addr, FastHeader *hdr, float on
 // back) become NaN, in that launch where the store comes after the timeout and in every later
 // launch until the workspace is initialised again.
 __device__ __forceinline__ bool GaveUp(FastHeader *hdr) {
-  return __hip_atomic_load(&hdr->error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;
+  return __hip_atomic_load(Global(&hdr->error), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;
 }
 
 // Called by one thread after the workgroup's last barrier.
 __device__ __forceinline__ void FinishWorkgroup(FastHeader *hdr, unsigned total) {
-  const unsigned n = atomicAdd(&hdr->done, 1u);
+  const unsigned n = __hip_atomic_fetch_add(Global(&hdr->done), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   if (n + 1 == total) {
-    __hip_atomic_store(&hdr->done, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(&hdr->ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(Global(&hdr->done), 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(Global(&hdr->ticket), 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 }
 
 __device__ __forceinline__ void PublishEdge(float *addr, float v) {
   unsigned u = __float_as_uint(v);
   if (u == kSentinel) u = 0x7fc00000u;
-  __hip_atomic_store(reinterpret_cast<unsigned *>(addr), u, __ATOMIC_RELAXED,
+  __hip_atomic_store(Global(reinterpret_cast<unsigned *>(addr)), u, __ATOMIC_RELAXED,
                      __HIP_MEMORY_SCOPE_AGENT);
 }
 
@@ -394,13 +404,13 @@ __device__ __forceinline__ CutWords CutOf(float *cut, int b, int nchunks) {
 __device__ __forceinline__ void WaitCount(unsigned *word, unsigned want, FastHeader *hdr) {
   int spins = 0;
   for (;;) {
-    if (__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == want) return;
+    if (__hip_atomic_load(Global(word), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == want) return;
     ++spins;
     if ((spins & 255) == 0 &&
-        __hip_atomic_load(&hdr->error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)
+        __hip_atomic_load(Global(&hdr->error), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)
       return;
     if (spins > kSpinLimit) {
-      __hip_atomic_store(&hdr->error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(Global(&hdr->error), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       return;
     }
     __builtin_amdgcn_s_sleep(2);
@@ -474,7 +484,7 @@ __device__ __forceinline__ float WaveCutJoin(CutShared &sh, const CutWords cw, i
   const unsigned *wb = reinterpret_cast<const unsigned *>(cw.beta);
   float scale = 0.0f;
   for (int spins = 0;; ++spins) {
-    const unsigned us = __hip_atomic_load(reinterpret_cast<const unsigned *>(cw.scale), __ATOMIC_RELAXED,
+    const unsigned us = __hip_atomic_load(Global(reinterpret_cast<const unsigned *>(cw.scale)), __ATOMIC_RELAXED,
                                           __HIP_MEMORY_SCOPE_AGENT);
     bool missing = false;
     for (int s0 = lane; s0 <= ns; s0 += kWave * kBatch) {
@@ -482,8 +492,8 @@ __device__ __forceinline__ float WaveCutJoin(CutShared &sh, const CutWords cw, i
 #pragma unroll
       for (int i = 0; i < kBatch; ++i) {
         const int s = min(s0 + i * kWave, ns);
-        ua[i] = __hip_atomic_load(wa + s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        ub[i] = __hip_atomic_load(wb + (ns - s), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ua[i] = __hip_atomic_load(Global(wa + s), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ub[i] = __hip_atomic_load(Global(wb + (ns - s)), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
 #pragma unroll
       for (int i = 0; i < kBatch; ++i) {
@@ -501,10 +511,10 @@ __device__ __forceinline__ float WaveCutJoin(CutShared &sh, const CutWords cw, i
     // bounded like every wait: what is missing stays a NaN, the score comes out as not finite
     // and the error flag turns the results into NaN
     if ((spins & 255) == 255 &&
-        __hip_atomic_load(&hdr->error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)
+        __hip_atomic_load(Global(&hdr->error), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)
       break;
     if (spins > kSpinLimit) {
-      __hip_atomic_store(&hdr->error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(Global(&hdr->error), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       break;
     }
     __builtin_amdgcn_s_sleep(1);
@@ -627,9 +637,8 @@ __device__ __forceinline__ void MiForwardChunk(
 
   const int T1 = modified ? Tn : Tn + 1;
   const int LS = Tn + 1;  // floats per row of log_deriv (the two-kernel pair's tensor)
-  const float *pxb = px + (size_t)g.b * S * T1;
-  const float *pyb = py + (size_t)g.b * (S + 1) * Tn;
-  float *pb = kWriteP ? p + (size_t)g.b * (S + 1) * (Tn + 1) : nullptr;
+  const GFloat *pxb = Global(px) + (size_t)g.b * S * T1;
+  GFloat *pb = kWriteP ? Global(p) + (size_t)g.b * (S + 1) * (Tn + 1) : nullptr;
   // (kBidir: the run of blocks of this chunk of this half in the launch's slab)
   float *ldb = !kKeep ? nullptr
                : kBidir ? log_deriv + (size_t)g.b * SlabFloatsPerSequence(S, Tn, modified) +
@@ -782,7 +791,7 @@ __device__ __forceinline__ void MiForwardChunk(
       // where own columns j .. j+3 of the row lie: the mirrored half stores the lattice's cell
       // (ns - row, nt - column) one column to the right of its place, columns descending
       const ptrdiff_t at = (ptrdiff_t)(g.s0 + row_i) * LS + g.t0 + j;
-      float *dst = pb + at;
+      GFloat *dst = pb + at;
       float ld[4] = {0.f, 0.f, 0.f, 0.f};
       if (kKeep) {
         // What arrived along px at each step: for row 0 of the chunk the edge wavefront's sum
@@ -1063,7 +1072,7 @@ struct ZeroGeom {
 __device__ __forceinline__ void ZeroItem(const ZeroGeom &z, int r, int c) {
   const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
   if (r < z.S && c < z.T1) {
-    float *dst = z.gx + (size_t)r * z.T1 + c;
+    GFloat *dst = Global(z.gx) + (size_t)r * z.T1 + c;
     const bool row_in = r >= z.xs0 && r < z.xs1;
     if (row_in && c >= z.xt0 && c + 3 < z.xt1) {
       // the sweep assigns all four
@@ -1076,7 +1085,7 @@ __device__ __forceinline__ void ZeroItem(const ZeroGeom &z, int r, int c) {
     }
   }
   if (r <= z.S && c < z.Tn) {
-    float *dst = z.gy + (size_t)r * z.Tn + c;
+    GFloat *dst = Global(z.gy) + (size_t)r * z.Tn + c;
     const bool row_in = r >= z.xs0 && r < z.ys1;
     if (row_in && c >= z.xt0 && c + 3 < z.yt1) {
       // the sweep assigns all four
@@ -1112,12 +1121,12 @@ __device__ __forceinline__ void MiBackwardChunk(
   g.c = chunk;
   const int T1 = modified ? Tn : Tn + 1;
   const int off = modified ? -1 : 0;
-  float *gxb = px_grad + (size_t)g.b * S * T1;
-  float *gyb = py_grad + (size_t)g.b * (S + 1) * Tn;
+  GFloat *gxb = Global(px_grad) + (size_t)g.b * S * T1;
+  GFloat *gyb = Global(py_grad) + (size_t)g.b * (S + 1) * Tn;
 
   if (zero_only) {
     ZeroGeom zg;
-    zg.gx = gxb; zg.gy = gyb; zg.S = S; zg.T1 = T1; zg.Tn = Tn;
+    zg.gx = px_grad + (size_t)g.b * S * T1; zg.gy = py_grad + (size_t)g.b * (S + 1) * Tn; zg.S = S; zg.T1 = T1; zg.Tn = Tn;
     zg.xs0 = box.ok ? box.s0 : 0; zg.xs1 = box.ok ? box.s1 : 0;
     zg.xt0 = box.ok ? box.t0 : 0; zg.xt1 = box.ok ? box.t1 + off + 1 : 0;
     zg.ys1 = box.ok ? box.s1 + 1 : 0; zg.yt1 = box.ok ? box.t1 : 0;
@@ -1337,9 +1346,9 @@ __device__ __forceinline__ void MiBackwardChunk(
       // OUT of that lattice cell along px / py: both gradients land at that cell's own index,
       // columns descending.
       const int sm = g.s0 + g.ns - row_i;
-      float *dy = mirror ? gyb + (ptrdiff_t)sm * Tn + g.t0 + g.nt - jd - 3
+      GFloat *dy = mirror ? gyb + (ptrdiff_t)sm * Tn + g.t0 + g.nt - jd - 3
                          : gyb + (ptrdiff_t)s * Tn + g.t0 + jd - 1;
-      float *dx = mirror ? gxb + (ptrdiff_t)sm * T1 + g.t0 + g.nt - jd - 3
+      GFloat *dx = mirror ? gxb + (ptrdiff_t)sm * T1 + g.t0 + g.nt - jd - 3
                          : gxb + (ptrdiff_t)(s - 1) * T1 + g.t0 + jd - 1 + g.skew;
       if (inner) {  // uniform: every cell of the block has both edges inside the box
         const float4 c4 = make_float4(cv[0], cv[1], cv[2], cv[3]), h4 = make_float4(hv[0], hv[1], hv[2], hv[3]);
@@ -1668,7 +1677,7 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiBidirKernel(const Bidir
   __shared__ Box boxes[kBoxes];
   if (threadIdx.x == 0) {
     ts.k = k;
-    sh.ticket = atomicAdd(&k.hdr->ticket, 1u);
+    sh.ticket = __hip_atomic_fetch_add(Global(&k.hdr->ticket), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   for (int i = (int)threadIdx.x - kWave; i >= 0 && i < min(k.B, kBoxes); i += blockDim.x - kWave)
     boxes[i] = LoadBox(k.boundary, i, k.S, k.Tn);
@@ -1681,7 +1690,7 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiBidirKernel(const Bidir
   for (bool first = true;; first = false) {
     if (!first) {
       __syncthreads();  // the previous task's last LDS reads are done, its stores complete
-      if (threadIdx.x == 0) sh.ticket = atomicAdd(&k.hdr->ticket, 1u);
+      if (threadIdx.x == 0) sh.ticket = __hip_atomic_fetch_add(Global(&k.hdr->ticket), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
     const unsigned ticket = sh.ticket;
@@ -1730,7 +1739,7 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiBidirKernel(const Bidir
       // before this barrier: whichever compute unit sweeps this chunk back will see them
       __syncthreads();
       if (threadIdx.x == 0)
-        __hip_atomic_fetch_add(cw.stored, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_fetch_add(Global(cw.stored), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       continue;
     }
 
@@ -1762,12 +1771,12 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiBidirKernel(const Bidir
     // task to say so puts them back into their initial state.
     __syncthreads();
     if (threadIdx.x == 0)
-      sh.last = __hip_atomic_fetch_add(cw.depart, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
+      sh.last = __hip_atomic_fetch_add(Global(cw.depart), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
                 kSentinel + per_seq;
     __syncthreads();
     if (sh.last)
       for (int i = threadIdx.x; i < cw.words; i += blockDim.x)
-        __hip_atomic_store(reinterpret_cast<unsigned *>(cw.depart) - 1 + i, kSentinel, __ATOMIC_RELAXED,
+        __hip_atomic_store(Global(reinterpret_cast<unsigned *>(cw.depart) - 1 + i), kSentinel, __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_AGENT);
   }
   if (threadIdx.x == 0) FinishWorkgroup(k.hdr, gridDim.x);
