@@ -705,7 +705,9 @@ __device__ __forceinline__ void MiForwardChunk(
   };
   // a loaded quad in ascending order of own columns (`at` = the index it was loaded from)
   auto unmirror = [&](float4 v, int at, bool rim) {
-    if (rim && g.b == 0) v = ShiftQuad(v, at);  // the only sequence whose rows can start the tensor
+    // (a quad can start in front of the tensor for the first sequences: always for the first
+    // row of sequence 0, and for later ones where a sequence is shorter than a quad)
+    if (rim) v = ShiftQuad(v, at);
     return mirror ? Rev4(v) : v;
   };
   // `inner` is uniform over the workgroup: the masking code for blocks on the rim of the box is
@@ -1275,7 +1277,7 @@ __device__ __forceinline__ void MiBackwardChunk(
       float4 qd = AsFloat4(r.d[it]);
       float4 qs = kKept ? qd : AsFloat4(r.s[it]), qx = kKept ? qd : AsFloat4(r.x[it]);
       // (the slab's quads are whole by construction)
-      if (!kBidir && !inner && g.b == 0) {  // the only sequence whose rows can start the tensor
+      if (!kBidir && !inner) {  // (a quad can start in front of the tensor: see ShiftQuad)
         asm volatile("");
         const int jd0 = kb * kW + 4 * mm - q * g.skew;
         qd = ShiftQuad(qd, idx_d[it] + jd0);

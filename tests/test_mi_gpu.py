@@ -157,6 +157,28 @@ def test_random_multi_chunk_cases_vs_oracle(device):
 
 
 @pytest.mark.parametrize("modified", [False, True])
+def test_sequences_shorter_than_a_quad(device, modified):
+    """Lattices of one to three cells a side, several to a batch: the 16-byte loads of every
+    sequence then start in front of the sequence's own first element (for the mirrored half of the
+    single launch up to three floats back), for the first sequences in front of the tensor."""
+    rng = np.random.default_rng(77)
+    for S, T in ((1, 1), (1, 2), (2, 2), (1, 3), (2, 3), (3, 3)):
+        if modified and T < S:
+            continue
+        B = 7
+        T1 = T if modified else T + 1
+        px = rng.standard_normal((B, S, T1)).astype(np.float32)
+        py = rng.standard_normal((B, S + 1, T)).astype(np.float32)
+        full = np.tile(np.array([[0, 0, S, T]], np.int64), (B, 1))
+        for bd in (None, full):
+            if bd is None and not modified:
+                px[:, :, -1] = -np.inf
+            ans, p = omi.mi_forward(px, py, bd)
+            gx, gy = omi.mi_backward(px, py, bd, p)
+            check(f"S{S}T{T}", px, py, bd, (ans, p, gx, gy), device)
+
+
+@pytest.mark.parametrize("modified", [False, True])
 def test_wide_lattice_more_rows_than_a_wavefront(device, modified):
     # S+1 > 256 exercises the row loop of a workgroup; long T exercises many steps.
     rng = np.random.default_rng(5)
