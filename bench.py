@@ -36,7 +36,7 @@ BWD_BYTES_PER_CELL = 16
 # HBM bytes per launch on the default workload, from rocprofv3's FETCH_SIZE / WRITE_SIZE counters
 # scaled by a 256 MiB device copy (profiles/mi_bidir_kernel_c4_hbm_traffic.md).  Reported only
 # for the default shape; any other --B/--S/--T prints null.
-MEASURED_TRAFFIC_BYTES = {"mi_forward_backward": 160290000, "mi_forward": 50140000, "mi_backward": 69280000}
+MEASURED_TRAFFIC_BYTES = {"mi_forward_backward": 134950000, "mi_forward": 50140000, "mi_backward": 69270000}
 MEASURED_TRAFFIC_BYTES_PLAIN_PAIR = {"mi_forward": 50060000, "mi_backward": 86030000}  # --no-keep
 
 
