@@ -147,8 +147,9 @@ K2AMD_API int k2amd_mi_backward_kept(const void *px, const void *py, const int64
  * k2amd_mi_forward_backward_supported(...) says whether a call will be served (1) or returns
  * K2AMD_ERR_UNSUPPORTED (0; use the two calls).  k2amd_mi_forward_backward_advised(...) says
  * whether it is also the faster way on the current device (1): it is while the device has a compute
- * unit for every half-sweep, 2 * B * ceil((S+1)/64) of them, at once; beyond that the two calls,
- * whose kernels share compute units, take less time, and a host that has the choice makes them. */
+ * unit for every two of the 2 * B * ceil((S+1)/64) half-sweeps, and on long lattices (T >= 1000) at
+ * any batch size; otherwise the two calls, whose kernels share compute units, take less time (by
+ * up to a fifth), and a host that has the choice makes them. */
 K2AMD_API int k2amd_mi_forward_backward_supported(int B, int S, int T, int modified, int dtype,
                                         int has_workspace);
 K2AMD_API int k2amd_mi_forward_backward_advised(int B, int S, int T, int modified, int dtype,

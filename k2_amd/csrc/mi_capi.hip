@@ -207,7 +207,7 @@ int k2amd_mi_forward_backward_supported(int B, int S, int T, int modified, int d
 int k2amd_mi_forward_backward_advised(int B, int S, int T, int modified, int dtype,
                                       int has_workspace) {
   return k2amd_mi_forward_backward_supported(B, S, T, modified, dtype, has_workspace) &&
-         (MiFusedAdvised(B, S) || PathIs("single-launch"));
+         (MiFusedAdvised(B, S, T) || PathIs("single-launch"));
 }
 
 size_t k2amd_mi_forward_backward_scratch_bytes(int B, int S, int T, int modified, int dtype) {

@@ -1897,14 +1897,17 @@ bool MiFusedSupports(int B, int S, int Tn, int modified) {
 }
 
 // Whether the single launch is the faster way to run both recursions of this shape on the current
-// device: it is while every forward half-sweep finds a compute unit at once (the launch then lasts
-// as long as one sequence's two half-length fronts).  With more half-sweeps than units they queue,
-// one workgroup to a unit, and the two launches, which place two workgroups on a unit, take less
-// time (B = 128 at S = 200, T = 1000: 181 us against 201).
-bool MiFusedAdvised(int B, int S) {
+// device.  It is, by far, while every forward half-sweep finds a compute unit at once (the launch
+// then lasts as long as one sequence's two half-length fronts: B = 32, S = 200, T = 1000 takes 58 us
+// against 79 for the pair), and still by a few per cent with up to two half-sweeps per unit.  With
+// more of them they queue, one workgroup to a unit, where the pair places two: the pair then wins
+// on short lattices (B = 512, S = 100, T = 500: 199 us against 225; T = 700: 474 against 493) and
+// the single launch on long ones (B = 512 and 1024, S = 200, T = 1000: 625 against 645 us, 1263
+// against 1278).
+bool MiFusedAdvised(int B, int S, int Tn) {
   const int units = ComputeUnits();
   const long long nchunks = (S + 1 + kRows - 1) / kRows;
-  return units > 0 && 2ll * B * nchunks <= units;
+  return units > 0 && (2ll * B * nchunks <= 2ll * units || Tn >= 1000);
 }
 
 // Floats of scratch per call of the single launch: the log-derivatives of both halves of every

@@ -37,7 +37,7 @@ int MiBackwardFast(const float *px, const float *p, const float *log_deriv,
 // read, by the launch itself).  MiFusedSupports: whether that kernel serves the shape.
 bool MiFusedSupports(int B, int S, int Tn, int modified);
 // Whether it is also the faster way on the current device (else: the two launches).
-bool MiFusedAdvised(int B, int S);
+bool MiFusedAdvised(int B, int S, int Tn);
 size_t MiFusedScratchElems(int B, int S, int Tn, int modified);
 int MiForwardBackwardFast(const float *px, const float *py, const int64_t *boundary, float *ans,
                           float *scratch, float *ans_grad, float *px_grad, float *py_grad, int B,

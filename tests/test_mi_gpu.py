@@ -434,8 +434,8 @@ def test_single_launch_serves_any_batch_and_says_what_it_does_not(device):
     np.testing.assert_allclose(scores.cpu().numpy(), a, rtol=1e-4, atol=1e-5)
     np.testing.assert_allclose(gx.cpu().numpy(), wx, rtol=1e-4, atol=1e-5)
     np.testing.assert_allclose(gy.cpu().numpy(), wy, rtol=1e-4, atol=1e-5)
-    # With more half-sweeps than compute units the two launches are the faster way, the library says
-    # so, and the Python layer follows: its results are then the pair's bits.
+    # With many more (short) half-sweeps than compute units the two launches are the faster way, the
+    # library says so, and the Python layer follows: its results are then the pair's bits.
     assert capi.mi_forward_backward_advised(bx[:4].contiguous(), by[:4].contiguous())
     assert not capi.mi_forward_backward_advised(bx, by)
     assert not capi.mi_forward_backward_advised(px, py)
