@@ -65,6 +65,42 @@ def _lattice_buffers(px: Tensor, py: Tensor, want_grad: bool) -> Tuple[Optional[
     return buf, None
 
 
+def recursion_values(px: Tensor, py: Tensor, boundary: Optional[Tensor], want_grad: bool):
+    """(scores, px_grad, py_grad) of contiguous px, py: the recursion and, when gradients may be
+    wanted, the backward recursion with ans_grad = 1 straight away, as the reference's Function does
+    (k2/python/k2/mutual_information.py:157-169).  No autograd here: the Function below and the
+    loss nodes of rnnt_loss.py, which are autograd nodes themselves, both call it."""
+    B = px.shape[0]
+    px_grad, py_grad = None, None
+    if want_grad and _single_launch(px, py):
+        # both recursions in one launch, seeded with 1 per sequence
+        (ans, px_grad, py_grad) = native.mutual_information_forward_backward(px, py, boundary, None)
+    else:
+        # the backward runs right away, so the forward can hand it the px-edge log-derivatives
+        # instead of p (which nothing else reads)
+        p, log_deriv = _lattice_buffers(px, py, want_grad)
+        ans = native.mutual_information_forward(px, py, boundary, p, log_deriv)
+        if want_grad:
+            ans_grad = torch.ones(B, device=px.device, dtype=px.dtype)
+            (px_grad, py_grad) = native.mutual_information_backward(px, py, boundary, p, ans_grad,
+                                                                    log_deriv)
+    return ans, px_grad, py_grad
+
+
+def check_recursion_inputs(px: Tensor, py: Tensor, boundary: Optional[Tensor]) -> None:
+    """The asserts of k2/python/k2/mutual_information.py:268-289."""
+    assert px.ndim == 3, px.shape
+    B, S, T1 = px.shape
+    T = py.shape[-1]
+    assert px.shape[-1] in [T, T + 1], (px.shape, T)
+    assert py.shape == (B, S + 1, T), (py.shape, B, S, T)
+    assert px.dtype == py.dtype, (px.dtype, py.dtype)
+    if boundary is not None:
+        assert boundary.dtype == torch.int64, boundary.dtype
+        assert boundary.shape == (B, 4), (boundary.shape, B)
+        _check_boundary(boundary, S, T)
+
+
 class MutualInformationRecursionFunction(torch.autograd.Function):
     """Mirrors k2/python/k2/mutual_information.py:24-182: the forward runs the recursion and, when
     gradients may be wanted, the backward recursion with ans_grad = 1 straight away; autograd's
@@ -81,19 +117,7 @@ class MutualInformationRecursionFunction(torch.autograd.Function):
             assert boundary.shape == (B, 4), (boundary.shape, B)
 
         want_grad = return_grad or px.requires_grad or py.requires_grad
-        px_grad, py_grad = None, None
-        if want_grad and _single_launch(px, py):
-            # both recursions in one launch, seeded with 1 per sequence
-            (ans, px_grad, py_grad) = native.mutual_information_forward_backward(px, py, boundary, None)
-        else:
-            # the backward runs right away, so the forward can hand it the px-edge log-derivatives
-            # instead of p (which nothing else reads)
-            p, log_deriv = _lattice_buffers(px, py, want_grad)
-            ans = native.mutual_information_forward(px, py, boundary, p, log_deriv)
-            if want_grad:
-                ans_grad = torch.ones(B, device=px.device, dtype=px.dtype)
-                (px_grad, py_grad) = native.mutual_information_backward(px, py, boundary, p, ans_grad,
-                                                                        log_deriv)
+        ans, px_grad, py_grad = recursion_values(px, py, boundary, want_grad)
         if want_grad:
             ctx.save_for_backward(px_grad, py_grad)
         assert len(pxy_grads) == 2, len(pxy_grads)
@@ -122,17 +146,7 @@ def mutual_information_recursion(
     (scores, (px_grad, py_grad)) when return_grad is set, the grads being the occupation
     probabilities d scores.sum() / d px, py.
     """
-    assert px.ndim == 3, px.shape
-    B, S, T1 = px.shape
-    T = py.shape[-1]
-    assert px.shape[-1] in [T, T + 1], (px.shape, T)
-    assert py.shape == (B, S + 1, T), (py.shape, B, S, T)
-    assert px.dtype == py.dtype, (px.dtype, py.dtype)
-    if boundary is not None:
-        assert boundary.dtype == torch.int64, boundary.dtype
-        assert boundary.shape == (B, 4), (boundary.shape, B)
-        _check_boundary(boundary, S, T)
-
+    check_recursion_inputs(px, py, boundary)
     px, py = px.contiguous(), py.contiguous()
     pxy_grads = [None, None]
     scores = MutualInformationRecursionFunction.apply(px, py, pxy_grads, boundary, return_grad)

@@ -11,7 +11,8 @@ import torch
 from torch import Tensor
 
 from . import capi, native
-from .mutual_information import boundary_rows, mutual_information_recursion
+from .mutual_information import (boundary_rows, check_recursion_inputs, mutual_information_recursion,
+                                 recursion_values)
 
 _RNNT_TYPES = ("regular", "modified", "constrained")
 
@@ -116,11 +117,16 @@ class _Scores(torch.autograd.Function):
     recursion has the occupation probabilities ready when it returns (as the reference's does,
     k2/python/k2/mutual_information.py:162-169); what arrives at the scores in the backward pass
     scales them per sequence inside the builder's gradient kernels (``seq_scale``), where the
-    reference runs two elementwise products first (mutual_information.py:177-182).  Returns
-    (scores, px_grad, py_grad); the last two are None unless asked for or needed."""
+    reference runs two elementwise products first (mutual_information.py:177-182).  The node also
+    negates and reduces the scores (the reference's last two torch ops, rnnt_loss.py:331-338): a
+    graph of one node instead of three costs the host some 20 us less per step, which is what the
+    small configurations are bound by.  Returns (loss, px_grad, py_grad); the last two are None
+    unless asked for or needed."""
 
     @staticmethod
-    def forward(ctx, kind, rnnt_type, delay_penalty, return_grad, *args):
+    def forward(ctx, kind, rnnt_type, delay_penalty, return_grad, reduction, *args):
+        if reduction not in ("none", "mean", "sum"):
+            raise ValueError(f"reduction should be ('none' | 'mean' | 'sum'), given {reduction}")
         boundary = {"joint": 4, "joiner": 8}.get(kind, 5)
         boundary = args[boundary]
         need = return_grad or any(ctx.needs_input_grad)
@@ -151,21 +157,28 @@ class _Scores(torch.autograd.Function):
             saved = (logits, norm)
         if delay_penalty > 0.0:
             px = _delay_penalty(px, boundary, rnnt_type, delay_penalty)
-        out = mutual_information_recursion(px=px, py=py, boundary=boundary, return_grad=need)
-        scores, (px_grad, py_grad) = out if need else (out, (None, None))
+        check_recursion_inputs(px, py, boundary)
+        scores, px_grad, py_grad = recursion_values(px.contiguous(), py.contiguous(), boundary, need)
         ctx.kind, ctx.args, ctx.n_saved = kind, args, len(saved)
+        ctx.reduction, ctx.batch = reduction, scores.shape[0]
         if need:
             ctx.save_for_backward(*saved, px_grad, py_grad)
             ctx.mark_non_differentiable(px_grad, py_grad)
-        return scores, px_grad, py_grad
+        return _reduce(scores, reduction), px_grad, py_grad
 
     @staticmethod
-    def backward(ctx, scores_grad, _px_grad_grad, _py_grad_grad):
+    def backward(ctx, loss_grad, _px_grad_grad, _py_grad_grad):
         args = ctx.args
-        if scores_grad is None:
-            return (None,) * (4 + len(args))
+        if loss_grad is None:
+            return (None,) * (5 + len(args))
         saved, (px_grad, py_grad) = ctx.saved_tensors[:ctx.n_saved], ctx.saved_tensors[ctx.n_saved:]
-        scale = scores_grad.contiguous()
+        # what reaches each sequence's score: the loss is minus the scores, their sum or their mean
+        if ctx.reduction == "none":
+            scale = loss_grad.neg()
+        else:
+            # (a division for the mean, as torch's own backward of it: the same bits)
+            scale = loss_grad.neg() if ctx.reduction == "sum" else loss_grad / float(-ctx.batch)
+            scale = scale.expand(ctx.batch).contiguous()
         if ctx.kind == "simple":
             _, _, symbols, termination_symbol, rnnt_code, boundary = args
             grads = native.logprobs_simple_backward(px_grad, py_grad, symbols, boundary, saved,
@@ -186,7 +199,7 @@ class _Scores(torch.autograd.Function):
             grads = (native.logprobs_pruned_backward(saved[0], saved[1], px_grad, py_grad, symbols,
                                                      ranges, boundary, termination_symbol, rnnt_code,
                                                      hat, scale),)
-        return (None, None, None, None) + tuple(grads) + (None,) * (len(args) - len(grads))
+        return (None, None, None, None, None) + tuple(grads) + (None,) * (len(args) - len(grads))
 
 
 class _PruneGather(torch.autograd.Function):
@@ -270,9 +283,8 @@ def rnnt_loss_simple(
 ) -> Union[Tensor, Tuple[Tensor, Tuple[Tensor, Tensor]]]:
     """k2.rnnt_loss_simple (k2/python/k2/rnnt_loss.py:228-338)."""
     args = _simple_args(lm, am, symbols, termination_symbol, rnnt_type, boundary)
-    negated_loss, px_grad, py_grad = _Scores.apply("simple", rnnt_type, float(delay_penalty),
-                                                   bool(return_grad), *args)
-    loss = _reduce(negated_loss, reduction)
+    loss, px_grad, py_grad = _Scores.apply("simple", rnnt_type, float(delay_penalty),
+                                           bool(return_grad), reduction, *args)
     return (loss, (px_grad, py_grad)) if return_grad else loss
 
 
@@ -311,8 +323,7 @@ def rnnt_loss(
 ) -> Tensor:
     """k2.rnnt_loss (k2/python/k2/rnnt_loss.py:450-540)."""
     args = _joint_args(logits, symbols, termination_symbol, rnnt_type, boundary)
-    negated_loss = _Scores.apply("joint", rnnt_type, float(delay_penalty), False, *args)[0]
-    return _reduce(negated_loss, reduction)
+    return _Scores.apply("joint", rnnt_type, float(delay_penalty), False, reduction, *args)[0]
 
 
 def _monotonic_lower_bound(x: Tensor) -> Tensor:
@@ -475,8 +486,7 @@ def rnnt_loss_pruned(
     builder to get_hat_logprobs_pruned (:1430-1447)."""
     checked = _hat_args if use_hat_loss else _pruned_args
     args = checked(logits, symbols, ranges, termination_symbol, boundary, rnnt_type)
-    negated_loss = _Scores.apply("pruned", rnnt_type, float(delay_penalty), False, *args)[0]
-    return _reduce(negated_loss, reduction)
+    return _Scores.apply("pruned", rnnt_type, float(delay_penalty), False, reduction, *args)[0]
 
 
 def rnnt_loss_pruned_joiner(
@@ -516,8 +526,7 @@ def rnnt_loss_pruned_joiner(
     _validate_st_lengths(S, T, rnnt_type == "regular", boundary)
     args = (am, lm, _dev_i64(ranges, am), weight, bias, _dev_i64(symbols, am), int(termination_symbol),
             capi.RNNT_TYPES[rnnt_type], _dev_i64(boundary, am), capi.JOINER_PRECISIONS[precision])
-    negated_loss = _Scores.apply("joiner", rnnt_type, float(delay_penalty), False, *args)[0]
-    return _reduce(negated_loss, reduction)
+    return _Scores.apply("joiner", rnnt_type, float(delay_penalty), False, reduction, *args)[0]
 
 
 def get_rnnt_logprobs_smoothed(
