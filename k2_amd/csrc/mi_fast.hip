@@ -1319,45 +1319,74 @@ __device__ __forceinline__ void MiBackwardChunk(
   // The gradient G a cell at position m saw is what the chain left at position m + 1, which for
   // the last position of a block lies in the block to its right (computed one iteration earlier;
   // its slot in g is not written again before the chain reaches the block two to the left).
+  // Where a storer lane's two items (rows mq and mq + 32, quad mm) of block 0 go; block kb lies
+  // kb * 32 floats further on (back, in the mirrored half).  Worked out once: per block the
+  // storers only add.
+  //   py_grad[s][t0 + jd - 1 + e]   for destination columns 1..nt
+  //   px_grad[s-1][t0 + jd - 1 + skew + e]   for destination columns (1 - skew)..nt
+  // The mirrored half's destination cell (row, column) is the lattice's cell (ns - row,
+  // nt - column), and what flows into it along its px / py edge is the flow OUT of that lattice
+  // cell along px / py: both gradients land at that cell's own index, columns descending.
+  // (Set by the storers when their loop starts, and their last block is stored inside their
+  // branch: pointers that were live where the roles part would cost every role their registers.)
+  GFloat *dy0[2], *dx0[2];
+  const ptrdiff_t block_step = mirror ? -kW : kW;
+  auto storer_bases = [&]() {
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+      const int q = mq + 32 * it;
+      const int row_i = g.row0 + q;
+      const int jd = 4 * mm - q * g.skew;
+      const int s = g.s0 + row_i, sm = g.s0 + g.ns - row_i;
+      dy0[it] = mirror ? gyb + (ptrdiff_t)sm * Tn + g.t0 + g.nt - jd - 3 : gyb + (ptrdiff_t)s * Tn + g.t0 + jd - 1;
+      dx0[it] = mirror ? gxb + (ptrdiff_t)sm * T1 + g.t0 + g.nt - jd - 3
+                       : gxb + (ptrdiff_t)(s - 1) * T1 + g.t0 + jd - 1 + g.skew;
+    }
+  };
   auto store_block = [&](int kb) {
     if (kb >= g.nblocks) return;
     const bool inner = interior(kb);
+    const int ring = __builtin_amdgcn_readfirstlane(kb % 3);
+    const int pq = ring * kQuadsPerBlock + mm;
+    const int pq_right = mm + 1 < kQuadsPerBlock ? pq + 1 : (ring == 2 ? 0 : ring + 1) * kQuadsPerBlock;
+    // Both items' operands are asked for before either is used (one LDS latency per block) where
+    // the registers allow it: the plain backward's loaders hold three tensors' loads, and its
+    // kernel must stay within the registers that let two workgroups share a compute unit.
+    float4 e4[2], o4[2], g4[2], gr[2];
+    auto fetch = [&](int it) {
+      const int q = mq + 32 * it;
+      e4[it] = lds.e[q][pq];
+      o4[it] = lds.ome[q][pq];
+      g4[it] = lds.g[q][pq];
+      gr[it] = lds.g[q][pq_right];
+      // Only three floats of g4 and one of gr are used, and the compiler would fetch just those
+      // with 4-byte reads: lanes that are whole quads apart then share 16 of the 64 banks (4-way
+      // conflicts).  Whole-quad reads are conflict-free.
+      asm volatile("" : "+v"(g4[it].x), "+v"(g4[it].y), "+v"(g4[it].z), "+v"(g4[it].w));
+      asm volatile("" : "+v"(gr[it].x), "+v"(gr[it].y), "+v"(gr[it].z), "+v"(gr[it].w));
+    };
+    if (kKept) {
+      fetch(0);
+      fetch(1);
+    }
 #pragma unroll
     for (int it = 0; it < 2; ++it) {
       const int q = mq + 32 * it;
       const int row_i = g.row0 + q;
       if (row_i > g.ns) continue;
-      const int pq = (kb % 3) * kQuadsPerBlock + mm;
-      const int pq_right = mm + 1 < kQuadsPerBlock ? pq + 1 : ((kb + 1) % 3) * kQuadsPerBlock;
-      const float4 e4 = lds.e[q][pq], o4 = lds.ome[q][pq];
-      float4 g4 = lds.g[q][pq], gr = lds.g[q][pq_right];
-      // Only three floats of g4 and one of gr are used, and the compiler would fetch just those
-      // with 4-byte reads: lanes that are whole quads apart then share 16 of the 64 banks (4-way
-      // conflicts).  Whole-quad reads are conflict-free.
-      asm volatile("" : "+v"(g4.x), "+v"(g4.y), "+v"(g4.z), "+v"(g4.w));
-      asm volatile("" : "+v"(gr.x), "+v"(gr.y), "+v"(gr.z), "+v"(gr.w));
-      const float gv[4] = {g4.y, g4.z, g4.w, gr.x};
-      const float hv[4] = {e4.x * gv[0], e4.y * gv[1], e4.z * gv[2], e4.w * gv[3]};
-      const float cv[4] = {o4.x * gv[0], o4.y * gv[1], o4.z * gv[2], o4.w * gv[3]};
-      const int jd = kb * kW + 4 * mm - q * g.skew;
-      const int s = g.s0 + row_i;
-      // py_grad[s][t0 + jd - 1 + e]   for destination columns 1..nt
-      // px_grad[s-1][t0 + jd - 1 + skew + e]   for destination columns (1 - skew)..nt
-      // The mirrored half's destination cell (row, column) is the lattice's cell
-      // (ns - row, nt - column), and what flows into it along its px / py edge is the flow
-      // OUT of that lattice cell along px / py: both gradients land at that cell's own index,
-      // columns descending.
-      const int sm = g.s0 + g.ns - row_i;
-      GFloat *dy = mirror ? gyb + (ptrdiff_t)sm * Tn + g.t0 + g.nt - jd - 3
-                         : gyb + (ptrdiff_t)s * Tn + g.t0 + jd - 1;
-      GFloat *dx = mirror ? gxb + (ptrdiff_t)sm * T1 + g.t0 + g.nt - jd - 3
-                         : gxb + (ptrdiff_t)(s - 1) * T1 + g.t0 + jd - 1 + g.skew;
+      if (!kKept) fetch(it);
+      const float gv[4] = {g4[it].y, g4[it].z, g4[it].w, gr[it].x};
+      const float hv[4] = {e4[it].x * gv[0], e4[it].y * gv[1], e4[it].z * gv[2], e4[it].w * gv[3]};
+      const float cv[4] = {o4[it].x * gv[0], o4[it].y * gv[1], o4[it].z * gv[2], o4[it].w * gv[3]};
+      GFloat *dy = dy0[it] + kb * block_step;
+      GFloat *dx = dx0[it] + kb * block_step;
       if (inner) {  // uniform: every cell of the block has both edges inside the box
         const float4 c4 = make_float4(cv[0], cv[1], cv[2], cv[3]), h4 = make_float4(hv[0], hv[1], hv[2], hv[3]);
         StoreQuad(dy, kBidir && mirror ? Rev4(c4) : c4);
         if (row_i >= 1) StoreQuad(dx, kBidir && mirror ? Rev4(h4) : h4);
       } else {
         asm volatile("");  // keeps this path a branch of its own
+        const int jd = kb * kW + 4 * mm - q * g.skew;
 #pragma unroll
         for (int e = 0; e < 4; ++e)
           if (jd + e >= 1 && jd + e <= g.nt && (!kBidir || jd + e + q * g.skew <= n_last))
@@ -1523,10 +1552,12 @@ __device__ __forceinline__ void MiBackwardChunk(
 #pragma unroll
     for (int i = 0; i < kSets; ++i) wait_all(sets[i]);
   } else if (role == kStorer) {
+    storer_bases();
     for (int kb = top; kb >= 0; --kb) {
       store_block(kb + 1);
       LdsBarrier();
     }
+    store_block(0);
   } else if (role == kEdge) {
     for (int kb = top; kb >= 0; --kb) {
       publish_block(kb + 1);
@@ -1535,7 +1566,6 @@ __device__ __forceinline__ void MiBackwardChunk(
     }
   }
   K2AMD_TRACE_MARK(half, 6);
-  if (role == kStorer) store_block(0);
   if (role == kEdge) publish_block(0);
   if (overwrite_ans_grad && ans_grad != nullptr && role == kChain && g.c == 0 && lane == 0 && !mirror)
     ans_grad[g.b] = GaveUp(hdr) ? __builtin_nanf("") : g_origin;
