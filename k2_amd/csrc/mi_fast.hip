@@ -375,6 +375,8 @@ struct CutShared {
   float total;   // the sequence's score, from the join of this task
   float scale;   // the gradient of the sequence's score
   int split_ok;  // the score is finite: the halves sweep back from the cut
+  int departed_set;   // the task has already said that it is through with the cut words,
+  unsigned departed;  // and this is what the counter held before
   int last;
   unsigned ticket;
 };
@@ -1469,6 +1471,8 @@ __device__ __forceinline__ void MiBackwardChunk(
 
   const int top = g.nblocks - 1;
   BwdRegs sets[kSets];
+  unsigned departed_early = 0;  // (chain wavefront, lane 0, single launch)
+  auto sh_of = [](const BidirJoin *j) { return j->sh; };
   if (kBidir) {
     // The chain wavefront joins the halves on the cut; the loaders wait for the forward sweeps'
     // last log-derivatives (all of the sequence's: the counter is per sequence) and fetch the
@@ -1487,6 +1491,10 @@ __device__ __forceinline__ void MiBackwardChunk(
         sh.scale = scale;
         sh.split_ok = ok;
         if (join->ans != nullptr && ok) *join->ans = GaveUp(hdr) ? __builtin_nanf("") : total;
+        // This task is through with the cut words: said now, so that the count is back by the
+        // time the sweep ends (it is looked at there; a trip to memory off the launch's tail).
+        departed_early = __hip_atomic_fetch_add(Global(join->cw.depart), 1u, __ATOMIC_RELAXED,
+                                                __HIP_MEMORY_SCOPE_AGENT);
       }
       K2AMD_TRACE_MARK(half, 1);
     } else if (role == kLoader) {
@@ -1503,6 +1511,10 @@ __device__ __forceinline__ void MiBackwardChunk(
       if (role == kLoader) {
 #pragma unroll
         for (int i = 0; i < kSets; ++i) wait_all(sets[i]);
+      }
+      if (threadIdx.x == 0) {
+        sh.departed = departed_early;
+        sh.departed_set = 1;
       }
       return;
     }
@@ -1566,6 +1578,10 @@ __device__ __forceinline__ void MiBackwardChunk(
     }
   }
   K2AMD_TRACE_MARK(half, 6);
+  if (kBidir && threadIdx.x == 0) {
+    sh_of(join)->departed = departed_early;
+    sh_of(join)->departed_set = 1;
+  }
   if (role == kEdge) publish_block(0);
   if (overwrite_ans_grad && ans_grad != nullptr && role == kChain && g.c == 0 && lane == 0 && !mirror)
     ans_grad[g.b] = GaveUp(hdr) ? __builtin_nanf("") : g_origin;
@@ -1777,6 +1793,7 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiBidirKernel(const Bidir
 
     // Backward sweep of a chunk, or the sequence's last task: both start from the cut, whose
     // words they wait for themselves.
+    if (threadIdx.x == 0) sh.departed_set = 0;
     if (!last) {
       if (threadIdx.x == 0 && !mirror && chunk == 0 && !box.ok) k.ans[seq] = __builtin_nanf("");
       if (box.ok)
@@ -1802,9 +1819,13 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiBidirKernel(const Bidir
     // This task is through with the sequence's cut words (where it read them at all).  The last
     // task to say so puts them back into their initial state.
     __syncthreads();
-    if (threadIdx.x == 0)
-      sh.last = __hip_atomic_fetch_add(Global(cw.depart), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
-                kSentinel + per_seq;
+    if (threadIdx.x == 0) {
+      const unsigned before = sh.departed_set
+                                  ? sh.departed
+                                  : __hip_atomic_fetch_add(Global(cw.depart), 1u, __ATOMIC_RELAXED,
+                                                           __HIP_MEMORY_SCOPE_AGENT);
+      sh.last = before == kSentinel + per_seq;
+    }
     __syncthreads();
     if (sh.last)
       for (int i = threadIdx.x; i < cw.words; i += blockDim.x)
