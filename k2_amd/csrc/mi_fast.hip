@@ -29,8 +29,8 @@
 // they differ from a sentinel, and writes the sentinel back once it has the value, so the buffer
 // is clean again when the kernel ends.  Each word is self-validating, so no fences and no cache
 // flushes are needed.  Workgroups take their chunk from a ticket counter, which guarantees that
-// the chunk a workgroup waits for has already started; the last workgroup to finish resets the
-// counter.  The workspace therefore needs ONE initialisation (k2amd_mi_workspace_init) and no
+// the chunk a workgroup waits for has already started; the workgroup that draws a launch's last
+// ticket puts the counter back.  The workspace therefore needs ONE initialisation (k2amd_mi_workspace_init) and no
 // per-call setup kernel.  Every wait is bounded; a timeout raises the header's error flag, after
 // which every later wait returns at once.
 //
@@ -92,8 +92,8 @@ typedef Layout<4> BwdLayout;
 static_assert(kBlockItems == 2 * kWave * kStorerWaves, "two work items per storer lane");
 
 struct FastHeader {
-  unsigned ticket;  // next chunk to hand out; reset by the last workgroup of a launch
-  unsigned done;    // workgroups finished in this launch
+  unsigned ticket;  // next chunk to hand out; put back by the drawer of a launch's last ticket
+  unsigned done;    // (not used any more; stays 0)
   unsigned error;   // set when a bounded wait timed out (sticky until re-initialised)
   unsigned pad[61];
 };
@@ -340,13 +340,13 @@ __device__ __forceinline__ bool GaveUp(FastHeader *hdr) {
   return __hip_atomic_load(Global(&hdr->error), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;
 }
 
-// Called by one thread after the workgroup's last barrier.
-__device__ __forceinline__ void FinishWorkgroup(FastHeader *hdr, unsigned total) {
-  const unsigned n = __hip_atomic_fetch_add(Global(&hdr->done), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  if (n + 1 == total) {
-    __hip_atomic_store(Global(&hdr->done), 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+// Called by the thread that drew ticket `ticket` of the `total` that a launch draws in all: the
+// one that drew the last of them puts the counter back for the next launch (nobody draws after
+// it; no counter of finished workgroups, whose answer every workgroup would have to wait for
+// before it ends).
+__device__ __forceinline__ void PutTicketsBack(FastHeader *hdr, unsigned ticket, unsigned total) {
+  if (ticket + 1 == total)
     __hip_atomic_store(Global(&hdr->ticket), 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
 }
 
 __device__ __forceinline__ void PublishEdge(float *addr, float v) {
@@ -1019,7 +1019,7 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiForwardFastKernel(
                                         ans, log_deriv, hdr, edge, B, S, Tn, modified, nchunks,
                                         edge_stride, (int)(ticket / nchunks), (int)(ticket % nchunks),
                                         Half{}, nullptr);
-  if (threadIdx.x == 0) FinishWorkgroup(hdr, gridDim.x);
+  if (threadIdx.x == 0) PutTicketsBack(hdr, lds.ticket, gridDim.x);
 }
 
 // ------------------------------------------------------------------------------ backward
@@ -1608,7 +1608,7 @@ __global__ __launch_bounds__(BwdLayout::kThreads) void MiBackwardFastKernel(
                                 (int)(unit / nchunks),
                                 zero_only ? (int)(unit % nchunks) : nchunks - 1 - (int)(unit % nchunks),
                                 zero_only, Half{}, nullptr);
-  if (threadIdx.x == 0) FinishWorkgroup(hdr, gridDim.x);
+  if (threadIdx.x == 0) PutTicketsBack(hdr, lds.ticket, gridDim.x);
 }
 
 // ------------------------------------------------------------------------------ single launch
@@ -1832,7 +1832,8 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiBidirKernel(const Bidir
         __hip_atomic_store(Global(reinterpret_cast<unsigned *>(cw.depart) - 1 + i), kSentinel, __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_AGENT);
   }
-  if (threadIdx.x == 0) FinishWorkgroup(k.hdr, gridDim.x);
+  // (every workgroup draws exactly one ticket past the tasks)
+  if (threadIdx.x == 0) PutTicketsBack(k.hdr, sh.ticket, ntasks + gridDim.x);
 }
 
 // A sweeping workgroup wants a compute unit to itself (its chain wavefront sets the pace of the

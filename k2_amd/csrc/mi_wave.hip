@@ -129,12 +129,10 @@ struct WaveGeom {
   int B, S, Tn, nchunks, edge_stride;
 };
 
-__device__ __forceinline__ void FinishWave(WaveHeader *hdr, unsigned total) {
-  const unsigned n = atomicAdd(&hdr->done, 1u);
-  if (n + 1 == total) {
-    __hip_atomic_store(&hdr->done, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(&hdr->ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
+// The workgroup that drew the last of a launch's tickets puts the counter back for the next
+// launch (nobody draws after it).
+__device__ __forceinline__ void PutTicketsBack(WaveHeader *hdr, unsigned ticket, unsigned total) {
+  if (ticket + 1 == total) __hip_atomic_store(&hdr->ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // The special cells of the forward recursion are expressed in its operands, so that every cell
@@ -224,7 +222,7 @@ __global__ __launch_bounds__(kRows) void MiWaveForwardKernel(
     }
     if (i == ns) ans[b] = GaveUp(hdr) ? __builtin_nan("") : P;
   }
-  if (lane == 0) FinishWave(hdr, gridDim.x);
+  if (lane == 0) PutTicketsBack(hdr, ticket, gridDim.x);
 }
 
 // exp(term1 - total) with the reference's guards (see PxDeriv in mi_generic_impl.h)
@@ -340,7 +338,7 @@ __global__ __launch_bounds__(kRows) void MiWaveBackwardKernel(
     // a lane's last cell is (i, 0): the origin's gradient is what reached the start
     if (i == 0 && overwrite_ans_grad) ans_grad[b] = GaveUp(hdr) ? __builtin_nan("") : G;
   }
-  if (lane == 0) FinishWave(hdr, gridDim.x);
+  if (lane == 0) PutTicketsBack(hdr, ticket, gridDim.x);
 }
 
 // px_grad / py_grad outside the boundary boxes (the sweep assigns everything inside them).
