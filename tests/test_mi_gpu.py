@@ -191,6 +191,21 @@ def test_wide_lattice_more_rows_than_a_wavefront(device, modified):
     check("wide", px, py, bd, (ans, p, gx, gy), device)
 
 
+@pytest.mark.parametrize("modified", [False, True])
+def test_single_launch_at_its_row_limit(device, modified):
+    """S + 2 = 2056 rows, the most the single launch's join keeps in LDS: 33 chunks a half, the
+    join's words fetched in nine batches a pass.  fp32 (the pipelined kernels in all their
+    variants, the single launch among them)."""
+    rng = np.random.default_rng(11)
+    B, S, T = 2, 2054, (2070 if modified else 37)
+    px = rng.normal(-1.5, 1, (B, S, T if modified else T + 1)).astype(np.float32)
+    py = rng.normal(-1.5, 1, (B, S + 1, T)).astype(np.float32)
+    bd = np.array([[0, 0, S, T], [3, 1, S - 40, T - 2]], dtype=np.int64)
+    ans, p = omi.mi_forward(px, py, bd)
+    gx, gy = omi.mi_backward(px, py, bd, p)
+    check("tall", px, py, bd, (ans, p, gx, gy), device)
+
+
 @pytest.mark.parametrize("B", [80, 150])
 @pytest.mark.parametrize("modified", [False, True])
 def test_more_workgroups_than_compute_units(device, modified, B):
