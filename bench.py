@@ -8,8 +8,11 @@ in HBM and taken in turn from eight copies, so that every step reads them from H
 from what the step before left in the 256 MB Infinity Cache.
 
 Prints ONE JSON line.  `value` counts ACTIVE lattice cells, sum_b (S_b+1)(T_b+1), per second of
-fwd+bwd wall time on the GPU; `roofline` prices the step's kernel (the slower of the two where
-two launches are asked for) against the HBM peak with its algorithmic bytes; `cache_resident` is
+fwd+bwd wall time on the GPU: the steps alone between two synchronisations.  `roofline` prices the
+step's kernel (the slower of the two where two launches are asked for) against the HBM peak with
+its algorithmic bytes and its average launch duration, which HIP events measure in a second pass
+over the same steps (one event per ten launches of the single launch: an event between two
+launches costs the GPU 3-4 us, which neither figure should carry); `cache_resident` is
 the same measurement with one copy of the inputs; `cpu_baseline` is the reference's CPU loop on
 this host.  `secondary`, `other_configs` and `fused_joiner` are further workloads through the Python
 API (configs 3, 2, 5, and config 3's shape with the joiner inside the loss), none of them `value`.
@@ -31,6 +34,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # Algorithmic bytes per lattice cell, fp32: forward reads px, py and writes p (12 B); backward
 # reads px, p and writes px_grad, py_grad (16 B; the backward never needs py).
 FWD_BYTES_PER_CELL = 12
+EVENT_GROUP = 10  # launches between two events of the pass that times the kernels
 BWD_BYTES_PER_CELL = 16
 
 # HBM bytes per launch on the default workload, from rocprofv3's FETCH_SIZE / WRITE_SIZE counters
@@ -378,9 +382,6 @@ def main():
             x, y = sets[turn[0] % len(sets)]
             turn[0] += 1
             if single:
-                # one event per launch: launch k lasts from its event to the next launch's
-                if ev is not None:
-                    ev[0].record()
                 return capi.mi_forward_backward(x, y, bd, ones, overwrite_ans_grad=False)
             if ev is not None:
                 ev[0].record()
@@ -395,25 +396,42 @@ def main():
         for _ in range(args.warmup):
             step()
         torch.cuda.synchronize()
-        events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
-        torch.cuda.synchronize()
+        # The timed region: exactly args.steps steps between two synchronisations, nothing else on
+        # the stream (an event recorded between two launches costs the GPU 3-4 us, 7 % of this
+        # step).  The kernels' durations come from a second pass over the same steps.
         t0 = time.perf_counter()
         for k in range(args.steps):
-            step(events[k])
-        if single:
-            events[-1][2].record()
+            step()
         torch.cuda.synchronize()
         wall = time.perf_counter() - t0
         m = {"ms_per_step": wall / args.steps * 1e3, "input_mb": len(sets) * (px.numel() + py.numel()) * 4 // 1000000}
+        events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+        torch.cuda.synchronize()
         if single:
-            # one kernel does the step: its algorithmic bytes are the forward's plus the backward's
-            ends = [e[0] for e in events[1:]] + [events[-1][2]]
-            both_ms = np.array([e[0].elapsed_time(end) for e, end in zip(events, ends)])
+            # one kernel does the step: its algorithmic bytes are the forward's plus the backward's.
+            # An event every EVENT_GROUP launches: the average launch (kernel + the gap to the next
+            # one) of each group, without an event's own cost inside every launch.
+            group = max(1, min(EVENT_GROUP, args.steps))
+            marks = []
+            for k in range(args.steps):
+                if k % group == 0:
+                    events[k][0].record()
+                    marks.append(k)
+                step()
+            events[-1][2].record()
+            torch.cuda.synchronize()
+            ends = [events[k][0] for k in marks[1:]] + [events[-1][2]]
+            counts = [b - a for a, b in zip(marks, marks[1:] + [args.steps])]
+            both_ms = np.array([events[k][0].elapsed_time(end) / n for k, end, n in zip(marks, ends, counts)])
             m.update(dom="mi_forward_backward", dom_ms=float(both_ms.mean()), dom_bytes=both_bytes,
                      both_avg=float(both_ms.mean()),
                      kernel_times={"mi_forward_backward_avg_us": float(both_ms.mean()) * 1e3,
-                                   "mi_forward_backward_min_us": float(both_ms.min()) * 1e3})
+                                   "mi_forward_backward_min_us": float(both_ms.min()) * 1e3,
+                                   "launches_per_event": group})
         else:
+            for k in range(args.steps):
+                step(events[k])
+            torch.cuda.synchronize()
             fwd_ms = np.array([e[0].elapsed_time(e[1]) for e in events])
             bwd_ms = np.array([e[1].elapsed_time(e[2]) for e in events])
             # Roofline of the dominant kernel (the one with the longer average launch).
