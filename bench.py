@@ -161,7 +161,7 @@ def pruned_secondary(dev, steps=50, cpu=True):
         "logits_GBps": logits_bytes / t_pruned / 1e9,
         "frac_of_hbm_peak": logits_bytes / t_pruned / 1e9 / HBM_PEAK_GBS,
         "simple_pass_plus_prune_ranges_ms": t_ranges * 1e3,
-        "loss": float(loss),
+        "loss": float(loss.detach()),
     }
     if cpu:
         n = B  # utterances in the CPU sample: the whole batch
