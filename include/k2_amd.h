@@ -270,9 +270,12 @@ K2AMD_API int k2amd_rnnt_prune_gather_backward(const void *grad, const int64_t *
  *   px, py, normalizers [B][T][R]: as k2amd_rnnt_logprobs_pruned_forward.
  *   precision: K2AMD_JOINER_F32 multiplies in fp32 on the matrix cores; K2AMD_JOINER_BF16 rounds the
  *   activations, the weight and the logits' gradients to bfloat16 for the products (fp32 sums).
- *   workspace: k2amd_rnnt_joiner_pruned_workspace_bytes(...) bytes of device memory (0 = shape
- *   not served: D a multiple of 64 up to 512, R <= 32 and <= S + 1; any C); contents need not
- *   survive between the two calls.
+ *   workspace: device memory, k2amd_rnnt_joiner_pruned_forward_workspace_bytes(...) bytes for the
+ *   forward (the weight in the operand type) and k2amd_rnnt_joiner_pruned_workspace_bytes(...)
+ *   for the backward (the weight twice, and what its first kernel hands its second: the
+ *   activations and the logits' gradients in the operand type, B T R x (D + C) elements); 0 =
+ *   shape not served: D a multiple of 64 up to 512, R <= 32 and <= S + 1; any C.  Contents need
+ *   not survive between the two calls.
  * The backward takes what the forward took, the normalizers it wrote and the gradients w.r.t. its
  * px / py (seq_scale as for the other builders), and writes am_grad [B][T][D], lm_grad [B][S+1][D],
  * weight_grad [C][D], bias_grad [C] (or NULL).  lm_grad, weight_grad and bias_grad are sums formed
@@ -280,6 +283,8 @@ K2AMD_API int k2amd_rnnt_prune_gather_backward(const void *grad, const int64_t *
 enum k2amd_joiner_precision { K2AMD_JOINER_F32 = 0, K2AMD_JOINER_BF16 = 1 };
 K2AMD_API size_t k2amd_rnnt_joiner_pruned_workspace_bytes(int B, int S, int T, int R, int C, int D,
                                                           int precision);
+K2AMD_API size_t k2amd_rnnt_joiner_pruned_forward_workspace_bytes(int B, int S, int T, int R, int C,
+                                                                  int D, int precision);
 K2AMD_API int k2amd_rnnt_joiner_pruned_forward(
     const void *am, const void *lm, const int64_t *ranges, const void *weight, const void *bias,
     const int64_t *symbols, const int64_t *boundary, void *px, void *py, void *normalizers, int B,

@@ -48,6 +48,7 @@ _SIGNATURES = {
     "k2amd_rnnt_hat_logprobs_pruned_forward": ([_vp] * 7 + [_ci] * 7 + [_vp], _ci),
     "k2amd_rnnt_hat_logprobs_pruned_backward": ([_vp] * 9 + [_ci] * 7 + [_vp], _ci),
     "k2amd_rnnt_joiner_pruned_workspace_bytes": ([_ci] * 7, _sz),
+    "k2amd_rnnt_joiner_pruned_forward_workspace_bytes": ([_ci] * 7, _sz),
     "k2amd_rnnt_joiner_pruned_forward": ([_vp] * 10 + [_ci] * 9 + [_vp, _sz, _vp], _ci),
     "k2amd_rnnt_joiner_pruned_backward": ([_vp] * 15 + [_ci] * 9 + [_vp, _sz, _vp], _ci),
     "k2amd_rnnt_prune_ranges": ([_vp] * 4 + [_ci] * 6 + [_vp], _ci),
@@ -470,8 +471,9 @@ JOINER_PRECISIONS = {"fp32": 0, "bf16": 1}
 
 
 def _joiner_shapes(am, lm, ranges, weight, bias, symbols, boundary, termination_symbol, rnnt_type,
-                   precision):
-    """Checks every tensor of the fused joiner calls; returns (B, S, T, R, C, D, workspace)."""
+                   precision, forward):
+    """Checks every tensor of the fused joiner calls; returns (B, S, T, R, C, D, workspace), the
+    workspace of the size the forward (or the backward) call asks for."""
     dev = am.device
     if am.dtype != torch.float32:
         raise RuntimeError(f"k2_amd: the fused joiner takes float32 tensors, am is {am.dtype}")
@@ -491,7 +493,9 @@ def _joiner_shapes(am, lm, ranges, weight, bias, symbols, boundary, termination_
     expect(symbols, "symbols", torch.int64, dev, (B, S))
     expect_optional(boundary, "boundary", torch.int64, dev, (B, 4))
     _symbol(termination_symbol, C)
-    nbytes = lib().k2amd_rnnt_joiner_pruned_workspace_bytes(B, S, T, R, C, D, precision)
+    size_of = (lib().k2amd_rnnt_joiner_pruned_forward_workspace_bytes if forward
+               else lib().k2amd_rnnt_joiner_pruned_workspace_bytes)
+    nbytes = size_of(B, S, T, R, C, D, precision)
     if nbytes == 0:
         raise RuntimeError(f"k2_amd: the fused joiner does not serve B={B} S={S} T={T} R={R} C={C} D={D} "
                            "(D must be a multiple of 64 up to 512, R at most 32 and S + 1)")
@@ -504,7 +508,7 @@ def joiner_pruned_forward(am, lm, ranges, weight, bias, symbols, termination_sym
     """tanh(am[b,t] + lm[b,ranges[b,t,k]]) . weight^T + bias and get_rnnt_logprobs_pruned on it in one
     pass: returns (px, py, normalizers [B][T][R]); the logits never exist in memory."""
     B, S, T, R, C, D, ws = _joiner_shapes(am, lm, ranges, weight, bias, symbols, boundary,
-                                          termination_symbol, rnnt_type, precision)
+                                          termination_symbol, rnnt_type, precision, True)
     dev = am.device
     px = torch.empty(B, S, _t1(T, rnnt_type), dtype=torch.float32, device=dev)
     py = torch.empty(B, S + 1, T, dtype=torch.float32, device=dev)
@@ -522,7 +526,7 @@ def joiner_pruned_backward(am, lm, ranges, weight, bias, symbols, termination_sy
     """Gradients of sum_b seq_scale[b] * score_b through the fused joiner: returns (am_grad, lm_grad,
     weight_grad, bias_grad or None)."""
     B, S, T, R, C, D, ws = _joiner_shapes(am, lm, ranges, weight, bias, symbols, boundary,
-                                          termination_symbol, rnnt_type, precision)
+                                          termination_symbol, rnnt_type, precision, False)
     dev = am.device
     expect(norm, "normalizers", torch.float32, dev, (B, T, R))
     _expect_lattice_grads(px_grad, py_grad, seq_scale, torch.float32, dev, B, S, T, rnnt_type)

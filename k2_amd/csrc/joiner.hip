@@ -8,8 +8,10 @@
 // The [B][T][R][C] logits only ever exist as tiles in registers: the forward multiplies a tile of
 // rows by the weight on the matrix cores, folds each tile of columns into a running log-sum-exp and
 // picks out the two logits a row contributes; the backward multiplies again and forms
-// d logits = -softmax (gx + gy) + gx [c == symbol] + gy [c == blank] on the fly, once per tile of
-// rows (for the gradients of am and lm) and once per slice of columns (for those of the weight).
+// d logits = -softmax (gx + gy) + gx [c == symbol] + gy [c == blank] on the fly, tile of rows by
+// tile of rows, for the gradients of am and lm, and leaves the activations and d logits in the
+// caller's workspace (in the operand type and in the order a product over the rows consumes them)
+// for a second kernel that forms the gradients of the weight and the bias.
 //
 // One row of the product is (b, t, k); a tile holds whole frames (b, t), R rows each, so the sum
 // over k that am's gradient needs stays inside a tile.  Operands: `F32` multiplies fp32 by fp32
@@ -138,6 +140,12 @@ struct JoinerArgs {
   const void *wc;   // weight copy, rows d (Dpad), k = c (Cpad)
   float *px, *py, *norm;        // forward outputs (norm [B][T][R])
   const float4 *hdr;            // backward: per row {gx, gy, symbol, norm}
+  // backward, written by the rows kernel for the weight kernel after it, both as operands of a
+  // product over k = row (see BOperand; a step of k is one tile of rows): tanh(..) with rows d,
+  // d logits with rows c; and the sums of d logits over each tile's rows, [tile][Cpad]
+  void *hs, *dzs;
+  float *bias_part;
+  int tiles;                    // tiles of rows of the rows kernel
   float *am_grad, *lm_grad, *weight_grad, *bias_grad;
   int B, S, Tn, R, C, D, blank, rnnt_type;
   int Cpad, Dpad;               // C, D rounded up to whole tiles of kNTile
@@ -232,53 +240,6 @@ __device__ __forceinline__ void StageActivations(const JoinerArgs &a, const RowM
         ht[(size_t)(4 * q + 2) * ldt + m] = Mode::From(v.z);
         ht[(size_t)(4 * q + 3) * ldt + m] = Mode::From(v.w);
       }
-    }
-  }
-}
-
-// The same for the weight gradient in bfloat16, which also wants the activations transposed,
-// ht[d][m] (k = row contiguous).  An item is four adjacent columns of four adjacent rows: the
-// transposed copy is then written eight bytes at a time (four rows of one column) instead of one
-// two-byte store per element, whose lanes fell sixteen to an LDS bank.  Consecutive threads take
-// consecutive groups of rows first, so that those stores of a wavefront are contiguous.
-template <typename Mode, int MT>
-__device__ __forceinline__ void StageActivationsBoth(const JoinerArgs &a, const RowMeta *meta, int rows,
-                                                     typename Mode::Elem *h, int ldh,
-                                                     typename Mode::Elem *ht, int ldt) {
-  static_assert(sizeof(typename Mode::Elem) == 2, "bfloat16 tiles");
-  constexpr int kGroups = MT / 4;
-  const int qpr = a.D >> 2, items = kGroups * qpr;
-  for (int it = threadIdx.x; it < items; it += kThreads) {
-    const int mg = it % kGroups, q = it / kGroups;
-    float4 x[4], y[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int m = mg * 4 + r;
-      x[r] = make_float4(0.f, 0.f, 0.f, 0.f);
-      y[r] = x[r];
-      if (m < rows) {
-        const RowMeta rm = meta[m];
-        x[r] = *reinterpret_cast<const float4 *>(a.am + (size_t)rm.bt * a.D + 4 * q);
-        y[r] = *reinterpret_cast<const float4 *>(a.lm + (size_t)rm.lmrow * a.D + 4 * q);
-      }
-    }
-    unsigned short t[4][4];  // [row][column]
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const float4 v = make_float4(Tanh(x[r].x + y[r].x), Tanh(x[r].y + y[r].y), Tanh(x[r].z + y[r].z),
-                                   Tanh(x[r].w + y[r].w));
-      t[r][0] = ToBf16(v.x); t[r][1] = ToBf16(v.y); t[r][2] = ToBf16(v.z); t[r][3] = ToBf16(v.w);
-      uint2 row;
-      row.x = (unsigned)t[r][0] | ((unsigned)t[r][1] << 16);
-      row.y = (unsigned)t[r][2] | ((unsigned)t[r][3] << 16);
-      *reinterpret_cast<uint2 *>(h + (size_t)(mg * 4 + r) * ldh + 4 * q) = row;
-    }
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      uint2 colv;
-      colv.x = (unsigned)t[0][e] | ((unsigned)t[1][e] << 16);
-      colv.y = (unsigned)t[2][e] | ((unsigned)t[3][e] << 16);
-      *reinterpret_cast<uint2 *>(ht + (size_t)(4 * q + e) * ldt + mg * 4) = colv;
     }
   }
 }
@@ -525,6 +486,30 @@ __global__ __launch_bounds__(kThreads) void JoinerBackwardRowsKernel(const Joine
   __syncthreads();
   StageActivations<Mode, MT, false, 8>(a, meta, rows, h, ldh, nullptr, 0);
   __syncthreads();
+  {  // The tile's activations go to the workspace as an operand with k = row: this tile is step
+     // blockIdx.x of k, and a 16-byte group holds consecutive rows of one column d.
+    static_assert(MT == Mode::kChunk, "a tile of rows is one step of k");
+    constexpr int kPer = 16 / sizeof(Elem);
+    uint4 *dst = static_cast<uint4 *>(a.hs);
+    const int groups = (a.D / 32) * kFragQuads;
+    for (int g = threadIdx.x; g < groups; g += kThreads) {
+      const int nb = g / kFragQuads, r = g % kFragQuads, i = r >> 6, l = r & 63;
+      const Elem *src = h + (size_t)((l >> 5) * (Mode::kChunk / 2) + i * kPer) * ldh + nb * 32 + (l & 31);
+      uint4 out;
+      if constexpr (sizeof(Elem) == 4) {
+        out = make_uint4(AsBits(Mode::To(src[0])), AsBits(Mode::To(src[ldh])), AsBits(Mode::To(src[2 * ldh])),
+                         AsBits(Mode::To(src[3 * ldh])));
+      } else {
+        unsigned w32[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          w32[e] = (unsigned)(unsigned short)src[(size_t)(2 * e) * ldh] |
+                   ((unsigned)(unsigned short)src[(size_t)(2 * e + 1) * ldh] << 16);
+        out = make_uint4(w32[0], w32[1], w32[2], w32[3]);
+      }
+      dst[((size_t)nb * a.tiles + blockIdx.x) * kFragQuads + r] = out;
+    }
+  }
 
   const int lane = threadIdx.x & 63, col = lane & 31, half = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the same in all lanes: a scalar
@@ -547,14 +532,44 @@ __global__ __launch_bounds__(kThreads) void JoinerBackwardRowsKernel(const Joine
     TileProduct<Mode, RB, kStepsD>(acc, h + (size_t)col * ldh + koff, ldh,
                                    BOperand(a.wk, (n0 >> 5) + wave, a.D / Mode::kChunk, 0), lane, a.D);
     const float bn = (n < a.C && a.bias != nullptr) ? a.bias[n] : 0.f;
+    float colsum = 0.f;
+    // d logits as an operand with k = row, for the weight kernel: block of columns (n0 >> 5) + wave,
+    // step blockIdx.x.  A lane holds runs of four consecutive rows of its column (AccRow), which
+    // are half a 16-byte group in bfloat16 and a whole one in fp32.
+    unsigned char *zblock = static_cast<unsigned char *>(a.dzs) +
+                            ((size_t)((n0 >> 5) + wave) * a.tiles + blockIdx.x) * kFragQuads * 16;
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = rb * 32 + AccRow(r, half);
-        const float v = n < a.C ? LogitGrad(acc[rb][r] + bn, n, hdr[row], a.blank) : 0.f;
-        dz[(size_t)row * ldz + wave * 32 + col] = Mode::From(v);
+      for (int j = 0; j < 4; ++j) {
+        Elem run[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int r = j * 4 + e;
+          const int row = rb * 32 + AccRow(r, half);
+          const float v = n < a.C ? LogitGrad(acc[rb][r] + bn, n, hdr[row], a.blank) : 0.f;
+          run[e] = Mode::From(v);
+          colsum += Mode::To(run[e]);
+          dz[(size_t)row * ldz + wave * 32 + col] = run[e];
+        }
+        const int k = rb * 32 + j * 8 + half * 4;  // the run's first row = its position in the step of k
+        constexpr int kHalfChunk = Mode::kChunk / 2, kPer = 16 / (int)sizeof(Elem);
+        const int kin = k % kHalfChunk;
+        unsigned char *at = zblock + ((size_t)(kin / kPer) * 64 + (k / kHalfChunk) * 32 + col) * 16 +
+                            (kin % kPer) * sizeof(Elem);
+        if constexpr (sizeof(Elem) == 4) {
+          *reinterpret_cast<uint4 *>(at) = make_uint4(AsBits(Mode::To(run[0])), AsBits(Mode::To(run[1])),
+                                                      AsBits(Mode::To(run[2])), AsBits(Mode::To(run[3])));
+        } else {
+          uint2 p;
+          p.x = (unsigned)(unsigned short)run[0] | ((unsigned)(unsigned short)run[1] << 16);
+          p.y = (unsigned)(unsigned short)run[2] | ((unsigned)(unsigned short)run[3] << 16);
+          *reinterpret_cast<uint2 *>(at) = p;
+        }
       }
+    // the column's sum over the tile's rows (the two halves of the wavefront hold 16 RB rows each)
+    colsum += __shfl_xor(colsum, 32, kWave);
+    if (half == 0) a.bias_part[(size_t)blockIdx.x * a.Cpad + n] = colsum;
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
@@ -613,136 +628,88 @@ __global__ __launch_bounds__(kThreads) void JoinerBackwardRowsKernel(const Joine
 
 // ------------------------------------------------------- backward, gradients of weight and bias
 //
-// A workgroup owns kSlice columns c of d logits and every `groups`-th tile of 64 rows; it keeps its
-// [kSlice][D] block of the weight's gradient in accumulators over all of its tiles:
-//   logits slice = h . weight[c-slice]^T     (k = D; with fewer 32 x 32 blocks than wavefronts, k is
-//                                             split between them and the halves meet in LDS)
-//   d logits slice -> LDS, transposed [c][row]
-//   weight_grad[c][d] += sum over rows of d logits[row][c] h[row][d]   (k = rows of the tile)
-// and adds it to weight_grad (zeroed by the launcher) with atomic adds at the end.
-template <typename Mode, int kSlice, int kD>
-__global__ __launch_bounds__(kThreads) void JoinerBackwardWeightKernel(const JoinerArgs a, int tiles,
-                                                                        int groups) {
-  constexpr int MT = 64;
-  constexpr bool kBf = sizeof(typename Mode::Elem) == 2;
-  constexpr int kColBlocks = kSlice / 32;               // 32-column blocks of the slice
-  constexpr int kBlocks = 2 * kColBlocks;               // blocks of the logits slice
-  constexpr int kSplit = kWaves / kBlocks;              // wavefronts per block: shares of k
-  constexpr int kDGroups = kWaves / kColBlocks;         // wavefronts per column block in the gradient
-  constexpr int kMaxDB = (kMaxD / 32) / kDGroups;       // 32-column blocks of D per wavefront
-  static_assert(kBlocks * kSplit == kWaves && (kSplit == 1 || kSplit == 2), "wavefront roles");
-  typedef typename Mode::Elem Elem;
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  const int ldh = (kD > 0 ? kD : a.D) + Mode::kPad;  // a constant where D is one: LDS offsets become immediates
-  constexpr int ldz = MT + Mode::kPad;  // d logits, transposed: [c][row]
-  constexpr int ldt = MT + Mode::kPad;  // h, transposed: [d][row] (bfloat16 only)
-  Elem *h = reinterpret_cast<Elem *>(smem);
-  Elem *dzt = h + (size_t)MT * ldh;
-  Elem *ht = dzt + (size_t)kSlice * ldz;
-  float4 *hdr = reinterpret_cast<float4 *>(ht + (kBf ? (size_t)a.D * ldt : 0));
-  RowMeta *meta = reinterpret_cast<RowMeta *>(hdr + MT);
-
-  const int slice = blockIdx.x / groups, group = blockIdx.x - slice * groups;
-  const int c0 = slice * kSlice;
+//   weight_grad[c][d] = sum over rows of d logits[row][c] h[row][d]
+// is a product over k = row of two operands that the rows kernel has left in the workspace in the
+// order the multiplies consume them, so this kernel is nothing but loads and multiplies: no LDS, no
+// barrier.  A workgroup of four wavefronts (one per SIMD, so that a wavefront has the registers for
+// eight accumulator blocks and two sets of operands) owns 128 columns c x 256 columns d of the
+// gradient and one share of the steps of k; wavefront w takes two blocks of c and four of d.  The
+// workgroups that share a share of k are eight apart in the grid, which puts them on one XCD: what
+// one of them has fetched the others find in that XCD's L2.  The sums meet in weight_grad
+// (zeroed by the launcher) through atomic adds; the workgroups of the first block of d also add up
+// their tiles' sums of d logits for bias_grad.
+constexpr int kWgThreads = 256;
+constexpr int kWgCBlocks = 2, kWgDBlocks = 4;  // per wavefront
+template <typename Mode>
+__global__ __launch_bounds__(kWgThreads) void JoinerWeightGradKernel(const JoinerArgs a, int dtiles, int shares) {
+  const int share = blockIdx.x % shares, combo = blockIdx.x / shares;
+  const int ct = combo / dtiles, dt = combo - ct * dtiles;
   const int lane = threadIdx.x & 63, col = lane & 31, half = lane >> 5;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the same in all lanes: a scalar
-  const int koff = half * (Mode::kChunk / 2);
-  // the block of the logits slice this wavefront multiplies, and its share of k
-  const int blk = wave % kBlocks, ks = wave / kBlocks, rb = blk / kColBlocks, cb = blk % kColBlocks;
-  const int n = c0 + cb * 32 + col;  // its column of logits (< Cpad: slices tile Cpad)
-  const int kshare = a.D / kSplit;
-  // its blocks of the gradient: columns c0 + gcb*32 .. +31, d blocks dgrp, dgrp + kDGroups, ..
-  const int gcb = wave % kColBlocks, dgrp = wave / kColBlocks, ndb = a.D / 32;
-  Acc16 wacc[kMaxDB];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int cb0 = ct * 4 + (wave & 1) * kWgCBlocks, db0 = dt * 8 + (wave >> 1) * kWgDBlocks;
+  const int ncb = a.Cpad / 32, ndb = a.D / 32;
+  const int t0 = (int)((long long)a.tiles * share / shares), t1 = (int)((long long)a.tiles * (share + 1) / shares);
+  bool c_ok[kWgCBlocks], d_ok[kWgDBlocks];
 #pragma unroll
-  for (int i = 0; i < kMaxDB; ++i)
+  for (int i = 0; i < kWgCBlocks; ++i) c_ok[i] = cb0 + i < ncb;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) wacc[i][r] = 0.f;
-  float bsum = 0.f;
-  const float bn = (n < a.C && a.bias != nullptr) ? a.bias[n] : 0.f;
-
-  for (int tile = group; tile < tiles; tile += groups) {
-    const long long f0 = (long long)tile * a.tpt;
-    const int rows = LoadMeta<MT>(a, f0, meta);
-    for (int m = threadIdx.x; m < MT; m += kThreads)
-      hdr[m] = m < rows ? a.hdr[(size_t)f0 * a.R + m] : make_float4(0.f, 0.f, -1.f, 3.0e38f);  // padding: exp(. - norm) = 0
-    __syncthreads();
-    if constexpr (kBf) StageActivationsBoth<Mode, MT>(a, meta, rows, h, ldh, ht, ldt);
-    else StageActivations<Mode, MT, false, 2>(a, meta, rows, h, ldh, nullptr, 0);
-    __syncthreads();
-    Acc16 acc[1];
+  for (int j = 0; j < kWgDBlocks; ++j) d_ok[j] = db0 + j < ndb;
+  Acc16 acc[kWgCBlocks][kWgDBlocks];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[0][r] = 0.f;
-    TileProduct<Mode, 1, kD / kSplit / Mode::kChunk>(acc, h + (size_t)(rb * 32 + col) * ldh + ks * kshare + koff,
-                                                     ldh, BOperand(a.wk, (c0 >> 5) + cb, a.D / Mode::kChunk, ks * kshare / Mode::kChunk), lane, kshare);
-    if constexpr (kSplit == 2) {  // the upper share of k parks its sums where the block's d logits will go
-      float *park = reinterpret_cast<float *>(dzt);
-      if (ks == 1) {
+  for (int i = 0; i < kWgCBlocks; ++i)
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          park[(size_t)(cb * 32 + col) * ldz + rb * 32 + AccRow(r, half)] = acc[0][r];
-      }
-      __syncthreads();
-      if (ks == 0) {
+    for (int j = 0; j < kWgDBlocks; ++j)
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          acc[0][r] += park[(size_t)(cb * 32 + col) * ldz + rb * 32 + AccRow(r, half)];
-      }
-    }
-    if (ks == 0) {
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  struct Operands {
+    Frag z[kWgCBlocks], h[kWgDBlocks];
+  };
+  auto load = [&](Operands &o, int t) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = rb * 32 + AccRow(r, half);
-        const float v = n < a.C ? LogitGrad(acc[0][r] + bn, n, hdr[row], a.blank) : 0.f;
-        dzt[(size_t)(cb * 32 + col) * ldz + row] = Mode::From(v);
-      }
-    }
-    __syncthreads();
-    if (threadIdx.x < kSlice) {
-      float s = 0.f;
-      for (int m = 0; m < MT; ++m) s += Mode::To(dzt[(size_t)threadIdx.x * ldz + m]);
-      bsum += s;
+    for (int i = 0; i < kWgCBlocks; ++i)
+      if (c_ok[i]) o.z[i] = LoadFragB(BOperand(a.dzs, cb0 + i, a.tiles, t), lane);
+#pragma unroll
+    for (int j = 0; j < kWgDBlocks; ++j)
+      if (d_ok[j]) o.h[j] = LoadFragB(BOperand(a.hs, db0 + j, a.tiles, t), lane);
+  };
+  auto multiply = [&](const Operands &o) {
+#pragma unroll
+    for (int i = 0; i < kWgCBlocks; ++i)
+#pragma unroll
+      for (int j = 0; j < kWgDBlocks; ++j)
+        if (c_ok[i] && d_ok[j]) Mode::Mma(acc[i][j], o.z[i], o.h[j]);
+  };
+  if (t0 < t1 && c_ok[0] && d_ok[0]) {
+    Operands o0, o1;
+    load(o0, t0);
+    for (int t = t0; t < t1; t += 2) {
+      load(o1, t + 1 < t1 ? t + 1 : t);
+      multiply(o0);
+      load(o0, t + 2 < t1 ? t + 2 : t);
+      if (t + 1 < t1) multiply(o1);
     }
 #pragma unroll
-    for (int kc = 0; kc < MT / Mode::kChunk; ++kc) {
-      const Frag fa = LoadFrag(dzt + (size_t)(gcb * 32 + col) * ldz + kc * Mode::kChunk + koff);
+    for (int i = 0; i < kWgCBlocks; ++i)
 #pragma unroll
-      for (int i = 0; i < kMaxDB; ++i) {
-        const int db = dgrp + kDGroups * i;
-        if (db < ndb) {
-          const int d = db * 32 + col;
-          Frag fb;
-          if (kBf) {
-            fb = LoadFrag(ht + (size_t)d * ldt + kc * Mode::kChunk + koff);
-          } else {
-            const float *hf = reinterpret_cast<const float *>(h);
-            unsigned u[16];
+      for (int j = 0; j < kWgDBlocks; ++j) {
+        if (!c_ok[i] || !d_ok[j]) continue;
+        const int d = (db0 + j) * 32 + col;
 #pragma unroll
-            for (int j = 0; j < 16; ++j)
-              u[j] = AsBits(hf[(size_t)(kc * 32 + half * 16 + j) * ldh + d]);
-#pragma unroll
-            for (int q = 0; q < 4; ++q) fb.q[q] = make_uint4(u[4 * q], u[4 * q + 1], u[4 * q + 2], u[4 * q + 3]);
-          }
-          Mode::Mma(wacc[i], fa, fb);
+        for (int r = 0; r < 16; ++r) {
+          const int c = (cb0 + i) * 32 + AccRow(r, half);
+          if (c < a.C) atomicAdd(a.weight_grad + (size_t)c * a.D + d, acc[i][j][r]);
         }
       }
-    }
-    __syncthreads();  // the next tile's staging overwrites h, dzt, hdr
   }
-#pragma unroll
-  for (int i = 0; i < kMaxDB; ++i) {
-    const int db = dgrp + kDGroups * i;
-    if (db < ndb) {
-      const int d = db * 32 + col;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int c = c0 + gcb * 32 + AccRow(r, half);
-        if (c < a.C) atomicAdd(a.weight_grad + (size_t)c * a.D + d, wacc[i][r]);
-      }
+  if (dt == 0 && a.bias_grad != nullptr) {
+    const int c = ct * 128 + (int)(threadIdx.x & 127);
+    if (c < a.C) {
+      float sum = 0.f;
+      for (int t = t0 + (int)(threadIdx.x >> 7); t < t1; t += kWgThreads / 128)
+        sum += a.bias_part[(size_t)t * a.Cpad + c];
+      atomicAdd(a.bias_grad + c, sum);
     }
   }
-  if (threadIdx.x < kSlice && c0 + (int)threadIdx.x < a.C && a.bias_grad != nullptr)
-    atomicAdd(a.bias_grad + c0 + threadIdx.x, bsum);
 }
 
 // ---------------------------------------------------------------------------- small kernels
@@ -846,8 +813,10 @@ bool JoinerShapeOk(int B, int S, int T, int R, int C, int D) {
 }
 
 struct WorkspaceLayout {
-  size_t wk, wc, hdr, total;
+  size_t wk, wc, hdr, forward_total, hs, dzs, bias_part, total;
 };
+// rows per tile of the backward's rows kernel, which is one step of k of the weight kernel
+int RowsTile(int precision) { return precision == K2AMD_JOINER_BF16 ? 64 : 32; }
 WorkspaceLayout LayoutOf(int B, int T, int R, int C, int D, int precision) {
   const size_t e = ElemBytes(precision);
   const size_t Cpad = RoundUp(C, kNTile), Dpad = RoundUp(D, kNTile);
@@ -855,7 +824,14 @@ WorkspaceLayout LayoutOf(int B, int T, int R, int C, int D, int precision) {
   w.wk = 0;
   w.wc = (Cpad * D * e + 255) / 256 * 256;
   w.hdr = w.wc + (Dpad * Cpad * e + 255) / 256 * 256;
-  w.total = w.hdr + (size_t)B * T * R * sizeof(float4);
+  w.forward_total = w.wc;  // the forward multiplies by the first copy only
+  const size_t tpt = RowsTile(precision) / R;
+  const size_t tiles = tpt > 0 ? ((size_t)B * T + tpt - 1) / tpt : 0;
+  const size_t padded_rows = tiles * RowsTile(precision);
+  w.hs = (w.hdr + (size_t)B * T * R * sizeof(float4) + 255) / 256 * 256;
+  w.dzs = w.hs + (padded_rows * D * e + 255) / 256 * 256;
+  w.bias_part = w.dzs + (padded_rows * Cpad * e + 255) / 256 * 256;
+  w.total = w.bias_part + tiles * Cpad * sizeof(float);
   return w;
 }
 
@@ -883,6 +859,9 @@ JoinerArgs MakeArgs(const float *am, const float *lm, const int64_t *ranges, con
   a.wk = ws + w.wk;
   a.wc = ws + w.wc;
   a.hdr = reinterpret_cast<const float4 *>(ws + w.hdr);
+  a.hs = ws + w.hs;
+  a.dzs = ws + w.dzs;
+  a.bias_part = reinterpret_cast<float *>(ws + w.bias_part);
   return a;
 }
 
@@ -941,27 +920,16 @@ int BackwardImpl(const float *weight, JoinerArgs a, const float *px_grad, const 
     rc = AllowLds(kernel, lds);
     if (rc != K2AMD_OK) return rc;
     const long long tiles = (a.frames + r.tpt - 1) / r.tpt;
+    r.tiles = (int)tiles;
+    a.tiles = (int)tiles;
     hipLaunchKernelGGL(kernel, dim3((unsigned)tiles), dim3(kThreads), lds, st, r);
   }
-  {  // gradients of weight and bias: slices of columns x groups of tiles of 64 rows
-    constexpr int kSlice = kBf ? 128 : 64;
-    JoinerArgs w = a;
-    w.tpt = 64 / a.R;
-    const size_t lds = (size_t)64 * (a.D + Mode::kPad) * sizeof(Elem) +
-                       (size_t)kSlice * (64 + Mode::kPad) * sizeof(Elem) +
-                       (kBf ? (size_t)a.D * (64 + Mode::kPad) * sizeof(Elem) : 0) +
-                       64 * (sizeof(float4) + sizeof(RowMeta));
-    auto kernel = a.D == kMaxD ? JoinerBackwardWeightKernel<Mode, kSlice, kMaxD>
-                               : JoinerBackwardWeightKernel<Mode, kSlice, 0>;
-    rc = AllowLds(kernel, lds);
-    if (rc != K2AMD_OK) return rc;
-    const long long tiles = (a.frames + w.tpt - 1) / w.tpt;
-    const int slices = a.Cpad / kSlice;
-    int groups = 256 / slices;  // one workgroup per compute unit
-    if (groups < 1) groups = 1;
-    if (groups > tiles) groups = (int)tiles;
-    hipLaunchKernelGGL(kernel, dim3((unsigned)(slices * groups)), dim3(kThreads), lds, st, w, (int)tiles,
-                       groups);
+  {  // gradients of weight and bias: blocks of 128 x 256 of the gradient x shares of the rows
+    const int ctiles = a.Cpad / 128, dtiles = (a.D + 255) / 256;
+    int shares = 256 / (ctiles * dtiles) / 8 * 8;  // one workgroup per compute unit; a multiple of the XCDs
+    if (shares < 8) shares = 8;
+    hipLaunchKernelGGL(JoinerWeightGradKernel<Mode>, dim3((unsigned)(ctiles * dtiles * shares)),
+                       dim3(kWgThreads), 0, st, a, dtiles, shares);
   }
   return LaunchStatus();
 }
@@ -980,6 +948,13 @@ size_t k2amd_rnnt_joiner_pruned_workspace_bytes(int B, int S, int T, int R, int 
   return LayoutOf(B, T, R, C, D, precision).total;
 }
 
+size_t k2amd_rnnt_joiner_pruned_forward_workspace_bytes(int B, int S, int T, int R, int C, int D,
+                                                        int precision) {
+  if (!JoinerShapeOk(B, S, T, R, C, D)) return 0;
+  if (precision != K2AMD_JOINER_F32 && precision != K2AMD_JOINER_BF16) return 0;
+  return LayoutOf(B, T, R, C, D, precision).forward_total;
+}
+
 int k2amd_rnnt_joiner_pruned_forward(const void *am, const void *lm, const int64_t *ranges,
                                      const void *weight, const void *bias, const int64_t *symbols,
                                      const int64_t *boundary, void *px, void *py, void *normalizers,
@@ -995,7 +970,7 @@ int k2amd_rnnt_joiner_pruned_forward(const void *am, const void *lm, const int64
   if (!am || !lm || !ranges || !weight || !px || !py || !normalizers || (!symbols && S > 0))
     return K2AMD_ERR_INVALID_ARGUMENT;
   if (workspace == nullptr ||
-      workspace_bytes < k2amd_rnnt_joiner_pruned_workspace_bytes(B, S, T, R, C, D, precision))
+      workspace_bytes < k2amd_rnnt_joiner_pruned_forward_workspace_bytes(B, S, T, R, C, D, precision))
     return K2AMD_ERR_WORKSPACE;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool bf = precision == K2AMD_JOINER_BF16;

@@ -1491,10 +1491,6 @@ __device__ __forceinline__ void MiBackwardChunk(
         sh.scale = scale;
         sh.split_ok = ok;
         if (join->ans != nullptr && ok) *join->ans = GaveUp(hdr) ? __builtin_nanf("") : total;
-        // This task is through with the cut words: said now, so that the count is back by the
-        // time the sweep ends (it is looked at there; a trip to memory off the launch's tail).
-        departed_early = __hip_atomic_fetch_add(Global(join->cw.depart), 1u, __ATOMIC_RELAXED,
-                                                __HIP_MEMORY_SCOPE_AGENT);
       }
       K2AMD_TRACE_MARK(half, 1);
     } else if (role == kLoader) {
@@ -1507,6 +1503,15 @@ __device__ __forceinline__ void MiBackwardChunk(
       for (int i = 0; i < kSets; ++i) load_block(top - 1 - i, sets[i]);
     }
     LdsBarrier();
+    // This task is through with the sequence's words: the chain has read the cut and, behind the
+    // barrier, the loaders have seen the count of the forward sweeps' stores.  Said now, so that
+    // the answer is back by the time the sweep ends (it is looked at there; a trip to memory off
+    // the launch's tail), and not before the barrier: the task that departs last puts every word
+    // of the sequence back, that count included, and a loader still waiting for it to reach its
+    // final value would then wait until its bound expires.
+    if (role == kChain && lane == 0)
+      departed_early = __hip_atomic_fetch_add(Global(join->cw.depart), 1u, __ATOMIC_RELAXED,
+                                              __HIP_MEMORY_SCOPE_AGENT);
     if (!sh.split_ok) {
       if (role == kLoader) {
 #pragma unroll
