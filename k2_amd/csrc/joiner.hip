@@ -200,14 +200,16 @@ __device__ __forceinline__ int LoadMeta(const JoinerArgs &a, long long f0, RowMe
 
 // h[m][:] = tanh(am[frame] + lm[lmrow]) for the tile's rows (zeros beyond them), in the operand
 // type; kTransposed also keeps a copy ht[d][m] (k = row contiguous, for the weight gradient).
-template <typename Mode, int MT, bool kTransposed, int kBatch>
+template <typename Mode, int MT, bool kTransposed, int kBatch, int kD>
 __device__ __forceinline__ void StageActivations(const JoinerArgs &a, const RowMeta *meta, int rows,
                                                  typename Mode::Elem *h, int ldh,
                                                  typename Mode::Elem *ht, int ldt) {
   // A thread's items in batches of kBatch: all loads of a batch are asked for before the first is
   // used (one trip to memory per batch instead of one per item; the batch is sized to the registers
   // the caller has left).
-  const int qpr = a.D >> 2, items = MT * qpr;
+  // (kD > 0: the joiner dimension is known when compiling, and the divisions below are shifts)
+  const int dim = kD > 0 ? kD : a.D;
+  const int qpr = dim >> 2, items = MT * qpr;
   for (int base = threadIdx.x; base < items; base += kThreads * kBatch) {
     float4 x[kBatch], y[kBatch];
     int at[kBatch];  // m * qpr + q, or -1 beyond the tile's items
@@ -221,8 +223,8 @@ __device__ __forceinline__ void StageActivations(const JoinerArgs &a, const RowM
         const int m = idx / qpr, q = idx - m * qpr;
         if (m < rows) {
           const RowMeta rm = meta[m];
-          x[j] = *reinterpret_cast<const float4 *>(a.am + (size_t)rm.bt * a.D + 4 * q);
-          y[j] = *reinterpret_cast<const float4 *>(a.lm + (size_t)rm.lmrow * a.D + 4 * q);
+          x[j] = *reinterpret_cast<const float4 *>(a.am + (size_t)rm.bt * dim + 4 * q);
+          y[j] = *reinterpret_cast<const float4 *>(a.lm + (size_t)rm.lmrow * dim + 4 * q);
         }
       }
     }
@@ -341,7 +343,7 @@ __global__ __launch_bounds__(kThreads) void JoinerForwardKernel(const JoinerArgs
   const int rows = LoadMeta<MT>(a, f0, meta);
   for (int m = threadIdx.x; m < MT; m += kThreads) { zsym[m] = 0.f; zblank[m] = 0.f; }
   __syncthreads();
-  StageActivations<Mode, MT, false, 8>(a, meta, rows, h, ldh, nullptr, 0);
+  StageActivations<Mode, MT, false, 8, kD>(a, meta, rows, h, ldh, nullptr, 0);
   __syncthreads();
 
   const int lane = threadIdx.x & 63, col = lane & 31, half = lane >> 5;
@@ -484,7 +486,7 @@ __global__ __launch_bounds__(kThreads) void JoinerBackwardRowsKernel(const Joine
   for (int m = threadIdx.x; m < MT; m += kThreads)
     hdr[m] = m < rows ? a.hdr[(size_t)f0 * a.R + m] : make_float4(0.f, 0.f, -1.f, 3.0e38f);  // padding: exp(. - norm) = 0
   __syncthreads();
-  StageActivations<Mode, MT, false, 8>(a, meta, rows, h, ldh, nullptr, 0);
+  StageActivations<Mode, MT, false, 8, kD>(a, meta, rows, h, ldh, nullptr, 0);
   __syncthreads();
   {  // The tile's activations go to the workspace as an operand with k = row: this tile is step
      // blockIdx.x of k, and a 16-byte group holds consecutive rows of one column d.
