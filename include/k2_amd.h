@@ -273,8 +273,9 @@ K2AMD_API int k2amd_rnnt_prune_gather_backward(const void *grad, const int64_t *
  *   workspace: device memory, k2amd_rnnt_joiner_pruned_forward_workspace_bytes(...) bytes for the
  *   forward (the weight in the operand type) and k2amd_rnnt_joiner_pruned_workspace_bytes(...)
  *   for the backward (the weight twice, and what its first kernel hands its second: the
- *   activations and the logits' gradients in the operand type, B T R x (D + C) elements); 0 =
- *   shape not served: D a multiple of 64 up to 512, R <= 32 and <= S + 1; any C.  Contents need
+ *   activations and the logits' gradients in the operand type, B T R x (D + C) elements or, where
+ *   that is more than 128 Mi elements, as many; the backward then goes through the rows in
+ *   passes); 0 = shape not served: D a multiple of 64 up to 512, R <= 32 and <= S + 1; any C.  Contents need
  *   not survive between the two calls.
  * The backward takes what the forward took, the normalizers it wrote and the gradients w.r.t. its
  * px / py (seq_scale as for the other builders), and writes am_grad [B][T][D], lm_grad [B][S+1][D],

@@ -145,7 +145,9 @@ struct JoinerArgs {
   // d logits with rows c; and the sums of d logits over each tile's rows, [tile][Cpad]
   void *hs, *dzs;
   float *bias_part;
-  int tiles;                    // tiles of rows of the rows kernel
+  int tiles;                    // tiles of rows in the pass at hand: the steps of k of its operands
+  int tile0;                    // the pass's first tile (the backward goes through the rows in passes
+                                // that fit the workspace)
   float *am_grad, *lm_grad, *weight_grad, *bias_grad;
   int B, S, Tn, R, C, D, blank, rnnt_type;
   int Cpad, Dpad;               // C, D rounded up to whole tiles of kNTile
@@ -481,7 +483,7 @@ __global__ __launch_bounds__(kThreads) void JoinerBackwardRowsKernel(const Joine
   float4 *hdr = reinterpret_cast<float4 *>(dz + (size_t)MT * ldz);
   RowMeta *meta = reinterpret_cast<RowMeta *>(hdr + MT);
 
-  const long long f0 = (long long)blockIdx.x * a.tpt;
+  const long long f0 = ((long long)a.tile0 + blockIdx.x) * a.tpt;
   const int rows = LoadMeta<MT>(a, f0, meta);
   for (int m = threadIdx.x; m < MT; m += kThreads)
     hdr[m] = m < rows ? a.hdr[(size_t)f0 * a.R + m] : make_float4(0.f, 0.f, -1.f, 3.0e38f);  // padding: exp(. - norm) = 0
@@ -819,6 +821,19 @@ struct WorkspaceLayout {
 };
 // rows per tile of the backward's rows kernel, which is one step of k of the weight kernel
 int RowsTile(int precision) { return precision == K2AMD_JOINER_BF16 ? 64 : 32; }
+// The backward goes through the tiles in passes of equal size whose operands (activations and
+// logit gradients of the pass's rows) stay within this many elements (256 MB in bfloat16, 512 MB
+// in fp32), so that what it keeps does not grow with B T R x C.
+#ifndef K2AMD_JOINER_PASS_ELEMS
+#define K2AMD_JOINER_PASS_ELEMS ((size_t)128 << 20)
+#endif
+constexpr size_t kPassElems = K2AMD_JOINER_PASS_ELEMS;
+size_t TilesPerPass(size_t tiles, int C, int D, int precision) {
+  const size_t per_tile = (size_t)RowsTile(precision) * ((size_t)D + RoundUp(C, kNTile));
+  const size_t most = kPassElems / per_tile > 0 ? kPassElems / per_tile : 1;
+  const size_t passes = (tiles + most - 1) / most;
+  return passes > 0 ? (tiles + passes - 1) / passes : 0;
+}
 WorkspaceLayout LayoutOf(int B, int T, int R, int C, int D, int precision) {
   const size_t e = ElemBytes(precision);
   const size_t Cpad = RoundUp(C, kNTile), Dpad = RoundUp(D, kNTile);
@@ -829,11 +844,12 @@ WorkspaceLayout LayoutOf(int B, int T, int R, int C, int D, int precision) {
   w.forward_total = w.wc;  // the forward multiplies by the first copy only
   const size_t tpt = RowsTile(precision) / R;
   const size_t tiles = tpt > 0 ? ((size_t)B * T + tpt - 1) / tpt : 0;
-  const size_t padded_rows = tiles * RowsTile(precision);
+  const size_t pass_tiles = TilesPerPass(tiles, C, D, precision);
+  const size_t padded_rows = pass_tiles * RowsTile(precision);
   w.hs = (w.hdr + (size_t)B * T * R * sizeof(float4) + 255) / 256 * 256;
   w.dzs = w.hs + (padded_rows * D * e + 255) / 256 * 256;
   w.bias_part = w.dzs + (padded_rows * Cpad * e + 255) / 256 * 256;
-  w.total = w.bias_part + tiles * Cpad * sizeof(float);
+  w.total = w.bias_part + pass_tiles * Cpad * sizeof(float);
   return w;
 }
 
@@ -912,24 +928,25 @@ int BackwardImpl(const float *weight, JoinerArgs a, const float *px_grad, const 
   if (rows == 0) return LaunchStatus();
   hipLaunchKernelGGL(JoinerRowHeaderKernel, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, st, a,
                      px_grad, py_grad, seq_scale, const_cast<float4 *>(a.hdr));
-  {  // gradients of am and lm: tiles of 32 (fp32) or 64 (bfloat16) rows
-    constexpr int RB = kBf ? 2 : 1, MT = 32 * RB;
-    JoinerArgs r = a;
-    r.tpt = MT / a.R;
-    const size_t lds = (size_t)MT * (a.D + Mode::kPad + kNTile + Mode::kPad) * sizeof(Elem) +
-                       MT * (sizeof(float4) + sizeof(RowMeta));
-    auto kernel = a.D == kMaxD ? JoinerBackwardRowsKernel<Mode, RB, kMaxD> : JoinerBackwardRowsKernel<Mode, RB, 0>;
-    rc = AllowLds(kernel, lds);
-    if (rc != K2AMD_OK) return rc;
-    const long long tiles = (a.frames + r.tpt - 1) / r.tpt;
-    r.tiles = (int)tiles;
-    a.tiles = (int)tiles;
-    hipLaunchKernelGGL(kernel, dim3((unsigned)tiles), dim3(kThreads), lds, st, r);
-  }
-  {  // gradients of weight and bias: blocks of 128 x 256 of the gradient x shares of the rows
-    const int ctiles = a.Cpad / 128, dtiles = (a.D + 255) / 256;
-    int shares = 256 / (ctiles * dtiles) / 8 * 8;  // one workgroup per compute unit; a multiple of the XCDs
-    if (shares < 8) shares = 8;
+  // Gradients of am and lm, tile by tile of 32 (fp32) or 64 (bfloat16) rows, and then those of the
+  // weight and the bias from what that kernel left in the workspace (blocks of 128 x 256 of the
+  // gradient x shares of the rows), pass by pass.
+  constexpr int RB = kBf ? 2 : 1, MT = 32 * RB;
+  a.tpt = MT / a.R;
+  const size_t lds = (size_t)MT * (a.D + Mode::kPad + kNTile + Mode::kPad) * sizeof(Elem) +
+                     MT * (sizeof(float4) + sizeof(RowMeta));
+  auto kernel = a.D == kMaxD ? JoinerBackwardRowsKernel<Mode, RB, kMaxD> : JoinerBackwardRowsKernel<Mode, RB, 0>;
+  rc = AllowLds(kernel, lds);
+  if (rc != K2AMD_OK) return rc;
+  const long long tiles = (a.frames + a.tpt - 1) / a.tpt;
+  const long long pass_tiles = (long long)TilesPerPass((size_t)tiles, a.C, a.D, kBf ? K2AMD_JOINER_BF16 : K2AMD_JOINER_F32);
+  const int ctiles = a.Cpad / 128, dtiles = (a.D + 255) / 256;
+  int shares = 256 / (ctiles * dtiles) / 8 * 8;  // one workgroup per compute unit; a multiple of the XCDs
+  if (shares < 8) shares = 8;
+  for (long long first = 0; first < tiles; first += pass_tiles) {
+    a.tile0 = (int)first;
+    a.tiles = (int)(tiles - first < pass_tiles ? tiles - first : pass_tiles);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)a.tiles), dim3(kThreads), lds, st, a);
     hipLaunchKernelGGL(JoinerWeightGradKernel<Mode>, dim3((unsigned)(ctiles * dtiles * shares)),
                        dim3(kWgThreads), 0, st, a, dtiles, shares);
   }
