@@ -251,32 +251,30 @@ __device__ __forceinline__ void StageActivations(const JoinerArgs &a, const RowM
 // acc[rb] += A[rows rb*32 .. +31][0..K) . B[n][0..K)^T for the wavefront's 32 columns n: A in LDS
 // (row stride lda elements), B rows in global memory, both k-contiguous.  kSteps > 0: the number of
 // steps of k is known when compiling and the loop is unrolled completely, B asked for Mode::kAhead steps
-// and A one step ahead of their use (the compiler counts outstanding loads exactly in straight-line
-// code; around a loop it waits for all of them at every iteration).  kSteps == 0: any K, that loop.
+// ahead of its use (the compiler counts outstanding loads exactly in straight-line code; around a
+// loop it waits for all of them at every iteration).  kSteps == 0: any K, that loop.
 template <typename Mode, int RB, int kSteps>
 __device__ __forceinline__ void TileProduct(Acc16 (&acc)[RB], const typename Mode::Elem *a_lane,
                                             int lda, const uint4 *b_block, int lane, int K) {
   constexpr int kChunk = Mode::kChunk;
   if constexpr (kSteps > 0) {
     constexpr int kAhead = Mode::kAhead;  // steps of k between asking for B and using it
-    Frag fb[kAhead + 1], fa[2][RB];
+    Frag fb[kAhead + 1], fa[RB];
 #pragma unroll
     for (int i = 0; i < kAhead; ++i)
       if (i < kSteps) fb[i] = LoadFragB(b_block + (size_t)i * kFragQuads, lane);
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb) fa[0][rb] = LoadFrag(a_lane + (size_t)rb * 32 * lda);
-#pragma unroll
     for (int kc = 0; kc < kSteps; ++kc) {
       if (kc + kAhead < kSteps)
         fb[(kc + kAhead) % (kAhead + 1)] = LoadFragB(b_block + (size_t)(kc + kAhead) * kFragQuads, lane);
-      if (kc + 1 < kSteps) {
+      // A comes from LDS when its step begins: a second set of its fragments, asked for a step
+      // ahead, cost the forward kernel the registers it then spilled (155 -> 132 us in bfloat16
+      // without); the SIMD's other wavefront multiplies while this one waits for LDS.
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb)
-          fa[(kc + 1) & 1][rb] = LoadFrag(a_lane + (size_t)rb * 32 * lda + (size_t)(kc + 1) * kChunk);
-      }
+      for (int rb = 0; rb < RB; ++rb) fa[rb] = LoadFrag(a_lane + (size_t)rb * 32 * lda + (size_t)kc * kChunk);
       __builtin_amdgcn_sched_barrier(0);  // the requests above stay above the multiplies below
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb) Mode::Mma(acc[rb], fa[kc & 1][rb], fb[kc % (kAhead + 1)]);
+      for (int rb = 0; rb < RB; ++rb) Mode::Mma(acc[rb], fa[rb], fb[kc % (kAhead + 1)]);
       __builtin_amdgcn_sched_barrier(0);
     }
   } else {
