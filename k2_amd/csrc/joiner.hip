@@ -27,6 +27,8 @@
 // operand per step of k is 64 bytes (16 floats or 32 bfloat16): four 16-byte loads.  Which k a lane
 // feeds to which multiply is the same for both operands, which is all the instruction needs.
 // Workgroups are eight wavefronts, two per SIMD.
+#include <cstdlib>
+
 #include "common.h"
 
 namespace k2amd {
@@ -841,14 +843,18 @@ struct WorkspaceLayout {
 int RowsTile(int precision) { return precision == K2AMD_JOINER_BF16 ? 64 : 32; }
 // The backward goes through the tiles in passes of equal size whose operands (activations and
 // logit gradients of the pass's rows) stay within this many elements (256 MB in bfloat16, 512 MB
-// in fp32), so that what it keeps does not grow with B T R x C.
-#ifndef K2AMD_JOINER_PASS_ELEMS
-#define K2AMD_JOINER_PASS_ELEMS ((size_t)128 << 20)
-#endif
-constexpr size_t kPassElems = K2AMD_JOINER_PASS_ELEMS;
+// in fp32), so that what it keeps does not grow with B T R x C.  The environment variable
+// K2AMD_JOINER_PASS_ELEMS sets another bound (read at every call: the tests use it to go through
+// several passes at small shapes).
+constexpr size_t kPassElems = (size_t)128 << 20;
+size_t PassElems() {
+  const char *text = std::getenv("K2AMD_JOINER_PASS_ELEMS");
+  const long long given = text != nullptr ? std::atoll(text) : 0;
+  return given > 0 ? (size_t)given : kPassElems;
+}
 size_t TilesPerPass(size_t tiles, int C, int D, int precision) {
   const size_t per_tile = (size_t)RowsTile(precision) * ((size_t)D + RoundUp(C, kNTile));
-  const size_t most = kPassElems / per_tile > 0 ? kPassElems / per_tile : 1;
+  const size_t most = PassElems() / per_tile > 0 ? PassElems() / per_tile : 1;
   const size_t passes = (tiles + most - 1) / most;
   return passes > 0 ? (tiles + passes - 1) / passes : 0;
 }

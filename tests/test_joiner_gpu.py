@@ -125,6 +125,36 @@ def test_forward_small_shapes_fp32(device, rnnt_type):
         np.testing.assert_allclose(norm.cpu().numpy(), want_norm, rtol=1e-4, atol=1e-5)
 
 
+@pytest.mark.parametrize("precision", ["fp32", "bf16"])
+def test_backward_in_several_passes(device, precision, monkeypatch):
+    """The backward keeps the activations and the logits' gradients of the rows it has gone through
+    in its workspace, up to a bound; beyond it, it goes through the rows in passes.  With the
+    bound lowered (the library reads K2AMD_JOINER_PASS_ELEMS at every call) a small shape takes
+    several passes: same gradients as in one pass, up to the order of the sums."""
+    from k2_amd import capi
+    seed, B, T, S, C, D, R, with_bias = 7, 3, 57, 14, 300, 128, 4, True
+    c = joiner_case(seed, B, T, S, C, D, R, "regular", with_bias)
+    logits, px, py = chain_fp64(c)
+    _, gx, gy = omi.mi(px, py, c["boundary"])
+    gx, gy = gx.astype(np.float32), gy.astype(np.float32)
+    scale = np.linspace(0.5, 1.5, B).astype(np.float32)
+    _, _, norm = run_forward(c, device, precision)
+    args = (B, S, T, R, C, D, capi.JOINER_PRECISIONS[precision])
+    whole = capi.lib().k2amd_rnnt_joiner_pruned_workspace_bytes(*args)
+    one = run_backward(c, device, precision, norm, gx, gy, scale)
+    rows_tile = 64 if precision == "bf16" else 32
+    monkeypatch.setenv("K2AMD_JOINER_PASS_ELEMS", str(2 * rows_tile * (D + 512)))  # two tiles a pass
+    assert capi.lib().k2amd_rnnt_joiner_pruned_workspace_bytes(*args) < whole
+    several = run_backward(c, device, precision, norm, gx, gy, scale)
+    monkeypatch.delenv("K2AMD_JOINER_PASS_ELEMS")
+    for name, g, w in zip(("am_grad", "lm_grad", "weight_grad", "bias_grad"), several, one):
+        close(f"{precision} {name}", g, w, 1e-5, 1e-6)
+    if precision == "fp32":
+        for name, g, w in zip(("am_grad", "lm_grad", "weight_grad", "bias_grad"), several,
+                              closed_form_grads(c, logits, gx, gy, scale)):
+            close(name, g, w, 1e-4, 1e-5)
+
+
 @pytest.mark.parametrize("rnnt_type", TYPES)
 def test_backward_small_shapes_fp32(device, rnnt_type):
     for seed, B, T, S, C, D, R, with_bias in SMALL:
