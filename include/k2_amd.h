@@ -275,7 +275,8 @@ K2AMD_API int k2amd_rnnt_prune_gather_backward(const void *grad, const int64_t *
  *   for the backward (the weight twice, and what its first kernel hands its second: the
  *   activations and the logits' gradients in the operand type, B T R x (D + C) elements or, where
  *   that is more than 128 Mi elements, as many; the backward then goes through the rows in
- *   passes); 0 = shape not served: D a multiple of 64 up to 512, R <= 32 and <= S + 1; any C.  Contents need
+ *   passes; the environment variable K2AMD_JOINER_PASS_ELEMS, read at every call, sets another
+ *   bound); 0 = shape not served: D a multiple of 64 up to 512, R <= 32 and <= S + 1; any C.  Contents need
  *   not survive between the two calls.
  * The backward takes what the forward took, the normalizers it wrote and the gradients w.r.t. its
  * px / py (seq_scale as for the other builders), and writes am_grad [B][T][D], lm_grad [B][S+1][D],
