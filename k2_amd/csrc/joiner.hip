@@ -482,6 +482,7 @@ __global__ __launch_bounds__(kThreads) void JoinerBackwardRowsKernel(const Joine
   float *stage = reinterpret_cast<float *>(dz);  // after the last column tile
   float4 *hdr = reinterpret_cast<float4 *>(dz + (size_t)MT * ldz);
   RowMeta *meta = reinterpret_cast<RowMeta *>(hdr + MT);
+  unsigned long long *run_ends = reinterpret_cast<unsigned long long *>(meta + MT);  // [32]
 
   const long long f0 = ((long long)a.tile0 + blockIdx.x) * a.tpt;
   const int rows = LoadMeta<MT>(a, f0, meta);
@@ -584,9 +585,32 @@ __global__ __launch_bounds__(kThreads) void JoinerBackwardRowsKernel(const Joine
     __syncthreads();
   }
 
-  const int part = threadIdx.x / kStageCols, c = threadIdx.x % kStageCols;
+  const int c = threadIdx.x % kStageCols;
+  const int part = __builtin_amdgcn_readfirstlane(threadIdx.x / kStageCols);  // the same in a wavefront
   constexpr int kParts = kThreads / kStageCols;
   const int nf = rows / a.R;
+  // What the sums below need to know about the tile's rows does not depend on the column: where a
+  // run of equal lm rows ends (bit fl of a position's word: after frame fl).  Worked out once per
+  // tile, one thread per position k; the loops over the columns are then reads and adds.
+  constexpr int kTakes = 2;
+  static_assert(MT <= 64, "a bit per frame");
+  if ((int)threadIdx.x < a.R) {
+    const int k = threadIdx.x;
+    unsigned long long ends = 0;
+    int key = meta[k].lmrow;
+    for (int fl = 0; fl < nf; ++fl) {
+      const int next = fl + 1 < nf ? meta[(fl + 1) * a.R + k].lmrow : -1;
+      if (next != key) ends |= 1ull << fl;
+      key = next;
+    }
+    run_ends[k] = ends;
+  }
+  auto ends_of = [&](int k) -> unsigned long long {  // (after the first barrier below)
+    const unsigned long long ends = run_ends[k];
+    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)ends);
+    const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(ends >> 32));
+    return ((unsigned long long)hi << 32) | lo;
+  };
   for (int d0 = 0; d0 < a.D; d0 += kStageCols) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
@@ -605,45 +629,56 @@ __global__ __launch_bounds__(kThreads) void JoinerBackwardRowsKernel(const Joine
     }
     __syncthreads();
     if (d0 + c < a.D) {
-      // (The loops below ask for four LDS values at a time before they use any: with one read per
-      // iteration, each waiting for the one before it, they took a third of the kernel.)
+      // am_grad[frame] = the sum of the frame's R rows; four values asked for before any is used
+      // (one read per iteration, each waiting for the one before it, is what these loops cost).
+      const int frame_step = a.R * kLdStage;
       for (int fl = part; fl < nf; fl += kParts) {
+        const float *src = stage + fl * frame_step + c;
         float sum = 0.f;
-        const float *src = stage + (size_t)fl * a.R * kLdStage + c;
-        for (int k0 = 0; k0 < a.R; k0 += 4) {
-          float v[4];
-#pragma unroll
-          for (int j = 0; j < 4; ++j) v[j] = src[(size_t)min(k0 + j, a.R - 1) * kLdStage];
-#pragma unroll
-          for (int j = 0; j < 4; ++j)
-            if (k0 + j < a.R) sum += v[j];
+        int k = 0;
+        for (; k + 4 <= a.R; k += 4) {
+          const float v0 = src[0], v1 = src[kLdStage], v2 = src[2 * kLdStage], v3 = src[3 * kLdStage];
+          sum += v0; sum += v1; sum += v2; sum += v3;
+          src += 4 * kLdStage;
         }
+        for (; k < a.R; ++k, src += kLdStage) sum += *src;
         a.am_grad[(size_t)(f0 + fl) * a.D + d0 + c] = sum;
       }
-      for (int k = part; k < a.R; k += kParts) {
-        int key = -1;
-        float sum = 0.f;
-        for (int fl0 = 0; fl0 < nf; fl0 += 4) {
-          int keys[4];
-          float v[4];
+      // lm_grad[lm row] += the sum of each run of frames that took that row at position k
+      for (int kb = part; kb < a.R; kb += kTakes * kParts) {
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const int row = min(fl0 + j, nf - 1) * a.R + k;
-            keys[j] = meta[row].lmrow;
-            v[j] = stage[row * kLdStage + c];
+        for (int t = 0; t < kTakes; ++t) {
+          const int k = kb + t * kParts;
+          if (k >= a.R) break;
+          unsigned long long ends = ends_of(k);
+          const float *src = stage + k * kLdStage + c;
+          float sum = 0.f;
+          int fl = 0;
+          for (; fl + 4 <= nf; fl += 4) {
+            const float v[4] = {src[0], src[frame_step], src[2 * frame_step], src[3 * frame_step]};
+            src += 4 * frame_step;
+            const unsigned four = (unsigned)(ends >> fl) & 15u;
+            if (four == 0) {  // (the common case: the run goes on)
+              sum += v[0]; sum += v[1]; sum += v[2]; sum += v[3];
+              continue;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              sum += v[j];
+              if (four >> j & 1) {
+                atomicAdd(a.lm_grad + (size_t)meta[(fl + j) * a.R + k].lmrow * a.D + d0 + c, sum);
+                sum = 0.f;
+              }
+            }
           }
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            if (fl0 + j >= nf) break;
-            if (keys[j] != key) {
-              if (key >= 0) atomicAdd(a.lm_grad + (size_t)key * a.D + d0 + c, sum);
-              key = keys[j];
+          for (; fl < nf; ++fl, src += frame_step) {
+            sum += *src;
+            if (ends >> fl & 1) {
+              atomicAdd(a.lm_grad + (size_t)meta[fl * a.R + k].lmrow * a.D + d0 + c, sum);
               sum = 0.f;
             }
-            sum += v[j];
           }
         }
-        if (key >= 0) atomicAdd(a.lm_grad + (size_t)key * a.D + d0 + c, sum);
       }
     }
     __syncthreads();
@@ -958,7 +993,7 @@ int BackwardImpl(const float *weight, JoinerArgs a, const float *px_grad, const 
   constexpr int RB = kBf ? 2 : 1, MT = 32 * RB;
   a.tpt = MT / a.R;
   const size_t lds = (size_t)MT * (a.D + Mode::kPad + kNTile + Mode::kPad) * sizeof(Elem) +
-                     MT * (sizeof(float4) + sizeof(RowMeta));
+                     MT * (sizeof(float4) + sizeof(RowMeta)) + 32 * sizeof(unsigned long long);
   auto kernel = a.D == kMaxD ? JoinerBackwardRowsKernel<Mode, RB, kMaxD> : JoinerBackwardRowsKernel<Mode, RB, 0>;
   rc = AllowLds(kernel, lds);
   if (rc != K2AMD_OK) return rc;
