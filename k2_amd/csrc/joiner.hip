@@ -365,21 +365,42 @@ __global__ __launch_bounds__(kThreads) void JoinerForwardKernel(const JoinerArgs
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[rb][r] = 0.f;
     TileProduct<Mode, RB, kStepsD>(acc, a_lane, ldh, BOperand(a.wk, (n0 >> 5) + wave, a.D / Mode::kChunk, 0), lane, a.D);
-    if (n < a.C) {
-      const float bn = a.bias != nullptr ? a.bias[n] : 0.f;
+    const float bn = (n < a.C && a.bias != nullptr) ? a.bias[n] : 0.f;
+    if (n0 == 0) {
+      // the first tile of columns starts the running pairs: no exponential (a lane whose column
+      // lies beyond C keeps the empty pair)
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if (n < a.C) { run_m[rb][r] = acc[rb][r] + bn; run_s[rb][r] = 1.0f; }
+    } else if (n < a.C) {
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int row = rb * 32 + AccRow(r, half);
           const float z = acc[rb][r] + bn;
           const float m = run_m[rb][r], d = z - m;
           const float e = __expf(-fabsf(d));
           run_s[rb][r] = d > 0 ? run_s[rb][r] * e + 1.0f : run_s[rb][r] + e;
           run_m[rb][r] = d > 0 ? z : m;
-          if (n == meta[row].sym) zsym[row] = z;
-          if (n == a.blank) zblank[row] = z;
         }
+    }
+    if (n < a.C) {
+      // the two logits a row contributes: the lane that holds one parks it
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = rb * 32 + AccRow(r, half);
+          if (n == meta[row].sym) zsym[row] = acc[rb][r] + bn;
+        }
+      if (n == a.blank) {
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) zblank[rb * 32 + AccRow(r, half)] = acc[rb][r] + bn;
+      }
     }
   }
   // (max, sum) of a row: over the 32 lanes that hold its columns, then over the wavefronts.  The
