@@ -796,11 +796,31 @@ __global__ __launch_bounds__(kWgThreads) void JoinerWeightGradKernel(const Joine
 
 // The weight [C][D] in the operand type and in the order the multiplies read it (see BOperand):
 // wk with rows n = c (Cpad of them, zeros beyond C) and k = d; wc with rows n = d (Dpad) and k = c
-// (Cpad, zeros beyond C and D).  One thread per 16-byte group.
+// (Cpad, zeros beyond C and D).  One thread per 16-byte group.  The same launch fills the tensors
+// that the kernels after it only write in part (px, py: -inf) or add to (the sums of atomic adds).
+struct Fills {
+  float *at[3];
+  size_t n[3];
+  float value;
+};
 template <typename Mode>
 __global__ void JoinerPrepWeightKernel(const float *__restrict__ weight, uint4 *wk, uint4 *wc, int C,
-                                       int D, int Cpad, int Dpad) {
+                                       int D, int Cpad, int Dpad, const Fills fills) {
   typedef typename Mode::Elem Elem;
+#pragma unroll
+  for (int f = 0; f < 3; ++f) {
+    float *at = fills.at[f];
+    const size_t n = fills.n[f];
+    if (at == nullptr || n == 0) continue;
+    // whole 16-byte groups where the tensor's address allows, single floats around them
+    const size_t head = ((16 - (reinterpret_cast<size_t>(at) & 15)) & 15) / sizeof(float);
+    const size_t lead = head < n ? head : n, quads = (n - lead) / 4;
+    const size_t first = (size_t)blockIdx.x * blockDim.x + threadIdx.x, stride = (size_t)gridDim.x * blockDim.x;
+    const float4 four = make_float4(fills.value, fills.value, fills.value, fills.value);
+    for (size_t i = first; i < quads; i += stride) reinterpret_cast<float4 *>(at + lead)[i] = four;
+    if (first < lead) at[first] = fills.value;
+    if (first < n - lead - 4 * quads) at[lead + 4 * quads + first] = fills.value;
+  }
   constexpr int kPer = 16 / sizeof(Elem);  // elements per group
   const size_t nk = (size_t)Cpad * D / kPer, nc = wc != nullptr ? (size_t)Dpad * Cpad / kPer : 0;
   for (size_t g = (size_t)blockIdx.x * blockDim.x + threadIdx.x; g < nk + nc;
@@ -831,13 +851,6 @@ __global__ void JoinerPrepWeightKernel(const float *__restrict__ weight, uint4 *
     }
     (second ? wc : wk)[j] = out;
   }
-}
-
-__global__ void JoinerFillKernel(float *a, size_t na, float va, float *b, size_t nb, float vb) {
-  const size_t first = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const size_t stride = (size_t)gridDim.x * blockDim.x;
-  for (size_t i = first; i < na; i += stride) a[i] = va;
-  for (size_t i = first; i < nb; i += stride) b[i] = vb;
 }
 
 // px[b,s,t] += py[b,s+1,t] (k2/python/k2/rnnt_loss.py:1345-1346); T1 == Tn here.
@@ -964,22 +977,22 @@ JoinerArgs MakeArgs(const float *am, const float *lm, const int64_t *ranges, con
 }
 
 template <typename Mode>
-int PrepWeights(const float *weight, const JoinerArgs &a, bool both, hipStream_t st) {
-  hipLaunchKernelGGL(JoinerPrepWeightKernel<Mode>, dim3(512), dim3(256), 0, st, weight,
+int PrepWeights(const float *weight, const JoinerArgs &a, bool both, const Fills &fills, hipStream_t st) {
+  hipLaunchKernelGGL(JoinerPrepWeightKernel<Mode>, dim3(1024), dim3(256), 0, st, weight,
                      static_cast<uint4 *>(const_cast<void *>(a.wk)),
-                     both ? static_cast<uint4 *>(const_cast<void *>(a.wc)) : nullptr, a.C, a.D, a.Cpad, a.Dpad);
+                     both ? static_cast<uint4 *>(const_cast<void *>(a.wc)) : nullptr, a.C, a.D, a.Cpad,
+                     a.Dpad, fills);
   return LaunchStatus();
 }
 
 template <typename Mode, int RB>
 int ForwardImpl(const float *weight, JoinerArgs a, hipStream_t st) {
   constexpr int MT = 32 * RB;
-  int rc = PrepWeights<Mode>(weight, a, false, st);
-  if (rc != K2AMD_OK) return rc;
   const size_t npx = (size_t)a.B * a.S * (a.rnnt_type == K2AMD_REGULAR ? a.Tn + 1 : a.Tn);
   const size_t npy = (size_t)a.B * (a.S + 1) * a.Tn;
-  hipLaunchKernelGGL(JoinerFillKernel, dim3(512), dim3(256), 0, st, a.px, npx, Real<float>::NegInf(),
-                     a.py, npy, Real<float>::NegInf());
+  const Fills fills{{a.px, a.py, nullptr}, {npx, npy, 0}, Real<float>::NegInf()};
+  int rc = PrepWeights<Mode>(weight, a, false, fills, st);
+  if (rc != K2AMD_OK) return rc;
   const size_t lds = (size_t)MT * (a.D + Mode::kPad) * sizeof(typename Mode::Elem) +
                      MT * (sizeof(RowMeta) + (2 + 2 * kWaves) * sizeof(float));
   auto kernel = a.D == kMaxD ? JoinerForwardKernel<Mode, RB, kMaxD> : JoinerForwardKernel<Mode, RB, 0>;
@@ -997,14 +1010,12 @@ int BackwardImpl(const float *weight, JoinerArgs a, const float *px_grad, const 
                  const float *seq_scale, hipStream_t st) {
   typedef typename Mode::Elem Elem;
   constexpr bool kBf = sizeof(Elem) == 2;
-  int rc = PrepWeights<Mode>(weight, a, true, st);
+  const Fills fills{{a.lm_grad, a.weight_grad, a.bias_grad},
+                    {(size_t)a.B * (a.S + 1) * a.D, (size_t)a.C * a.D, a.bias_grad != nullptr ? (size_t)a.C : 0},
+                    0.f};
+  int rc = PrepWeights<Mode>(weight, a, true, fills, st);
   if (rc != K2AMD_OK) return rc;
   const long long rows = a.frames * a.R;
-  hipLaunchKernelGGL(JoinerFillKernel, dim3(512), dim3(256), 0, st, a.lm_grad,
-                     (size_t)a.B * (a.S + 1) * a.D, 0.f, a.weight_grad, (size_t)a.C * a.D, 0.f);
-  if (a.bias_grad != nullptr)
-    hipLaunchKernelGGL(JoinerFillKernel, dim3(4), dim3(256), 0, st, a.bias_grad, (size_t)a.C, 0.f,
-                       static_cast<float *>(nullptr), (size_t)0, 0.f);
   if (rows == 0) return LaunchStatus();
   hipLaunchKernelGGL(JoinerRowHeaderKernel, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, st, a,
                      px_grad, py_grad, seq_scale, const_cast<float4 *>(a.hdr));
