@@ -363,7 +363,10 @@ def logprobs_simple_backward(px_grad, py_grad, symbols, boundary, saved, termina
     _symbol(termination_symbol, C)
     lm_grad = torch.empty_like(lm_probs)
     am_grad = torch.empty_like(am_probs)
-    q = torch.empty_like(denom)
+    # the products' operand [B][S+1][T], then the gradients' sums along s (per 32 rows) and along t
+    # (per 64 frames)
+    rows = B * (S + 1)
+    q = torch.empty(rows * T + B * ((S + 32) // 32) * T + 2 * rows * ((T + 63) // 64), dtype=dt, device=dev)
     dev = am_probs.device
     with torch.cuda.device(dev):
         check(lib().k2amd_rnnt_logprobs_simple_backward(

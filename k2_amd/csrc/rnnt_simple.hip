@@ -6,9 +6,9 @@
 // the log, adds the maxima back and emits
 // px / py directly, so the normaliser never makes a round trip through HBM as a separate tensor
 // apart from the `denom` buffer kept for the backward.
-// Backward: Q = (dpx + dpy) / denom, two more batched products (Q * am_probs, Q^T * lm_probs)
-// scaled by the saved exponentials; the symbol terms of the am gradient ride in that product's
-// epilogue, the termination terms and the lm gradient's gathered terms have small kernels.
+// Backward: one pass over dpx, dpy writes Q = (dpx + dpy) / denom and their sums along s and t;
+// two more batched products (Q * am_probs, Q^T * lm_probs) scaled by the saved exponentials,
+// whose epilogues add the gathered terms (symbol and termination columns) from those sums.
 #include "common.h"
 
 namespace k2amd {
@@ -86,6 +86,33 @@ constexpr int kTile = 64, kTileK = 16, kPad = 4;
 constexpr int kStageColumns = 64, kMaxHits = 4;
 constexpr int kStageInts = kStageColumns * (1 + kMaxHits);
 
+// What an epilogue loads for a thread's elements (all in one column n, rows `rows`, clamped into
+// the matrix by the caller), in rounds so that the loads of one round are in flight together: the
+// compiler cannot move a load across a store that might alias it or out of a branch, and one
+// dependent round trip per element is what a tile's epilogue would otherwise cost.
+//   pre[r] = epi.Prepare(b, m, n, column)            what every element loads
+//   for k < Epilogue::kLevels: if any element of the wavefront has epi.Wants(k, column, pre[r]):
+//       epi.Extra(k, b, m, n, column, pre[r])         for every element; loads without branches
+//                                                    (from clamped addresses), values by select
+template <typename Epilogue, int R>
+__device__ __forceinline__ void PrepareElements(const Epilogue &epi, int b, const int (&rows)[R],
+                                                int n, const typename Epilogue::ColumnData &column,
+                                                typename Epilogue::ElementData (&pre)[R]) {
+#pragma unroll
+  for (int r = 0; r < R; ++r) pre[r] = epi.Prepare(b, rows[r], n, column);
+  if constexpr (Epilogue::kLevels > 0) {
+#pragma unroll
+    for (int k = 0; k < Epilogue::kLevels; ++k) {
+      bool wanted = false;
+#pragma unroll
+      for (int r = 0; r < R; ++r) wanted |= epi.Wants(k, column, pre[r]);
+      if (!__any(wanted)) continue;
+#pragma unroll
+      for (int r = 0; r < R; ++r) epi.Extra(k, b, rows[r], n, column, pre[r]);
+    }
+  }
+}
+
 // fp64: one 64 x 64 output tile per workgroup, K in steps of 16 staged through LDS as As[k][m],
 // Bs[k][n] (scalar, bounds-checked loads: any stride works), 16 x 16 threads with 4 x 4 outputs
 // each on the vector ALUs.
@@ -142,11 +169,10 @@ __global__ __launch_bounds__(256) void BatchedProductKernel(const T *__restrict_
     if (n >= N) continue;
     const auto column = epi.Column(b, n, n - n0, stage);
     typename Epilogue::ElementData pre[4];
+    int rows[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int m = m0 + ty * 4 + i;
-      if (m < M) pre[i] = epi.Prepare(b, m, n, column);
-    }
+    for (int i = 0; i < 4; ++i) rows[i] = min(m0 + ty * 4 + i, M - 1);
+    PrepareElements(epi, b, rows, n, column, pre);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int m = m0 + ty * 4 + i;
@@ -232,15 +258,19 @@ __global__ __launch_bounds__(256) void ProductSplitKKernel(const float *__restri
   Acc16 acc;
 #pragma unroll
   for (int i = 0; i < 16; ++i) acc[i] = 0;
+  float ra[kAhead][8], rb[kAhead][8];
+  const int c_last = c_end - 1;
   if (c_begin < c_end) {
-    float ra[kAhead][8], rb[kAhead][8];
-    const int c_last = c_end - 1;
 #pragma unroll
     for (int d = 0; d < kAhead; ++d) {
       const int k = min(c_begin + d, c_last) * kChunk + half * 8;
       oa.Full(k, ra[d]);
       ob.Full(k, rb[d]);
     }
+  }
+  // (here: what the staging waits for is covered by the operands' first loads)
+  if constexpr (Epilogue::kStaged) epi.Stage(b, n0, kMfmaTile, stage);
+  if (c_begin < c_end) {
     int c = c_begin;
     for (; c + kAhead <= c_end; c += kAhead) {
 #pragma unroll
@@ -281,15 +311,13 @@ __global__ __launch_bounds__(256) void ProductSplitKKernel(const float *__restri
 #pragma unroll
   for (int r = 0; r < 16; ++r) part[wave][(r >> 2) * 8 + half * 4 + (r & 3)][col] = acc[r];
   __syncthreads();
-  if constexpr (Epilogue::kStaged) epi.Stage(b, n0, kMfmaTile, stage);
   if (n >= N) return;
   const auto column = epi.Column(b, n, col, stage);
   typename Epilogue::ElementData pre[4];
+  int rows[4];
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const int m = m0 + wave * 8 + half * 4 + r;
-    if (m < M) pre[r] = epi.Prepare(b, m, n, column);
-  }
+  for (int r = 0; r < 4; ++r) rows[r] = min(m0 + wave * 8 + half * 4 + r, M - 1);
+  PrepareElements(epi, b, rows, n, column, pre);
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const int row = wave * 8 + half * 4 + r;
@@ -438,6 +466,8 @@ __global__ __launch_bounds__(256) void ProductLdsKernel(const float *__restrict_
   };
   sa.Fetch(0, ra);
   sb.Fetch(0, rb);
+  // (here: what the staging waits for is covered by the operands' first loads)
+  if constexpr (Epilogue::kStaged) epi.Stage(b, n0, kTile, stage);
   sa.Park(As[0], ra);
   sb.Park(Bs[0], rb);
   sa.Fetch(kKc, ra);
@@ -448,16 +478,14 @@ __global__ __launch_bounds__(256) void ProductLdsKernel(const float *__restrict_
     chunk(c, fa[0], fb[0], fa[1], fb[1]);
     if (c + 1 < chunks) chunk(c + 1, fa[1], fb[1], fa[0], fb[0]);
   }
-  if constexpr (Epilogue::kStaged) epi.Stage(b, n0, kTile, stage);
   const int n = n0 + qn + col;
   if (n >= N) return;
   const auto column = epi.Column(b, n, qn + col, stage);
   typename Epilogue::ElementData pre[16];
+  int rows[16];
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int m = m0 + qm + (r >> 2) * 8 + half * 4 + (r & 3);
-    if (m < M) pre[r] = epi.Prepare(b, m, n, column);
-  }
+  for (int r = 0; r < 16; ++r) rows[r] = min(m0 + qm + (r >> 2) * 8 + half * 4 + (r & 3), M - 1);
+  PrepareElements(epi, b, rows, n, column, pre);
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const int m = m0 + qm + (r >> 2) * 8 + half * 4 + (r & 3);
@@ -518,7 +546,10 @@ void LaunchProduct(const T *A, MatView av, const T *Bm, MatView bv, int M, int N
   if (M <= 0 || N <= 0 || B <= 0) return;
   if constexpr (sizeof(T) == 4) {
     const long long big_tiles = (long long)((N + 63) / 64) * ((M + 63) / 64) * B;
-    if (big_tiles >= 512)  // two workgroups per compute unit without splitting K
+    // The 64 x 64 tiles once they give every compute unit two workgroups; four where K is short:
+    // the operands then matter little and a 32 x 32 tile's epilogue is a quarter as long per thread
+    // (B=16 T=250 S=50 C=500, the am gradient, K = 51: 15.4 us against 18.4 us).
+    if (big_tiles >= (K <= 128 ? 1024 : 512))
       LaunchLds<kAKFast, kBKFast>(A, av, Bm, bv, M, N, K, B, epi, st);
     else
       LaunchSplitK(A, av, Bm, bv, M, N, K, B, epi, st);
@@ -556,13 +587,12 @@ struct GradView {
   }
 };
 
-// Epilogues work in two steps so that a thread can issue the loads of all its elements before
-// the first store (the compiler cannot move a load across a store that might alias it, and one
-// dependent round trip per element is what the tile's epilogue would otherwise cost):
+// Epilogues work in steps so that a thread can issue the loads of all its elements before the
+// first store (see PrepareElements):
 //   epi.Stage(b, n0, width, scratch)          (only if Epilogue::kStaged; whole workgroup, has
 //                                              barriers) what depends on the tile's columns
 //   column = epi.Column(b, n, n - n0, scratch)   what depends on (b, n) only
-//   pre    = epi.Prepare(b, m, n, column)        loads for element (m, n)
+//   PrepareElements: epi.Prepare, then epi.Wants / epi.Extra for Epilogue::kLevels rounds
 //   epi.Finish(b, m, n, acc, column, pre)        arithmetic and stores
 
 // Forward epilogue: (m, n) = (s, t).  Also writes the -inf column px[b,s,T] of a regular lattice
@@ -582,6 +612,7 @@ struct ForwardEpilogue {
     T lm_max, lm_blank, sym_sum;  // sym_sum = am[b,t,sym] + lm[b,s,sym], -inf without a symbol
   };
   static constexpr bool kStaged = false;
+  static constexpr int kLevels = 0;
   __device__ __forceinline__ ColumnData Column(int b, int t, int, const int *) const {
     ColumnData c;
     c.amr = am + ((size_t)b * Tn + t) * C;
@@ -619,27 +650,58 @@ struct ForwardEpilogue {
   }
 };
 
-// Backward epilogue: out[b][m][n] = -scale[b][m][n] * acc  (scale = the saved exponentials).
+// Epilogue of the lm gradient, (m, n) = (s, c):
+//   lm_grad[b,s,c] = -lm_probs[b,s,c] * acc + (c == symbols[b,s]) * sum_t Gx(b,s,t)
+//                    + (c == blank) * sum_t Gy(b,s,t).
+// The two sums come from QSumsKernel as one value per chunk of t and are added here in the order
+// of the chunks.
 template <typename T>
-struct ScaleEpilogue {
-  const T *scale;
+struct LmGradEpilogue {
+  const T *scale;  // lm_probs
   T *out;
-  int M, N;
+  const int64_t *symbols;
+  const T *row_x, *row_y;  // [B][S+1][chunks]
+  int S, N, chunks, blank;
   struct ColumnData {};
-  struct ElementData { T scale; };
+  struct ElementData {
+    T scale, sum_x, sum_y;
+    bool takes_x, takes_y;
+  };
   static constexpr bool kStaged = false;
+  static constexpr int kLevels = 1;
   __device__ __forceinline__ ColumnData Column(int, int, int, const int *) const { return ColumnData(); }
-  __device__ __forceinline__ ElementData Prepare(int b, int m, int n, const ColumnData &) const {
-    return ElementData{scale[((size_t)b * M + m) * N + n]};
+  __device__ __forceinline__ ElementData Prepare(int b, int s, int c, const ColumnData &) const {
+    ElementData e;
+    e.scale = scale[((size_t)b * (S + 1) + s) * N + c];
+    e.sum_x = e.sum_y = 0;
+    const int64_t sym = S > 0 ? symbols[(size_t)b * S + min(s, S - 1)] : -1;
+    e.takes_x = s < S && sym == c;
+    e.takes_y = c == blank;
+    return e;
   }
-  __device__ __forceinline__ void Finish(int b, int m, int n, T acc, const ColumnData &,
+  __device__ __forceinline__ bool Wants(int, const ColumnData &, const ElementData &e) const {
+    return e.takes_x || e.takes_y;
+  }
+  __device__ __forceinline__ void Extra(int, int b, int s, int, const ColumnData &, ElementData &e) const {
+    const size_t first = ((size_t)b * (S + 1) + s) * chunks;
+    T sx = 0, sy = 0;
+    for (int k = 0; k < chunks; ++k) {
+      sx += row_x[first + k];
+      sy += row_y[first + k];
+    }
+    e.sum_x = e.takes_x ? sx : T(0);
+    e.sum_y = e.takes_y ? sy : T(0);
+  }
+  __device__ __forceinline__ void Finish(int b, int s, int c, T acc, const ColumnData &,
                                          const ElementData &e) const {
-    out[((size_t)b * M + m) * N + n] = -e.scale * acc;
+    out[((size_t)b * (S + 1) + s) * N + c] = (-e.scale * acc + e.sum_x) + e.sum_y;
   }
 };
 
 // Epilogue of the am gradient, (m, n) = (t, c):
-//   am_grad[b,t,c] = -am_probs[b,t,c] * acc + sum over s with symbols[b,s] == c of Gx(b,s,t).
+//   am_grad[b,t,c] = -am_probs[b,t,c] * acc + sum over s with symbols[b,s] == c of Gx(b,s,t)
+//                    + (c == blank) * sum over s of Gy(b,s,t)
+// (the latter from QSumsKernel as one value per group of rows s, added here in the groups' order).
 // Stage lists, for each of the tile's columns, the positions s whose symbol is that column (up
 // to kMaxHits, sorted; longer lists are rescanned per element), so that the symbol terms cost a
 // tile one pass over the sequence's symbols instead of a launch of their own.  The terms of an
@@ -651,10 +713,16 @@ struct AmGradEpilogue {
   T *out;
   GradView<T> gv;
   const int64_t *symbols;
-  int M, N;  // Tn, C
+  const T *col_y;  // [B][groups][Tn]
+  int M, N;        // Tn, C
+  int blank, groups;
+  static constexpr int kLevels = kMaxHits + 1;
   struct ColumnData {
     int hits;  // positions s with symbols[b,s] == c (all of them, also beyond kMaxHits)
     int s[kMaxHits];
+    T scale;          // of sequence b
+    int64_t t_cut;    // regular lattice with a boundary: px_grad[b, :, t_cut] does not count
+    bool is_blank;
   };
   struct ElementData { T scale, sym_sum; };
   __device__ void Stage(int b, int n0, int width, int *scratch) const {
@@ -682,27 +750,44 @@ struct AmGradEpilogue {
     }
     __syncthreads();
   }
-  __device__ __forceinline__ ColumnData Column(int, int, int local, const int *scratch) const {
+  __device__ __forceinline__ ColumnData Column(int b, int c, int local, const int *scratch) const {
     ColumnData col;
+    col.is_blank = c == blank;
     col.hits = scratch[local];
 #pragma unroll
     for (int k = 0; k < kMaxHits; ++k) col.s[k] = scratch[kStageColumns + local * kMaxHits + k];
+    col.scale = gv.Scale(b);
+    col.t_cut = gv.rnnt_type == K2AMD_REGULAR && gv.boundary != nullptr ? gv.boundary[4 * b + 3] : -1;
     return col;
   }
-  __device__ __forceinline__ ElementData Prepare(int b, int t, int c, const ColumnData &col) const {
-    ElementData e;
-    e.scale = scale[((size_t)b * M + t) * N + c];
-    e.sym_sum = 0;
+  __device__ __forceinline__ ElementData Prepare(int b, int t, int c, const ColumnData &) const {
+    return ElementData{scale[((size_t)b * M + t) * N + c], T(0)};
+  }
+  // Rounds 0 .. kMaxHits-1: the column's k-th position s; the last round: the blank column's sums.
+  __device__ __forceinline__ bool Wants(int k, const ColumnData &col, const ElementData &) const {
+    return k < kMaxHits ? k < col.hits : col.is_blank;
+  }
+  __device__ __forceinline__ void Extra(int k, int b, int t, int c, const ColumnData &col,
+                                        ElementData &e) const {
+    if (k == kMaxHits) {
+      T sum = 0;
+      for (int g = 0; g < groups; ++g) sum += col_y[((size_t)b * groups + g) * M + t];
+      if (col.is_blank) e.sym_sum += sum;
+      return;
+    }
     if (col.hits <= kMaxHits) {
-#pragma unroll
-      for (int k = 0; k < kMaxHits; ++k)
-        if (k < col.hits) e.sym_sum += gv.Gx(b, col.s[k], t);
-    } else {
+      // Gx(b, s, t) of GradView, the load from position 0 where this column has no k-th position
+      // (a round only runs where some column has one, so S > 0)
+      const bool mine = k < col.hits;
+      const int T1 = gv.rnnt_type == K2AMD_REGULAR ? gv.Tn + 1 : gv.Tn;
+      const T raw = gv.px_grad[((size_t)b * gv.S + (mine ? col.s[k] : 0)) * T1 + t];
+      const T g = MulRounded(raw, col.scale);
+      if (mine && t != col.t_cut) e.sym_sum += g;
+    } else if (k == 0) {  // a longer list: every position of the sequence, in order
       const int64_t *sym = symbols + (size_t)b * gv.S;
       for (int s = 0; s < gv.S; ++s)
         if (sym[s] == c) e.sym_sum += gv.Gx(b, s, t);
     }
-    return e;
   }
   __device__ __forceinline__ void Finish(int b, int t, int c, T acc, const ColumnData &,
                                          const ElementData &e) const {
@@ -734,64 +819,104 @@ __global__ void ConstrainedKernelS(T *__restrict__ px, const T *__restrict__ py,
   }
 }
 
-template <typename T>
-__global__ void QKernel(GradView<T> gv, const T *__restrict__ denom, T *__restrict__ q, int B) {
-  const size_t n = (size_t)B * (gv.S + 1) * gv.Tn;
-  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-       i += (size_t)gridDim.x * blockDim.x) {
-    const int t = (int)(i % gv.Tn);
-    const int s = (int)((i / gv.Tn) % (gv.S + 1));
-    const int b = (int)(i / ((size_t)gv.Tn * (gv.S + 1)));
-    q[i] = (gv.Gx(b, s, t) + gv.Gy(b, s, t)) / denom[i];
-  }
-}
+// One pass over the lattice's gradients for the whole backward:
+//   q[b,s,t] = (Gx + Gy) / denom                   the A operand of the two products
+//   col_y[b,g,t] = sum of Gy(b,s,t) over group g's kSumsGroup rows s
+//                                                  the termination terms of the am gradient
+//   row_x / row_y[b,s,chunk] = sum of Gx / Gy over the chunk's kSumsChunk values of t
+//                                                  the gathered terms of the lm gradient
+// One workgroup per (chunk of t, group of s, b); each of its four wavefronts takes kSumsRows
+// consecutive rows and requests all it reads at once, from addresses clamped into the tensors
+// (one round trip to memory instead of one per row).  The consumers add the groups / chunks in
+// order, and every sum here is added in a fixed order: no result depends on scheduling.
+constexpr int kSumsChunk = 64, kSumsRows = 8, kSumsGroup = 4 * kSumsRows;
 
-// lm_grad[b,s,sym[b,s]] += sum_t Gx; lm_grad[b,s,blank] += sum_t Gy.  One wavefront per (b,s).
-template <typename T>
-__global__ __launch_bounds__(256) void LmGatherTermsKernel(GradView<T> gv,
-                                                           const int64_t *__restrict__ symbols,
-                                                           T *__restrict__ lm_grad, int B, int C,
-                                                           int blank) {
-  const int lane = threadIdx.x & (kWave - 1);
-  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (row >= B * (gv.S + 1)) return;
-  const int b = row / (gv.S + 1), s = row - b * (gv.S + 1);
-  T sx = 0, sy = 0;
-  for (int t = lane; t < gv.Tn; t += kWave) {
-    sx += gv.Gx(b, s, t);
-    sy += gv.Gy(b, s, t);
-  }
-  sx = WaveSumS(sx);
-  sy = WaveSumS(sy);
-  if (lane == 0) {
-    T *g = lm_grad + (size_t)row * C;
-    if (s < gv.S) {
-      const int64_t sym = symbols[(size_t)b * gv.S + s];
-      if (sym >= 0 && sym < C) g[sym] += sx;
+inline int SumsChunks(int Tn) { return (Tn + kSumsChunk - 1) / kSumsChunk; }
+inline int SumsGroups(int S) { return (S + kSumsGroup) / kSumsGroup; }  // of the S + 1 rows
+
+// Sums each of a lane's 2^kLog values over the wavefront.  Every step halves the values a lane
+// still carries (it hands the other half to the lane it pairs with), so the 2^kLog sums cost
+// 2^kLog - 1 + (6 - kLog) exchanges instead of 6 each.  Returns the complete sum of value
+// number (lane >> (6 - kLog)), the same in every lane that shares the number.
+template <typename T, int kLog>
+__device__ __forceinline__ T WaveSumsTransposed(T (&v)[1 << kLog], int lane) {
+  static_assert(kLog >= 1 && kLog <= 6, "");
+#pragma unroll
+  for (int step = 0; step < kLog; ++step) {
+    const int n = (1 << kLog) >> (step + 1), off = kWave >> (step + 1);
+    const bool upper = (lane & off) != 0;
+#pragma unroll
+    for (int i = 0; i < n; ++i) {
+      const T keep = upper ? v[i + n] : v[i];
+      const T send = upper ? v[i] : v[i + n];
+      v[i] = keep + __shfl_xor(send, off, kWave);
     }
-    g[blank] += sy;
   }
+  T r = v[0];
+#pragma unroll
+  for (int off = kWave >> (kLog + 1); off > 0; off >>= 1) r += __shfl_xor(r, off, kWave);
+  return r;
 }
 
-// am_grad[b,t,blank] += sum_s Gy(b,s,t).  One thread per (b,t); the reads of consecutive threads
-// are consecutive.
 template <typename T>
-__global__ void AmBlankTermKernel(GradView<T> gv, T *__restrict__ am_grad, int B, int C,
-                                  int blank) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= B * gv.Tn) return;
-  const int b = i / gv.Tn, t = i - b * gv.Tn;
-  T sy = 0;
-  int s = 0;
-  for (; s + 8 <= gv.S + 1; s += 8) {  // eight rows' loads in flight at a time
-    T v[8];
+__global__ __launch_bounds__(256) void QSumsKernel(GradView<T> gv, const T *__restrict__ denom,
+                                                   T *__restrict__ q, T *__restrict__ col_y,
+                                                   T *__restrict__ row_x, T *__restrict__ row_y,
+                                                   int chunks, int groups) {
+  __shared__ T col[4][kSumsChunk];
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+  const int chunk = blockIdx.x, group = blockIdx.y, b = blockIdx.z;
+  const int S = gv.S, Tn = gv.Tn;
+  const int t = chunk * kSumsChunk + lane;
+  const bool inside = t < Tn;
+  const int tc = min(t, Tn - 1);
+  const int s0 = group * kSumsGroup + wave * kSumsRows;
+  const bool regular = gv.rnnt_type == K2AMD_REGULAR;
+  const bool constrained = gv.rnnt_type == K2AMD_CONSTRAINED;
+  const int T1 = regular ? Tn + 1 : Tn;
+  const T scale = gv.Scale(b);
+  const bool cut = regular && gv.boundary != nullptr && gv.boundary[4 * b + 3] == t;
+  // rows s0 - 1 .. s0 + kSumsRows - 1 of px_grad (the first one only feeds a constrained lattice's
+  // Gy), rows s0 .. of py_grad and denom
+  T px_raw[kSumsRows + 1], py_raw[kSumsRows], den[kSumsRows];
 #pragma unroll
-    for (int k = 0; k < 8; ++k) v[k] = gv.Gy(b, s + k, t);
-#pragma unroll
-    for (int k = 0; k < 8; ++k) sy += v[k];
+  for (int j = 0; j <= kSumsRows; ++j) {
+    const int s = min(max(s0 + j - 1, 0), S - 1);
+    px_raw[j] = S > 0 && (j > 0 || constrained) ? gv.px_grad[((size_t)b * S + s) * T1 + tc] : T(0);
   }
-  for (; s <= gv.S; ++s) sy += gv.Gy(b, s, t);
-  am_grad[(size_t)i * C + blank] += sy;
+#pragma unroll
+  for (int j = 0; j < kSumsRows; ++j) {
+    const size_t i = ((size_t)b * (S + 1) + min(s0 + j, S)) * Tn + tc;
+    py_raw[j] = gv.py_grad[i];
+    den[j] = denom[i];
+  }
+  T sums[2 * kSumsRows];  // of row j: Gx in 2 j, Gy in 2 j + 1
+  T cy = 0;
+  T gx_below = 0;  // Gx(b, s - 1, t)
+  if (constrained && s0 >= 1 && s0 - 1 < S && inside && !cut) gx_below = MulRounded(px_raw[0], scale);
+#pragma unroll
+  for (int j = 0; j < kSumsRows; ++j) {
+    const int s = s0 + j;
+    const bool live = inside && s <= S;
+    const T gx = live && s < S && !cut ? MulRounded(px_raw[j + 1], scale) : T(0);
+    T gy = live ? MulRounded(py_raw[j], scale) : T(0);
+    if (constrained && live && s >= 1) gy += gx_below;
+    gx_below = gx;
+    if (live) q[((size_t)b * (S + 1) + s) * Tn + t] = (gx + gy) / den[j];
+    cy += gy;
+    sums[2 * j] = gx;
+    sums[2 * j + 1] = gy;
+  }
+  const T total = WaveSumsTransposed<T, 4>(sums, lane);
+  if ((lane & 3) == 0) {
+    const int which = lane >> 2, s = s0 + (which >> 1);
+    if (s <= S) ((which & 1) ? row_y : row_x)[((size_t)b * (S + 1) + s) * chunks + chunk] = total;
+  }
+  col[wave][lane] = cy;
+  __syncthreads();
+  if (wave == 0 && inside)
+    col_y[((size_t)b * groups + group) * Tn + t] =
+        (col[0][lane] + col[1][lane]) + (col[2][lane] + col[3][lane]);
 }
 
 template <typename T>
@@ -822,25 +947,27 @@ int SimpleBackward(const T *px_grad, const T *py_grad, const T *seq_scale, const
                    int rnnt_type, hipStream_t st) {
   if (B == 0) return K2AMD_OK;
   GradView<T> gv{px_grad, py_grad, seq_scale, boundary, S, Tn, rnnt_type};
-  if (Tn > 0) {
-    hipLaunchKernelGGL(QKernel<T>, dim3(512), dim3(256), 0, st, gv, denom, q, B);
-    {  // lm_grad[b][s][c] = -lm_probs * sum_t q[b][s][t] * am_probs[b][t][c]
-      ScaleEpilogue<T> epi{lm_probs, lm_grad, S + 1, C};
-      MatView av{(size_t)(S + 1) * Tn, Tn, 1};  // A(m=s, k=t) = q[b][s][t]
-      MatView bv{(size_t)Tn * C, C, 1};         // B(k=t, n=c) = am_probs[b][t][c]
-      LaunchProduct<T, true, false>((const T *)q, av, am_probs, bv, S + 1, C, Tn, B, epi, st);
-    }
-    {  // am_grad[b][t][c] = -am_probs * sum_s q[b][s][t] * lm_probs[b][s][c]
-      AmGradEpilogue<T> epi{am_probs, am_grad, gv, symbols, Tn, C};
-      MatView av{(size_t)(S + 1) * Tn, 1, Tn};   // A(m=t, k=s) = q[b][s][t]
-      MatView bv{(size_t)(S + 1) * C, C, 1};     // B(k=s, n=c) = lm_probs[b][s][c]
-      LaunchProduct<T, false, false>((const T *)q, av, lm_probs, bv, Tn, C, S + 1, B, epi, st);
-    }
-    hipLaunchKernelGGL(AmBlankTermKernel<T>, dim3((B * Tn + 255) / 256), dim3(256), 0, st, gv, am_grad, B, C, blank);
-  } else {
+  if (Tn == 0) {  // no am rows; every term of the lm gradient is an empty sum
     hipLaunchKernelGGL(ZeroKernelS<T>, dim3(256), dim3(256), 0, st, lm_grad, (size_t)B * (S + 1) * C);
+    return LaunchStatus();
   }
-  hipLaunchKernelGGL(LmGatherTermsKernel<T>, dim3((B * (S + 1) + 3) / 4), dim3(256), 0, st, gv, symbols, lm_grad, B, C, blank);
+  const int chunks = SumsChunks(Tn), groups = SumsGroups(S);
+  T *col_y = q + (size_t)B * (S + 1) * Tn;
+  T *row_x = col_y + (size_t)B * groups * Tn;
+  T *row_y = row_x + (size_t)B * (S + 1) * chunks;
+  hipLaunchKernelGGL(QSumsKernel<T>, dim3(chunks, groups, B), dim3(256), 0, st, gv, denom, q, col_y, row_x, row_y, chunks, groups);
+  {  // lm_grad[b][s][c] = -lm_probs * sum_t q[b][s][t] * am_probs[b][t][c]  (+ the gathered terms)
+    LmGradEpilogue<T> epi{lm_probs, lm_grad, symbols, row_x, row_y, S, C, chunks, blank};
+    MatView av{(size_t)(S + 1) * Tn, Tn, 1};  // A(m=s, k=t) = q[b][s][t]
+    MatView bv{(size_t)Tn * C, C, 1};         // B(k=t, n=c) = am_probs[b][t][c]
+    LaunchProduct<T, true, false>((const T *)q, av, am_probs, bv, S + 1, C, Tn, B, epi, st);
+  }
+  {  // am_grad[b][t][c] = -am_probs * sum_s q[b][s][t] * lm_probs[b][s][c]  (+ symbol and blank terms)
+    AmGradEpilogue<T> epi{am_probs, am_grad, gv, symbols, col_y, Tn, C, blank, groups};
+    MatView av{(size_t)(S + 1) * Tn, 1, Tn};   // A(m=t, k=s) = q[b][s][t]
+    MatView bv{(size_t)(S + 1) * C, C, 1};     // B(k=s, n=c) = lm_probs[b][s][c]
+    LaunchProduct<T, false, false>((const T *)q, av, lm_probs, bv, Tn, C, S + 1, B, epi, st);
+  }
   return LaunchStatus();
 }
 

@@ -176,9 +176,10 @@ class _Scores(torch.autograd.Function):
         if ctx.reduction == "none":
             scale = loss_grad.neg()
         else:
-            # (a division for the mean, as torch's own backward of it: the same bits)
-            scale = loss_grad.neg() if ctx.reduction == "sum" else loss_grad / float(-ctx.batch)
-            scale = scale.expand(ctx.batch).contiguous()
+            # (a division for the mean, as torch's own backward of it: the same bits; the op on the
+            # expanded scalar writes the [B] tensor in one launch)
+            scale = loss_grad.expand(ctx.batch)
+            scale = (scale.neg() if ctx.reduction == "sum" else scale / float(-ctx.batch)).contiguous()
         if ctx.kind == "simple":
             _, _, symbols, termination_symbol, rnnt_code, boundary = args
             grads = native.logprobs_simple_backward(px_grad, py_grad, symbols, boundary, saved,
