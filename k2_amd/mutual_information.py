@@ -28,10 +28,40 @@ def boundary_rows(boundary: Tensor) -> Tuple[Tuple[int, int, int, int], ...]:
     hit = _boundary_copies.get(ident)
     if hit is not None and hit[0]() is boundary and hit[1] == boundary._version:
         return hit[2]
-    rows = tuple(tuple(r) for r in boundary.tolist())
+    early = _boundary_reads.pop(ident, None)
+    if early is not None and early[0]() is boundary and early[1] == boundary._version:
+        early[3].synchronize()  # the copy alone, not what was queued after it
+        rows = tuple(tuple(r) for r in early[2].tolist())
+    else:
+        rows = tuple(tuple(r) for r in boundary.tolist())
     _boundary_copies[ident] = (weakref.ref(boundary, lambda _, i=ident: _boundary_copies.pop(i, None)),
                                boundary._version, rows)
     return rows
+
+
+# copies to the host under way: id(tensor) -> (weak reference, version counter, pinned tensor, event)
+_boundary_reads = {}
+
+
+def begin_boundary_read(boundary: Optional[Tensor]) -> None:
+    """Starts the copy that boundary_rows needs, without waiting for it: a loss function calls this
+    before it queues the kernels that do not depend on the boundary's values being valid, so that
+    the checks after them (k2/python/k2/mutual_information.py:284-289, which the reference reaches
+    after get_rnnt_logprobs' kernels too, k2/python/k2/rnnt_loss.py:295-330) find the rows on the
+    host instead of waiting for those kernels and leaving the device idle meanwhile.  Nothing to do
+    for a tensor whose rows are already here, and for host tensors."""
+    if boundary is None or not boundary.is_cuda:
+        return
+    ident = id(boundary)
+    hit = _boundary_copies.get(ident)
+    if hit is not None and hit[0]() is boundary and hit[1] == boundary._version:
+        return
+    pinned = torch.empty(boundary.shape, dtype=boundary.dtype, pin_memory=True)
+    pinned.copy_(boundary, non_blocking=True)
+    event = torch.cuda.Event()
+    event.record(torch.cuda.current_stream(boundary.device))
+    _boundary_reads[ident] = (weakref.ref(boundary, lambda _, i=ident: _boundary_reads.pop(i, None)),
+                              boundary._version, pinned, event)
 
 
 def _check_boundary(boundary: Tensor, S: int, T: int) -> None:

@@ -11,8 +11,8 @@ import torch
 from torch import Tensor
 
 from . import capi, native
-from .mutual_information import (boundary_rows, check_recursion_inputs, mutual_information_recursion,
-                                 recursion_values)
+from .mutual_information import (begin_boundary_read, boundary_rows, check_recursion_inputs,
+                                 mutual_information_recursion, recursion_values)
 
 _RNNT_TYPES = ("regular", "modified", "constrained")
 
@@ -129,6 +129,7 @@ class _Scores(torch.autograd.Function):
             raise ValueError(f"reduction should be ('none' | 'mean' | 'sum'), given {reduction}")
         boundary = {"joint": 4, "joiner": 8}.get(kind, 5)
         boundary = args[boundary]
+        begin_boundary_read(boundary)  # for check_recursion_inputs below, behind the builder's kernels
         need = return_grad or any(ctx.needs_input_grad)
         # no zero tensors for the gradients of px_grad / py_grad, which nothing differentiates
         ctx.set_materialize_grads(False)

@@ -1,5 +1,5 @@
-"""Host-side checks of the Python layer that need no GPU: the shared host copy of a boundary
-tensor and the integer arithmetic of the s_range adjustment."""
+"""Host-side checks of the Python layer: the shared host copy of a boundary tensor (its early,
+non-blocking read needs a device) and the integer arithmetic of the s_range adjustment."""
 import gc
 import importlib
 
@@ -25,6 +25,41 @@ def test_boundary_rows_are_read_once_per_tensor_version():
     del other
     gc.collect()
     assert key not in kmi._boundary_copies                  # the copy goes with its tensor
+
+
+def test_an_early_read_is_for_host_tensors_a_no_op():
+    bd = torch.tensor([[0, 0, 3, 7]], dtype=torch.int64)
+    kmi.begin_boundary_read(bd)
+    kmi.begin_boundary_read(None)
+    assert id(bd) not in kmi._boundary_reads
+    assert kmi.boundary_rows(bd) == ((0, 0, 3, 7),)
+
+
+@pytest.mark.gpu
+def test_an_early_read_of_a_device_boundary_gives_the_same_rows(device):
+    """begin_boundary_read starts the copy, boundary_rows waits for it alone; a tensor written in
+    between is read again, and rows already on the host are not asked for twice."""
+    want = ((0, 0, 3, 7), (1, 2, 4, 9))
+    bd = torch.tensor(want, dtype=torch.int64, device=device)
+    kmi.begin_boundary_read(bd)
+    assert id(bd) in kmi._boundary_reads
+    big = torch.randn(4096, 4096, device=device)
+    for _ in range(4):                                      # work queued behind the copy
+        big = big @ big * 1e-3
+    assert kmi.boundary_rows(bd) == want
+    assert id(bd) not in kmi._boundary_reads
+    kmi.begin_boundary_read(bd)                             # the rows are here already
+    assert id(bd) not in kmi._boundary_reads
+    other = bd.clone()
+    kmi.begin_boundary_read(other)
+    other[0, 2] = 2                                         # written after the copy was queued
+    assert kmi.boundary_rows(other) == ((0, 0, 2, 7), (1, 2, 4, 9))
+    third = bd.clone()
+    kmi.begin_boundary_read(third)
+    key = id(third)
+    del third
+    gc.collect()
+    assert key not in kmi._boundary_reads                   # a read nobody asked the rows of
 
 
 def test_range_asserts_follow_the_reference():
