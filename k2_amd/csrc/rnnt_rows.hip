@@ -312,8 +312,10 @@ template <typename T, bool kHat>
 __global__ __launch_bounds__(kRowsPerBlock *kWave) void RowGradKernel(
     const T *__restrict__ logits, T *__restrict__ logits_grad, long long rows, int C, int blank) {
   const int lane = threadIdx.x & (kWave - 1);
-  const long long row = (long long)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
-  if (row >= rows) return;
+  // Last row first: the forward pass read the rows in ascending order, so of a tensor larger than
+  // the 256 MB memory-side cache it is the tail that is still there.
+  const long long row = rows - 1 - ((long long)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6));
+  if (row < 0) return;
   const T *x = logits + (size_t)row * C;
   T *dx = logits_grad + (size_t)row * C;
   typedef typename Vec16<T>::type V;
