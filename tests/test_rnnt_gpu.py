@@ -501,8 +501,8 @@ def test_logprobs_simple_fp32_products_vs_fp64(device, rnnt_type):
     rng = np.random.default_rng(91)
     shapes = ((3, 37, 9, 50),        # small, rows not a multiple of four: split-K kernel, scalar loads
               (2, 70, 66, 132),      # split-K kernel, 16-byte loads, K = 132 = 8 x 16 + 4
-              (16, 250, 50, 500),    # config 2: the am gradient takes the LDS kernel
-              (64, 203, 70, 130),    # LDS kernel everywhere, scalar loads, ragged in every axis
+              (16, 250, 50, 500),    # config 2: split-K kernel everywhere (the am gradient's K is short)
+              (96, 203, 70, 130),    # LDS kernel everywhere, scalar loads, ragged in every axis
               (32, 500, 100, 500))   # config 3: LDS kernel, 16-byte loads
     for (B, T, S, C) in shapes:
         c = cases.rnnt_case(B + T, B, T, S, C, t_lo=max(T // 2, S), s_lo=S // 2, modified=rnnt_type != "regular")
@@ -725,6 +725,30 @@ def test_config2_network_gradients_full_size(device):
         np.testing.assert_allclose(got, own[k], rtol=1e-4, atol=1e-5, err_msg="c2 " + name)
         # signed sums of ~100 occupation probabilities: the arbitration's percentile is absolute
         three_way("c2 " + name, got, f32[k], f64[k], mode="absolute")
+
+
+@pytest.mark.parametrize("few_symbols", [False, True])
+def test_simple_gradients_where_the_am_gradient_takes_the_larger_tiles(device, few_symbols):
+    """B=32, T=250, S=33, V=500: 1024 tiles of 64 x 64 in the am gradient, the fewest with which
+    its product of K = S + 1 = 34 takes the LDS kernel (sixteen elements per thread in the
+    epilogue's load rounds, ragged tiles in T and V, two groups of rows in the blank column's
+    sums).  With the symbols as drawn (a column lists 0-3 positions) and with two classes only
+    (every list overflows: the rescanning path).  lm.grad / am.grad against the fp64 closed form
+    (tests/closed_forms.py) on the occupation probabilities that the GPU itself returned."""
+    import k2_amd as k2
+    B, T, S, C = 32, 250, 33, 500
+    c = cases.rnnt_case(77, B, T, S, C, t_lo=150, s_lo=20)
+    symbols = 1 + c["symbols"] % 2 if few_symbols else c["symbols"]
+    w = np.linspace(0.5, 1.5, B).astype(np.float32)
+    lm = dev(c["lm"], device).requires_grad_(True)
+    am = dev(c["am"], device).requires_grad_(True)
+    loss, (gx, gy) = k2.rnnt_loss_simple(lm, am, dev(symbols, device), 0, dev(c["boundary"], device),
+                                         reduction="none", return_grad=True)
+    (loss * dev(w, device)).sum().backward()
+    gx, gy = gx.cpu().numpy(), gy.cpu().numpy()
+    (want,) = cf.simple_grads(c["lm"], c["am"], symbols, 0, (gx,), (gy,), w)
+    for name, got, k in (("lm.grad", lm.grad.cpu().numpy(), 0), ("am.grad", am.grad.cpu().numpy(), 1)):
+        np.testing.assert_allclose(got, want[k], rtol=1e-4, atol=1e-5, err_msg=name)
 
 
 def test_config3_logits_gradient_full_size(device):
