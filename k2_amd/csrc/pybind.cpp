@@ -13,6 +13,7 @@
 // PyTorch-ROCm names its HIP devices "cuda"; these are the guard and stream types that go with it
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <ATen/hip/HIPEvent.h>
 
 #include <algorithm>
 #include <map>
@@ -647,8 +648,44 @@ std::vector<torch::Tensor> PrunedRangesToLattice(torch::Tensor ranges, torch::Te
 
 }  // namespace
 
+// The rows of a [B][4] boundary tensor on their way to the host: a non-blocking copy into pinned
+// memory on the tensor's current stream and an event behind it.  Rows() waits for that event
+// alone (not for what was queued after the copy) and returns the rows as tuples of Python
+// integers, what k2's range asserts read (k2/python/k2/mutual_information.py:284-289).
+class BoundaryRead {
+ public:
+  explicit BoundaryRead(const torch::Tensor &boundary) {
+    TORCH_CHECK(boundary.is_cuda() && boundary.dim() == 2 && boundary.size(1) == 4 &&
+                    boundary.scalar_type() == torch::kLong,
+                "boundary must be a [B][4] int64 tensor on the device");
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(boundary.device());
+    pinned_ = torch::empty(boundary.sizes(), torch::TensorOptions().dtype(torch::kLong).pinned_memory(true));
+    pinned_.copy_(boundary, /*non_blocking=*/true);
+    event_.record(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(boundary.device().index()));
+  }
+  pybind11::tuple Rows() {
+    {
+      pybind11::gil_scoped_release release;
+      event_.synchronize();
+    }
+    const int64_t B = pinned_.size(0);
+    const int64_t *v = pinned_.data_ptr<int64_t>();
+    pybind11::tuple rows(B);
+    for (int64_t b = 0; b < B; ++b)
+      rows[b] = pybind11::make_tuple(v[4 * b], v[4 * b + 1], v[4 * b + 2], v[4 * b + 3]);
+    return rows;
+  }
+
+ private:
+  torch::Tensor pinned_;
+  at::cuda::CUDAEvent event_;
+};
+
 PYBIND11_MODULE(_k2_amd, m) {
   m.doc() = "MI355X host layer of the k2 mutual-information recursion";
+  pybind11::class_<BoundaryRead>(m, "BoundaryRead")
+      .def(pybind11::init<const torch::Tensor &>(), pybind11::arg("boundary"))
+      .def("rows", &BoundaryRead::Rows);
   m.def("mutual_information_forward", &MutualInformationForward, pybind11::arg("px"),
         pybind11::arg("py"), pybind11::arg("boundary"), pybind11::arg("p"),
         pybind11::arg("log_deriv") = pybind11::none());

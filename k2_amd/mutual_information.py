@@ -30,8 +30,7 @@ def boundary_rows(boundary: Tensor) -> Tuple[Tuple[int, int, int, int], ...]:
         return hit[2]
     early = _boundary_reads.pop(ident, None)
     if early is not None and early[0]() is boundary and early[1] == boundary._version:
-        early[3].synchronize()  # the copy alone, not what was queued after it
-        rows = tuple(tuple(r) for r in early[2].tolist())
+        rows = early[2].rows()  # waits for the copy alone, not for what was queued after it
     else:
         rows = tuple(tuple(r) for r in boundary.tolist())
     _boundary_copies[ident] = (weakref.ref(boundary, lambda _, i=ident: _boundary_copies.pop(i, None)),
@@ -39,13 +38,14 @@ def boundary_rows(boundary: Tensor) -> Tuple[Tuple[int, int, int, int], ...]:
     return rows
 
 
-# copies to the host under way: id(tensor) -> (weak reference, version counter, pinned tensor, event)
+# copies to the host under way: id(tensor) -> (weak reference, version counter, native.boundary_read)
 _boundary_reads = {}
 
 
 def begin_boundary_read(boundary: Optional[Tensor]) -> None:
     """Starts the copy that boundary_rows needs, without waiting for it: a loss function calls this
-    before it queues the kernels that do not depend on the boundary's values being valid, so that
+    before it queues the kernels that do not depend on the boundary's values being valid (a
+    non-blocking copy into pinned memory and an event behind it), so that
     the checks after them (k2/python/k2/mutual_information.py:284-289, which the reference reaches
     after get_rnnt_logprobs' kernels too, k2/python/k2/rnnt_loss.py:295-330) find the rows on the
     host instead of waiting for those kernels and leaving the device idle meanwhile.  Nothing to do
@@ -56,12 +56,8 @@ def begin_boundary_read(boundary: Optional[Tensor]) -> None:
     hit = _boundary_copies.get(ident)
     if hit is not None and hit[0]() is boundary and hit[1] == boundary._version:
         return
-    pinned = torch.empty(boundary.shape, dtype=boundary.dtype, pin_memory=True)
-    pinned.copy_(boundary, non_blocking=True)
-    event = torch.cuda.Event()
-    event.record(torch.cuda.current_stream(boundary.device))
     _boundary_reads[ident] = (weakref.ref(boundary, lambda _, i=ident: _boundary_reads.pop(i, None)),
-                              boundary._version, pinned, event)
+                              boundary._version, native.boundary_read(boundary))
 
 
 def _check_boundary(boundary: Tensor, S: int, T: int) -> None:

@@ -22,6 +22,29 @@ def _require_device(t: torch.Tensor):
             "k2_amd runs on MI355X only: got a tensor on %s (there is no CPU path)" % t.device)
 
 
+class _BoundaryRead:
+    """The host layer's BoundaryRead with torch's Python API, where the extension is not built."""
+
+    def __init__(self, boundary: torch.Tensor):
+        self.pinned = torch.empty(boundary.shape, dtype=boundary.dtype, pin_memory=True)
+        self.pinned.copy_(boundary, non_blocking=True)
+        self.event = torch.cuda.Event()
+        self.event.record(torch.cuda.current_stream(boundary.device))
+
+    def rows(self):
+        self.event.synchronize()  # the copy alone, not what was queued after it
+        return tuple(tuple(r) for r in self.pinned.tolist())
+
+
+def boundary_read(boundary: torch.Tensor):
+    """Starts the copy of a [B][4] int64 device tensor to the host without waiting for it;
+    ``.rows()`` of the returned object waits for that copy alone and gives the rows as tuples of
+    Python integers."""
+    if _ext is not None and boundary.dtype == torch.int64 and boundary.dim() == 2 and boundary.shape[1] == 4:
+        return _ext.BoundaryRead(boundary)
+    return _BoundaryRead(boundary)
+
+
 def mutual_information_recover_workspaces() -> int:
     """Waits for the streams that the pipelined fp32 kernels have run on and reads the error flag
     of each scratch buffer.  Where a kernel gave up a bounded wait (its scores came out as NaN,
