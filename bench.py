@@ -315,6 +315,93 @@ def other_configs(dev, steps=50):
     return out
 
 
+def next_rows(dev, steps=30):
+    """The rows either side of the path that the library also serves, each once at a BASELINE shape:
+    pruned_ranges_to_lattice and the HAT pruned loss on config 3's shape, the smoothed loss on
+    config 2's, joint_mutual_information_recursion (two px / py pairs) on config 4's.  HIP-event
+    time per call through the k2-style API (forward + backward for the losses, a fresh boundary
+    tensor per step as in the other secondary figures), with the bytes each has to move at least."""
+    import torch
+    import cases
+    import k2_amd as k2
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps * 1e-3
+
+    def entry(workload, t, nbytes, what):
+        return {"workload": workload, "ms_per_call": t * 1e3, "algorithmic_bytes": int(nbytes),
+                "bytes_counted": what, "GBps": nbytes / t / 1e9, "frac_of_hbm_peak": nbytes / t / 1e9 / HBM_PEAK_GBS}
+
+    out = {}
+    B, T, S, C, R = 32, 500, 100, 500, 5
+    c = cases.rnnt_case(3, B, T, S, C, t_lo=300, s_lo=50)
+    lm, am = torch.from_numpy(c["lm"]).to(dev), torch.from_numpy(c["am"]).to(dev)
+    sym, bd = torch.from_numpy(c["symbols"]).to(dev), torch.from_numpy(c["boundary"]).to(dev)
+    _, (gx, gy) = k2.rnnt_loss_simple(lm, am, sym, 0, bd, reduction="sum", return_grad=True)
+    ranges = k2.get_rnnt_prune_ranges(gx, gy, bd, R)
+    del lm, am, gx, gy
+    logits = torch.from_numpy(
+        np.random.default_rng(33).standard_normal((B, T, R, C)).astype(np.float32)).to(dev)
+    ranges32, frames = ranges.to(torch.int32), bd[:, 3].to(torch.int32).contiguous()
+    lattice, arc_map = k2.pruned_ranges_to_lattice(ranges32, frames, sym, logits)
+    arcs = int(arc_map.numel())
+    t = timed(lambda: k2.pruned_ranges_to_lattice(ranges32, frames, sym, logits))
+    out["pruned_ranges_to_lattice"] = entry(
+        f"pruned_ranges_to_lattice, fp32 logits, B={B} T={T} S={S} V={C} s_range={R} (config 3's shape): "
+        f"{arcs} arcs; two host reads of the counts per call, as in the reference", t,
+        arcs * (16 + 4 + 4) + ranges32.numel() * 4,
+        "arc records 16 B + arc_map 4 B written and one logit read per arc, ranges read once")
+
+    logits.requires_grad_(True)
+
+    def hat():
+        logits.grad = None
+        k2.rnnt_loss_pruned(logits, sym, ranges, 0, bd.clone(), reduction="sum", use_hat_loss=True).backward()
+
+    out["hat_pruned_loss"] = entry(
+        f"rnnt_loss_pruned(use_hat_loss=True) fwd+bwd, fp32, regular, B={B} T={T} S={S} V={C} s_range={R}",
+        timed(hat), 3 * logits.numel() * 4, "logits read forward, read + gradient written backward")
+    del logits
+
+    B, T, S, C = 16, 250, 50, 500
+    c = cases.rnnt_case(2, B, T, S, C, t_lo=150, s_lo=20)
+    lm = torch.from_numpy(c["lm"]).to(dev).requires_grad_(True)
+    am = torch.from_numpy(c["am"]).to(dev).requires_grad_(True)
+    sym, bd = torch.from_numpy(c["symbols"]).to(dev), torch.from_numpy(c["boundary"]).to(dev)
+
+    def smoothed():
+        lm.grad = None
+        am.grad = None
+        k2.rnnt_loss_smoothed(lm, am, sym, 0, lm_only_scale=0.25, am_only_scale=0.1, boundary=bd.clone(),
+                              reduction="sum").backward()
+
+    out["smoothed_loss"] = entry(
+        f"rnnt_loss_smoothed fwd+bwd, fp32, regular, B={B} T={T} S={S} V={C} (config 2's shape)",
+        timed(smoothed), 2 * 4 * (lm.numel() + am.numel()), "lm, am read forward; their gradients written backward")
+    del lm, am
+
+    B, S, T = 32, 200, 1000
+    c = cases.c4_case(B=B, S=S, T=T)
+    px, py, bd = (torch.from_numpy(c[k]).to(dev) for k in ("px", "py", "boundary"))
+    pxs, pys = (px * 0.75, px * 0.25), (py * 0.75, py * 0.25)
+    t = timed(lambda: k2.joint_mutual_information_recursion(pxs, pys, bd))
+    out["joint_mutual_information_recursion"] = entry(
+        f"joint_mutual_information_recursion, two px / py pairs, fp32, modified, B={B} S={S} T={T} (config 4's shape)",
+        t, 4 * (2 + 1 + 1 + 2) * (px.numel() + py.numel()),
+        "the pairs read and their sum written, the sum read by the recursion, the occupation "
+        "probabilities written, then read with the pairs for the inner products (full box)")
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -501,6 +588,7 @@ def main():
         out["secondary"] = pruned_secondary(dev, cpu=not args.no_cpu)
         out["other_configs"] = other_configs(dev)
         out["fused_joiner"] = fused_joiner(dev)
+        out["next_rows"] = next_rows(dev)
     print(json.dumps(out))
 
 
