@@ -186,10 +186,12 @@ K2AMD_API int k2amd_rnnt_logprobs_simple_forward(
     int T, int C, int termination_symbol, int rnnt_type, int dtype, void *stream);
 
 /* Gradient of the above w.r.t. lm and am (what torch autograd derives from
- * k2/python/k2/rnnt_loss.py:172-223).  q_scratch is scratch of
- * B * ((S+1) * T + ceil((S+1) / 32) * T + 2 * (S+1) * ceil(T / 64)) elements: the [B][S+1][T]
- * operand of the two products, then the gradients' sums along s ([B][T] per 32 rows) and along t
- * ([B][S+1] per 64 frames, for px_grad and for py_grad).                                         */
+ * k2/python/k2/rnnt_loss.py:172-223).  q_scratch is device scratch of
+ * k2amd_rnnt_logprobs_simple_backward_scratch_elements(B, S, T) elements of the tensors' type
+ * (= B * ((S+1) * T + ceil((S+1) / 32) * T + 2 * (S+1) * ceil(T / 64)): the [B][S+1][T] operand
+ * of the two products, then the gradients' sums along s ([B][T] per 32 rows) and along t
+ * ([B][S+1] per 64 frames, for px_grad and for py_grad)).                                        */
+K2AMD_API size_t k2amd_rnnt_logprobs_simple_backward_scratch_elements(int B, int S, int T);
 K2AMD_API int k2amd_rnnt_logprobs_simple_backward(
     const void *px_grad, const void *py_grad, const void *seq_scale, const int64_t *symbols,
     const int64_t *boundary,

@@ -41,6 +41,7 @@ _SIGNATURES = {
     "k2amd_mi_forward_backward": ([_vp] * 5 + [_sz] + [_vp] * 3 + [_ci] * 6 + [_vp, _sz, _vp], _ci),
     "k2amd_rnnt_logprobs_simple_forward": ([_vp] * 11 + [_ci] * 7 + [_vp], _ci),
     "k2amd_rnnt_logprobs_simple_backward": ([_vp] * 11 + [_ci] * 7 + [_vp], _ci),
+    "k2amd_rnnt_logprobs_simple_backward_scratch_elements": ([_ci] * 3, ctypes.c_size_t),
     "k2amd_rnnt_logprobs_joint_forward": ([_vp] * 6 + [_ci] * 7 + [_vp], _ci),
     "k2amd_rnnt_logprobs_joint_backward": ([_vp] * 8 + [_ci] * 7 + [_vp], _ci),
     "k2amd_rnnt_logprobs_pruned_forward": ([_vp] * 7 + [_ci] * 8 + [_vp], _ci),
@@ -363,10 +364,8 @@ def logprobs_simple_backward(px_grad, py_grad, symbols, boundary, saved, termina
     _symbol(termination_symbol, C)
     lm_grad = torch.empty_like(lm_probs)
     am_grad = torch.empty_like(am_probs)
-    # the products' operand [B][S+1][T], then the gradients' sums along s (per 32 rows) and along t
-    # (per 64 frames)
-    rows = B * (S + 1)
-    q = torch.empty(rows * T + B * ((S + 32) // 32) * T + 2 * rows * ((T + 63) // 64), dtype=dt, device=dev)
+    # the products' operand [B][S+1][T], then the gradients' sums along s and along t
+    q = torch.empty(lib().k2amd_rnnt_logprobs_simple_backward_scratch_elements(B, S, T), dtype=dt, device=dev)
     dev = am_probs.device
     with torch.cuda.device(dev):
         check(lib().k2amd_rnnt_logprobs_simple_backward(

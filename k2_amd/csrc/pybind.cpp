@@ -403,11 +403,9 @@ std::vector<torch::Tensor> LogprobsSimpleBackward(torch::Tensor px_grad, torch::
   const void *scale = ScalePtr(seq_scale, px_grad);
   c10::hip::HIPGuardMasqueradingAsCUDA guard(am_probs.device());
   torch::Tensor lm_grad = torch::empty_like(lm_probs), am_grad = torch::empty_like(am_probs);
-  // the products' operand [B][S+1][T], then the gradients' sums along s (per 32 rows) and along t
-  // (per 64 frames)
-  const int64_t rows = (int64_t)B * (S + 1);
+  // the products' operand [B][S+1][T], then the gradients' sums along s and along t
   torch::Tensor q = torch::empty(
-      {rows * T + (int64_t)B * ((S + 32) / 32) * T + 2 * rows * ((T + 63) / 64)}, denom.options());
+      {static_cast<int64_t>(k2amd_rnnt_logprobs_simple_backward_scratch_elements(B, S, T))}, denom.options());
   void *stream = StreamOf(am_probs);
   {
     pybind11::gil_scoped_release release;

@@ -1002,6 +1002,12 @@ int k2amd_rnnt_logprobs_simple_forward(const void *lm, const void *am, const int
   return SimpleForward<double>((const double *)lm, (const double *)am, symbols, boundary, (double *)px, (double *)py, (double *)lm_probs, (double *)am_probs, (double *)lm_max, (double *)am_max, (double *)denom, B, S, T, C, termination_symbol, rnnt_type, st);
 }
 
+size_t k2amd_rnnt_logprobs_simple_backward_scratch_elements(int B, int S, int T) {
+  if (B <= 0 || S < 0 || T <= 0) return 0;
+  const size_t rows = (size_t)B * (S + 1);
+  return rows * T + (size_t)B * SumsGroups(S) * T + 2 * rows * SumsChunks(T);
+}
+
 int k2amd_rnnt_logprobs_simple_backward(const void *px_grad, const void *py_grad,
                                         const void *seq_scale, const int64_t *symbols, const int64_t *boundary,
                                         const void *lm_probs, const void *am_probs,
