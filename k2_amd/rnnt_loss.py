@@ -546,7 +546,7 @@ def get_rnnt_logprobs_smoothed(
     against a unigram lm averaged over the batch).
 
     Not on the accelerated path's critical list: the joint part (the only one of size
-    [B][S+1][T] x C) is the fused kernel of get_rnnt_logprobs; the two marginal parts are a few
+    [B][S+1][T] x C) is the fused kernel of get_rnnt_logprobs; the two marginal parts are a dozen
     torch ops on the device over [B][S+1][C] and [B][T][C]."""
     assert lm.ndim == 3, lm.shape
     assert am.ndim == 3, am.shape
@@ -565,35 +565,31 @@ def get_rnnt_logprobs_smoothed(
     px, py = _LogprobsSimple.apply(lm, am, symbols, blank,
                                    capi.RNNT_TYPES["regular" if regular else "modified"], None)
 
+    # The two marginal parts in probability space, as the reference defines them
+    # (k2/python/k2/rnnt_loss.py:1608-1677), written with log_softmax (one kernel forward, one
+    # backward) where the reference spells the max, the exponentials, their sum and its log out:
+    #   lm only:  log softmax(lm)                                     [B][S+1][C]
+    #   am only:  log softmax(am + log unigram), unigram = the batch's mean of softmax(lm) + tiny
+    # (its normaliser log sum_c e^am unigram_c is exactly that log-softmax's).
     tiny = torch.finfo(lm.dtype).tiny
-    am_top = am.amax(dim=2, keepdim=True)                        # [B][T][1]
-    lm_top = lm.amax(dim=2, keepdim=True)                        # [B][S+1][1]
-    am_lin = (am - am_top).exp()
-    lm_lin = (lm - lm_top).exp()
-    lm_mass = lm_lin.sum(dim=2, keepdim=True)                    # [B][S+1][1]
-    unigram = (lm_lin / lm_mass).mean(dim=(0, 1)) + tiny         # [C]
-    am_only_norm = (torch.mv(am_lin.reshape(-1, C), unigram).reshape(B, 1, T).log()
-                    + am_top.transpose(1, 2))                    # [B][1][T]
-    log_unigram = unigram.log()
-    lm_only_norm = lm_mass.log() + lm_top                        # [B][S+1][1]
+    lm_only = torch.log_softmax(lm, dim=2)                                   # [B][S+1][C]
+    log_unigram = (lm_only.exp().mean(dim=(0, 1)) + tiny).log()              # [C]
+    am_only = torch.log_softmax(am + log_unigram, dim=2)                     # [B][T][C]
 
-    sym_am = torch.gather(am.transpose(1, 2), 1, symbols.unsqueeze(2).expand(B, S, T))  # [B][S][T]
-    sym_lm = torch.gather(lm[:, :S], 2, symbols.unsqueeze(2))                           # [B][S][1]
-    px_am_only = sym_am + log_unigram[symbols].unsqueeze(2) - am_only_norm
+    px_am_only = torch.gather(am_only.transpose(1, 2), 1, symbols.unsqueeze(2).expand(B, S, T))  # [B][S][T]
     if regular:  # no symbol can be emitted one past the last frame
         px_am_only = torch.nn.functional.pad(px_am_only, (0, 1), value=float("-inf"))
-    px_lm_only = sym_lm - lm_only_norm[:, :S]
-
-    blank_am = am[:, :, blank].unsqueeze(1)                      # [B][1][T]
-    blank_lm = lm[:, :, blank].unsqueeze(2)                      # [B][S+1][1]
-    py_am_only = blank_am + log_unigram[blank] - am_only_norm
-    py_lm_only = blank_lm - lm_only_norm
+    px_lm_only = torch.gather(lm_only[:, :S], 2, symbols.unsqueeze(2))       # [B][S][1]
+    py_am_only = am_only[:, :, blank].unsqueeze(1)                           # [B][1][T]
+    py_lm_only = lm_only[:, :, blank].unsqueeze(2)                           # [B][S+1][1]
 
     joint_scale = 1.0 - lm_only_scale - am_only_scale
     lm_only_scale = 1.0e-20 if lm_only_scale == 0.0 else lm_only_scale
     am_only_scale = 1.0e-20 if am_only_scale == 0.0 else am_only_scale
-    px_mix = px * joint_scale + px_lm_only * lm_only_scale + px_am_only * am_only_scale
-    py_mix = py * joint_scale + py_lm_only * lm_only_scale + py_am_only * am_only_scale
+    px_mix = torch.add(torch.add(px * joint_scale, px_lm_only, alpha=lm_only_scale), px_am_only,
+                       alpha=am_only_scale)
+    py_mix = torch.add(torch.add(py * joint_scale, py_lm_only, alpha=lm_only_scale), py_am_only,
+                       alpha=am_only_scale)
 
     if regular:
         px_mix = fix_for_boundary(px_mix, _dev_i64(boundary, px_mix))
