@@ -357,7 +357,7 @@ def next_rows(dev, steps=30):
     t = timed(lambda: k2.pruned_ranges_to_lattice(ranges32, frames, sym, logits))
     out["pruned_ranges_to_lattice"] = entry(
         f"pruned_ranges_to_lattice, fp32 logits, B={B} T={T} S={S} V={C} s_range={R} (config 3's shape): "
-        f"{arcs} arcs; two host reads of the counts per call, as in the reference", t,
+        f"{arcs} arcs; one host read of the two counts per call", t,
         arcs * (16 + 4 + 4) + ranges32.numel() * 4,
         "arc records 16 B + arc_map 4 B written and one logit read per arc, ranges read once")
 

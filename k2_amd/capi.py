@@ -606,15 +606,15 @@ def pruned_ranges_to_lattice(ranges, frames, symbols, logits):
     i32 = dict(dtype=torch.int32, device=dev)
     arc_local = torch.empty(B, T * R + 1, **i32)
     seq_arcs = torch.empty(max(B, 1), **i32)
-    state_splits = torch.empty(B + 1, **i32)
-    arc_base = torch.empty(B + 1, **i32)
+    splits = torch.empty(2, B + 1, **i32)  # one buffer: the two totals come to the host in one copy
+    state_splits, arc_base = splits[0], splits[1]
     code = {torch.float32: F32, torch.float64: F64, torch.float16: F16}.get(logits.dtype)
     if code is None:
         raise RuntimeError(f"k2_amd: unsupported logits dtype {logits.dtype}")
     with torch.cuda.device(dev):
         check(lib().k2amd_lattice_count(ptr(ranges), ptr(frames), ptr(arc_local), ptr(seq_arcs),
                                         ptr(state_splits), ptr(arc_base), B, T, R, stream_ptr(dev)))
-        n_states, n_arcs = int(state_splits[B]), int(arc_base[B])  # the one host read, as in k2
+        n_states, n_arcs = splits[:, B].tolist()  # the one host read, as in k2
         arc_splits = torch.empty(n_states + 1, **i32)
         arcs = torch.empty(n_arcs, 4, **i32)
         arc_map = torch.empty(n_arcs, **i32)

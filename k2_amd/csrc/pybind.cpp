@@ -625,14 +625,17 @@ std::vector<torch::Tensor> PrunedRangesToLattice(torch::Tensor ranges, torch::Te
   c10::hip::HIPGuardMasqueradingAsCUDA guard(ranges.device());
   auto i32 = ranges.options();
   torch::Tensor arc_local = torch::empty({B, T * R + 1}, i32), seq_arcs = torch::empty({std::max(B, 1)}, i32);
-  torch::Tensor state_splits = torch::empty({B + 1}, i32), arc_base = torch::empty({B + 1}, i32);
+  // (one buffer for the two prefix sums: their totals then come to the host in one copy)
+  torch::Tensor splits = torch::empty({2, B + 1}, i32);
+  torch::Tensor state_splits = splits[0], arc_base = splits[1];
   void *stream = StreamOf(ranges);
   Check(k2amd_lattice_count(ranges.data_ptr<int32_t>(), frames.data_ptr<int32_t>(),
                             arc_local.data_ptr<int32_t>(), seq_arcs.data_ptr<int32_t>(),
                             state_splits.data_ptr<int32_t>(), arc_base.data_ptr<int32_t>(), B, T, R,
                             stream));
   // the one host read on this path (the reference reads the same totals to size its arrays)
-  const int n_states = state_splits[B].item<int32_t>(), n_arcs = arc_base[B].item<int32_t>();
+  const torch::Tensor totals = splits.select(1, B).cpu();
+  const int n_states = totals[0].item<int32_t>(), n_arcs = totals[1].item<int32_t>();
   torch::Tensor arc_splits = B > 0 ? torch::empty({n_states + 1}, i32) : torch::zeros({1}, i32);
   torch::Tensor arcs = torch::empty({n_arcs, 4}, i32), arc_map = torch::empty({n_arcs}, i32);
   const int64_t strides[4] = {logits.stride(0), logits.stride(1), logits.stride(2), logits.stride(3)};
