@@ -396,9 +396,9 @@ def next_rows(dev, steps=30):
     t = timed(lambda: k2.joint_mutual_information_recursion(pxs, pys, bd))
     out["joint_mutual_information_recursion"] = entry(
         f"joint_mutual_information_recursion, two px / py pairs, fp32, modified, B={B} S={S} T={T} (config 4's shape)",
-        t, 4 * (2 + 1 + 1 + 2) * (px.numel() + py.numel()),
-        "the pairs read and their sum written, the sum read by the recursion, the occupation "
-        "probabilities written, then read with the pairs for the inner products (full box)")
+        t, 4 * (2 + 1 + 1 + 1 + 3) * (px.numel() + py.numel()),
+        "the two pairs read and their sum written, the sum read by the recursion, the occupation "
+        "probabilities written, then read once with the two pairs for the split (full box)")
     return out
 
 

@@ -161,6 +161,19 @@ K2AMD_API int k2amd_mi_forward_backward(const void *px, const void *py, const in
                               int overwrite_ans_grad, void *workspace, size_t workspace_bytes,
                               void *stream);
 
+/* The split of a joint score over the N inputs of joint_mutual_information_recursion
+ * (k2/python/k2/mutual_information.py:404-417, torch ops there: stack, clamp, product, sum):
+ *   prods[n][b] = sum_k px_grad[b][k] * max(px_n[b][k], lowest) + the same over py_grad, py_n,
+ * lowest = the most negative finite value of the type (an input of -inf carries no occupation).
+ * px, py: HOST arrays of N device pointers, each tensor [B][kx] resp. [B][ky] elements, dense;
+ * N <= 8 (else K2AMD_ERR_UNSUPPORTED); prods [N][B]; partial: device scratch of
+ * k2amd_mi_joint_products_scratch_elements(N, B) elements of the type.                          */
+K2AMD_API size_t k2amd_mi_joint_products_scratch_elements(int N, int B);
+K2AMD_API int k2amd_mi_joint_products(const void *const *px, const void *const *py, int N,
+                                      const void *px_grad, const void *py_grad, void *prods,
+                                      void *partial, int B, long long kx, long long ky, int dtype,
+                                      void *stream);
+
 /* ------------------------------------------------------------------ RNN-T log-prob builders
  *
  * Common conventions: symbols [B][S] int64 in [0,C); boundary [B][4] int64 or NULL;

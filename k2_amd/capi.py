@@ -39,6 +39,9 @@ _SIGNATURES = {
     "k2amd_mi_forward_backward_advised": ([_ci] * 6, _ci),
     "k2amd_mi_forward_backward_scratch_bytes": ([_ci] * 5, _sz),
     "k2amd_mi_forward_backward": ([_vp] * 5 + [_sz] + [_vp] * 3 + [_ci] * 6 + [_vp, _sz, _vp], _ci),
+    "k2amd_mi_joint_products_scratch_elements": ([_ci] * 2, ctypes.c_size_t),
+    "k2amd_mi_joint_products": ([_vp, _vp, _ci, _vp, _vp, _vp, _vp, _ci, ctypes.c_longlong, ctypes.c_longlong,
+                                 _ci, _vp], _ci),
     "k2amd_rnnt_logprobs_simple_forward": ([_vp] * 11 + [_ci] * 7 + [_vp], _ci),
     "k2amd_rnnt_logprobs_simple_backward": ([_vp] * 11 + [_ci] * 7 + [_vp], _ci),
     "k2amd_rnnt_logprobs_simple_backward_scratch_elements": ([_ci] * 3, ctypes.c_size_t),
@@ -297,6 +300,35 @@ def mi_forward_backward(px, py, boundary, ans_grad, overwrite_ans_grad=True):
                                               B, S, T, modified, dt, int(overwrite_ans_grad), ptr(ws),
                                               0 if ws is None else ws.numel(), stream_ptr(px.device)))
     return ans, px_grad, py_grad
+
+
+JOINT_MAX_INPUTS = 8
+
+
+def mi_joint_products(px, py, px_grad, py_grad):
+    """prods [N][B] of joint_mutual_information_recursion: px, py sequences of N tensors shaped
+    like px_grad [B][S][T1] and py_grad [B][S+1][T] (same dtype and device, contiguous)."""
+    N = len(px)
+    if N < 1 or len(py) != N or N > JOINT_MAX_INPUTS:
+        raise RuntimeError(f"k2_amd: 1 to {JOINT_MAX_INPUTS} pairs of inputs, got {N} and {len(py)}")
+    dt, dev = _float_dtype(px_grad, "px_grad")
+    B = px_grad.shape[0]
+    expect(px_grad, "px_grad", dt, dev, tuple(px_grad.shape))
+    expect(py_grad, "py_grad", dt, dev, (B,) + tuple(py_grad.shape[1:]))
+    for n in range(N):
+        expect(px[n], f"px[{n}]", dt, dev, tuple(px_grad.shape))
+        expect(py[n], f"py[{n}]", dt, dev, tuple(py_grad.shape))
+    kx = px_grad.numel() // B if B else 0
+    ky = py_grad.numel() // B if B else 0
+    prods = torch.empty(N, B, dtype=dt, device=dev)
+    partial = torch.empty(lib().k2amd_mi_joint_products_scratch_elements(N, B), dtype=dt, device=dev)
+    xs = (ctypes.c_void_p * N)(*[ptr(t) for t in px])
+    ys = (ctypes.c_void_p * N)(*[ptr(t) for t in py])
+    with torch.cuda.device(dev):
+        check(lib().k2amd_mi_joint_products(ctypes.addressof(xs), ctypes.addressof(ys), N, ptr(px_grad),
+                                            ptr(py_grad), ptr(prods), ptr(partial), B, kx, ky,
+                                            dtype_code(px_grad), stream_ptr(dev)))
+    return prods
 
 
 def _t1(T, rnnt_type):

@@ -649,6 +649,46 @@ std::vector<torch::Tensor> PrunedRangesToLattice(torch::Tensor ranges, torch::Te
 
 }  // namespace
 
+namespace {
+
+// prods [N][B] of joint_mutual_information_recursion (k2/python/k2/mutual_information.py:404-417):
+// px, py lists of N tensors shaped like px_grad and py_grad.
+torch::Tensor MutualInformationJointProducts(std::vector<torch::Tensor> px, std::vector<torch::Tensor> py,
+                                             torch::Tensor px_grad, torch::Tensor py_grad) {
+  const int N = static_cast<int>(px.size());
+  TORCH_CHECK(N >= 1 && py.size() == px.size(), "as many px as py, at least one of each");
+  ExpectFloat(px_grad, "px_grad", 3);
+  const auto dtype = px_grad.scalar_type();
+  const auto dev = px_grad.device();
+  auto same = [&](const torch::Tensor &t, const char *name, const torch::Tensor &like) {
+    RequireDevice(t, name);
+    TORCH_CHECK(t.scalar_type() == dtype && t.device() == dev && t.sizes() == like.sizes(), "k2_amd: ",
+                name, " must be ", dtype, " ", like.sizes(), " on ", dev, ", got ", t.scalar_type(), " ",
+                t.sizes(), " on ", t.device());
+  };
+  TORCH_CHECK(py_grad.dim() == 3 && py_grad.size(0) == px_grad.size(0), "py_grad must be [B][S+1][T]");
+  same(py_grad, "py_grad", py_grad);
+  std::vector<const void *> xs(N), ys(N);
+  for (int n = 0; n < N; ++n) {
+    same(px[n], "px[n]", px_grad);
+    same(py[n], "py[n]", py_grad);
+    xs[n] = px[n].data_ptr();
+    ys[n] = py[n].data_ptr();
+  }
+  const int B = px_grad.size(0);
+  const long long kx = B ? px_grad.numel() / B : 0, ky = B ? py_grad.numel() / B : 0;
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(dev);
+  torch::Tensor prods = torch::empty({N, B}, px_grad.options());
+  torch::Tensor partial = torch::empty(
+      {static_cast<int64_t>(k2amd_mi_joint_products_scratch_elements(N, B))}, px_grad.options());
+  void *stream = StreamOf(px_grad);
+  Check(k2amd_mi_joint_products(xs.data(), ys.data(), N, px_grad.data_ptr(), py_grad.data_ptr(),
+                                prods.data_ptr(), partial.data_ptr(), B, kx, ky, DtypeCode(px_grad), stream));
+  return prods;
+}
+
+}  // namespace
+
 // The rows of a [B][4] boundary tensor on their way to the host: a non-blocking copy into pinned
 // memory on the tensor's current stream and an event behind it.  Rows() waits for that event
 // alone (not for what was queued after the copy) and returns the rows as tuples of Python
@@ -691,6 +731,8 @@ PYBIND11_MODULE(_k2_amd, m) {
         pybind11::arg("py"), pybind11::arg("boundary"), pybind11::arg("p"),
         pybind11::arg("log_deriv") = pybind11::none());
   m.def("mutual_information_recover_workspaces", &MutualInformationRecoverWorkspaces);
+  m.def("mutual_information_joint_products", &MutualInformationJointProducts, pybind11::arg("px"),
+        pybind11::arg("py"), pybind11::arg("px_grad"), pybind11::arg("py_grad"));
   m.def("mutual_information_keeps_log_deriv", &MutualInformationKeepsLogDeriv, pybind11::arg("px"),
         pybind11::arg("py"));
   m.def("mutual_information_backward", &MutualInformationBackward, pybind11::arg("px"),

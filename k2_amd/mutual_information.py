@@ -180,6 +180,39 @@ def mutual_information_recursion(
     return (scores, (px_grad, py_grad)) if return_grad else scores
 
 
+class _JointProducts(torch.autograd.Function):
+    """prods [N][B] = sum_k px_grad[b][k] * clamp(px[n][b][k]) + the same over py, clamp(v) =
+    max(v, most negative finite value): the split of the joint score, one native pass over every
+    tensor where the reference stacks, clamps, multiplies and sums with torch ops
+    (k2/python/k2/mutual_information.py:404-417).  Differentiable in the inputs like that chain
+    (the occupation probabilities are constants there, too)."""
+
+    @staticmethod
+    def forward(ctx, px_grad, py_grad, *inputs):
+        N = len(inputs) // 2
+        px, py = inputs[:N], inputs[N:]
+        ctx.save_for_backward(px_grad, py_grad, *inputs)
+        return native.mutual_information_joint_products([x.contiguous() for x in px],
+                                                        [y.contiguous() for y in py], px_grad, py_grad)
+
+    @staticmethod
+    def backward(ctx, g):  # g [N][B]
+        px_grad, py_grad = ctx.saved_tensors[:2]
+        inputs = ctx.saved_tensors[2:]
+        N = len(inputs) // 2
+        lowest = torch.finfo(px_grad.dtype).min
+        grads = []
+        for i, v in enumerate(inputs):
+            if not ctx.needs_input_grad[2 + i]:
+                grads.append(None)
+                continue
+            occupation = px_grad if i < N else py_grad
+            # d clamp(v) / d v = 1 where v >= lowest (torch.clamp's own rule), else 0
+            grads.append(torch.where(v >= lowest, g[i % N].reshape(-1, 1, 1) * occupation,
+                                     torch.zeros((), dtype=v.dtype, device=v.device)))
+        return (None, None) + tuple(grads)
+
+
 def _inner_product(a: Tensor, b: Tensor) -> Tensor:
     """Batched dot product over the last axis: [..., N] x [..., N] -> [...]."""
     return (a * b).sum(dim=-1)
@@ -207,10 +240,18 @@ def joint_mutual_information_recursion(
         assert boundary.shape == (B, 4)
         _check_boundary(boundary, S, T)
 
-    px_cat = torch.stack(list(px), dim=0)  # [N][B][S][T1]
-    py_cat = torch.stack(list(py), dim=0)  # [N][B][S+1][T]
-    px_tot = px_cat.sum(dim=0).contiguous()
-    py_tot = py_cat.sum(dim=0).contiguous()
+    fused = N <= native.JOINT_MAX_INPUTS and B > 0
+    if fused:  # the sum of the inputs without a stacked copy of them (nothing differentiates it)
+        with torch.no_grad():
+            px_tot, py_tot = px[0], py[0]
+            for x, y in zip(px[1:], py[1:]):
+                px_tot, py_tot = px_tot + x, py_tot + y
+            px_tot, py_tot = px_tot.contiguous(), py_tot.contiguous()
+    else:
+        px_cat = torch.stack(list(px), dim=0)  # [N][B][S][T1]
+        py_cat = torch.stack(list(py), dim=0)  # [N][B][S+1][T]
+        px_tot = px_cat.sum(dim=0).contiguous()
+        py_tot = py_cat.sum(dim=0).contiguous()
     if _single_launch(px_tot, py_tot):
         (tot_probs, px_grad, py_grad) = native.mutual_information_forward_backward(
             px_tot, py_tot, boundary, None)
@@ -222,10 +263,13 @@ def joint_mutual_information_recursion(
                                                                 log_deriv)
     # -inf inputs carry zero occupation: clamp them to the most negative finite value so that
     # 0 * -inf does not produce NaN (k2/python/k2/mutual_information.py:410-411)
-    lowest = torch.finfo(px_cat.dtype).min
-    x_prods = _inner_product(px_grad.reshape(1, B, -1), px_cat.reshape(N, B, -1).clamp(min=lowest))
-    y_prods = _inner_product(py_grad.reshape(1, B, -1), py_cat.reshape(N, B, -1).clamp(min=lowest))
-    prods = x_prods + y_prods  # [N][B]
+    if fused:
+        prods = _JointProducts.apply(px_grad, py_grad, *px, *py)  # [N][B]
+    else:
+        lowest = torch.finfo(px_cat.dtype).min
+        x_prods = _inner_product(px_grad.reshape(1, B, -1), px_cat.reshape(N, B, -1).clamp(min=lowest))
+        y_prods = _inner_product(py_grad.reshape(1, B, -1), py_cat.reshape(N, B, -1).clamp(min=lowest))
+        prods = x_prods + y_prods  # [N][B]
     # the first element absorbs the gap between the sum of logs and the log of the sum
     with torch.no_grad():
         offset = tot_probs - prods.sum(dim=0)

@@ -45,6 +45,19 @@ def boundary_read(boundary: torch.Tensor):
     return _BoundaryRead(boundary)
 
 
+JOINT_MAX_INPUTS = capi.JOINT_MAX_INPUTS
+
+
+def mutual_information_joint_products(px, py, px_grad: torch.Tensor, py_grad: torch.Tensor) -> torch.Tensor:
+    """prods [N][B] = sum_k px_grad[b][k] * max(px[n][b][k], lowest finite) + the same over py: the
+    split of a joint score over the N inputs of joint_mutual_information_recursion
+    (k2/python/k2/mutual_information.py:404-417), every tensor read once."""
+    _require_device(px_grad)
+    if _ext is not None:
+        return _ext.mutual_information_joint_products(list(px), list(py), px_grad, py_grad)
+    return capi.mi_joint_products(list(px), list(py), px_grad, py_grad)
+
+
 def mutual_information_recover_workspaces() -> int:
     """Waits for the streams that the pipelined fp32 kernels have run on and reads the error flag
     of each scratch buffer.  Where a kernel gave up a bounded wait (its scores came out as NaN,

@@ -601,3 +601,44 @@ def test_fp64_headline_shape_on_the_wave_kernels(device, monkeypatch):
             bd = cases.random_boundary(rng, B, S, T, modified)
             for boundary in (None, bd):
                 against_oracle(f"modified={modified} B={B} S={S} T={T} bd={boundary is not None}", px, py, boundary)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_joint_recursion_split_matches_the_torch_chain(device, dtype):
+    """The fused split of joint_mutual_information_recursion against the reference's chain of torch
+    ops (stack, clamp, product, sum; k2/python/k2/mutual_information.py:404-417) on the same
+    occupation probabilities: values and the gradients to every input, with -inf entries in the
+    inputs, sizes that are no multiple of anything, one to three pairs."""
+    import importlib
+    kmi = importlib.import_module("k2_amd.mutual_information")
+    g = torch.Generator().manual_seed(5)
+    B, S, T = 3, 7, 41
+    lowest = torch.finfo(dtype).min
+    rtol = 2e-5 if dtype == torch.float32 else 1e-12
+    for N in (1, 2, 3):
+        def leaf(*shape):
+            return (torch.randn(*shape, generator=g, dtype=torch.float64) - 2).to(dtype).to(device).requires_grad_(True)
+        px = [leaf(B, S, T + 1) for _ in range(N)]
+        py = [leaf(B, S + 1, T) for _ in range(N)]
+        px_grad = torch.rand(B, S, T + 1, generator=g, dtype=torch.float64).to(dtype).to(device)
+        py_grad = torch.rand(B, S + 1, T, generator=g, dtype=torch.float64).to(dtype).to(device)
+        with torch.no_grad():
+            px[0][0, 1, 5] = float("-inf")
+            px_grad[0, 1, 5] = 0.0
+            py[N - 1][2, 0, 0] = float("-inf")
+            py_grad[2, 0, 0] = 0.0
+        w = torch.randn(N, B, generator=g, dtype=torch.float64).to(dtype).to(device)
+        got = kmi._JointProducts.apply(px_grad, py_grad, *px, *py)
+        (got * w).sum().backward()
+        got_grads = [t.grad.clone() for t in px + py]
+        for t in px + py:
+            t.grad = None
+        px_cat, py_cat = torch.stack(px), torch.stack(py)
+        want = ((px_grad.reshape(1, B, -1) * px_cat.reshape(N, B, -1).clamp(min=lowest)).sum(-1)
+                + (py_grad.reshape(1, B, -1) * py_cat.reshape(N, B, -1).clamp(min=lowest)).sum(-1))
+        (want * w).sum().backward()
+        assert got.shape == (N, B) and torch.isfinite(got).all()
+        torch.testing.assert_close(got, want.detach(), rtol=rtol, atol=0)
+        for a, t in zip(got_grads, px + py):
+            torch.testing.assert_close(a, t.grad, rtol=rtol, atol=0)
