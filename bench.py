@@ -40,7 +40,7 @@ BWD_BYTES_PER_CELL = 16
 # HBM bytes per launch on the default workload, from rocprofv3's FETCH_SIZE / WRITE_SIZE counters
 # scaled by a 256 MiB device copy (profiles/mi_bidir_kernel_c4_hbm_traffic.md).  Reported only
 # for the default shape; any other --B/--S/--T prints null.
-MEASURED_TRAFFIC_BYTES = {"mi_forward_backward": 141140000, "mi_forward": 50120000, "mi_backward": 69230000}
+MEASURED_TRAFFIC_BYTES = {"mi_forward_backward": 141090000, "mi_forward": 50120000, "mi_backward": 69230000}
 MEASURED_TRAFFIC_BYTES_PLAIN_PAIR = {"mi_forward": 50040000, "mi_backward": 85940000}  # --no-keep
 
 
