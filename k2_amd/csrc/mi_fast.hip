@@ -38,12 +38,17 @@
 // backward alone, and both in one launch for callers that want the gradients with the scores.
 // In that launch, and in the two-call pair that goes with it, the forward hands the backward the
 // logarithm of every cell's px-edge derivative in a tensor that takes p's place, so the backward
-// reads one value per cell.  In the single launch a workgroup also waits for a LATER ticket (the
-// chunk below it, once it sweeps backward), so its launcher requires that all workgroups be
-// resident at once.
+// reads one value per cell.  The single launch hands its work out as tasks through the same ticket
+// counter to persistent workgroups; a task only ever waits for tasks with EARLIER tickets, which
+// running workgroups hold, so the launch makes progress with any number of resident workgroups
+// (deadlock freedom depends on exactly that: no task may wait for a later ticket).
 //
 // Arithmetic is the reference's log-domain recursion (k2/python/csrc/torch/
 // mutual_information_cpu.cu:89-121, log-add of k2/csrc/utils.h:511-563) with hardware exp2/log2.
+// The forward sweeps of the single launch carry p in base-2 logarithms and relative to a FRAME
+// (a multiple of 64 that follows the values block by block, see ChainStep2 and Frames): p never
+// leaves that launch, and values of a few hundred carry an ulp of 1e-5 where the thousands that
+// p itself reaches carry 2.4e-4 and more.
 #include <algorithm>
 #include <atomic>
 #include <cstdlib>
@@ -92,9 +97,9 @@ typedef Layout<4> BwdLayout;
 static_assert(kBlockItems == 2 * kWave * kStorerWaves, "two work items per storer lane");
 
 struct FastHeader {
-  unsigned ticket;  // next chunk to hand out; put back by the drawer of a launch's last ticket
-  unsigned done;    // (not used any more; stays 0)
-  unsigned error;   // set when a bounded wait timed out (sticky until re-initialised)
+  unsigned ticket;    // next chunk to hand out; put back by the drawer of a launch's last ticket
+  unsigned reserved;  // stays 0
+  unsigned error;     // set when a bounded wait timed out (sticky until re-initialised)
   unsigned pad[61];
 };
 
@@ -131,6 +136,87 @@ __device__ __forceinline__ float ChainStep(float P, float fx, float fy) {
   const float e = __builtin_amdgcn_exp2f(-__builtin_fabsf(d) * kLog2e);
   return __builtin_fmaf(__builtin_amdgcn_logf(1.0f + e), kLn2, mx);
 }
+
+// The same step in base-2 logarithms (P, fx, fy all scaled by log2 e): the dependent multiply in
+// front of the exponential and the one behind the logarithm are gone,
+//     P' = max + log2(1 + exp2(-|inc - x|)).
+// Used where p never leaves the launch (the single launch): a p that went through a scaling is
+// one rounding away from the reference's, which matters where p itself is handed on, and does
+// not where only differences of p (the log-derivatives) and the score are.
+__device__ __forceinline__ float ChainStep2(float P, float fx, float fy) {
+  float x, mx, d, inc = fx;
+  asm volatile(
+      "v_add_f32 %[x], %[P], %[fy]\n\t"
+      "s_nop 0\n\t"
+      "v_add_f32_dpp %[inc], %[P], %[inc] wave_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32 %[mx], %[inc], %[x]\n\t"
+      "v_sub_f32 %[d], %[inc], %[x]"
+      : [x] "=&v"(x), [inc] "+&v"(inc), [mx] "=&v"(mx), [d] "=&v"(d)
+      : [P] "v"(P), [fy] "v"(fy));
+  const float e = __builtin_amdgcn_exp2f(-__builtin_fabsf(d));
+  return mx + __builtin_amdgcn_logf(1.0f + e);
+}
+
+// Frames.  A forward sweep of the single launch keeps, per chunk and per 32-step block, a FRAME: a
+// multiple of 64 (so that adding and subtracting frames is exact) that is subtracted from every
+// value the chain carries in that block.  ANY sequence of frames gives the same mathematics; a
+// frame near the values keeps them small, and with them their rounding errors.  The chain
+// wavefront moves its values from one block's frame to the next at the block boundary and picks
+// the frame two blocks ahead (so that a barrier lies between the choice and every other
+// wavefront's use of it) by extrapolating the largest live value; a chunk's first two blocks take
+// the frame of the first words that arrive from the chunk above.  Between chunks every published
+// block of edge words comes with its frame (one more self-validating word); on the cut every
+// chunk publishes the frame of its last block next to its 64 values.
+constexpr int kFrameRing = 8;
+constexpr float kFrameUnit = 64.0f;
+__device__ __forceinline__ float RoundToFrame(float v) {
+  v = fminf(fmaxf(v, -1.0e9f), 1.0e9f);
+  return kFrameUnit * __builtin_rintf(v * (1.0f / kFrameUnit));
+}
+
+// The gauge.  Adding a constant to every px and another to every py of a sequence changes the score
+// by a known amount (every path from the origin to the end cell takes the same number of edges of
+// either kind) and the gradients not at all.  The single launch subtracts from px and py (in
+// base-2 logarithms) the means of a small sample of each, rounded to sixteenths, before the chain
+// sees them: what the chain then carries grows like the logarithm of the number of paths instead
+// of like the sum of the log-probabilities along one, and the frames have little left to follow.
+// ANY pair of constants gives the same mathematics, but every task of a sequence must use the
+// SAME pair: all of them take it from the same sixteen floats of the sequence's first px and py
+// row with the same arithmetic (GaugeOf), and the join adds back what the pair took off the score.
+struct Gauge {
+  float x, y;  // subtracted from px * log2(e), py * log2(e)
+};
+// The sample: lanes 0..15 of a wavefront hold the first 16 floats of the sequence's first px row,
+// lanes 16..31 those of its first py row (lattice coordinates; `valid`: the float exists).  Each
+// constant is the mean of the sample's values that lie within kGaugeBand of its largest one (an
+// edge that is blocked or all but blocked says nothing about the edges that the paths that matter
+// take), in base-2 logarithms, rounded to sixteenths.  Reductions over rows of 16 lanes in a fixed
+// order: every wavefront of every task gets the same bits.
+constexpr int kGaugeSample = 16;
+constexpr float kGaugeBand = 20.0f;
+#define K2AMD_ROW_BUTTERFLY_F(v, op)                                                          \
+  v = op(v, __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), 0xB1, 0xf, 0xf, true)));  \
+  v = op(v, __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), 0x4E, 0xf, 0xf, true)));  \
+  v = op(v, __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), 0x141, 0xf, 0xf, true))); \
+  v = op(v, __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), 0x140, 0xf, 0xf, true)))
+__device__ __forceinline__ float GaugeMaxF(float a, float b) { return fmaxf(a, b); }
+__device__ __forceinline__ float GaugeAddF(float a, float b) { return a + b; }
+__device__ __forceinline__ Gauge GaugeOf(float v, bool valid, int ns) {
+  const bool ok = valid && __builtin_fabsf(v) < 1.0e29f;  // (NaN: not ok)
+  float top = ok ? v : -3.0e38f;
+  K2AMD_ROW_BUTTERFLY_F(top, GaugeMaxF);
+  const bool in = ok && v >= top - kGaugeBand;
+  float sum = in ? v : 0.0f, cnt = in ? 1.0f : 0.0f;
+  K2AMD_ROW_BUTTERFLY_F(sum, GaugeAddF);
+  K2AMD_ROW_BUTTERFLY_F(cnt, GaugeAddF);
+  const float mean = cnt > 0.0f ? sum / cnt * kLog2e : 0.0f;
+  const float r = __builtin_rintf(fminf(fmaxf(mean, -1.0e6f), 1.0e6f) * 16.0f) * (1.0f / 16.0f);
+  Gauge g;
+  g.x = ns > 0 ? __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(r), 0)) : 0.0f;
+  g.y = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(r), kGaugeSample));
+  return g;
+}
+#undef K2AMD_ROW_BUTTERFLY_F
 
 // Everything these kernels reach through a pointer is device memory, and they say so: the tasks
 // of the single launch get their pointers from a structure in LDS, where the compiler cannot see
@@ -273,6 +359,11 @@ struct Half {
 // which device-coherent stores send to memory as the partial lines they are).
 // Blocks a chunk of a half can have: its positions end one past the cut diagonal, and the cut
 // lies half way along the lattice's longest path.
+// Floats per (sequence, chunk + 1) row of the edge buffer: the edge words of every step a chunk can
+// have, then one frame word per block (single launch).
+__host__ __device__ inline int EdgeWords(int Tn) { return (int)(((size_t)Tn + 2 + kRows + kW + 3) / 4 * 4 + kW); }
+__host__ __device__ inline int EdgeStride(int Tn) { return EdgeWords(Tn) + (EdgeWords(Tn) / kW + 4 + 3) / 4 * 4; }
+
 constexpr int kSlabBlockFloats = kRows * kW;
 __host__ __device__ inline int SlabBlocks(int S, int Tn, int modified) {
   const int diagonals = Tn + (modified ? 0 : S);
@@ -304,7 +395,7 @@ __global__ void FastWsInitKernel(FastHeader *hdr, unsigned *edge, size_t n) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i == 0) {
     hdr->ticket = 0;
-    hdr->done = 0;
+    hdr->reserved = 0;
     hdr->error = 0;
   }
   for (size_t k = i; k < n; k += (size_t)gridDim.x * blockDim.x) edge[k] = kSentinel;
@@ -366,12 +457,15 @@ __device__ __forceinline__ void PublishCut(float *addr, float v) { PublishEdge(a
 // ---- the cut of the single launch (see MiBidirKernel) ----
 constexpr int kCutRows = 2056;  // lattice rows (S + 2 at most) the single launch serves
 constexpr int kCutWordsPerSeqHeader = 16;
+constexpr int kCutChunks = (kCutRows + kRows - 1) / kRows;  // chunks a half can have
 
 struct CutShared {
   // alpha / beta of the sequence's cut cells by lattice row, then exp(alpha + beta - best); also
   // the two rotating rows of the exact recursion
   float a[kCutRows];
   float b[kCutRows];
+  // the frames of the chunks' values on the cut (see Frames), by chunk of each half
+  float fa[kCutChunks], fb[kCutChunks];
   float total;   // the sequence's score, from the join of this task
   float scale;   // the gradient of the sequence's score
   int split_ok;  // the score is finite: the halves sweep back from the cut
@@ -383,22 +477,31 @@ struct CutShared {
 
 // Per sequence, in the workspace: depart (readers of the cut finished), the gradient of the
 // sequence's score, stored (forward sweeps whose log-derivatives have all reached memory), then
-// alpha by own row of the first half and beta by own row of the second.  Counters count up from
+// alpha by own row of the first half and beta by own row of the second (base-2 logarithms, each
+// chunk's 64 relative to the chunk's frame), then those frames by chunk.  Counters count up from
 // the sentinel, which is what the workspace is initialised to.
 struct CutWords {
   unsigned *depart, *stored;
-  float *scale, *alpha, *beta;
+  float *scale, *alpha, *beta, *frame_alpha, *frame_beta;
+  float *gauge;  // two words: what the sweeps subtracted from px and py (see Gauge)
   int words;
 };
+__host__ __device__ inline int CutFrameWords(int nchunks) { return (nchunks + 3) / 4 * 4; }
+__host__ __device__ inline int CutWordsPerSequence(int nchunks) {
+  return kCutWordsPerSeqHeader + 2 * nchunks * kRows + 2 * CutFrameWords(nchunks);
+}
 __device__ __forceinline__ CutWords CutOf(float *cut, int b, int nchunks) {
   CutWords w;
-  w.words = kCutWordsPerSeqHeader + 2 * nchunks * kRows;
+  w.words = CutWordsPerSequence(nchunks);
   float *base = cut + (size_t)b * w.words;
   w.depart = reinterpret_cast<unsigned *>(base) + 1;
   w.scale = base + 2;
   w.stored = reinterpret_cast<unsigned *>(base) + 3;
+  w.gauge = base + 4;
   w.alpha = base + kCutWordsPerSeqHeader;
   w.beta = w.alpha + nchunks * kRows;
+  w.frame_alpha = w.beta + nchunks * kRows;
+  w.frame_beta = w.frame_alpha + CutFrameWords(nchunks);
   return w;
 }
 
@@ -475,7 +578,7 @@ struct BidirJoin {
 // values BEFORE they are added, which keeps the shares exact to a few ulps of themselves.
 // (Inlined: as a function of its own it would take the words' addresses and hand back its results
 // through scratch memory, a trip there for each.)
-__device__ __forceinline__ float WaveCutJoin(CutShared &sh, const CutWords cw, int ns, int row0,
+__device__ __forceinline__ float WaveCutJoin(CutShared &sh, const CutWords cw, int ns, int py_edges, int row0,
                                              int mirror, FastHeader *hdr, float *seed_out,
                                              float *scale_out) {
   const int lane = threadIdx.x & (kWave - 1);
@@ -484,10 +587,20 @@ __device__ __forceinline__ float WaveCutJoin(CutShared &sh, const CutWords cw, i
   constexpr int kBatch = 4;
   const unsigned *wa = reinterpret_cast<const unsigned *>(cw.alpha);
   const unsigned *wb = reinterpret_cast<const unsigned *>(cw.beta);
-  float scale = 0.0f;
+  const unsigned *wfa = reinterpret_cast<const unsigned *>(cw.frame_alpha);
+  const unsigned *wfb = reinterpret_cast<const unsigned *>(cw.frame_beta);
+  const int nchunks = ns / kRows + 1;  // chunks that hold rows of this sequence
+  float scale = 0.0f, gauge_x = 0.0f, gauge_y = 0.0f;
   for (int spins = 0;; ++spins) {
     const unsigned us = __hip_atomic_load(Global(reinterpret_cast<const unsigned *>(cw.scale)), __ATOMIC_RELAXED,
                                           __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned ugx = __hip_atomic_load(Global(reinterpret_cast<const unsigned *>(cw.gauge)), __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned ugy = __hip_atomic_load(Global(reinterpret_cast<const unsigned *>(cw.gauge) + 1), __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+    const int fc = min(lane, nchunks - 1);
+    const unsigned ufa = __hip_atomic_load(Global(wfa + fc), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned ufb = __hip_atomic_load(Global(wfb + fc), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     bool missing = false;
     for (int s0 = lane; s0 <= ns; s0 += kWave * kBatch) {
       unsigned ua[kBatch], ub[kBatch];
@@ -507,8 +620,16 @@ __device__ __forceinline__ float WaveCutJoin(CutShared &sh, const CutWords cw, i
         }
       }
     }
-    missing |= us == kSentinel;
+    static_assert(kCutChunks <= kWave, "one lane per chunk's frame");
+    if (lane < nchunks) {
+      missing |= ufa == kSentinel || ufb == kSentinel;
+      sh.fa[lane] = __uint_as_float(ufa);
+      sh.fb[lane] = __uint_as_float(ufb);
+    }
+    missing |= us == kSentinel || ugx == kSentinel || ugy == kSentinel;
     scale = __uint_as_float(us);
+    gauge_x = __uint_as_float(ugx);
+    gauge_y = __uint_as_float(ugy);
     if (!__any(missing)) break;
     // bounded like every wait: what is missing stays a NaN, the score comes out as not finite
     // and the error flag turns the results into NaN
@@ -522,13 +643,15 @@ __device__ __forceinline__ float WaveCutJoin(CutShared &sh, const CutWords cw, i
     __builtin_amdgcn_s_sleep(1);
   }
   __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  // Lattice row s is own row s of the first half (chunk s / 64) and own row ns - s of the second.
   float best = -3.0e38f;
   int best_s = 0x7fffffff;
   for (int s = lane; s <= ns; s += kWave) {
-    const float u = sh.a[s] + sh.b[s];
+    const float u = (sh.a[s] + sh.b[s]) + (sh.fa[s / kRows] + sh.fb[(ns - s) / kRows]);
     if (u > best) { best = u; best_s = s; }
   }
-  // the largest sum, the smallest row among equals
+  // the largest sum (to the rounding of the frames' sum: any cell near the best one serves as the
+  // reference), the smallest row among equals
   const float wave_best = WaveMaxF(best);
   best_s = WaveMinI(best == wave_best ? best_s : 0x7fffffff);
   const int at = best_s <= ns ? best_s : 0;  // (no candidate at all: every sum was NaN)
@@ -536,11 +659,15 @@ __device__ __forceinline__ float WaveCutJoin(CutShared &sh, const CutWords cw, i
   // the compiler from moving them.
   __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
   const float a_ref = sh.a[at], b_ref = sh.b[at];
+  const float fa_ref = sh.fa[at / kRows], fb_ref = sh.fb[(ns - at) / kRows];
   const bool reachable = a_ref + b_ref > kLogZeroTest;
   __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
   float sum = 0.0f;
   for (int s = lane; s <= ns; s += kWave) {
-    const float w = reachable ? expf((sh.a[s] - a_ref) + (sh.b[s] - b_ref)) : 0.0f;
+    // differences of values of like size first, the (exact) differences of the frames added to them
+    const float da = (sh.a[s] - a_ref) + (sh.fa[s / kRows] - fa_ref);
+    const float db = (sh.b[s] - b_ref) + (sh.fb[(ns - s) / kRows] - fb_ref);
+    const float w = reachable ? __builtin_amdgcn_exp2f(da + db) : 0.0f;
     sh.a[s] = w;
     sum += w;
   }
@@ -551,7 +678,13 @@ __device__ __forceinline__ float WaveCutJoin(CutShared &sh, const CutWords cw, i
   const float share = sh.a[s_own];
   *seed_out = reachable && own <= ns ? share / sum * scale : 0.0f;
   *scale_out = scale;
-  return reachable ? (a_ref + b_ref) + logf(sum) : NegInfF();
+  // The score in natural logarithms: the best cell's values and the sum (small), the two frames
+  // (thousands, exact) and what the gauge took off every path (ns px edges, py_edges py edges),
+  // added in double so that the one rounding that matters is the last.
+  const double log2_score = ((double)a_ref + (double)b_ref) + (double)__builtin_amdgcn_logf(sum) +
+                            ((double)fa_ref + (double)fb_ref) + (double)ns * (double)gauge_x +
+                            (double)py_edges * (double)gauge_y;
+  return reachable ? (float)(log2_score * 0.69314718055994530942) : NegInfF();
 }
 
 // ------------------------------------------------------------------------------ forward
@@ -572,6 +705,9 @@ struct FwdLds {
   // px of the row above the chunk (the last row of the chunk above), block by block: written by
   // the loaders one block ahead of the rest, read by the edge wavefront
   float px_above[4][kW];
+  // the chunk's frame of each recent block (single launch, see Frames), and what it lies above
+  // the block before's; slot kb % kFrameRing
+  float frame[kFrameRing], shift[kFrameRing];
   unsigned ticket;
 };
 
@@ -608,7 +744,8 @@ __device__ __forceinline__ void MiForwardChunk(
     FwdLds &lds, const float *__restrict__ px, const float *__restrict__ py, const Box &box,
     float *__restrict__ p, float *__restrict__ ans,
     float *__restrict__ log_deriv, FastHeader *hdr, float *edge, int B, int S, int Tn,
-    int modified, int nchunks, int edge_stride, int seq, int chunk, Half half, float *cut_out) {
+    int modified, int nchunks, int edge_stride, int seq, int chunk, Half half, float *cut_out,
+    float *cut_frame_out, float *gauge_out) {
   static_assert(!kBidir || (kKeep && !kWriteP), "the halves keep the log-derivatives only");
   ChunkGeom g;
   g.b = seq;
@@ -630,6 +767,7 @@ __device__ __forceinline__ void MiForwardChunk(
   g.nblocks = blocks_of(g.row0);
   if (kBidir && g.nblocks == 0) {  // no cell of these rows lies in the half
     if (threadIdx.x < kRows) PublishCut(cut_out + threadIdx.x, kLogZero);
+    if (threadIdx.x == 0) PublishCut(cut_frame_out, 0.0f);
     return;
   }
   const bool has_down = g.row0 + kRows <= g.ns && blocks_of(g.row0 + kRows) > 0;
@@ -648,8 +786,27 @@ __device__ __forceinline__ void MiForwardChunk(
                         : log_deriv + (size_t)g.b * (S + 1) * LS;
   float *edge_out = edge + ((size_t)g.b * nchunks + g.c + 1) * edge_stride;  // read by chunk c+1
   float *edge_in = edge + ((size_t)g.b * nchunks + g.c) * edge_stride;
+  // (single launch) the frames of the published blocks: one word per block behind a row's edge words
+  float *frame_out = edge_out + EdgeWords(Tn), *frame_in = edge_in + EdgeWords(Tn);
+  // The blocks of the chunk above whose words this chunk takes (it takes their frames with them),
+  // and the same for the chunk below and this chunk's blocks: both sides work it out alike.
+  auto frames_lo = [&]() { return max(edge_shift, 0) / kW; };
+  auto frames_hi = [&](int blocks_above, int blocks_below) {
+    return (min(blocks_above * kW - 1, blocks_below * kW - 1 + edge_shift)) / kW;
+  };
+  // natural logarithms in the two-launch kernels, base-2 ones less the gauge in the single launch
+  const float in_scale = kBidir ? kLog2e : 1.0f;
+  // what block kb's frame lies above block kb-1's (a multiple of 64; kb >= 1)
+  auto frame_step = [&](int kb) { return lds.shift[kb & (kFrameRing - 1)]; };
 
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  Gauge gauge{0.0f, 0.0f};  // (set in the prologue by the wavefronts that scale inputs)
+  // where the gauge's sample lies: the first floats of the box's first px and py row
+  const int gauge_idx_x = (g.b * S + g.s0) * T1 + g.t0, gauge_idx_y = (g.b * (S + 1) + g.s0) * Tn + g.t0;
+  // lanes 0..15: px, 16..31: py (the row's valid columns; px has no row at all where ns = 0)
+  const bool gauge_valid = lane < 2 * kGaugeSample &&
+                           ((lane & kGaugeSample) ? (lane & (kGaugeSample - 1)) < g.nt
+                                                  : g.ns > 0 && (lane & (kGaugeSample - 1)) < g.nt + 1 - modified);
   typedef FwdLayout L;
   constexpr int kLoadItems = L::kLoadItems, kRowStep = L::kRowStep;
   const int role = RoleOf<L>(wave);
@@ -731,8 +888,8 @@ __device__ __forceinline__ void MiForwardChunk(
         const float in_x[4] = {qx.x, qx.y, qx.z, qx.w}, in_y[4] = {qy.x, qy.y, qy.z, qy.w};
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          vx[e] = rowx_ok[it] ? fmaxf(in_x[e], kLogZero) : kLogZero;
-          vy[e] = rowy_ok[it] ? fmaxf(in_y[e], kLogZero) : kLogZero;
+          vx[e] = rowx_ok[it] ? fmaxf(__builtin_fmaf(in_x[e], in_scale, -gauge.x), kLogZero) : kLogZero;
+          vy[e] = rowy_ok[it] ? fmaxf(__builtin_fmaf(in_y[e], in_scale, -gauge.y), kLogZero) : kLogZero;
         }
       } else {
         asm volatile("");
@@ -745,8 +902,8 @@ __device__ __forceinline__ void MiForwardChunk(
         for (int e = 0; e < 4; ++e) {
           const bool okx = rowx_ok[it] && jx + e >= 0 && jx + e <= hi_x;
           const bool oky = rowy_ok[it] && jp + e >= 0 && jp + e <= hi_y;
-          vx[e] = okx ? fmaxf(in_x[e], kLogZero) : kLogZero;
-          vy[e] = oky ? fmaxf(in_y[e], kLogZero) : kLogZero;
+          vx[e] = okx ? fmaxf(__builtin_fmaf(in_x[e], in_scale, -gauge.x), kLogZero) : kLogZero;
+          vy[e] = oky ? fmaxf(__builtin_fmaf(in_y[e], in_scale, -gauge.y), kLogZero) : kLogZero;
         }
       }
       const int pq = (kb % 3) * kQuadsPerBlock + mm;
@@ -764,7 +921,7 @@ __device__ __forceinline__ void MiForwardChunk(
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const int jx = (kb + 1) * kW + 4 * mm + e - 1 + g.skew;
-      v[e] = g.c > 0 && jx >= 0 && jx <= hi_x ? fmaxf(in[e], kLogZero) : kLogZero;
+      v[e] = g.c > 0 && jx >= 0 && jx <= hi_x ? fmaxf(__builtin_fmaf(in[e], in_scale, -gauge.x), kLogZero) : kLogZero;
     }
     *reinterpret_cast<float4 *>(&lds.px_above[(kb + 1) & 3][4 * mm]) = make_float4(v[0], v[1], v[2], v[3]);
   };
@@ -816,7 +973,10 @@ __device__ __forceinline__ void MiForwardChunk(
             asm volatile("" : "+v"(b4.x), "+v"(b4.y), "+v"(b4.z), "+v"(b4.w));
             before = b4.w;
           } else {
+            // (single launch: the chain moved that value into this block's frame with the same
+            // subtraction before lane q saw it)
             before = kb > 0 ? lds.last[(kb + 2) % 3][q - 1] : kLogZero;
+            if (kBidir && kb > 0) before = fmaxf(before, -1.0e36f) - frame_step(kb);
           }
           t1[0] = before + x4.x; t1[1] = a.x + x4.y; t1[2] = a.y + x4.z; t1[3] = a.z + x4.w;
         }
@@ -854,6 +1014,29 @@ __device__ __forceinline__ void MiForwardChunk(
     }
   };
 
+  // (single launch) The frame of block kb + 2, chosen in iteration kb by the first storer wavefront
+  // (off the chain's path; a barrier lies between the choice and every use: the edge wavefront's
+  // in iteration kb + 1, the chain's in kb + 2, the storers' in kb + 3): half way between the
+  // largest and the smallest live value at the end of block kb - 2, the last one whose results all
+  // storers have passed on, but never far below the largest (rows behind an all but blocked edge
+  // carry no weight).  The gauge has taken the trend out of the values, so what they were four
+  // blocks earlier is a fair guess of what they will be.
+  auto choose_frame = [&](int kb) {
+    const int to = (kb + 2) & (kFrameRing - 1), from = (kb + 1) & (kFrameRing - 1);
+    float next = lds.frame[from];
+    if (kb >= 2) {
+      const float v = lds.last[(kb - 2) % 3][lane];
+      const bool live = g.row0 + lane <= g.ns && v > kLogZeroTest;
+      const float top = WaveMaxF(live ? v : -3.0e38f), bottom = -WaveMaxF(live ? -v : -3.0e38f);
+      if (top > kLogZeroTest)
+        next = RoundToFrame(lds.frame[(kb - 2) & (kFrameRing - 1)] + (top - fminf(0.5f * (top - bottom), 256.0f)));
+    }
+    if (lane == 0) {
+      lds.shift[to] = next - lds.frame[from];
+      lds.frame[to] = next;
+    }
+  };
+
   // ---- edge wavefront ----------------------------------------------------------------------
   // Lanes 0..31 prepare, for each step n of block kb, what arrives at lane 0 along px:
   //     p[row0-1][..] (taken from the chunk above) + px[row0-1][..]
@@ -866,32 +1049,78 @@ __device__ __forceinline__ void MiForwardChunk(
     const int jx = kb * kW + lane - 1 + g.skew;
     float v = kLogZero;
     if (g.c > 0 && lane < kW && jx >= 0 && jx <= hi_x)
-      v = fmaxf(mirror ? pxb[(size_t)(g.s0 + g.ns - g.row0) * T1 + g.t0 + hi_x - jx]
-                       : pxb[(size_t)(g.s0 + g.row0 - 1) * T1 + g.t0 + jx], kLogZero);
+      v = fmaxf(__builtin_fmaf(mirror ? pxb[(size_t)(g.s0 + g.ns - g.row0) * T1 + g.t0 + hi_x - jx]
+                                      : pxb[(size_t)(g.s0 + g.row0 - 1) * T1 + g.t0 + jx],
+                               in_scale, -gauge.x), kLogZero);
     return v;
   };
+  // (single launch) frames of the chunk above that this wavefront has taken so far: the newest
+  // one and the one before it, by block of the chunk above; wave-uniform
+  int up_taken = frames_lo() - 1;
+  float up_frame_new = 0.0f, up_frame_old = 0.0f;
+  const int up_hi = kBidir && g.c > 0 && nblocks_up > 0 ? frames_hi(nblocks_up, g.nblocks) : -1;
   auto take_block = [&](int kb, float px_above) {
-    if (lane < kW && kb < g.nblocks) {
-      const int n = kb * kW + lane;
-      float v = kLogZero;
-      if (g.c == 0) {
-        if (n == 0) v = 0.0f;  // the origin: p[s_begin][t_begin] = 0 "arrives" at step 0
+    if (kb >= g.nblocks) return;  // (uniform)
+    const int n = kb * kW + lane;
+    const int idx = n + edge_shift;
+    const bool word = lane < kW && g.c > 0 && idx >= 0 && idx < nblocks_up * kW;
+    // Lanes 32 and 33 take the frames of the blocks above that this block's words lie in, where
+    // they have not been taken yet (blocks come in order, so at most two are new, and two only
+    // for this chunk's first block), in the same trip to memory as the words.
+    const int j_last = min((kb * kW + kW - 1 + edge_shift) / kW, up_hi);
+    const int j_want = lane - kW + up_taken + 1;  // lane 32: the next one, lane 33: the one after
+    const bool frame = kBidir && (lane == kW || lane == kW + 1) && j_want <= j_last;
+    float v = kLogZero;
+    if (word || frame) v = TakeEdge(word ? edge_in + idx : frame_in + j_want, hdr, word ? kLogZero : 0.0f);
+    float own = 0.0f;  // (single launch) this block's frame
+    if (kBidir) {
+      const int got = min(j_last - up_taken, 2);  // (uniform) frames taken just now: <= 0, 1 or 2
+      if (got == 2) {
+        up_frame_old = LaneF(v, kW);
+        up_frame_new = LaneF(v, kW + 1);
+      } else if (got == 1) {
+        up_frame_old = up_frame_new;
+        up_frame_new = LaneF(v, kW);
+      }
+      if (got > 0) up_taken += got;
+      if (kb == 0) {
+        // a chunk's first two blocks take the frame of the first words that arrive (chunk 0: 0)
+        own = got == 2 ? up_frame_old : (got == 1 ? up_frame_new : 0.0f);
+        if (lane == 0) {
+          lds.frame[0] = own;
+          lds.frame[1] = own;
+          lds.shift[0] = 0.0f;
+          lds.shift[1] = 0.0f;
+        }
       } else {
-        const int idx = n + edge_shift;
-        if (idx >= 0 && idx < nblocks_up * kW) v = TakeEdge(edge_in + idx, hdr, kLogZero) + px_above;
+        own = lds.frame[kb & (kFrameRing - 1)];  // chosen by the chain two iterations ago
+      }
+    }
+    if (lane < kW) {
+      if (g.c == 0) {
+        v = n == 0 ? 0.0f : kLogZero;  // the origin: p[s_begin][t_begin] = 0 "arrives" at step 0
+      } else if (word) {
+        // (single launch) from the frame of the block above that the word lies in to this block's
+        if (kBidir) v = fmaxf(v, -1.0e36f) + ((idx / kW == up_taken ? up_frame_new : up_frame_old) - own);
+        v += px_above;
       }
       reinterpret_cast<float *>(lds.fx[kWave])[(kb % 3) * kW + lane] = v;
     }
   };
   // lanes 32..63: hand block kb of the last row to the chunk below.  Only words the chunk below
   // will take are published, so the buffer ends the launch clean.
+  const int down_hi = kBidir && has_down ? frames_hi(g.nblocks, nblocks_down) : -1;
   auto publish_block = [&](int kb) {
-    if (has_down && kb >= 0 && lane >= kW) {
+    if (has_down && kb >= 0) {
       const int n = kb * kW + (lane - kW);
-      // the chunk below takes word n at its step n - edge_shift, which must exist
-      if (n >= edge_shift && n - edge_shift < nblocks_down * kW)
-        PublishEdge(edge_out + n, reinterpret_cast<const float *>(
-                                      &lds.fy[kWave - 1][0])[(kb % 3) * kW + (lane - kW)]);
+      // the chunk below takes word n at its step n - edge_shift, which must exist; (single launch)
+      // lane 0 sends the block's frame along, in the same instruction
+      const bool word = lane >= kW && n >= edge_shift && n - edge_shift < nblocks_down * kW;
+      const bool frame = kBidir && lane == 0 && kb >= frames_lo() && kb <= down_hi;
+      if (word || frame)
+        PublishEdge(word ? edge_out + n : frame_out + kb,
+                    word ? reinterpret_cast<const float *>(&lds.fy[kWave - 1][0])[(kb % 3) * kW + (lane - kW)]
+                         : lds.frame[kb & (kFrameRing - 1)]);
     }
   };
 
@@ -901,7 +1130,9 @@ __device__ __forceinline__ void MiForwardChunk(
   auto chain_block = [&](int kb) {
     const int base = (kb % 3) * kQuadsPerBlock;
     P = fmaxf(P, -1.0e36f);  // lanes idling on the stand-in for -inf must never reach -inf itself
+    const float into_frame = kBidir ? frame_step(kb) : 0.0f;  // (0 for the chunk's first block)
     float4 nfx = lds.fx[fx_row][base], nfy = lds.fy[lane][base];
+    if (kBidir) P -= into_frame;  // into this block's frame (see Frames)
 #pragma unroll
     for (int k = 0; k < kQuadsPerBlock; ++k) {
       const float4 fx4 = nfx, fy4 = nfy;
@@ -914,7 +1145,7 @@ __device__ __forceinline__ void MiForwardChunk(
       float out[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        P = ChainStep(P, fxs[e], fys[e]);
+        P = kBidir ? ChainStep2(P, fxs[e], fys[e]) : ChainStep(P, fxs[e], fys[e]);
         out[e] = P;
       }
       lds.fy[lane][base + k] = make_float4(out[0], out[1], out[2], out[3]);
@@ -935,13 +1166,36 @@ __device__ __forceinline__ void MiForwardChunk(
   constexpr int kFwdSets = kBidir ? K2AMD_FWD_SETS : 2;
   FwdRegs sets[kFwdSets];
   if (role == kLoader) {
+    float gauge_v = 0.0f;
+    if (kBidir) {  // the gauge's sample, in the same trip to memory as block 0
+      // (a float that exists, for every lane: the tensor's first one where the lane has no sample)
+      const GFloat *src = !gauge_valid ? Global(px)
+                          : (lane & kGaugeSample) ? Global(py) + gauge_idx_y + (lane & (kGaugeSample - 1))
+                                                  : Global(px) + gauge_idx_x + (lane & (kGaugeSample - 1));
+      asm volatile("global_load_dword %0, %1, off" : "=v"(gauge_v) : "v"(src) : "memory");
+    }
     load_block(0, sets[0]);
     WaitLoads<0>(sets[0]);
+    if (kBidir) {
+      // (every load of this wavefront has landed; nothing reads the sample in front of this)
+      asm volatile("" : "+v"(gauge_v));
+      gauge = GaugeOf(gauge_v, gauge_valid, g.ns);
+      if (gauge_out != nullptr && mid == 0) {
+        PublishCut(gauge_out, gauge.x);
+        PublishCut(gauge_out + 1, gauge.y);
+      }
+    }
     commit_block(0, sets[0]);
     commit_above(0, sets[0]);
 #pragma unroll
     for (int i = 0; i < kFwdSets; ++i) load_block(1 + i, sets[i]);
   } else if (role == kEdge) {
+    if (kBidir && g.c > 0) {  // the same sample, the same arithmetic: the same gauge
+      const GFloat *src = (lane & kGaugeSample) ? Global(py) + gauge_idx_y : Global(px) + gauge_idx_x;
+      float v = 0.0f;
+      if (gauge_valid) v = src[lane & (kGaugeSample - 1)];
+      gauge = GaugeOf(v, gauge_valid, g.ns);
+    }
     take_block(0, edge_px(0));
   }
   K2AMD_TRACE_MARK(half, 4);
@@ -977,6 +1231,7 @@ __device__ __forceinline__ void MiForwardChunk(
   } else if (role == kStorer) {
     for (int kb = 0; kb < g.nblocks; ++kb) {
       store_block(kb - 1);
+      if (kBidir && wave == 2 + L::kLoaderWaves) choose_frame(kb);
       LdsBarrier();
     }
   } else if (role == kEdge) {
@@ -1000,6 +1255,7 @@ __device__ __forceinline__ void MiForwardChunk(
     const int at = ((g.nblocks - 1) % 3) * kW + (n_last - (g.nblocks - 1) * kW);
     const bool on_cut = half.dmax - g.row0 * g.skew == n_last && g.row0 + lane <= g.ns;
     PublishCut(cut_out + lane, on_cut ? reinterpret_cast<const float *>(&lds.fy[lane][0])[at] : kLogZero);
+    if (lane == 0) PublishCut(cut_frame_out, lds.frame[(g.nblocks - 1) & (kFrameRing - 1)]);
   }
   if (kBidir) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the coherent stores above
 }
@@ -1018,7 +1274,7 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiForwardFastKernel(
   MiForwardChunk<kKeep, kWriteP, false>(lds, px, py, LoadBox(boundary, (int)(ticket / nchunks), S, Tn), p,
                                         ans, log_deriv, hdr, edge, B, S, Tn, modified, nchunks,
                                         edge_stride, (int)(ticket / nchunks), (int)(ticket % nchunks),
-                                        Half{}, nullptr);
+                                        Half{}, nullptr, nullptr, nullptr);
   if (threadIdx.x == 0) PutTicketsBack(hdr, lds.ticket, gridDim.x);
 }
 
@@ -1247,7 +1503,7 @@ __device__ __forceinline__ void MiBackwardChunk(
   // p[src], px[src] (k2/python/csrc/torch/mutual_information_cpu.cu:195-211).
   auto flow = [&](float pd, float ps, float xs, float *e_out, float *o_out) {
     const float total = __builtin_isfinite(pd) ? pd : 0.0f;
-    const float d1 = __expf(kKept ? pd : (ps + xs) - total);
+    const float d1 = kBidir ? __builtin_amdgcn_exp2f(pd) : __expf(kKept ? pd : (ps + xs) - total);
     const bool fin = __builtin_isfinite(d1);
     *e_out = fin ? d1 : 0.0f;
     *o_out = fin ? 1.0f - d1 : 0.0f;
@@ -1483,7 +1739,7 @@ __device__ __forceinline__ void MiBackwardChunk(
     if (role == kChain) {
       float scale;
       K2AMD_TRACE_MARK(half, 7);
-      const float total = WaveCutJoin(sh, join->cw, g.ns, g.row0, mirror, hdr, &G, &scale);
+      const float total = WaveCutJoin(sh, join->cw, g.ns, modified ? g.nt - g.ns : g.nt, g.row0, mirror, hdr, &G, &scale);
       K2AMD_TRACE_MARK(half, 3);
       if (lane == 0) {
         const bool ok = total > kLogZeroTest;  // a finite score
@@ -1675,11 +1931,13 @@ struct TaskShared {
   Box box;
 };
 __device__ __attribute__((noinline)) void BidirForwardTask(FwdLds &lds, const TaskShared &t, int seq,
-                                                           int chunk, Half half, float *cut_out) {
+                                                           int chunk, Half half, float *cut_out,
+                                                           float *cut_frame_out, float *gauge_out) {
   const BidirArgs &k = t.k;
   MiForwardChunk<true, false, true>(lds, k.px, k.py, t.box, nullptr, k.ans, k.scratch, k.hdr,
                                     half.mirror ? k.edge1 : k.edge0, k.B, k.S, k.Tn, k.modified,
-                                    k.nchunks, k.edge_stride, seq, chunk, half, cut_out);
+                                    k.nchunks, k.edge_stride, seq, chunk, half, cut_out, cut_frame_out,
+                                    gauge_out);
 }
 // (what the join needs comes as arguments of its own: a structure handed over by address would
 // live in scratch memory, a trip there for every field the sweep reads)
@@ -1787,7 +2045,9 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiBidirKernel(const Bidir
     if (fwd) {
       if (!mirror && chunk == 0 && threadIdx.x == 0)
         PublishCut(cw.scale, k.ans_grad != nullptr ? k.ans_grad[seq] : 1.0f);
-      BidirForwardTask(lds.fwd, ts, seq, chunk, half, (mirror ? cw.beta : cw.alpha) + chunk * kRows);
+      BidirForwardTask(lds.fwd, ts, seq, chunk, half, (mirror ? cw.beta : cw.alpha) + chunk * kRows,
+                       (mirror ? cw.frame_beta : cw.frame_alpha) + chunk,
+                       !mirror && chunk == 0 ? cw.gauge : nullptr);
       // every wavefront has waited for its stores (device-coherent ones, see StoreQuadCoherent)
       // before this barrier: whichever compute unit sweeps this chunk back will see them
       __syncthreads();
@@ -1810,7 +2070,7 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiBidirKernel(const Bidir
       // which the last task to leave the sequence resets, and this task is among those.
       if (threadIdx.x < kWave) {
         float seed, scale = 0.0f;
-        const float total = box.ok ? WaveCutJoin(sh, cw, ns, 0, 0, k.hdr, &seed, &scale) : 0.0f;
+        const float total = box.ok ? WaveCutJoin(sh, cw, ns, k.modified ? nt - ns : nt, 0, 0, k.hdr, &seed, &scale) : 0.0f;
         if (threadIdx.x == 0) {
           sh.total = total;
           sh.scale = scale;
@@ -1864,8 +2124,8 @@ bool MiFastSupports(int B, int S, int Tn, int modified) {
 // the words of the cut of every sequence.
 size_t MiFastWorkspaceBytes(int B, int S, int Tn) {
   const int nchunks = (S + 1 + kRows - 1) / kRows;
-  const size_t edge_stride = ((size_t)Tn + 2 + kRows + kW + 3) / 4 * 4 + kW;
-  const size_t cut_words = kCutWordsPerSeqHeader + 2 * (size_t)nchunks * kRows;
+  const size_t edge_stride = EdgeStride(Tn);
+  const size_t cut_words = CutWordsPerSequence(nchunks);
   return sizeof(FastHeader) + (2 * (size_t)B * (nchunks + 1) * edge_stride + (size_t)B * cut_words) * sizeof(float);
 }
 
@@ -1912,7 +2172,7 @@ int MiForwardFast(const float *px, const float *py, const int64_t *boundary, flo
                   size_t workspace_bytes, hipStream_t stream) {
   if (workspace == nullptr || workspace_bytes < MiFastWorkspaceBytes(B, S, Tn)) return K2AMD_ERR_WORKSPACE;
   const int nchunks = (S + 1 + kRows - 1) / kRows;
-  const int edge_stride = (int)(((size_t)Tn + 2 + kRows + kW + 3) / 4 * 4 + kW);
+  const int edge_stride = EdgeStride(Tn);
   FastHeader *hdr = static_cast<FastHeader *>(workspace);
   float *edge = reinterpret_cast<float *>(hdr + 1);
   const dim3 grid((unsigned)(B * nchunks)), block(FwdLayout::kThreads);
@@ -1934,7 +2194,7 @@ int MiBackwardFast(const float *px, const float *p, const float *log_deriv,
                    hipStream_t stream) {
   if (workspace == nullptr || workspace_bytes < MiFastWorkspaceBytes(B, S, Tn)) return K2AMD_ERR_WORKSPACE;
   const int nchunks = (S + 1 + kRows - 1) / kRows;
-  const int edge_stride = (int)(((size_t)Tn + 2 + kRows + kW + 3) / 4 * 4 + kW);
+  const int edge_stride = EdgeStride(Tn);
   FastHeader *hdr = static_cast<FastHeader *>(workspace);
   float *edge = reinterpret_cast<float *>(hdr + 1);
   // B * nchunks sweeping workgroups + as many that only clear
@@ -1983,7 +2243,7 @@ int MiForwardBackwardFast(const float *px, const float *py, const int64_t *bound
   const int units = ComputeUnits();
   if (units <= 0) return K2AMD_ERR_LAUNCH;
   const int nchunks = (S + 1 + kRows - 1) / kRows;
-  const int edge_stride = (int)(((size_t)Tn + 2 + kRows + kW + 3) / 4 * 4 + kW);
+  const int edge_stride = EdgeStride(Tn);
   FastHeader *hdr = static_cast<FastHeader *>(workspace);
   float *edge0 = reinterpret_cast<float *>(hdr + 1);
   float *edge1 = edge0 + (size_t)B * (nchunks + 1) * edge_stride;

@@ -36,6 +36,10 @@ def mi_case(seed, dtype=np.float32, max_B=10, max_S=16, max_T=500, force=None):
     if force is not None:
         modified = bool(force.get("modified", modified))
         rand_bd = force.get("rand_bd", rand_bd)
+        big_px = force.get("big_px", big_px)
+        big_py = force.get("big_py", big_py)
+        random_px = force.get("random_px", random_px)
+        random_py = force.get("random_py", random_py)
     if modified and T < S:
         T = S + int(rng.integers(0, 31))
     T1 = T if modified else T + 1

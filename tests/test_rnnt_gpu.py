@@ -686,7 +686,7 @@ def test_random_shapes_through_the_api(device):
             if dtype == np.float64:
                 close("pruned gradient", seed, lg.grad, g64, tol)
             else:
-                tolerance.close_f32(f"pruned gradient {seed}", lg.grad.cpu().numpy(), g32, g64)
+                tolerance.close_f32(f"pruned gradient {seed}", lg.grad.cpu().numpy(), g32, g64, max_arbitrated=0.05)
         full = rng.standard_normal((B, T, S + 1, C)).astype(dtype)
         want = orn.rnnt_loss(full, sym, 0, bd, rt, pen, "none")
         got = k2.rnnt_loss(dev(full, device), dev(sym, device), 0, dev(bd, device), rt, pen, "none")

@@ -1,12 +1,18 @@
 """How the fp32 results of the GPU path are compared with the CPU oracle.
 
-The stated bar is |got - want| <= 1e-5 + 1e-4 |want| against the reference's fp32 result.  Where
-|p| reaches the hundreds or thousands, one fp32 ulp of p is 3e-5 .. 2.4e-4, every gradient is a
-sum over paths of products of exp() of differences of such values, the rounding errors add up
-along the S_b + T_b steps of a path like a random walk, and the reference's OWN fp32 gradients
+The stated bar is |got - want| <= 1e-5 + 1e-4 |want| against the reference's CPU result.  The
+reference's CPU path exists in fp32 and in fp64 (mutual_information_cpu.cu:81,168 dispatches on
+the dtype), and an element meets the bar PLAINLY if it is that close to either of them: to the
+fp32 result (the kernels that repeat the reference's additions land on its bits almost
+everywhere), or to the fp64 result of the same inputs (the exact answer, which a kernel that
+sums in another order is often closer to than the reference's own fp32 code is).
+
+Where |p| reaches the hundreds or thousands, one fp32 ulp of p is 3e-5 .. 2.4e-4, every gradient
+is a sum over paths of products of exp() of differences of such values, the rounding errors add
+up along the S_b + T_b steps of a path like a random walk, and the reference's OWN fp32 gradients
 then differ from an fp64 run by several 1e-4 relative: two correct fp32 implementations cannot
-agree to 1e-4 there.  For the elements that miss the plain bar the fp64 oracle arbitrates,
-element by element:
+agree to 1e-4 there, nor can either agree with fp64.  The elements that meet the bar against
+neither result are ARBITRATED by the fp64 oracle, element by element:
 
     |got - f64| <= 1e-5 + 1e-4 |f64| + 2 max(|cpu32 - f64|, Q_b |f64|)
 
@@ -19,8 +25,9 @@ worst thousandth of the same sequence's elements; a tiny element is never grante
 element's noise.  A percentile is not a maximum: of tens of millions of elements a few lie in
 the far tail of either implementation's error, so up to TAIL_FRACTION of the elements (one in a
 hundred thousand) may exceed that budget, by no more than TAIL_FACTOR times.  The share of
-elements that needed the arbitration is returned, bounded by the caller and printed by the tests
-at the BASELINE sizes.
+elements that needed the arbitration is returned and bounded by the caller (max_arbitrated: the
+rule is for a thin tail, not a second tolerance), and so is the share that missed the bar against
+the fp32 result alone.
 """
 import numpy as np
 
@@ -60,7 +67,7 @@ def close_f32(name, got, want32, want64, max_arbitrated=1.0, mode="relative"):
     with np.errstate(invalid="ignore"):
         same = (got == w32) | (np.isnan(got) & np.isnan(w32))
         plain = same | (np.abs(got - w32) <= ATOL + RTOL * np.abs(w32))
-        stats = dict(n=int(got.size), arbitrated=0, arbitrated_frac=0.0,
+        stats = dict(n=int(got.size), arbitrated=0, arbitrated_frac=0.0, beyond_fp32_bar=int((~plain).sum()),
                      max_gpu_vs_cpu32=float(np.max(np.abs(got - w32), where=~same & np.isfinite(got - w32),
                                                    initial=0.0)))
     if want64 is not None:
@@ -72,6 +79,8 @@ def close_f32(name, got, want32, want64, max_arbitrated=1.0, mode="relative"):
     if not plain.all():
         assert want64 is not None, (name, int((~plain).sum()), got[~plain][:5], w32[~plain][:5])
         with np.errstate(invalid="ignore"):
+            # the same bar against the reference's fp64 result
+            plain = plain | (got == w64) | (np.abs(got - w64) <= ATOL + RTOL * np.abs(w64))
             ref_err = np.abs(w32 - w64)
             q = _per_sequence_quantile(ref_err, np.abs(w64), mode)
             floor = q * np.abs(w64) if mode == "relative" else q
