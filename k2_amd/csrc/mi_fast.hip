@@ -401,7 +401,9 @@ __global__ void FastWsInitKernel(FastHeader *hdr, unsigned *edge, size_t n) {
   for (size_t k = i; k < n; k += (size_t)gridDim.x * blockDim.x) edge[k] = kSentinel;
 }
 
-// Waits for one published word, takes it and leaves the sentinel behind.
+// Waits for one published word, takes it and leaves the sentinel behind.  One poll in flight at
+// a time: several polls of the same word a quarter of a trip apart (so that it is looked at more
+// often than once per trip) made every hand-over slower, not faster (a launch of 56 us took 70).
 __device__ __forceinline__ float TakeEdge(float *addr, FastHeader *hdr, float on_timeout) {
   unsigned *word = reinterpret_cast<unsigned *>(addr);
   int spins = 0;
@@ -1210,6 +1212,9 @@ __device__ __forceinline__ void MiForwardChunk(
   if (role == kChain) {
     for (int kb = 0; kb < g.nblocks; ++kb) {
       chain_block(kb);
+#ifdef K2AMD_MI_TRACE
+      if (kBidir && kb < 24) K2AMD_TRACE_MARK(half, 8 + kb);
+#endif
       LdsBarrier();
     }
   } else if (role == kLoader) {
@@ -1892,7 +1897,7 @@ __global__ __launch_bounds__(BwdLayout::kThreads) void MiBackwardFastKernel(
 //
 // Work is handed out as TASKS through the ticket counter to a fixed set of persistent workgroups
 // (one per compute unit): first the forward sweeps of all (sequence, half, 64-row chunk), then the
-// clearing of what lies outside the boxes, then the backward sweeps, then one task per sequence
+// backward sweeps, then the clearing of what lies outside the boxes, then one task per sequence
 // for the lattices the split cannot serve.  A task only ever waits for tasks with EARLIER
 // tickets (a chunk's producer; for the backward sweeps and the last kind of task, all forward
 // sweeps of the sequence), and a ticket is only taken by a workgroup that is running, so the
@@ -1995,8 +2000,14 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiBidirKernel(const Bidir
   auto box_of = [&](int seq) { return seq < kBoxes ? boxes[seq] : LoadBox(k.boundary, seq, k.S, k.Tn); };
   const int nchunks = k.nchunks;
   const unsigned per_seq = 2u * nchunks, nsweep = (unsigned)k.B * per_seq;
-  const unsigned first_clear = nsweep, first_bwd = first_clear + (unsigned)k.B * nchunks;
-  const unsigned first_last = first_bwd + nsweep, ntasks = first_last + (unsigned)k.B;
+  // Tickets: the forward half-sweeps, the backward half-sweeps, the clearing of what lies outside
+  // the boxes, one last task per sequence.  (The clearing writes a fifth as many bytes as the
+  // sweeps move, and placed between the two kinds of sweeps, where workgroups whose forward
+  // sweeps end early are free for it, it slowed the long sequences' forward sweeps down while
+  // their inputs come from HBM: 56.5 us per launch against 54.1 with the clearing behind the
+  // backward sweeps, drawn by workgroups whose backward sweeps end early.)
+  const unsigned first_bwd = nsweep, first_clear = first_bwd + nsweep;
+  const unsigned first_last = first_clear + (unsigned)k.B * nchunks, ntasks = first_last + (unsigned)k.B;
   const int skew = k.modified ? 0 : 1;
   for (bool first = true;; first = false) {
     if (!first) {
@@ -2011,11 +2022,11 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiBidirKernel(const Bidir
       unsigned long long *at;
       __device__ void mark(int i) { if (at != nullptr && threadIdx.x == 0) at[i] = wall_clock64(); }
       __device__ ~Tracer() { mark(2); }
-    } tracer{k.trace != nullptr ? k.trace + 8 * (size_t)ticket : nullptr};
+    } tracer{k.trace != nullptr ? k.trace + 32 * (size_t)ticket : nullptr};
     tracer.mark(0);
 #endif
 
-    if (ticket >= first_clear && ticket < first_bwd) {  // what no sweep assigns
+    if (ticket >= first_clear && ticket < first_last) {  // what no sweep assigns
       const unsigned unit = ticket - first_clear;
       if (threadIdx.x == 0) ts.box = box_of((int)(unit / nchunks));
       __syncthreads();
@@ -2023,7 +2034,7 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiBidirKernel(const Bidir
       continue;
     }
 
-    const bool fwd = ticket < first_clear, last = ticket >= first_last;
+    const bool fwd = ticket < first_bwd, last = ticket >= first_last;
     const unsigned unit = fwd ? ticket : (last ? 0u : ticket - first_bwd);
     const int seq = last ? (int)(ticket - first_last) : (int)(unit / per_seq);
     const int mirror = last ? 0 : (int)((unit % per_seq) / nchunks);
@@ -2038,7 +2049,7 @@ __global__ __launch_bounds__(FwdLayout::kThreads) void MiBidirKernel(const Bidir
     half.mirror = mirror;
     half.dmax = mirror ? diagonals - dcut : dcut;
 #ifdef K2AMD_MI_TRACE
-    half.trace = k.trace != nullptr ? k.trace + 8 * (size_t)ticket : nullptr;
+    half.trace = k.trace != nullptr ? k.trace + 32 * (size_t)ticket : nullptr;
 #endif
     const CutWords cw = CutOf(k.cut, seq, nchunks);
 
