@@ -151,6 +151,35 @@ def mi(px, py, boundary=None, backend="port"):
     return ans, gx, gy
 
 
+def joint_mi(pxs, pys, boundary=None, backend="port"):
+    """k2.joint_mutual_information_recursion (k2/python/k2/mutual_information.py:314-423): the
+    recursion on the sums of the N px and N py, and the split of its score over the inputs,
+    prods[n][b] = <occupation of the px edges, px_n> + <occupation of the py edges, py_n> with
+    -inf inputs clamped to the dtype's most negative finite number, the rest of the score added to
+    prods[0].  Returns (prods[N][B], px_occupation, py_occupation): the gradient of
+    sum(w * prods) to px_n is w[n][b] times the occupation wherever px_n is above that clamp, the
+    score itself carrying no gradient in the reference (it is computed outside autograd)."""
+    N = len(pxs)
+    assert len(pys) == N and N > 0
+    dtype = np.asarray(pxs[0]).dtype
+    px_tot = np.zeros_like(np.asarray(pxs[0]))
+    py_tot = np.zeros_like(np.asarray(pys[0]))
+    for n in range(N):  # torch.stack(...).sum(dim=0) adds the inputs in their order
+        px_tot = px_tot + np.asarray(pxs[n], dtype=dtype)
+        py_tot = py_tot + np.asarray(pys[n], dtype=dtype)
+    tot, gx, gy = mi(px_tot, py_tot, boundary, backend=backend)
+    lo = np.finfo(dtype).min
+    B = px_tot.shape[0]
+    prods = np.zeros((N, B), dtype=dtype)
+    for n in range(N):
+        cx = np.maximum(np.asarray(pxs[n], dtype=dtype), lo).reshape(B, -1)
+        cy = np.maximum(np.asarray(pys[n], dtype=dtype), lo).reshape(B, -1)
+        prods[n] = (np.einsum("bk,bk->b", gx.reshape(B, -1).astype(np.float64), cx.astype(np.float64)) +
+                    np.einsum("bk,bk->b", gy.reshape(B, -1).astype(np.float64), cy.astype(np.float64))).astype(dtype)
+    prods[0] += tot - prods.sum(axis=0)
+    return prods, gx, gy
+
+
 def log_add(x, y, dtype=np.float32):
     lib = port_lib()
     if dtype == np.float32:

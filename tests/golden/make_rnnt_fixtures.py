@@ -97,7 +97,7 @@ class Recorder:
 
 def main():
     omi.build_ref()
-    rl, _ = _load_reference()
+    rl, mi = _load_reference()
     rec = Recorder()
     torch.manual_seed(0)
     torch.set_num_threads(1)
@@ -208,6 +208,81 @@ def main():
                                       rnnt_type=rt, boundary=boundary)
         rec.add(name, am=am, lm=lm, symbols=symbols, boundary=boundary, rnnt_type=np.array(rt),
                 px=px, py=py)
+
+    # ---- joint_mutual_information_recursion: the split over the inputs and its gradients --------
+    joint = [
+        # name,     N, B, S,  T, modified, boundary
+        ("joint0", 1, 2, 5, 9, False, False),
+        ("joint1", 2, 3, 7, 12, False, True),
+        ("joint2", 3, 2, 6, 15, True, True),
+        ("joint3", 2, 2, 70, 90, True, True),     # two chunks of rows
+        ("joint4", 3, 2, 9, 40, False, False),
+        ("joint5", 2, 3, 4, 4, True, False),
+    ]
+    for seed, (name, N, B, S, T, modified, wb) in enumerate(joint):
+        rng = np.random.default_rng(400 + seed)
+        T1 = T if modified else T + 1
+        pxs = [torch.from_numpy(rng.normal(-1.0, 1.0, (B, S, T1)).astype(np.float32)).requires_grad_(True)
+               for _ in range(N)]
+        pys = [torch.from_numpy(rng.normal(-1.0, 1.0, (B, S + 1, T)).astype(np.float32)).requires_grad_(True)
+               for _ in range(N)]
+        if not modified and not wb:
+            with torch.no_grad():
+                pxs[0][:, :, -1] = -np.inf   # the reference's convention for the last column
+        boundary = None
+        if wb:
+            rows = []
+            for _ in range(B):
+                s_len = int(rng.integers(S // 2, S + 1))
+                t_len = int(rng.integers(max(T // 2, s_len), T + 1))
+                s0 = int(rng.integers(0, S - s_len + 1))
+                t0 = int(rng.integers(0, T - t_len + 1))
+                rows.append([s0, t0, s0 + s_len, t0 + t_len])
+            boundary = torch.tensor(rows, dtype=torch.int64)
+        prods = mi.joint_mutual_information_recursion(px=pxs, py=pys, boundary=boundary)
+        w = torch.from_numpy(rng.uniform(0.5, 1.5, (N, B)).astype(np.float32))
+        (prods * w).sum().backward()
+        arrays = dict(boundary=boundary, modified=np.array(modified), weights=w, prods=prods,
+                      n=np.array(N))
+        for i in range(N):
+            arrays[f"px{i}"] = pxs[i]
+            arrays[f"py{i}"] = pys[i]
+            arrays[f"px{i}_grad"] = pxs[i].grad
+            arrays[f"py{i}_grad"] = pys[i].grad
+        rec.add(name, **arrays)
+
+    # ---- gradients of the smoothed and of the HAT pruned loss to the network outputs -------------
+    variants = [
+        # name,    B, T,  S, C, rnnt_type,     R, lm_only, am_only
+        ("grad0", 2, 17, 5, 7, "regular", 3, 0.25, 0.0),
+        ("grad1", 2, 23, 6, 9, "modified", 4, 0.0, 0.3),
+        ("grad2", 3, 30, 8, 8, "regular", 5, 0.2, 0.1),
+        ("grad3", 2, 20, 6, 6, "constrained", 3, 0.15, 0.25),
+    ]
+    for seed, (name, B, T, S, C, rt, R, lm_only, am_only) in enumerate(variants):
+        rng = np.random.default_rng(500 + seed)
+        am, lm, symbols, boundary = _inputs(rng, B, T, S, C, np.float32, True, rt != "regular",
+                                            max(T // 2, S), S // 2)
+        w = torch.from_numpy(rng.uniform(0.5, 1.5, B).astype(np.float32))
+        am_g = am.clone().requires_grad_(True)
+        lm_g = lm.clone().requires_grad_(True)
+        smoothed = rl.rnnt_loss_smoothed(lm=lm_g, am=am_g, symbols=symbols, termination_symbol=0,
+                                         lm_only_scale=lm_only, am_only_scale=am_only,
+                                         boundary=boundary, rnnt_type=rt, reduction="none")
+        (smoothed * w).sum().backward()
+        _, (gx, gy) = rl.rnnt_loss_simple(lm=lm, am=am, symbols=symbols, termination_symbol=0,
+                                          boundary=boundary, rnnt_type=rt, reduction="none",
+                                          return_grad=True)
+        ranges = rl.get_rnnt_prune_ranges(px_grad=gx, py_grad=gy, boundary=boundary, s_range=R)
+        am_p, lm_p = rl.do_rnnt_pruning(am=am, lm=lm, ranges=ranges)
+        logits = (am_p + lm_p).clone().requires_grad_(True)
+        hat = rl.rnnt_loss_pruned(logits=logits, symbols=symbols, ranges=ranges, termination_symbol=0,
+                                  boundary=boundary, rnnt_type=rt, reduction="none", use_hat_loss=True)
+        (hat * w).sum().backward()
+        rec.add(name, am=am, lm=lm, symbols=symbols, boundary=boundary, rnnt_type=np.array(rt),
+                weights=w, lm_only_scale=np.array(lm_only), am_only_scale=np.array(am_only),
+                smoothed_loss=smoothed, smoothed_am_grad=am_g.grad, smoothed_lm_grad=lm_g.grad,
+                ranges=ranges, hat_logits=logits.detach(), hat_loss=hat, hat_logits_grad=logits.grad)
 
     rec.out["names"] = np.array(rec.names)
     rec.out["torch_version"] = np.array(torch.__version__)

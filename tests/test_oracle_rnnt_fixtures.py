@@ -175,3 +175,35 @@ def test_delay_penalty_by_brute_force(rnnt_type, with_boundary):
         t = np.arange(gx.shape[2])
         expected = -(gx[b] * ((T_b - 1) / 2 - t)[None, :]).sum()
         assert (a[b] - b0[b]) / eps == pytest.approx(expected, rel=1e-4, abs=1e-6)
+
+
+@pytest.mark.parametrize("name", [f"joint{i}" for i in range(6)])
+def test_joint_recursion_matches_the_reference(fx, name):
+    """oracle.mi.joint_mi against k2.joint_mutual_information_recursion's recorded split and the
+    gradients torch's autograd gave for it (k2/python/k2/mutual_information.py:314-423)."""
+    from oracle import mi as omi
+    N = int(fx.get(name, "n"))
+    pxs = [fx.get(name, f"px{i}") for i in range(N)]
+    pys = [fx.get(name, f"py{i}") for i in range(N)]
+    prods, gx, gy = omi.joint_mi(pxs, pys, fx.get(name, "boundary"))
+    # the elements are differences of sums of hundreds of terms: absolute tolerance scaled by the
+    # size of the terms' sum
+    np.testing.assert_allclose(prods, fx.get(name, "prods"), rtol=1e-4, atol=1e-4)
+    w = fx.get(name, "weights")
+    lo = np.finfo(np.float32).min
+    for i in range(N):
+        np.testing.assert_allclose(np.where(pxs[i] > lo, w[i][:, None, None] * gx, 0.0), fx.get(name, f"px{i}_grad"), **F32)
+        np.testing.assert_allclose(np.where(pys[i] > lo, w[i][:, None, None] * gy, 0.0), fx.get(name, f"py{i}_grad"), **F32)
+
+
+@pytest.mark.parametrize("name", [f"grad{i}" for i in range(4)])
+def test_smoothed_and_hat_losses_of_the_gradient_cases(fx, name):
+    am, lm, sym, bd = (fx.get(name, k) for k in ("am", "lm", "symbols", "boundary"))
+    rt = str(fx.get(name, "rnnt_type"))
+    np.testing.assert_allclose(
+        orn.rnnt_loss_smoothed(lm, am, sym, 0, float(fx.get(name, "lm_only_scale")),
+                               float(fx.get(name, "am_only_scale")), bd, rt, 0.0, "none"),
+        fx.get(name, "smoothed_loss"), **F32)
+    np.testing.assert_allclose(
+        orn.rnnt_loss_pruned(fx.get(name, "hat_logits"), sym, fx.get(name, "ranges"), 0, bd, rt, 0.0, "none", True),
+        fx.get(name, "hat_loss"), **F32)

@@ -900,3 +900,68 @@ def test_reference_logprobs_where_the_shifted_exponentials_underflow(device):
         fin = np.isfinite(want_px)
         np.testing.assert_allclose(px[fin], want_px[fin], rtol=1e-4, atol=1e-5, err_msg=name)
         np.testing.assert_allclose(py, want_py, rtol=1e-4, atol=1e-5, err_msg=name)
+
+
+def test_reference_joint_recursion_fixtures(device):
+    """joint_mutual_information_recursion (k2/python/k2/mutual_information.py:314-423) on inputs
+    recorded with the reference's own outputs: the split of the score over N = 1, 2, 3 pairs of
+    inputs, and the gradient of a weighted sum of its elements to every input."""
+    import k2_amd as k2
+    names, get = _fixtures()
+    tol = dict(rtol=1e-4, atol=1e-5)
+    seen = 0
+    for name in names:
+        if not name.startswith("joint"):
+            continue
+        seen += 1
+        N = int(get(name, "n"))
+        bd = dev(get(name, "boundary"), device)
+        pxs = [dev(get(name, f"px{i}"), device).requires_grad_(True) for i in range(N)]
+        pys = [dev(get(name, f"py{i}"), device).requires_grad_(True) for i in range(N)]
+        prods = k2.joint_mutual_information_recursion(pxs, pys, bd)
+        assert tuple(prods.shape) == get(name, "prods").shape, name
+        np.testing.assert_allclose(prods.detach().cpu().numpy(), get(name, "prods"), err_msg=name, **tol)
+        w = get(name, "weights")
+        (prods * dev(w, device)).sum().backward()
+        # the gradients are weighted occupation probabilities: where an element misses the plain
+        # bar against the reference's fp32 result the fp64 oracle arbitrates (tolerance.py)
+        _, gx64, gy64 = omi.joint_mi([get(name, f"px{i}").astype(np.float64) for i in range(N)],
+                                     [get(name, f"py{i}").astype(np.float64) for i in range(N)], get(name, "boundary"))
+        lo = np.finfo(np.float32).min
+        for i in range(N):
+            for what, t, occ in (("px", pxs[i], gx64), ("py", pys[i], gy64)):
+                want = get(name, f"{what}{i}_grad")
+                want64 = np.where(get(name, f"{what}{i}") > lo, w[i].astype(np.float64)[:, None, None] * occ, 0.0)
+                tolerance.close_f32(f"{name} {what}{i}.grad", t.grad.cpu().numpy(), want, want64, max_arbitrated=0.01)
+    assert seen >= 6
+
+
+def test_reference_smoothed_and_hat_gradient_fixtures(device):
+    """The gradients of rnnt_loss_smoothed to lm / am and of rnnt_loss_pruned(use_hat_loss=True) to
+    the logits (k2/python/k2/rnnt_loss.py:1471-1829, 992-1177), against what the reference's chain
+    and torch's autograd gave on the same inputs."""
+    import k2_amd as k2
+    names, get = _fixtures()
+    tol = dict(rtol=1e-4, atol=1e-5)
+    seen = 0
+    for name in names:
+        if not name.startswith("grad"):
+            continue
+        seen += 1
+        rt = str(get(name, "rnnt_type"))
+        sym_d, bd_d, w = dev(get(name, "symbols"), device), dev(get(name, "boundary"), device), dev(get(name, "weights"), device)
+        lm_d = dev(get(name, "lm"), device).requires_grad_(True)
+        am_d = dev(get(name, "am"), device).requires_grad_(True)
+        smoothed = k2.rnnt_loss_smoothed(lm_d, am_d, sym_d, 0, float(get(name, "lm_only_scale")),
+                                         float(get(name, "am_only_scale")), bd_d, rt, 0.0, "none")
+        (smoothed * w).sum().backward()
+        np.testing.assert_allclose(smoothed.detach().cpu().numpy(), get(name, "smoothed_loss"), err_msg=name, **tol)
+        np.testing.assert_allclose(lm_d.grad.cpu().numpy(), get(name, "smoothed_lm_grad"), err_msg=name, **tol)
+        np.testing.assert_allclose(am_d.grad.cpu().numpy(), get(name, "smoothed_am_grad"), err_msg=name, **tol)
+        logits = dev(get(name, "hat_logits"), device).requires_grad_(True)
+        ranges = dev(get(name, "ranges"), device)
+        hat = k2.rnnt_loss_pruned(logits, sym_d, ranges, 0, bd_d, rt, 0.0, "none", use_hat_loss=True)
+        (hat * w).sum().backward()
+        np.testing.assert_allclose(hat.detach().cpu().numpy(), get(name, "hat_loss"), err_msg=name, **tol)
+        np.testing.assert_allclose(logits.grad.cpu().numpy(), get(name, "hat_logits_grad"), err_msg=name, **tol)
+    assert seen >= 4
