@@ -64,6 +64,14 @@ K2AMD_API int k2amd_mi_workspace_init(void *workspace, size_t workspace_bytes, v
  * are those of every later call until the workspace is initialised again; the kernels make that
  * visible without this call by writing NaN to ans (and to the ans_grad they hand back). */
 K2AMD_API int k2amd_mi_workspace_status(const void *workspace, void *stream);
+/* The same question without the wait: queues, on `stream`, a copy of the workspace's error flag
+ * into *host_flag (4 bytes of pinned host memory that must stay valid until the stream has passed
+ * this point) and returns at once.  Once the stream has passed it, *host_flag != 0 says what
+ * K2AMD_ERR_TIMEOUT says above.  For hosts that wait on the stream anyway (the reference's Python
+ * layer reads `boundary` on the host in every call, k2/python/k2/mutual_information.py:287): the
+ * flag rides along with that read, and a launch that gave up is reported at the caller's next
+ * call instead of as NaN scores from then on.  No counterpart in the reference. */
+K2AMD_API int k2amd_mi_workspace_status_async(const void *workspace, unsigned *host_flag, void *stream);
 
 /* Replaces _k2.mutual_information_forward (k2/python/csrc/torch/mutual_information.cu:26-44,
  * CPU semantics of k2/python/csrc/torch/mutual_information_cpu.cu:50-124):

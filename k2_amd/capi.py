@@ -28,6 +28,7 @@ _SIGNATURES = {
     "k2amd_mi_workspace_bytes": ([_ci, _ci, _ci, _ci, _ci], _sz),
     "k2amd_mi_workspace_init": ([_vp, _sz, _vp], _ci),
     "k2amd_mi_workspace_status": ([_vp, _vp], _ci),
+    "k2amd_mi_workspace_status_async": ([_vp, _vp, _vp], _ci),
     "k2amd_mi_forward": ([_vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp, _sz, _vp], _ci),
     "k2amd_mi_forward_noalloc": ([_vp] * 5 + [_ci] * 5 + [_vp], _ci),
     "k2amd_mi_backward": ([_vp, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci,

@@ -90,6 +90,15 @@ int k2amd_mi_workspace_status(const void *workspace, void *stream) {
   return header[2] != 0 ? K2AMD_ERR_TIMEOUT : K2AMD_OK;  // FastHeader::error
 }
 
+int k2amd_mi_workspace_status_async(const void *workspace, unsigned *host_flag, void *stream) {
+  if (workspace == nullptr || host_flag == nullptr) return K2AMD_ERR_INVALID_ARGUMENT;
+  // FastHeader::error is the third word of the buffer
+  if (hipMemcpyAsync(host_flag, static_cast<const unsigned *>(workspace) + 2, sizeof(unsigned),
+                     hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream)) != hipSuccess)
+    return K2AMD_ERR_LAUNCH;
+  return K2AMD_OK;
+}
+
 int k2amd_mi_keeps_log_deriv(int B, int S, int T, int modified, int dtype, int has_workspace) {
   return dtype == K2AMD_F32 && has_workspace && ShapeOk(B, S, T) && B > 0 && !ForceGeneric() &&
          MiFastSupports(B, S, T, modified ? 1 : 0);

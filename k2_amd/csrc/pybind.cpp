@@ -42,6 +42,13 @@ struct WorkspaceCache {
   std::mutex mu;
   std::map<std::pair<int, void *>, torch::Tensor> bufs;
 
+  // the buffer of (device, stream) if there is one
+  torch::Tensor Find(const torch::Device &dev, void *stream) {
+    std::lock_guard<std::mutex> lock(mu);
+    auto it = bufs.find(std::make_pair(static_cast<int>(dev.index()), stream));
+    return it == bufs.end() ? torch::Tensor() : it->second;
+  }
+
   torch::Tensor Get(size_t bytes, const torch::Device &dev, void *stream) {
     if (bytes == 0) return torch::Tensor();
     std::lock_guard<std::mutex> lock(mu);
@@ -79,6 +86,17 @@ int64_t MutualInformationRecoverWorkspaces() {
     }
   }
   return recovered;
+}
+
+// The buffer that the pipelined kernels use on `like`'s device and current stream, or None where
+// no call has needed one yet (for diagnostics and for tests that force its error flag from the
+// host).  No counterpart in the reference.
+pybind11::object MutualInformationWorkspace(const torch::Tensor &like) {
+  TORCH_CHECK(like.is_cuda(), "k2_amd: a device tensor names the device");
+  void *stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(like.device().index()).stream();
+  torch::Tensor ws = Cache().Find(like.device(), stream);
+  if (!ws.defined()) return pybind11::none();
+  return pybind11::cast(ws);
 }
 
 WorkspaceCache &Cache() {
@@ -693,6 +711,10 @@ torch::Tensor MutualInformationJointProducts(std::vector<torch::Tensor> px, std:
 // memory on the tensor's current stream and an event behind it.  Rows() waits for that event
 // alone (not for what was queued after the copy) and returns the rows as tuples of Python
 // integers, what k2's range asserts read (k2/python/k2/mutual_information.py:284-289).
+// The error flag of the stream's workspace for the pipelined kernels rides along: a launch that
+// gave up a bounded wait (its scores came out as NaN, and so would those of every later launch on
+// that workspace) is reported here, at the caller's next call, as a RuntimeError, and the
+// workspace is initialised again so that the call after that one works.
 class BoundaryRead {
  public:
   explicit BoundaryRead(const torch::Tensor &boundary) {
@@ -700,14 +722,31 @@ class BoundaryRead {
                     boundary.scalar_type() == torch::kLong,
                 "boundary must be a [B][4] int64 tensor on the device");
     c10::hip::HIPGuardMasqueradingAsCUDA guard(boundary.device());
+    auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(boundary.device().index());
     pinned_ = torch::empty(boundary.sizes(), torch::TensorOptions().dtype(torch::kLong).pinned_memory(true));
     pinned_.copy_(boundary, /*non_blocking=*/true);
-    event_.record(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(boundary.device().index()));
+    stream_ = stream.stream();
+    workspace_ = Cache().Find(boundary.device(), stream_);
+    if (workspace_.defined()) {
+      flag_ = torch::zeros({1}, torch::TensorOptions().dtype(torch::kInt).pinned_memory(true));
+      Check(k2amd_mi_workspace_status_async(workspace_.data_ptr(),
+                                            reinterpret_cast<unsigned *>(flag_.data_ptr<int>()), stream_));
+    }
+    event_.record(stream);
   }
   pybind11::tuple Rows() {
     {
       pybind11::gil_scoped_release release;
       event_.synchronize();
+    }
+    if (flag_.defined() && flag_.data_ptr<int>()[0] != 0) {
+      flag_.data_ptr<int>()[0] = 0;  // (reported once)
+      c10::hip::HIPGuardMasqueradingAsCUDA guard(workspace_.device());
+      Check(k2amd_mi_workspace_init(workspace_.data_ptr(), static_cast<size_t>(workspace_.numel()), stream_));
+      TORCH_CHECK(false, "k2_amd: ", k2amd_status_string(K2AMD_ERR_TIMEOUT),
+                  ": an earlier launch of the mutual-information kernels on this stream gave up waiting for a "
+                  "neighbouring workgroup, so its scores and gradients (NaN) are invalid; the workspace has "
+                  "been initialised again, the next call will work");
     }
     const int64_t B = pinned_.size(0);
     const int64_t *v = pinned_.data_ptr<int64_t>();
@@ -718,7 +757,8 @@ class BoundaryRead {
   }
 
  private:
-  torch::Tensor pinned_;
+  torch::Tensor pinned_, flag_, workspace_;
+  void *stream_ = nullptr;
   at::cuda::CUDAEvent event_;
 };
 
@@ -731,6 +771,7 @@ PYBIND11_MODULE(_k2_amd, m) {
         pybind11::arg("py"), pybind11::arg("boundary"), pybind11::arg("p"),
         pybind11::arg("log_deriv") = pybind11::none());
   m.def("mutual_information_recover_workspaces", &MutualInformationRecoverWorkspaces);
+  m.def("mutual_information_workspace", &MutualInformationWorkspace, pybind11::arg("like"));
   m.def("mutual_information_joint_products", &MutualInformationJointProducts, pybind11::arg("px"),
         pybind11::arg("py"), pybind11::arg("px_grad"), pybind11::arg("py_grad"));
   m.def("mutual_information_keeps_log_deriv", &MutualInformationKeepsLogDeriv, pybind11::arg("px"),

@@ -31,6 +31,10 @@ def boundary_rows(boundary: Tensor) -> Tuple[Tuple[int, int, int, int], ...]:
     early = _boundary_reads.pop(ident, None)
     if early is not None and early[0]() is boundary and early[1] == boundary._version:
         rows = early[2].rows()  # waits for the copy alone, not for what was queued after it
+    elif boundary.is_cuda and boundary.dtype == torch.int64 and boundary.dim() == 2 and boundary.shape[1] == 4:
+        # the same read, begun and waited for here: what rides along with it (the error flag of the
+        # stream's workspace, native.boundary_read) is looked at in every call that reads a boundary
+        rows = native.boundary_read(boundary).rows()
     else:
         rows = tuple(tuple(r) for r in boundary.tolist())
     _boundary_copies[ident] = (weakref.ref(boundary, lambda _, i=ident: _boundary_copies.pop(i, None)),

@@ -23,16 +23,37 @@ def _require_device(t: torch.Tensor):
 
 
 class _BoundaryRead:
-    """The host layer's BoundaryRead with torch's Python API, where the extension is not built."""
+    """The host layer's BoundaryRead with torch's Python API, where the extension is not built:
+    the copy of ``boundary`` to the host, and with it the error flag of the stream's workspace
+    (a launch that gave up a bounded wait is reported by ``rows()`` as a RuntimeError, once, and
+    the workspace initialised again)."""
 
     def __init__(self, boundary: torch.Tensor):
         self.pinned = torch.empty(boundary.shape, dtype=boundary.dtype, pin_memory=True)
         self.pinned.copy_(boundary, non_blocking=True)
+        stream = torch.cuda.current_stream(boundary.device)
+        self.key = (boundary.device.index, stream.cuda_stream)
+        self.workspace = capi._workspaces.get(self.key)
+        self.flag = None
+        if self.workspace is not None:
+            self.flag = torch.zeros(1, dtype=torch.int32, pin_memory=True)
+            with torch.cuda.device(boundary.device):
+                capi.check(capi.lib().k2amd_mi_workspace_status_async(
+                    self.workspace.data_ptr(), self.flag.data_ptr(), self.key[1]))
         self.event = torch.cuda.Event()
-        self.event.record(torch.cuda.current_stream(boundary.device))
+        self.event.record(stream)
 
     def rows(self):
         self.event.synchronize()  # the copy alone, not what was queued after it
+        if self.flag is not None and int(self.flag[0]) != 0:
+            self.flag[0] = 0
+            with torch.cuda.device(self.key[0]):
+                capi.check(capi.lib().k2amd_mi_workspace_init(self.workspace.data_ptr(), self.workspace.numel(),
+                                                              self.key[1]))
+            raise RuntimeError(
+                "k2_amd: in-kernel wait timed out: an earlier launch of the mutual-information kernels on this "
+                "stream gave up waiting for a neighbouring workgroup, so its scores and gradients (NaN) are "
+                "invalid; the workspace has been initialised again, the next call will work")
         return tuple(tuple(r) for r in self.pinned.tolist())
 
 

@@ -622,6 +622,39 @@ def test_a_wait_that_gave_up_is_loud(device):
     assert native.mutual_information_recover_workspaces() == 0
 
 
+@pytest.mark.parametrize("host", ["extension", "ctypes"])
+def test_a_wait_that_gave_up_raises_at_the_next_call(device, host, monkeypatch):
+    """Through the API: after a launch whose bounded wait expired (the flag is forced from the
+    host, so every kernel ends normally), the NEXT call that reads its boundary raises a
+    RuntimeError that names the timeout, without a status call by the user, and the call after
+    that one works again: no NaN is handed on silently.  Both host layers."""
+    import k2_amd as k2
+    from k2_amd import capi, native
+    if host == "ctypes":
+        monkeypatch.setattr(native, "_ext", None)
+    elif native._ext is None:
+        pytest.skip("the C++ host module is not built")
+    rng = np.random.default_rng(19)
+    B, S, T = 3, 90, 120
+    px = torch.from_numpy(rng.normal(-2, 1, (B, S, T + 1)).astype(np.float32)).to(device)
+    py = torch.from_numpy(rng.normal(-2, 1, (B, S + 1, T)).astype(np.float32)).to(device)
+    bd = torch.tensor([[0, 0, S, T], [1, 2, 80, 100], [0, 0, 64, 64]], dtype=torch.int64, device=device)
+    good, (gx, gy) = k2.mutual_information_recursion(px, py, bd.clone(), return_grad=True)
+    assert torch.isfinite(good).all()
+    if host == "ctypes":
+        ws = capi._workspaces[(px.device.index, torch.cuda.current_stream(device).cuda_stream)]
+    else:
+        ws = native._ext.mutual_information_workspace(px)
+    assert ws is not None
+    torch.cuda.synchronize(device)
+    ws[:16].view(torch.int32)[2] = 1                         # FastHeader::error
+    with pytest.raises(RuntimeError, match="timed out"):
+        k2.mutual_information_recursion(px, py, bd.clone(), return_grad=True)
+    again, (gx2, gy2) = k2.mutual_information_recursion(px, py, bd.clone(), return_grad=True)
+    assert torch.equal(again, good) and torch.equal(gx2, gx) and torch.equal(gy2, gy)
+    assert native.mutual_information_recover_workspaces() == 0
+
+
 def test_single_launches_on_two_streams(device):
     """Two streams issue the single launch at the same time, each with its own workspace.  The
     clearing workgroups of a launch never wait and leave, so what must be resident together is
