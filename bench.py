@@ -35,6 +35,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # reads px, p and writes px_grad, py_grad (16 B; the backward never needs py).
 FWD_BYTES_PER_CELL = 12
 EVENT_GROUP = 10  # launches between two events of the pass that times the kernels
+REPEATS = 5       # the timed region (--steps steps between two synchronisations) is run this often
 BWD_BYTES_PER_CELL = 16
 
 # HBM bytes per launch on the default workload, from rocprofv3's FETCH_SIZE / WRITE_SIZE counters
@@ -121,6 +122,10 @@ def pruned_secondary(dev, steps=50, cpu=True):
     sym, bd = torch.from_numpy(c["symbols"]).to(dev), torch.from_numpy(c["boundary"]).to(dev)
     logits = torch.from_numpy(np.random.default_rng(33).standard_normal((B, T, R, C)).astype(np.float32)).to(dev)
     logits.requires_grad_(True)
+    # Three copies taken in turn (480 MB): a step's logits then come from HBM, not from what the
+    # steps before left in the 256 MB Infinity Cache, which holds one copy (160 MB) whole.
+    logits_sets = [logits] + [logits.detach().clone().requires_grad_(True) for _ in range(LOGITS_SETS - 1)]
+    turn = [0]
 
     # A training loop brings a new boundary tensor with every batch, and the functions read its
     # values on the host once per tensor (a device-to-host copy that waits for the stream): every
@@ -130,27 +135,33 @@ def pruned_secondary(dev, steps=50, cpu=True):
         _, (gx, gy) = k2.rnnt_loss_simple(lm, am, sym, 0, b, reduction="sum", return_grad=True)
         return k2.get_rnnt_prune_ranges(gx, gy, b, R)
 
-    def pruned(ranges):
-        logits.grad = None
-        loss = k2.rnnt_loss_pruned(logits, sym, ranges, 0, bd.clone(), reduction="sum")
+    def pruned(ranges, n_sets):
+        x = logits_sets[turn[0] % n_sets]
+        turn[0] += 1
+        x.grad = None
+        loss = k2.rnnt_loss_pruned(x, sym, ranges, 0, bd.clone(), reduction="sum")
         loss.backward()
         return loss
 
     ranges = simple_and_ranges()
-    for _ in range(3):
-        pruned(ranges)
-    ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+    for _ in range(2 * LOGITS_SETS):
+        pruned(ranges, LOGITS_SETS)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
     torch.cuda.synchronize()
     ev[0].record()
     for _ in range(steps):
         ranges = simple_and_ranges()
     ev[1].record()
     for _ in range(steps):
-        loss = pruned(ranges)
+        loss = pruned(ranges, LOGITS_SETS)
     ev[2].record()
+    for _ in range(steps):
+        pruned(ranges, 1)
+    ev[3].record()
     torch.cuda.synchronize()
     t_ranges = ev[0].elapsed_time(ev[1]) / steps * 1e-3
     t_pruned = ev[1].elapsed_time(ev[2]) / steps * 1e-3
+    t_cached = ev[2].elapsed_time(ev[3]) / steps * 1e-3
     # one read of the logits forward, one read + one write backward, fp32
     logits_bytes = 3 * logits.numel() * 4
     out = {
@@ -158,8 +169,18 @@ def pruned_secondary(dev, steps=50, cpu=True):
                     "(BASELINE config 3), ranges from an rnnt_loss_simple pass; a fresh boundary "
                     "tensor in every step (one host read of it per step, as in a training loop)",
         "value": B / t_pruned, "unit": "utterances/s", "ms_per_step": t_pruned * 1e3,
+        "logits": f"taken in turn from {LOGITS_SETS} copies, {LOGITS_SETS * logits.numel() * 4 // 1000000} MB in "
+                  "all: they come from HBM",
         "logits_GBps": logits_bytes / t_pruned / 1e9,
         "frac_of_hbm_peak": logits_bytes / t_pruned / 1e9 / HBM_PEAK_GBS,
+        "roofline": {"bound": "hbm", "achieved": logits_bytes / t_pruned / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": logits_bytes / t_pruned / 1e9 / HBM_PEAK_GBS,
+                     "bytes": "the logits read forward, read again and their gradient written backward (480 MB); "
+                              "the whole step through the API, host launches included",
+                     **PROFILED_KERNELS["c3_pruned"]},
+        "cache_resident": {"logits": "the same 160 MB tensor every step, which the Infinity Cache holds",
+                           "ms_per_step": t_cached * 1e3, "value": B / t_cached,
+                           "logits_GBps": logits_bytes / t_cached / 1e9},
         "simple_pass_plus_prune_ranges_ms": t_ranges * 1e3,
         "loss": float(loss.detach()),
     }
@@ -183,6 +204,16 @@ def pruned_secondary(dev, steps=50, cpu=True):
 
 
 MFMA_PEAK_TFLOPS = {"fp32": 157.3, "bf16": 2500.0}  # MI355X published dense matrix rates
+LOGITS_SETS = 3  # copies of config 3's logits the secondary figures rotate over (see pruned_secondary)
+# The dominant kernel of the secondary workloads and its average duration in the committed kernel
+# trace of this file's default run (rocprofv3 --kernel-trace --stats; not measured by the run).
+PROFILED_KERNELS = {
+    "c3_pruned": {"kernel": "RowGradKernel (grid 5120000)", "kernel_avg_us": 52.8,
+                  "kernel_source": "profiles/mi_bidir_kernel_c4_kernel_trace.md, the default run's table "
+                                   "(recorded when every step read the same 160 MB of logits)"},
+    "c5_joint": {"kernel": "RowGradKernel (grid 11673600)", "kernel_avg_us": 113.6,
+                 "kernel_source": "profiles/mi_bidir_kernel_c4_kernel_trace.md, the default run's table"},
+}
 
 
 def fused_joiner(dev, steps=20):
@@ -311,7 +342,13 @@ def other_configs(dev, steps=50):
     out["c5_rnnt_loss"] = {
         "workload": "rnnt_loss fwd+bwd, fp32, regular, B=8 T=300 S=75 V=500 (BASELINE config 5)",
         "ms_per_step": t * 1e3, "utterances_per_s": B / t, "logits_GBps": nbytes / t / 1e9,
-        "frac_of_hbm_peak": nbytes / t / 1e9 / HBM_PEAK_GBS}
+        "frac_of_hbm_peak": nbytes / t / 1e9 / HBM_PEAK_GBS,
+        "logits": "one 365 MB tensor, larger than the 256 MB Infinity Cache: read from HBM in every step",
+        "roofline": {"bound": "hbm", "achieved": nbytes / t / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": nbytes / t / 1e9 / HBM_PEAK_GBS,
+                     "bytes": "the logits read forward, read again and their gradient written backward (1.09 GB); "
+                              "the whole step through the API, host launches included",
+                     **PROFILED_KERNELS["c5_joint"]}}
     return out
 
 
@@ -362,15 +399,20 @@ def next_rows(dev, steps=30):
         "arc records 16 B + arc_map 4 B written and one logit read per arc, ranges read once")
 
     logits.requires_grad_(True)
+    logits_sets = [logits] + [logits.detach().clone().requires_grad_(True) for _ in range(LOGITS_SETS - 1)]
+    turn = [0]
 
     def hat():
-        logits.grad = None
-        k2.rnnt_loss_pruned(logits, sym, ranges, 0, bd.clone(), reduction="sum", use_hat_loss=True).backward()
+        x = logits_sets[turn[0] % LOGITS_SETS]
+        turn[0] += 1
+        x.grad = None
+        k2.rnnt_loss_pruned(x, sym, ranges, 0, bd.clone(), reduction="sum", use_hat_loss=True).backward()
 
     out["hat_pruned_loss"] = entry(
-        f"rnnt_loss_pruned(use_hat_loss=True) fwd+bwd, fp32, regular, B={B} T={T} S={S} V={C} s_range={R}",
+        f"rnnt_loss_pruned(use_hat_loss=True) fwd+bwd, fp32, regular, B={B} T={T} S={S} V={C} s_range={R}; "
+        f"logits taken in turn from {LOGITS_SETS} copies (from HBM)",
         timed(hat), 3 * logits.numel() * 4, "logits read forward, read + gradient written backward")
-    del logits
+    del logits, logits_sets
 
     B, T, S, C = 16, 250, 50, 500
     c = cases.rnnt_case(2, B, T, S, C, t_lo=150, s_lo=20)
@@ -486,12 +528,17 @@ def main():
         # The timed region: exactly args.steps steps between two synchronisations, nothing else on
         # the stream (an event recorded between two launches costs the GPU 3-4 us, 7 % of this
         # step).  The kernels' durations come from a second pass over the same steps.
-        t0 = time.perf_counter()
-        for k in range(args.steps):
-            step()
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
-        m = {"ms_per_step": wall / args.steps * 1e3, "input_mb": len(sets) * (px.numel() + py.numel()) * 4 // 1000000}
+        # The region is run REPEATS times and the median reported (a region of 20 steps lasts a
+        # millisecond: one sample of it says little).
+        walls = []
+        for _ in range(REPEATS):
+            t0 = time.perf_counter()
+            for k in range(args.steps):
+                step()
+            torch.cuda.synchronize()
+            walls.append((time.perf_counter() - t0) / args.steps * 1e3)
+        m = {"ms_per_step": float(np.median(walls)), "ms_per_step_repeats": walls,
+             "input_mb": len(sets) * (px.numel() + py.numel()) * 4 // 1000000}
         events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
         torch.cuda.synchronize()
         if single:
@@ -557,6 +604,9 @@ def main():
                                f"S={S} T={T}, random boundary (BASELINE config 4)",
                    "active_cells": active, "full_box_cells": full, "log_deriv_kept": bool(keep),
                    "launches_per_step": 1 if single else 2, "input_sets": args.input_sets,
+                   "timed_region": f"{args.steps} steps between two synchronisations, run {REPEATS} times; "
+                                   "ms_per_step is the median of the runs",
+                   "ms_per_step_of_each_run": m["ms_per_step_repeats"],
                    "inputs": ("the same px / py every step: at this size the Infinity Cache serves them from "
                               "the second step on, as it does after the builder kernels of the loss functions"
                               if args.input_sets == 1 else
@@ -565,6 +615,9 @@ def main():
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
                      "traffic": traffic_table.get(dom) if (B, S, T) == (32, 200, 1000) else None,
+                     "traffic_source": "rocprofv3 FETCH_SIZE + WRITE_SIZE of this kernel on this workload, from the "
+                                       "committed profile (profiles/mi_bidir_kernel_c4_hbm_traffic.md); not "
+                                       "measured by this run",
                      "kernel": dom,
                      "kernel_avg_us": dom_ms * 1e3},
         "kernels": dict(m["kernel_times"],

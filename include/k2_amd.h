@@ -98,6 +98,11 @@ K2AMD_API int k2amd_mi_forward(const void *px, const void *py, const int64_t *bo
 K2AMD_API int k2amd_mi_forward_noalloc(const void *px, const void *py, const int64_t *boundary,
                                        void *p, void *ans, int B, int S, int T, int modified,
                                        int dtype, void *stream);
+/* k2amd_mi_workspace_status for the static array of the current device: synchronises `stream` and
+ * returns K2AMD_ERR_TIMEOUT if the last k2amd_mi_forward_noalloc on this device gave up a wait
+ * (its ans then holds NaN).  Ask before the next such call: every call starts by clearing the flag
+ * with the rest of the array.  No counterpart in the reference.                                  */
+K2AMD_API int k2amd_mi_noalloc_status(void *stream);
 
 /* Replaces _k2.mutual_information_backward (k2/python/csrc/torch/mutual_information.cu:46-67,
  * semantics of k2/python/csrc/torch/mutual_information_cpu.cu:128-255).  Writes EVERY element of
@@ -207,18 +212,20 @@ K2AMD_API int k2amd_rnnt_logprobs_simple_forward(
     int T, int C, int termination_symbol, int rnnt_type, int dtype, void *stream);
 
 /* Gradient of the above w.r.t. lm and am (what torch autograd derives from
- * k2/python/k2/rnnt_loss.py:172-223).  q_scratch is device scratch of
- * k2amd_rnnt_logprobs_simple_backward_scratch_elements(B, S, T) elements of the tensors' type
+ * k2/python/k2/rnnt_loss.py:172-223).  q_scratch is device scratch of q_scratch_elements
+ * elements of the tensors' type, at least
+ * k2amd_rnnt_logprobs_simple_backward_scratch_elements(B, S, T)
  * (= B * ((S+1) * T + ceil((S+1) / 32) * T + 2 * (S+1) * ceil(T / 64)): the [B][S+1][T] operand
  * of the two products, then the gradients' sums along s ([B][T] per 32 rows) and along t
- * ([B][S+1] per 64 frames, for px_grad and for py_grad)).                                        */
+ * ([B][S+1] per 64 frames, for px_grad and for py_grad)); less is refused with
+ * K2AMD_ERR_WORKSPACE before anything is launched.                                               */
 K2AMD_API size_t k2amd_rnnt_logprobs_simple_backward_scratch_elements(int B, int S, int T);
 K2AMD_API int k2amd_rnnt_logprobs_simple_backward(
     const void *px_grad, const void *py_grad, const void *seq_scale, const int64_t *symbols,
     const int64_t *boundary,
     const void *lm_probs, const void *am_probs, const void *denom, void *lm_grad, void *am_grad,
-    void *q_scratch, int B, int S, int T, int C, int termination_symbol, int rnnt_type, int dtype,
-    void *stream);
+    void *q_scratch, size_t q_scratch_elements, int B, int S, int T, int C, int termination_symbol,
+    int rnnt_type, int dtype, void *stream);
 
 /* Replaces get_rnnt_logprobs_joint (k2/python/k2/rnnt_loss.py:341-447): logits [B][T][S+1][C];
  * normalizers [B][T][S+1] = logsumexp over C is written for the backward.                        */

@@ -29,6 +29,7 @@ _SIGNATURES = {
     "k2amd_mi_workspace_init": ([_vp, _sz, _vp], _ci),
     "k2amd_mi_workspace_status": ([_vp, _vp], _ci),
     "k2amd_mi_workspace_status_async": ([_vp, _vp, _vp], _ci),
+    "k2amd_mi_noalloc_status": ([_vp], _ci),
     "k2amd_mi_forward": ([_vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp, _sz, _vp], _ci),
     "k2amd_mi_forward_noalloc": ([_vp] * 5 + [_ci] * 5 + [_vp], _ci),
     "k2amd_mi_backward": ([_vp, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci,
@@ -44,7 +45,7 @@ _SIGNATURES = {
     "k2amd_mi_joint_products": ([_vp, _vp, _ci, _vp, _vp, _vp, _vp, _ci, ctypes.c_longlong, ctypes.c_longlong,
                                  _ci, _vp], _ci),
     "k2amd_rnnt_logprobs_simple_forward": ([_vp] * 11 + [_ci] * 7 + [_vp], _ci),
-    "k2amd_rnnt_logprobs_simple_backward": ([_vp] * 11 + [_ci] * 7 + [_vp], _ci),
+    "k2amd_rnnt_logprobs_simple_backward": ([_vp] * 11 + [ctypes.c_size_t] + [_ci] * 7 + [_vp], _ci),
     "k2amd_rnnt_logprobs_simple_backward_scratch_elements": ([_ci] * 3, ctypes.c_size_t),
     "k2amd_rnnt_logprobs_joint_forward": ([_vp] * 6 + [_ci] * 7 + [_vp], _ci),
     "k2amd_rnnt_logprobs_joint_backward": ([_vp] * 8 + [_ci] * 7 + [_vp], _ci),
@@ -403,7 +404,7 @@ def logprobs_simple_backward(px_grad, py_grad, symbols, boundary, saved, termina
     with torch.cuda.device(dev):
         check(lib().k2amd_rnnt_logprobs_simple_backward(
             ptr(px_grad), ptr(py_grad), ptr(seq_scale), ptr(symbols), ptr(boundary), ptr(lm_probs),
-            ptr(am_probs), ptr(denom), ptr(lm_grad), ptr(am_grad), ptr(q), B, S, T, C, termination_symbol,
+            ptr(am_probs), ptr(denom), ptr(lm_grad), ptr(am_grad), ptr(q), q.numel(), B, S, T, C, termination_symbol,
             rnnt_type, dtype_code(am_probs), stream_ptr(dev)))
     return lm_grad, am_grad
 

@@ -897,6 +897,13 @@ __global__ void JoinerRowHeaderKernel(const JoinerArgs a, const float *__restric
 int RoundUp(int v, int m) { return (v + m - 1) / m * m; }
 size_t ElemBytes(int precision) { return precision == K2AMD_JOINER_BF16 ? 2 : 4; }
 
+// A lattice without frames: the regular one still has its px column T, which the reference pads
+// with -inf (k2/python/k2/rnnt_loss.py:1310-1319).
+__global__ void JoinerFillKernel(float *__restrict__ dst, size_t n, float v) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+    dst[i] = v;
+}
+
 bool JoinerShapeOk(int B, int S, int T, int R, int C, int D) {
   if (B < 0 || S < 0 || T < 0 || R < 1 || C < 1) return false;
   if (D < 64 || D > kMaxD || D % 64 != 0 || R > 32 || R > S + 1 || C > (1 << 20)) return false;
@@ -1076,7 +1083,17 @@ int k2amd_rnnt_joiner_pruned_forward(const void *am, const void *lm, const int64
   if (rnnt_type != K2AMD_REGULAR && rnnt_type != K2AMD_MODIFIED && rnnt_type != K2AMD_CONSTRAINED)
     return K2AMD_ERR_INVALID_ARGUMENT;
   if (rnnt_type != K2AMD_REGULAR && T < S) return K2AMD_ERR_INVALID_ARGUMENT;
-  if (B == 0 || T == 0) return K2AMD_OK;
+  if (B == 0) return K2AMD_OK;
+  if (T == 0) {  // no frames: py is empty, px is its one -inf column where the lattice is regular
+    if (rnnt_type == K2AMD_REGULAR && S > 0) {
+      if (!px) return K2AMD_ERR_INVALID_ARGUMENT;
+      const size_t n = (size_t)B * S;
+      hipLaunchKernelGGL(JoinerFillKernel, dim3((unsigned)std::min<size_t>((n + 255) / 256, 1024)), dim3(256), 0,
+                         static_cast<hipStream_t>(stream), (float *)px, n, -__builtin_huge_valf());
+      return LaunchStatus();
+    }
+    return K2AMD_OK;
+  }
   if (!am || !lm || !ranges || !weight || !px || !py || !normalizers || (!symbols && S > 0))
     return K2AMD_ERR_INVALID_ARGUMENT;
   if (workspace == nullptr ||

@@ -145,7 +145,11 @@ int k2amd_mi_forward_keep(const void *px, const void *py, const int64_t *boundar
 int k2amd_mi_forward_noalloc(const void *px, const void *py, const int64_t *boundary, void *p,
                              void *ans, int B, int S, int T, int modified, int dtype, void *stream) {
   if (!ShapeOk(B, S, T) || (dtype != K2AMD_F32 && dtype != K2AMD_F64)) return K2AMD_ERR_INVALID_ARGUMENT;
-  const size_t need = k2amd_mi_workspace_bytes(B, S, T, modified, dtype);
+  // scratch only where the pipelined kernels will take the shape: what the exact kernels serve
+  // (no rows or no columns, tensors of 2 GiB and more) needs none and is never refused for it
+  const bool pipelined = !ForceGeneric() && B > 0 &&
+                         (dtype == K2AMD_F32 ? MiFastSupports(B, S, T, modified ? 1 : 0) : MiWaveSupports(B, S, T));
+  const size_t need = pipelined ? k2amd_mi_workspace_bytes(B, S, T, modified, dtype) : 0;
   if (need > kScratchBytes) return K2AMD_ERR_SCRATCH_LIMIT;
   // set-up (also for B == 0, so that a caller can have it done ahead of its first real call)
   void *ws = ScratchOfCurrentDevice();
@@ -161,6 +165,12 @@ int k2amd_mi_forward_noalloc(const void *px, const void *py, const int64_t *boun
   }
   return k2amd_mi_forward_keep(px, py, boundary, p, ans, nullptr, B, S, T, modified, dtype,
                                need > 0 ? ws : nullptr, need, stream);
+}
+
+int k2amd_mi_noalloc_status(void *stream) {
+  void *ws = ScratchOfCurrentDevice();
+  if (ws == nullptr) return K2AMD_ERR_LAUNCH;
+  return k2amd_mi_workspace_status(ws, stream);
 }
 
 int k2amd_mi_backward(const void *px, const void *py, const int64_t *boundary, const void *p,

@@ -430,7 +430,7 @@ std::vector<torch::Tensor> LogprobsSimpleBackward(torch::Tensor px_grad, torch::
     Check(k2amd_rnnt_logprobs_simple_backward(
         px_grad.data_ptr(), py_grad.data_ptr(), scale, I64(symbols), I64(boundary), lm_probs.data_ptr(),
         am_probs.data_ptr(), denom.data_ptr(), lm_grad.data_ptr(), am_grad.data_ptr(), q.data_ptr(),
-        B, S, T, C, termination_symbol, rnnt_type, DtypeCode(am_probs), stream));
+        static_cast<size_t>(q.numel()), B, S, T, C, termination_symbol, rnnt_type, DtypeCode(am_probs), stream));
   }
   return {lm_grad, am_grad};
 }

@@ -1012,10 +1012,12 @@ int k2amd_rnnt_logprobs_simple_backward(const void *px_grad, const void *py_grad
                                         const void *seq_scale, const int64_t *symbols, const int64_t *boundary,
                                         const void *lm_probs, const void *am_probs,
                                         const void *denom, void *lm_grad, void *am_grad,
-                                        void *q_scratch, int B, int S, int T, int C,
-                                        int termination_symbol, int rnnt_type, int dtype,
-                                        void *stream) {
+                                        void *q_scratch, size_t q_scratch_elements, int B, int S,
+                                        int T, int C, int termination_symbol, int rnnt_type,
+                                        int dtype, void *stream) {
   if (!ArgsOk(B, S, T, C, termination_symbol, rnnt_type, dtype)) return K2AMD_ERR_INVALID_ARGUMENT;
+  if (q_scratch == nullptr || q_scratch_elements < k2amd_rnnt_logprobs_simple_backward_scratch_elements(B, S, T))
+    return B == 0 ? K2AMD_OK : K2AMD_ERR_WORKSPACE;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == K2AMD_F32)
     return SimpleBackward<float>((const float *)px_grad, (const float *)py_grad, (const float *)seq_scale, symbols, boundary, (const float *)lm_probs, (const float *)am_probs, (const float *)denom, (float *)lm_grad, (float *)am_grad, (float *)q_scratch, B, S, T, C, termination_symbol, rnnt_type, st);

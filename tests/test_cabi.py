@@ -68,6 +68,14 @@ def test_invalid_arguments_return_codes_without_a_gpu():
     assert lib.k2amd_mi_keeps_log_deriv(0, 10, 20, 0, 0, 1) == 0
     assert lib.k2amd_rnnt_prune_ranges(None, None, None, None, 1, 4, 4, 0, 9, 0, None) == 1
     assert lib.k2amd_rnnt_logprobs_joint_forward(None, None, None, None, None, None, 1, 1, 1, 4, 9, 0, 0, None) == 1
+    # the simple builder's backward: scratch smaller than its query function says is refused
+    # before anything is launched (B=2 S=5 T=9 C=7: 2 * (6*9 + 1*9 + 2*6*1) = 150 elements)
+    need = lib.k2amd_rnnt_logprobs_simple_backward_scratch_elements(2, 5, 9)
+    assert need == 150
+    args = lambda n: (one, one, None, one, None, one, one, one, one, one, one, n, 2, 5, 9, 7, 0, 0, 0, None)
+    assert lib.k2amd_rnnt_logprobs_simple_backward(*args(need - 1)) == 3
+    assert lib.k2amd_rnnt_logprobs_simple_backward(one, one, None, one, None, one, one, one, one, one, None, need,
+                                                   2, 5, 9, 7, 0, 0, 0, None) == 3
     # an empty batch is a no-op
     assert lib.k2amd_mi_forward(None, None, None, None, None, 0, 3, 3, 0, 0, None, 0, None) == 0
     with pytest.raises(RuntimeError):

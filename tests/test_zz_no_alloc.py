@@ -44,11 +44,19 @@ def test_noalloc_forward_equals_the_workspace_entry_point(device):
     _both(small, device)
     _both(cases.mi_case(77, dtype=np.float64, max_B=3, max_S=20, max_T=40), device)   # the fp64 kernels, same array
     _both(big, device)
-    # beyond the static array: refused with its own status, nothing launched
+    # A shape that the pipelined kernels take and whose scratch is beyond the static array: refused
+    # with its own status, nothing launched.  (Null pointers: were the refusal ever to fail, the
+    # call would be turned down for them instead of reaching a kernel.)
     lib = capi.lib()
-    one = 1  # never dereferenced
-    assert lib.k2amd_mi_workspace_bytes(4096, 200, 1000, 1, 0) > (8 << 20)
-    assert lib.k2amd_mi_forward_noalloc(one, one, None, one, one, 4096, 200, 1000, 1, 0, None) == 6
+    assert lib.k2amd_mi_keeps_log_deriv(2048, 100, 500, 1, 0, 1) == 1
+    assert lib.k2amd_mi_workspace_bytes(2048, 100, 500, 1, 0) > (8 << 20)
+    assert lib.k2amd_mi_forward_noalloc(None, None, None, None, None, 2048, 100, 500, 1, 0, None) == 6
+    # what the exact kernels serve without scratch is not refused for the array's size: a lattice
+    # of 2 GiB and more gets as far as the check of its pointers
+    assert lib.k2amd_mi_keeps_log_deriv(4096, 200, 1000, 1, 0, 1) == 0
+    assert lib.k2amd_mi_forward_noalloc(None, None, None, None, None, 4096, 200, 1000, 1, 0, None) == 1
     with pytest.raises(RuntimeError, match="static array"):
         capi.check(6)
     assert lib.k2amd_mi_forward_noalloc(None, None, None, None, None, 0, 3, 3, 0, 0, None) == 0
+    # no wait gave up in any of the calls above (the flag sits in the static array)
+    assert lib.k2amd_mi_noalloc_status(torch.cuda.current_stream(device).cuda_stream) == 0
