@@ -227,6 +227,46 @@ K2AMD_API int k2amd_rnnt_logprobs_simple_backward(
     void *q_scratch, size_t q_scratch_elements, int B, int S, int T, int C, int termination_symbol,
     int rnnt_type, int dtype, void *stream);
 
+/* The terms that get_rnnt_logprobs_smoothed (k2/python/k2/rnnt_loss.py:1471-1704) adds to
+ * get_rnnt_logprobs, and the mix of the three:
+ *   px[b,s,t] = joint_scale * px_joint[b,s,t] + lm_only_scale * log softmax(lm[b,s])[sym[b,s]]
+ *                                             + am_only_scale * log softmax(am[b,t] + log unigram)[sym[b,s]]
+ * and py alike with the termination symbol; joint_scale = 1 - lm_only_scale - am_only_scale,
+ * unigram = the mean over all B (S+1) rows of softmax(lm) + tiny, a scale of exactly 0 counts as
+ * 1e-20 as in the reference.  After the mix: px[b,:,T] = px[b,:,boundary[b,3]] = -inf on a regular
+ * lattice, px[b,s,t] += py[b,s+1,t] on a constrained one.
+ * Inputs besides lm and am: what k2amd_rnnt_logprobs_simple_forward wrote for the same lm and am
+ * on a REGULAR (if rnnt_type is regular) or MODIFIED (otherwise) lattice with a null boundary:
+ * px_joint, py_joint, lm_probs, am_probs, lm_max, am_max.  Outputs: px [B][S][T+1 or T],
+ * py [B][S+1][T] (neither may overlap px_joint / py_joint), and for the backward lm_norm [B][S+1]
+ * (log sum_c exp lm), am_norm [B][T] (log sum_c exp(am) unigram[c]) and unigram [2][C] (the
+ * unigram, then its log).  scratch: k2amd_rnnt_smoothed_scratch_elements(B, S, T, C) elements of
+ * the tensors' type (= C * max(ceil(B (S+1) / 16), 1 + ceil(B T / 16)): per-workgroup column
+ * sums); less is refused with K2AMD_ERR_WORKSPACE before anything is launched.
+ * The vocabulary must fit the kernels' LDS arrays: (2 C + S) * sizeof(element) <= 64 KiB, else
+ * K2AMD_ERR_UNSUPPORTED (k2amd_rnnt_smoothed_supported tells beforehand).                         */
+K2AMD_API size_t k2amd_rnnt_smoothed_scratch_elements(int B, int S, int T, int C);
+K2AMD_API int k2amd_rnnt_smoothed_supported(int B, int S, int T, int C, int dtype);
+K2AMD_API int k2amd_rnnt_smoothed_forward(
+    const void *lm, const void *am, const int64_t *symbols, const int64_t *boundary,
+    const void *lm_probs, const void *am_probs, const void *lm_max, const void *am_max,
+    const void *px_joint, const void *py_joint, void *px, void *py, void *lm_norm, void *am_norm,
+    void *unigram, void *scratch, size_t scratch_elements, double lm_only_scale, double am_only_scale,
+    int B, int S, int T, int C, int termination_symbol, int rnnt_type, int dtype, void *stream);
+
+/* Gradient of the two marginal terms above (what torch autograd derives from
+ * k2/python/k2/rnnt_loss.py:1608-1690), ADDED to lm_grad [B][S+1][C] and am_grad [B][T][C].  The
+ * joint term's gradient is k2amd_rnnt_logprobs_simple_backward's on the same px_grad / py_grad,
+ * boundary and rnnt_type with seq_scale[b] * joint_scale in place of seq_scale[b]; it writes
+ * lm_grad and am_grad and so has to run first.  px_grad / py_grad are the gradients that reach
+ * the mixed px / py.                                                                              */
+K2AMD_API int k2amd_rnnt_smoothed_backward(
+    const void *px_grad, const void *py_grad, const void *seq_scale, const int64_t *symbols,
+    const int64_t *boundary, const void *lm_probs, const void *am_probs, const void *lm_max,
+    const void *am_max, const void *lm_norm, const void *am_norm, const void *unigram, void *lm_grad,
+    void *am_grad, void *scratch, size_t scratch_elements, double lm_only_scale, double am_only_scale,
+    int B, int S, int T, int C, int termination_symbol, int rnnt_type, int dtype, void *stream);
+
 /* Replaces get_rnnt_logprobs_joint (k2/python/k2/rnnt_loss.py:341-447): logits [B][T][S+1][C];
  * normalizers [B][T][S+1] = logsumexp over C is written for the backward.                        */
 K2AMD_API int k2amd_rnnt_logprobs_joint_forward(

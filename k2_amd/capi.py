@@ -47,6 +47,12 @@ _SIGNATURES = {
     "k2amd_rnnt_logprobs_simple_forward": ([_vp] * 11 + [_ci] * 7 + [_vp], _ci),
     "k2amd_rnnt_logprobs_simple_backward": ([_vp] * 11 + [ctypes.c_size_t] + [_ci] * 7 + [_vp], _ci),
     "k2amd_rnnt_logprobs_simple_backward_scratch_elements": ([_ci] * 3, ctypes.c_size_t),
+    "k2amd_rnnt_smoothed_scratch_elements": ([_ci] * 4, ctypes.c_size_t),
+    "k2amd_rnnt_smoothed_supported": ([_ci] * 5, _ci),
+    "k2amd_rnnt_smoothed_forward": ([_vp] * 16 + [ctypes.c_size_t, ctypes.c_double, ctypes.c_double] + [_ci] * 7
+                                    + [_vp], _ci),
+    "k2amd_rnnt_smoothed_backward": ([_vp] * 15 + [ctypes.c_size_t, ctypes.c_double, ctypes.c_double] + [_ci] * 7
+                                     + [_vp], _ci),
     "k2amd_rnnt_logprobs_joint_forward": ([_vp] * 6 + [_ci] * 7 + [_vp], _ci),
     "k2amd_rnnt_logprobs_joint_backward": ([_vp] * 8 + [_ci] * 7 + [_vp], _ci),
     "k2amd_rnnt_logprobs_pruned_forward": ([_vp] * 7 + [_ci] * 8 + [_vp], _ci),
@@ -406,6 +412,88 @@ def logprobs_simple_backward(px_grad, py_grad, symbols, boundary, saved, termina
             ptr(px_grad), ptr(py_grad), ptr(seq_scale), ptr(symbols), ptr(boundary), ptr(lm_probs),
             ptr(am_probs), ptr(denom), ptr(lm_grad), ptr(am_grad), ptr(q), q.numel(), B, S, T, C, termination_symbol,
             rnnt_type, dtype_code(am_probs), stream_ptr(dev)))
+    return lm_grad, am_grad
+
+
+def smoothed_supported(lm, am):
+    """Whether the smoothed builder's kernels take these tensors (the vocabulary has to fit their
+    LDS arrays)."""
+    B, T, C = am.shape
+    return bool(lib().k2amd_rnnt_smoothed_supported(B, lm.shape[1] - 1, T, C, dtype_code(am)))
+
+
+def logprobs_smoothed_forward(lm, am, symbols, termination_symbol, lm_only_scale, am_only_scale, rnnt_type,
+                              boundary):
+    """C-ABI get_rnnt_logprobs_smoothed: the simple builder on the lattice without a boundary, then
+    the marginal terms and the mix.  Returns (px, py, saved), ``saved`` = (lm_probs, am_probs, denom,
+    lm_max, am_max, lm_norm, am_norm, unigram) for the backward."""
+    dt, dev = _float_dtype(am, "am")
+    B, T, C = _dims(am, "am", 3)
+    S = _dims(lm, "lm", 3)[1] - 1
+    _rnnt_type(rnnt_type)
+    expect(am, "am", dt, dev, (B, T, C))
+    expect(lm, "lm", dt, dev, (B, S + 1, C))
+    expect(symbols, "symbols", torch.int64, dev, (B, S))
+    expect_optional(boundary, "boundary", torch.int64, dev, (B, 4))
+    _symbol(termination_symbol, C)
+    joint_type = REGULAR if rnnt_type == REGULAR else MODIFIED
+    px_joint = torch.empty(B, S, _t1(T, rnnt_type), dtype=dt, device=dev)
+    py_joint = torch.empty(B, S + 1, T, dtype=dt, device=dev)
+    px, py = torch.empty_like(px_joint), torch.empty_like(py_joint)
+    lm_probs, am_probs = torch.empty_like(lm), torch.empty_like(am)
+    lm_max, lm_norm = (torch.empty(B, S + 1, dtype=dt, device=dev) for _ in range(2))
+    am_max, am_norm = (torch.empty(B, T, dtype=dt, device=dev) for _ in range(2))
+    denom = torch.empty(B, S + 1, T, dtype=dt, device=dev)
+    unigram = torch.empty(2, C, dtype=dt, device=dev)
+    scratch = torch.empty(lib().k2amd_rnnt_smoothed_scratch_elements(B, S, T, C), dtype=dt, device=dev)
+    with torch.cuda.device(dev):
+        check(lib().k2amd_rnnt_logprobs_simple_forward(
+            ptr(lm), ptr(am), ptr(symbols), None, ptr(px_joint), ptr(py_joint), ptr(lm_probs), ptr(am_probs),
+            ptr(lm_max), ptr(am_max), ptr(denom), B, S, T, C, termination_symbol, joint_type, dtype_code(am),
+            stream_ptr(dev)))
+        check(lib().k2amd_rnnt_smoothed_forward(
+            ptr(lm), ptr(am), ptr(symbols), ptr(boundary), ptr(lm_probs), ptr(am_probs), ptr(lm_max), ptr(am_max),
+            ptr(px_joint), ptr(py_joint), ptr(px), ptr(py), ptr(lm_norm), ptr(am_norm), ptr(unigram), ptr(scratch),
+            scratch.numel(), float(lm_only_scale), float(am_only_scale), B, S, T, C, termination_symbol, rnnt_type,
+            dtype_code(am), stream_ptr(dev)))
+    return px, py, (lm_probs, am_probs, denom, lm_max, am_max, lm_norm, am_norm, unigram)
+
+
+def logprobs_smoothed_backward(px_grad, py_grad, symbols, boundary, saved, termination_symbol, lm_only_scale,
+                               am_only_scale, rnnt_type, seq_scale=None):
+    """(lm_grad, am_grad): the simple builder's backward with the gradients scaled by
+    1 - lm_only_scale - am_only_scale, then the marginal terms' gradients added."""
+    lm_probs, am_probs, denom, lm_max, am_max, lm_norm, am_norm, unigram = saved
+    dt, dev = _float_dtype(am_probs, "am_probs")
+    B, T, C = _dims(am_probs, "am_probs", 3)
+    S = _dims(lm_probs, "lm_probs", 3)[1] - 1
+    _rnnt_type(rnnt_type)
+    expect(am_probs, "am_probs", dt, dev, (B, T, C))
+    expect(lm_probs, "lm_probs", dt, dev, (B, S + 1, C))
+    expect(denom, "denom", dt, dev, (B, S + 1, T))
+    for t, name, shape in ((lm_max, "lm_max", (B, S + 1)), (lm_norm, "lm_norm", (B, S + 1)), (am_max, "am_max", (B, T)),
+                           (am_norm, "am_norm", (B, T)), (unigram, "unigram", (2, C))):
+        expect(t, name, dt, dev, shape)
+    expect(symbols, "symbols", torch.int64, dev, (B, S))
+    expect_optional(boundary, "boundary", torch.int64, dev, (B, 4))
+    _expect_lattice_grads(px_grad, py_grad, seq_scale, dt, dev, B, S, T, rnnt_type)
+    _symbol(termination_symbol, C)
+    joint_scale = 1.0 - float(lm_only_scale) - float(am_only_scale)
+    joint_seq_scale = (torch.full((B,), joint_scale, dtype=dt, device=dev) if seq_scale is None
+                       else seq_scale * joint_scale)
+    lm_grad, am_grad = torch.empty_like(lm_probs), torch.empty_like(am_probs)
+    q = torch.empty(lib().k2amd_rnnt_logprobs_simple_backward_scratch_elements(B, S, T), dtype=dt, device=dev)
+    scratch = torch.empty(lib().k2amd_rnnt_smoothed_scratch_elements(B, S, T, C), dtype=dt, device=dev)
+    with torch.cuda.device(dev):
+        check(lib().k2amd_rnnt_logprobs_simple_backward(
+            ptr(px_grad), ptr(py_grad), ptr(joint_seq_scale), ptr(symbols), ptr(boundary), ptr(lm_probs),
+            ptr(am_probs), ptr(denom), ptr(lm_grad), ptr(am_grad), ptr(q), q.numel(), B, S, T, C, termination_symbol,
+            rnnt_type, dtype_code(am_probs), stream_ptr(dev)))
+        check(lib().k2amd_rnnt_smoothed_backward(
+            ptr(px_grad), ptr(py_grad), ptr(seq_scale), ptr(symbols), ptr(boundary), ptr(lm_probs), ptr(am_probs),
+            ptr(lm_max), ptr(am_max), ptr(lm_norm), ptr(am_norm), ptr(unigram), ptr(lm_grad), ptr(am_grad),
+            ptr(scratch), scratch.numel(), float(lm_only_scale), float(am_only_scale), B, S, T, C,
+            termination_symbol, rnnt_type, dtype_code(am_probs), stream_ptr(dev)))
     return lm_grad, am_grad
 
 

@@ -435,6 +435,102 @@ std::vector<torch::Tensor> LogprobsSimpleBackward(torch::Tensor px_grad, torch::
   return {lm_grad, am_grad};
 }
 
+// get_rnnt_logprobs_smoothed (k2/python/k2/rnnt_loss.py:1471-1704): the simple builder on the
+// lattice without a boundary, then the marginal terms and the mix.  Returns (px, py, lm_probs,
+// am_probs, denom, lm_max, am_max, lm_norm, am_norm, unigram); all but the first two are for the
+// backward.
+std::vector<torch::Tensor> LogprobsSmoothedForward(torch::Tensor lm, torch::Tensor am, torch::Tensor symbols,
+                                                   int termination_symbol, double lm_only_scale,
+                                                   double am_only_scale, int rnnt_type,
+                                                   torch::optional<torch::Tensor> boundary) {
+  ExpectFloat(am, "am", 3);
+  ExpectFloat(lm, "lm", 3);
+  ExpectRnntType(rnnt_type);
+  const int B = am.size(0), T = am.size(1), C = am.size(2), S = lm.size(1) - 1;
+  Expect(lm, "lm", am.scalar_type(), am.device(), {B, S + 1, C});
+  Expect(symbols, "symbols", torch::kLong, am.device(), {B, S});
+  ExpectOptional(boundary, "boundary", torch::kLong, am.device(), {B, 4});
+  ExpectSymbol(termination_symbol, C);
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(am.device());
+  auto opt = am.options();
+  const int joint_type = rnnt_type == K2AMD_REGULAR ? K2AMD_REGULAR : K2AMD_MODIFIED;
+  torch::Tensor px_joint = torch::empty({B, S, T1Of(T, rnnt_type)}, opt), py_joint = torch::empty({B, S + 1, T}, opt);
+  torch::Tensor px = torch::empty_like(px_joint), py = torch::empty_like(py_joint);
+  torch::Tensor lm_probs = torch::empty_like(lm), am_probs = torch::empty_like(am);
+  torch::Tensor lm_max = torch::empty({B, S + 1}, opt), am_max = torch::empty({B, T}, opt);
+  torch::Tensor lm_norm = torch::empty({B, S + 1}, opt), am_norm = torch::empty({B, T}, opt);
+  torch::Tensor denom = torch::empty({B, S + 1, T}, opt), unigram = torch::empty({2, C}, opt);
+  torch::Tensor scratch =
+      torch::empty({static_cast<int64_t>(k2amd_rnnt_smoothed_scratch_elements(B, S, T, C))}, opt);
+  void *stream = StreamOf(am);
+  {
+    pybind11::gil_scoped_release release;
+    Check(k2amd_rnnt_logprobs_simple_forward(
+        lm.data_ptr(), am.data_ptr(), I64(symbols), nullptr, px_joint.data_ptr(), py_joint.data_ptr(),
+        lm_probs.data_ptr(), am_probs.data_ptr(), lm_max.data_ptr(), am_max.data_ptr(), denom.data_ptr(), B, S, T,
+        C, termination_symbol, joint_type, DtypeCode(am), stream));
+    Check(k2amd_rnnt_smoothed_forward(
+        lm.data_ptr(), am.data_ptr(), I64(symbols), I64(boundary), lm_probs.data_ptr(), am_probs.data_ptr(),
+        lm_max.data_ptr(), am_max.data_ptr(), px_joint.data_ptr(), py_joint.data_ptr(), px.data_ptr(),
+        py.data_ptr(), lm_norm.data_ptr(), am_norm.data_ptr(), unigram.data_ptr(), scratch.data_ptr(),
+        static_cast<size_t>(scratch.numel()), lm_only_scale, am_only_scale, B, S, T, C, termination_symbol,
+        rnnt_type, DtypeCode(am), stream));
+  }
+  return {px, py, lm_probs, am_probs, denom, lm_max, am_max, lm_norm, am_norm, unigram};
+}
+
+// (lm_grad, am_grad): the simple builder's backward with the gradients scaled by
+// 1 - lm_only_scale - am_only_scale, then the marginal terms' gradients added.
+std::vector<torch::Tensor> LogprobsSmoothedBackward(
+    torch::Tensor px_grad, torch::Tensor py_grad, torch::Tensor symbols, torch::optional<torch::Tensor> boundary,
+    torch::Tensor lm_probs, torch::Tensor am_probs, torch::Tensor denom, torch::Tensor lm_max, torch::Tensor am_max,
+    torch::Tensor lm_norm, torch::Tensor am_norm, torch::Tensor unigram, int termination_symbol,
+    double lm_only_scale, double am_only_scale, int rnnt_type, torch::optional<torch::Tensor> seq_scale) {
+  ExpectFloat(am_probs, "am_probs", 3);
+  ExpectFloat(lm_probs, "lm_probs", 3);
+  ExpectRnntType(rnnt_type);
+  const int B = am_probs.size(0), T = am_probs.size(1), C = am_probs.size(2), S = lm_probs.size(1) - 1;
+  const auto dtype = am_probs.scalar_type();
+  const auto dev = am_probs.device();
+  Expect(lm_probs, "lm_probs", dtype, dev, {B, S + 1, C});
+  Expect(denom, "denom", dtype, dev, {B, S + 1, T});
+  Expect(lm_max, "lm_max", dtype, dev, {B, S + 1});
+  Expect(lm_norm, "lm_norm", dtype, dev, {B, S + 1});
+  Expect(am_max, "am_max", dtype, dev, {B, T});
+  Expect(am_norm, "am_norm", dtype, dev, {B, T});
+  Expect(unigram, "unigram", dtype, dev, {2, C});
+  Expect(symbols, "symbols", torch::kLong, dev, {B, S});
+  ExpectOptional(boundary, "boundary", torch::kLong, dev, {B, 4});
+  ExpectLatticeGrads(px_grad, py_grad, seq_scale, dtype, dev, B, S, T, rnnt_type);
+  ExpectSymbol(termination_symbol, C);
+  const void *scale = ScalePtr(seq_scale, px_grad);
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(dev);
+  const double joint_scale = 1.0 - lm_only_scale - am_only_scale;
+  torch::Tensor joint_seq_scale = scale != nullptr ? (*seq_scale * joint_scale).contiguous()
+                                                   : torch::full({B}, joint_scale, am_probs.options());
+  torch::Tensor lm_grad = torch::empty_like(lm_probs), am_grad = torch::empty_like(am_probs);
+  torch::Tensor q = torch::empty(
+      {static_cast<int64_t>(k2amd_rnnt_logprobs_simple_backward_scratch_elements(B, S, T))}, denom.options());
+  torch::Tensor scratch =
+      torch::empty({static_cast<int64_t>(k2amd_rnnt_smoothed_scratch_elements(B, S, T, C))}, denom.options());
+  void *stream = StreamOf(am_probs);
+  {
+    pybind11::gil_scoped_release release;
+    Check(k2amd_rnnt_logprobs_simple_backward(
+        px_grad.data_ptr(), py_grad.data_ptr(), joint_seq_scale.data_ptr(), I64(symbols), I64(boundary),
+        lm_probs.data_ptr(), am_probs.data_ptr(), denom.data_ptr(), lm_grad.data_ptr(), am_grad.data_ptr(),
+        q.data_ptr(), static_cast<size_t>(q.numel()), B, S, T, C, termination_symbol, rnnt_type,
+        DtypeCode(am_probs), stream));
+    Check(k2amd_rnnt_smoothed_backward(
+        px_grad.data_ptr(), py_grad.data_ptr(), scale, I64(symbols), I64(boundary), lm_probs.data_ptr(),
+        am_probs.data_ptr(), lm_max.data_ptr(), am_max.data_ptr(), lm_norm.data_ptr(), am_norm.data_ptr(),
+        unigram.data_ptr(), lm_grad.data_ptr(), am_grad.data_ptr(), scratch.data_ptr(),
+        static_cast<size_t>(scratch.numel()), lm_only_scale, am_only_scale, B, S, T, C, termination_symbol,
+        rnnt_type, DtypeCode(am_probs), stream));
+  }
+  return {lm_grad, am_grad};
+}
+
 // get_rnnt_logprobs_joint: returns (px, py, normalizers)
 std::vector<torch::Tensor> LogprobsJointForward(torch::Tensor logits, torch::Tensor symbols,
                                                 int termination_symbol, int rnnt_type,
@@ -789,6 +885,11 @@ PYBIND11_MODULE(_k2_amd, m) {
   m.def("version", []() { return k2amd_version(); });
   m.def("logprobs_simple_forward", &LogprobsSimpleForward);
   m.def("logprobs_simple_backward", &LogprobsSimpleBackward);
+  m.def("logprobs_smoothed_forward", &LogprobsSmoothedForward);
+  m.def("logprobs_smoothed_backward", &LogprobsSmoothedBackward);
+  m.def("smoothed_supported", [](int B, int S, int T, int C, int dtype) {
+    return k2amd_rnnt_smoothed_supported(B, S, T, C, dtype) != 0;
+  });
   m.def("logprobs_joint_forward", &LogprobsJointForward);
   m.def("logprobs_joint_backward", &LogprobsJointBackward);
   m.def("logprobs_pruned_forward", &LogprobsPrunedForward);

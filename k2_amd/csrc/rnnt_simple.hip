@@ -1016,8 +1016,10 @@ int k2amd_rnnt_logprobs_simple_backward(const void *px_grad, const void *py_grad
                                         int T, int C, int termination_symbol, int rnnt_type,
                                         int dtype, void *stream) {
   if (!ArgsOk(B, S, T, C, termination_symbol, rnnt_type, dtype)) return K2AMD_ERR_INVALID_ARGUMENT;
-  if (q_scratch == nullptr || q_scratch_elements < k2amd_rnnt_logprobs_simple_backward_scratch_elements(B, S, T))
-    return B == 0 ? K2AMD_OK : K2AMD_ERR_WORKSPACE;
+  {  // no frames or no sequences: nothing is asked for, and a null pointer is as good as any
+    const size_t need = k2amd_rnnt_logprobs_simple_backward_scratch_elements(B, S, T);
+    if (need > 0 && (q_scratch == nullptr || q_scratch_elements < need)) return K2AMD_ERR_WORKSPACE;
+  }
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == K2AMD_F32)
     return SimpleBackward<float>((const float *)px_grad, (const float *)py_grad, (const float *)seq_scale, symbols, boundary, (const float *)lm_probs, (const float *)am_probs, (const float *)denom, (float *)lm_grad, (float *)am_grad, (float *)q_scratch, B, S, T, C, termination_symbol, rnnt_type, st);

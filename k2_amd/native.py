@@ -198,6 +198,37 @@ def logprobs_simple_backward(px_grad, py_grad, symbols, boundary, saved, termina
                                          termination_symbol, rnnt_type, seq_scale)
 
 
+def smoothed_supported(lm, am):
+    """Whether the smoothed builder's kernels take these tensors (their vocabulary has to fit the
+    kernels' LDS arrays)."""
+    if _ext is not None:
+        return _ext.smoothed_supported(am.shape[0], lm.shape[1] - 1, am.shape[1], am.shape[2], capi.dtype_code(am))
+    return capi.smoothed_supported(lm, am)
+
+
+def logprobs_smoothed_forward(lm, am, symbols, termination_symbol, lm_only_scale, am_only_scale, rnnt_type,
+                              boundary):
+    """(px, py, saved) of get_rnnt_logprobs_smoothed; ``saved`` goes to logprobs_smoothed_backward."""
+    _require_device(am)
+    if _ext is not None:
+        out = _ext.logprobs_smoothed_forward(lm, am, symbols, termination_symbol, lm_only_scale, am_only_scale,
+                                             rnnt_type, boundary)
+        return out[0], out[1], tuple(out[2:])
+    return capi.logprobs_smoothed_forward(lm, am, symbols, termination_symbol, lm_only_scale, am_only_scale,
+                                          rnnt_type, boundary)
+
+
+def logprobs_smoothed_backward(px_grad, py_grad, symbols, boundary, saved, termination_symbol, lm_only_scale,
+                               am_only_scale, rnnt_type, seq_scale=None):
+    _require_device(px_grad)
+    if _ext is not None:
+        return tuple(_ext.logprobs_smoothed_backward(px_grad, py_grad, symbols, boundary, *saved,
+                                                     termination_symbol, lm_only_scale, am_only_scale, rnnt_type,
+                                                     seq_scale))
+    return capi.logprobs_smoothed_backward(px_grad, py_grad, symbols, boundary, saved, termination_symbol,
+                                           lm_only_scale, am_only_scale, rnnt_type, seq_scale)
+
+
 def logprobs_joint_forward(logits, symbols, termination_symbol, rnnt_type, boundary):
     _require_device(logits)
     if _ext is not None:

@@ -5,6 +5,7 @@ Where the reference chains 15-25 torch ops per call, each builder here is one fu
 (plus its hand-written backward), reached through a torch.autograd.Function so that
 ``loss.backward()`` works as before.  Tensors must live on a ROCm device.
 """
+import os
 from typing import Optional, Tuple, Union
 
 import torch
@@ -69,6 +70,36 @@ class _LogprobsSimple(torch.autograd.Function):
             px_grad.contiguous(), py_grad.contiguous(), symbols, boundary, ctx.saved_tensors,
             termination_symbol, rnnt_code)
         return lm_grad, am_grad, None, None, None, None
+
+
+class _LogprobsSmoothed(torch.autograd.Function):
+    """get_rnnt_logprobs_smoothed in the library's kernels: the simple builder, then the marginal
+    terms and the mix (k2_amd/csrc/rnnt_smoothed.hip)."""
+
+    @staticmethod
+    def forward(ctx, lm, am, symbols, termination_symbol, lm_only_scale, am_only_scale, rnnt_code, boundary):
+        px, py, saved = native.logprobs_smoothed_forward(lm.contiguous(), am.contiguous(), symbols,
+                                                        termination_symbol, lm_only_scale, am_only_scale,
+                                                        rnnt_code, boundary)
+        ctx.save_for_backward(*saved)
+        ctx.meta = (symbols, boundary, termination_symbol, lm_only_scale, am_only_scale, rnnt_code)
+        return px, py
+
+    @staticmethod
+    def backward(ctx, px_grad, py_grad):
+        symbols, boundary, termination_symbol, lm_only_scale, am_only_scale, rnnt_code = ctx.meta
+        lm_grad, am_grad = native.logprobs_smoothed_backward(
+            px_grad.contiguous(), py_grad.contiguous(), symbols, boundary, ctx.saved_tensors,
+            termination_symbol, lm_only_scale, am_only_scale, rnnt_code)
+        return lm_grad, am_grad, None, None, None, None, None, None
+
+
+def smoothed_kernels_enabled() -> bool:
+    """The marginal terms of get_rnnt_logprobs_smoothed have two implementations on the device:
+    torch ops (the default) and the library's own kernels, which so far have run only in their
+    host-thread build (tests/test_cpu_build_smoothed.py), never on a GPU; K2AMD_SMOOTHED_KERNELS=1
+    selects them."""
+    return os.environ.get("K2AMD_SMOOTHED_KERNELS", "0") == "1"
 
 
 class _LogprobsJoint(torch.autograd.Function):
@@ -545,9 +576,10 @@ def get_rnnt_logprobs_smoothed(
     log domain, the joint log-probs with "lm only" log-probs and "am only" log-probs (the latter
     against a unigram lm averaged over the batch).
 
-    Not on the accelerated path's critical list: the joint part (the only one of size
-    [B][S+1][T] x C) is the fused kernel of get_rnnt_logprobs; the two marginal parts are a dozen
-    torch ops on the device over [B][S+1][C] and [B][T][C]."""
+    The joint part (the only one of size [B][S+1][T] x C) is the fused kernel of
+    get_rnnt_logprobs.  The two marginal parts, over [B][S+1][C] and [B][T][C], and the mix are a
+    dozen torch ops on the device, or with K2AMD_SMOOTHED_KERNELS=1 the library's own kernels (see
+    smoothed_kernels_enabled)."""
     assert lm.ndim == 3, lm.shape
     assert am.ndim == 3, am.shape
     assert lm.shape[0] == am.shape[0], (lm.shape, am.shape)
@@ -560,6 +592,9 @@ def get_rnnt_logprobs_smoothed(
     regular = rnnt_type == "regular"
     symbols = _dev_i64(symbols, am)
     blank = int(termination_symbol)
+    if smoothed_kernels_enabled() and B > 0 and native.smoothed_supported(lm, am):
+        return _LogprobsSmoothed.apply(lm, am, symbols, blank, float(lm_only_scale), float(am_only_scale),
+                                       capi.RNNT_TYPES[rnnt_type], _dev_i64(boundary, am))
 
     # joint part, before the boundary fix / the "constrained" add (both come after interpolation)
     px, py = _LogprobsSimple.apply(lm, am, symbols, blank,

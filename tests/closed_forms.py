@@ -139,3 +139,53 @@ def _pruned_logits_grad(logits, symbols, ranges, blank, gxs, gys, scale, rnnt_ty
                 g[..., 0] = gxb * sig - gyb * (1.0 - sig)
             out[b] = scale[b] * g
     return outs
+
+
+def smoothed_grads(lm, am, symbols, blank, lm_only_scale, am_only_scale, gx, gy, scale, rnnt_type="regular"):
+    """(lm_grad, am_grad) of sum_b scale[b] * rnnt_loss_smoothed(...)[b]
+    (k2/python/k2/rnnt_loss.py:1471-1704).  Every lattice edge carries
+        joint_scale * log softmax(lm_s + am_t) + lm_only_scale * log softmax(lm_s)
+                                               + am_only_scale * log softmax(am_t + log unigram),
+    unigram = mean over all B (S+1) rows of softmax(lm) + tiny.  The joint term is the simple
+    loss's gradient times joint_scale.  With Wx, Wy the symbol / blank weights of a row summed over
+    its frames, the lm-only term gives row (b, s) of lm
+        lm_only_scale * (softmax(lm_s) (Wx + Wy) - Wx onehot(symbol_s) - Wy onehot(blank));
+    the am-only term gives row (b, t) of am the same shape of expression, dz, with the weights summed
+    over s and the symbol one-hots weighted one by one, and through the unigram it reaches every
+    row of lm:  softmax(lm_s) (dU - <softmax(lm_s), dU>) / (B (S+1)),  dU = sum_{b,t} dz / unigram."""
+    def one(gx, gy):
+        B, T, C = am.shape
+        S = lm.shape[1] - 1
+        joint_scale = 1.0 - lm_only_scale - am_only_scale
+        ls = lm_only_scale or 1.0e-20
+        as_ = am_only_scale or 1.0e-20
+        lm_g, am_g = _simple_grads(lm, am, symbols, blank, gx, gy, scale, rnnt_type, None)
+        lm_g *= joint_scale
+        am_g *= joint_scale
+        GX, GY = _edge_weights(gx, gy, rnnt_type)
+        w = np.asarray(scale, np.float64)
+        pl = _softmax(lm)                                              # [B][S+1][C]
+        unigram = pl.mean(axis=(0, 1)) + np.finfo(lm.dtype).tiny
+        pa = _softmax(am.astype(np.float64) + np.log(unigram))         # [B][T][C]
+        # lm only
+        wx, wy = GX.sum(axis=2), GY.sum(axis=2)                        # [B][S+1]
+        g = pl * (wx + wy)[..., None]
+        g[..., blank] -= wy
+        for b in range(B):
+            if S > 0:
+                np.subtract.at(g[b], (np.arange(S), symbols[b]), wx[b, :S])
+        lm_g += ls * w[:, None, None] * g
+        # am only
+        vx, vy = GX.sum(axis=1), GY.sum(axis=1)                        # [B][T]
+        dz = pa * (vx + vy)[..., None]
+        dz[..., blank] -= vy
+        for b in range(B):
+            if S > 0:
+                np.subtract.at(dz[b], (np.arange(T)[None, :].repeat(S, 0), symbols[b][:, None].repeat(T, 1)),
+                               GX[b, :S])
+        dz *= as_ * w[:, None, None]
+        am_g += dz
+        du = dz.sum(axis=(0, 1)) / unigram / (B * (S + 1))             # d loss / d softmax(lm)[b][s][c], any b, s
+        lm_g += pl * (du - (pl * du).sum(axis=-1, keepdims=True))
+        return lm_g, am_g
+    return _alternatives(lambda a, b: [one(x, y) for x, y in zip(a, b)], gx, gy)

@@ -1,0 +1,168 @@
+// A stand-in for <hip/hip_runtime.h> that runs HIP kernels on host threads, for tests only: the
+// same kernel source is compiled with g++ and every launch runs its workgroups one after the
+// other, each workgroup's work-items as threads of their own, so that barriers and wavefront
+// exchanges keep their meaning.  It covers the portable subset the row kernels use (no inline
+// assembly, no DPP, no matrix instructions) and lets a host sanitizer and a CPU debugger see the
+// kernels' indexing.  Slow by design: sizes stay small.
+#ifndef K2_AMD_TESTS_CPU_BUILD_HIP_RUNTIME_H_
+#define K2_AMD_TESTS_CPU_BUILD_HIP_RUNTIME_H_
+
+#include <math.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <string.h>
+
+#include <algorithm>
+#include <barrier>
+#include <cmath>
+#include <memory>
+#include <thread>
+#include <vector>
+
+#define __global__
+#define __device__
+#define __host__
+#define __forceinline__ inline __attribute__((always_inline))
+#define __launch_bounds__(...)
+#define __shared__ static
+// dynamic LDS, as HIP spells it
+#define HIP_DYNAMIC_SHARED(type, var) type *var = reinterpret_cast<type *>(hip_threads::state().dynamic_lds);
+
+typedef int hipError_t;
+constexpr hipError_t hipSuccess = 0;
+typedef void *hipStream_t;
+inline hipError_t hipGetLastError() { return hipSuccess; }
+
+struct dim3 {
+  unsigned x, y, z;
+  dim3(unsigned x_ = 1, unsigned y_ = 1, unsigned z_ = 1) : x(x_), y(y_), z(z_) {}
+};
+
+namespace hip_threads {
+
+constexpr int kWaveSize = 64;
+
+struct Wave {
+  std::unique_ptr<std::barrier<>> barrier;
+  int lanes;
+  // one exchange value per lane, two sets used in turn: a lane that is already writing for the
+  // next exchange cannot disturb one that still reads the last (each exchange has a barrier, so
+  // no lane is ever two exchanges ahead of another)
+  alignas(8) unsigned char slot[2][kWaveSize][8];
+};
+
+struct State {
+  unsigned char *dynamic_lds = nullptr;
+  std::barrier<> *block_barrier = nullptr;
+  std::vector<Wave> *waves = nullptr;
+};
+
+inline State &state() {
+  static State s;
+  return s;
+}
+
+struct Index {
+  unsigned x, y, z;
+};
+inline thread_local Index thread_idx, block_idx;
+inline thread_local int flat_thread;
+inline thread_local unsigned exchanges;  // this work-item's count of wavefront exchanges in the workgroup
+inline Index block_dim, grid_dim;
+
+inline Wave &my_wave() { return (*state().waves)[flat_thread / kWaveSize]; }
+
+template <typename T>
+inline T exchange(T v, int src_lane) {
+  static_assert(sizeof(T) <= 8, "");
+  Wave &w = my_wave();
+  const int lane = flat_thread % kWaveSize;
+  const unsigned set = exchanges++ & 1;
+  memcpy(w.slot[set][lane], &v, sizeof(T));
+  w.barrier->arrive_and_wait();
+  T r = v;  // a source outside the wavefront gives the lane's own value back; kernels must not rely on it
+  if (src_lane >= 0 && src_lane < w.lanes) memcpy(&r, w.slot[set][src_lane], sizeof(T));
+  return r;
+}
+
+template <typename Kernel, typename... Args>
+void launch(Kernel kernel, dim3 grid, dim3 block, size_t dynamic_lds_bytes, Args... args) {
+  const int threads = (int)(block.x * block.y * block.z);
+  const size_t blocks = (size_t)grid.x * grid.y * grid.z;
+  if (threads == 0 || blocks == 0) return;
+  block_dim = {block.x, block.y, block.z};
+  grid_dim = {grid.x, grid.y, grid.z};
+  // exactly the bytes asked for, on the heap: a sanitizer sees an access beyond them
+  std::unique_ptr<unsigned char[]> lds(new unsigned char[std::max<size_t>(dynamic_lds_bytes, 1)]);
+  state().dynamic_lds = lds.get();
+  // One set of threads for the whole launch; the workgroups run one after the other.  A work-item
+  // that leaves the kernel drops out of its wavefront's and its workgroup's barriers, as exited
+  // lanes and wavefronts do on the hardware, so those barriers are made anew for every workgroup.
+  std::unique_ptr<std::barrier<>> block_barrier;
+  std::vector<Wave> waves((threads + kWaveSize - 1) / kWaveSize);
+  auto fresh = [&] {
+    block_barrier.reset(new std::barrier<>(threads));
+    for (size_t w = 0; w < waves.size(); ++w) {
+      waves[w].lanes = std::min(kWaveSize, threads - (int)w * kWaveSize);
+      waves[w].barrier.reset(new std::barrier<>(waves[w].lanes));
+    }
+    state().block_barrier = block_barrier.get();
+  };
+  fresh();
+  state().waves = &waves;
+  std::barrier<> between(threads);
+  std::vector<std::thread> pool;
+  pool.reserve(threads);
+  for (int t = 0; t < threads; ++t)
+    pool.emplace_back([&, t] {
+      flat_thread = t;
+      thread_idx = {t % block.x, (t / block.x) % block.y, t / (block.x * block.y)};
+      for (size_t k = 0; k < blocks; ++k) {
+        exchanges = 0;
+        block_idx = {(unsigned)(k % grid.x), (unsigned)((k / grid.x) % grid.y), (unsigned)(k / ((size_t)grid.x * grid.y))};
+        kernel(args...);
+        my_wave().barrier->arrive_and_drop();
+        state().block_barrier->arrive_and_drop();
+        between.arrive_and_wait();
+        if (t == 0) fresh();
+        between.arrive_and_wait();
+      }
+    });
+  for (auto &th : pool) th.join();
+  state().dynamic_lds = nullptr;
+  state().block_barrier = nullptr;
+  state().waves = nullptr;
+}
+
+}  // namespace hip_threads
+
+#define threadIdx hip_threads::thread_idx
+#define blockIdx hip_threads::block_idx
+#define blockDim hip_threads::block_dim
+#define gridDim hip_threads::grid_dim
+
+#define hipLaunchKernelGGL(kernel, grid, block, lds_bytes, stream, ...) \
+  hip_threads::launch(kernel, grid, block, lds_bytes, __VA_ARGS__)
+
+inline void __syncthreads() { hip_threads::state().block_barrier->arrive_and_wait(); }
+
+template <typename T>
+inline T __shfl_xor(T v, int mask, int width = hip_threads::kWaveSize) {
+  (void)width;
+  return hip_threads::exchange(v, (hip_threads::flat_thread % hip_threads::kWaveSize) ^ mask);
+}
+template <typename T>
+inline T __shfl(T v, int src_lane, int width = hip_threads::kWaveSize) {
+  (void)width;
+  return hip_threads::exchange(v, src_lane);
+}
+inline int __any(int predicate) {
+  int r = predicate != 0;
+  for (int off = 32; off > 0; off >>= 1) r |= __shfl_xor(r, off);
+  return r;
+}
+
+using std::max;
+using std::min;
+
+#endif  // K2_AMD_TESTS_CPU_BUILD_HIP_RUNTIME_H_

@@ -70,3 +70,23 @@ def test_pruned_closed_form_equals_autograd(rnnt_type, hat):
     got = cf.pruned_logits_grad(logits, c["symbols"], ranges, 0, gx, gy, np.where(ok.numpy(), w, 0.0),
                                 rnnt_type, hat=hat)
     np.testing.assert_allclose(got, lg.grad.numpy(), rtol=1e-9, atol=1e-12)
+
+
+@pytest.mark.parametrize("scales", [(0.25, 0.1), (0.0, 0.3), (0.4, 0.0)])
+@pytest.mark.parametrize("rnnt_type", TYPES)
+def test_smoothed_closed_form_equals_autograd(rnnt_type, scales):
+    B, T, S, C = 3, 9, 4, 6
+    c = cases.rnnt_case(65, B, T, S, C, dtype=np.float64, t_lo=6, s_lo=2, modified=rnnt_type != "regular")
+    bd = torch.from_numpy(c["boundary"])
+    w = np.linspace(0.5, 1.5, B)
+    lm = torch.from_numpy(c["lm"]).requires_grad_(True)
+    am = torch.from_numpy(c["am"]).requires_grad_(True)
+    px, py = torch_ref.logprobs_smoothed(lm, am, torch.from_numpy(c["symbols"]), 0, scales[0], scales[1],
+                                         rnnt_type, bd)
+    (-torch_ref.mi_scores(px, py, bd) * torch.from_numpy(w)).sum().backward()
+    opx, opy = orn.logprobs_smoothed(c["lm"], c["am"], c["symbols"], 0, scales[0], scales[1], c["boundary"],
+                                     rnnt_type)
+    _, gx, gy = omi.mi(opx, opy, c["boundary"])
+    lm_g, am_g = cf.smoothed_grads(c["lm"], c["am"], c["symbols"], 0, scales[0], scales[1], gx, gy, w, rnnt_type)
+    np.testing.assert_allclose(lm_g, lm.grad.numpy(), rtol=1e-9, atol=1e-12)
+    np.testing.assert_allclose(am_g, am.grad.numpy(), rtol=1e-9, atol=1e-12)
