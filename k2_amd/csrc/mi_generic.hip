@@ -18,7 +18,7 @@ template <typename T>
 __global__ __launch_bounds__(kThreads) void MiForwardGenericKernel(
     const T *__restrict__ px, const T *__restrict__ py, const int64_t *__restrict__ boundary,
     T *__restrict__ p, T *__restrict__ ans, int S, int Tn, int modified) {
-  extern __shared__ unsigned char smem_raw[];
+  HIP_DYNAMIC_SHARED(unsigned char, smem_raw)
   T *prev = reinterpret_cast<T *>(smem_raw);
   T *cur = prev + (S + 2);
   const int b = blockIdx.x;
@@ -36,7 +36,7 @@ __global__ __launch_bounds__(kThreads) void MiBackwardGenericKernel(
     const T *__restrict__ px, const T *__restrict__ p, const int64_t *__restrict__ boundary,
     T *__restrict__ ans_grad, T *__restrict__ px_grad, T *__restrict__ py_grad, int S, int Tn,
     int modified, int overwrite_ans_grad) {
-  extern __shared__ unsigned char smem_raw[];
+  HIP_DYNAMIC_SHARED(unsigned char, smem_raw)
   T *gprev = reinterpret_cast<T *>(smem_raw);
   T *gcur = gprev + (S + 2);
   const int b = blockIdx.x;

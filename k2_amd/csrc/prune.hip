@@ -124,7 +124,7 @@ void LaunchArgmax(const T *px_grad, const T *py_grad, int64_t *ranges, int S, in
 // written over the raw arg-max values.
 __global__ __launch_bounds__(kPruneThreads) void PruneFinishKernel(
     const int64_t *__restrict__ boundary, int64_t *__restrict__ ranges, int Tn, int modified, int R) {
-  extern __shared__ int lds[];
+  HIP_DYNAMIC_SHARED(int, lds)
   int *buf0 = lds, *buf1 = lds + Tn;
   const int b = blockIdx.x;
   const int64_t s_end = boundary[4 * b + 2], t_end = boundary[4 * b + 3];
@@ -196,7 +196,7 @@ template <typename T, int kVec>
 __global__ __launch_bounds__(kGatherThreads) void GatherBackwardKernel(
     const T *__restrict__ grad, const int64_t *__restrict__ ranges, T *__restrict__ lm_grad, int S1,
     int TR, int D) {
-  extern __shared__ unsigned char gather_smem[];
+  HIP_DYNAMIC_SHARED(unsigned char, gather_smem)
   int *found = reinterpret_cast<int *>(gather_smem);  // [TR] row numbers, in order
   __shared__ int counts[kGatherThreads + 1];
   const int b = blockIdx.x / S1, s = blockIdx.x - b * S1;

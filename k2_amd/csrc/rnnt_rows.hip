@@ -338,6 +338,9 @@ __global__ __launch_bounds__(kRowsPerBlock *kWave) void RowGradKernel(
   terms.norm = dx[3];
   terms.blank = blank;
   terms.sg = kHat ? Sigmoid(x[0]) : T(0);
+  // every lane has the record before any lane's store below overwrites it: a wavefront's lanes
+  // run in lockstep, so this emits no instruction; it states the dependence
+  __builtin_amdgcn_wave_barrier();
   if (vectorised) {
     V *dv = reinterpret_cast<V *>(dx);
     V outv[kMaxVecs];
@@ -359,8 +362,7 @@ __global__ __launch_bounds__(kRowsPerBlock *kWave) void RowGradKernel(
     }
     return;
   }
-  // rows that are not read as vectors: every lane holds the record in registers before the
-  // first store of the loop below can reach it (a wavefront's loads complete in order)
+  // rows that are not read as vectors
   for (int c = lane; c < C; c += kWave) dx[c] = terms.template At<false>(x[c], c);
 }
 

@@ -13,6 +13,7 @@
 #include <string.h>
 
 #include <algorithm>
+#include <atomic>
 #include <barrier>
 #include <cmath>
 #include <memory>
@@ -110,7 +111,8 @@ void launch(Kernel kernel, dim3 grid, dim3 block, size_t dynamic_lds_bytes, Args
   };
   fresh();
   state().waves = &waves;
-  std::barrier<> between(threads);
+  auto renew = [&]() noexcept { fresh(); };  // runs once all have arrived, before any goes on
+  std::barrier<decltype(renew)> between(threads, renew);
   std::vector<std::thread> pool;
   pool.reserve(threads);
   for (int t = 0; t < threads; ++t)
@@ -123,8 +125,6 @@ void launch(Kernel kernel, dim3 grid, dim3 block, size_t dynamic_lds_bytes, Args
         kernel(args...);
         my_wave().barrier->arrive_and_drop();
         state().block_barrier->arrive_and_drop();
-        between.arrive_and_wait();
-        if (t == 0) fresh();
         between.arrive_and_wait();
       }
     });
@@ -156,6 +156,9 @@ inline T __shfl(T v, int src_lane, int width = hip_threads::kWaveSize) {
   (void)width;
   return hip_threads::exchange(v, src_lane);
 }
+// On the hardware a scheduling fence that emits nothing (a wavefront's lanes run in lockstep);
+// here the lanes are free-running threads, so it has to be a real barrier over the wavefront.
+inline void __builtin_amdgcn_wave_barrier() { hip_threads::my_wave().barrier->arrive_and_wait(); }
 inline int __any(int predicate) {
   int r = predicate != 0;
   for (int off = 32; off > 0; off >>= 1) r |= __shfl_xor(r, off);
@@ -164,5 +167,56 @@ inline int __any(int predicate) {
 
 using std::max;
 using std::min;
+
+// ---- vector types (no alignment beyond the element's: host buffers need not be 16-byte aligned) --
+struct float2 { float x, y; };
+struct float4 { float x, y, z, w; };
+struct double2 { double x, y; };
+struct int2 { int x, y; };
+struct int4 { int x, y, z, w; };
+inline float2 make_float2(float x, float y) { return {x, y}; }
+inline float4 make_float4(float x, float y, float z, float w) { return {x, y, z, w}; }
+inline double2 make_double2(double x, double y) { return {x, y}; }
+inline int2 make_int2(int x, int y) { return {x, y}; }
+inline int4 make_int4(int x, int y, int z, int w) { return {x, y, z, w}; }
+
+// ---- atomics: work-items of one workgroup are threads, so these have to be real ----------------
+template <typename T>
+inline T atomicAdd(T *address, T value) { return std::atomic_ref<T>(*address).fetch_add(value); }
+template <typename T>
+inline T unsafeAtomicAdd(T *address, T value) { return atomicAdd(address, value); }
+template <typename T>
+inline T atomicMax(T *address, T value) {
+  std::atomic_ref<T> a(*address);
+  T old = a.load();
+  while (old < value && !a.compare_exchange_weak(old, value)) {}
+  return old;
+}
+
+inline float __expf(float x) { return expf(x); }
+inline float __logf(float x) { return logf(x); }
+
+// ---- IEEE half, as storage with a conversion (hip_fp16.h's __half) -----------------------------
+struct __half { uint16_t bits; };
+inline float __half2float(__half h) {
+  const uint32_t sign = (uint32_t)(h.bits & 0x8000u) << 16, exponent = (h.bits >> 10) & 0x1fu, mantissa = h.bits & 0x3ffu;
+  uint32_t u;
+  if (exponent == 0) {
+    if (mantissa == 0) {
+      u = sign;
+    } else {  // subnormal: value = mantissa * 2^-24
+      float f = (float)mantissa * 5.9604644775390625e-8f;
+      memcpy(&u, &f, 4);
+      u |= sign;
+    }
+  } else if (exponent == 31) {
+    u = sign | 0x7f800000u | (mantissa << 13);
+  } else {
+    u = sign | ((exponent + 112) << 23) | (mantissa << 13);
+  }
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+}
 
 #endif  // K2_AMD_TESTS_CPU_BUILD_HIP_RUNTIME_H_

@@ -1,0 +1,120 @@
+"""The library's portable HIP kernels compiled for the host (tests only).
+
+k2_amd/csrc/{rnnt_rows, prune, lattice, mi_joint, mi_generic, rnnt_smoothed}.hip use nothing but
+plain HIP (LDS, barriers, wavefront shuffles, atomics): g++ compiles the SAME sources over the
+thread stand-in of tests/cpu_build/hip/hip_runtime.h into one shared library, whose C-ABI entry
+points then take numpy buffers.  The ctypes signatures are k2_amd/capi.py's own table, so a wrong
+entry there shows up here as well.  The kernels that need the hardware (inline assembly, DPP,
+matrix instructions: mi_fast, mi_wave, rnnt_simple's products, joiner) are not part of it.
+
+Fenced arrays: a numpy array whose last byte sits directly in front of an inaccessible page (or
+whose first byte directly behind one), so that a kernel reading or writing past the end of a
+tensor stops the test run with a segmentation fault instead of passing unnoticed.
+"""
+import ctypes
+import mmap
+import os
+import subprocess
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(ROOT, "k2_amd", "csrc")
+SHIM = os.path.join(HERE, "cpu_build")
+OUT = os.path.join(SHIM, "_build")
+PORTABLE = ["rnnt_rows", "prune", "lattice", "mi_joint", "mi_generic", "rnnt_smoothed"]
+# -ffp-contract=off: a * b + c rounds twice, as in the reference's CPU loops (the exact
+# mutual-information kernels are compared with them bit for bit)
+FLAGS = ["-std=c++20", "-O1", "-g", "-fPIC", "-pthread", "-ffp-contract=off", f"-I{SHIM}", f"-I{CSRC}"]
+
+_lib = None
+
+
+def build():
+    """Compiles the portable sources and tests/cpu_build/entry.cc into _build/libk2amd_cpu.so."""
+    os.makedirs(OUT, exist_ok=True)
+    jobs = []
+    for name in PORTABLE + ["entry"]:
+        src = os.path.join(CSRC, name + ".hip") if name != "entry" else os.path.join(SHIM, "entry.cc")
+        obj = os.path.join(OUT, name + ".o")
+        jobs.append((src, obj, subprocess.Popen(["g++", *FLAGS, "-x", "c++", "-c", src, "-o", obj],
+                                                stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+    for src, _, proc in jobs:
+        out, _ = proc.communicate()
+        assert proc.returncode == 0, f"g++ failed on {src}\n{out}"
+    path = os.path.join(OUT, "libk2amd_cpu.so")
+    proc = subprocess.run(["g++", "-shared", "-pthread", "-o", path, *[j[1] for j in jobs]],
+                          stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert proc.returncode == 0, proc.stdout
+    return path
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        from k2_amd import capi
+        _lib = ctypes.CDLL(build())
+        for name, (argtypes, restype) in capi._SIGNATURES.items():
+            if hasattr(_lib, name):
+                fn = getattr(_lib, name)
+                fn.argtypes, fn.restype = argtypes, restype
+        vp, ci = ctypes.c_void_p, ctypes.c_int
+        _lib.cpu_mi_forward_generic.argtypes = [vp] * 5 + [ci] * 5
+        _lib.cpu_mi_backward_generic.argtypes = [vp] * 6 + [ci] * 6
+    return _lib
+
+
+_PAGE = mmap.PAGESIZE
+_libc = ctypes.CDLL(None, use_errno=True)
+_libc.mprotect.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+
+
+class Fenced:
+    """``.a``: an array of the given shape and dtype next to a page that may not be touched:
+    behind its last element (at="end", the default) or in front of its first (at="start").  The
+    other side, up to the page boundary, carries a pattern that ``intact()`` checks."""
+
+    PATTERN = 0xA5
+
+    def __init__(self, shape, dtype, fill=None, at="end"):
+        dtype = np.dtype(dtype)
+        n = int(np.prod(shape, dtype=np.int64))
+        nbytes = n * dtype.itemsize
+        pages = max(1, -(-nbytes // _PAGE))
+        self.map = mmap.mmap(-1, (pages + 1) * _PAGE)
+        self.buf = np.frombuffer(self.map, dtype=np.uint8)
+        base = self.buf.ctypes.data
+        assert base % _PAGE == 0
+        if at == "end":
+            guard, start = base + pages * _PAGE, pages * _PAGE - nbytes
+            self.slack = slice(0, start)
+        else:
+            guard, start = base, _PAGE
+            self.slack = slice(_PAGE + nbytes, (pages + 1) * _PAGE)
+        self.buf[self.slack] = self.PATTERN
+        if _libc.mprotect(guard, _PAGE, 0) != 0:
+            raise OSError(ctypes.get_errno(), "mprotect")
+        self.a = self.buf[start:start + nbytes].view(dtype).reshape(shape)
+        if fill is not None:
+            self.a[...] = fill
+
+    def intact(self):
+        return bool((self.buf[self.slack] == self.PATTERN).all())
+
+
+def fenced(array, at="end"):
+    """A fenced copy of ``array`` (None stays None)."""
+    if array is None:
+        return None
+    f = Fenced(array.shape, array.dtype, at=at)
+    f.a[...] = array
+    return f
+
+
+def p(x):
+    """The pointer ctypes passes for a Fenced, a numpy array or None."""
+    if x is None:
+        return None
+    a = x.a if isinstance(x, Fenced) else x
+    return ctypes.c_void_p(a.ctypes.data)

@@ -39,15 +39,8 @@ def _compile(args, out):
 
 @pytest.fixture(scope="module")
 def lib():
-    path = _compile(["-shared", "-fPIC", "-x", "c++", SRC], os.path.join(OUT, "libsmoothed_cpu.so"))
-    lib = ctypes.CDLL(path)
-    vp, i64p, ci, cd, sz = ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_double, ctypes.c_size_t
-    lib.k2amd_rnnt_smoothed_scratch_elements.restype = sz
-    lib.k2amd_rnnt_smoothed_scratch_elements.argtypes = [ci] * 4
-    lib.k2amd_rnnt_smoothed_supported.argtypes = [ci] * 5
-    lib.k2amd_rnnt_smoothed_forward.argtypes = [vp, vp, i64p, i64p] + [vp] * 12 + [sz, cd, cd] + [ci] * 7 + [vp]
-    lib.k2amd_rnnt_smoothed_backward.argtypes = [vp, vp, vp, i64p, i64p] + [vp] * 10 + [sz, cd, cd] + [ci] * 7 + [vp]
-    return lib
+    import cpu_kernels
+    return cpu_kernels.lib()  # the host build of all portable kernels, k2_amd/capi.py's signatures
 
 
 def _p(a):
