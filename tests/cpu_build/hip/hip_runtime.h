@@ -50,6 +50,7 @@ struct Wave {
   // next exchange cannot disturb one that still reads the last (each exchange has a barrier, so
   // no lane is ever two exchanges ahead of another)
   alignas(8) unsigned char slot[2][kWaveSize][8];
+  float matrix_a[2][kWaveSize], matrix_b[2][kWaveSize];  // the operands of a matrix instruction, likewise
 };
 
 struct State {
@@ -156,6 +157,33 @@ inline T __shfl(T v, int src_lane, int width = hip_threads::kWaveSize) {
   (void)width;
   return hip_threads::exchange(v, src_lane);
 }
+// ---- what the fp32 matrix-core products of rnnt_simple.hip use --------------------------------
+// clang's ext_vector_type for FLOAT vectors (the only ones in the files of the host build)
+#define ext_vector_type(n) vector_size(4 * (n))
+#define __builtin_amdgcn_fence(...) ((void)0)
+#define __builtin_amdgcn_sched_barrier(mask) ((void)0)
+inline void __builtin_amdgcn_s_barrier() { __syncthreads(); }
+
+// v_mfma_f32_32x32x2_f32: D = A (32 x 2) * B (2 x 32) + C over the wavefront.  Lane l supplies
+// A[l % 32][l / 32] and B[l / 32][l % 32] and holds, in element v of its 16, D[i][l % 32] with
+// i = 8 (v / 4) + 4 (l / 32) + v % 4.
+typedef float hip_threads_float16 __attribute__((vector_size(64)));
+inline hip_threads_float16 __builtin_amdgcn_mfma_f32_32x32x2f32(float a, float b, hip_threads_float16 c, int, int,
+                                                               int) {
+  hip_threads::Wave &w = hip_threads::my_wave();
+  const int lane = hip_threads::flat_thread % hip_threads::kWaveSize;
+  const unsigned set = hip_threads::exchanges++ & 1;
+  w.matrix_a[set][lane] = a;
+  w.matrix_b[set][lane] = b;
+  w.barrier->arrive_and_wait();
+  const int j = lane % 32;
+  for (int v = 0; v < 16; ++v) {
+    const int i = 8 * (v / 4) + 4 * (lane / 32) + v % 4;
+    c[v] += w.matrix_a[set][i] * w.matrix_b[set][j] + w.matrix_a[set][i + 32] * w.matrix_b[set][j + 32];
+  }
+  return c;
+}
+
 // On the hardware a scheduling fence that emits nothing (a wavefront's lanes run in lockstep);
 // here the lanes are free-running threads, so it has to be a real barrier over the wavefront.
 inline void __builtin_amdgcn_wave_barrier() { hip_threads::my_wave().barrier->arrive_and_wait(); }

@@ -298,3 +298,147 @@ def test_joint_products(lib, dtype):
                          for n in range(N)])
         np.testing.assert_allclose(prods.a, want, **(dict(rtol=1e-12) if dtype == np.float64 else dict(rtol=2e-5)))
         assert prods.intact() and scratch.intact()
+
+
+# ---- get_rnnt_logprobs (rnnt_simple.hip) and the smoothed builder on top of it ------------------
+
+def _simple_forward(lib, c, rnnt_type, bd, at="end"):
+    lm, am, sym = c["lm"], c["am"], c["symbols"]
+    dt = lm.dtype
+    B, T, C = am.shape
+    S = lm.shape[1] - 1
+    T1 = T + 1 if rnnt_type == "regular" else T
+    out = dict(px=Fenced((B, S, T1), dt, np.nan, at), py=Fenced((B, S + 1, T), dt, np.nan, at),
+               lm_probs=Fenced(lm.shape, dt, np.nan, at), am_probs=Fenced(am.shape, dt, np.nan, at),
+               lm_max=Fenced((B, S + 1), dt, np.nan, at), am_max=Fenced((B, T), dt, np.nan, at),
+               denom=Fenced((B, S + 1, T), dt, np.nan, at),
+               lm=fenced(lm, at), am=fenced(am, at), sym=fenced(sym, at), bd=fenced(bd, at))
+    assert lib.k2amd_rnnt_logprobs_simple_forward(
+        p(out["lm"]), p(out["am"]), p(out["sym"]), p(out["bd"]), p(out["px"]), p(out["py"]), p(out["lm_probs"]),
+        p(out["am_probs"]), p(out["lm_max"]), p(out["am_max"]), p(out["denom"]), B, S, T, C, 0, CODES[rnnt_type],
+        dcode(dt), None) == 0
+    for k in ("px", "py", "lm_probs", "am_probs", "lm_max", "am_max", "denom"):
+        assert out[k].intact(), k
+    return out
+
+
+def _simple_backward(lib, f, gx, gy, w, rnnt_type, at="end"):
+    dt = f["lm"].a.dtype
+    B, T, C = f["am"].a.shape
+    S = f["lm"].a.shape[1] - 1
+    keep = Inputs(at)
+    lm_grad, am_grad = Fenced(f["lm"].a.shape, dt, np.nan, at), Fenced(f["am"].a.shape, dt, np.nan, at)
+    n = lib.k2amd_rnnt_logprobs_simple_backward_scratch_elements(B, S, T)
+    q = Fenced((n,), dt, np.nan, at)
+    args = (keep(gx.astype(dt)), keep(gy.astype(dt)), None if w is None else keep(w.astype(dt)), p(f["sym"]),
+            p(f["bd"]), p(f["lm_probs"]), p(f["am_probs"]), p(f["denom"]), p(lm_grad), p(am_grad), p(q))
+    dims = (B, S, T, C, 0, CODES[rnnt_type], dcode(dt), None)
+    if n > 0:
+        assert lib.k2amd_rnnt_logprobs_simple_backward(*args, n - 1, *dims) == 3  # too little scratch: refused
+        assert np.isnan(lm_grad.a).all()
+    assert lib.k2amd_rnnt_logprobs_simple_backward(*args, n, *dims) == 0
+    assert lm_grad.intact() and am_grad.intact() and q.intact()
+    return lm_grad, am_grad
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("rnnt_type", TYPES)
+def test_simple_builder(lib, rnnt_type, dtype):
+    """Forward against the oracle, backward against the closed form; fp32 through the emulated
+    matrix instruction (the kernel for small products), fp64 on the vector path."""
+    at = "start" if rnnt_type == "constrained" else "end"
+    for k, (B, T, S, C) in enumerate(((2, 9, 4, 7), (1, 70, 33, 70), (3, 33, 0, 5))):
+        c = cases.rnnt_case(700 + k, B, T, S, C, dtype=dtype, t_lo=max(S, T - 3), s_lo=max(0, S - 2),
+                            modified=rnnt_type != "regular")
+        if S > 1:
+            c["symbols"][:, 1] = c["symbols"][:, 0]
+        bd = c["boundary"] if k != 1 else None
+        f = _simple_forward(lib, c, rnnt_type, bd, at)
+        wpx, wpy = orn.logprobs_simple(c["lm"], c["am"], c["symbols"], 0, rnnt_type, bd)
+        np.testing.assert_allclose(f["px"].a, wpx, **TOL[np.dtype(dtype)])
+        np.testing.assert_allclose(f["py"].a, wpy, **TOL[np.dtype(dtype)])
+        _, gx, gy = omi.mi(wpx.astype(np.float64), wpy.astype(np.float64), bd)
+        w = np.linspace(0.5, 1.5, B)
+        want_lm, want_am = cf.simple_grads(c["lm"], c["am"], c["symbols"], 0, gx, gy, -w, rnnt_type)
+        lm_grad, am_grad = _simple_backward(lib, f, gx, gy, w, rnnt_type, at)
+        tol = dict(rtol=1e-8, atol=1e-10) if dtype == np.float64 else dict(rtol=1e-3, atol=1e-5)
+        np.testing.assert_allclose(lm_grad.a, want_lm, **tol)
+        np.testing.assert_allclose(am_grad.a, want_am, **tol)
+
+
+def test_simple_builder_without_frames(lib):
+    """T = 0: px is its one -inf column, the lm gradient all zeros; the backward needs no scratch
+    and takes a null pointer for it."""
+    B, S, C = 2, 3, 5
+    c = cases.rnnt_case(710, B, 0, S, C, dtype=np.float32, with_boundary=False)
+    f = _simple_forward(lib, c, "regular", None)
+    assert np.isneginf(f["px"].a).all()
+    lm_grad = Fenced(c["lm"].shape, np.float32, np.nan)
+    assert lib.k2amd_rnnt_logprobs_simple_backward_scratch_elements(B, S, 0) == 0
+    assert lib.k2amd_rnnt_logprobs_simple_backward(None, None, None, p(f["sym"]), None, p(f["lm_probs"]), None, None,
+                                                   p(lm_grad), None, None, 0, B, S, 0, C, 0, 0, 0, None) == 0
+    assert (lm_grad.a == 0).all() and lm_grad.intact()
+
+
+@pytest.mark.skipif(os.environ.get("K2AMD_SLOW_CPU_TESTS", "0") != "1",
+                    reason="ten minutes on eight cores: run with K2AMD_SLOW_CPU_TESTS=1")
+def test_simple_builder_lds_tiled_products(lib):
+    """A shape large enough for the 64 x 64 LDS-tiled product kernel (it takes over at 512 tiles):
+    the forward product (both operands contiguous along k) and the am-gradient product (neither).
+    Hundreds of workgroups of 256 threads each: slow on the host, so not part of the default run."""
+    B, T, S, C = 16, 1000, 127, 130
+    c = cases.rnnt_case(720, B, T, S, C, dtype=np.float32, t_lo=900, s_lo=100)
+    f = _simple_forward(lib, c, "regular", c["boundary"])
+    wpx, wpy = orn.logprobs_simple(c["lm"], c["am"], c["symbols"], 0, "regular", c["boundary"])
+    np.testing.assert_allclose(f["px"].a, wpx, rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(f["py"].a, wpy, rtol=1e-4, atol=1e-5)
+    rng = np.random.default_rng(721)
+    gx, gy = rng.uniform(0, 1e-2, wpx.shape), rng.uniform(0, 1e-2, wpy.shape)
+    gx[:, :, T] = 0.0
+    for b in range(B):
+        gx[b, :, c["boundary"][b, 3]] = 0.0
+    lm_grad, am_grad = _simple_backward(lib, f, gx, gy, None, "regular")
+    for b in (0, B - 1):  # the closed form holds a [S+1][T][C] tensor per sequence: two of them will do
+        one = {k: c[k][b:b + 1] for k in ("lm", "am", "symbols")}
+        want_lm, want_am = cf.simple_grads(one["lm"], one["am"], one["symbols"], 0, gx[b:b + 1], gy[b:b + 1],
+                                           -np.ones(1), "regular")
+        np.testing.assert_allclose(lm_grad.a[b:b + 1], want_lm, rtol=1e-3, atol=1e-5)
+        np.testing.assert_allclose(am_grad.a[b:b + 1], want_am, rtol=1e-3, atol=1e-5)
+
+
+@pytest.mark.parametrize("rnnt_type", TYPES)
+def test_smoothed_chain_end_to_end(lib, rnnt_type):
+    """The two calls per direction that make up get_rnnt_logprobs_smoothed, all in the kernels:
+    simple builder without a boundary, mix; simple builder's backward with the scaled weights,
+    marginal terms added.  Against the oracle and the closed-form gradients."""
+    B, T, S, C = 3, 11, 6, 70
+    scales = (0.25, 0.1)
+    c = cases.rnnt_case(730, B, T, S, C, dtype=np.float64, t_lo=8, s_lo=3, modified=rnnt_type != "regular")
+    bd = c["boundary"]
+    f = _simple_forward(lib, c, "regular" if rnnt_type == "regular" else "modified", None)
+    T1 = T + 1 if rnnt_type == "regular" else T
+    dt = np.float64
+    px, py = Fenced((B, S, T1), dt, np.nan), Fenced((B, S + 1, T), dt, np.nan)
+    lm_norm, am_norm, unigram = Fenced((B, S + 1), dt, np.nan), Fenced((B, T), dt, np.nan), Fenced((2, C), dt, np.nan)
+    n = lib.k2amd_rnnt_smoothed_scratch_elements(B, S, T, C)
+    scratch, fbd = Fenced((n,), dt, np.nan), fenced(bd)
+    dims = (B, S, T, C, 0, CODES[rnnt_type], 1, None)
+    assert lib.k2amd_rnnt_smoothed_forward(
+        p(f["lm"]), p(f["am"]), p(f["sym"]), p(fbd), p(f["lm_probs"]), p(f["am_probs"]), p(f["lm_max"]),
+        p(f["am_max"]), p(f["px"]), p(f["py"]), p(px), p(py), p(lm_norm), p(am_norm), p(unigram), p(scratch), n,
+        *scales, *dims) == 0
+    wpx, wpy = orn.logprobs_smoothed(c["lm"], c["am"], c["symbols"], 0, scales[0], scales[1], bd, rnnt_type)
+    np.testing.assert_allclose(px.a, wpx, rtol=1e-10, atol=1e-10)
+    np.testing.assert_allclose(py.a, wpy, rtol=1e-10, atol=1e-10)
+    _, gx, gy = omi.mi(wpx, wpy, bd)
+    w = np.linspace(0.5, 1.5, B)
+    f["bd"] = fbd  # the backward of the joint term sees the real boundary and lattice type
+    lm_grad, am_grad = _simple_backward(lib, f, gx, gy, w * (1.0 - scales[0] - scales[1]), rnnt_type)
+    keep = Inputs()
+    assert lib.k2amd_rnnt_smoothed_backward(
+        keep(gx), keep(gy), keep(w), p(f["sym"]), p(fbd), p(f["lm_probs"]), p(f["am_probs"]), p(f["lm_max"]),
+        p(f["am_max"]), p(lm_norm), p(am_norm), p(unigram), p(lm_grad), p(am_grad), p(scratch), n, *scales,
+        *dims) == 0
+    want_lm, want_am = cf.smoothed_grads(c["lm"], c["am"], c["symbols"], 0, scales[0], scales[1], gx, gy, -w, rnnt_type)
+    np.testing.assert_allclose(lm_grad.a, want_lm, rtol=1e-8, atol=1e-10)
+    np.testing.assert_allclose(am_grad.a, want_am, rtol=1e-8, atol=1e-10)
