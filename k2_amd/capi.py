@@ -104,10 +104,15 @@ def dtype_code(t):
     raise RuntimeError(f"k2_amd: unsupported dtype {t.dtype} (float32 / float64 only)")
 
 
+def _on_device(t):
+    """The one place that decides whether a tensor's memory is the GPU's."""
+    return t.is_cuda
+
+
 def ptr(t):
     if t is None:
         return None
-    assert t.is_cuda and t.is_contiguous(), "k2_amd C-ABI takes contiguous device tensors"
+    assert _on_device(t) and t.is_contiguous(), "k2_amd C-ABI takes contiguous device tensors"
     return t.data_ptr()
 
 
@@ -117,7 +122,7 @@ def expect(t, name, dtype, device, shape):
     tensor would be read out of bounds or at the wrong element size."""
     if not isinstance(t, torch.Tensor):
         raise RuntimeError(f"k2_amd: {name} must be a tensor")
-    if not t.is_cuda:
+    if not _on_device(t):
         raise RuntimeError(f"k2_amd runs on MI355X only: {name} is on {t.device} (there is no CPU path)")
     if t.dtype != dtype or t.device != device or tuple(t.shape) != tuple(shape):
         raise RuntimeError(f"k2_amd: {name} must be {dtype} {list(shape)} on {device}, "
@@ -134,7 +139,7 @@ def expect_optional(t, name, dtype, device, shape):
 def _float_dtype(t, name):
     if not isinstance(t, torch.Tensor) or t.dtype not in (torch.float32, torch.float64):
         raise RuntimeError(f"k2_amd: {name} must be a float32 or float64 tensor")
-    if not t.is_cuda:
+    if not _on_device(t):
         raise RuntimeError(f"k2_amd runs on MI355X only: {name} is on {t.device} (there is no CPU path)")
     return t.dtype, t.device
 
@@ -743,7 +748,7 @@ def pruned_ranges_to_lattice(ranges, frames, symbols, logits):
         if B == 0:
             arc_splits.zero_()
         strides = (ctypes.c_int64 * 4)(*logits.stride())
-        assert logits.is_cuda
+        assert _on_device(logits)
         check(lib().k2amd_lattice_fill(ptr(ranges), ptr(frames), ptr(symbols), logits.data_ptr(),
                                        ctypes.addressof(strides), ptr(state_splits), ptr(arc_base),
                                        ptr(arc_local), ptr(arc_splits), ptr(arcs), ptr(arc_map), B, T,

@@ -4,6 +4,32 @@
 #include "common.h"
 #include "mi_internal.h"
 
+// The host build has mi_capi.hip itself (argument checks and kernel selection) but none of the
+// kernels that need the hardware: their launchers say "not served", as they do on the GPU for a
+// shape outside their range, and every call then takes the exact kernels of mi_generic.hip.
+namespace k2amd {
+bool MiFastSupports(int, int, int, int) { return false; }
+size_t MiFastWorkspaceBytes(int, int, int) { return 0; }
+int MiFastWorkspaceInit(void *, size_t, hipStream_t) { return K2AMD_OK; }
+int MiForwardFast(const float *, const float *, const int64_t *, float *, float *, float *, int, int, int, int,
+                  void *, size_t, hipStream_t) { return K2AMD_ERR_UNSUPPORTED; }
+int MiBackwardFast(const float *, const float *, const float *, const int64_t *, float *, float *, float *, int,
+                   int, int, int, int, void *, size_t, hipStream_t) { return K2AMD_ERR_UNSUPPORTED; }
+bool MiFusedSupports(int, int, int, int) { return false; }
+bool MiFusedAdvised(int, int, int) { return false; }
+size_t MiFusedScratchElems(int, int, int, int) { return 0; }
+int MiForwardBackwardFast(const float *, const float *, const int64_t *, float *, float *, float *, float *,
+                          float *, int, int, int, int, int, void *, size_t, hipStream_t) {
+  return K2AMD_ERR_UNSUPPORTED;
+}
+bool MiWaveSupports(int, int, int) { return false; }
+size_t MiWaveWorkspaceBytes(int, int, int) { return 0; }
+int MiForwardWave(const double *, const double *, const int64_t *, double *, double *, int, int, int, int, void *,
+                  size_t, hipStream_t) { return K2AMD_ERR_UNSUPPORTED; }
+int MiBackwardWave(const double *, const double *, const int64_t *, double *, double *, double *, int, int, int,
+                   int, int, void *, size_t, hipStream_t) { return K2AMD_ERR_UNSUPPORTED; }
+}  // namespace k2amd
+
 extern "C" {
 
 int cpu_mi_forward_generic(const void *px, const void *py, const int64_t *boundary, void *p, void *ans, int B,

@@ -7,7 +7,9 @@ operand layout: g++ compiles the SAME sources over the thread stand-in of
 tests/cpu_build/hip/hip_runtime.h into one shared library, whose C-ABI entry points then take
 numpy buffers.  The ctypes signatures are k2_amd/capi.py's own table, so a wrong entry there
 shows up here as well.  The kernels that need more of the hardware (inline assembly, DPP, spin
-waits between workgroups: mi_fast, mi_wave, joiner) are not part of it.
+waits between workgroups: mi_fast, mi_wave, joiner) are not part of it; mi_capi.hip (the MI
+entry points' argument checks and kernel selection) is, with launchers for those kernels that
+say "not served" (tests/cpu_build/entry.cc), so every MI call takes the exact kernels.
 
 Fenced arrays: a numpy array whose last byte sits directly in front of an inaccessible page (or
 whose first byte directly behind one), so that a kernel reading or writing past the end of a
@@ -25,7 +27,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(ROOT, "k2_amd", "csrc")
 SHIM = os.path.join(HERE, "cpu_build")
 OUT = os.path.join(SHIM, "_build")
-PORTABLE = ["rnnt_rows", "prune", "lattice", "mi_joint", "mi_generic", "rnnt_smoothed", "rnnt_simple"]
+PORTABLE = ["rnnt_rows", "prune", "lattice", "mi_joint", "mi_generic", "rnnt_smoothed", "rnnt_simple", "mi_capi"]
 # -ffp-contract=off: a * b + c rounds twice, as in the reference's CPU loops (the exact
 # mutual-information kernels are compared with them bit for bit)
 FLAGS = ["-std=c++20", "-O1", "-g", "-fPIC", "-pthread", "-ffp-contract=off", f"-I{SHIM}", f"-I{CSRC}"]

@@ -1,0 +1,246 @@
+"""The Python host layer (k2_amd/capi.py's wrappers, k2_amd/rnnt_loss.py's autograd Functions)
+run on CPU tensors against the host build of the kernels (tests/cpu_kernels.py).
+
+The product never does this: it takes device tensors and fails without the GPU library.  Here a
+fixture swaps, for the duration of a test, the library handle for the host build and the three
+places where the wrappers touch the device (the device check, the stream, the device guard), so
+that the very code that marshals arguments on the GPU box is exercised without one: argument
+order and count of every C-ABI call, the buffers it allocates and their shapes, what is saved for
+the backward, and the chaining of the autograd Functions.  Gradients are compared with torch
+autograd over the plain-torch definitions (tests/torch_ref.py)."""
+import contextlib
+
+import numpy as np
+import pytest
+import torch
+
+import cases
+import cpu_kernels as ck
+import torch_ref
+from oracle import mi as omi
+from oracle import rnnt as orn
+
+TYPES = ["regular", "modified", "constrained"]
+
+
+@pytest.fixture
+def host_on_cpu(monkeypatch):
+    from k2_amd import capi, native
+    cpu_lib = ck.lib()
+    monkeypatch.setattr(capi, "lib", lambda: cpu_lib)
+    monkeypatch.setattr(capi, "_on_device", lambda t: True)
+    monkeypatch.setattr(capi, "stream_ptr", lambda device: None)
+    monkeypatch.setattr(torch.cuda, "device", lambda device: contextlib.nullcontext())
+    monkeypatch.setattr(native, "_ext", None)              # the ctypes host: same C-ABI calls as the extension's
+    monkeypatch.setattr(native, "_require_device", lambda t: None)
+    return capi
+
+
+def _weighted(px, py, seed):
+    """A scalar function of the lattice's log-probs with fixed random weights (zero where px is
+    -inf: the last column of a regular lattice and the boundary cut)."""
+    g = torch.Generator().manual_seed(seed)
+    wx = torch.rand(px.shape, generator=g, dtype=torch.float64).to(px.dtype)
+    wy = torch.rand(py.shape, generator=g, dtype=torch.float64).to(py.dtype)
+    finite = torch.isfinite(px)
+    return (torch.where(finite, px, torch.zeros_like(px)) * wx).sum() + (py * wy).sum()
+
+
+def _case(seed, B, T, S, C, rnnt_type, dtype=np.float64):
+    c = cases.rnnt_case(seed, B, T, S, C, dtype=dtype, t_lo=max(S, T - 3), s_lo=max(1, S - 2),
+                        modified=rnnt_type != "regular")
+    c["symbols"][:, 1] = c["symbols"][:, 0]
+    return c
+
+
+def _t(c, *keys):
+    return [None if c[k] is None else torch.from_numpy(c[k]) for k in keys]
+
+
+@pytest.mark.parametrize("rnnt_type", TYPES)
+def test_simple_and_smoothed_builders_through_autograd(host_on_cpu, rnnt_type, monkeypatch):
+    import k2_amd as k2
+    c = _case(801, 3, 11, 6, 70, rnnt_type)
+    sym, bd = _t(c, "symbols", "boundary")
+    for smoothed in (False, True):
+        for kernels in ((False, True) if smoothed else (False,)):
+            monkeypatch.setenv("K2AMD_SMOOTHED_KERNELS", "1" if kernels else "0")
+            lm, am = (x.requires_grad_(True) for x in _t(c, "lm", "am"))
+            lm_r, am_r = (x.requires_grad_(True) for x in _t(c, "lm", "am"))
+            if smoothed:
+                px, py = k2.get_rnnt_logprobs_smoothed(lm, am, sym, 0, 0.25, 0.1, boundary=bd, rnnt_type=rnnt_type)
+                rpx, rpy = torch_ref.logprobs_smoothed(lm_r, am_r, sym, 0, 0.25, 0.1, rnnt_type, bd)
+            else:
+                px, py = k2.get_rnnt_logprobs(lm, am, sym, 0, rnnt_type=rnnt_type, boundary=bd)
+                rpx, rpy = torch_ref.logprobs_simple(lm_r, am_r, sym, 0, rnnt_type, bd)
+            np.testing.assert_allclose(px.detach().numpy(), rpx.detach().numpy(), rtol=1e-10, atol=1e-10)
+            np.testing.assert_allclose(py.detach().numpy(), rpy.detach().numpy(), rtol=1e-10, atol=1e-10)
+            _weighted(px, py, 5).backward()
+            _weighted(rpx, rpy, 5).backward()
+            np.testing.assert_allclose(lm.grad.numpy(), lm_r.grad.numpy(), rtol=1e-8, atol=1e-10)
+            np.testing.assert_allclose(am.grad.numpy(), am_r.grad.numpy(), rtol=1e-8, atol=1e-10)
+
+
+def test_smoothed_kernels_with_float32_and_a_per_sequence_scale(host_on_cpu, monkeypatch):
+    """The smoothed wrappers directly, fp32, with seq_scale (the loss functions' way of passing
+    the gradient that reaches each score)."""
+    capi = host_on_cpu
+    c = _case(802, 3, 13, 5, 33, "regular", np.float32)
+    lm, am, sym, bd = _t(c, "lm", "am", "symbols", "boundary")
+    assert capi.smoothed_supported(lm, am)
+    px, py, saved = capi.logprobs_smoothed_forward(lm, am, sym, 0, 0.25, 0.1, 0, bd)
+    wpx, wpy = orn.logprobs_smoothed(c["lm"], c["am"], c["symbols"], 0, 0.25, 0.1, c["boundary"], "regular")
+    np.testing.assert_allclose(px.numpy(), wpx, rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(py.numpy(), wpy, rtol=1e-4, atol=1e-5)
+    _, gx, gy = omi.mi(wpx.astype(np.float64), wpy.astype(np.float64), c["boundary"])
+    scale = torch.linspace(0.5, 1.5, 3)
+    lm_g, am_g = capi.logprobs_smoothed_backward(torch.from_numpy(gx.astype(np.float32)),
+                                                 torch.from_numpy(gy.astype(np.float32)), sym, bd, saved, 0, 0.25,
+                                                 0.1, 0, scale)
+    import closed_forms as cf
+    want_lm, want_am = cf.smoothed_grads(c["lm"], c["am"], c["symbols"], 0, 0.25, 0.1, gx, gy, -scale.numpy(),
+                                         "regular")
+    np.testing.assert_allclose(lm_g.numpy(), want_lm, rtol=1e-3, atol=1e-5)
+    np.testing.assert_allclose(am_g.numpy(), want_am, rtol=1e-3, atol=1e-5)
+
+
+@pytest.mark.parametrize("rnnt_type", TYPES)
+def test_joint_and_pruned_builders_through_autograd(host_on_cpu, rnnt_type):
+    import k2_amd as k2
+    B, T, S, C, R = 2, 9, 5, 37, 3
+    c = _case(803, B, T, S, C, rnnt_type)
+    sym, bd = _t(c, "symbols", "boundary")
+    rng = np.random.default_rng(804)
+    logits = torch.from_numpy(rng.standard_normal((B, T, S + 1, C))).requires_grad_(True)
+    ref = logits.detach().clone().requires_grad_(True)
+    px, py = k2.get_rnnt_logprobs_joint(logits, sym, 0, rnnt_type=rnnt_type, boundary=bd)
+    rpx, rpy = torch_ref.logprobs_from_logits(ref, sym, 0, rnnt_type, bd)
+    np.testing.assert_allclose(px.detach().numpy(), rpx.detach().numpy(), rtol=1e-10, atol=1e-10)
+    _weighted(px, py, 6).backward()
+    _weighted(rpx, rpy, 6).backward()
+    np.testing.assert_allclose(logits.grad.numpy(), ref.grad.numpy(), rtol=1e-8, atol=1e-10)
+
+    start = np.sort(rng.integers(0, S - R + 2, (B, T)), axis=1)
+    start[:, 0], start[:, -2:] = 0, S - R + 1
+    ranges = torch.from_numpy((np.maximum.accumulate(start, axis=1)[:, :, None] + np.arange(R)).astype(np.int64))
+    for hat in (False, True):
+        logits = torch.from_numpy(rng.standard_normal((B, T, R, C))).requires_grad_(True)
+        ref = logits.detach().clone().requires_grad_(True)
+        builder = k2.get_hat_logprobs_pruned if hat else k2.get_rnnt_logprobs_pruned
+        px, py = builder(logits, sym, ranges, 0, boundary=bd, rnnt_type=rnnt_type)
+        rpx, rpy = torch_ref.logprobs_pruned(ref, sym, ranges, 0, bd, rnnt_type, hat=hat)
+        finite = torch.isfinite(rpx)
+        assert torch.equal(torch.isfinite(px), finite)
+        np.testing.assert_allclose(px.detach()[finite].numpy(), rpx.detach()[finite].numpy(), rtol=1e-10, atol=1e-10)
+        # py outside the band is -inf on both sides: weigh the band only
+        band = torch.isfinite(rpy)
+        assert torch.equal(torch.isfinite(py), band)
+        g = torch.Generator().manual_seed(7)
+        wx, wy = torch.rand(px.shape, generator=g, dtype=torch.float64), torch.rand(py.shape, generator=g, dtype=torch.float64)
+        zero = torch.zeros((), dtype=torch.float64)
+        for a, b in ((px, py), (rpx, rpy)):
+            (torch.where(finite, a, zero) * wx).sum().add((torch.where(band, b, zero) * wy).sum()).backward()
+        np.testing.assert_allclose(logits.grad.numpy(), ref.grad.numpy(), rtol=1e-8, atol=1e-10)
+
+
+def test_prune_ranges_pruning_and_lattice(host_on_cpu):
+    import k2_amd as k2
+    capi = host_on_cpu
+    B, T, S, C, R = 3, 17, 8, 12, 4
+    c = _case(805, B, T, S, C, "regular", np.float32)
+    px, py = orn.logprobs_simple(c["lm"], c["am"], c["symbols"], 0, "regular", c["boundary"])
+    _, gx, gy = omi.mi(px, py, c["boundary"])
+    bd = torch.from_numpy(c["boundary"])
+    ranges = k2.get_rnnt_prune_ranges(torch.from_numpy(gx), torch.from_numpy(gy), bd, R)
+    want = orn.prune_ranges(gx, gy, c["boundary"], R)
+    assert np.array_equal(ranges.numpy(), want)
+
+    D = 24
+    rng = np.random.default_rng(806)
+    am = torch.from_numpy(rng.standard_normal((B, T, D)).astype(np.float32)).requires_grad_(True)
+    lm = torch.from_numpy(rng.standard_normal((B, S + 1, D)).astype(np.float32)).requires_grad_(True)
+    am_p, lm_p = k2.do_rnnt_pruning(am, lm, ranges)
+    want_lm = torch.gather(lm.detach().unsqueeze(1).expand(B, T, S + 1, D), 2,
+                           ranges.reshape(B, T, R, 1).expand(B, T, R, D))
+    assert torch.equal(lm_p.detach(), want_lm)
+    assert torch.equal(am_p.detach(), am.detach().unsqueeze(2).expand(B, T, R, D))
+    w = torch.from_numpy(rng.standard_normal((B, T, R, D)).astype(np.float32))
+    (lm_p * w).sum().backward()
+    want_g = torch.zeros(B, S + 1, D).index_put_(
+        (torch.arange(B).reshape(B, 1, 1).expand(B, T, R), ranges), w, accumulate=True)
+    np.testing.assert_allclose(lm.grad.numpy(), want_g.numpy(), rtol=1e-5, atol=1e-5)
+
+    from oracle import lattice as olat
+    logits = rng.standard_normal((B, T, ranges.shape[2], C)).astype(np.float32)
+    frames = c["boundary"][:, 3].astype(np.int32)
+    state_splits, arc_splits, arcs, arc_map = capi.pruned_ranges_to_lattice(
+        ranges.to(torch.int32), torch.from_numpy(frames), torch.from_numpy(c["symbols"]), torch.from_numpy(logits))
+    w_state, w_arc, w_arcs, w_scores, w_map = olat.pruned_ranges_to_lattice(
+        ranges.numpy().astype(np.int32), frames, c["symbols"], logits)
+    assert np.array_equal(state_splits.numpy(), w_state) and np.array_equal(arc_splits.numpy(), w_arc)
+    assert np.array_equal(arcs.numpy()[:, :3], w_arcs) and np.array_equal(arc_map.numpy(), w_map)
+    assert np.array_equal(arcs.numpy()[:, 3].copy().view(np.float32), w_scores.astype(np.float32))
+
+
+def test_joint_products_wrapper(host_on_cpu):
+    capi = host_on_cpu
+    rng = np.random.default_rng(807)
+    N, B, S, T = 3, 2, 4, 7
+    pxs = [torch.from_numpy(-rng.uniform(0, 3, (B, S, T + 1))) for _ in range(N)]
+    pys = [torch.from_numpy(-rng.uniform(0, 3, (B, S + 1, T))) for _ in range(N)]
+    gx, gy = torch.from_numpy(rng.uniform(0, 1, (B, S, T + 1))), torch.from_numpy(rng.uniform(0, 1, (B, S + 1, T)))
+    prods = capi.mi_joint_products(pxs, pys, gx, gy)
+    want = torch.stack([(x * gx).sum(dim=(1, 2)) + (y * gy).sum(dim=(1, 2)) for x, y in zip(pxs, pys)])
+    np.testing.assert_allclose(prods.numpy(), want.numpy(), rtol=1e-12)
+
+
+# ---- the whole Python API on the host: the GPU tests' own bodies, with device = cpu --------------
+# mi_capi.hip is part of the host build with the hardware kernels' launchers saying "not served",
+# so mutual_information_recursion and every loss function run end to end (on the exact kernels).
+
+def _gpu_test(name):
+    import test_rnnt_gpu
+    return getattr(test_rnnt_gpu, name)
+
+
+@pytest.mark.parametrize("name", ["test_reference_chain_fixtures",
+                                  "test_reference_prune_ranges_on_ties_and_near_ties",
+                                  "test_reference_logprobs_where_the_shifted_exponentials_underflow",
+                                  "test_reference_joint_recursion_fixtures",
+                                  "test_reference_smoothed_and_hat_gradient_fixtures"])
+def test_reference_fixtures_through_the_api(host_on_cpu, name, monkeypatch):
+    """Everything recorded from the reference's own Python chain (tests/golden/rnnt_ref_fixtures.npz)
+    through k2_amd's API on CPU tensors: losses, occupation probabilities, gradients to the network
+    outputs, prune ranges bit for bit; the smoothed loss once with torch ops for its marginal
+    terms and once with the library's kernels."""
+    if "chain" in name:  # every second chain, the smoothed loss in it with the library's kernels
+        monkeypatch.setenv("K2AMD_SMOOTHED_KERNELS", "1")
+        _gpu_test(name)(torch.device("cpu"), every=2)
+        return
+    _gpu_test(name)(torch.device("cpu"))
+    if "smoothed" in name:
+        monkeypatch.setenv("K2AMD_SMOOTHED_KERNELS", "1")
+        _gpu_test(name)(torch.device("cpu"))
+
+
+@pytest.mark.parametrize("rnnt_type", TYPES)
+def test_smoothed_loss_with_the_kernels(host_on_cpu, rnnt_type, monkeypatch):
+    """rnnt_loss_smoothed end to end (values against the oracle, gradients against autograd over the
+    definition, scales (0, 0) == rnnt_loss_simple, invariance to per-frame constants) with the
+    marginal terms in the library's kernels."""
+    monkeypatch.setenv("K2AMD_SMOOTHED_KERNELS", "1")
+    _gpu_test("test_smoothed_loss_values_gradients_and_identities")(torch.device("cpu"), rnnt_type)
+
+
+@pytest.mark.parametrize("name", ["test_rnnt_loss_gradient", "test_rnnt_loss_empty_reference",
+                                  "test_mutual_information_against_itself_and_finite_differences"])
+def test_reference_scenarios_through_the_api(host_on_cpu, name):
+    """Scenarios of the reference's own tests (rnnt_loss_test.py, mutual_information_test.py) as
+    tests/test_reference_scenarios_gpu.py restates them, at the sizes the host build can afford."""
+    import test_reference_scenarios_gpu
+    getattr(test_reference_scenarios_gpu, name)(torch.device("cpu"))
+
+
+def test_joint_recursion_split_through_the_api(host_on_cpu):
+    import test_mi_gpu
+    test_mi_gpu.test_joint_recursion_split_matches_the_torch_chain(torch.device("cpu"), torch.float32)

@@ -817,16 +817,15 @@ def _fixtures():
     return [str(n) for n in f["names"]], get
 
 
-def test_reference_chain_fixtures(device):
+def test_reference_chain_fixtures(device, every=1):
     """Every function of the path on the inputs recorded with the reference's outputs: losses,
     occupation probabilities and network-output gradients within the fp32 tolerance, prune ranges
     (both rules) bit for bit from the reference's own gradients."""
     import k2_amd as k2
     names, get = _fixtures()
     tol = dict(rtol=1e-4, atol=1e-5)
-    for name in names:
-        if not name.startswith("chain"):
-            continue
+    # (every: the host-build run of this body, tests/test_cpu_build_host_layer.py, takes every second chain)
+    for name in [n for n in names if n.startswith("chain")][::every]:
         am, lm, sym, bd = (get(name, k) for k in ("am", "lm", "symbols", "boundary"))
         rt, dp, R = str(get(name, "rnnt_type")), float(get(name, "delay_penalty")), int(get(name, "s_range"))
         w = dev(get(name, "weights"), device)
