@@ -213,23 +213,6 @@ def test_refusals(device):
         capi.joiner_pruned_forward(*args(), 37, None, 0)
 
 
-def test_no_frames_at_all(device):
-    """T = 0: py is empty, and a regular lattice still has its px column T, which the reference
-    pads with -inf (k2/python/k2/rnnt_loss.py:1310-1319); nothing may be left as allocated."""
-    from k2_amd import capi
-    B, S, R, C, D = 2, 5, 3, 11, 64
-    rng = np.random.default_rng(3)
-    am = torch.zeros(B, 0, D, device=device)
-    lm = dev(rng.standard_normal((B, S + 1, D)).astype(np.float32), device)
-    ranges = torch.zeros(B, 0, R, dtype=torch.int64, device=device)
-    weight = dev(rng.standard_normal((C, D)).astype(np.float32), device)
-    symbols = dev(rng.integers(1, C, (B, S)).astype(np.int64), device)
-    px, py, _ = capi.joiner_pruned_forward(am, lm, ranges, weight, None, symbols, 0, None, 0)
-    torch.cuda.synchronize(device)
-    assert tuple(px.shape) == (B, S, 1) and tuple(py.shape) == (B, S + 1, 0)
-    assert torch.isneginf(px).all()
-
-
 def test_config3_shape_through_the_api(device):
     """BASELINE config 3's shape (B=32, T=500, S=100, V=500, s_range=5) with a joiner of D=512,
     through k2_amd.rnnt_loss_pruned_joiner and autograd: the loss per utterance against the fp64

@@ -5,7 +5,8 @@ pair of host layers is compared in tests/test_mi_gpu.py.)
 
 Written while no GPU was at hand and not run on one yet; the ctypes side has run against the host
 build of the kernels (tests/test_cpu_build_host_layer.py), the extension's side in all other GPU
-tests.  The file's name puts it behind the tests that have run on a GPU."""
+tests.  Also here: the fused joiner's case without frames, written at the same time.  The file's
+name puts it behind the tests that have run on a GPU."""
 import numpy as np
 import pytest
 import torch
@@ -101,3 +102,20 @@ def test_pruning_and_lattice(device, hosts, dtype):
     frames = bd[:, 3].to(torch.int32).contiguous()
     _same(native.pruned_ranges_to_lattice(ranges.to(torch.int32), frames, sym, logits),
           capi.pruned_ranges_to_lattice(ranges.to(torch.int32), frames, sym, logits), "lattice")
+
+
+def test_fused_joiner_without_frames(device):
+    """T = 0: py is empty, and a regular lattice still has its px column T, which the reference
+    pads with -inf (k2/python/k2/rnnt_loss.py:1310-1319); nothing may be left as allocated."""
+    from k2_amd import capi
+    B, S, R, C, D = 2, 5, 3, 11, 64
+    rng = np.random.default_rng(3)
+    am = torch.zeros(B, 0, D, device=device)
+    lm = dev(rng.standard_normal((B, S + 1, D)).astype(np.float32), device)
+    ranges = torch.zeros(B, 0, R, dtype=torch.int64, device=device)
+    weight = dev(rng.standard_normal((C, D)).astype(np.float32), device)
+    symbols = dev(rng.integers(1, C, (B, S)).astype(np.int64), device)
+    px, py, _ = capi.joiner_pruned_forward(am, lm, ranges, weight, None, symbols, 0, None, 0)
+    torch.cuda.synchronize(device)
+    assert tuple(px.shape) == (B, S, 1) and tuple(py.shape) == (B, S + 1, 0)
+    assert torch.isneginf(px).all()
