@@ -638,10 +638,16 @@ def main():
         out["cpu_baseline"] = cpu_baseline(c)
     if not args.no_secondary:
         del px, py, p
-        out["secondary"] = pruned_secondary(dev, cpu=not args.no_cpu)
-        out["other_configs"] = other_configs(dev)
-        out["fused_joiner"] = fused_joiner(dev)
-        out["next_rows"] = next_rows(dev)
+        # None of these is `value`: a failure in one of them is reported in its field and does not
+        # take the headline's line with it.
+        for field, part in (("secondary", lambda: pruned_secondary(dev, cpu=not args.no_cpu)),
+                            ("other_configs", lambda: other_configs(dev)),
+                            ("fused_joiner", lambda: fused_joiner(dev)),
+                            ("next_rows", lambda: next_rows(dev))):
+            try:
+                out[field] = part()
+            except Exception as e:  # noqa: BLE001 - whatever it is, the line below still has to come out
+                out[field] = {"error": f"{type(e).__name__}: {e}"}
     print(json.dumps(out))
 
 
