@@ -243,7 +243,7 @@ K2AMD_API int k2amd_rnnt_logprobs_simple_backward(
  * unigram, then its log).  scratch: k2amd_rnnt_smoothed_scratch_elements(B, S, T, C) elements of
  * the tensors' type (= C * max(ceil(B (S+1) / 16), 1 + ceil(B T / 16)): per-workgroup column
  * sums); less is refused with K2AMD_ERR_WORKSPACE before anything is launched.
- * The vocabulary must fit the kernels' LDS arrays: (2 C + S) * sizeof(element) <= 64 KiB, else
+ * The vocabulary must fit the kernels' LDS arrays: (2 C + S) * sizeof(element) + 12 S <= 64 KiB, else
  * K2AMD_ERR_UNSUPPORTED (k2amd_rnnt_smoothed_supported tells beforehand).                         */
 K2AMD_API size_t k2amd_rnnt_smoothed_scratch_elements(int B, int S, int T, int C);
 K2AMD_API int k2amd_rnnt_smoothed_supported(int B, int S, int T, int C, int dtype);

@@ -175,8 +175,14 @@ struct LatticeGrads {
 //     dz[c] = am_scale * ( sum over s with symbols[b][s] == c of Gx(b,s,t)  +  (c == blank) vy
 //                          - p[c] (vx + vy) )
 // is added to am_grad[b][t], and the group's sum of dz over its rows is written to partial[group]
-// (the gradient that reaches log unigram).  LDS: the row being built [C], the group's sums [C],
-// Gx of the row's frame [S].
+// (the gradient that reaches log unigram).
+// The symbols' terms: positions that carry the same symbol are chained once per sequence
+// (lead_of[s] = the symbol if s is its first position, else -1; next_of[s] = the next position
+// with the same symbol, or -1), so that per row the first position's lane adds up its chain in
+// ascending s and writes one column: a fixed order, no two lanes on one column, and a cost per row
+// of the longest chain rather than of S.
+// LDS: the row being built [C], the group's sums [C], Gx of the row's frame [S]; then as ints the
+// sequence's symbols [S], lead_of [S], next_of [S].
 template <typename T>
 __global__ __launch_bounds__(64) void AmOnlyGradKernel(LatticeGrads<T> g, const int64_t *__restrict__ symbols,
                                                        const T *__restrict__ am_probs,
@@ -190,11 +196,33 @@ __global__ __launch_bounds__(64) void AmOnlyGradKernel(LatticeGrads<T> g, const 
   T *acc = dz + C;                           // [C]
   T *gx_of = acc + C;                        // [S]
   const int lane = threadIdx.x, S = g.S, Tn = g.Tn;
+  int *sym_of = reinterpret_cast<int *>(gx_of + S);  // [S]
+  int *lead_of = sym_of + S;                         // [S]
+  int *next_of = lead_of + S;                        // [S]
   for (int c = lane; c < C; c += kWave) acc[c] = T(0);
   const long long row0 = (long long)blockIdx.x * kRowsPerGroup;
+  int chained_b = -1;  // the sequence whose chains the LDS arrays hold
   for (int r = 0; r < kRowsPerGroup && row0 + r < rows; ++r) {
     const long long row = row0 + r;
     const int b = (int)(row / Tn), t = (int)(row - (long long)b * Tn);
+    if (b != chained_b) {  // the same for every lane
+      chained_b = b;
+      const int64_t *sym = symbols + (size_t)b * S;
+      for (int s = lane; s < S; s += kWave) sym_of[s] = sym[s] >= 0 && sym[s] < C ? (int)sym[s] : -1;
+      __syncthreads();
+      for (int s = lane; s < S; s += kWave) {
+        const int mine = sym_of[s];
+        bool first = mine >= 0;
+        int next = -1;
+        if (mine >= 0) {
+          for (int k = 0; k < s && first; ++k) first = sym_of[k] != mine;
+          for (int k = s + 1; k < S && next < 0; ++k)
+            if (sym_of[k] == mine) next = k;
+        }
+        lead_of[s] = first ? mine : -1;
+        next_of[s] = next;
+      }
+    }
     T vx = 0, vy = 0;
     for (int s = lane; s <= S; s += kWave) {
       const T gx = g.Gx(b, s, t);
@@ -208,21 +236,22 @@ __global__ __launch_bounds__(64) void AmOnlyGradKernel(LatticeGrads<T> g, const 
     const T *p = am_probs + (size_t)row * C;
     for (int c = lane; c < C; c += kWave)
       dz[c] = am_scale * ((c == blank ? vy : T(0)) - p[c] * unigram[c] * inv_sum * (vx + vy));
-    __syncthreads();  // gx_of was written by other lanes than the ones that read it below
-    // the symbols' terms, position by position so that a repeated symbol adds in a fixed order;
-    // column c belongs to lane c % 64 here as in the loops around
-    const int64_t *sym_of = symbols + (size_t)b * S;
-    for (int s = 0; s < S; ++s) {
-      const int64_t sym = sym_of[s];
-      if (sym >= 0 && sym < C && (int)(sym & (kWave - 1)) == lane) dz[sym] += am_scale * gx_of[s];
+    __syncthreads();  // dz, gx_of and the chains are read by other lanes than the ones that wrote them
+    for (int s = lane; s < S; s += kWave) {
+      const int c = lead_of[s];
+      if (c < 0) continue;
+      T v = gx_of[s];
+      for (int k = next_of[s]; k >= 0; k = next_of[k]) v += gx_of[k];
+      dz[c] += am_scale * v;
     }
+    __syncthreads();
     T *out = am_grad + (size_t)row * C;
     for (int c = lane; c < C; c += kWave) {
       const T v = dz[c];
       out[c] += v;
       acc[c] += v;
     }
-    __syncthreads();  // before the next row overwrites gx_of
+    __syncthreads();  // before the next row overwrites dz and gx_of
   }
   for (int c = lane; c < C; c += kWave) partial[(size_t)blockIdx.x * C + c] = acc[c];
 }
@@ -279,8 +308,8 @@ __global__ __launch_bounds__(256) void LmOnlyGradKernel(LatticeGrads<T> g, const
 
 constexpr size_t kLdsLimit = 64 * 1024;  // what a launch may ask for without a function attribute
 
-template <typename T>
-size_t BackwardLdsBytes(int S, int C) { return ((size_t)2 * C + S) * sizeof(T); }
+// AmOnlyGradKernel's arrays: 2 C + S elements, then 3 S ints
+inline size_t BackwardLdsBytes(int S, int C, size_t elem) { return ((size_t)2 * C + S) * elem + (size_t)3 * S * 4; }
 
 bool ArgsOk(int B, int S, int T, int C, int blank, int rnnt_type, int dtype) {
   if (B < 0 || S < 0 || T < 0 || C <= 0 || blank < 0 || blank >= C) return false;
@@ -291,8 +320,7 @@ bool ArgsOk(int B, int S, int T, int C, int blank, int rnnt_type, int dtype) {
 
 // The vocabulary has to fit the workgroups' LDS arrays, and grid sizes 32 bits.
 bool Served(int B, int S, int T, int C, int dtype) {
-  const size_t elem = dtype == K2AMD_F64 ? 8 : 4;
-  if (((size_t)2 * C + S) * elem > kLdsLimit) return false;
+  if (BackwardLdsBytes(S, C, dtype == K2AMD_F64 ? 8 : 4) > kLdsLimit) return false;
   const long long lim = 1ll << 30;
   return (long long)B * (S + 1) < lim && (long long)B * T < lim;
 }
@@ -342,7 +370,7 @@ int SmoothedBackward(const T *px_grad, const T *py_grad, const T *seq_scale, con
   LatticeGrads<T> g{px_grad, py_grad, seq_scale, boundary, S, Tn, rnnt_type};
   T *d_unigram = scratch, *partial = scratch + C;
   if (groups > 0)
-    hipLaunchKernelGGL(AmOnlyGradKernel<T>, dim3((unsigned)groups), dim3(64), BackwardLdsBytes<T>(S, C), st, g,
+    hipLaunchKernelGGL(AmOnlyGradKernel<T>, dim3((unsigned)groups), dim3(64), BackwardLdsBytes(S, C, sizeof(T)), st, g,
                        symbols, am_probs, am_max, am_norm, unigram, am_grad, partial, am_rows, C, blank,
                        (T)am_only_scale);
   hipLaunchKernelGGL(UnigramGradKernel<T>, dim3((C + 255) / 256), dim3(256), 0, st, (const T *)partial, unigram,

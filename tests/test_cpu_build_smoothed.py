@@ -163,7 +163,7 @@ def test_shapes_at_the_edges(lib):
 
 
 def test_refusals(lib):
-    assert lib.k2amd_rnnt_smoothed_supported(2, 10, 20, 8192, 0) == 0      # (2 C + S) * 4 B > 64 KiB
+    assert lib.k2amd_rnnt_smoothed_supported(2, 10, 20, 8192, 0) == 0      # (2 C + S) * 4 B + 12 S > 64 KiB
     assert lib.k2amd_rnnt_smoothed_supported(2, 10, 20, 8000, 0) == 1
     assert lib.k2amd_rnnt_smoothed_supported(2, 10, 20, 4096, 1) == 0
     assert lib.k2amd_rnnt_smoothed_supported(2, 10, 20, 4000, 1) == 1
