@@ -244,3 +244,25 @@ def test_reference_scenarios_through_the_api(host_on_cpu, name):
 def test_joint_recursion_split_through_the_api(host_on_cpu):
     import test_mi_gpu
     test_mi_gpu.test_joint_recursion_split_matches_the_torch_chain(torch.device("cpu"), torch.float32)
+
+
+def test_no_allocation_entry_point_on_the_exact_kernels(host_on_cpu):
+    """k2amd_mi_forward_noalloc where no pipelined kernel serves the shape (always, in the host
+    build): it asks for no scratch, is not refused for the static array's size whatever the shape,
+    gives what k2amd_mi_forward gives, and its status call answers."""
+    capi = host_on_cpu
+    lib = capi.lib()
+    c = cases.mi_case(901, dtype=np.float32, max_B=3, max_S=20, max_T=40)
+    px, py = torch.from_numpy(c["px"]), torch.from_numpy(c["py"])
+    bd = None if c["boundary"] is None else torch.from_numpy(c["boundary"])
+    B, S, T = c["B"], c["S"], c["T"]
+    p1, p2 = torch.empty(B, S + 1, T + 1), torch.empty(B, S + 1, T + 1)
+    want = capi.mi_forward(px, py, bd, p1)
+    got = capi.mi_forward_noalloc(px, py, bd, p2, torch.empty(B))
+    assert torch.equal(got, want)
+    ans, _ = omi.mi_forward(c["px"], c["py"], c["boundary"])
+    np.testing.assert_array_equal(got.numpy(), ans)
+    # a lattice of 2 GiB and more: not refused for scratch, turned down for its null pointers
+    assert lib.k2amd_mi_forward_noalloc(None, None, None, None, None, 4096, 200, 1000, 1, 0, None) == 1
+    assert lib.k2amd_mi_forward_noalloc(None, None, None, None, None, 0, 3, 3, 0, 0, None) == 0
+    assert lib.k2amd_mi_noalloc_status(None) == 0
