@@ -10,7 +10,15 @@
 namespace k2amd {
 bool MiFastSupports(int, int, int, int) { return false; }
 size_t MiFastWorkspaceBytes(int, int, int) { return 0; }
-int MiFastWorkspaceInit(void *, size_t, hipStream_t) { return K2AMD_OK; }
+// (the fp64 wave kernels ARE part of the host build and share the fp32 kernels' workspace layout:
+// a header of 64 words, zero, then words that hold the sentinel while nothing is published)
+int MiFastWorkspaceInit(void *workspace, size_t workspace_bytes, hipStream_t) {
+  if (workspace == nullptr || workspace_bytes < 256) return K2AMD_ERR_WORKSPACE;
+  unsigned *words = static_cast<unsigned *>(workspace);
+  for (size_t i = 0; i < 64; ++i) words[i] = 0;
+  for (size_t i = 64; i < workspace_bytes / 4; ++i) words[i] = 0x7fc5a5a5u;
+  return K2AMD_OK;
+}
 int MiForwardFast(const float *, const float *, const int64_t *, float *, float *, float *, int, int, int, int,
                   void *, size_t, hipStream_t) { return K2AMD_ERR_UNSUPPORTED; }
 int MiBackwardFast(const float *, const float *, const float *, const int64_t *, float *, float *, float *, int,
@@ -22,12 +30,6 @@ int MiForwardBackwardFast(const float *, const float *, const int64_t *, float *
                           float *, int, int, int, int, int, void *, size_t, hipStream_t) {
   return K2AMD_ERR_UNSUPPORTED;
 }
-bool MiWaveSupports(int, int, int) { return false; }
-size_t MiWaveWorkspaceBytes(int, int, int) { return 0; }
-int MiForwardWave(const double *, const double *, const int64_t *, double *, double *, int, int, int, int, void *,
-                  size_t, hipStream_t) { return K2AMD_ERR_UNSUPPORTED; }
-int MiBackwardWave(const double *, const double *, const int64_t *, double *, double *, double *, int, int, int,
-                   int, int, void *, size_t, hipStream_t) { return K2AMD_ERR_UNSUPPORTED; }
 }  // namespace k2amd
 
 extern "C" {

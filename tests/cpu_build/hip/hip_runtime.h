@@ -10,6 +10,7 @@
 #include <math.h>
 #include <stddef.h>
 #include <stdint.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <algorithm>
@@ -196,6 +197,33 @@ inline hip_threads_float16 __builtin_amdgcn_mfma_f32_32x32x2f32(float a, float b
     c[v] += w.matrix_a[set][i] * w.matrix_b[set][j] + w.matrix_a[set][i + 32] * w.matrix_b[set][j + 32];
   }
   return c;
+}
+
+// ---- what the fp64 wave kernels (mi_wave.hip) use ------------------------------------------------
+#define __HIP_MEMORY_SCOPE_AGENT 0
+#define __hip_atomic_load(address, order, scope) hip_threads::atomic_load(address)
+#define __hip_atomic_store(address, value, order, scope) hip_threads::atomic_store(address, value)
+namespace hip_threads {
+template <typename T>
+inline T atomic_load(T *address) { return std::atomic_ref<T>(*address).load(std::memory_order_seq_cst); }
+template <typename T, typename V>
+inline void atomic_store(T *address, V value) { std::atomic_ref<T>(*address).store((T)value, std::memory_order_seq_cst); }
+}  // namespace hip_threads
+inline void __builtin_amdgcn_s_sleep(int) { std::this_thread::yield(); }
+inline float __builtin_amdgcn_rcpf(float x) { return 1.0f / x; }
+template <typename T>
+inline T __builtin_amdgcn_readlane(T v, int lane) { return hip_threads::exchange(v, lane); }
+template <typename T>
+inline T __builtin_amdgcn_readfirstlane(T v) { return hip_threads::exchange(v, 0); }  // (lane 0 is live wherever it is used)
+// DPP moves over the whole wavefront: wave_shr:1 (0x138: lane l takes lane l - 1, lane 0 keeps
+// `old`) and wave_shl:1 (0x130: lane l takes lane l + 1, lane 63 keeps `old`); all rows and banks
+// enabled, as the kernels ask for.  Other controls are not emulated.
+inline int __builtin_amdgcn_update_dpp(int old, int src, int ctrl, int row_mask, int bank_mask, bool bound_ctrl) {
+  if ((ctrl != 0x138 && ctrl != 0x130) || row_mask != 0xf || bank_mask != 0xf || bound_ctrl) abort();
+  const int lane = hip_threads::flat_thread % hip_threads::kWaveSize;
+  const int from = ctrl == 0x138 ? lane - 1 : lane + 1;
+  const int got = hip_threads::exchange(src, std::min(std::max(from, 0), hip_threads::kWaveSize - 1));
+  return from < 0 || from >= hip_threads::my_wave().lanes ? old : got;
 }
 
 // On the hardware a scheduling fence that emits nothing (a wavefront's lanes run in lockstep);

@@ -27,7 +27,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(ROOT, "k2_amd", "csrc")
 SHIM = os.path.join(HERE, "cpu_build")
 OUT = os.path.join(SHIM, "_build")
-PORTABLE = ["rnnt_rows", "prune", "lattice", "mi_joint", "mi_generic", "rnnt_smoothed", "rnnt_simple", "mi_capi"]
+PORTABLE = ["rnnt_rows", "prune", "lattice", "mi_joint", "mi_generic", "rnnt_smoothed", "rnnt_simple", "mi_capi", "mi_wave"]
 # -ffp-contract=off: a * b + c rounds twice, as in the reference's CPU loops (the exact
 # mutual-information kernels are compared with them bit for bit)
 FLAGS = ["-std=c++20", "-O1", "-g", "-fPIC", "-pthread", "-ffp-contract=off", f"-I{SHIM}", f"-I{CSRC}"]

@@ -9,6 +9,7 @@ order and count of every C-ABI call, the buffers it allocates and their shapes, 
 the backward, and the chaining of the autograd Functions.  Gradients are compared with torch
 autograd over the plain-torch definitions (tests/torch_ref.py)."""
 import contextlib
+import types
 
 import numpy as np
 import pytest
@@ -31,6 +32,11 @@ def host_on_cpu(monkeypatch):
     monkeypatch.setattr(capi, "_on_device", lambda t: True)
     monkeypatch.setattr(capi, "stream_ptr", lambda device: None)
     monkeypatch.setattr(torch.cuda, "device", lambda device: contextlib.nullcontext())
+    # (for the workspace cache of the pipelined kernels, which is kept per device and stream)
+    monkeypatch.setattr(torch.cuda, "current_stream", lambda device=None: types.SimpleNamespace(cuda_stream=0))
+    monkeypatch.setattr(torch.cuda, "current_device", lambda: 0)
+    monkeypatch.setattr(torch.cuda, "synchronize", lambda device=None: None)
+    monkeypatch.setattr(capi, "_workspaces", {})
     monkeypatch.setattr(native, "_ext", None)              # the ctypes host: same C-ABI calls as the extension's
     monkeypatch.setattr(native, "_require_device", lambda t: None)
     return capi
@@ -211,16 +217,15 @@ def _gpu_test(name):
 def test_reference_fixtures_through_the_api(host_on_cpu, name, monkeypatch):
     """Everything recorded from the reference's own Python chain (tests/golden/rnnt_ref_fixtures.npz)
     through k2_amd's API on CPU tensors: losses, occupation probabilities, gradients to the network
-    outputs, prune ranges bit for bit; the smoothed loss once with torch ops for its marginal
-    terms and once with the library's kernels."""
+    outputs, prune ranges bit for bit; the smoothed loss with the library's kernels for
+    its marginal terms."""
     if "chain" in name:  # every second chain, the smoothed loss in it with the library's kernels
         monkeypatch.setenv("K2AMD_SMOOTHED_KERNELS", "1")
         _gpu_test(name)(torch.device("cpu"), every=2)
         return
-    _gpu_test(name)(torch.device("cpu"))
-    if "smoothed" in name:
+    if "smoothed" in name:  # (with torch ops for the marginal terms this test runs on the GPU)
         monkeypatch.setenv("K2AMD_SMOOTHED_KERNELS", "1")
-        _gpu_test(name)(torch.device("cpu"))
+    _gpu_test(name)(torch.device("cpu"))
 
 
 @pytest.mark.parametrize("rnnt_type", TYPES)
@@ -266,3 +271,35 @@ def test_no_allocation_entry_point_on_the_exact_kernels(host_on_cpu):
     assert lib.k2amd_mi_forward_noalloc(None, None, None, None, None, 4096, 200, 1000, 1, 0, None) == 1
     assert lib.k2amd_mi_forward_noalloc(None, None, None, None, None, 0, 3, 3, 0, 0, None) == 0
     assert lib.k2amd_mi_noalloc_status(None) == 0
+
+
+@pytest.mark.parametrize("modified", [False, True])
+def test_fp64_pipelined_kernels(host_on_cpu, modified):
+    """mi_wave.hip (one wavefront per chunk of 64 rows, chunks of a sequence handing their border
+    over through words in the workspace, lane shifts by DPP) against the fp64 oracle: lattices of
+    one to three chunks, boundaries, both lattice types; the workspace is back in its initial
+    state after every call.  Workgroups run one after the other here, in ticket order, which the
+    kernels' own rule (a chunk waits only for chunks with earlier tickets) makes sufficient."""
+    capi = host_on_cpu
+    seen_chunks = set()
+    for seed, max_s in ((910, 20), (911, 100), (912, 190), (913, 130), (914, 70)):
+        c = cases.mi_case(seed, dtype=np.float64, max_B=3, max_S=max_s, max_T=60,
+                          force={"modified": modified, "rand_bd": seed % 2 == 0})
+        B, S, T = c["B"], c["S"], c["T"]
+        seen_chunks.add(S // 64 + 1)
+        px, py = torch.from_numpy(c["px"]), torch.from_numpy(c["py"])
+        bd = None if c["boundary"] is None else torch.from_numpy(c["boundary"])
+        assert capi.lib().k2amd_mi_workspace_bytes(B, S, T, int(modified), 1) > 0
+        p = torch.empty(B, S + 1, T + 1, dtype=torch.float64)
+        ans = capi.mi_forward(px, py, bd, p)
+        want_ans, want_p = omi.mi_forward(c["px"], c["py"], c["boundary"])
+        np.testing.assert_allclose(ans.numpy(), want_ans, rtol=1e-10, atol=1e-10)
+        g = torch.full((B,), 1.0, dtype=torch.float64)
+        gx, gy = capi.mi_backward(px, py, bd, p, g, overwrite_ans_grad=True)
+        want_gx, want_gy = omi.mi_backward(c["px"], c["py"], c["boundary"], want_p)
+        np.testing.assert_allclose(gx.numpy(), want_gx, rtol=1e-9, atol=1e-10)
+        np.testing.assert_allclose(gy.numpy(), want_gy, rtol=1e-9, atol=1e-10)
+        finite = np.isfinite(want_ans)
+        np.testing.assert_allclose(g.numpy()[finite], 1.0, rtol=1e-9)
+        assert capi.mi_workspace_is_clean(px.device)
+    assert len(seen_chunks) >= 2, seen_chunks
