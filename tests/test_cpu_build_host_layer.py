@@ -9,6 +9,7 @@ order and count of every C-ABI call, the buffers it allocates and their shapes, 
 the backward, and the chaining of the autograd Functions.  Gradients are compared with torch
 autograd over the plain-torch definitions (tests/torch_ref.py)."""
 import contextlib
+import os
 import types
 
 import numpy as np
@@ -22,6 +23,9 @@ from oracle import mi as omi
 from oracle import rnnt as orn
 
 TYPES = ["regular", "modified", "constrained"]
+# what takes a quarter of a minute and more on eight cores runs with K2AMD_SLOW_CPU_TESTS=1 only
+slow = pytest.mark.skipif(os.environ.get("K2AMD_SLOW_CPU_TESTS", "0") != "1",
+                          reason="slow on the host: run with K2AMD_SLOW_CPU_TESTS=1")
 
 
 @pytest.fixture
@@ -212,7 +216,7 @@ def _gpu_test(name):
 @pytest.mark.parametrize("name", ["test_reference_chain_fixtures",
                                   "test_reference_prune_ranges_on_ties_and_near_ties",
                                   "test_reference_logprobs_where_the_shifted_exponentials_underflow",
-                                  "test_reference_joint_recursion_fixtures",
+                                  pytest.param("test_reference_joint_recursion_fixtures", marks=slow),
                                   "test_reference_smoothed_and_hat_gradient_fixtures"])
 def test_reference_fixtures_through_the_api(host_on_cpu, name, monkeypatch):
     """Everything recorded from the reference's own Python chain (tests/golden/rnnt_ref_fixtures.npz)
@@ -237,7 +241,7 @@ def test_smoothed_loss_with_the_kernels(host_on_cpu, rnnt_type, monkeypatch):
     _gpu_test("test_smoothed_loss_values_gradients_and_identities")(torch.device("cpu"), rnnt_type)
 
 
-@pytest.mark.parametrize("name", ["test_rnnt_loss_gradient", "test_rnnt_loss_empty_reference",
+@pytest.mark.parametrize("name", [pytest.param("test_rnnt_loss_gradient", marks=slow), "test_rnnt_loss_empty_reference",
                                   "test_mutual_information_against_itself_and_finite_differences"])
 def test_reference_scenarios_through_the_api(host_on_cpu, name):
     """Scenarios of the reference's own tests (rnnt_loss_test.py, mutual_information_test.py) as
@@ -246,6 +250,7 @@ def test_reference_scenarios_through_the_api(host_on_cpu, name):
     getattr(test_reference_scenarios_gpu, name)(torch.device("cpu"))
 
 
+@slow
 def test_joint_recursion_split_through_the_api(host_on_cpu):
     import test_mi_gpu
     test_mi_gpu.test_joint_recursion_split_matches_the_torch_chain(torch.device("cpu"), torch.float32)
@@ -282,7 +287,7 @@ def test_fp64_pipelined_kernels(host_on_cpu, modified):
     kernels' own rule (a chunk waits only for chunks with earlier tickets) makes sufficient."""
     capi = host_on_cpu
     seen_chunks = set()
-    for seed, max_s in ((910, 20), (911, 100), (912, 190), (913, 130), (914, 70)):
+    for seed, max_s in ((910, 20), (912, 190), (913, 130)):
         c = cases.mi_case(seed, dtype=np.float64, max_B=3, max_S=max_s, max_T=60,
                           force={"modified": modified, "rand_bd": seed % 2 == 0})
         B, S, T = c["B"], c["S"], c["T"]

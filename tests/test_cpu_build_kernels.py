@@ -132,7 +132,7 @@ def test_joint_builder(lib, rnnt_type, dtype):
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("rnnt_type", TYPES)
 def test_pruned_builders(lib, rnnt_type, dtype, hat):
-    for k, C in enumerate(ROW_CLASSES if rnnt_type == "regular" else ROW_CLASSES[1:6:2]):
+    for k, C in enumerate(ROW_CLASSES[::2] + ROW_CLASSES[5:6] if rnnt_type == "regular" else ROW_CLASSES[1:6:2]):
         B, T, S, R = 2, 9 + k, 5, 1 + k % 4
         c = cases.rnnt_case(620 + k, B, T, S, C, dtype=dtype, t_lo=7, s_lo=3, modified=rnnt_type != "regular")
         rng = np.random.default_rng(630 + k)
