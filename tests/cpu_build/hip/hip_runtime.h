@@ -1,9 +1,16 @@
 // A stand-in for <hip/hip_runtime.h> that runs HIP kernels on host threads, for tests only: the
 // same kernel source is compiled with g++ and every launch runs its workgroups one after the
 // other, each workgroup's work-items as threads of their own, so that barriers and wavefront
-// exchanges keep their meaning.  It covers the portable subset the row kernels use (no inline
-// assembly, no DPP, no matrix instructions) and lets a host sanitizer and a CPU debugger see the
-// kernels' indexing.  Slow by design: sizes stay small.
+// exchanges keep their meaning, and a host sanitizer or a CPU debugger sees the kernels' indexing.
+//
+// What it has: launches with static and dynamic LDS, __syncthreads, the __shfl family, atomics,
+// vector types, __half as storage, and of the gfx9 builtins readlane / readfirstlane, the two
+// whole-wavefront DPP shifts, v_mfma_f32_32x32x2_f32 (from its documented operand layout),
+// wave_barrier (a real barrier here: the lanes are free-running threads, not in lockstep) and
+// no-ops for fences and scheduling hints.  What it does not have: inline assembly, other DPP
+// controls, bfloat16 vectors, concurrency BETWEEN workgroups (a kernel whose workgroups wait for
+// one another must only ever wait for workgroups that started earlier).  Slow by design: sizes
+// stay small.
 #ifndef K2_AMD_TESTS_CPU_BUILD_HIP_RUNTIME_H_
 #define K2_AMD_TESTS_CPU_BUILD_HIP_RUNTIME_H_
 
