@@ -241,10 +241,11 @@ K2AMD_API int k2amd_rnnt_logprobs_simple_backward(
  * py [B][S+1][T] (neither may overlap px_joint / py_joint), and for the backward lm_norm [B][S+1]
  * (log sum_c exp lm), am_norm [B][T] (log sum_c exp(am) unigram[c]) and unigram [2][C] (the
  * unigram, then its log).  scratch: k2amd_rnnt_smoothed_scratch_elements(B, S, T, C) elements of
- * the tensors' type (= C * max(ceil(B (S+1) / 16), 1 + ceil(B T / 16)): per-workgroup column
- * sums); less is refused with K2AMD_ERR_WORKSPACE before anything is launched.
- * The vocabulary must fit the kernels' LDS arrays: (2 C + S) * sizeof(element) + 12 S <= 64 KiB, else
- * K2AMD_ERR_UNSUPPORTED (k2amd_rnnt_smoothed_supported tells beforehand).                         */
+ * the tensors' type (row sums of the lattice's gradients, per-row weights and the partial column
+ * sums over chunks of rows: 4 B (S+1) + 3 B T + C (ceil(B T / 64) + ceil(B (S+1) / 64) + 1) at
+ * most, chunks capped at 64 each); less is refused with K2AMD_ERR_WORKSPACE before anything is
+ * launched.  No limit on the vocabulary; k2amd_rnnt_smoothed_supported tells whether the row
+ * counts fit the kernels' 32-bit indexing.                                                         */
 K2AMD_API size_t k2amd_rnnt_smoothed_scratch_elements(int B, int S, int T, int C);
 K2AMD_API int k2amd_rnnt_smoothed_supported(int B, int S, int T, int C, int dtype);
 K2AMD_API int k2amd_rnnt_smoothed_forward(

@@ -421,8 +421,8 @@ def logprobs_simple_backward(px_grad, py_grad, symbols, boundary, saved, termina
 
 
 def smoothed_supported(lm, am):
-    """Whether the smoothed builder's kernels take these tensors (the vocabulary has to fit their
-    LDS arrays)."""
+    """Whether the smoothed builder's kernels take these tensors (their row counts have to fit the
+    kernels' 32-bit indexing)."""
     B, T, C = am.shape
     return bool(lib().k2amd_rnnt_smoothed_supported(B, lm.shape[1] - 1, T, C, dtype_code(am)))
 

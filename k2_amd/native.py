@@ -199,8 +199,8 @@ def logprobs_simple_backward(px_grad, py_grad, symbols, boundary, saved, termina
 
 
 def smoothed_supported(lm, am):
-    """Whether the smoothed builder's kernels take these tensors (their vocabulary has to fit the
-    kernels' LDS arrays)."""
+    """Whether the smoothed builder's kernels take these tensors (their row counts have to fit the
+    kernels' 32-bit indexing)."""
     if _ext is not None:
         return _ext.smoothed_supported(am.shape[0], lm.shape[1] - 1, am.shape[1], am.shape[2], capi.dtype_code(am))
     return capi.smoothed_supported(lm, am)
