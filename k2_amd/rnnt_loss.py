@@ -168,6 +168,11 @@ class _Scores(torch.autograd.Function):
             lm, am, symbols, termination_symbol, rnnt_code, _ = args
             px, py, saved = native.logprobs_simple_forward(lm.contiguous(), am.contiguous(), symbols,
                                                          termination_symbol, rnnt_code, boundary)
+        elif kind == "smoothed":
+            lm, am, symbols, termination_symbol, rnnt_code, _, lm_only_scale, am_only_scale = args
+            px, py, saved = native.logprobs_smoothed_forward(lm.contiguous(), am.contiguous(), symbols,
+                                                           termination_symbol, lm_only_scale, am_only_scale,
+                                                           rnnt_code, boundary)
         elif kind == "joint":
             logits, symbols, termination_symbol, rnnt_code, _ = args
             logits = logits.contiguous()
@@ -216,6 +221,11 @@ class _Scores(torch.autograd.Function):
             _, _, symbols, termination_symbol, rnnt_code, boundary = args
             grads = native.logprobs_simple_backward(px_grad, py_grad, symbols, boundary, saved,
                                                     termination_symbol, rnnt_code, scale)
+        elif ctx.kind == "smoothed":
+            _, _, symbols, termination_symbol, rnnt_code, boundary, lm_only_scale, am_only_scale = args
+            grads = native.logprobs_smoothed_backward(px_grad, py_grad, symbols, boundary, saved,
+                                                      termination_symbol, lm_only_scale, am_only_scale,
+                                                      rnnt_code, scale)
         elif ctx.kind == "joint":
             _, symbols, termination_symbol, rnnt_code, boundary = args
             grads = (native.logprobs_joint_backward(saved[0], saved[1], px_grad, py_grad, symbols,
@@ -647,6 +657,12 @@ def rnnt_loss_smoothed(
     return_grad: bool = False,
 ) -> Union[Tuple[Tensor, Tuple[Tensor, Tensor]], Tensor]:
     """k2.rnnt_loss_smoothed (k2/python/k2/rnnt_loss.py:1707-1829)."""
+    if smoothed_kernels_enabled() and am.ndim == 3 and am.shape[0] > 0 and native.smoothed_supported(lm, am):
+        # builder, recursion and reduction as one graph node, like the other losses
+        args = _simple_args(lm, am, symbols, termination_symbol, rnnt_type, boundary)
+        loss, px_grad, py_grad = _Scores.apply("smoothed", rnnt_type, float(delay_penalty), bool(return_grad),
+                                               reduction, *args, float(lm_only_scale), float(am_only_scale))
+        return (loss, (px_grad, py_grad)) if return_grad else loss
     px, py = get_rnnt_logprobs_smoothed(lm=lm, am=am, symbols=symbols,
                                         termination_symbol=termination_symbol,
                                         lm_only_scale=lm_only_scale, am_only_scale=am_only_scale,
