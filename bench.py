@@ -109,15 +109,16 @@ def _cpu_pruned_loss(logits, symbols, ranges, boundary, blank=0):
     return -Lattice.apply(px, py).sum()
 
 
-def pruned_secondary(dev, steps=50, cpu=True):
+def pruned_secondary(dev, steps=None, cpu=True):
     """Second figure asked for next to the headline: pruned RNN-T loss forward + backward on
     BASELINE config 3 (B=32, T=500, S=100, V=500, s_range=5, regular lattice) in utterances/s,
     beside the CPU route on a sample of the same utterances."""
+    steps = steps or SECONDARY_STEPS["pruned_secondary"]
     import torch
     import cases
     import k2_amd as k2
-    B, T, S, C, R = 32, 500, 100, 500, 5
-    c = cases.rnnt_case(3, B, T, S, C, t_lo=300, s_lo=50)
+    B, T, S, C, R = (SHAPES["c3"][k] for k in ("B", "T", "S", "C", "R"))
+    c = cases.rnnt_case(3, B, T, S, C, t_lo=SHAPES["c3"]["t_lo"], s_lo=SHAPES["c3"]["s_lo"])
     lm, am = torch.from_numpy(c["lm"]).to(dev), torch.from_numpy(c["am"]).to(dev)
     sym, bd = torch.from_numpy(c["symbols"]).to(dev), torch.from_numpy(c["boundary"]).to(dev)
     logits = torch.from_numpy(np.random.default_rng(33).standard_normal((B, T, R, C)).astype(np.float32)).to(dev)
@@ -204,6 +205,14 @@ def pruned_secondary(dev, steps=50, cpu=True):
 
 
 MFMA_PEAK_TFLOPS = {"fp32": 157.3, "bf16": 2500.0}  # MI355X published dense matrix rates
+# BASELINE's configurations as the secondary workloads use them: B, T, S, V (, s_range), and the
+# smallest T_b / S_b of the random boundaries.  (One place, so that a test can run this file's
+# control flow on toy sizes.)
+SHAPES = {"c2": dict(B=16, T=250, S=50, C=500, t_lo=150, s_lo=20),
+          "c3": dict(B=32, T=500, S=100, C=500, R=5, t_lo=300, s_lo=50),
+          "c5": dict(B=8, T=300, S=75, C=500, t_lo=200, s_lo=40),
+          "c4": dict(B=32, S=200, T=1000)}
+SECONDARY_STEPS = {"pruned_secondary": 50, "other_configs": 50, "fused_joiner": 20, "next_rows": 30}
 LOGITS_SETS = 3  # copies of config 3's logits the secondary figures rotate over (see pruned_secondary)
 # The dominant kernel of the secondary workloads and its average duration in the committed kernel
 # trace of this file's default run (rocprofv3 --kernel-trace --stats; not measured by the run).
@@ -216,18 +225,20 @@ PROFILED_KERNELS = {
 }
 
 
-def fused_joiner(dev, steps=20):
+def fused_joiner(dev, steps=None):
     """The pruned loss with the joiner inside it (k2_amd.rnnt_loss_pruned_joiner) on BASELINE config
     3's shape with a joiner of D=512, forward + backward, beside the chain it replaces on the same
     device (do_rnnt_pruning, torch's tanh and linear, rnnt_loss_pruned).  FLOPs counted: the three
     products an implementation cannot avoid (logits, their gradient times the weight, the
     weight's gradient), 2 * B*T*s_range * D * V each; what the fused kernels multiply again when they
     recompute is not counted."""
+    steps = steps or SECONDARY_STEPS["fused_joiner"]
     import torch
     import cases
     import k2_amd as k2
-    B, T, S, C, R, D = 32, 500, 100, 500, 5, 512
-    c = cases.rnnt_case(3, B, T, S, C, t_lo=300, s_lo=50)
+    B, T, S, C, R = (SHAPES["c3"][k] for k in ("B", "T", "S", "C", "R"))
+    D = 512
+    c = cases.rnnt_case(3, B, T, S, C, t_lo=SHAPES["c3"]["t_lo"], s_lo=SHAPES["c3"]["s_lo"])
     lm0, am0 = torch.from_numpy(c["lm"]).to(dev), torch.from_numpy(c["am"]).to(dev)
     sym, bd = torch.from_numpy(c["symbols"]).to(dev), torch.from_numpy(c["boundary"]).to(dev)
     _, (gx, gy) = k2.rnnt_loss_simple(lm0, am0, sym, 0, bd, reduction="sum", return_grad=True)
@@ -285,10 +296,11 @@ def fused_joiner(dev, steps=20):
     return out
 
 
-def other_configs(dev, steps=50):
+def other_configs(dev, steps=None):
     """The two remaining BASELINE configurations, forward + backward through the k2-style API with
     gradients to the network outputs: config 2 (rnnt_loss_simple, B=16 T=250 S=50 V=500) and
     config 5 (rnnt_loss on the full joiner lattice, B=8 T=300 S=75 V=500)."""
+    steps = steps or SECONDARY_STEPS["other_configs"]
     import torch
     import cases
     import k2_amd as k2
@@ -306,8 +318,8 @@ def other_configs(dev, steps=50):
         return e0.elapsed_time(e1) / steps * 1e-3
 
     out = {}
-    B, T, S, C = 16, 250, 50, 500
-    c = cases.rnnt_case(2, B, T, S, C, t_lo=150, s_lo=20)
+    B, T, S, C = (SHAPES["c2"][k] for k in ("B", "T", "S", "C"))
+    c = cases.rnnt_case(2, B, T, S, C, t_lo=SHAPES["c2"]["t_lo"], s_lo=SHAPES["c2"]["s_lo"])
     lm = torch.from_numpy(c["lm"]).to(dev).requires_grad_(True)
     am = torch.from_numpy(c["am"]).to(dev).requires_grad_(True)
     sym, bd = torch.from_numpy(c["symbols"]).to(dev), torch.from_numpy(c["boundary"]).to(dev)
@@ -326,8 +338,8 @@ def other_configs(dev, steps=50):
         "frac_of_hbm_peak": nbytes / t / 1e9 / HBM_PEAK_GBS}
     del lm, am
 
-    B, T, S, C = 8, 300, 75, 500
-    c = cases.rnnt_case(5, B, T, S, C, t_lo=200, s_lo=40)
+    B, T, S, C = (SHAPES["c5"][k] for k in ("B", "T", "S", "C"))
+    c = cases.rnnt_case(5, B, T, S, C, t_lo=SHAPES["c5"]["t_lo"], s_lo=SHAPES["c5"]["s_lo"])
     logits = torch.from_numpy(
         np.random.default_rng(55).standard_normal((B, T, S + 1, C)).astype(np.float32)).to(dev)
     logits.requires_grad_(True)
@@ -352,12 +364,13 @@ def other_configs(dev, steps=50):
     return out
 
 
-def next_rows(dev, steps=30):
+def next_rows(dev, steps=None):
     """The rows either side of the path that the library also serves, each once at a BASELINE shape:
     pruned_ranges_to_lattice and the HAT pruned loss on config 3's shape, the smoothed loss on
     config 2's, joint_mutual_information_recursion (two px / py pairs) on config 4's.  HIP-event
     time per call through the k2-style API (forward + backward for the losses, a fresh boundary
     tensor per step as in the other secondary figures), with the bytes each has to move at least."""
+    steps = steps or SECONDARY_STEPS["next_rows"]
     import torch
     import cases
     import k2_amd as k2
@@ -379,8 +392,8 @@ def next_rows(dev, steps=30):
                 "bytes_counted": what, "GBps": nbytes / t / 1e9, "frac_of_hbm_peak": nbytes / t / 1e9 / HBM_PEAK_GBS}
 
     out = {}
-    B, T, S, C, R = 32, 500, 100, 500, 5
-    c = cases.rnnt_case(3, B, T, S, C, t_lo=300, s_lo=50)
+    B, T, S, C, R = (SHAPES["c3"][k] for k in ("B", "T", "S", "C", "R"))
+    c = cases.rnnt_case(3, B, T, S, C, t_lo=SHAPES["c3"]["t_lo"], s_lo=SHAPES["c3"]["s_lo"])
     lm, am = torch.from_numpy(c["lm"]).to(dev), torch.from_numpy(c["am"]).to(dev)
     sym, bd = torch.from_numpy(c["symbols"]).to(dev), torch.from_numpy(c["boundary"]).to(dev)
     _, (gx, gy) = k2.rnnt_loss_simple(lm, am, sym, 0, bd, reduction="sum", return_grad=True)
@@ -414,8 +427,8 @@ def next_rows(dev, steps=30):
         timed(hat), 3 * logits.numel() * 4, "logits read forward, read + gradient written backward")
     del logits, logits_sets
 
-    B, T, S, C = 16, 250, 50, 500
-    c = cases.rnnt_case(2, B, T, S, C, t_lo=150, s_lo=20)
+    B, T, S, C = (SHAPES["c2"][k] for k in ("B", "T", "S", "C"))
+    c = cases.rnnt_case(2, B, T, S, C, t_lo=SHAPES["c2"]["t_lo"], s_lo=SHAPES["c2"]["s_lo"])
     lm = torch.from_numpy(c["lm"]).to(dev).requires_grad_(True)
     am = torch.from_numpy(c["am"]).to(dev).requires_grad_(True)
     sym, bd = torch.from_numpy(c["symbols"]).to(dev), torch.from_numpy(c["boundary"]).to(dev)
@@ -431,7 +444,7 @@ def next_rows(dev, steps=30):
         timed(smoothed), 2 * 4 * (lm.numel() + am.numel()), "lm, am read forward; their gradients written backward")
     del lm, am
 
-    B, S, T = 32, 200, 1000
+    B, S, T = (SHAPES["c4"][k] for k in ("B", "S", "T"))
     c = cases.c4_case(B=B, S=S, T=T)
     px, py, bd = (torch.from_numpy(c[k]).to(dev) for k in ("px", "py", "boundary"))
     pxs, pys = (px * 0.75, px * 0.25), (py * 0.75, py * 0.25)
@@ -465,6 +478,9 @@ def main():
                          "(8 copies at the default shape are 410 MB); 1 = the same inputs every step")
     ap.add_argument("--no-cache-resident", action="store_true",
                     help="skip the second measurement on one copy of the inputs ('cache_resident')")
+    ap.add_argument("--device", default="cuda:0",
+                    help="where the tensors live; anything but a GPU only makes sense under a test that "
+                         "stands in for the library (the library itself refuses host tensors)")
     ap.add_argument("--B", type=int, default=32)
     ap.add_argument("--S", type=int, default=200)
     ap.add_argument("--T", type=int, default=1000)
@@ -482,7 +498,7 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(1)
-    dev = torch.device("cuda", 0)
+    dev = torch.device(args.device)
     c = cases.c4_case(B=args.B, S=args.S, T=args.T)
     px = torch.from_numpy(c["px"]).to(dev)
     py = torch.from_numpy(c["py"]).to(dev)
