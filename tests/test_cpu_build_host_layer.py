@@ -308,3 +308,12 @@ def test_fp64_pipelined_kernels(host_on_cpu, modified):
         np.testing.assert_allclose(g.numpy()[finite], 1.0, rtol=1e-9)
         assert capi.mi_workspace_is_clean(px.device)
     assert len(seen_chunks) >= 2, seen_chunks
+
+
+def test_smoke_entry_point_runs(host_on_cpu, capsys):
+    """__graft_entry__.smoke()'s own body on CPU tensors (the exact and the fp64 pipelined kernels;
+    the single launch is not in the host build and its branch is skipped, as on any shape it does
+    not serve)."""
+    import __graft_entry__
+    __graft_entry__.smoke("cpu")
+    assert "smoke ok" in capsys.readouterr().out
