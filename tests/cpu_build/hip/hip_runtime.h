@@ -73,6 +73,7 @@ struct Wave {
   // no lane is ever two exchanges ahead of another)
   alignas(8) unsigned char slot[2][kWaveSize][8];
   float matrix_a[2][kWaveSize], matrix_b[2][kWaveSize];  // the operands of a matrix instruction, likewise
+  float matrix_a8[2][kWaveSize][8], matrix_b8[2][kWaveSize][8];
 };
 
 struct State {
@@ -206,6 +207,44 @@ inline hip_threads_float16 __builtin_amdgcn_mfma_f32_32x32x2f32(float a, float b
   return c;
 }
 
+// ---- what the fused joiner (joiner.hip) uses besides ------------------------------------------------
+// bfloat16: eight of them as one 16-byte value, and the hardware's conversion (round to nearest
+// even; NaN stays NaN).  The host compiler has no such type; the test's build replaces the two
+// places of the source that spell it (tests/cpu_kernels.py).
+struct hip_threads_bf16x8 { unsigned short v[8]; };
+inline unsigned short hip_threads_to_bf16(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40u);
+  return (unsigned short)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+// v_mfma_f32_32x32x16_bf16: as the fp32 one above with sixteen k per step: lane l supplies eight
+// consecutive k of row / column l % 32, the lower half of the wavefront the first eight.
+inline hip_threads_float16 __builtin_amdgcn_mfma_f32_32x32x16_bf16(hip_threads_bf16x8 a, hip_threads_bf16x8 b,
+                                                                   hip_threads_float16 c, int, int, int) {
+  hip_threads::Wave &w = hip_threads::my_wave();
+  const int lane = hip_threads::flat_thread % hip_threads::kWaveSize;
+  const unsigned set = hip_threads::exchanges++ & 1;
+  for (int e = 0; e < 8; ++e) {
+    uint32_t ua = (uint32_t)a.v[e] << 16, ub = (uint32_t)b.v[e] << 16;
+    memcpy(&w.matrix_a8[set][lane][e], &ua, 4);
+    memcpy(&w.matrix_b8[set][lane][e], &ub, 4);
+  }
+  w.barrier->arrive_and_wait();
+  const int j = lane % 32;
+  for (int v = 0; v < 16; ++v) {
+    const int i = 8 * (v / 4) + 4 * (lane / 32) + v % 4;
+    float sum = 0;
+    for (int half = 0; half < 2; ++half)
+      for (int e = 0; e < 8; ++e) sum += w.matrix_a8[set][i + 32 * half][e] * w.matrix_b8[set][j + 32 * half][e];
+    c[v] += sum;
+  }
+  return c;
+}
+inline float __builtin_amdgcn_exp2f(float x) { return exp2f(x); }
+enum hipFuncAttribute { hipFuncAttributeMaxDynamicSharedMemorySize };
+inline hipError_t hipFuncSetAttribute(const void *, hipFuncAttribute, int) { return hipSuccess; }
+
 // ---- what the fp64 wave kernels (mi_wave.hip) use ------------------------------------------------
 #define __HIP_MEMORY_SCOPE_AGENT 0
 #define __hip_atomic_load(address, order, scope) hip_threads::atomic_load(address)
@@ -222,12 +261,16 @@ template <typename T>
 inline T __builtin_amdgcn_readlane(T v, int lane) { return hip_threads::exchange(v, lane); }
 template <typename T>
 inline T __builtin_amdgcn_readfirstlane(T v) { return hip_threads::exchange(v, 0); }  // (lane 0 is live wherever it is used)
-// DPP moves over the whole wavefront: wave_shr:1 (0x138: lane l takes lane l - 1, lane 0 keeps
-// `old`) and wave_shl:1 (0x130: lane l takes lane l + 1, lane 63 keeps `old`); all rows and banks
-// enabled, as the kernels ask for.  Other controls are not emulated.
+// DPP moves: within quads (quad_perm), and over the whole wavefront wave_shr:1 (0x138: lane l
+// takes lane l - 1, lane 0 keeps `old`) and wave_shl:1 (0x130: lane l takes lane l + 1, lane 63
+// keeps `old`); all rows and banks enabled, as the kernels ask for.  Other controls are not emulated.
 inline int __builtin_amdgcn_update_dpp(int old, int src, int ctrl, int row_mask, int bank_mask, bool bound_ctrl) {
-  if ((ctrl != 0x138 && ctrl != 0x130) || row_mask != 0xf || bank_mask != 0xf || bound_ctrl) abort();
   const int lane = hip_threads::flat_thread % hip_threads::kWaveSize;
+  if (ctrl >= 0 && ctrl < 0x100) {  // quad_perm: lane 4 q + i takes lane 4 q + ((ctrl >> 2 i) & 3); always in range
+    if (row_mask != 0xf || bank_mask != 0xf) abort();
+    return hip_threads::exchange(src, (lane & ~3) | ((ctrl >> (2 * (lane & 3))) & 3));
+  }
+  if ((ctrl != 0x138 && ctrl != 0x130) || row_mask != 0xf || bank_mask != 0xf || bound_ctrl) abort();
   const int from = ctrl == 0x138 ? lane - 1 : lane + 1;
   const int got = hip_threads::exchange(src, std::min(std::max(from, 0), hip_threads::kWaveSize - 1));
   return from < 0 || from >= hip_threads::my_wave().lanes ? old : got;
@@ -249,11 +292,15 @@ using std::min;
 struct float2 { float x, y; };
 struct float4 { float x, y, z, w; };
 struct double2 { double x, y; };
+struct uint2 { unsigned x, y; };
+struct uint4 { unsigned x, y, z, w; };
 struct int2 { int x, y; };
 struct int4 { int x, y, z, w; };
 inline float2 make_float2(float x, float y) { return {x, y}; }
 inline float4 make_float4(float x, float y, float z, float w) { return {x, y, z, w}; }
 inline double2 make_double2(double x, double y) { return {x, y}; }
+inline uint2 make_uint2(unsigned x, unsigned y) { return {x, y}; }
+inline uint4 make_uint4(unsigned x, unsigned y, unsigned z, unsigned w) { return {x, y, z, w}; }
 inline int2 make_int2(int x, int y) { return {x, y}; }
 inline int4 make_int4(int x, int y, int z, int w) { return {x, y, z, w}; }
 

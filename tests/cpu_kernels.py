@@ -1,15 +1,17 @@
-"""The library's portable HIP kernels compiled for the host (tests only).
+"""The library's HIP kernels compiled for the host (tests only): every kernel file but mi_fast.hip.
 
-k2_amd/csrc/{rnnt_rows, prune, lattice, mi_joint, mi_generic, rnnt_smoothed}.hip use nothing but
-plain HIP (LDS, barriers, wavefront shuffles, atomics), and rnnt_simple.hip besides that one
-matrix instruction (v_mfma_f32_32x32x2_f32), which the stand-in computes from its documented
-operand layout: g++ compiles the SAME sources over the thread stand-in of
+g++ compiles the SAME sources as the GPU library over the thread stand-in of
 tests/cpu_build/hip/hip_runtime.h into one shared library, whose C-ABI entry points then take
-numpy buffers.  The ctypes signatures are k2_amd/capi.py's own table, so a wrong entry there
-shows up here as well.  The kernels that need more of the hardware (inline assembly, DPP, spin
-waits between workgroups: mi_fast, mi_wave, joiner) are not part of it; mi_capi.hip (the MI
-entry points' argument checks and kernel selection) is, with launchers for those kernels that
-say "not served" (tests/cpu_build/entry.cc), so every MI call takes the exact kernels.
+numpy buffers (or CPU tensors, through the product's own Python layer).  Most files use nothing
+but plain HIP (LDS, barriers, wavefront shuffles, atomics); rnnt_simple.hip and joiner.hip besides
+that the two matrix instructions (fp32 and bfloat16 operands), which the stand-in computes from
+their documented operand layouts, mi_wave.hip two DPP lane shifts, readlane and agent-scope
+atomics.  joiner.hip is compiled from a copy in which three lines that the host compiler cannot
+parse are replaced (JOINER_EDITS below, nothing else).  The ctypes signatures are k2_amd/capi.py's
+own table, so a wrong entry there shows up here as well.  mi_fast.hip (inline assembly
+throughout) is not part of it; mi_capi.hip (the MI entry points' argument checks and kernel
+selection) is, with launchers for mi_fast's kernels that say "not served"
+(tests/cpu_build/entry.cc), so MI calls take the exact or the fp64 pipelined kernels.
 
 Fenced arrays: a numpy array whose last byte sits directly in front of an inaccessible page (or
 whose first byte directly behind one), so that a kernel reading or writing past the end of a
@@ -35,12 +37,35 @@ FLAGS = ["-std=c++20", "-O1", "-g", "-fPIC", "-pthread", "-ffp-contract=off", f"
 _lib = None
 
 
+# joiner.hip spells three things the host compiler cannot parse; the host build compiles a copy in
+# which exactly these lines are replaced (each must be found the stated number of times), and not
+# a character else.
+JOINER_EDITS = [
+    ("typedef __bf16 Bf8 __attribute__((ext_vector_type(8)));", "typedef hip_threads_bf16x8 Bf8;", 1),
+    ("return __builtin_bit_cast(unsigned short, static_cast<__bf16>(f));", "return hip_threads_to_bf16(f);", 1),
+    ("extern __shared__ __attribute__((aligned(16))) unsigned char smem[];", "HIP_DYNAMIC_SHARED(unsigned char, smem)", None),
+]
+
+
+def _joiner_source():
+    text = open(os.path.join(CSRC, "joiner.hip")).read()
+    for old, new, count in JOINER_EDITS:
+        assert text.count(old) >= 1 and (count is None or text.count(old) == count), old
+        text = text.replace(old, new)
+    path = os.path.join(OUT, "joiner_host.hip")
+    with open(path, "w") as f:
+        f.write(text)
+    return path
+
+
 def build():
     """Compiles the portable sources and tests/cpu_build/entry.cc into _build/libk2amd_cpu.so."""
     os.makedirs(OUT, exist_ok=True)
     jobs = []
-    for name in PORTABLE + ["entry"]:
+    for name in PORTABLE + ["joiner", "entry"]:
         src = os.path.join(CSRC, name + ".hip") if name != "entry" else os.path.join(SHIM, "entry.cc")
+        if name == "joiner":
+            src = _joiner_source()
         obj = os.path.join(OUT, name + ".o")
         jobs.append((src, obj, subprocess.Popen(["g++", *FLAGS, "-x", "c++", "-c", src, "-o", obj],
                                                 stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))

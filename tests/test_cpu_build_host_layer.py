@@ -317,3 +317,50 @@ def test_smoke_entry_point_runs(host_on_cpu, capsys):
     import __graft_entry__
     __graft_entry__.smoke("cpu")
     assert "smoke ok" in capsys.readouterr().out
+
+
+# ---- the fused joiner: built for the host from a copy of joiner.hip in which the three lines that
+# spell bfloat16 vectors and aligned dynamic LDS are replaced (tests/cpu_kernels.py); the matrix
+# instructions of both operand types and the quad DPP moves come from the stand-in -----------------
+
+@pytest.mark.parametrize("rnnt_type", TYPES)
+def test_fused_joiner_fp32(host_on_cpu, rnnt_type):
+    import test_joiner_gpu as tj
+    cpu = torch.device("cpu")
+    for seed, B, T, S, C, D, R, with_bias in ((1, 2, 9, 4, 11, 64, 3, True), (2, 1, 7, 3, 70, 128, 2, False)):
+        c = tj.joiner_case(seed, B, T, S, C, D, R, rnnt_type, with_bias)
+        logits, px, py = tj.chain_fp64(c)
+        gpx, gpy, norm = tj.run_forward(c, cpu, "fp32")
+        tag = f"{rnnt_type} seed {seed}"
+        tj.close(tag + " px", gpx.numpy(), px, 1e-4, 1e-5 / max(np.abs(px[np.isfinite(px)]).max(), 1e-30))
+        tj.close(tag + " py", gpy.numpy(), py, 1e-4, 1e-5 / max(np.abs(py[np.isfinite(py)]).max(), 1e-30))
+        _, gx, gy = omi.mi(px, py, c["boundary"])
+        gx, gy = gx.astype(np.float32), gy.astype(np.float32)
+        scale = np.linspace(0.5, 1.5, B).astype(np.float32)
+        want = tj.closed_form_grads(c, logits, gx, gy, scale)
+        got = tj.run_backward(c, cpu, "fp32", norm, gx, gy, scale)
+        for name, g, w in zip(("am_grad", "lm_grad", "weight_grad", "bias_grad"), got, want):
+            if g is None:
+                assert name == "bias_grad" and not with_bias
+                continue
+            tj.close(f"{tag} {name}", g, w, 1e-4, 1e-5)
+
+
+def test_fused_joiner_bf16_and_no_frames(host_on_cpu):
+    import test_joiner_gpu as tj
+    from k2_amd import capi
+    cpu = torch.device("cpu")
+    c = tj.joiner_case(3, 2, 9, 4, 11, 64, 3, "regular", True)
+    logits, px, py = tj.chain_fp64(c)
+    gpx, gpy, norm = tj.run_forward(c, cpu, "bf16")
+    fin = np.isfinite(px)
+    assert np.array_equal(np.isfinite(gpx.numpy()), fin)
+    assert np.abs(gpx.numpy()[fin] - px[fin]).max() < 3e-2 and np.abs(gpy.numpy()[np.isfinite(py)] - py[np.isfinite(py)]).max() < 3e-2
+    # no frames at all: py is empty, px is its one -inf column
+    B, S, R, C, D = 2, 5, 3, 11, 64
+    rng = np.random.default_rng(3)
+    lm = torch.from_numpy(rng.standard_normal((B, S + 1, D)).astype(np.float32))
+    px0, py0, _ = capi.joiner_pruned_forward(torch.zeros(B, 0, D), lm, torch.zeros(B, 0, R, dtype=torch.int64),
+                                             torch.from_numpy(rng.standard_normal((C, D)).astype(np.float32)), None,
+                                             torch.from_numpy(rng.integers(1, C, (B, S)).astype(np.int64)), 0, None, 0)
+    assert tuple(px0.shape) == (B, S, 1) and tuple(py0.shape) == (B, S + 1, 0) and torch.isneginf(px0).all()
