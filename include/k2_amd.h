@@ -373,6 +373,24 @@ K2AMD_API int k2amd_rnnt_joiner_pruned_backward(
     void *bias_grad, int B, int S, int T, int R, int C, int D, int termination_symbol, int rnnt_type,
     int precision, void *workspace, size_t workspace_bytes, void *stream);
 
+/* The same pair with get_hat_logprobs_pruned (k2/python/k2/rnnt_loss.py:992-1177) in place of
+ * get_rnnt_logprobs_pruned, i.e. rnnt_loss_pruned(use_hat_loss=True) on the joiner's logits: column 0
+ * is the blank, py = log sigmoid(logits[..., 0]), normalizers = logsumexp over columns 1..C-1,
+ * px = logits[..., symbol] - normalizers + log(1 - sigmoid(logits[..., 0])).  Arguments, workspace
+ * and limits as above, without termination_symbol; C >= 2.  The reference has no such call (its
+ * chain is do_rnnt_pruning -> the caller's joiner -> get_hat_logprobs_pruned).                   */
+K2AMD_API int k2amd_rnnt_joiner_hat_pruned_forward(
+    const void *am, const void *lm, const int64_t *ranges, const void *weight, const void *bias,
+    const int64_t *symbols, const int64_t *boundary, void *px, void *py, void *normalizers, int B,
+    int S, int T, int R, int C, int D, int rnnt_type, int precision, void *workspace,
+    size_t workspace_bytes, void *stream);
+K2AMD_API int k2amd_rnnt_joiner_hat_pruned_backward(
+    const void *am, const void *lm, const int64_t *ranges, const void *weight, const void *bias,
+    const int64_t *symbols, const int64_t *boundary, const void *normalizers, const void *px_grad,
+    const void *py_grad, const void *seq_scale, void *am_grad, void *lm_grad, void *weight_grad,
+    void *bias_grad, int B, int S, int T, int R, int C, int D, int rnnt_type, int precision,
+    void *workspace, size_t workspace_bytes, void *stream);
+
 /* ------------------------------------------------------------------ lattice
  *
  * Replaces _k2.pruned_ranges_to_lattice (k2/python/csrc/torch/pruned_ranges_to_lattice.cu:60-263):

@@ -63,6 +63,8 @@ _SIGNATURES = {
     "k2amd_rnnt_joiner_pruned_forward_workspace_bytes": ([_ci] * 7, _sz),
     "k2amd_rnnt_joiner_pruned_forward": ([_vp] * 10 + [_ci] * 9 + [_vp, _sz, _vp], _ci),
     "k2amd_rnnt_joiner_pruned_backward": ([_vp] * 15 + [_ci] * 9 + [_vp, _sz, _vp], _ci),
+    "k2amd_rnnt_joiner_hat_pruned_forward": ([_vp] * 10 + [_ci] * 8 + [_vp, _sz, _vp], _ci),
+    "k2amd_rnnt_joiner_hat_pruned_backward": ([_vp] * 15 + [_ci] * 8 + [_vp, _sz, _vp], _ci),
     "k2amd_rnnt_prune_ranges": ([_vp] * 4 + [_ci] * 6 + [_vp], _ci),
     "k2amd_rnnt_prune_gather": ([_vp] * 3 + [_ci] * 6 + [_vp], _ci),
     "k2amd_rnnt_prune_gather_backward": ([_vp] * 3 + [_ci] * 6 + [_vp], _ci),
@@ -633,9 +635,12 @@ def _joiner_shapes(am, lm, ranges, weight, bias, symbols, boundary, termination_
 
 
 def joiner_pruned_forward(am, lm, ranges, weight, bias, symbols, termination_symbol, boundary,
-                          rnnt_type, precision=0):
+                          rnnt_type, precision=0, hat=False):
     """tanh(am[b,t] + lm[b,ranges[b,t,k]]) . weight^T + bias and get_rnnt_logprobs_pruned on it in one
-    pass: returns (px, py, normalizers [B][T][R]); the logits never exist in memory."""
+    pass: returns (px, py, normalizers [B][T][R]); the logits never exist in memory.  ``hat``:
+    get_hat_logprobs_pruned instead (column 0 is the blank; termination_symbol must be 0)."""
+    if hat and int(termination_symbol) != 0:
+        raise RuntimeError("k2_amd: the hybrid autoregressive transducer's blank is symbol 0")
     B, S, T, R, C, D, ws = _joiner_shapes(am, lm, ranges, weight, bias, symbols, boundary,
                                           termination_symbol, rnnt_type, precision, True)
     dev = am.device
@@ -643,15 +648,21 @@ def joiner_pruned_forward(am, lm, ranges, weight, bias, symbols, termination_sym
     py = torch.empty(B, S + 1, T, dtype=torch.float32, device=dev)
     norm = torch.empty(B, T, R, dtype=torch.float32, device=dev)
     with torch.cuda.device(dev):
-        check(lib().k2amd_rnnt_joiner_pruned_forward(
-            ptr(am), ptr(lm), ptr(ranges), ptr(weight), ptr(bias), ptr(symbols), ptr(boundary),
-            ptr(px), ptr(py), ptr(norm), B, S, T, R, C, D, termination_symbol, rnnt_type, precision,
-            ptr(ws), ws.numel(), stream_ptr(dev)))
+        if hat:
+            check(lib().k2amd_rnnt_joiner_hat_pruned_forward(
+                ptr(am), ptr(lm), ptr(ranges), ptr(weight), ptr(bias), ptr(symbols), ptr(boundary),
+                ptr(px), ptr(py), ptr(norm), B, S, T, R, C, D, rnnt_type, precision,
+                ptr(ws), ws.numel(), stream_ptr(dev)))
+        else:
+            check(lib().k2amd_rnnt_joiner_pruned_forward(
+                ptr(am), ptr(lm), ptr(ranges), ptr(weight), ptr(bias), ptr(symbols), ptr(boundary),
+                ptr(px), ptr(py), ptr(norm), B, S, T, R, C, D, termination_symbol, rnnt_type, precision,
+                ptr(ws), ws.numel(), stream_ptr(dev)))
     return px, py, norm
 
 
 def joiner_pruned_backward(am, lm, ranges, weight, bias, symbols, termination_symbol, boundary,
-                           rnnt_type, norm, px_grad, py_grad, seq_scale=None, precision=0):
+                           rnnt_type, norm, px_grad, py_grad, seq_scale=None, precision=0, hat=False):
     """Gradients of sum_b seq_scale[b] * score_b through the fused joiner: returns (am_grad, lm_grad,
     weight_grad, bias_grad or None)."""
     B, S, T, R, C, D, ws = _joiner_shapes(am, lm, ranges, weight, bias, symbols, boundary,
@@ -664,11 +675,18 @@ def joiner_pruned_backward(am, lm, ranges, weight, bias, symbols, termination_sy
     weight_grad = torch.empty_like(weight)
     bias_grad = torch.empty_like(bias) if bias is not None else None
     with torch.cuda.device(dev):
-        check(lib().k2amd_rnnt_joiner_pruned_backward(
-            ptr(am), ptr(lm), ptr(ranges), ptr(weight), ptr(bias), ptr(symbols), ptr(boundary),
-            ptr(norm), ptr(px_grad), ptr(py_grad), ptr(seq_scale), ptr(am_grad), ptr(lm_grad),
-            ptr(weight_grad), ptr(bias_grad), B, S, T, R, C, D, termination_symbol, rnnt_type,
-            precision, ptr(ws), ws.numel(), stream_ptr(dev)))
+        if hat:
+            check(lib().k2amd_rnnt_joiner_hat_pruned_backward(
+                ptr(am), ptr(lm), ptr(ranges), ptr(weight), ptr(bias), ptr(symbols), ptr(boundary),
+                ptr(norm), ptr(px_grad), ptr(py_grad), ptr(seq_scale), ptr(am_grad), ptr(lm_grad),
+                ptr(weight_grad), ptr(bias_grad), B, S, T, R, C, D, rnnt_type,
+                precision, ptr(ws), ws.numel(), stream_ptr(dev)))
+        else:
+            check(lib().k2amd_rnnt_joiner_pruned_backward(
+                ptr(am), ptr(lm), ptr(ranges), ptr(weight), ptr(bias), ptr(symbols), ptr(boundary),
+                ptr(norm), ptr(px_grad), ptr(py_grad), ptr(seq_scale), ptr(am_grad), ptr(lm_grad),
+                ptr(weight_grad), ptr(bias_grad), B, S, T, R, C, D, termination_symbol, rnnt_type,
+                precision, ptr(ws), ws.numel(), stream_ptr(dev)))
     return am_grad, lm_grad, weight_grad, bias_grad
 
 

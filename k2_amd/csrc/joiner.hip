@@ -324,10 +324,29 @@ __device__ __forceinline__ float LogitGrad(float z, int n, const float4 g, int b
   return v;
 }
 
+// The same for the hybrid autoregressive transducer (k2/python/k2/rnnt_loss.py:992-1177): column 0
+// is the blank with its own sigmoid sg, py = log sg, and the other columns share a softmax whose
+// normaliser g.w leaves column 0 out, px = z[symbol] - norm + log(1 - sg):
+//   d/d z[0] = gy (1 - sg) - gx sg,   d/d z[n >= 1] = -exp(z[n] - norm) gx,   + gx at the symbol.
+__device__ __forceinline__ float LogitGradHat(float z, int n, const float4 g) {
+  float v;
+  if (n == 0) {
+    const float e = __expf(-fabsf(z));
+    const float sg = (z >= 0 ? 1.0f : e) / (1.0f + e);
+    v = g.y * (1.0f - sg) - g.x * sg;
+  } else {
+    v = -__expf(z - g.w) * g.x;
+  }
+  if (n == (int)g.z) v += g.x;
+  return v;
+}
+
 // ---------------------------------------------------------------------------------- forward
 //
 // LDS: h [MT][D + pad]; row meta; the two picked logits per row; per wavefront (max, sum) per row.
-template <typename Mode, int RB, int kD>
+// kHat: get_hat_logprobs_pruned in place of get_rnnt_logprobs_pruned: the normaliser leaves column 0
+// out, py = log sigmoid(z[0]), px = z[symbol] - norm + (py - z[0]) (a.blank is 0).
+template <typename Mode, int RB, int kD, bool kHat>
 __global__ __launch_bounds__(kThreads) void JoinerForwardKernel(const JoinerArgs a) {
   constexpr int kStepsD = kD / Mode::kChunk;  // 0: D only known at run time
   constexpr int MT = 32 * RB;
@@ -368,12 +387,13 @@ __global__ __launch_bounds__(kThreads) void JoinerForwardKernel(const JoinerArgs
     const float bn = (n < a.C && a.bias != nullptr) ? a.bias[n] : 0.f;
     if (n0 == 0) {
       // the first tile of columns starts the running pairs: no exponential (a lane whose column
-      // lies beyond C keeps the empty pair)
+      // lies beyond C keeps the empty pair, and so does the one of column 0 where that column has
+      // its own sigmoid)
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
         for (int r = 0; r < 16; ++r)
-          if (n < a.C) { run_m[rb][r] = acc[rb][r] + bn; run_s[rb][r] = 1.0f; }
+          if (n < a.C && !(kHat && n == 0)) { run_m[rb][r] = acc[rb][r] + bn; run_s[rb][r] = 1.0f; }
     } else if (n < a.C) {
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb)
@@ -470,9 +490,16 @@ __global__ __launch_bounds__(kThreads) void JoinerForwardKernel(const JoinerArgs
     a.norm[(size_t)f0 * a.R + row] = norm;
     const int T1 = a.rnnt_type == K2AMD_REGULAR ? a.Tn + 1 : a.Tn;
     const bool has_blank = a.blank >= 0 && a.blank < a.C;
-    a.py[((size_t)b * (a.S + 1) + rm.s) * a.Tn + t] = has_blank ? zblank[row] - norm : Real<float>::NegInf();
+    float shift = 0.f, yv = has_blank ? zblank[row] - norm : Real<float>::NegInf();
+    if constexpr (kHat) {
+      const float z0 = zblank[row];
+      yv = fminf(z0, 0.f) - log1pf(__expf(-fabsf(z0)));  // log sigmoid(z0)
+      shift = yv - z0;                                   // log(1 - sigmoid(z0))
+    }
+    a.py[((size_t)b * (a.S + 1) + rm.s) * a.Tn + t] = yv;
     if (rm.s < a.S) {
       float v = rm.sym >= 0 ? zsym[row] - norm : Real<float>::NegInf();
+      if constexpr (kHat) v += shift;  // (-inf stays -inf)
       if (a.rnnt_type == K2AMD_REGULAR && a.boundary != nullptr && a.boundary[4 * b + 3] == t)
         v = Real<float>::NegInf();
       a.px[((size_t)b * a.S + rm.s) * T1 + t] = v;
@@ -488,7 +515,7 @@ __global__ __launch_bounds__(kThreads) void JoinerForwardKernel(const JoinerArgs
 // through LDS 128 columns at a time: am_grad[frame] is the sum over the frame's R rows (plain
 // stores: a frame lies in one tile), lm_grad[b, s] collects its rows with atomic adds (runs of
 // equal s along t are added up first).
-template <typename Mode, int RB, int kD>
+template <typename Mode, int RB, int kD, bool kHat>
 __global__ __launch_bounds__(kThreads) void JoinerBackwardRowsKernel(const JoinerArgs a) {
   constexpr int kStepsD = kD / Mode::kChunk;  // 0: D only known at run time
   constexpr int MT = 32 * RB;
@@ -573,7 +600,8 @@ __global__ __launch_bounds__(kThreads) void JoinerBackwardRowsKernel(const Joine
         for (int e = 0; e < 4; ++e) {
           const int r = j * 4 + e;
           const int row = rb * 32 + AccRow(r, half);
-          const float v = n < a.C ? LogitGrad(acc[rb][r] + bn, n, hdr[row], a.blank) : 0.f;
+          const float z = acc[rb][r] + bn;
+          const float v = n < a.C ? (kHat ? LogitGradHat(z, n, hdr[row]) : LogitGrad(z, n, hdr[row], a.blank)) : 0.f;
           run[e] = Mode::From(v);
           colsum += Mode::To(run[e]);
           dz[(size_t)row * ldz + wave * 32 + col] = run[e];
@@ -993,7 +1021,7 @@ int PrepWeights(const float *weight, const JoinerArgs &a, bool both, const Fills
 }
 
 template <typename Mode, int RB>
-int ForwardImpl(const float *weight, JoinerArgs a, hipStream_t st) {
+int ForwardImpl(const float *weight, JoinerArgs a, bool hat, hipStream_t st) {
   constexpr int MT = 32 * RB;
   const size_t npx = (size_t)a.B * a.S * (a.rnnt_type == K2AMD_REGULAR ? a.Tn + 1 : a.Tn);
   const size_t npy = (size_t)a.B * (a.S + 1) * a.Tn;
@@ -1002,7 +1030,8 @@ int ForwardImpl(const float *weight, JoinerArgs a, hipStream_t st) {
   if (rc != K2AMD_OK) return rc;
   const size_t lds = (size_t)MT * (a.D + Mode::kPad) * sizeof(typename Mode::Elem) +
                      MT * (sizeof(RowMeta) + (2 + 2 * kWaves) * sizeof(float));
-  auto kernel = a.D == kMaxD ? JoinerForwardKernel<Mode, RB, kMaxD> : JoinerForwardKernel<Mode, RB, 0>;
+  auto kernel = hat ? (a.D == kMaxD ? JoinerForwardKernel<Mode, RB, kMaxD, true> : JoinerForwardKernel<Mode, RB, 0, true>)
+                    : (a.D == kMaxD ? JoinerForwardKernel<Mode, RB, kMaxD, false> : JoinerForwardKernel<Mode, RB, 0, false>);
   rc = AllowLds(kernel, lds);
   if (rc != K2AMD_OK) return rc;
   const long long tiles = (a.frames + a.tpt - 1) / a.tpt;
@@ -1014,7 +1043,7 @@ int ForwardImpl(const float *weight, JoinerArgs a, hipStream_t st) {
 
 template <typename Mode>
 int BackwardImpl(const float *weight, JoinerArgs a, const float *px_grad, const float *py_grad,
-                 const float *seq_scale, hipStream_t st) {
+                 const float *seq_scale, bool hat, hipStream_t st) {
   typedef typename Mode::Elem Elem;
   constexpr bool kBf = sizeof(Elem) == 2;
   const Fills fills{{a.lm_grad, a.weight_grad, a.bias_grad},
@@ -1033,7 +1062,8 @@ int BackwardImpl(const float *weight, JoinerArgs a, const float *px_grad, const 
   a.tpt = MT / a.R;
   const size_t lds = (size_t)MT * (a.D + Mode::kPad + kNTile + Mode::kPad) * sizeof(Elem) +
                      MT * (sizeof(float4) + sizeof(RowMeta)) + 32 * sizeof(unsigned long long);
-  auto kernel = a.D == kMaxD ? JoinerBackwardRowsKernel<Mode, RB, kMaxD> : JoinerBackwardRowsKernel<Mode, RB, 0>;
+  auto kernel = hat ? (a.D == kMaxD ? JoinerBackwardRowsKernel<Mode, RB, kMaxD, true> : JoinerBackwardRowsKernel<Mode, RB, 0, true>)
+                    : (a.D == kMaxD ? JoinerBackwardRowsKernel<Mode, RB, kMaxD, false> : JoinerBackwardRowsKernel<Mode, RB, 0, false>);
   rc = AllowLds(kernel, lds);
   if (rc != K2AMD_OK) return rc;
   const long long tiles = (a.frames + a.tpt - 1) / a.tpt;
@@ -1072,13 +1102,17 @@ size_t k2amd_rnnt_joiner_pruned_forward_workspace_bytes(int B, int S, int T, int
   return LayoutOf(B, T, R, C, D, precision).forward_total;
 }
 
-int k2amd_rnnt_joiner_pruned_forward(const void *am, const void *lm, const int64_t *ranges,
-                                     const void *weight, const void *bias, const int64_t *symbols,
-                                     const int64_t *boundary, void *px, void *py, void *normalizers,
-                                     int B, int S, int T, int R, int C, int D, int termination_symbol,
-                                     int rnnt_type, int precision, void *workspace,
-                                     size_t workspace_bytes, void *stream) {
+}  // extern "C"
+
+// hat: the hybrid autoregressive transducer's log-probs (column 0 is the blank, termination_symbol 0)
+static int JoinerForwardEntry(const void *am, const void *lm, const int64_t *ranges,
+                              const void *weight, const void *bias, const int64_t *symbols,
+                              const int64_t *boundary, void *px, void *py, void *normalizers,
+                              int B, int S, int T, int R, int C, int D, int termination_symbol,
+                              int rnnt_type, int precision, bool hat, void *workspace,
+                              size_t workspace_bytes, void *stream) {
   if (!JoinerShapeOk(B, S, T, R, C, D)) return K2AMD_ERR_UNSUPPORTED;
+  if (hat && C < 2) return K2AMD_ERR_INVALID_ARGUMENT;
   if (precision != K2AMD_JOINER_F32 && precision != K2AMD_JOINER_BF16) return K2AMD_ERR_INVALID_ARGUMENT;
   if (rnnt_type != K2AMD_REGULAR && rnnt_type != K2AMD_MODIFIED && rnnt_type != K2AMD_CONSTRAINED)
     return K2AMD_ERR_INVALID_ARGUMENT;
@@ -1105,19 +1139,20 @@ int k2amd_rnnt_joiner_pruned_forward(const void *am, const void *lm, const int64
                           boundary, B, S, T, R, C, D, termination_symbol, rnnt_type, 64, workspace,
                           precision);
   a.px = (float *)px; a.py = (float *)py; a.norm = (float *)normalizers;
-  return bf ? ForwardImpl<Bf16, 2>((const float *)weight, a, st)
-            : ForwardImpl<F32, 2>((const float *)weight, a, st);
+  return bf ? ForwardImpl<Bf16, 2>((const float *)weight, a, hat, st)
+            : ForwardImpl<F32, 2>((const float *)weight, a, hat, st);
 }
 
-int k2amd_rnnt_joiner_pruned_backward(const void *am, const void *lm, const int64_t *ranges,
-                                      const void *weight, const void *bias, const int64_t *symbols,
-                                      const int64_t *boundary, const void *normalizers,
-                                      const void *px_grad, const void *py_grad, const void *seq_scale,
-                                      void *am_grad, void *lm_grad, void *weight_grad, void *bias_grad,
-                                      int B, int S, int T, int R, int C, int D, int termination_symbol,
-                                      int rnnt_type, int precision, void *workspace,
-                                      size_t workspace_bytes, void *stream) {
+static int JoinerBackwardEntry(const void *am, const void *lm, const int64_t *ranges,
+                               const void *weight, const void *bias, const int64_t *symbols,
+                               const int64_t *boundary, const void *normalizers,
+                               const void *px_grad, const void *py_grad, const void *seq_scale,
+                               void *am_grad, void *lm_grad, void *weight_grad, void *bias_grad,
+                               int B, int S, int T, int R, int C, int D, int termination_symbol,
+                               int rnnt_type, int precision, bool hat, void *workspace,
+                               size_t workspace_bytes, void *stream) {
   if (!JoinerShapeOk(B, S, T, R, C, D)) return K2AMD_ERR_UNSUPPORTED;
+  if (hat && C < 2) return K2AMD_ERR_INVALID_ARGUMENT;
   if (precision != K2AMD_JOINER_F32 && precision != K2AMD_JOINER_BF16) return K2AMD_ERR_INVALID_ARGUMENT;
   if (rnnt_type != K2AMD_REGULAR && rnnt_type != K2AMD_MODIFIED && rnnt_type != K2AMD_CONSTRAINED)
     return K2AMD_ERR_INVALID_ARGUMENT;
@@ -1138,9 +1173,55 @@ int k2amd_rnnt_joiner_pruned_backward(const void *am, const void *lm, const int6
   a.am_grad = (float *)am_grad; a.lm_grad = (float *)lm_grad;
   a.weight_grad = (float *)weight_grad; a.bias_grad = (float *)bias_grad;
   return bf ? BackwardImpl<Bf16>((const float *)weight, a, (const float *)px_grad,
-                                 (const float *)py_grad, (const float *)seq_scale, st)
+                                 (const float *)py_grad, (const float *)seq_scale, hat, st)
             : BackwardImpl<F32>((const float *)weight, a, (const float *)px_grad,
-                                (const float *)py_grad, (const float *)seq_scale, st);
+                                (const float *)py_grad, (const float *)seq_scale, hat, st);
+}
+
+extern "C" {
+
+int k2amd_rnnt_joiner_pruned_forward(const void *am, const void *lm, const int64_t *ranges,
+                                     const void *weight, const void *bias, const int64_t *symbols,
+                                     const int64_t *boundary, void *px, void *py, void *normalizers,
+                                     int B, int S, int T, int R, int C, int D, int termination_symbol,
+                                     int rnnt_type, int precision, void *workspace,
+                                     size_t workspace_bytes, void *stream) {
+  return JoinerForwardEntry(am, lm, ranges, weight, bias, symbols, boundary, px, py, normalizers, B, S, T, R, C, D,
+                            termination_symbol, rnnt_type, precision, false, workspace, workspace_bytes, stream);
+}
+
+int k2amd_rnnt_joiner_pruned_backward(const void *am, const void *lm, const int64_t *ranges,
+                                      const void *weight, const void *bias, const int64_t *symbols,
+                                      const int64_t *boundary, const void *normalizers,
+                                      const void *px_grad, const void *py_grad, const void *seq_scale,
+                                      void *am_grad, void *lm_grad, void *weight_grad, void *bias_grad,
+                                      int B, int S, int T, int R, int C, int D, int termination_symbol,
+                                      int rnnt_type, int precision, void *workspace,
+                                      size_t workspace_bytes, void *stream) {
+  return JoinerBackwardEntry(am, lm, ranges, weight, bias, symbols, boundary, normalizers, px_grad, py_grad,
+                             seq_scale, am_grad, lm_grad, weight_grad, bias_grad, B, S, T, R, C, D,
+                             termination_symbol, rnnt_type, precision, false, workspace, workspace_bytes, stream);
+}
+
+int k2amd_rnnt_joiner_hat_pruned_forward(const void *am, const void *lm, const int64_t *ranges,
+                                         const void *weight, const void *bias, const int64_t *symbols,
+                                         const int64_t *boundary, void *px, void *py, void *normalizers,
+                                         int B, int S, int T, int R, int C, int D, int rnnt_type,
+                                         int precision, void *workspace, size_t workspace_bytes, void *stream) {
+  return JoinerForwardEntry(am, lm, ranges, weight, bias, symbols, boundary, px, py, normalizers, B, S, T, R, C, D,
+                            0, rnnt_type, precision, true, workspace, workspace_bytes, stream);
+}
+
+int k2amd_rnnt_joiner_hat_pruned_backward(const void *am, const void *lm, const int64_t *ranges,
+                                          const void *weight, const void *bias, const int64_t *symbols,
+                                          const int64_t *boundary, const void *normalizers,
+                                          const void *px_grad, const void *py_grad, const void *seq_scale,
+                                          void *am_grad, void *lm_grad, void *weight_grad, void *bias_grad,
+                                          int B, int S, int T, int R, int C, int D, int rnnt_type, int precision,
+                                          void *workspace, size_t workspace_bytes, void *stream) {
+  return JoinerBackwardEntry(am, lm, ranges, weight, bias, symbols, boundary, normalizers, px_grad, py_grad,
+                             seq_scale, am_grad, lm_grad, weight_grad, bias_grad, B, S, T, R, C, D, 0, rnnt_type,
+                             precision, true, workspace, workspace_bytes, stream);
 }
 
 }  // extern "C"

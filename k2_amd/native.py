@@ -266,16 +266,16 @@ def logprobs_pruned_backward(logits, norm, px_grad, py_grad, symbols, ranges, bo
 
 
 def joiner_pruned_forward(am, lm, ranges, weight, bias, symbols, termination_symbol, boundary,
-                          rnnt_type, precision):
+                          rnnt_type, precision, hat=False):
     _require_device(am)
     return capi.joiner_pruned_forward(am, lm, ranges, weight, bias, symbols, termination_symbol,
-                                      boundary, rnnt_type, precision)
+                                      boundary, rnnt_type, precision, hat)
 
 
 def joiner_pruned_backward(am, lm, ranges, weight, bias, symbols, termination_symbol, boundary,
-                           rnnt_type, norm, px_grad, py_grad, seq_scale, precision):
+                           rnnt_type, norm, px_grad, py_grad, seq_scale, precision, hat=False):
     return capi.joiner_pruned_backward(am, lm, ranges, weight, bias, symbols, termination_symbol,
-                                       boundary, rnnt_type, norm, px_grad, py_grad, seq_scale, precision)
+                                       boundary, rnnt_type, norm, px_grad, py_grad, seq_scale, precision, hat)
 
 
 def prune_ranges(px_grad, py_grad, boundary, s_range):

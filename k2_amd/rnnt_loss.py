@@ -180,11 +180,11 @@ class _Scores(torch.autograd.Function):
                                                          rnnt_code, boundary)
             saved = (logits, norm)
         elif kind == "joiner":
-            am, lm, ranges, weight, bias, symbols, termination_symbol, rnnt_code, _, precision = args
+            am, lm, ranges, weight, bias, symbols, termination_symbol, rnnt_code, _, precision, hat = args
             am, lm, weight = am.contiguous(), lm.contiguous(), weight.contiguous()
             bias = bias.contiguous() if bias is not None else None
             px, py, norm = native.joiner_pruned_forward(am, lm, ranges, weight, bias, symbols,
-                                                        termination_symbol, boundary, rnnt_code, precision)
+                                                        termination_symbol, boundary, rnnt_code, precision, hat)
             saved = (am, lm, weight, norm) + ((bias,) if bias is not None else ())
         else:
             logits, symbols, ranges, termination_symbol, rnnt_code, _, hat = args
@@ -231,11 +231,11 @@ class _Scores(torch.autograd.Function):
             grads = (native.logprobs_joint_backward(saved[0], saved[1], px_grad, py_grad, symbols,
                                                     boundary, termination_symbol, rnnt_code, scale),)
         elif ctx.kind == "joiner":
-            _, _, ranges, _, bias, symbols, termination_symbol, rnnt_code, boundary, precision = args
+            _, _, ranges, _, bias, symbols, termination_symbol, rnnt_code, boundary, precision, hat = args
             am, lm, weight, norm = saved[:4]
             d_am, d_lm, d_w, d_b = native.joiner_pruned_backward(
                 am, lm, ranges, weight, saved[4] if bias is not None else None, symbols,
-                termination_symbol, boundary, rnnt_code, norm, px_grad, py_grad, scale, precision)
+                termination_symbol, boundary, rnnt_code, norm, px_grad, py_grad, scale, precision, hat)
             grads = (d_am, d_lm, None, d_w, d_b)
         else:
             _, symbols, ranges, termination_symbol, rnnt_code, boundary, hat = args
@@ -545,6 +545,7 @@ def rnnt_loss_pruned_joiner(
     delay_penalty: float = 0.0,
     reduction: Optional[str] = "mean",
     precision: str = "fp32",
+    use_hat_loss: bool = False,
 ) -> Tensor:
     """do_rnnt_pruning -> joiner -> rnnt_loss_pruned (k2/python/k2/rnnt_loss.py:913-954, the
     caller's joiner, :1351-1468) as one call for the usual joiner,
@@ -555,7 +556,17 @@ def rnnt_loss_pruned_joiner(
     get_rnnt_prune_ranges, weight [C][D] and bias [C] (or None) those of the output layer.  The
     [B][T][s_range][C] logits are never stored; gradients flow to am, lm, weight and bias.
     ``precision``: "fp32" multiplies in fp32; "bf16" rounds the activations, the weight and the logits'
-    gradients to bfloat16 for the matrix products (fp32 accumulation), as autocast would."""
+    gradients to bfloat16 for the matrix products (fp32 accumulation), as autocast would.
+    ``use_hat_loss``: as in rnnt_loss_pruned (k2/python/k2/rnnt_loss.py:1439-1447), the hybrid
+    autoregressive transducer's log-probs, termination_symbol 0.  That variant of the kernels has
+    so far run in its host-thread build only (tests/test_cpu_build_host_layer.py), never on a GPU:
+    it is refused unless K2AMD_JOINER_HAT=1 is set; the three separate steps serve meanwhile."""
+    if use_hat_loss:
+        assert termination_symbol == 0, "the hybrid autoregressive transducer's blank is symbol 0"
+        if os.environ.get("K2AMD_JOINER_HAT", "0") != "1":
+            raise RuntimeError("k2_amd: rnnt_loss_pruned_joiner(use_hat_loss=True) has not run on a GPU yet and is "
+                               "off by default: set K2AMD_JOINER_HAT=1 to use it, or call do_rnnt_pruning, the "
+                               "joiner and rnnt_loss_pruned(use_hat_loss=True) one after the other")
     assert am.ndim == 3 and lm.ndim == 3, (am.shape, lm.shape)
     (B, T, D) = am.shape
     assert lm.shape[0] == B and lm.shape[2] == D, (am.shape, lm.shape)
@@ -568,7 +579,8 @@ def rnnt_loss_pruned_joiner(
     assert precision in capi.JOINER_PRECISIONS, precision
     _validate_st_lengths(S, T, rnnt_type == "regular", boundary)
     args = (am, lm, _dev_i64(ranges, am), weight, bias, _dev_i64(symbols, am), int(termination_symbol),
-            capi.RNNT_TYPES[rnnt_type], _dev_i64(boundary, am), capi.JOINER_PRECISIONS[precision])
+            capi.RNNT_TYPES[rnnt_type], _dev_i64(boundary, am), capi.JOINER_PRECISIONS[precision],
+            bool(use_hat_loss))
     return _Scores.apply("joiner", rnnt_type, float(delay_penalty), False, reduction, *args)[0]
 
 

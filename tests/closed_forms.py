@@ -133,10 +133,10 @@ def _pruned_logits_grad(logits, symbols, ranges, blank, gxs, gys, scale, rnnt_ty
                 # log px = l[sym] - logsumexp(l[1:]) + log(1 - sig);  log py = log sig
                 g = np.zeros(logits[b].shape, np.float64)
                 g[..., 1:] = P * gxb[..., None]
+                g[..., 0] = gxb * sig - gyb * (1.0 - sig)
+            # (after column 0 is in place: a label equal to 0 takes its -gx there as anywhere else)
             np.put_along_axis(g, sym[..., None],
                               np.take_along_axis(g, sym[..., None], axis=2) - gxb[..., None], axis=2)
-            if hat:
-                g[..., 0] = gxb * sig - gyb * (1.0 - sig)
             out[b] = scale[b] * g
     return outs
 

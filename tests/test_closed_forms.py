@@ -90,3 +90,33 @@ def test_smoothed_closed_form_equals_autograd(rnnt_type, scales):
     lm_g, am_g = cf.smoothed_grads(c["lm"], c["am"], c["symbols"], 0, scales[0], scales[1], gx, gy, w, rnnt_type)
     np.testing.assert_allclose(lm_g, lm.grad.numpy(), rtol=1e-9, atol=1e-12)
     np.testing.assert_allclose(am_g, am.grad.numpy(), rtol=1e-9, atol=1e-12)
+
+
+def test_hat_closed_form_with_a_label_equal_to_zero():
+    """A label equal to 0 under HAT is outside what the variant is meant for (0 is the blank), and
+    there k2's code (px = logits[symbol] - logsumexp(logits[1:]) + log(1 - sigmoid(logits[0])),
+    rnnt_loss.py:1115-1160) and the textbook distribution part ways; the kernels and the closed
+    form follow k2's code.  Pinned by central differences over the oracle's restatement of it."""
+    B, T, S, R, C = 2, 6, 4, 2, 5
+    c = cases.rnnt_case(66, B, T, S, C, dtype=np.float64, t_lo=5, s_lo=3)
+    c["symbols"][:, 1] = 0
+    rng = np.random.default_rng(67)
+    ranges = _random_ranges(rng, B, T, S, R)
+    logits = rng.standard_normal((B, T, R, C))
+    px, py = orn.hat_logprobs_pruned(logits, c["symbols"], ranges, 0, c["boundary"], "regular")
+    fx, fy = np.isfinite(px), np.isfinite(py)
+    wx, wy = np.where(fx, rng.uniform(0.1, 1.0, px.shape), 0.0), np.where(fy, rng.uniform(0.1, 1.0, py.shape), 0.0)
+
+    def value(x):
+        a, b = orn.hat_logprobs_pruned(x, c["symbols"], ranges, 0, c["boundary"], "regular")
+        return (np.where(fx, a, 0.0) * wx).sum() + (np.where(fy, b, 0.0) * wy).sum()
+
+    got = cf.pruned_logits_grad(logits, c["symbols"], ranges, 0, wx, wy, -np.ones(B), "regular", hat=True)
+    want = np.zeros_like(logits)
+    eps = 1e-6
+    for i in np.ndindex(logits.shape):
+        up, down = logits.copy(), logits.copy()
+        up[i] += eps
+        down[i] -= eps
+        want[i] = (value(up) - value(down)) / (2 * eps)
+    np.testing.assert_allclose(got, want, rtol=1e-6, atol=1e-8)

@@ -323,22 +323,29 @@ def test_smoke_entry_point_runs(host_on_cpu, capsys):
 # spell bfloat16 vectors and aligned dynamic LDS are replaced (tests/cpu_kernels.py); the matrix
 # instructions of both operand types and the quad DPP moves come from the stand-in -----------------
 
+@pytest.mark.parametrize("hat", [False, True])
 @pytest.mark.parametrize("rnnt_type", TYPES)
-def test_fused_joiner_fp32(host_on_cpu, rnnt_type):
+def test_fused_joiner_fp32(host_on_cpu, rnnt_type, hat):
+    """hat: the hybrid autoregressive transducer's log-probs inside the fused kernels (column 0 with
+    its own sigmoid, the normaliser over the other columns)."""
     import test_joiner_gpu as tj
     cpu = torch.device("cpu")
-    for seed, B, T, S, C, D, R, with_bias in ((1, 2, 9, 4, 11, 64, 3, True), (2, 1, 7, 3, 70, 128, 2, False)):
+    # the second shape has more than one tile of 256 columns: column 0 is left out of the
+    # normaliser in the first tile only
+    for seed, B, T, S, C, D, R, with_bias in ((1, 2, 9, 4, 11, 64, 3, True), (2, 1, 7, 3, 300, 128, 2, False)):
         c = tj.joiner_case(seed, B, T, S, C, D, R, rnnt_type, with_bias)
-        logits, px, py = tj.chain_fp64(c)
-        gpx, gpy, norm = tj.run_forward(c, cpu, "fp32")
+        if hat:
+            c["symbols"][:, 0] = 0  # the blank's column as an ordinary symbol
+        logits, px, py = tj.chain_fp64(c, hat)
+        gpx, gpy, norm = tj.run_forward(c, cpu, "fp32", hat)
         tag = f"{rnnt_type} seed {seed}"
         tj.close(tag + " px", gpx.numpy(), px, 1e-4, 1e-5 / max(np.abs(px[np.isfinite(px)]).max(), 1e-30))
         tj.close(tag + " py", gpy.numpy(), py, 1e-4, 1e-5 / max(np.abs(py[np.isfinite(py)]).max(), 1e-30))
         _, gx, gy = omi.mi(px, py, c["boundary"])
         gx, gy = gx.astype(np.float32), gy.astype(np.float32)
         scale = np.linspace(0.5, 1.5, B).astype(np.float32)
-        want = tj.closed_form_grads(c, logits, gx, gy, scale)
-        got = tj.run_backward(c, cpu, "fp32", norm, gx, gy, scale)
+        want = tj.closed_form_grads(c, logits, gx, gy, scale, hat)
+        got = tj.run_backward(c, cpu, "fp32", norm, gx, gy, scale, hat)
         for name, g, w in zip(("am_grad", "lm_grad", "weight_grad", "bias_grad"), got, want):
             if g is None:
                 assert name == "bias_grad" and not with_bias
@@ -364,3 +371,29 @@ def test_fused_joiner_bf16_and_no_frames(host_on_cpu):
                                              torch.from_numpy(rng.standard_normal((C, D)).astype(np.float32)), None,
                                              torch.from_numpy(rng.integers(1, C, (B, S)).astype(np.int64)), 0, None, 0)
     assert tuple(px0.shape) == (B, S, 1) and tuple(py0.shape) == (B, S + 1, 0) and torch.isneginf(px0).all()
+
+
+def test_hat_loss_through_the_fused_joiner(host_on_cpu, monkeypatch):
+    """rnnt_loss_pruned_joiner(use_hat_loss=True) against the three steps it replaces
+    (do_rnnt_pruning, tanh + linear, rnnt_loss_pruned(use_hat_loss=True)): loss and the gradients
+    to am, lm, weight and bias; refused while its switch is off."""
+    import k2_amd as k2
+    import test_joiner_gpu as tj
+    c = tj.joiner_case(5, 2, 9, 4, 11, 64, 3, "regular", True)
+    t = lambda k, grad=False: torch.from_numpy(c[k]).requires_grad_(grad)
+    sym, bd, ranges = t("symbols"), t("boundary"), t("ranges")
+    a1, l1, w1, b1 = t("am", True), t("lm", True), t("weight", True), t("bias", True)
+    with pytest.raises(RuntimeError, match="K2AMD_JOINER_HAT"):
+        k2.rnnt_loss_pruned_joiner(a1, l1, ranges, w1, b1, sym, 0, bd, reduction="sum", use_hat_loss=True)
+    monkeypatch.setenv("K2AMD_JOINER_HAT", "1")
+    fused = k2.rnnt_loss_pruned_joiner(a1, l1, ranges, w1, b1, sym, 0, bd, reduction="sum", use_hat_loss=True)
+    fused.backward()
+    a2, l2, w2, b2 = t("am", True), t("lm", True), t("weight", True), t("bias", True)
+    am_p, lm_p = k2.do_rnnt_pruning(a2, l2, ranges)
+    logits = torch.nn.functional.linear(torch.tanh(am_p + lm_p), w2, b2)
+    steps = k2.rnnt_loss_pruned(logits, sym, ranges, 0, bd, reduction="sum", use_hat_loss=True)
+    steps.backward()
+    np.testing.assert_allclose(fused.item(), steps.item(), rtol=1e-5)
+    for name, x, y in (("am", a1, a2), ("lm", l1, l2), ("weight", w1, w2), ("bias", b1, b2)):
+        scale = float(y.grad.abs().max())
+        np.testing.assert_allclose(x.grad.numpy(), y.grad.numpy(), rtol=1e-4, atol=1e-5 * scale, err_msg=name)

@@ -42,21 +42,22 @@ def joiner_case(seed, B, T, S, C, D, R, rnnt_type="regular", with_bias=True, t_l
                 ranges=ranges, symbols=c["symbols"], boundary=c["boundary"], rnnt_type=rnnt_type)
 
 
-def chain_fp64(c):
+def chain_fp64(c, hat=False):
     """logits, px, py of the chain in fp64 on the fp32 inputs."""
     f = lambda x: None if x is None else x.astype(np.float64)
     logits = orn.joiner_pruned_logits(f(c["am"]), f(c["lm"]), c["ranges"], f(c["weight"]), f(c["bias"]))
-    px, py = orn.logprobs_pruned(logits, c["symbols"], c["ranges"], 0, c["boundary"], c["rnnt_type"])
+    builder = orn.hat_logprobs_pruned if hat else orn.logprobs_pruned
+    px, py = builder(logits, c["symbols"], c["ranges"], 0, c["boundary"], c["rnnt_type"])
     return logits, px, py
 
 
-def closed_form_grads(c, logits, gx, gy, scale):
+def closed_form_grads(c, logits, gx, gy, scale, hat=False):
     """fp64 gradients of sum_b scale[b] * score_b w.r.t. am, lm, weight, bias, given the gradients
     gx, gy of the scores w.r.t. px, py: the closed form for the logits, then the chain rule through
     the linear layer, tanh and the gather."""
     B, T, R = c["ranges"].shape
     d_logits = -cf.pruned_logits_grad(logits, c["symbols"], c["ranges"], 0, gx.astype(np.float64),
-                                      gy.astype(np.float64), scale.astype(np.float64), c["rnnt_type"])
+                                      gy.astype(np.float64), scale.astype(np.float64), c["rnnt_type"], hat=hat)
     am, lm, w = c["am"].astype(np.float64), c["lm"].astype(np.float64), c["weight"].astype(np.float64)
     h = np.tanh(am[:, :, None, :] + lm[np.arange(B)[:, None, None], c["ranges"], :])
     d_w = np.einsum("btkc,btkd->cd", d_logits, h, optimize=True)
@@ -82,21 +83,21 @@ def close(name, got, want, rtol, atol_of_max):
     assert worst <= 1.0, (name, worst)
 
 
-def run_forward(c, device, precision):
+def run_forward(c, device, precision, hat=False):
     from k2_amd import capi
     return capi.joiner_pruned_forward(dev(c["am"], device), dev(c["lm"], device), dev(c["ranges"], device),
                                       dev(c["weight"], device), dev(c["bias"], device), dev(c["symbols"], device),
                                       0, dev(c["boundary"], device), capi.RNNT_TYPES[c["rnnt_type"]],
-                                      capi.JOINER_PRECISIONS[precision])
+                                      capi.JOINER_PRECISIONS[precision], hat)
 
 
-def run_backward(c, device, precision, norm, gx, gy, scale):
+def run_backward(c, device, precision, norm, gx, gy, scale, hat=False):
     from k2_amd import capi
     out = capi.joiner_pruned_backward(dev(c["am"], device), dev(c["lm"], device), dev(c["ranges"], device),
                                       dev(c["weight"], device), dev(c["bias"], device), dev(c["symbols"], device),
                                       0, dev(c["boundary"], device), capi.RNNT_TYPES[c["rnnt_type"]], norm,
                                       dev(gx, device), dev(gy, device), dev(scale, device),
-                                      capi.JOINER_PRECISIONS[precision])
+                                      capi.JOINER_PRECISIONS[precision], hat)
     torch.cuda.synchronize()
     return [None if t is None else t.cpu().numpy() for t in out]
 
