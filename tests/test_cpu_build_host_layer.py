@@ -323,8 +323,10 @@ def test_smoke_entry_point_runs(host_on_cpu, capsys):
 # spell bfloat16 vectors and aligned dynamic LDS are replaced (tests/cpu_kernels.py); the matrix
 # instructions of both operand types and the quad DPP moves come from the stand-in -----------------
 
-@pytest.mark.parametrize("hat", [False, True])
-@pytest.mark.parametrize("rnnt_type", TYPES)
+@pytest.mark.parametrize("rnnt_type,hat", [("regular", False), ("constrained", True), ("modified", True),
+                                           pytest.param("modified", False, marks=slow),
+                                           pytest.param("constrained", False, marks=slow),
+                                           pytest.param("regular", True, marks=slow)])
 def test_fused_joiner_fp32(host_on_cpu, rnnt_type, hat):
     """hat: the hybrid autoregressive transducer's log-probs inside the fused kernels (column 0 with
     its own sigmoid, the normaliser over the other columns)."""
