@@ -3,14 +3,20 @@
 // other, each workgroup's work-items as threads of their own, so that barriers and wavefront
 // exchanges keep their meaning, and a host sanitizer or a CPU debugger sees the kernels' indexing.
 //
-// What it has: launches with static and dynamic LDS, __syncthreads, the __shfl family, atomics,
-// vector types, __half as storage, and of the gfx9 builtins readlane / readfirstlane, the two
-// whole-wavefront DPP shifts, v_mfma_f32_32x32x2_f32 (from its documented operand layout),
-// wave_barrier (a real barrier here: the lanes are free-running threads, not in lockstep) and
-// no-ops for fences and scheduling hints.  What it does not have: inline assembly, other DPP
-// controls, bfloat16 vectors, concurrency BETWEEN workgroups (a kernel whose workgroups wait for
-// one another must only ever wait for workgroups that started earlier).  Slow by design: sizes
-// stay small.
+// What it has: launches with static and dynamic LDS, __syncthreads, the __shfl family, atomics
+// (also the agent-scope builtins), vector types, __half as storage, and of the gfx9 builtins
+// readlane / readfirstlane, the DPP moves that the kernels use (quad permutations, mirrored rows,
+// the two whole-wavefront shifts), the matrix instructions v_mfma_f32_32x32x2_f32 and
+// v_mfma_f32_32x32x16_bf16 (from their documented operand layouts), exp2 / log2 / rcp,
+// wave_barrier and fences at wavefront scope (real barriers here: the lanes are free-running
+// threads, not in lockstep), s_barrier, s_sleep, and no-ops for other fences and scheduling hints;
+// helpers that do what three instructions do which the kernels spell in assembly (the host build
+// compiles copies of those sources with calls to the helpers in the assembly's place).  What it
+// does not have: inline assembly, other DPP controls, bfloat16 arithmetic.  Workgroups do not
+// overlap unless hip_threads::concurrent_workgroups asks for it (then every workgroup is a child
+// process): a kernel whose workgroups wait for one another must only ever wait for workgroups that
+// started earlier, as on the device, where a later one may not be resident yet.  Slow by design:
+// sizes stay small.
 #ifndef K2_AMD_TESTS_CPU_BUILD_HIP_RUNTIME_H_
 #define K2_AMD_TESTS_CPU_BUILD_HIP_RUNTIME_H_
 
@@ -19,6 +25,9 @@
 #include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
+
+#include <sys/wait.h>
+#include <unistd.h>
 
 #include <algorithm>
 #include <atomic>
@@ -110,19 +119,24 @@ inline T exchange(T v, int src_lane) {
   return r;
 }
 
+// 0: the workgroups of a launch run one after the other in this process.  n > 0: every workgroup
+// runs in a child process of its own (its threads, its own copy of the kernel's static LDS
+// variables), n of them at a time, started in the order of their indices: workgroups then really
+// overlap, as on the device, and what they hand to each other goes through whatever memory the
+// caller has mapped as shared between processes (every buffer a kernel writes has to be; the
+// kernels' arguments are copied at the fork).  For tests of what workgroups say to each other.
+inline int concurrent_workgroups = 0;
+
 template <typename Kernel, typename... Args>
-void launch(Kernel kernel, dim3 grid, dim3 block, size_t dynamic_lds_bytes, Args... args) {
+void run_workgroups(Kernel kernel, dim3 grid, dim3 block, size_t dynamic_lds_bytes, size_t first, size_t last,
+                    Args... args) {
   const int threads = (int)(block.x * block.y * block.z);
-  const size_t blocks = (size_t)grid.x * grid.y * grid.z;
-  if (threads == 0 || blocks == 0) return;
-  block_dim = {block.x, block.y, block.z};
-  grid_dim = {grid.x, grid.y, grid.z};
   // exactly the bytes asked for, on the heap: a sanitizer sees an access beyond them
   std::unique_ptr<unsigned char[]> lds(new unsigned char[std::max<size_t>(dynamic_lds_bytes, 1)]);
   state().dynamic_lds = lds.get();
-  // One set of threads for the whole launch; the workgroups run one after the other.  A work-item
-  // that leaves the kernel drops out of its wavefront's and its workgroup's barriers, as exited
-  // lanes and wavefronts do on the hardware, so those barriers are made anew for every workgroup.
+  // One set of threads for all of them.  A work-item that leaves the kernel drops out of its
+  // wavefront's and its workgroup's barriers, as exited lanes and wavefronts do on the hardware, so
+  // those barriers are made anew for every workgroup.
   std::unique_ptr<std::barrier<>> block_barrier;
   std::vector<Wave> waves((threads + kWaveSize - 1) / kWaveSize);
   auto fresh = [&] {
@@ -143,7 +157,7 @@ void launch(Kernel kernel, dim3 grid, dim3 block, size_t dynamic_lds_bytes, Args
     pool.emplace_back([&, t] {
       flat_thread = t;
       thread_idx = {t % block.x, (t / block.x) % block.y, t / (block.x * block.y)};
-      for (size_t k = 0; k < blocks; ++k) {
+      for (size_t k = first; k < last; ++k) {
         exchanges = 0;
         block_idx = {(unsigned)(k % grid.x), (unsigned)((k / grid.x) % grid.y), (unsigned)(k / ((size_t)grid.x * grid.y))};
         kernel(args...);
@@ -156,6 +170,35 @@ void launch(Kernel kernel, dim3 grid, dim3 block, size_t dynamic_lds_bytes, Args
   state().dynamic_lds = nullptr;
   state().block_barrier = nullptr;
   state().waves = nullptr;
+}
+
+template <typename Kernel, typename... Args>
+void launch(Kernel kernel, dim3 grid, dim3 block, size_t dynamic_lds_bytes, Args... args) {
+  const int threads = (int)(block.x * block.y * block.z);
+  const size_t blocks = (size_t)grid.x * grid.y * grid.z;
+  if (threads == 0 || blocks == 0) return;
+  block_dim = {block.x, block.y, block.z};
+  grid_dim = {grid.x, grid.y, grid.z};
+  if (concurrent_workgroups <= 0) {
+    run_workgroups(kernel, grid, block, dynamic_lds_bytes, 0, blocks, args...);
+    return;
+  }
+  size_t started = 0, alive = 0;
+  while (started < blocks || alive > 0) {
+    while (started < blocks && alive < (size_t)concurrent_workgroups) {
+      const pid_t child = fork();
+      if (child < 0) abort();
+      if (child == 0) {
+        run_workgroups(kernel, grid, block, dynamic_lds_bytes, started, started + 1, args...);
+        _exit(0);
+      }
+      ++started;
+      ++alive;
+    }
+    int status = 0;
+    if (wait(&status) < 0 || !WIFEXITED(status) || WEXITSTATUS(status) != 0) abort();
+    --alive;
+  }
 }
 
 }  // namespace hip_threads
@@ -183,7 +226,12 @@ inline T __shfl(T v, int src_lane, int width = hip_threads::kWaveSize) {
 // ---- what the fp32 matrix-core products of rnnt_simple.hip use --------------------------------
 // clang's ext_vector_type for FLOAT vectors (the only ones in the files of the host build)
 #define ext_vector_type(n) vector_size(4 * (n))
-#define __builtin_amdgcn_fence(...) ((void)0)
+// A fence orders one thread's accesses, which the sequentially consistent atomics and the barriers
+// of this stand-in do already; at wavefront scope the kernels use it where the lanes of one
+// wavefront hand values to each other through LDS and rely on running in lockstep, so here it is
+// a barrier over the wavefront (every live lane has to reach it, as it does on the hardware).
+inline void hip_threads_fence(int, const char *scope, const char * = nullptr);
+#define __builtin_amdgcn_fence(...) hip_threads_fence(__VA_ARGS__)
 #define __builtin_amdgcn_sched_barrier(mask) ((void)0)
 inline void __builtin_amdgcn_s_barrier() { __syncthreads(); }
 
@@ -242,6 +290,14 @@ inline hip_threads_float16 __builtin_amdgcn_mfma_f32_32x32x16_bf16(hip_threads_b
   return c;
 }
 inline float __builtin_amdgcn_exp2f(float x) { return exp2f(x); }
+inline float __builtin_amdgcn_logf(float x) { return log2f(x); }
+inline void __builtin_amdgcn_s_setprio(int) {}
+inline unsigned __float_as_uint(float f) { unsigned u; memcpy(&u, &f, 4); return u; }
+inline float __uint_as_float(unsigned u) { float f; memcpy(&f, &u, 4); return f; }
+enum hipDeviceAttribute_t { hipDeviceAttributeMultiprocessorCount };
+// (the compute units of the device that the library is written for: the single launch sizes its
+// grid with it and the kernel selection compares with it)
+inline hipError_t hipDeviceGetAttribute(int *value, hipDeviceAttribute_t, int) { *value = 256; return hipSuccess; }
 enum hipFuncAttribute { hipFuncAttributeMaxDynamicSharedMemorySize };
 inline hipError_t hipFuncSetAttribute(const void *, hipFuncAttribute, int) { return hipSuccess; }
 
@@ -249,13 +305,19 @@ inline hipError_t hipFuncSetAttribute(const void *, hipFuncAttribute, int) { ret
 #define __HIP_MEMORY_SCOPE_AGENT 0
 #define __hip_atomic_load(address, order, scope) hip_threads::atomic_load(address)
 #define __hip_atomic_store(address, value, order, scope) hip_threads::atomic_store(address, value)
+#define __hip_atomic_fetch_add(address, value, order, scope) std::atomic_ref(*(address)).fetch_add(value)
 namespace hip_threads {
 template <typename T>
 inline T atomic_load(T *address) { return std::atomic_ref<T>(*address).load(std::memory_order_seq_cst); }
 template <typename T, typename V>
 inline void atomic_store(T *address, V value) { std::atomic_ref<T>(*address).store((T)value, std::memory_order_seq_cst); }
 }  // namespace hip_threads
-inline void __builtin_amdgcn_s_sleep(int) { std::this_thread::yield(); }
+// (a poll loop's pause; with workgroups in processes of their own the poller sleeps, so that the
+// hundreds of threads of the workgroup it waits for get the cores, and a bounded wait of a million
+// polls does not run out while they are still being scheduled)
+inline void __builtin_amdgcn_s_sleep(int) {
+  if (hip_threads::concurrent_workgroups > 0) usleep(20); else std::this_thread::yield();
+}
 inline float __builtin_amdgcn_rcpf(float x) { return 1.0f / x; }
 template <typename T>
 inline T __builtin_amdgcn_readlane(T v, int lane) { return hip_threads::exchange(v, lane); }
@@ -263,12 +325,18 @@ template <typename T>
 inline T __builtin_amdgcn_readfirstlane(T v) { return hip_threads::exchange(v, 0); }  // (lane 0 is live wherever it is used)
 // DPP moves: within quads (quad_perm), and over the whole wavefront wave_shr:1 (0x138: lane l
 // takes lane l - 1, lane 0 keeps `old`) and wave_shl:1 (0x130: lane l takes lane l + 1, lane 63
-// keeps `old`); all rows and banks enabled, as the kernels ask for.  Other controls are not emulated.
-inline int __builtin_amdgcn_update_dpp(int old, int src, int ctrl, int row_mask, int bank_mask, bool bound_ctrl) {
+// keeps `old`), mirrored rows; all rows and banks enabled, as the kernels ask for.  Other controls
+// are not emulated.
+inline int hip_threads_update_dpp(int old, int src, int ctrl, int row_mask, int bank_mask, bool bound_ctrl) {
   const int lane = hip_threads::flat_thread % hip_threads::kWaveSize;
   if (ctrl >= 0 && ctrl < 0x100) {  // quad_perm: lane 4 q + i takes lane 4 q + ((ctrl >> 2 i) & 3); always in range
     if (row_mask != 0xf || bank_mask != 0xf) abort();
     return hip_threads::exchange(src, (lane & ~3) | ((ctrl >> (2 * (lane & 3))) & 3));
+  }
+  if (ctrl == 0x140 || ctrl == 0x141) {  // row_mirror, row_half_mirror: lane i of a row of 16 (8) takes lane 15 - i (7 - i)
+    if (row_mask != 0xf || bank_mask != 0xf) abort();
+    const int width = ctrl == 0x140 ? 16 : 8;
+    return hip_threads::exchange(src, (lane & ~(width - 1)) | (width - 1 - (lane & (width - 1))));
   }
   if ((ctrl != 0x138 && ctrl != 0x130) || row_mask != 0xf || bank_mask != 0xf || bound_ctrl) abort();
   const int from = ctrl == 0x138 ? lane - 1 : lane + 1;
@@ -276,9 +344,58 @@ inline int __builtin_amdgcn_update_dpp(int old, int src, int ctrl, int row_mask,
   return from < 0 || from >= hip_threads::my_wave().lanes ? old : got;
 }
 
+template <typename T>  // int or unsigned
+inline T __builtin_amdgcn_update_dpp(T old, T src, int ctrl, int row_mask, int bank_mask, bool bound_ctrl) {
+  static_assert(sizeof(T) == 4, "");
+  return (T)hip_threads_update_dpp((int)old, (int)src, ctrl, row_mask, bank_mask, bound_ctrl);
+}
+
+// The two DPP instructions that the pipelined kernels spell in assembly, for the copy of
+// mi_fast.hip that the host build compiles (tests/cpu_kernels.py puts these calls in the place of
+// the assembly blocks):
+//   v_add_f32_dpp inc, P, inc wave_shr:1   inc = P(lane - 1) + inc; lane 0 has no source lane and
+//                                          is left alone
+//   v_mul_f32_dpp t, G, t wave_shl:1       t = G(lane + 1) * t; lane 63 likewise
+inline float hip_threads_add_from_lane_above(float P, float inc) {
+  const int lane = hip_threads::flat_thread % hip_threads::kWaveSize;
+  const float above = hip_threads::exchange(P, std::max(lane - 1, 0));
+  return lane == 0 ? inc : above + inc;
+}
+inline float hip_threads_mul_from_lane_below(float G, float t) {
+  const int lane = hip_threads::flat_thread % hip_threads::kWaveSize;
+  const float below = hip_threads::exchange(G, std::min(lane + 1, hip_threads::kWaveSize - 1));
+  return lane == hip_threads::kWaveSize - 1 ? t : below * t;
+}
+// buffer_load_dwordx4 ... offen through a raw buffer resource (words 0 and 1: the base address,
+// word 2: the size in bytes): every dword is range-checked by itself and reads as 0 when any of
+// its bytes lies at or beyond the size.
+struct hip_threads_int4 { int x, y, z, w; };
+struct hip_threads_float4 { float x, y, z, w; };
+inline hip_threads_float4 hip_threads_buffer_load4(hip_threads_int4 resource, int byte_offset) {
+  const unsigned long long base = (unsigned long long)(unsigned)resource.x | ((unsigned long long)(unsigned)resource.y << 32);
+  const unsigned size = (unsigned)resource.z;
+  float out[4];
+  for (int i = 0; i < 4; ++i) {
+    const unsigned long long at = (unsigned long long)(unsigned)byte_offset + 4ull * i;
+    out[i] = 0.0f;
+    if (at + 4 <= size) memcpy(&out[i], reinterpret_cast<const void *>(base + at), 4);
+  }
+  return {out[0], out[1], out[2], out[3]};
+}
+
 // On the hardware a scheduling fence that emits nothing (a wavefront's lanes run in lockstep);
 // here the lanes are free-running threads, so it has to be a real barrier over the wavefront.
 inline void __builtin_amdgcn_wave_barrier() { hip_threads::my_wave().barrier->arrive_and_wait(); }
+// (HIP_THREADS_FENCES_ARE_NOT_BARRIERS: for the thread sanitizer's test of itself, which has to
+// report the race that this barrier prevents)
+inline void hip_threads_fence(int, const char *scope, const char *) {
+  std::atomic_thread_fence(std::memory_order_seq_cst);
+#ifndef HIP_THREADS_FENCES_ARE_NOT_BARRIERS
+  if (strcmp(scope, "wavefront") == 0) __builtin_amdgcn_wave_barrier();
+#else
+  (void)scope;
+#endif
+}
 inline int __any(int predicate) {
   int r = predicate != 0;
   for (int off = 32; off > 0; off >>= 1) r |= __shfl_xor(r, off);

@@ -1,4 +1,4 @@
-"""The library's HIP kernels compiled for the host (tests only): every kernel file but mi_fast.hip.
+"""The library's HIP kernels compiled for the host (tests only): every kernel file.
 
 g++ compiles the SAME sources as the GPU library over the thread stand-in of
 tests/cpu_build/hip/hip_runtime.h into one shared library, whose C-ABI entry points then take
@@ -6,12 +6,17 @@ numpy buffers (or CPU tensors, through the product's own Python layer).  Most fi
 but plain HIP (LDS, barriers, wavefront shuffles, atomics); rnnt_simple.hip and joiner.hip besides
 that the two matrix instructions (fp32 and bfloat16 operands), which the stand-in computes from
 their documented operand layouts, mi_wave.hip two DPP lane shifts, readlane and agent-scope
-atomics.  joiner.hip is compiled from a copy in which three lines that the host compiler cannot
-parse are replaced (JOINER_EDITS below, nothing else).  The ctypes signatures are k2_amd/capi.py's
-own table, so a wrong entry there shows up here as well.  mi_fast.hip (inline assembly
-throughout) is not part of it; mi_capi.hip (the MI entry points' argument checks and kernel
-selection) is, with launchers for mi_fast's kernels that say "not served"
-(tests/cpu_build/entry.cc), so MI calls take the exact or the fp64 pipelined kernels.
+atomics.  Two files are compiled from copies in which the lines that the host compiler cannot
+parse are replaced, and not a character else (EDITS below): joiner.hip (three spellings) and
+mi_fast.hip, the pipelined mutual-information kernels and the single launch, whose inline assembly
+(two DPP arithmetic instructions, buffer loads, coherent loads and stores, wait counts) gives way
+to calls that do what the instructions do.  The ctypes signatures are k2_amd/capi.py's own table,
+so a wrong entry there shows up here as well.
+
+What the host build cannot show: anything that depends on workgroups running at the same time
+(they run one after the other here, which the kernels allow: every wait of theirs is for a
+workgroup that started earlier), the memory model of the device (coherence between compute units,
+wait counts), and timing.
 
 Fenced arrays: a numpy array whose last byte sits directly in front of an inaccessible page (or
 whose first byte directly behind one), so that a kernel reading or writing past the end of a
@@ -20,6 +25,7 @@ tensor stops the test run with a segmentation fault instead of passing unnoticed
 import ctypes
 import mmap
 import os
+import re
 import subprocess
 
 import numpy as np
@@ -37,22 +43,69 @@ FLAGS = ["-std=c++20", "-O1", "-g", "-fPIC", "-pthread", "-ffp-contract=off", f"
 _lib = None
 
 
-# joiner.hip spells three things the host compiler cannot parse; the host build compiles a copy in
-# which exactly these lines are replaced (each must be found the stated number of times), and not
-# a character else.
-JOINER_EDITS = [
-    ("typedef __bf16 Bf8 __attribute__((ext_vector_type(8)));", "typedef hip_threads_bf16x8 Bf8;", 1),
-    ("return __builtin_bit_cast(unsigned short, static_cast<__bf16>(f));", "return hip_threads_to_bf16(f);", 1),
-    ("extern __shared__ __attribute__((aligned(16))) unsigned char smem[];", "HIP_DYNAMIC_SHARED(unsigned char, smem)", None),
-]
+# Two sources hold lines that the host compiler cannot parse; the host build compiles copies in
+# which exactly these are replaced and not a character else.  (old, new, count): a literal that
+# must be found `count` times (None: at least once); a compiled pattern replaces every match.
+EDITS = {
+    "joiner": [
+        ("typedef __bf16 Bf8 __attribute__((ext_vector_type(8)));", "typedef hip_threads_bf16x8 Bf8;", 1),
+        ("return __builtin_bit_cast(unsigned short, static_cast<__bf16>(f));", "return hip_threads_to_bf16(f);", 1),
+        ("extern __shared__ __attribute__((aligned(16))) unsigned char smem[];", "HIP_DYNAMIC_SHARED(unsigned char, smem)", None),
+    ],
+    "mi_fast": [
+        # the first half of a forward chain step (twice: natural and base-2 logarithms)
+        ("""  asm volatile(
+      "v_add_f32 %[x], %[P], %[fy]\\n\\t"
+      "s_nop 0\\n\\t"
+      "v_add_f32_dpp %[inc], %[P], %[inc] wave_shr:1 row_mask:0xf bank_mask:0xf\\n\\t"
+      "v_max_f32 %[mx], %[inc], %[x]\\n\\t"
+      "v_sub_f32 %[d], %[inc], %[x]"
+      : [x] "=&v"(x), [inc] "+&v"(inc), [mx] "=&v"(mx), [d] "=&v"(d)
+      : [P] "v"(P), [fy] "v"(fy));
+""", """  x = P + fy;
+  inc = hip_threads_add_from_lane_above(P, inc);
+  mx = fmaxf(inc, x);
+  d = inc - x;
+""", 2),
+        # a backward chain step
+        ("""        asm volatile(
+            "s_nop 1\\n\\t"
+            "v_mul_f32_dpp %[t], %[G], %[t] wave_shl:1 row_mask:0xf bank_mask:0xf\\n\\t"
+            "v_fmac_f32 %[t], %[O], %[G]"
+            : [t] "+&v"(ts[e])
+            : [O] "v"(os[e]), [G] "v"(G));
+""", """        ts[e] = __builtin_fmaf(os[e], G, hip_threads_mul_from_lane_below(G, ts[e]));
+""", 1),
+        ('asm volatile("buffer_load_dwordx4 %0, %1, %2, 0 offen" : "=v"(v) : "v"(off), "s"(rs) : "memory");',
+         "v = hip_threads_buffer_load4(rs, off);", 1),
+        ('asm volatile("buffer_load_dwordx4 %0, %1, %2, 0 offen sc1" : "=v"(v) : "v"(off), "s"(rs) : "memory");',
+         "v = hip_threads_buffer_load4(rs, off);", 1),
+        ('asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(ptr), "v"(w) : "memory");', "memcpy(ptr, &w, 16);", 1),
+        ('asm volatile("global_load_dword %0, %1, off" : "=v"(gauge_v) : "v"(src) : "memory");', "gauge_v = *src;", 1),
+        # waits for loads, and empty statements that only pin registers or keep branches apart
+        (re.compile(r'asm volatile\("s_waitcnt[^;]*;'), ";", 4),
+        (re.compile(r'asm volatile\(""[^;]*;'), ";", 10),
+        # vector types whose elements the kernels name .x to .w
+        ("typedef int int4v __attribute__((ext_vector_type(4)));", "typedef hip_threads_int4 int4v;", 1),
+        ("typedef float float4v __attribute__((ext_vector_type(4)));", "typedef hip_threads_float4 float4v;", 1),
+        ("typedef float QuadU __attribute__((ext_vector_type(4), aligned(4)));", "typedef hip_threads_float4 QuadU;", 1),
+        # without address spaces this overload is the one in front of it
+        ("__device__ __forceinline__ void StoreQuad(float *ptr, float4 v) { StoreQuad(Global(ptr), v); }\n", "", 1),
+    ],
+}
 
 
-def _joiner_source():
-    text = open(os.path.join(CSRC, "joiner.hip")).read()
-    for old, new, count in JOINER_EDITS:
-        assert text.count(old) >= 1 and (count is None or text.count(old) == count), old
-        text = text.replace(old, new)
-    path = os.path.join(OUT, "joiner_host.hip")
+def _edited_source(name):
+    text = open(os.path.join(CSRC, name + ".hip")).read()
+    for old, new, count in EDITS[name]:
+        if isinstance(old, str):
+            found = text.count(old)
+            text = text.replace(old, new)
+        else:
+            text, found = old.subn(new, text)
+        assert found >= 1 and (count is None or found == count), (name, old, found)
+    assert "asm" not in re.sub(r"//[^\n]*", "", text).replace("assembly", ""), name
+    path = os.path.join(OUT, name + "_host.hip")
     with open(path, "w") as f:
         f.write(text)
     return path
@@ -62,10 +115,10 @@ def build():
     """Compiles the portable sources and tests/cpu_build/entry.cc into _build/libk2amd_cpu.so."""
     os.makedirs(OUT, exist_ok=True)
     jobs = []
-    for name in PORTABLE + ["joiner", "entry"]:
+    for name in PORTABLE + list(EDITS) + ["entry"]:
         src = os.path.join(CSRC, name + ".hip") if name != "entry" else os.path.join(SHIM, "entry.cc")
-        if name == "joiner":
-            src = _joiner_source()
+        if name in EDITS:
+            src = _edited_source(name)
         obj = os.path.join(OUT, name + ".o")
         jobs.append((src, obj, subprocess.Popen(["g++", *FLAGS, "-x", "c++", "-c", src, "-o", obj],
                                                 stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))

@@ -1,8 +1,9 @@
 """bench.py's control flow on toy sizes and CPU tensors, over the host build of the kernels: every
 section runs, the one JSON line comes out with the fields the contract names, the median of the
-repeated timed region is what it says, a section that cannot run (the fused joiner: its kernels
-are not in the host build) is reported in its field without taking the line with it.  Figures are
-meaningless here; the point is that a mistake in the script shows before a GPU is spent on it."""
+repeated timed region is what it says, a section that fails (the fused joiner's, made to: at
+D = 512 it takes minutes on threads, and it ran through once this way while this was written) is
+reported in its field without taking the line with it.  Figures are meaningless here; the point
+is that a mistake in the script shows before a GPU is spent on it."""
 import contextlib
 import io
 import json
@@ -60,6 +61,10 @@ def test_every_section_runs_and_the_line_is_whole(monkeypatch):
                                            "c5": dict(B=2, T=9, S=4, C=7, t_lo=7, s_lo=2),
                                            "c4": dict(B=2, S=5, T=12)})
     monkeypatch.setattr(bench, "SECONDARY_STEPS", {k: 2 for k in bench.SECONDARY_STEPS})
+
+    def failing_section(dev, steps=None):
+        raise RuntimeError("made to fail")
+    monkeypatch.setattr(bench, "fused_joiner", failing_section)
     monkeypatch.setattr(sys, "argv", ["bench.py", "--device", "cpu", "--B", "2", "--S", "5", "--T", "12", "--steps", "3",
                                       "--warmup", "1", "--input-sets", "2"])
     out = io.StringIO()
@@ -85,7 +90,7 @@ def test_every_section_runs_and_the_line_is_whole(monkeypatch):
     assert "roofline" in line["other_configs"]["c5_rnnt_loss"]
     assert set(line["next_rows"]) == {"pruned_ranges_to_lattice", "hat_pruned_loss", "smoothed_loss",
                                       "joint_mutual_information_recursion"}
-    assert "error" in line["fused_joiner"]  # its kernels need the hardware; the line stands all the same
+    assert "made to fail" in line["fused_joiner"]["error"]  # the line stands all the same
 
 
 def test_more_than_one_gpu_is_declined(monkeypatch, capsys):

@@ -1,10 +1,11 @@
-"""The portable HIP kernels of the library, compiled for the host (tests/cpu_kernels.py) and run
-through their C-ABI on numpy buffers that end at an inaccessible page: the same parity checks as
-the GPU tests make, without a GPU, plus the certainty that no kernel reads or writes past the
-end of a tensor at these shapes (that would end the run with a segmentation fault).
+"""The library's HIP kernels, compiled for the host (tests/cpu_kernels.py) and run through their
+C-ABI on numpy buffers that end at an inaccessible page: the same parity checks as the GPU tests
+make, without a GPU, plus the certainty that no kernel reads or writes past the end of a tensor at
+these shapes (that would end the run with a segmentation fault).  (The pipelined fp32
+mutual-information kernels and the single launch: tests/test_cpu_build_pipelined.py.)
 
 This is a second line behind the GPU tests, not a replacement: the host compiler is not hipcc,
-every work-item is a thread here, and the kernels that need the hardware are not covered."""
+every work-item is a thread here and the workgroups of a launch run one after the other."""
 import ctypes
 import os
 
