@@ -11,7 +11,8 @@
 //   program rounds repeats window seed
 //
 // Random small shapes (one to three chunks, one to four blocks, boxes, both lattice types), the
-// pair of launches with the log-derivative tensor and the single launch.
+// pair of launches with the log-derivative tensor, the single launch, and the fp64 pair
+// (k2_amd/csrc/mi_wave.hip: one wavefront per chunk, the same hand-over between chunks).
 #include <sys/mman.h>
 
 #include <algorithm>
@@ -40,22 +41,64 @@ struct Outputs {
   float *p, *log_deriv, *ans, *seed, *px_grad, *py_grad;
 };
 
-bool SameBits(const char *what, const float *a, const float *b, size_t n) {
-  if (memcmp(a, b, n * sizeof(float)) == 0) return true;
-  for (size_t i = 0; i < n; ++i)
-    if (memcmp(a + i, b + i, 4) != 0) {
-      printf("%s differs at %zu: %.9g against %.9g\n", what, i, a[i], b[i]);
-      break;
-    }
-  return false;
-}
-
 bool Clean(const unsigned *ws, size_t words) {
   for (size_t i = 0; i < 3; ++i)
     if (ws[i] != 0) return false;
   for (size_t i = 64; i < words; ++i)
     if (ws[i] != 0x7fc5a5a5u) return false;
   return true;
+}
+
+template <typename T>
+bool SameBits(const char *what, const T *a, const T *b, size_t n) {
+  if (memcmp(a, b, n * sizeof(T)) == 0) return true;
+  for (size_t i = 0; i < n; ++i)
+    if (memcmp(a + i, b + i, sizeof(T)) != 0) {
+      printf("%s differs at %zu: %.17g against %.17g\n", what, i, (double)a[i], (double)b[i]);
+      break;
+    }
+  return false;
+}
+
+// the fp64 pair, in order and `repeats` times overlapping
+bool DoublePair(const float *px32, const float *py32, const int64_t *boundary, int B, int S, int T, int modified,
+                size_t nx, size_t ny, size_t np, int repeats, int window) {
+  const size_t ws_bytes = k2amd_mi_workspace_bytes(B, S, T, modified, K2AMD_F64);
+  if (ws_bytes == 0) return true;  // (not served: the exact kernels have no hand-over)
+  double *px = Shared<double>(nx), *py = Shared<double>(ny);
+  for (size_t i = 0; i < nx; ++i) px[i] = px32[i];
+  for (size_t i = 0; i < ny; ++i) py[i] = py32[i];
+  unsigned *ws = Shared<unsigned>(ws_bytes / 4);
+  bool ok = k2amd_mi_workspace_init(ws, ws_bytes, nullptr) == K2AMD_OK;
+  double *p[2], *ans[2], *seed[2], *gx[2], *gy[2];
+  for (int i = 0; i < 2; ++i) {
+    p[i] = Shared<double>(np); ans[i] = Shared<double>(B); seed[i] = Shared<double>(B);
+    gx[i] = Shared<double>(nx); gy[i] = Shared<double>(ny);
+  }
+  for (int run = 0; ok && run <= repeats; ++run) {
+    const int o = run == 0 ? 0 : 1;
+    hip_threads::concurrent_workgroups = run == 0 ? 0 : window;
+    memset(p[o], 0, np * 8); memset(gx[o], 0, nx * 8); memset(gy[o], 0, ny * 8);
+    for (int b = 0; b < B; ++b) { ans[o][b] = 0.0; seed[o][b] = 0.5 + 0.25 * b; }
+    int status = k2amd_mi_forward(px, py, boundary, p[o], ans[o], B, S, T, modified, K2AMD_F64, ws, ws_bytes, nullptr);
+    if (status == K2AMD_OK)
+      status = k2amd_mi_backward(px, py, boundary, p[o], seed[o], gx[o], gy[o], B, S, T, modified, K2AMD_F64, 1, ws,
+                                 ws_bytes, nullptr);
+    hip_threads::concurrent_workgroups = 0;
+    if (status == K2AMD_OK) status = k2amd_mi_workspace_status(ws, nullptr);
+    ok = status == K2AMD_OK && Clean(ws, ws_bytes / 4);
+    if (!ok) printf("fp64 pair run %d: status %d or workspace not clean\n", run, status);
+    if (ok && run > 0) {
+      ok = SameBits("ans", ans[0], ans[1], B) && SameBits("ans_grad", seed[0], seed[1], B) && SameBits("p", p[0], p[1], np) &&
+           SameBits("px_grad", gx[0], gx[1], nx) && SameBits("py_grad", gy[0], gy[1], ny);
+      if (!ok) printf("fp64 pair run %d: not the bits of the run in order\n", run);
+    }
+  }
+  for (int i = 0; i < 2; ++i) {
+    Release(p[i], np); Release(ans[i], B); Release(seed[i], B); Release(gx[i], nx); Release(gy[i], ny);
+  }
+  Release(ws, ws_bytes / 4); Release(px, nx); Release(py, ny);
+  return ok;
 }
 
 }  // namespace
@@ -122,6 +165,7 @@ int main(int argc, char **argv) {
         if (!same) { printf("route %d run %d: not the bits of the run in order\n", route, run); return 1; }
       }
     }
+    if (!DoublePair(px, py, boundary, B, S, T, modified, nx, ny, np, repeats, window)) return 1;
     for (Outputs &o : out) {
       Release(o.p, np); Release(o.log_deriv, np); Release(o.ans, B); Release(o.seed, B); Release(o.px_grad, nx); Release(o.py_grad, ny);
     }

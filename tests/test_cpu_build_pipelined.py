@@ -481,7 +481,8 @@ def test_overlapping_workgroups_give_the_bits_of_workgroups_in_order():
     counters in shared memory.  What a launch computes does not depend on how its workgroups
     interleave, so every output has to have the bits of the run with the workgroups in order; the
     workspace has to be clean and no wait expired.  Random shapes of one to three chunks, the pair
-    with the log-derivative tensor and the single launch, three overlapping runs each.
+    with the log-derivative tensor, the single launch and the fp64 pair (mi_wave.hip), three
+    overlapping runs each.
 
     That the workgroups do overlap is shown by a control: the same program over a copy of the
     kernels in which the take of a word between chunks does not wait for it.  In order that is
