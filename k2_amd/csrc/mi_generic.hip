@@ -5,6 +5,15 @@
 // term for term, so these kernels are the exact-semantics path: every dtype, every size, every
 // -inf / NaN corner.
 // They are latency-bound by design; the throughput path for fp32 lives in mi_fast.hip.
+//
+// The sweep keeps the previous step's values in two LDS rows of S + 2 elements.  A sequence with
+// more rows than 64 KiB of LDS hold (S > 8190 in fp32, 4094 in fp64) is swept by the same
+// kernels without those rows (kRowsInLds = false): the previous step is read back from what the
+// workgroup itself stored in p, px_grad and py_grad, with the same bits as a result.
+// K2AMD_MI_GENERIC_ROWS=global selects that form for every shape (tests and comparisons).
+#include <cstdlib>
+#include <cstring>
+
 #include "common.h"
 #include "mi_generic_impl.h"
 #include "mi_internal.h"
@@ -14,31 +23,34 @@ namespace {
 
 constexpr int kThreads = 256;
 
-template <typename T>
+template <typename T, bool kRowsInLds>
 __global__ __launch_bounds__(kThreads) void MiForwardGenericKernel(
     const T *__restrict__ px, const T *__restrict__ py, const int64_t *__restrict__ boundary,
     T *__restrict__ p, T *__restrict__ ans, int S, int Tn, int modified) {
   HIP_DYNAMIC_SHARED(unsigned char, smem_raw)
-  T *prev = reinterpret_cast<T *>(smem_raw);
-  T *cur = prev + (S + 2);
   const int b = blockIdx.x;
   const Box box = LoadBox(boundary, b, S, Tn);
   if (!box.ok) {
     if (threadIdx.x == 0) ans[b] = std::numeric_limits<T>::quiet_NaN();
     return;
   }
-  const T end = MiForwardGenericSeq<T>(px, py, box, p, b, S, Tn, modified, Tn + 1, prev, cur);
+  T end;
+  if (kRowsInLds) {
+    T *prev = reinterpret_cast<T *>(smem_raw);
+    T *cur = prev + (S + 2);
+    end = MiForwardGenericSeq<T>(px, py, box, p, b, S, Tn, modified, Tn + 1, prev, cur);
+  } else {
+    end = MiForwardRowsFromP<T>(px, py, box, p, b, S, Tn, modified, Tn + 1);
+  }
   if (threadIdx.x == 0) ans[b] = end;
 }
 
-template <typename T>
+template <typename T, bool kRowsInLds>
 __global__ __launch_bounds__(kThreads) void MiBackwardGenericKernel(
     const T *__restrict__ px, const T *__restrict__ p, const int64_t *__restrict__ boundary,
     T *__restrict__ ans_grad, T *__restrict__ px_grad, T *__restrict__ py_grad, int S, int Tn,
     int modified, int overwrite_ans_grad) {
   HIP_DYNAMIC_SHARED(unsigned char, smem_raw)
-  T *gprev = reinterpret_cast<T *>(smem_raw);
-  T *gcur = gprev + (S + 2);
   const int b = blockIdx.x;
   const Box box = LoadBox(boundary, b, S, Tn);
   const int T1 = modified ? Tn : Tn + 1;
@@ -64,26 +76,40 @@ __global__ __launch_bounds__(kThreads) void MiBackwardGenericKernel(
     }
   }
   if (!box.ok) return;
-  const T at_origin = MiBackwardGenericSeq<T>(px, p, box, ans_grad[b], px_grad, py_grad, b, S, Tn,
-                                              modified, Tn + 1, gprev, gcur);
+  T at_origin;
+  if (kRowsInLds) {
+    T *gprev = reinterpret_cast<T *>(smem_raw);
+    T *gcur = gprev + (S + 2);
+    at_origin = MiBackwardGenericSeq<T>(px, p, box, ans_grad[b], px_grad, py_grad, b, S, Tn,
+                                        modified, Tn + 1, gprev, gcur);
+  } else {
+    at_origin = MiBackwardRowsFromGrads<T>(px, p, box, ans_grad[b], px_grad, py_grad, b, S, Tn,
+                                           modified, Tn + 1);
+  }
   if (overwrite_ans_grad && threadIdx.x == 0) ans_grad[b] = at_origin;
 }
 
-}  // namespace
+constexpr size_t kLdsRowsLimit = 64 * 1024;
 
-size_t MiGenericMaxRows(int dtype) {
-  // two rotating LDS rows of S+2 values must fit the 64 KiB a workgroup may ask for
-  const size_t elem = dtype == K2AMD_F64 ? 8 : 4;
-  return (64 * 1024) / (2 * elem) - 2;
+// Whether a sequence's two rows go to LDS: they have to fit, and the switch must not say otherwise.
+bool RowsInLds(size_t smem) {
+  if (smem > kLdsRowsLimit) return false;
+  const char *e = std::getenv("K2AMD_MI_GENERIC_ROWS");
+  return !(e != nullptr && std::strcmp(e, "global") == 0);
 }
+
+}  // namespace
 
 template <typename T>
 int MiForwardGeneric(const T *px, const T *py, const int64_t *boundary, T *p, T *ans, int B,
                      int S, int Tn, int modified, hipStream_t stream) {
   const size_t smem = 2 * (size_t)(S + 2) * sizeof(T);
-  if (smem > 64 * 1024) return K2AMD_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL(MiForwardGenericKernel<T>, dim3(B), dim3(kThreads), smem, stream, px, py,
-                     boundary, p, ans, S, Tn, modified);
+  if (RowsInLds(smem))
+    hipLaunchKernelGGL((MiForwardGenericKernel<T, true>), dim3(B), dim3(kThreads), smem, stream, px,
+                       py, boundary, p, ans, S, Tn, modified);
+  else
+    hipLaunchKernelGGL((MiForwardGenericKernel<T, false>), dim3(B), dim3(kThreads), 0, stream, px,
+                       py, boundary, p, ans, S, Tn, modified);
   return LaunchStatus();
 }
 
@@ -92,9 +118,12 @@ int MiBackwardGeneric(const T *px, const T *p, const int64_t *boundary, T *ans_g
                       T *py_grad, int B, int S, int Tn, int modified, int overwrite_ans_grad,
                       hipStream_t stream) {
   const size_t smem = 2 * (size_t)(S + 2) * sizeof(T);
-  if (smem > 64 * 1024) return K2AMD_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL(MiBackwardGenericKernel<T>, dim3(B), dim3(kThreads), smem, stream, px, p,
-                     boundary, ans_grad, px_grad, py_grad, S, Tn, modified, overwrite_ans_grad);
+  if (RowsInLds(smem))
+    hipLaunchKernelGGL((MiBackwardGenericKernel<T, true>), dim3(B), dim3(kThreads), smem, stream, px,
+                       p, boundary, ans_grad, px_grad, py_grad, S, Tn, modified, overwrite_ans_grad);
+  else
+    hipLaunchKernelGGL((MiBackwardGenericKernel<T, false>), dim3(B), dim3(kThreads), 0, stream, px,
+                       p, boundary, ans_grad, px_grad, py_grad, S, Tn, modified, overwrite_ans_grad);
   return LaunchStatus();
 }
 

@@ -16,7 +16,6 @@ template <typename T>
 int MiBackwardGeneric(const T *px, const T *p, const int64_t *boundary, T *ans_grad, T *px_grad,
                       T *py_grad, int B, int S, int Tn, int modified, int overwrite_ans_grad,
                       hipStream_t stream);
-size_t MiGenericMaxRows(int dtype);
 
 // fp32 throughput path: pipelined 63-row chunks, one chain wavefront per workgroup (mi_fast.hip).
 bool MiFastSupports(int B, int S, int Tn, int modified);

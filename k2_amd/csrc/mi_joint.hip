@@ -40,7 +40,7 @@ __global__ __launch_bounds__(256) void JointPartialKernel(JointInputs in, const 
                                                           T *__restrict__ partial, int B,
                                                           long long kx, long long ky) {
   __shared__ T sums[4];
-  const int chunk = blockIdx.x, b = blockIdx.y, n = blockIdx.z;
+  const int b = blockIdx.x / kJointChunks, chunk = blockIdx.x - b * kJointChunks, n = blockIdx.y;
   const long long lx = (kx + kJointChunks - 1) / kJointChunks, ly = (ky + kJointChunks - 1) / kJointChunks;
   const long long x0 = min((long long)chunk * lx, kx), x1 = min(x0 + lx, kx);
   const long long y0 = min((long long)chunk * ly, ky), y1 = min(y0 + ly, ky);
@@ -66,7 +66,7 @@ __global__ void JointFinishKernel(const T *__restrict__ partial, T *__restrict__
 template <typename T>
 int JointProducts(const JointInputs &in, int N, const T *px_grad, const T *py_grad, T *prods,
                   T *partial, int B, long long kx, long long ky, hipStream_t st) {
-  hipLaunchKernelGGL(JointPartialKernel<T>, dim3(kJointChunks, B, N), dim3(256), 0, st, in, px_grad,
+  hipLaunchKernelGGL(JointPartialKernel<T>, dim3((unsigned)B * kJointChunks, N), dim3(256), 0, st, in, px_grad,
                      py_grad, partial, B, kx, ky);
   hipLaunchKernelGGL(JointFinishKernel<T>, dim3((N * B + 255) / 256), dim3(256), 0, st, partial, prods, N * B);
   return LaunchStatus();
@@ -88,7 +88,7 @@ int k2amd_mi_joint_products(const void *const *px, const void *const *py, int N,
                             long long ky, int dtype, void *stream) {
   if (N < 1 || B < 0 || kx < 0 || ky < 0 || px == nullptr || py == nullptr) return K2AMD_ERR_INVALID_ARGUMENT;
   if (dtype != K2AMD_F32 && dtype != K2AMD_F64) return K2AMD_ERR_INVALID_ARGUMENT;
-  if (N > kJointMax || B > 65535) return K2AMD_ERR_UNSUPPORTED;
+  if (N > kJointMax || (long long)N * B >= (1ll << 31) / kJointChunks) return K2AMD_ERR_UNSUPPORTED;
   if (B == 0) return K2AMD_OK;
   JointInputs in{};
   for (int n = 0; n < N; ++n) {

@@ -1,6 +1,9 @@
 // Pruning side of the RNN-T path: the integer prune ranges and the lm gather / scatter.
 //   get_rnnt_prune_ranges  k2/python/k2/rnnt_loss.py:636-780
 //   do_rnnt_pruning        k2/python/k2/rnnt_loss.py:913-954
+#include <cstdlib>
+#include <cstring>
+
 #include "common.h"
 
 namespace k2amd {
@@ -8,17 +11,19 @@ namespace {
 
 constexpr int kPruneThreads = 256;
 
-// Reverse running minimum of n ints held in LDS (Hillis-Steele on two rotating buffers).
-// Returns the buffer that holds the result.  Every thread of the workgroup must call it.
-__device__ int *SuffixMin(int *a, int *b, int n) {
+// Reverse running minimum of n ints (Hillis-Steele on two rotating buffers whose elements lie
+// `stride` ints apart: LDS, or global memory that only this workgroup touches).  Returns the
+// buffer that holds the result.  Every thread of the workgroup must call it.
+typedef int __attribute__((may_alias)) ScanInt;  // the global buffers are halves of 64-bit words
+__device__ ScanInt *SuffixMin(ScanInt *a, ScanInt *b, int n, size_t stride) {
   for (int off = 1; off < n; off <<= 1) {
     for (int t = threadIdx.x; t < n; t += kPruneThreads) {
-      int v = a[t];
-      if (t + off < n) v = min(v, a[t + off]);
-      b[t] = v;
+      int v = a[t * stride];
+      if (t + off < n) v = min(v, a[(size_t)(t + off) * stride]);
+      b[t * stride] = v;
     }
     __syncthreads();
-    int *tmp = a; a = b; b = tmp;
+    ScanInt *tmp = a; a = b; b = tmp;
   }
   return a;
 }
@@ -40,13 +45,13 @@ constexpr int kArgSplit = 4;
 template <typename T, int kR>
 __global__ __launch_bounds__(kArgFrames * kArgSplit) void PruneArgmaxKernel(
     const T *__restrict__ px_grad, const T *__restrict__ py_grad, int64_t *__restrict__ ranges,
-    int S, int Tn, int modified, int R_any) {
+    int S, int Tn, int modified, int R_any, int frame_blocks) {
   __shared__ T best_v_s[kArgSplit][kArgFrames];
   __shared__ int best_w_s[kArgSplit][kArgFrames];
   const int R = kR > 0 ? kR : R_any;
-  const int b = blockIdx.y;
+  const int b = blockIdx.x / frame_blocks;
   const int tx = threadIdx.x % kArgFrames, grp = threadIdx.x / kArgFrames;
-  const int t = blockIdx.x * kArgFrames + tx;
+  const int t = (blockIdx.x - b * frame_blocks) * kArgFrames + tx;
   const int T1 = modified ? Tn : Tn + 1;
   const int S1 = S + 1;
   const int n_win = S1 - R + 1;
@@ -100,11 +105,13 @@ __global__ __launch_bounds__(kArgFrames * kArgSplit) void PruneArgmaxKernel(
 
 template <typename T>
 void LaunchArgmax(const T *px_grad, const T *py_grad, int64_t *ranges, int S, int Tn, int modified,
-                  int R, dim3 grid, hipStream_t st) {
-  const dim3 block(kArgFrames * kArgSplit);
+                  int R, int B, hipStream_t st) {
+  // one workgroup per (sequence, 64 frames), the sequence slowest
+  const int frame_blocks = (Tn + kArgFrames - 1) / kArgFrames;
+  const dim3 grid((unsigned)((size_t)B * frame_blocks)), block(kArgFrames * kArgSplit);
 #define K2AMD_ARGMAX(KR)                                                                         \
   hipLaunchKernelGGL((PruneArgmaxKernel<T, KR>), grid, block, 0, st, px_grad, py_grad, ranges, S, \
-                     Tn, modified, R)
+                     Tn, modified, R, frame_blocks)
   switch (R) {
     case 2: K2AMD_ARGMAX(2); break;
     case 3: K2AMD_ARGMAX(3); break;
@@ -120,27 +127,35 @@ void LaunchArgmax(const T *px_grad, const T *py_grad, int64_t *ranges, int S, in
 
 // Step 2: one workgroup per sequence.  Frames from t_end - 1 on are pinned to
 // max(s_end - R + 1, 0), then the two monotone passes of _adjust_pruning_lower_bound
-// (k2/python/k2/rnnt_loss.py:580-630, 749-766) run as log-step scans in LDS and the ranges are
-// written over the raw arg-max values.
+// (k2/python/k2/rnnt_loss.py:580-630, 749-766) run as log-step scans and the ranges are written
+// over the raw arg-max values.  The scans' two buffers of T ints lie in LDS (kInLds) or, for a T
+// whose buffers LDS does not hold, in the sequence's own part of `ranges`: frame t's two ints
+// are the halves of the 64-bit word ranges[b][t][0], which holds the raw arg-max until the first
+// loop has read it and the frame's final range only after the last loop has read both halves.
+template <bool kInLds>
 __global__ __launch_bounds__(kPruneThreads) void PruneFinishKernel(
-    const int64_t *__restrict__ boundary, int64_t *__restrict__ ranges, int Tn, int modified, int R) {
+    const int64_t *__restrict__ boundary, int64_t *ranges, int Tn, int modified, int R) {
   HIP_DYNAMIC_SHARED(int, lds)
-  int *buf0 = lds, *buf1 = lds + Tn;
   const int b = blockIdx.x;
+  const size_t stride = kInLds ? 1 : 2 * (size_t)R;
+  ScanInt *buf0 = kInLds ? lds : reinterpret_cast<ScanInt *>(ranges + (size_t)b * Tn * R);
+  ScanInt *buf1 = kInLds ? lds + Tn : buf0 + 1;
   const int64_t s_end = boundary[4 * b + 2], t_end = boundary[4 * b + 3];
   int64_t pad64 = s_end - R + 1;
   const int pad = pad64 < 0 ? 0 : (int)pad64;
-  for (int t = threadIdx.x; t < Tn; t += kPruneThreads)
-    buf0[t] = t < t_end - 1 ? (int)ranges[((size_t)b * Tn + t) * R] : pad;
+  for (int t = threadIdx.x; t < Tn; t += kPruneThreads) {
+    const int raw = (int)ranges[((size_t)b * Tn + t) * R];
+    buf0[t * stride] = t < t_end - 1 ? raw : pad;
+  }
   __syncthreads();
   const int ramp = (modified ? 2 : R) - 1;
-  int *cur = SuffixMin(buf0, buf1, Tn);
-  int *other = cur == buf0 ? buf1 : buf0;
-  for (int t = threadIdx.x; t < Tn; t += kPruneThreads) cur[t] = -(cur[t] - ramp * t);
+  ScanInt *cur = SuffixMin(buf0, buf1, Tn, stride);
+  ScanInt *other = cur == buf0 ? buf1 : buf0;
+  for (int t = threadIdx.x; t < Tn; t += kPruneThreads) cur[t * stride] = -(cur[t * stride] - ramp * t);
   __syncthreads();
-  cur = SuffixMin(cur, other, Tn);
+  cur = SuffixMin(cur, other, Tn, stride);
   for (int t = threadIdx.x; t < Tn; t += kPruneThreads) {
-    int v = cur[t];
+    int v = cur[t * stride];
     v = v < 0 ? 0 : v;
     const int64_t s_begin = -(int64_t)(v - ramp * t);
     int64_t *out = ranges + ((size_t)b * Tn + t) * R;
@@ -265,6 +280,15 @@ __global__ __launch_bounds__(kGatherThreads) void GatherBackwardKernel(
   }
 }
 
+constexpr size_t kFinishLdsLimit = 64 * 1024;
+
+// K2AMD_PRUNE_SCAN_ROWS=global: the finishing kernel's scans run in `ranges` itself at any T
+// (tests and comparisons; without it only where two rows of T ints exceed kFinishLdsLimit).
+bool FinishRowsInRanges() {
+  const char *e = std::getenv("K2AMD_PRUNE_SCAN_ROWS");
+  return e != nullptr && std::strcmp(e, "global") == 0;
+}
+
 unsigned GridFor(size_t n) {
   size_t blocks = (n + 255) / 256;
   return (unsigned)(blocks > 8192 ? 8192 : (blocks == 0 ? 1 : blocks));
@@ -285,15 +309,20 @@ int k2amd_rnnt_prune_ranges(const void *px_grad, const void *py_grad, const int6
     return K2AMD_ERR_INVALID_ARGUMENT;
   if (B == 0 || T == 0) return K2AMD_OK;
   const size_t smem = 2 * (size_t)T * sizeof(int);
-  if (smem > 64 * 1024 || (long long)S * T >= (1ll << 31) || B > 65535) return K2AMD_ERR_UNSUPPORTED;
+  // 32-bit element offsets inside a sequence, 32-bit workgroup counts
+  if ((long long)(S + 1) * ((long long)T + 1) >= (1ll << 31) ||
+      (long long)B * ((T + kArgFrames - 1) / kArgFrames) >= (1ll << 31))
+    return K2AMD_ERR_UNSUPPORTED;
   hipStream_t st = static_cast<hipStream_t>(stream);
   modified = modified ? 1 : 0;
-  const dim3 grid1((unsigned)((T + kArgFrames - 1) / kArgFrames), (unsigned)B);
   if (dtype == K2AMD_F32)
-    LaunchArgmax((const float *)px_grad, (const float *)py_grad, ranges, S, T, modified, s_range, grid1, st);
+    LaunchArgmax((const float *)px_grad, (const float *)py_grad, ranges, S, T, modified, s_range, B, st);
   else
-    LaunchArgmax((const double *)px_grad, (const double *)py_grad, ranges, S, T, modified, s_range, grid1, st);
-  hipLaunchKernelGGL(PruneFinishKernel, dim3(B), dim3(kPruneThreads), smem, st, boundary, ranges, T, modified, s_range);
+    LaunchArgmax((const double *)px_grad, (const double *)py_grad, ranges, S, T, modified, s_range, B, st);
+  if (smem <= kFinishLdsLimit && !FinishRowsInRanges())
+    hipLaunchKernelGGL(PruneFinishKernel<true>, dim3(B), dim3(kPruneThreads), smem, st, boundary, ranges, T, modified, s_range);
+  else
+    hipLaunchKernelGGL(PruneFinishKernel<false>, dim3(B), dim3(kPruneThreads), 0, st, boundary, ranges, T, modified, s_range);
   return LaunchStatus();
 }
 

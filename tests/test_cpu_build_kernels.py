@@ -80,6 +80,72 @@ def test_exact_mi_kernels_equal_the_cpu_loops_bit_for_bit(lib, dtype, modified):
             assert f.intact()
 
 
+def _exact_pair(lib, c, dtype, modified):
+    """p, ans, px_grad, py_grad of the exact kernels on fenced buffers."""
+    px, py, bd = c["px"], c["py"], c["boundary"]
+    B, S, T = c["B"], c["S"], c["T"]
+    fpx, fpy, fbd = fenced(px), fenced(py), fenced(bd)
+    pp, ans = Fenced((B, S + 1, T + 1), dtype, fill=np.nan), Fenced((B,), dtype, fill=np.nan)
+    assert lib.cpu_mi_forward_generic(p(fpx), p(fpy), p(fbd), p(pp), p(ans), B, S, T, int(modified),
+                                      dcode(dtype)) == 0
+    gx, gy = Fenced(px.shape, dtype, fill=np.nan), Fenced(py.shape, dtype, fill=np.nan)
+    ans_grad = Fenced((B,), dtype, fill=1.0)
+    assert lib.cpu_mi_backward_generic(p(fpx), p(pp), p(fbd), p(ans_grad), p(gx), p(gy), B, S, T,
+                                       int(modified), 1, dcode(dtype)) == 0
+    for f in (pp, ans, gx, gy, ans_grad):
+        assert f.intact()
+    return pp.a.copy(), ans.a.copy(), gx.a.copy(), gy.a.copy(), ans_grad.a.copy()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("modified", [False, True])
+def test_exact_mi_kernels_without_lds_rows_give_the_same_bits(lib, dtype, modified, monkeypatch):
+    """Sequences with more rows than LDS holds are swept with the previous step read back from p
+    and from px_grad / py_grad (mi_generic_impl.h); K2AMD_MI_GENERIC_ROWS=global selects that
+    form at any size.  Same bits as the CPU loops and as the form with the rows in LDS,
+    -inf entries and boundaries included."""
+    for seed in range(6):
+        c = cases.mi_case(900 + seed, dtype=dtype, max_B=3, max_S=40, max_T=70,
+                          force={"modified": modified, "rand_bd": seed % 3 != 0})
+        if seed % 2:
+            rng = np.random.default_rng(seed)
+            for name in ("px", "py"):
+                c[name][rng.random(c[name].shape) < 0.15] = -np.inf
+        monkeypatch.delenv("K2AMD_MI_GENERIC_ROWS", raising=False)
+        lds = _exact_pair(lib, c, dtype, modified)
+        monkeypatch.setenv("K2AMD_MI_GENERIC_ROWS", "global")
+        glob = _exact_pair(lib, c, dtype, modified)
+        want_ans, want_p = omi.mi_forward(c["px"], c["py"], c["boundary"])
+        want_gx, want_gy = omi.mi_backward(c["px"], c["py"], c["boundary"], want_p)
+        np.testing.assert_array_equal(glob[1], want_ans)
+        np.testing.assert_array_equal(glob[2], want_gx)
+        np.testing.assert_array_equal(glob[3], want_gy)
+        for a, b in zip(lds, glob):
+            np.testing.assert_array_equal(a.view(np.uint8), b.view(np.uint8))
+
+
+@pytest.mark.parametrize("dtype,S", [
+    (np.float32, 8200),
+    pytest.param(np.float64, 4100, marks=pytest.mark.skipif(
+        os.environ.get("K2AMD_SLOW_CPU_TESTS", "0") != "1", reason="slow on the host: run with K2AMD_SLOW_CPU_TESTS=1"))])
+def test_exact_mi_kernels_beyond_the_lds_rows(lib, dtype, S, monkeypatch):
+    """One sequence with more rows than two LDS rows of 64 KiB hold (S > 8190 in fp32, 4094 in
+    fp64): served, and with the bits of the CPU loops."""
+    monkeypatch.delenv("K2AMD_MI_GENERIC_ROWS", raising=False)
+    rng = np.random.default_rng(S)
+    B, T = 1, 2
+    c = {"B": B, "S": S, "T": T, "boundary": None,
+         "px": np.minimum(rng.normal(-2, 1, (B, S, T + 1)), 0).astype(dtype),
+         "py": np.minimum(rng.normal(-2, 1, (B, S + 1, T)), 0).astype(dtype)}
+    pp, ans, gx, gy, _ = _exact_pair(lib, c, dtype, False)
+    want_ans, want_p = omi.mi_forward(c["px"], c["py"], None)
+    want_gx, want_gy = omi.mi_backward(c["px"], c["py"], None, want_p)
+    np.testing.assert_array_equal(ans, want_ans)
+    np.testing.assert_array_equal(pp, want_p)
+    np.testing.assert_array_equal(gx, want_gx)
+    np.testing.assert_array_equal(gy, want_gy)
+
+
 # ---- the row kernels: get_rnnt_logprobs_joint / _pruned / HAT -----------------------------------
 
 def _random_ranges(rng, B, T, S, R):
@@ -198,6 +264,45 @@ def test_prune_ranges_bit_exact(lib, dtype, modified):
                                            int(modified), r_final, dcode(dtype), None) == 0
         np.testing.assert_array_equal(out.a, want)
         assert out.intact()
+
+
+@pytest.mark.parametrize("modified", [False, True])
+def test_prune_ranges_scans_inside_ranges_give_the_same_integers(lib, modified, monkeypatch):
+    """Where two rows of T ints exceed LDS the finishing kernel's scans run in the halves of
+    ranges[b][t][0] (prune.hip); K2AMD_PRUNE_SCAN_ROWS=global selects that at any T.  s_range = 1
+    is the case in which a frame owns nothing but that one word."""
+    monkeypatch.setenv("K2AMD_PRUNE_SCAN_ROWS", "global")
+    rt = "modified" if modified else "regular"
+    for k, (B, T, S, R) in enumerate(((2, 9, 5, 3), (1, 70, 20, 5), (3, 300, 33, 7), (2, 130, 4, 1), (1, 5, 1, 2), (2, 1, 1, 2))):
+        c = cases.rnnt_case(660 + k, B, T, S, 6, dtype=np.float32, t_lo=max(S, T - 3), s_lo=max(1, S - 2), modified=modified)
+        px, py = orn.logprobs_simple(c["lm"], c["am"], c["symbols"], 0, rt, c["boundary"])
+        _, gx, gy = omi.mi(px, py, c["boundary"])
+        want = orn.prune_ranges(gx, gy, c["boundary"], R)
+        keep = Inputs()
+        r_final = want.shape[2]
+        out = Fenced((B, T, r_final), np.int64, fill=-7)
+        assert lib.k2amd_rnnt_prune_ranges(keep(gx), keep(gy), keep(c["boundary"]), p(out), B, S, T,
+                                           int(modified), r_final, 0, None) == 0
+        np.testing.assert_array_equal(out.a, want)
+        assert out.intact()
+
+
+def test_prune_ranges_with_more_frames_than_lds_rows_hold(lib, monkeypatch):
+    """T = 8300 frames (two rows of T ints no longer fit 64 KiB): served, same integers as the
+    oracle.  Occupation counts drawn at random stand in for a recursion's gradients: the ranges
+    are a function of these two tensors and the boundary alone."""
+    monkeypatch.delenv("K2AMD_PRUNE_SCAN_ROWS", raising=False)
+    rng = np.random.default_rng(83)
+    B, T, S, R = 2, 8300, 6, 3
+    gx = rng.random((B, S, T + 1)).astype(np.float32)
+    gy = rng.random((B, S + 1, T)).astype(np.float32)
+    bd = np.array([[0, 0, S, T], [0, 0, S - 2, T - 11]], dtype=np.int64)
+    want = orn.prune_ranges(gx, gy, bd, R)
+    keep = Inputs()
+    out = Fenced((B, T, R), np.int64, fill=-7)
+    assert lib.k2amd_rnnt_prune_ranges(keep(gx), keep(gy), keep(bd), p(out), B, S, T, 0, R, 0, None) == 0
+    np.testing.assert_array_equal(out.a, want)
+    assert out.intact()
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
