@@ -319,6 +319,18 @@ K2AMD_API int k2amd_rnnt_prune_ranges(const void *px_grad, const void *py_grad,
                                       const int64_t *boundary, int64_t *ranges, int B, int S, int T,
                                       int modified, int s_range, int dtype, void *stream);
 
+/* Replaces the device work of get_rnnt_prune_ranges_deprecated (k2/python/k2/rnnt_loss.py:853-908):
+ * per frame the first arg-max over w of prefix[w + s_range] - prefix[w], where prefix[k] is the sum
+ * over rows i < k of px_grad[b,i,t] + py_grad[b,i,t] (px_grad's row S counts as 0), each prefix
+ * accumulated in double and rounded once to the input type (torch.cumsum on the CPU), the
+ * difference taken in the input type; then the padding and the running minima of
+ * k2amd_rnnt_prune_ranges.  s_range is the final value (min(s_range, S + 1), rnnt_loss.py:842-843).
+ * ranges [B][T][s_range] int64.                                                                  */
+K2AMD_API int k2amd_rnnt_prune_ranges_deprecated(const void *px_grad, const void *py_grad,
+                                                 const int64_t *boundary, int64_t *ranges, int B,
+                                                 int S, int T, int modified, int s_range, int dtype,
+                                                 void *stream);
+
 /* Replaces the gather of do_rnnt_pruning (k2/python/k2/rnnt_loss.py:947-953):
  * lm_pruned[b,t,k,:] = lm[b, ranges[b,t,k], :]; lm [B][S1][D].  Indices outside [0,S1) yield 0.  */
 K2AMD_API int k2amd_rnnt_prune_gather(const void *lm, const int64_t *ranges, void *lm_pruned, int B,

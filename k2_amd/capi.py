@@ -66,6 +66,7 @@ _SIGNATURES = {
     "k2amd_rnnt_joiner_hat_pruned_forward": ([_vp] * 10 + [_ci] * 8 + [_vp, _sz, _vp], _ci),
     "k2amd_rnnt_joiner_hat_pruned_backward": ([_vp] * 15 + [_ci] * 8 + [_vp, _sz, _vp], _ci),
     "k2amd_rnnt_prune_ranges": ([_vp] * 4 + [_ci] * 6 + [_vp], _ci),
+    "k2amd_rnnt_prune_ranges_deprecated": ([_vp] * 4 + [_ci] * 6 + [_vp], _ci),
     "k2amd_rnnt_prune_gather": ([_vp] * 3 + [_ci] * 6 + [_vp], _ci),
     "k2amd_rnnt_prune_gather_backward": ([_vp] * 3 + [_ci] * 6 + [_vp], _ci),
     "k2amd_lattice_count": ([_vp] * 6 + [_ci] * 3 + [_vp], _ci),
@@ -690,8 +691,9 @@ def joiner_pruned_backward(am, lm, ranges, weight, bias, symbols, termination_sy
     return am_grad, lm_grad, weight_grad, bias_grad
 
 
-def prune_ranges(px_grad, py_grad, boundary, s_range):
-    """``s_range`` is the final value (after the adjustments the Python layer applies)."""
+def prune_ranges(px_grad, py_grad, boundary, s_range, deprecated=False):
+    """``s_range`` is the final value (after the adjustments the Python layer applies);
+    ``deprecated``: the rule of get_rnnt_prune_ranges_deprecated instead."""
     dt, dev = _float_dtype(px_grad, "px_grad")
     B, S, T1 = _dims(px_grad, "px_grad", 3)
     T = _dims(py_grad, "py_grad", 3)[2]
@@ -704,9 +706,9 @@ def prune_ranges(px_grad, py_grad, boundary, s_range):
         raise RuntimeError(f"k2_amd: s_range {s_range} outside [1, S + 1 = {S + 1}]")
     ranges = torch.empty(B, T, s_range, dtype=torch.int64, device=px_grad.device)
     with torch.cuda.device(dev):
-        check(lib().k2amd_rnnt_prune_ranges(ptr(px_grad), ptr(py_grad), ptr(boundary), ptr(ranges),
-                                            B, S, T, int(T1 == T), s_range, dtype_code(px_grad),
-                                            stream_ptr(dev)))
+        entry = lib().k2amd_rnnt_prune_ranges_deprecated if deprecated else lib().k2amd_rnnt_prune_ranges
+        check(entry(ptr(px_grad), ptr(py_grad), ptr(boundary), ptr(ranges), B, S, T, int(T1 == T),
+                    s_range, dtype_code(px_grad), stream_ptr(dev)))
     return ranges
 
 

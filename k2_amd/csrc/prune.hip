@@ -1,5 +1,6 @@
 // Pruning side of the RNN-T path: the integer prune ranges and the lm gather / scatter.
-//   get_rnnt_prune_ranges  k2/python/k2/rnnt_loss.py:636-780
+//   get_rnnt_prune_ranges             k2/python/k2/rnnt_loss.py:636-780
+//   get_rnnt_prune_ranges_deprecated  k2/python/k2/rnnt_loss.py:786-910
 //   do_rnnt_pruning        k2/python/k2/rnnt_loss.py:913-954
 #include <cstdlib>
 #include <cstring>
@@ -123,6 +124,44 @@ void LaunchArgmax(const T *px_grad, const T *py_grad, int64_t *ranges, int S, in
     default: K2AMD_ARGMAX(0); break;
   }
 #undef K2AMD_ARGMAX
+}
+
+// Step 1 of get_rnnt_prune_ranges_deprecated (k2/python/k2/rnnt_loss.py:853-873): for every frame
+// the window of R rows with the largest total occupation
+//   prefix[w + R] - prefix[w],   prefix[k] = sum_{i<k} (px_grad[b,i,t] + py_grad[b,i,t])
+// with px_grad's row S counting as zero, first maximum over w = 0 .. S + 1 - R.  The occupation of a
+// cell is added in the input precision, as the reference's tensor addition does; a prefix is
+// accumulated in double and rounded to the input precision once, which is how torch.cumsum forms
+// it on the CPU; the difference of two prefixes is taken in the input precision again.  One
+// thread per frame (loads contiguous along t) keeps the leading and the trailing prefix as two
+// running sums, each the same function of the rows below it whoever computes it.
+template <typename T>
+__global__ __launch_bounds__(256) void PruneDeprecatedArgmaxKernel(
+    const T *__restrict__ px_grad, const T *__restrict__ py_grad, int64_t *__restrict__ ranges,
+    int S, int Tn, int modified, int R, int frame_blocks) {
+  const int b = blockIdx.x / frame_blocks;
+  const int t = (blockIdx.x - b * frame_blocks) * 256 + threadIdx.x;
+  if (t >= Tn) return;
+  const int T1 = modified ? Tn : Tn + 1;
+  const T *gx = px_grad + (size_t)b * S * T1;
+  const T *gy = py_grad + (size_t)b * (S + 1) * Tn;
+  auto occupation = [&](int s) -> T {
+    return (s < S ? gx[(size_t)s * T1 + t] : T(0)) + gy[(size_t)s * Tn + t];
+  };
+  double lead = 0, trail = 0;
+  for (int s = 0; s < R; ++s) lead += (double)occupation(s);
+  const int n_win = S + 2 - R;
+  T best_v = 0;
+  int best = -1;
+  for (int w = 0; w < n_win; ++w) {
+    const T v = (T)lead - (T)trail;
+    if (best < 0 || v > best_v) { best_v = v; best = w; }
+    if (w + 1 < n_win) {
+      lead += (double)occupation(w + R);
+      trail += (double)occupation(w);
+    }
+  }
+  ranges[((size_t)b * Tn + t) * R] = best < 0 ? 0 : best;
 }
 
 // Step 2: one workgroup per sequence.  Frames from t_end - 1 on are pinned to
@@ -319,6 +358,31 @@ int k2amd_rnnt_prune_ranges(const void *px_grad, const void *py_grad, const int6
     LaunchArgmax((const float *)px_grad, (const float *)py_grad, ranges, S, T, modified, s_range, B, st);
   else
     LaunchArgmax((const double *)px_grad, (const double *)py_grad, ranges, S, T, modified, s_range, B, st);
+  if (smem <= kFinishLdsLimit && !FinishRowsInRanges())
+    hipLaunchKernelGGL(PruneFinishKernel<true>, dim3(B), dim3(kPruneThreads), smem, st, boundary, ranges, T, modified, s_range);
+  else
+    hipLaunchKernelGGL(PruneFinishKernel<false>, dim3(B), dim3(kPruneThreads), 0, st, boundary, ranges, T, modified, s_range);
+  return LaunchStatus();
+}
+
+int k2amd_rnnt_prune_ranges_deprecated(const void *px_grad, const void *py_grad,
+                                       const int64_t *boundary, int64_t *ranges, int B, int S,
+                                       int T, int modified, int s_range, int dtype, void *stream) {
+  if (B < 0 || S < 0 || T < 0 || s_range < 1 || s_range > S + 1 || !boundary ||
+      (dtype != K2AMD_F32 && dtype != K2AMD_F64))
+    return K2AMD_ERR_INVALID_ARGUMENT;
+  if (B == 0 || T == 0) return K2AMD_OK;
+  const size_t smem = 2 * (size_t)T * sizeof(int);
+  const int frame_blocks = (T + 255) / 256;
+  if ((long long)(S + 1) * ((long long)T + 1) >= (1ll << 31) || (long long)B * frame_blocks >= (1ll << 31))
+    return K2AMD_ERR_UNSUPPORTED;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  modified = modified ? 1 : 0;
+  const dim3 grid((unsigned)((size_t)B * frame_blocks));
+  if (dtype == K2AMD_F32)
+    hipLaunchKernelGGL(PruneDeprecatedArgmaxKernel<float>, grid, dim3(256), 0, st, (const float *)px_grad, (const float *)py_grad, ranges, S, T, modified, s_range, frame_blocks);
+  else
+    hipLaunchKernelGGL(PruneDeprecatedArgmaxKernel<double>, grid, dim3(256), 0, st, (const double *)px_grad, (const double *)py_grad, ranges, S, T, modified, s_range, frame_blocks);
   if (smem <= kFinishLdsLimit && !FinishRowsInRanges())
     hipLaunchKernelGGL(PruneFinishKernel<true>, dim3(B), dim3(kPruneThreads), smem, st, boundary, ranges, T, modified, s_range);
   else

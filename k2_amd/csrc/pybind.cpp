@@ -653,9 +653,10 @@ torch::Tensor LogprobsPrunedBackward(torch::Tensor logits, torch::Tensor norm, t
   return grad;
 }
 
-// device part of get_rnnt_prune_ranges; s_range is the final value
+// device part of get_rnnt_prune_ranges (deprecated: of get_rnnt_prune_ranges_deprecated);
+// s_range is the final value
 torch::Tensor PruneRanges(torch::Tensor px_grad, torch::Tensor py_grad, torch::Tensor boundary,
-                          int s_range) {
+                          int s_range, bool deprecated) {
   ExpectFloat(px_grad, "px_grad", 3);
   ExpectFloat(py_grad, "py_grad", 3);
   const int B = px_grad.size(0), S = px_grad.size(1), T1 = px_grad.size(2), T = py_grad.size(2);
@@ -668,9 +669,9 @@ torch::Tensor PruneRanges(torch::Tensor px_grad, torch::Tensor py_grad, torch::T
   void *stream = StreamOf(px_grad);
   {
     pybind11::gil_scoped_release release;
-    Check(k2amd_rnnt_prune_ranges(px_grad.data_ptr(), py_grad.data_ptr(), I64(boundary),
-                                  ranges.data_ptr<int64_t>(), B, S, T, T1 == T ? 1 : 0, s_range,
-                                  DtypeCode(px_grad), stream));
+    auto entry = deprecated ? k2amd_rnnt_prune_ranges_deprecated : k2amd_rnnt_prune_ranges;
+    Check(entry(px_grad.data_ptr(), py_grad.data_ptr(), I64(boundary), ranges.data_ptr<int64_t>(),
+                B, S, T, T1 == T ? 1 : 0, s_range, DtypeCode(px_grad), stream));
   }
   return ranges;
 }
@@ -894,7 +895,8 @@ PYBIND11_MODULE(_k2_amd, m) {
   m.def("logprobs_joint_backward", &LogprobsJointBackward);
   m.def("logprobs_pruned_forward", &LogprobsPrunedForward);
   m.def("logprobs_pruned_backward", &LogprobsPrunedBackward);
-  m.def("prune_ranges", &PruneRanges);
+  m.def("prune_ranges", &PruneRanges, pybind11::arg("px_grad"), pybind11::arg("py_grad"),
+        pybind11::arg("boundary"), pybind11::arg("s_range"), pybind11::arg("deprecated") = false);
   m.def("prune_gather", &PruneGather);
   m.def("prune_gather_backward", &PruneGatherBackward);
   m.def("pruned_ranges_to_lattice", &PrunedRangesToLattice, pybind11::arg("ranges"),

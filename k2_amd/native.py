@@ -278,11 +278,11 @@ def joiner_pruned_backward(am, lm, ranges, weight, bias, symbols, termination_sy
                                        boundary, rnnt_type, norm, px_grad, py_grad, seq_scale, precision, hat)
 
 
-def prune_ranges(px_grad, py_grad, boundary, s_range):
+def prune_ranges(px_grad, py_grad, boundary, s_range, deprecated=False):
     _require_device(px_grad)
     if _ext is not None:
-        return _ext.prune_ranges(px_grad, py_grad, boundary, s_range)
-    return capi.prune_ranges(px_grad, py_grad, boundary, s_range)
+        return _ext.prune_ranges(px_grad, py_grad, boundary, s_range, deprecated)
+    return capi.prune_ranges(px_grad, py_grad, boundary, s_range, deprecated)
 
 
 def prune_gather(lm, ranges):

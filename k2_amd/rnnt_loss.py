@@ -697,7 +697,7 @@ def get_rnnt_prune_ranges_deprecated(
     """k2.get_rnnt_prune_ranges_deprecated (k2/python/k2/rnnt_loss.py:786-910): the older rule,
     which picks for every frame the window of s_range rows with the largest total occupation
     px_grad + py_grad (prefix sums over s), then applies the same padding and monotonicity
-    adjustment.  Kept for callers; torch ops on the device, not a fused kernel."""
+    adjustment.  Two launches, like get_rnnt_prune_ranges (csrc/prune.hip)."""
     (B, S, T1) = px_grad.shape
     T = py_grad.shape[-1]
     assert T1 in [T, T + 1], (T1, T)
@@ -714,17 +714,7 @@ def get_rnnt_prune_ranges_deprecated(
         assert s_range >= 2, \
             f"Pruning range for standard RNN-T should be equal to or greater than 2, " \
             f"or no valid paths could survive pruning. Given {s_range}"
-    dev = px_grad.device
-    boundary = boundary.to(dev)
-    pad = torch.nn.functional.pad
-    occupation = pad(px_grad, (0, 0, 0, 1)) + pad(py_grad, (0, T1 - T))   # [B][S+1][T1]
-    # torch's CPU cumsum, which the reference's values come from, accumulates fp32 input in double
-    # and rounds every prefix once; the device scan in fp32 would round along the way
-    prefix = torch.cumsum(pad(occupation, (0, 0, 1, 0)).double(), dim=1).to(occupation.dtype)  # [B][S+2][T1]
-    window = prefix[:, s_range:, :] - prefix[:, :-s_range, :]
-    s_begin = torch.argmax(window, dim=1)[:, :T]
-    live = torch.arange(T, device=dev).reshape(1, T) < boundary[:, 3].reshape(B, 1) - 1
-    parked = torch.clamp(boundary[:, 2].reshape(B, 1) - s_range + 1, min=0)
-    s_begin = torch.where(live, s_begin, parked)
-    s_begin = _adjust_pruning_lower_bound(s_begin, 2 if T1 == T else s_range)
-    return s_begin.reshape(B, T, 1) + torch.arange(s_range, device=dev)
+    # (the prefix sums over s are formed as torch.cumsum forms them on the CPU, where the
+    # reference's values come from: accumulated in double, every prefix rounded once)
+    return native.prune_ranges(px_grad.detach().contiguous(), py_grad.detach().contiguous(),
+                               _dev_i64(boundary, px_grad), int(s_range), deprecated=True)

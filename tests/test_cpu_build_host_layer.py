@@ -213,6 +213,11 @@ def _gpu_test(name):
     return getattr(test_rnnt_gpu, name)
 
 
+@pytest.mark.parametrize("modified", [False, True])
+def test_deprecated_prune_ranges_through_the_api(host_on_cpu, modified):
+    _gpu_test("test_deprecated_prune_ranges_matches_oracle")(torch.device("cpu"), modified)
+
+
 @pytest.mark.parametrize("name", ["test_reference_chain_fixtures",
                                   "test_reference_prune_ranges_on_ties_and_near_ties",
                                   "test_reference_logprobs_where_the_shifted_exponentials_underflow",

@@ -266,6 +266,42 @@ def test_prune_ranges_bit_exact(lib, dtype, modified):
         assert out.intact()
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("modified", [False, True])
+def test_deprecated_prune_ranges_bit_exact(lib, dtype, modified):
+    """k2amd_rnnt_prune_ranges_deprecated against the oracle's restatement of
+    get_rnnt_prune_ranges_deprecated (rnnt_loss.py:786-910), which the reference's recorded
+    ranges pin (tests/test_oracle_rnnt_fixtures.py): prefix sums accumulated in double and rounded
+    once, differences in the input type, first maximum."""
+    rt = "modified" if modified else "regular"
+    for k, (B, T, S, R) in enumerate(((2, 9, 5, 3), (1, 70, 20, 5), (3, 33, 33, 7), (2, 300, 4, 5), (1, 5, 1, 2),
+                                      (2, 40, 6, 7), (2, 12, 3, 1 if modified else 2))):
+        c = cases.rnnt_case(680 + k, B, T, S, 6, dtype=dtype, t_lo=max(S, T - 3), s_lo=max(1, S - 2), modified=modified)
+        px, py = orn.logprobs_simple(c["lm"], c["am"], c["symbols"], 0, rt, c["boundary"])
+        _, gx, gy = omi.mi(px, py, c["boundary"])
+        want = orn.prune_ranges_deprecated(gx, gy, c["boundary"], R)
+        keep = Inputs()
+        r_final = want.shape[2]
+        out = Fenced((B, T, r_final), np.int64, fill=-7)
+        assert lib.k2amd_rnnt_prune_ranges_deprecated(keep(gx), keep(gy), keep(c["boundary"]), p(out), B, S, T,
+                                                      int(modified), r_final, dcode(dtype), None) == 0
+        np.testing.assert_array_equal(out.a, want)
+        assert out.intact()
+    # sums that tie or differ in the last bits: rows of equal occupation
+    rng = np.random.default_rng(689)
+    B, T, S, R = 2, 50, 12, 3
+    T1 = T if modified else T + 1
+    gx = rng.integers(0, 3, (B, S, T1)).astype(dtype) * dtype(0.1)
+    gy = rng.integers(0, 3, (B, S + 1, T)).astype(dtype) * dtype(0.1)
+    bd = np.array([[0, 0, S, T], [0, 0, S - 1, T - 4]], dtype=np.int64)
+    want = orn.prune_ranges_deprecated(gx, gy, bd, R)
+    keep = Inputs()
+    out = Fenced((B, T, R), np.int64, fill=-7)
+    assert lib.k2amd_rnnt_prune_ranges_deprecated(keep(gx), keep(gy), keep(bd), p(out), B, S, T, int(modified),
+                                                  R, dcode(dtype), None) == 0
+    np.testing.assert_array_equal(out.a, want)
+
+
 @pytest.mark.parametrize("modified", [False, True])
 def test_prune_ranges_scans_inside_ranges_give_the_same_integers(lib, modified, monkeypatch):
     """Where two rows of T ints exceed LDS the finishing kernel's scans run in the halves of
