@@ -124,26 +124,30 @@ def test_exact_mi_kernels_without_lds_rows_give_the_same_bits(lib, dtype, modifi
             np.testing.assert_array_equal(a.view(np.uint8), b.view(np.uint8))
 
 
-@pytest.mark.parametrize("dtype,S", [
-    (np.float32, 8200),
-    pytest.param(np.float64, 4100, marks=pytest.mark.skipif(
-        os.environ.get("K2AMD_SLOW_CPU_TESTS", "0") != "1", reason="slow on the host: run with K2AMD_SLOW_CPU_TESTS=1"))])
-def test_exact_mi_kernels_beyond_the_lds_rows(lib, dtype, S, monkeypatch):
-    """One sequence with more rows than two LDS rows of 64 KiB hold (S > 8190 in fp32, 4094 in
-    fp64): served, and with the bits of the CPU loops."""
+@pytest.mark.parametrize("full", [False, pytest.param(True, marks=pytest.mark.skipif(
+    os.environ.get("K2AMD_SLOW_CPU_TESTS", "0") != "1", reason="slow on the host: run with K2AMD_SLOW_CPU_TESTS=1"))])
+@pytest.mark.parametrize("dtype,S", [(np.float32, 8200), (np.float64, 4100)])
+def test_exact_mi_kernels_beyond_the_lds_rows(lib, dtype, S, full, monkeypatch):
+    """Tensors with more rows than two LDS rows of 64 KiB hold (S > 8190 in fp32, 4094 in fp64):
+    served, and with the bits of the CPU loops.  The quick form sweeps boxes of a hundred rows at
+    either end of such a tensor (a barrier per step is what costs time on the host), the full
+    form all rows."""
     monkeypatch.delenv("K2AMD_MI_GENERIC_ROWS", raising=False)
     rng = np.random.default_rng(S)
-    B, T = 1, 2
-    c = {"B": B, "S": S, "T": T, "boundary": None,
+    B, T = 2, 2
+    bd = None if full else np.array([[S - 100, 0, S, T], [3, 1, 90, T]], dtype=np.int64)
+    c = {"B": B, "S": S, "T": T, "boundary": bd,
          "px": np.minimum(rng.normal(-2, 1, (B, S, T + 1)), 0).astype(dtype),
          "py": np.minimum(rng.normal(-2, 1, (B, S + 1, T)), 0).astype(dtype)}
     pp, ans, gx, gy, _ = _exact_pair(lib, c, dtype, False)
-    want_ans, want_p = omi.mi_forward(c["px"], c["py"], None)
-    want_gx, want_gy = omi.mi_backward(c["px"], c["py"], None, want_p)
+    want_ans, want_p = omi.mi_forward(c["px"], c["py"], bd)
+    want_gx, want_gy = omi.mi_backward(c["px"], c["py"], bd, want_p)
     np.testing.assert_array_equal(ans, want_ans)
-    np.testing.assert_array_equal(pp, want_p)
     np.testing.assert_array_equal(gx, want_gx)
     np.testing.assert_array_equal(gy, want_gy)
+    for b in range(B):
+        s0, t0, s1, t1 = (0, 0, S, T) if bd is None else bd[b]
+        np.testing.assert_array_equal(pp[b, s0:s1 + 1, t0:t1 + 1], want_p[b, s0:s1 + 1, t0:t1 + 1])
 
 
 # ---- the row kernels: get_rnnt_logprobs_joint / _pruned / HAT -----------------------------------

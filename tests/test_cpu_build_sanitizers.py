@@ -68,3 +68,16 @@ def test_simple_builder_and_fused_joiner(sanitizer):
 @slow
 def test_smoothed_builder_under_the_thread_sanitizer():
     _run(_program("smoothed_thread", "thread", [os.path.join(ck.SHIM, "smoothed_sanitizer_main.cc")]))
+
+
+ROWLESS = [os.path.join(ck.CSRC, "mi_generic.hip"), os.path.join(ck.CSRC, "prune.hip"),
+           os.path.join(ck.SHIM, "rowless_sanitizer_main.cc")]
+
+
+@slow
+@pytest.mark.parametrize("sanitizer", ["thread", "address,undefined"])
+def test_exact_recursion_and_prune_ranges_without_lds_rows(sanitizer):
+    """The forms that read the previous step back from the kernel's own output (mi_generic.hip past
+    8190 / 4094 rows, prune.hip past 8192 frames; selected here by their switches) and the kernel
+    of get_rnnt_prune_ranges_deprecated."""
+    _run(_program("rowless_" + sanitizer.split(",")[0], sanitizer, ROWLESS))
