@@ -34,7 +34,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(ROOT, "k2_amd", "csrc")
 SHIM = os.path.join(HERE, "cpu_build")
-OUT = os.path.join(SHIM, "_build")
+# (a directory per process where the suite runs in several: tests/conftest.py)
+OUT = os.path.join(SHIM, "_build", os.environ.get("PYTEST_XDIST_WORKER", ""))
 PORTABLE = ["rnnt_rows", "prune", "lattice", "mi_joint", "mi_generic", "rnnt_smoothed", "rnnt_simple", "mi_capi", "mi_wave"]
 # -ffp-contract=off: a * b + c rounds twice, as in the reference's CPU loops (the exact
 # mutual-information kernels are compared with them bit for bit)
@@ -130,6 +131,76 @@ def build():
                           stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     assert proc.returncode == 0, proc.stdout
     return path
+
+
+# The C++ host layer (k2_amd/csrc/pybind.cpp) for CPU tensors: a copy in which the places that
+# touch the device are replaced, and not a character else, linked against the host build of the
+# kernels.  What stays is what the GPU box runs of that file: every check, every allocation and
+# its shape, the order and count of the C-ABI arguments, what is returned.
+HOST_LAYER_PRELUDE = """
+namespace { struct HostStream { void *stream() const { return nullptr; } }; }
+"""
+HOST_LAYER_EDITS = [
+    ("#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>\n", "", 1),
+    ("#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>\n", "", 1),
+    ("#include <ATen/hip/HIPEvent.h>\n", HOST_LAYER_PRELUDE, 1),
+    # the device guard: nothing to guard
+    (re.compile(r"c10::hip::HIPGuardMasqueradingAsCUDA guard\([^;]*\);"), ";", None),
+    # torch's current stream of a device: the null stream of the stand-in
+    (re.compile(r"c10::hip::getCurrentHIPStreamMasqueradingAsCUDA\([^;]*?\)\.stream\(\)"), "nullptr", None),
+    ("auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(boundary.device().index());", "HostStream stream;", 1),
+    # the event behind the boundary copy: launches and copies are synchronous here
+    ("    event_.record(stream);\n", "", 1),
+    ("      event_.synchronize();\n", "", 1),
+    ("  at::cuda::CUDAEvent event_;\n", "", 1),
+    (".pinned_memory(true)", "", 2),
+    # "is on the device" becomes "is a tensor"
+    (".is_cuda()", ".defined()", None),
+    ("->is_cuda()", "->defined()", None),
+    ("PYBIND11_MODULE(_k2_amd, m)", "PYBIND11_MODULE(_k2_amd_host, m)", 1),
+    # (the process has usually loaded the GPU build of this module too, with a class of this name)
+    ('pybind11::class_<BoundaryRead>(m, "BoundaryRead")', 'pybind11::class_<BoundaryRead>(m, "BoundaryRead", pybind11::module_local())', 1),
+]
+
+_host_layer = None
+
+
+def host_layer():
+    """The module built from the edited copy of pybind.cpp (tests/cpu_build/_build/_k2_amd_host*.so)."""
+    global _host_layer
+    if _host_layer is not None:
+        return _host_layer
+    import importlib.util
+    import sysconfig
+    import pybind11
+    import torch
+    lib()  # the kernels it links against
+    text = open(os.path.join(CSRC, "pybind.cpp")).read()
+    for old, new, count in HOST_LAYER_EDITS:
+        if isinstance(old, str):
+            found = text.count(old)
+            text = text.replace(old, new)
+        else:
+            text, found = old.subn(new, text)
+        assert found >= 1 and (count is None or found == count), (old, found)
+    assert "hip" not in re.sub(r"//[^\n]*", "", text).lower().replace("hipstream", ""), "a device call is left"
+    src = os.path.join(OUT, "pybind_host.cpp")
+    with open(src, "w") as f:
+        f.write(text)
+    tdir = os.path.dirname(torch.__file__)
+    out = os.path.join(OUT, "_k2_amd_host" + sysconfig.get_config_var("EXT_SUFFIX"))
+    cmd = ["g++", "-O0", "-std=c++17", "-fPIC", "-shared", "-DTORCH_EXTENSION_NAME=_k2_amd_host",
+           "-DTORCH_API_INCLUDE_EXTENSION_H", f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+           f"-I{tdir}/include", f"-I{tdir}/include/torch/csrc/api/include", f"-I{sysconfig.get_paths()['include']}",
+           f"-I{pybind11.get_include()}", f"-I{os.path.join(ROOT, 'include')}", "-fvisibility=hidden", src, "-o", out,
+           f"-L{OUT}", "-lk2amd_cpu", "-Wl,-rpath,$ORIGIN", f"-L{tdir}/lib", f"-Wl,-rpath,{tdir}/lib",
+           "-ltorch", "-ltorch_cpu", "-lc10", "-ltorch_python"]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert proc.returncode == 0, proc.stdout[-4000:]
+    spec = importlib.util.spec_from_file_location("_k2_amd_host", out)
+    _host_layer = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(_host_layer)
+    return _host_layer
 
 
 def lib():

@@ -1,0 +1,176 @@
+"""The C++ host layer (k2_amd/csrc/pybind.cpp) on CPU tensors: a copy in which only the places
+that touch the device are replaced (tests/cpu_kernels.py::HOST_LAYER_EDITS: the device guard,
+torch's current stream, the event behind the boundary copy, pinned memory, "is on the device"),
+built against the host build of the kernels.  Everything else of that file runs as it runs on the
+GPU box: the checks, the allocations and their shapes, the order and count of the arguments of
+every C-ABI call, what comes back.
+
+It is compared with the ctypes host layer (k2_amd/capi.py), function by function and bit for
+bit, as tests/test_zw_host_layers_gpu.py and tests/test_mi_gpu.py compare the two on the GPU, and
+the loss functions run end to end through it against the reference's fixtures."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import cases
+import cpu_kernels as ck
+from test_cpu_build_host_layer import host_on_cpu  # noqa: F401  (a fixture)
+
+slow = pytest.mark.skipif(os.environ.get("K2AMD_SLOW_CPU_TESTS", "0") != "1",
+                          reason="slow on the host: run with K2AMD_SLOW_CPU_TESTS=1")
+CPU = torch.device("cpu")
+
+
+@pytest.fixture
+def hosts(host_on_cpu, monkeypatch):  # noqa: F811
+    """(native with the C++ host layer behind it, capi), both over the host build of the kernels."""
+    from k2_amd import native
+    monkeypatch.setattr(native, "_ext", ck.host_layer())
+    return native, host_on_cpu
+
+
+def _t(a):
+    return None if a is None else torch.from_numpy(np.ascontiguousarray(a))
+
+
+@slow
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("rnnt_type", ["regular", "modified", "constrained"])
+def test_builders_of_both_hosts(hosts, rnnt_type, dtype):
+    import test_zw_host_layers_gpu as zw
+    zw.test_builders(CPU, hosts, rnnt_type, dtype)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_pruning_and_lattice_of_both_hosts(hosts, dtype):
+    import test_zw_host_layers_gpu as zw
+    zw.test_pruning_and_lattice(CPU, hosts, dtype)
+
+
+@pytest.mark.parametrize("modified", [False, True])
+def test_deprecated_ranges_of_both_hosts(hosts, modified):
+    native, capi = hosts
+    B, T, S, R = 3, 41, 11, 4
+    rng = np.random.default_rng(94)
+    T1 = T if modified else T + 1
+    gx, gy = _t(rng.uniform(0, 1, (B, S, T1)).astype(np.float32)), _t(rng.uniform(0, 1, (B, S + 1, T)).astype(np.float32))
+    bd = _t(np.array([[0, 0, S, T], [0, 0, S - 2, T - 5], [0, 0, S - 1, T]], np.int64))
+    a, b = native.prune_ranges(gx, gy, bd, R, deprecated=True), capi.prune_ranges(gx, gy, bd, R, deprecated=True)
+    assert a.dtype == torch.int64 and torch.equal(a, b)
+    assert not torch.equal(a, native.prune_ranges(gx, gy, bd, R))  # (the two rules differ on random occupation)
+    from oracle import rnnt as orn
+    assert np.array_equal(a.numpy(), orn.prune_ranges_deprecated(gx.numpy(), gy.numpy(), bd.numpy(), R))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("rnnt_type", ["regular", "modified"])
+def test_smoothed_builder_of_both_hosts(hosts, rnnt_type, dtype):
+    native, capi = hosts
+    code = {"regular": 0, "modified": 1}[rnnt_type]
+    B, T, S, C = 3, 13, 5, 33
+    c = cases.rnnt_case(95, B, T, S, C, dtype=dtype, t_lo=max(S, T - 3), s_lo=max(1, S - 2), modified=rnnt_type != "regular")
+    lm, am, sym, bd = (_t(c[k]) for k in ("lm", "am", "symbols", "boundary"))
+    assert native.smoothed_supported(lm, am) and capi.smoothed_supported(lm, am)
+    a = native.logprobs_smoothed_forward(lm, am, sym, 0, 0.25, 0.1, code, bd)
+    b = capi.logprobs_smoothed_forward(lm, am, sym, 0, 0.25, 0.1, code, bd)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1]) and len(a[2]) == len(b[2])
+    for x, y in zip(a[2], b[2]):
+        assert torch.equal(x, y)
+    rng = np.random.default_rng(96)
+    T1 = T + 1 if rnnt_type == "regular" else T
+    gx, gy = _t(rng.uniform(0, 1, (B, S, T1)).astype(dtype)), _t(rng.uniform(0, 1, (B, S + 1, T)).astype(dtype))
+    for seq in (None, _t(np.linspace(0.5, 1.5, B).astype(dtype))):
+        ga = native.logprobs_smoothed_backward(gx, gy, sym, bd, a[2], 0, 0.25, 0.1, code, seq)
+        gb = capi.logprobs_smoothed_backward(gx, gy, sym, bd, b[2], 0, 0.25, 0.1, code, seq)
+        assert len(ga) == len(gb) == 2 and torch.equal(ga[0], gb[0]) and torch.equal(ga[1], gb[1])
+
+
+def test_recursion_of_both_hosts(hosts):
+    """The functions of the reference's names (mutual_information.cu:26-67) in both hosts: the pair,
+    the pair that hands the log-derivatives on, the single launch, a strided px made contiguous
+    by the C++ host, ans_grad overwritten."""
+    native, capi = hosts
+    ext = native._ext
+    rng = np.random.default_rng(77)
+    B, S, T = 2, 70, 40
+    px = _t(rng.standard_normal((B, S, T + 1)).astype(np.float32))
+    py = _t(rng.standard_normal((B, S + 1, T)).astype(np.float32))
+    bd = torch.tensor([[0, 0, S, T], [3, 5, 66, 33]], dtype=torch.int64)
+    p1, p2 = torch.empty(B, S + 1, T + 1), torch.empty(B, S + 1, T + 1)
+    ans1 = capi.mi_forward(px, py, bd, p1)
+    px_strided = torch.empty(B, S, 2 * px.shape[2])[:, :, ::2]
+    px_strided.copy_(px)
+    ans2 = ext.mutual_information_forward(px=px_strided, py=py, boundary=bd, p=p2)
+    g1, g2 = torch.full((B,), 2.0), torch.full((B,), 2.0)
+    gx1, gy1 = capi.mi_backward(px, py, bd, p1, g1, overwrite_ans_grad=True)
+    gx2, gy2 = ext.mutual_information_backward(px=px, py=py, boundary=bd, p=p2, ans_grad=g2)
+    for x, y in ((ans1, ans2), (gx1, gx2), (gy1, gy2), (g1, g2)):  # (p is undefined outside the boxes)
+        assert torch.equal(x, y)
+    assert ext.mutual_information_keeps_log_deriv(px=px, py=py) == bool(capi.mi_keeps_log_deriv(px, py))
+    if ext.mutual_information_keeps_log_deriv(px=px, py=py):
+        p3, kept = torch.empty(B, S + 1, T + 1), torch.full((B, S + 1, T + 1), float("nan"))
+        ans3 = ext.mutual_information_forward(px=px_strided, py=py, boundary=bd, p=p3, log_deriv=kept)
+        g3 = torch.full((B,), 2.0)
+        gx3, gy3 = ext.mutual_information_backward(px=px, py=py, boundary=bd, p=p3, ans_grad=g3, log_deriv=kept)
+        assert torch.equal(ans3, ans2) and torch.equal(gx3, gx2) and torch.equal(gy3, gy2) and torch.equal(g3, g2)
+        with pytest.raises(RuntimeError):  # wrong shape
+            ext.mutual_information_forward(px=px, py=py, boundary=bd, p=p3, log_deriv=kept[:, :-1])
+    assert ext.mutual_information_forward_backward_supported(px=px, py=py) == bool(capi.mi_forward_backward_supported(px, py))
+    if ext.mutual_information_forward_backward_supported(px=px, py=py):
+        g5, g6 = torch.full((B,), 2.0), torch.full((B,), 2.0)
+        ans5, gx5, gy5 = ext.mutual_information_forward_backward(px=px_strided, py=py, boundary=bd, ans_grad=g5)
+        ans6, gx6, gy6 = capi.mi_forward_backward(px, py, bd, g6, overwrite_ans_grad=True)
+        assert torch.equal(ans5, ans6) and torch.equal(gx5, gx6) and torch.equal(gy5, gy6) and torch.equal(g5, g6)
+        np.testing.assert_allclose(ans5.numpy(), ans2.numpy(), rtol=1e-4, atol=1e-5)
+    rows = ext.BoundaryRead(bd).rows()
+    assert rows == tuple(tuple(r) for r in bd.tolist())
+    ws = ext.mutual_information_workspace(px)
+    assert ws is not None and ws.dtype == torch.uint8
+    assert ext.mutual_information_recover_workspaces() == 0
+
+
+def test_joint_products_of_both_hosts(hosts):
+    native, capi = hosts
+    rng = np.random.default_rng(807)
+    N, B, S, T = 3, 2, 4, 7
+    pxs = [_t(-rng.uniform(0, 3, (B, S, T + 1))) for _ in range(N)]
+    pys = [_t(-rng.uniform(0, 3, (B, S + 1, T))) for _ in range(N)]
+    gx, gy = _t(rng.uniform(0, 1, (B, S, T + 1))), _t(rng.uniform(0, 1, (B, S + 1, T)))
+    assert torch.equal(native._ext.mutual_information_joint_products(pxs, pys, gx, gy),
+                       capi.mi_joint_products(pxs, pys, gx, gy))
+
+
+@pytest.mark.parametrize("name", ["test_reference_chain_fixtures",
+                                  "test_reference_prune_ranges_on_ties_and_near_ties",
+                                  pytest.param("test_reference_smoothed_and_hat_gradient_fixtures", marks=slow)])
+def test_reference_fixtures_through_the_api_over_the_cpp_host(hosts, name, monkeypatch):
+    """What was recorded from the reference's own Python chain, through k2_amd's API with the C++
+    host layer underneath: losses, occupation probabilities, gradients, both kinds of prune
+    ranges (every eighth chain; every second with the slow switch)."""
+    import test_rnnt_gpu
+    if "chain" in name:
+        monkeypatch.setenv("K2AMD_SMOOTHED_KERNELS", "1")
+        getattr(test_rnnt_gpu, name)(CPU, every=2 if os.environ.get("K2AMD_SLOW_CPU_TESTS", "0") == "1" else 8)
+        return
+    if "smoothed" in name:
+        monkeypatch.setenv("K2AMD_SMOOTHED_KERNELS", "1")
+    getattr(test_rnnt_gpu, name)(CPU)
+
+
+def test_recursion_scenario_over_the_cpp_host(hosts):
+    """mutual_information_recursion through its autograd Function with the C++ host layer
+    underneath (boundary read, workspace cache, the single launch or the pair as advised)."""
+    import k2_amd as k2
+    from oracle import mi as omi
+    c = cases.mi_case(41, dtype=np.float32, max_B=3, max_S=20, max_T=40, force={"rand_bd": True})
+    px, py = _t(c["px"]).requires_grad_(True), _t(c["py"]).requires_grad_(True)
+    scores = k2.mutual_information_recursion(px, py, _t(c["boundary"]))
+    want, gx, gy = omi.mi(c["px"], c["py"], c["boundary"])
+    np.testing.assert_allclose(scores.detach().numpy(), want, rtol=1e-4, atol=1e-5)
+    finite = np.isfinite(want)
+    scores[torch.from_numpy(finite)].sum().backward()
+    for b in np.nonzero(finite)[0]:
+        np.testing.assert_allclose(px.grad.numpy()[b], gx[b], rtol=1e-4, atol=1e-5)
+        np.testing.assert_allclose(py.grad.numpy()[b], gy[b], rtol=1e-4, atol=1e-5)

@@ -23,7 +23,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 SRC = os.path.join(ROOT, "k2_amd", "csrc", "rnnt_smoothed.hip")
 SHIM = os.path.join(HERE, "cpu_build")
-OUT = os.path.join(SHIM, "_build")
+OUT = os.path.join(SHIM, "_build", os.environ.get("PYTEST_XDIST_WORKER", ""))  # as tests/cpu_kernels.py
 TYPES = ["regular", "modified", "constrained"]
 CODES = {"regular": 0, "modified": 1, "constrained": 2}
 
