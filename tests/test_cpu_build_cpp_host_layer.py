@@ -35,9 +35,10 @@ def _t(a):
     return None if a is None else torch.from_numpy(np.ascontiguousarray(a))
 
 
-@slow
-@pytest.mark.parametrize("dtype", [np.float32, np.float64])
-@pytest.mark.parametrize("rnnt_type", ["regular", "modified", "constrained"])
+@pytest.mark.parametrize("rnnt_type,dtype", [
+    ("regular", np.float32), ("constrained", np.float64),
+    pytest.param("regular", np.float64, marks=slow), pytest.param("constrained", np.float32, marks=slow),
+    pytest.param("modified", np.float32, marks=slow), pytest.param("modified", np.float64, marks=slow)])
 def test_builders_of_both_hosts(hosts, rnnt_type, dtype):
     import test_zw_host_layers_gpu as zw
     zw.test_builders(CPU, hosts, rnnt_type, dtype)
