@@ -52,40 +52,15 @@ def test_pruning_and_lattice_of_both_hosts(hosts, dtype):
 
 @pytest.mark.parametrize("modified", [False, True])
 def test_deprecated_ranges_of_both_hosts(hosts, modified):
-    native, capi = hosts
-    B, T, S, R = 3, 41, 11, 4
-    rng = np.random.default_rng(94)
-    T1 = T if modified else T + 1
-    gx, gy = _t(rng.uniform(0, 1, (B, S, T1)).astype(np.float32)), _t(rng.uniform(0, 1, (B, S + 1, T)).astype(np.float32))
-    bd = _t(np.array([[0, 0, S, T], [0, 0, S - 2, T - 5], [0, 0, S - 1, T]], np.int64))
-    a, b = native.prune_ranges(gx, gy, bd, R, deprecated=True), capi.prune_ranges(gx, gy, bd, R, deprecated=True)
-    assert a.dtype == torch.int64 and torch.equal(a, b)
-    assert not torch.equal(a, native.prune_ranges(gx, gy, bd, R))  # (the two rules differ on random occupation)
-    from oracle import rnnt as orn
-    assert np.array_equal(a.numpy(), orn.prune_ranges_deprecated(gx.numpy(), gy.numpy(), bd.numpy(), R))
+    import test_zw_host_layers_gpu as zw
+    zw.test_deprecated_ranges(CPU, hosts, modified)
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("rnnt_type", ["regular", "modified"])
 def test_smoothed_builder_of_both_hosts(hosts, rnnt_type, dtype):
-    native, capi = hosts
-    code = {"regular": 0, "modified": 1}[rnnt_type]
-    B, T, S, C = 3, 13, 5, 33
-    c = cases.rnnt_case(95, B, T, S, C, dtype=dtype, t_lo=max(S, T - 3), s_lo=max(1, S - 2), modified=rnnt_type != "regular")
-    lm, am, sym, bd = (_t(c[k]) for k in ("lm", "am", "symbols", "boundary"))
-    assert native.smoothed_supported(lm, am) and capi.smoothed_supported(lm, am)
-    a = native.logprobs_smoothed_forward(lm, am, sym, 0, 0.25, 0.1, code, bd)
-    b = capi.logprobs_smoothed_forward(lm, am, sym, 0, 0.25, 0.1, code, bd)
-    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1]) and len(a[2]) == len(b[2])
-    for x, y in zip(a[2], b[2]):
-        assert torch.equal(x, y)
-    rng = np.random.default_rng(96)
-    T1 = T + 1 if rnnt_type == "regular" else T
-    gx, gy = _t(rng.uniform(0, 1, (B, S, T1)).astype(dtype)), _t(rng.uniform(0, 1, (B, S + 1, T)).astype(dtype))
-    for seq in (None, _t(np.linspace(0.5, 1.5, B).astype(dtype))):
-        ga = native.logprobs_smoothed_backward(gx, gy, sym, bd, a[2], 0, 0.25, 0.1, code, seq)
-        gb = capi.logprobs_smoothed_backward(gx, gy, sym, bd, b[2], 0, 0.25, 0.1, code, seq)
-        assert len(ga) == len(gb) == 2 and torch.equal(ga[0], gb[0]) and torch.equal(ga[1], gb[1])
+    import test_zw_host_layers_gpu as zw
+    zw.test_smoothed_builder(CPU, hosts, rnnt_type, dtype)
 
 
 def test_recursion_of_both_hosts(hosts):

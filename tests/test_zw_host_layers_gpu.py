@@ -7,6 +7,8 @@ Written while no GPU was at hand and not run on one yet; the ctypes side has run
 build of the kernels (tests/test_cpu_build_host_layer.py), the extension's side in all other GPU
 tests.  Also here: the fused joiner's case without frames, written at the same time.  The file's
 name puts it behind the tests that have run on a GPU."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -102,6 +104,45 @@ def test_pruning_and_lattice(device, hosts, dtype):
     frames = bd[:, 3].to(torch.int32).contiguous()
     _same(native.pruned_ranges_to_lattice(ranges.to(torch.int32), frames, sym, logits),
           capi.pruned_ranges_to_lattice(ranges.to(torch.int32), frames, sym, logits), "lattice")
+
+
+@pytest.mark.parametrize("modified", [False, True])
+def test_deprecated_ranges(device, hosts, modified):
+    native, capi = hosts
+    B, T, S, R = 3, 41, 11, 4
+    rng = np.random.default_rng(94)
+    T1 = T if modified else T + 1
+    gx, gy = dev(rng.uniform(0, 1, (B, S, T1)).astype(np.float32), device), dev(rng.uniform(0, 1, (B, S + 1, T)).astype(np.float32), device)
+    bd = dev(np.array([[0, 0, S, T], [0, 0, S - 2, T - 5], [0, 0, S - 1, T]], np.int64), device)
+    a, b = native.prune_ranges(gx, gy, bd, R, deprecated=True), capi.prune_ranges(gx, gy, bd, R, deprecated=True)
+    _same(a, b, "deprecated ranges")
+    assert not torch.equal(a, native.prune_ranges(gx, gy, bd, R))  # (the two rules differ on random occupation)
+    from oracle import rnnt as orn
+    assert np.array_equal(a.cpu().numpy(), orn.prune_ranges_deprecated(gx.cpu().numpy(), gy.cpu().numpy(), bd.cpu().numpy(), R))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("rnnt_type", ["regular", "modified"])
+def test_smoothed_builder(device, hosts, rnnt_type, dtype):
+    """The smoothed builder's own kernels through both hosts (they are called directly here,
+    whatever K2AMD_SMOOTHED_KERNELS says about the Python layer's choice)."""
+    native, capi = hosts
+    if torch.device(device).type != "cpu" and os.environ.get("K2AMD_SMOOTHED_KERNELS", "0") != "1":
+        pytest.skip("the smoothed builder's kernels have not run on a GPU yet: set K2AMD_SMOOTHED_KERNELS=1")
+    code = CODES[rnnt_type]
+    B, T, S, C = 3, 13, 5, 33
+    c = cases.rnnt_case(95, B, T, S, C, dtype=dtype, t_lo=max(S, T - 3), s_lo=max(1, S - 2), modified=rnnt_type != "regular")
+    lm, am, sym, bd = (dev(c[k], device) for k in ("lm", "am", "symbols", "boundary"))
+    assert native.smoothed_supported(lm, am) and capi.smoothed_supported(lm, am)
+    a = native.logprobs_smoothed_forward(lm, am, sym, 0, 0.25, 0.1, code, bd)
+    b = capi.logprobs_smoothed_forward(lm, am, sym, 0, 0.25, 0.1, code, bd)
+    _same(a, b, "smoothed forward")
+    rng = np.random.default_rng(96)
+    T1 = T + 1 if rnnt_type == "regular" else T
+    gx, gy = dev(rng.uniform(0, 1, (B, S, T1)).astype(dtype), device), dev(rng.uniform(0, 1, (B, S + 1, T)).astype(dtype), device)
+    for seq in (None, dev(np.linspace(0.5, 1.5, B).astype(dtype), device)):
+        _same(native.logprobs_smoothed_backward(gx, gy, sym, bd, a[2], 0, 0.25, 0.1, code, seq),
+              capi.logprobs_smoothed_backward(gx, gy, sym, bd, b[2], 0, 0.25, 0.1, code, seq), "smoothed backward")
 
 
 def test_fused_joiner_without_frames(device):
