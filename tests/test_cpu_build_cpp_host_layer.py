@@ -150,3 +150,31 @@ def test_recursion_scenario_over_the_cpp_host(hosts):
     for b in np.nonzero(finite)[0]:
         np.testing.assert_allclose(px.grad.numpy()[b], gx[b], rtol=1e-4, atol=1e-5)
         np.testing.assert_allclose(py.grad.numpy()[b], gy[b], rtol=1e-4, atol=1e-5)
+
+
+def test_error_flag_rides_with_the_cpp_hosts_boundary_read(hosts):
+    """The error flag of the stream's workspace rides with the C++ host's boundary read: forced
+    from the host, it turns the next read into a RuntimeError that names the timeout, once, and
+    the workspace is initialised again, so that the call after that works.  (Through the API this
+    runs on the GPU, tests/test_mi_gpu.py::test_a_wait_that_gave_up_raises_at_the_next_call: the
+    Python layer reads a host tensor's rows without this class.)"""
+    native, capi = hosts
+    ext = native._ext
+    rng = np.random.default_rng(19)
+    B, S, T = 2, 70, 40
+    px = _t(rng.normal(-2, 1, (B, S, T + 1)).astype(np.float32))
+    py = _t(rng.normal(-2, 1, (B, S + 1, T)).astype(np.float32))
+    bd = torch.tensor([[0, 0, S, T], [1, 2, 60, 33]], dtype=torch.int64)
+    p = torch.empty(B, S + 1, T + 1)
+    good = ext.mutual_information_forward(px=px, py=py, boundary=bd, p=p).clone()
+    assert torch.isfinite(good).all()
+    ws = ext.mutual_information_workspace(px)
+    assert ws is not None
+    ws[:16].view(torch.int32)[2] = 1                         # FastHeader::error
+    assert torch.isnan(ext.mutual_information_forward(px=px, py=py, boundary=bd, p=p)).all()
+    with pytest.raises(RuntimeError, match="timed out"):
+        ext.BoundaryRead(bd).rows()
+    assert int(ws[:16].view(torch.int32)[2]) == 0
+    assert ext.BoundaryRead(bd).rows() == tuple(tuple(r) for r in bd.tolist())
+    assert torch.equal(ext.mutual_information_forward(px=px, py=py, boundary=bd, p=p), good)
+    assert ext.mutual_information_recover_workspaces() == 0
