@@ -14,6 +14,7 @@ import pytest
 import torch
 
 import cases
+import tolerance
 from oracle import mi as omi
 from oracle import rnnt as orn
 
@@ -24,6 +25,25 @@ TOL = {np.dtype(np.float32): dict(rtol=1e-4, atol=1e-5), np.dtype(np.float64): d
 
 def dev(x, device):
     return None if x is None else torch.from_numpy(np.ascontiguousarray(x)).to(device)
+
+
+def _against_the_oracle(name, c, got):
+    """ans, px_grad, py_grad of the kernels against the CPU oracle: fp64 within 1e-10; fp32 within
+    1e-5 + 1e-4 |x| of the fp32 oracle, the elements that miss it arbitrated by the fp64 oracle
+    (tests/tolerance.py), 3 % of them at most."""
+    ans, _, gx, gy, _ = got
+    px, py, bd = c["px"], c["py"], c["boundary"]
+    want_ans, want_p = omi.mi_forward(px, py, bd)
+    want_gx, want_gy = omi.mi_backward(px, py, bd, want_p)
+    if px.dtype == np.float64:
+        for a, b in ((ans, want_ans), (gx, want_gx), (gy, want_gy)):
+            np.testing.assert_allclose(a, b, **TOL[np.dtype(np.float64)])
+        return
+    a64, p64 = omi.mi_forward(px.astype(np.float64), py.astype(np.float64), bd)
+    gx64, gy64 = omi.mi_backward(px.astype(np.float64), py.astype(np.float64), bd, p64)
+    tolerance.close_f32(name + " ans", ans, want_ans, a64, mode="absolute", max_arbitrated=0.03)
+    tolerance.close_f32(name + " px_grad", gx, want_gx, gx64, max_arbitrated=0.03)
+    tolerance.close_f32(name + " py_grad", gy, want_gy, gy64, max_arbitrated=0.03)
 
 
 def _exact_pair(c, device):
@@ -57,32 +77,27 @@ def test_exact_mi_kernels_without_lds_rows_give_the_same_bits(device, dtype, mod
         glob = _exact_pair(c, device)
         for name, a, b in zip(("ans", "p", "px_grad", "py_grad", "ans_grad"), lds, glob):
             assert np.array_equal(a.view(np.uint8), b.view(np.uint8)), (seed, name)
-        want_ans, want_p = omi.mi_forward(c["px"], c["py"], c["boundary"])
-        want_gx, want_gy = omi.mi_backward(c["px"], c["py"], c["boundary"], want_p)
-        tol = TOL[np.dtype(dtype)]
-        np.testing.assert_allclose(glob[0], want_ans, **tol)
-        np.testing.assert_allclose(glob[2], want_gx, **tol)
-        np.testing.assert_allclose(glob[3], want_gy, **tol)
+        _against_the_oracle(f"case {seed}", c, glob)
 
 
+@pytest.mark.parametrize("full", [False, True])
 @pytest.mark.parametrize("dtype,S", [(np.float32, 8200), (np.float64, 4100)])
-def test_exact_mi_kernels_beyond_the_lds_rows(device, dtype, S, monkeypatch):
-    """More rows than two LDS rows of 64 KiB hold (S > 8190 in fp32, 4094 in fp64), no workspace
-    in play (K2AMD_MI_PATH=generic): served, within the tolerance of the oracle."""
+def test_exact_mi_kernels_beyond_the_lds_rows(device, dtype, S, full, monkeypatch):
+    """Tensors with more rows than two LDS rows of 64 KiB hold (S > 8190 in fp32, 4094 in fp64), no
+    workspace in play (K2AMD_MI_PATH=generic): served, within the tolerance of the oracle.  Boxes
+    of a hundred rows at either end of such a tensor, or all of its rows; log-probabilities close
+    to zero, so that p stays small over thousands of rows and the comparison says something about
+    the kernels rather than about the conditioning of fp32 sums of that length."""
     monkeypatch.setenv("K2AMD_MI_PATH", "generic")
     monkeypatch.delenv("K2AMD_MI_GENERIC_ROWS", raising=False)
     rng = np.random.default_rng(S)
     B, T = 2, 3
-    c = {"B": B, "S": S, "T": T, "boundary": np.array([[0, 0, S, T], [5, 1, S - 7, T]], dtype=np.int64),
-         "px": np.minimum(rng.normal(-2, 1, (B, S, T + 1)), 0).astype(dtype),
-         "py": np.minimum(rng.normal(-2, 1, (B, S + 1, T)), 0).astype(dtype)}
-    ans, _, gx, gy, _ = _exact_pair(c, device)
-    want_ans, want_p = omi.mi_forward(c["px"], c["py"], c["boundary"])
-    want_gx, want_gy = omi.mi_backward(c["px"], c["py"], c["boundary"], want_p)
-    tol = TOL[np.dtype(dtype)]
-    np.testing.assert_allclose(ans, want_ans, **tol)
-    np.testing.assert_allclose(gx, want_gx, **tol)
-    np.testing.assert_allclose(gy, want_gy, **tol)
+    bd = np.array([[0, 0, S, T], [5, 1, S - 7, T]] if full else [[S - 100, 0, S, T], [3, 1, 90, T]], dtype=np.int64)
+    spread = 0.002 if full else 0.3
+    c = {"B": B, "S": S, "T": T, "boundary": bd,
+         "px": -rng.uniform(0, spread, (B, S, T + 1)).astype(dtype),
+         "py": -rng.uniform(0, spread, (B, S + 1, T)).astype(dtype)}
+    _against_the_oracle(f"S={S} full={full}", c, _exact_pair(c, device))
 
 
 @pytest.mark.parametrize("modified", [False, True])
