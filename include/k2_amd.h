@@ -55,7 +55,8 @@ K2AMD_API const char *k2amd_status_string(int status);
  * must run k2amd_mi_workspace_init() on it ONCE before its first use (and again after a
  * K2AMD_ERR_TIMEOUT); the kernels leave it ready for the next call, so a buffer sized for the
  * largest shape can be reused for any smaller one.  One workspace serves one stream at a time.
- * Passing workspace == NULL selects the exact one-workgroup-per-sequence kernels instead.
+ * Passing workspace == NULL selects the exact one-workgroup-per-sequence kernels instead, which
+ * take any S and T with (S + 1) (T + 1) < 2^31.
  */
 K2AMD_API size_t k2amd_mi_workspace_bytes(int B, int S, int T, int modified, int dtype);
 K2AMD_API int k2amd_mi_workspace_init(void *workspace, size_t workspace_bytes, void *stream);

@@ -168,3 +168,6 @@ def test_pybind_host_module_covers_every_builder_of_the_c_abi():
     with pytest.raises(RuntimeError, match="no CPU path"):
         native.prune_ranges(torch.zeros(1, 2, 5), torch.zeros(1, 3, 4),
                             torch.tensor([[0, 0, 2, 4]]), 2)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        native.prune_ranges(torch.zeros(1, 2, 5), torch.zeros(1, 3, 4),
+                            torch.tensor([[0, 0, 2, 4]]), 2, deprecated=True)
