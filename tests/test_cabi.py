@@ -171,3 +171,43 @@ def test_pybind_host_module_covers_every_builder_of_the_c_abi():
     with pytest.raises(RuntimeError, match="no CPU path"):
         native.prune_ranges(torch.zeros(1, 2, 5), torch.zeros(1, 3, 4),
                             torch.tensor([[0, 0, 2, 4]]), 2, deprecated=True)
+
+
+def test_header_is_plain_c_and_a_c_program_links_against_the_library(tmp_path):
+    """The boundary is a C ABI: include/k2_amd.h compiles as C99 without warnings, and a C program
+    built with gcc alone links against libk2amd.so and gets status codes back from calls that
+    are refused before anything touches a GPU."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    from k2_amd import capi
+    header = os.path.join(ROOT, "include", "k2_amd.h")
+    proc = subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-fsyntax-only", "-x", "c", header],
+                          stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert proc.returncode == 0, proc.stdout
+    src = tmp_path / "caller.c"
+    src.write_text('''
+#include <stdio.h>
+#include <string.h>
+#include "k2_amd.h"
+int main(void) {
+  if (k2amd_version() != K2AMD_VERSION) return 1;
+  if (strcmp(k2amd_status_string(K2AMD_OK), "ok") != 0) return 2;
+  /* negative sizes, an unknown dtype, a window longer than S + 1: refused, nothing launched */
+  if (k2amd_mi_forward(NULL, NULL, NULL, NULL, NULL, -1, 1, 1, 0, K2AMD_F32, NULL, 0, NULL) != K2AMD_ERR_INVALID_ARGUMENT) return 3;
+  if (k2amd_rnnt_prune_ranges(NULL, NULL, NULL, NULL, 1, 4, 4, 0, 9, K2AMD_F32, NULL) != K2AMD_ERR_INVALID_ARGUMENT) return 4;
+  if (k2amd_rnnt_prune_ranges_deprecated(NULL, NULL, NULL, NULL, 1, 4, 4, 0, 9, K2AMD_F32, NULL) != K2AMD_ERR_INVALID_ARGUMENT) return 5;
+  if (k2amd_mi_workspace_bytes(32, 200, 1000, 1, K2AMD_F32) == 0) return 6;
+  printf("c caller ok\\n");
+  return 0;
+}
+''')
+    lib_dir = os.path.dirname(capi._LIB_PATH)
+    exe = tmp_path / "caller"
+    proc = subprocess.run(["gcc", "-std=c99", "-Wall", f"-I{os.path.join(ROOT, 'include')}", str(src), "-o", str(exe),
+                           f"-L{lib_dir}", "-lk2amd", f"-Wl,-rpath,{lib_dir}"],
+                          stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert proc.returncode == 0, proc.stdout
+    proc = subprocess.run([str(exe)], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    assert proc.returncode == 0 and "c caller ok" in proc.stdout, (proc.returncode, proc.stdout)
