@@ -37,8 +37,8 @@ def _t(a):
 
 @pytest.mark.parametrize("rnnt_type,dtype", [
     ("regular", np.float32), ("constrained", np.float64),
-    pytest.param("regular", np.float64, marks=slow), pytest.param("constrained", np.float32, marks=slow),
-    pytest.param("modified", np.float32, marks=slow), pytest.param("modified", np.float64, marks=slow)])
+    ("modified", np.float32), pytest.param("regular", np.float64, marks=slow),
+    pytest.param("constrained", np.float32, marks=slow), pytest.param("modified", np.float64, marks=slow)])
 def test_builders_of_both_hosts(hosts, rnnt_type, dtype):
     import test_zw_host_layers_gpu as zw
     zw.test_builders(CPU, hosts, rnnt_type, dtype)

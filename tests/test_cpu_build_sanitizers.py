@@ -1,5 +1,5 @@
-"""The builders' kernels under host sanitizers (K2AMD_SLOW_CPU_TESTS=1: minutes each): programs of
-their own, built from the same kernel sources over the thread stand-in
+"""Kernels under host sanitizers (the builders' with K2AMD_SLOW_CPU_TESTS=1 only: minutes each; the
+exact recursion and the prune ranges without their LDS rows always): programs of their own, built from the same kernel sources over the thread stand-in
 (tests/cpu_build/hip/hip_runtime.h) and a small driver that calls the C-ABI on random inputs in
 heap buffers of exactly the documented sizes.
 
@@ -74,7 +74,6 @@ ROWLESS = [os.path.join(ck.CSRC, "mi_generic.hip"), os.path.join(ck.CSRC, "prune
            os.path.join(ck.SHIM, "rowless_sanitizer_main.cc")]
 
 
-@slow
 @pytest.mark.parametrize("sanitizer", ["thread", "address,undefined"])
 def test_exact_recursion_and_prune_ranges_without_lds_rows(sanitizer):
     """The forms that read the previous step back from the kernel's own output (mi_generic.hip past
