@@ -975,12 +975,15 @@ bool ArgsOk(int B, int S, int T, int C, int blank, int rnnt_type, int dtype) {
   if (B < 0 || S < 0 || T < 0 || C <= 0 || blank < 0 || blank >= C) return false;
   if (rnnt_type != K2AMD_REGULAR && rnnt_type != K2AMD_MODIFIED && rnnt_type != K2AMD_CONSTRAINED)
     return false;
-  if (B > 65535) return false;  // grid.z
-  {  // tile ids of the three products are ints
-    const long long ts = (S + 32) / 32, tt = (T + 31) / 32, tc = (C + 31) / 32, lim = 1ll << 30;
-    if (B * ts * tt > lim || B * ts * tc > lim || B * tt * tc > lim) return false;
-  }
   return dtype == K2AMD_F32 || dtype == K2AMD_F64;
+}
+
+// What the launches take of valid arguments: the batch is gridDim.z, tile ids of the three
+// products are ints.
+bool ShapeServed(int B, int S, int T, int C) {
+  if (B > 65535) return false;
+  const long long ts = (S + 32) / 32, tt = (T + 31) / 32, tc = (C + 31) / 32, lim = 1ll << 30;
+  return B * ts * tt <= lim && B * ts * tc <= lim && B * tt * tc <= lim;
 }
 
 }  // namespace
@@ -996,6 +999,7 @@ int k2amd_rnnt_logprobs_simple_forward(const void *lm, const void *am, const int
                                        int B, int S, int T, int C, int termination_symbol,
                                        int rnnt_type, int dtype, void *stream) {
   if (!ArgsOk(B, S, T, C, termination_symbol, rnnt_type, dtype)) return K2AMD_ERR_INVALID_ARGUMENT;
+  if (!ShapeServed(B, S, T, C)) return K2AMD_ERR_UNSUPPORTED;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == K2AMD_F32)
     return SimpleForward<float>((const float *)lm, (const float *)am, symbols, boundary, (float *)px, (float *)py, (float *)lm_probs, (float *)am_probs, (float *)lm_max, (float *)am_max, (float *)denom, B, S, T, C, termination_symbol, rnnt_type, st);
@@ -1016,6 +1020,7 @@ int k2amd_rnnt_logprobs_simple_backward(const void *px_grad, const void *py_grad
                                         int T, int C, int termination_symbol, int rnnt_type,
                                         int dtype, void *stream) {
   if (!ArgsOk(B, S, T, C, termination_symbol, rnnt_type, dtype)) return K2AMD_ERR_INVALID_ARGUMENT;
+  if (!ShapeServed(B, S, T, C)) return K2AMD_ERR_UNSUPPORTED;
   {  // no frames or no sequences: nothing is asked for, and a null pointer is as good as any
     const size_t need = k2amd_rnnt_logprobs_simple_backward_scratch_elements(B, S, T);
     if (need > 0 && (q_scratch == nullptr || q_scratch_elements < need)) return K2AMD_ERR_WORKSPACE;

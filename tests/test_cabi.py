@@ -70,6 +70,8 @@ def test_invalid_arguments_return_codes_without_a_gpu():
     assert lib.k2amd_rnnt_logprobs_joint_forward(None, None, None, None, None, None, 1, 1, 1, 4, 9, 0, 0, None) == 1
     # the simple builder's backward: scratch smaller than its query function says is refused
     # before anything is launched (B=2 S=5 T=9 C=7: 2 * (6*9 + 1*9 + 2*6*1) = 150 elements)
+    # a batch beyond the launches' grid is a valid call that this build does not serve
+    assert lib.k2amd_rnnt_logprobs_simple_forward(*([None] * 11), 70000, 5, 9, 7, 0, 0, 0, None) == 2
     need = lib.k2amd_rnnt_logprobs_simple_backward_scratch_elements(2, 5, 9)
     assert need == 150
     args = lambda n: (one, one, None, one, None, one, one, one, one, one, one, n, 2, 5, 9, 7, 0, 0, 0, None)
