@@ -369,25 +369,6 @@ def rnnt_loss(
     return _Scores.apply("joint", rnnt_type, float(delay_penalty), False, reduction, *args)[0]
 
 
-def _monotonic_lower_bound(x: Tensor) -> Tensor:
-    """k2/python/k2/rnnt_loss.py:543-577: reverse running minimum along the last axis."""
-    x = torch.flip(x, dims=(-1,))
-    x, _ = torch.cummin(x, dim=-1)
-    return torch.flip(x, dims=(-1,))
-
-
-def _adjust_pruning_lower_bound(s_begin: Tensor, s_range: int) -> Tensor:
-    """k2/python/k2/rnnt_loss.py:580-630 as torch ops (the fused kernel in
-    get_rnnt_prune_ranges does the same on the device in one launch)."""
-    (B, T) = s_begin.shape
-    ramp = (s_range - 1) * torch.arange(0, T, device=s_begin.device)
-    s_begin = _monotonic_lower_bound(s_begin)
-    s_begin = -(s_begin - ramp)
-    s_begin = _monotonic_lower_bound(s_begin)
-    s_begin = torch.clamp(s_begin, min=0)
-    return -(s_begin - ramp)
-
-
 def get_rnnt_prune_ranges(
     px_grad: Tensor,
     py_grad: Tensor,
