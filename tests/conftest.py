@@ -26,7 +26,10 @@ def pytest_cmdline_main(config):
     if hasattr(config, "workerinput") or not config.pluginmanager.hasplugin("xdist"):
         return
     option = config.option
-    workers = int(os.environ.get("K2AMD_TEST_WORKERS", CPU_SUITE_WORKERS))
+    try:
+        workers = int(os.environ.get("K2AMD_TEST_WORKERS", CPU_SUITE_WORKERS))
+    except ValueError:
+        workers = CPU_SUITE_WORKERS
     if (option.markexpr or "").strip() != "not gpu" or workers < 2:
         return
     if option.numprocesses is not None or option.dist != "no" or option.tx or option.collectonly or option.usepdb:
